@@ -1,0 +1,404 @@
+/*
+ * ktj.h — C ABI of the MI355X trace post-processing engine ("ktj" = kineto trace → JSON).
+ *
+ * The engine turns raw activity records into Chrome-trace JSON that is byte-identical to what
+ * libkineto's ChromeTraceLogger writes for the same records.  Everything below is plain C:
+ * opaque handle, pointers and sizes, int status codes (0 = ok, negative = error).  Nothing
+ * throws or aborts across this boundary.  One producer thread per engine, like the reference
+ * logger (libkineto/src/output_json.h:62-63).
+ *
+ * Reference interfaces each entry point replaces are cited as file:line relative to the
+ * pytorch/kineto tree.
+ */
+#ifndef KTJ_H_
+#define KTJ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------
+ * Status codes
+ * ---------------------------------------------------------------------------------------- */
+#define KTJ_OK 0
+#define KTJ_ERR_ARG (-1)      /* bad argument (null pointer, unknown id, out-of-range index)   */
+#define KTJ_ERR_STATE (-2)    /* call order violated (e.g. submit after finalize)               */
+#define KTJ_ERR_HIP (-3)      /* a HIP call failed; ktj_last_error() has the text               */
+#define KTJ_ERR_IO (-4)       /* output file could not be opened / written / renamed            */
+#define KTJ_ERR_NOMEM (-5)    /* host or device allocation failed                               */
+#define KTJ_ERR_LIMIT (-6)    /* input exceeds a documented limit                               */
+
+#define KTJ_NONE 0xFFFFFFFFu  /* "no string" / "no schema" sentinel for 32-bit ids              */
+
+/* ------------------------------------------------------------------------------------------
+ * Activity types: numeric values and category strings of libkineto::ActivityType
+ * (libkineto/include/ActivityType.h:19-62, names :80-111).
+ * ---------------------------------------------------------------------------------------- */
+enum {
+  KTJ_TYPE_CPU_OP = 0,
+  KTJ_TYPE_USER_ANNOTATION = 1,
+  KTJ_TYPE_GPU_USER_ANNOTATION = 2,
+  KTJ_TYPE_GPU_MEMCPY = 3,
+  KTJ_TYPE_GPU_MEMSET = 4,
+  KTJ_TYPE_CONCURRENT_KERNEL = 5,
+  KTJ_TYPE_EXTERNAL_CORRELATION = 6,
+  KTJ_TYPE_CUDA_RUNTIME = 7,
+  KTJ_TYPE_CUDA_DRIVER = 8,
+  KTJ_TYPE_CPU_INSTANT_EVENT = 9,
+  KTJ_TYPE_PYTHON_FUNCTION = 10,
+  KTJ_TYPE_OVERHEAD = 11,
+  KTJ_TYPE_MTIA_RUNTIME = 12,
+  KTJ_TYPE_MTIA_CCP_EVENTS = 13,
+  KTJ_TYPE_MTIA_INSIGHT = 14,
+  KTJ_TYPE_CUDA_SYNC = 15,
+  KTJ_TYPE_CUDA_EVENT = 16,
+  KTJ_TYPE_MTIA_COUNTERS = 17,
+  KTJ_TYPE_GLOW_RUNTIME = 18,
+  KTJ_TYPE_CUDA_PROFILER_RANGE = 19,
+  KTJ_TYPE_HPU_OP = 20,
+  KTJ_TYPE_XPU_RUNTIME = 21,
+  KTJ_TYPE_XPU_DRIVER = 22,
+  KTJ_TYPE_COLLECTIVE_COMM = 23,
+  KTJ_TYPE_PRIVATEUSE1_RUNTIME = 24,
+  KTJ_TYPE_PRIVATEUSE1_DRIVER = 25,
+  KTJ_TYPE_XPU_SCOPE_PROFILER = 26,
+  KTJ_TYPE_XPU_SYNC = 27,
+  KTJ_TYPE_HARDWARE_COUNTERS = 28,
+  KTJ_TYPE_COUNT = 29
+};
+
+/* Flow link types (libkineto/include/GenericTraceActivity.h:29-30). */
+#define KTJ_LINK_FWDBWD 1u
+#define KTJ_LINK_ASYNC_CPU_GPU 2u
+
+/* ------------------------------------------------------------------------------------------
+ * Raw activity records (the engine's input "activity buffers").  Packed arrays of fixed-size
+ * little-endian structs; sizes are multiples of 16 so that one lane reads 16 bytes at a time.
+ * ---------------------------------------------------------------------------------------- */
+
+/* Record classes for ktj_submit_records(). */
+enum {
+  KTJ_REC_GENERIC = 0,  /* ktj_generic_rec  */
+  KTJ_REC_RUNTIME = 1,  /* ktj_runtime_rec  */
+  KTJ_REC_DEVICE = 2,   /* ktj_device_rec   */
+  KTJ_REC_EXTCORR = 3   /* ktj_extcorr_rec  */
+};
+
+/*
+ * Generic activity: the fields of libkineto::GenericTraceActivity
+ * (libkineto/include/GenericTraceActivity.h:174-195) plus what ChromeTraceLogger reads from a
+ * linked activity (libkineto/src/output_json.cpp:871-874).  CPU-op spans submitted by a
+ * profiler client and every activity that arrives through ActivityLogger::handleActivity use
+ * this shape.
+ */
+typedef struct ktj_generic_rec {
+  int64_t start_ns;      /* startTime (absolute ns)                                            */
+  int64_t end_ns;        /* endTime; duration() = end_ns - start_ns                            */
+  int64_t resource;      /* resourceId(): thread id or stream id                               */
+  int64_t linked_corr;   /* linkedActivity()->correlationId(); read only if KTJ_GF_LINKED      */
+  uint64_t args_off;     /* first 8-byte slot of this record's values in the args blob         */
+  int32_t id;            /* correlationId() — GenericTraceActivity::id is int32                */
+  int32_t device;        /* deviceId() — process id for CPU ops                                */
+  uint32_t name_id;      /* string id of name()                                                */
+  uint32_t flow_id;      /* flow.id (uint32)                                                   */
+  uint32_t schema_id;    /* args schema, KTJ_NONE = no metadata                                */
+  uint8_t type;          /* KTJ_TYPE_*                                                         */
+  uint8_t flow_type;     /* flow.type (4 bits)                                                 */
+  uint8_t flags;         /* KTJ_GF_*                                                           */
+  uint8_t pad0;
+} ktj_generic_rec;       /* 64 bytes; getThreadId() is never printed and is not carried */
+
+#define KTJ_GF_FLOW_START 0x01u /* flow.start                                                  */
+#define KTJ_GF_LINKED 0x02u     /* linkedActivity() != nullptr                                 */
+
+/* Kinds of runtime rows: libkineto/src/RocLogger.h:74-81 (rocprof_activity_types). */
+enum {
+  KTJ_RT_DEFAULT = 0, /* rocprofRow        (RocLogger.h:101-118) */
+  KTJ_RT_KERNEL = 1,  /* rocprofKernelRow  (RocLogger.h:120-165) */
+  KTJ_RT_COPY = 2,    /* rocprofCopyRow    (RocLogger.h:167-194) */
+  KTJ_RT_MALLOC = 3   /* rocprofMallocRow  (RocLogger.h:196-214) */
+};
+
+/*
+ * Runtime-API row: union of rocprofRow / rocprofKernelRow / rocprofCopyRow / rocprofMallocRow.
+ * begin/end are in the host's approximate-clock domain and go through the clock model
+ * (libkineto/src/RocprofActivityApi.cpp:171-174).
+ */
+typedef struct ktj_runtime_rec {
+  uint64_t id;     /* correlation id                                                          */
+  uint64_t begin;
+  uint64_t end;
+  uint32_t cid;    /* runtime API operation id; name and flow-start come from the API table   */
+  uint32_t pid;
+  uint32_t tid;
+  uint32_t kind;   /* KTJ_RT_*                                                                */
+  union {
+    struct {
+      uint32_t grid[3];
+      uint32_t workgroup[3];
+      uint64_t group_segment_size;
+      uint64_t stream;          /* hipStream_t as integer; 0 = null stream                     */
+      uint32_t kernel_name_id;  /* "kernel" arg when the function pointer is known, else KTJ_NONE */
+      uint32_t pad;
+    } kernel;
+    struct {
+      uint64_t src;
+      uint64_t dst;
+      uint64_t size;
+      uint64_t stream;
+      uint32_t copy_kind;       /* hipMemcpyKind as integer                                    */
+      uint32_t pad;
+    } copy;
+    struct {
+      uint64_t ptr;
+      uint64_t size;
+    } malloc_;
+    uint64_t raw[7];
+  } u;
+} ktj_runtime_rec; /* 96 bytes */
+
+/* Device-row domains. */
+enum {
+  KTJ_DOM_KERNEL_DISPATCH = 0, /* rocprofAsyncRow, ROCPROFILER_BUFFER_TRACING_KERNEL_DISPATCH */
+  KTJ_DOM_MEMORY_COPY = 1,     /* rocprofAsyncRow, ROCPROFILER_BUFFER_TRACING_MEMORY_COPY     */
+  KTJ_DOM_MEMSET = 2           /* memset record shaped like CUpti_ActivityMemset
+                                  (libkineto/src/CuptiActivity.h:682-713)                      */
+};
+
+/* Copy directions: numeric values of rocprofiler_memory_copy_operation_t. */
+enum {
+  KTJ_COPY_NONE = 0,
+  KTJ_COPY_H2H = 1,
+  KTJ_COPY_H2D = 2,
+  KTJ_COPY_D2H = 3,
+  KTJ_COPY_D2D = 4
+};
+
+/*
+ * Device (asynchronous) row: rocprofAsyncRow (libkineto/src/RocLogger.h:216-240).  The kernel
+ * name std::string becomes a string id.  For KTJ_DOM_MEMSET rows `queue` carries the context id
+ * and `stream` must be set by the producer (no back-fill).
+ */
+typedef struct ktj_device_rec {
+  uint64_t id;       /* correlation id                                                        */
+  uint64_t begin;    /* device clock                                                          */
+  uint64_t end;
+  uint32_t domain;   /* KTJ_DOM_*                                                             */
+  uint32_t op;       /* KTJ_COPY_* for copies                                                 */
+  int32_t device;
+  uint32_t name_id;  /* kernel name, KTJ_NONE = empty                                         */
+  uint64_t queue;    /* HSA queue id                                                          */
+  uint64_t stream;   /* 0 = unknown: back-filled from the correlated runtime row              */
+  uint64_t bytes;    /* KTJ_DOM_MEMSET only                                                   */
+} ktj_device_rec;    /* 64 bytes */
+
+/* External-correlation pair, domain 0: (correlation id → CPU-op id)
+ * (libkineto/src/RocmActivityProfiler.cpp:135-148). */
+typedef struct ktj_extcorr_rec {
+  uint64_t correlation;
+  uint64_t external_id;
+} ktj_extcorr_rec; /* 16 bytes */
+
+/* ------------------------------------------------------------------------------------------
+ * Args schemas: the typed metadata of a generic activity, in emission order
+ * (libkineto/include/TypedMetadataJson.h:38-205).  A record's values live in the args blob as
+ * consecutive 8-byte slots starting at args_off; each field consumes `count` slots.
+ * ---------------------------------------------------------------------------------------- */
+enum {
+  KTJ_F_I64 = 0,   /* int64 via to_chars                                  (1 slot)            */
+  KTJ_F_U64 = 1,   /* uint64 via to_chars                                 (1 slot)            */
+  KTJ_F_F64 = 2,   /* double via fmt "{}"; non-finite values are quoted   (1 slot)            */
+  KTJ_F_BOOL = 3,  /* true / false                                        (1 slot)            */
+  KTJ_F_STR = 4,   /* slot = string id, emitted in double quotes          (1 slot)            */
+  KTJ_F_RAW = 5,   /* slot = string id, emitted verbatim (RawJson)        (1 slot)            */
+  KTJ_F_I64_ARRAY = 6 /* [a, b, c] with `count` int64 elements            (count slots)       */
+};
+
+typedef struct ktj_field {
+  uint32_t key_id; /* string id of the key; KTJ_NONE = the slot's string is a whole fragment   */
+  uint16_t type;   /* KTJ_F_*                                                                 */
+  uint16_t count;  /* slots consumed (1 except for arrays)                                    */
+} ktj_field;
+
+#define KTJ_MAX_SCHEMA_FIELDS 32
+
+/* ------------------------------------------------------------------------------------------
+ * Small host-side events (formatted by the host part of the library; O(#devices + #streams)).
+ * ---------------------------------------------------------------------------------------- */
+enum {
+  KTJ_INFO_DEVICE = 0,   /* ktj_device_info   */
+  KTJ_INFO_RESOURCE = 1, /* ktj_resource_info */
+  KTJ_INFO_OVERHEAD = 2, /* ktj_overhead_info */
+  KTJ_INFO_SPAN = 3      /* ktj_trace_span    */
+};
+
+typedef struct ktj_device_info {    /* libkineto/include/IActivityProfiler.h:48-53 */
+  int64_t id;
+  int64_t sort_index;
+  const char* name;
+  const char* label;
+  int64_t time_ns;
+} ktj_device_info;
+
+typedef struct ktj_resource_info {  /* libkineto/include/IActivityProfiler.h:63-70 */
+  int64_t id;
+  int64_t sort_index;
+  int64_t device_id;
+  const char* name;
+  int32_t host_thread;              /* ResourceType::HOST_THREAD */
+  int32_t pad;
+  int64_t time_ns;
+} ktj_resource_info;
+
+typedef struct ktj_overhead_info {  /* libkineto/include/output_base.h:41-44 */
+  const char* name;
+  int64_t time_ns;
+} ktj_overhead_info;
+
+typedef struct ktj_trace_span {     /* libkineto/include/TraceSpan.h:17-36 */
+  int64_t start_ns;
+  int64_t end_ns;
+  int32_t op_count;
+  int32_t iteration;
+  const char* name;
+  const char* prefix;
+} ktj_trace_span;
+
+/* Clock model for raw → wall-clock conversion. */
+typedef struct ktj_clock_model {
+  uint64_t t0_approx;   /* libkineto/src/ApproximateClock.cpp:83-90: for t > t0_approx the       */
+  int64_t t0;           /*   converter returns (int64)((double)(t - t0_approx) * scale) + t0     */
+  double scale;         /*   with the product taken in x87 extended precision; else 0           */
+  int64_t async_offset; /* added to device-row begin/end (RocprofActivityApi.cpp:166-170)       */
+  uint32_t runtime_mode; /* KTJ_CLOCK_* applied to runtime rows                                 */
+  uint32_t device_mode;  /* KTJ_CLOCK_* applied to device rows                                  */
+} ktj_clock_model;
+
+enum {
+  KTJ_CLOCK_IDENTITY = 0, /* timestamps already are wall-clock ns                               */
+  KTJ_CLOCK_CONVERT = 1,  /* apply the converter to begin and end separately
+                             (libkineto/src/CuptiTimestamp.h:29-51)                             */
+  KTJ_CLOCK_OFFSET = 2    /* add async_offset                                                   */
+};
+
+/* Counters of the post-processing stage (libkineto/src/GenericActivityProfiler.cpp:91-102,
+ * 329-340, 363-395) and per-stage timing measured with HIP events on the engine's stream. */
+#define KTJ_N_STAGES 12
+typedef struct ktj_stats {
+  uint64_t n_generic, n_runtime, n_device, n_extcorr;
+  uint64_t n_emitted;              /* activities written                                        */
+  uint64_t out_of_range_events;
+  uint64_t gpu_and_cpu_op_out_of_order;
+  uint64_t n_flow_events;
+  uint64_t n_linked;               /* activities that found a CPU op via external correlation   */
+  uint64_t n_blank_names;          /* names replaced by "unknown"                               */
+  uint64_t output_bytes;
+  uint64_t activity_bytes;         /* bytes of the sorted activity section                      */
+  float stage_ms[KTJ_N_STAGES];    /* see KTJ_STAGE_*                                           */
+  uint64_t stage_bytes[KTJ_N_STAGES]; /* algorithmic bytes moved by that stage                  */
+} ktj_stats;
+
+enum {
+  KTJ_STAGE_DICT = 0,     /* name / string dictionary sanitising                               */
+  KTJ_STAGE_DECODE = 1,   /* raw records → columns                                             */
+  KTJ_STAGE_CONVERT = 2,  /* clock conversion + window filter                                  */
+  KTJ_STAGE_JOIN = 3,     /* hash build + probe (ext-corr, runtime↔device, streams)            */
+  KTJ_STAGE_SORT = 4,     /* key build + stable radix sort                                     */
+  KTJ_STAGE_SIZE = 5,     /* exact byte length per record                                      */
+  KTJ_STAGE_SCAN = 6,     /* device-wide exclusive scan                                        */
+  KTJ_STAGE_EMIT = 7,     /* JSON formatting into the output buffer                            */
+  KTJ_STAGE_D2H = 8,      /* device → pinned host copy                                         */
+  KTJ_STAGE_FILE = 9,     /* write + rename (host)                                             */
+  KTJ_STAGE_TOTAL_GPU = 10 /* first kernel start → last kernel end                             */
+};
+
+typedef struct ktj_engine ktj_engine;
+
+/* ------------------------------------------------------------------------------------------
+ * Life cycle.  Replaces ChromeTraceLogger::ChromeTraceLogger / openTraceFile
+ * (libkineto/src/output_json.cpp:485-505): opens "<out_path>.tmp"; empty or NULL path means
+ * "/tmp/libkineto_activities_<pid>.json".  If the file cannot be opened the engine is still
+ * created and every later call is a silent no-op returning KTJ_OK, like the reference's
+ * `if (!traceOf_) return;`; ktj_finalize then returns KTJ_ERR_IO.
+ * With KTJ_CREATE_NO_FILE no file is opened or written: the document stays in the engine's
+ * buffers (ktj_output_device / ktj_output_host) and out_path is only the "traceName".
+ * ---------------------------------------------------------------------------------------- */
+#define KTJ_CREATE_NO_FILE 0x1u
+int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int hip_device,
+               uint32_t flags);
+void ktj_destroy(ktj_engine* e);
+const char* ktj_last_error(const ktj_engine* e);
+
+/* ChromeTraceLogger::handleTraceStart (output_json.cpp:445-479).  meta_kv holds n_kv key/value
+ * string pairs (2*n_kv pointers) in the order the caller's metadata map iterates, already merged
+ * with the environment metadata (output_json.cpp:433-443). */
+int ktj_trace_start(ktj_engine* e, const char* const* meta_kv, size_t n_kv,
+                    const char* device_properties);
+
+/* String dictionary: names, arg keys, arg string values, raw fragments.  offsets has n+1
+ * entries into blob.  *first_id receives the id of the first string; ids are consecutive. */
+int ktj_intern_strings(ktj_engine* e, const char* blob, const uint64_t* offsets, size_t n,
+                       uint32_t* first_id);
+
+/* Args schema registration (fields in emission order). */
+int ktj_register_schema(ktj_engine* e, const ktj_field* fields, size_t n_fields,
+                        uint32_t* schema_id);
+
+/* Args blob (8-byte slots) referenced by ktj_generic_rec::args_off.  Appends; *first_slot
+ * receives the slot index of the first appended value. */
+int ktj_submit_args(ktj_engine* e, const uint64_t* slots, size_t n_slots, uint64_t* first_slot);
+
+/* Runtime API table: RocprofLogger::opString (libkineto/src/RocprofLogger.cpp:751-760) and
+ * RuntimeActivity::flowStart (libkineto/src/RocprofActivity_inl.h:185-200).
+ * cid_name_ids[cid] = string id of the API name; flow_start_cids lists the cids that start an
+ * ac2g flow; malloc_cid is the cid of hipMalloc, whose rows carry a "bytes" arg
+ * (RocprofActivity_inl.h:265-277), or KTJ_NONE. */
+int ktj_set_api_table(ktj_engine* e, const uint32_t* cid_name_ids, size_t n_cids,
+                      const uint32_t* flow_start_cids, size_t n_flow_start, uint32_t malloc_cid);
+
+int ktj_set_clock_model(ktj_engine* e, const ktj_clock_model* model);
+
+/* Capture window for the out-of-range filter (GenericActivityProfiler.cpp:329-340). */
+int ktj_set_window(ktj_engine* e, int64_t start_ns, int64_t end_ns);
+
+/* Raw record submission: the bulk equivalent of the per-record handleActivity /
+ * handleGenericActivity calls (output_json.cpp:837-971) and of the profiler's per-row handlers
+ * (RocmActivityProfiler.cpp:150-213).  `packed` is host memory; the caller may free it when the
+ * call returns.  Arrival order is: all generic records, then all runtime rows, then all device
+ * rows, each in submission order. */
+int ktj_submit_records(ktj_engine* e, int rec_class, const void* packed, size_t n_records);
+
+/* Same, for records that already live in device memory of the engine's GPU (zero copy; the
+ * buffer must stay valid until ktj_finalize / ktj_process returns). */
+int ktj_submit_records_device(ktj_engine* e, int rec_class, const void* device_ptr,
+                              size_t n_records);
+
+/* handleDeviceInfo / handleResourceInfo / handleOverheadInfo / handleTraceSpan
+ * (output_json.cpp:507-658).  Strings are copied. */
+int ktj_submit_info(ktj_engine* e, int info_kind, const void* info);
+
+/* Runs decode → convert → join → sort → size → scan → emit on the GPU and leaves the finished
+ * document in a device buffer.  end_time_ns is finalizeTrace's endTime.  Idempotent inputs: may
+ * be called again after more ktj_submit_* calls (everything is re-processed). */
+int ktj_process(ktj_engine* e, int64_t end_time_ns);
+
+/* Device / host views of the finished document (valid until the next ktj_process/destroy). */
+int ktj_output_device(ktj_engine* e, const void** device_ptr, uint64_t* n_bytes);
+int ktj_output_host(ktj_engine* e, const char** host_ptr, uint64_t* n_bytes); /* pinned; D2H on first call */
+
+/* ChromeTraceLogger::finalizeTrace (output_json.cpp:1023-1028, 1066-1108): ktj_process if not
+ * done, D2H, write "<path>.tmp", remove + rename. */
+int ktj_finalize(ktj_engine* e, int64_t end_time_ns, uint64_t* bytes_written);
+
+int ktj_get_stats(ktj_engine* e, ktj_stats* out);
+
+/* Library identification; does not touch the GPU. */
+const char* ktj_version(void);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+#endif /* KTJ_H_ */
