@@ -175,20 +175,37 @@ size_t ktj_oracle_fmt_double(double v, char* out) {
   char* o = out;
   if (signbit(v)) { *o++ = '-'; v = -v; }
   if (v == 0.0) { *o++ = '0'; *o = 0; return (size_t)(o - out); }
-  char tmp[48];
-  int prec;
-  for (prec = 1; prec <= 17; ++prec) {
-    snprintf(tmp, sizeof tmp, "%.*e", prec - 1, v);
-    if (strtod(tmp, NULL) == v) break;
-  }
-  /* tmp = d[.ddd]e±XX */
+  /* Shortest-precision search: the first precision p at which some p-digit decimal reads back
+   * as v.  printf gives the p-digit decimal nearest to v; at a power of two the rounding
+   * interval is lopsided, so the p-digit neighbours are tried as well (the closest wins). */
   char digits[24];
-  int nd = 0;
-  const char* q = tmp;
-  for (; *q && *q != 'e'; ++q)
-    if (*q >= '0' && *q <= '9') digits[nd++] = *q;
-  int E = atoi(q + 1);
-  while (nd > 1 && digits[nd - 1] == '0') --nd; /* printf pads; shortest has no trailing zeros */
+  int nd = 0, E = 0;
+  for (int prec = 1; prec <= 17 && nd == 0; ++prec) {
+    char tmp[48];
+    snprintf(tmp, sizeof tmp, "%.*e", prec - 1, v);
+    unsigned long long m = 0;
+    const char* q = tmp;
+    for (; *q && *q != 'e'; ++q)
+      if (*q >= '0' && *q <= '9') m = m * 10 + (unsigned long long)(*q - '0');
+    const int e10 = atoi(q + 1);          /* v ~ m * 10^(e10 - (prec - 1)) */
+    unsigned long long best_m = 0;
+    int have = 0;
+    long double best_err = 0;
+    for (int delta = 0; delta < 3; ++delta) {
+      unsigned long long c = delta == 0 ? m : (delta == 1 ? m + 1 : m - 1);
+      if (c == 0) continue;
+      char cand[64];
+      snprintf(cand, sizeof cand, "%llue%d", c, e10 - (prec - 1));
+      if (strtod(cand, NULL) != v) continue;
+      long double err = fabsl(strtold(cand, NULL) - (long double)v);
+      if (!have || err < best_err) { have = 1; best_err = err; best_m = c; }
+    }
+    if (have) {
+      nd = snprintf(digits, sizeof digits, "%llu", best_m);
+      E = e10 - (prec - 1) + (nd - 1);    /* scientific exponent of the chosen digits */
+    }
+  }
+  while (nd > 1 && digits[nd - 1] == '0') --nd; /* shortest form has no trailing zeros */
   if (E >= -4 && E < 16) {
     if (E >= 0) {
       int i = 0;

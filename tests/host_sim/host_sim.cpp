@@ -1,0 +1,254 @@
+// Host-side simulation of the engine's data path, for CPU tests only.
+//
+// The engine's per-record logic (mat_core.h, fmt_core.h) and its host-formatted events
+// (host_events.cpp) compile as plain C++.  This file drives them sequentially in the same order
+// and with the same join semantics as the HIP kernels (last writer wins by arrival index,
+// output-partitioned tiles with clipping and deferred string copies), with std containers standing
+// in for the GPU hash tables, radix sort and scan.  It lets the byte-level logic be compared with
+// the oracle without a GPU.  It is not linked into libktj.so.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <unordered_map>
+#include <unordered_set>
+#include <vector>
+
+#include "../../kineto_amd/csrc/host_events.h"
+#include "../../kineto_amd/csrc/mat_core.h"
+
+using namespace ktj;
+
+namespace {
+
+struct Views {
+  std::string name_blob, arg_blob;
+  std::vector<uint64_t> name_off, arg_off;
+  std::vector<uint32_t> flags;
+};
+
+// same transformation the dictionary kernels perform
+void build_views(const ktj_stream* s, Views& v) {
+  v.name_off.push_back(0);
+  v.arg_off.push_back(0);
+  for (uint64_t i = 0; i < s->n_strings; ++i) {
+    const char* p = s->str_blob + s->str_off[i];
+    const uint64_t n = s->str_off[i + 1] - s->str_off[i];
+    uint32_t fl = 0;
+    bool blank = true, unknown = false;
+    std::string arg, name;
+    for (uint64_t k = 0; k < n; ++k) {
+      unsigned char c = (unsigned char)p[k];
+      if (c == '\n') continue;
+      if (c == '\\') c = '/';
+      arg += (char)c;
+      if (!(c == ' ' || c == '\t' || c == '\v' || c == '\f' || c == '\r')) blank = false;
+      if (c < 0x20 || c > 0x7e) unknown = true;
+      if (c == '"') name += '\\';
+      name += (char)c;
+    }
+    if (n == 6 && memcmp(p, "kernel", 6) == 0) name = "Kernel";
+    else if (unknown) { name = "unknown"; fl |= KTJ_SF_NAME_UNKNOWN; }
+    if (blank) fl |= KTJ_SF_ARG_BLANK;
+    v.name_blob += name; v.name_off.push_back(v.name_blob.size());
+    v.arg_blob += arg; v.arg_off.push_back(v.arg_blob.size());
+    v.flags.push_back(fl);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+// Returns a malloc'ed buffer with the complete document.
+int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t* out_n) {
+  Views v;
+  build_views(s, v);
+  EmitCtx ctx;
+  ctx.dict.name_blob = v.name_blob.data(); ctx.dict.name_off = v.name_off.data();
+  ctx.dict.arg_blob = v.arg_blob.data(); ctx.dict.arg_off = v.arg_off.data();
+  ctx.dict.flags = v.flags.data(); ctx.dict.n = (uint32_t)s->n_strings;
+  ctx.fields = s->fields; ctx.schemas = s->schemas; ctx.n_schemas = (uint32_t)s->n_schemas;
+  ctx.args = s->args; ctx.n_args = s->n_args; ctx.base_time_ns = s->base_time_ns;
+
+  ClockDev clk;
+  clk.t0_approx = s->clock.t0_approx; clk.t0 = s->clock.t0; memcpy(&clk.scale_bits, &s->clock.scale, 8);
+  clk.async_offset = s->clock.async_offset; clk.runtime_mode = s->clock.runtime_mode; clk.device_mode = s->clock.device_mode;
+
+  const uint64_t ng = s->n_generic, nr = s->n_runtime, nd = s->n_device;
+  std::vector<MatRow> mat(ng + nr + nd);
+
+  // tables (value = winning source index)
+  std::unordered_map<uint64_t, uint64_t> extcorr;          // correlation -> external id (last wins)
+  for (uint64_t i = 0; i < s->n_extcorr; ++i) extcorr[s->extcorr[i].correlation] = s->extcorr[i].external_id;
+  std::unordered_set<uint64_t> cpu_ids;
+  for (uint64_t i = 0; i < ng; ++i) cpu_ids.insert((uint64_t)(int64_t)s->generic[i].id);
+  auto ext_of = [&](uint64_t id) -> int32_t {
+    auto it = extcorr.find(narrow_corr_key(id));
+    if (it == extcorr.end()) return 0;
+    if (!cpu_ids.count(it->second)) return 0;
+    return (int32_t)(int64_t)it->second;
+  };
+  std::vector<uint8_t> flow_start(s->n_cids ? s->n_cids : 1, 0);
+  for (uint64_t i = 0; i < s->n_flow_start; ++i) if (s->flow_start_cids[i] < s->n_cids) flow_start[s->flow_start_cids[i]] = 1;
+
+  for (uint64_t i = 0; i < ng; ++i) mat[i] = mat_generic(s->generic[i]);
+
+  std::unordered_map<uint64_t, uint64_t> stream_src;       // full id -> runtime idx (last wins)
+  std::unordered_map<uint64_t, uint64_t> kernel_src, size_src;  // int-truncated id -> runtime idx (in range, last wins)
+  for (uint64_t i = 0; i < nr; ++i) {
+    const ktj_runtime_rec& r = s->runtime[i];
+    uint64_t b = r.begin, e = r.end;
+    convert_range(clk, clk.runtime_mode, &b, &e);
+    const int64_t ts = (int64_t)b, dur = (int64_t)(e - b);
+    const bool valid = !out_of_range(ts, dur, s->window_start_ns, s->window_end_ns);
+    const uint32_t name = r.cid < s->n_cids ? s->cid_name_ids[r.cid] : KTJ_NONE;
+    mat[ng + i] = mat_runtime(r, ts, dur, valid, ext_of(r.id), name, r.cid < s->n_cids && flow_start[r.cid], r.cid == s->malloc_cid);
+    const uint64_t sid = r.kind == KTJ_RT_KERNEL ? r.u.kernel.stream : r.kind == KTJ_RT_COPY ? r.u.copy.stream : 0;
+    if (sid) stream_src[r.id] = i;
+    if (valid) {
+      const uint64_t key = narrow_corr_key(r.id);
+      if (r.kind == KTJ_RT_KERNEL) kernel_src[key] = i;
+      else if (r.kind == KTJ_RT_COPY || r.kind == KTJ_RT_MALLOC) size_src[key] = i;
+    }
+  }
+  // stream back-fill
+  std::vector<uint64_t> dstream(nd);
+  for (uint64_t i = 0; i < nd; ++i) dstream[i] = s->device[i].stream;
+  if (!stream_src.empty()) {
+    for (uint64_t i = 0; i < nd; ++i) {
+      const ktj_device_rec& d = s->device[i];
+      if (d.domain == KTJ_DOM_MEMSET || dstream[i]) continue;
+      auto it = stream_src.find(d.id);
+      if (it != stream_src.end()) {
+        const ktj_runtime_rec& r = s->runtime[it->second];
+        dstream[i] = r.kind == KTJ_RT_KERNEL ? r.u.kernel.stream : r.u.copy.stream;
+      }
+    }
+    std::unordered_map<uint64_t, uint64_t> by_queue;
+    std::unordered_set<uint64_t> ambiguous;
+    for (uint64_t i = 0; i < nd; ++i) {
+      const ktj_device_rec& d = s->device[i];
+      if (d.domain == KTJ_DOM_MEMSET || !dstream[i] || !d.queue) continue;
+      auto it = by_queue.find(d.queue);
+      if (it == by_queue.end()) by_queue[d.queue] = dstream[i];
+      else if (it->second != dstream[i]) ambiguous.insert(d.queue);
+    }
+    for (uint64_t i = 0; i < nd; ++i) {
+      const ktj_device_rec& d = s->device[i];
+      if (d.domain == KTJ_DOM_MEMSET || dstream[i]) continue;
+      auto it = by_queue.find(d.queue);
+      if (it != by_queue.end() && !ambiguous.count(d.queue)) dstream[i] = it->second;
+    }
+    // dense index = 1 + number of distinct keys of the same device first seen earlier
+    struct Ent { int32_t dev; uint64_t key; uint64_t first; };
+    std::vector<Ent> ents;
+    auto key_of = [&](uint64_t i, uint64_t* key) {
+      const ktj_device_rec& d = s->device[i];
+      if (d.domain == KTJ_DOM_MEMSET) return false;
+      if (dstream[i]) *key = dstream[i]; else if (d.queue) *key = d.queue | (1ULL << 63); else return false;
+      return true;
+    };
+    for (uint64_t i = 0; i < nd; ++i) {
+      uint64_t key;
+      if (!key_of(i, &key)) continue;
+      bool found = false;
+      for (auto& e : ents) if (e.dev == s->device[i].device && e.key == key) { found = true; break; }
+      if (!found) ents.push_back({s->device[i].device, key, i});
+    }
+    for (uint64_t i = 0; i < nd; ++i) {
+      uint64_t key;
+      if (!key_of(i, &key)) continue;
+      uint64_t my_first = 0, rank = 1;
+      for (auto& e : ents) if (e.dev == s->device[i].device && e.key == key) my_first = e.first;
+      for (auto& e : ents) if (e.dev == s->device[i].device && e.first < my_first) ++rank;
+      dstream[i] = rank;
+    }
+  }
+  for (uint64_t i = 0; i < nd; ++i) {
+    const ktj_device_rec& d = s->device[i];
+    uint64_t b = d.begin, e = d.end;
+    convert_range(clk, clk.device_mode, &b, &e);
+    int64_t ts, dur;
+    device_times(d.domain, b, e, &ts, &dur);
+    const bool valid = !out_of_range(ts, dur, s->window_start_ns, s->window_end_ns);
+    const int64_t res = d.domain == KTJ_DOM_MEMSET ? (int64_t)d.stream : (int64_t)(dstream[i] ? dstream[i] : d.queue);
+    const uint64_t key = narrow_corr_key(d.id);
+    const ktj_runtime_rec* ksrc = nullptr;
+    bool has_size = false;
+    uint64_t size = 0;
+    if (d.domain != KTJ_DOM_MEMSET) {
+      auto si = size_src.find(key);
+      if (si != size_src.end()) {
+        const ktj_runtime_rec& r = s->runtime[si->second];
+        has_size = true;
+        size = r.kind == KTJ_RT_COPY ? r.u.copy.size : r.u.malloc_.size;
+      } else {
+        auto ki = kernel_src.find(key);
+        if (ki != kernel_src.end()) ksrc = &s->runtime[ki->second];
+      }
+    }
+    mat[ng + nr + i] = mat_device(d, ts, dur, res, valid, ext_of(d.id), ksrc, has_size, size);
+  }
+
+  // canonical order over valid rows
+  std::vector<uint64_t> perm;
+  for (uint64_t a = 0; a < mat.size(); ++a) if (mat[a].meta & KTJ_M_VALID) perm.push_back(a);
+  std::stable_sort(perm.begin(), perm.end(), [&](uint64_t x, uint64_t y) {
+    const MatRow &a = mat[x], &b = mat[y];
+    if (a.dev != b.dev) return a.dev < b.dev;
+    if (a.res != b.res) return a.res < b.res;
+    return a.ts < b.ts;
+  });
+  std::vector<uint64_t> offs(perm.size() + 1, 0);
+  for (size_t i = 0; i < perm.size(); ++i) {
+    CountWriter cw;
+    format_activity(cw, mat[perm[i]], ctx);
+    offs[i + 1] = offs[i] + cw.n;
+  }
+  const uint64_t act_bytes = offs.back();
+
+  std::string prefix, suffix;
+  append_trace_start(prefix, s->meta_kv, s->n_meta, s->device_properties, s->base_time_ns);
+  for (uint64_t i = 0; i < s->n_device_infos; ++i) append_device_info(prefix, s->device_infos[i], s->base_time_ns);
+  for (uint64_t i = 0; i < s->n_resource_infos; ++i) append_resource_info(prefix, s->resource_infos[i], s->base_time_ns);
+  for (uint64_t i = 0; i < s->n_overhead_infos; ++i) append_overhead_info(prefix, s->overhead_infos[i], s->base_time_ns);
+  for (uint64_t i = 0; i < s->n_spans; ++i) append_trace_span(suffix, s->spans[i], s->base_time_ns);
+  append_trace_end(suffix, s->end_time_ns, s->base_time_ns, s->trace_name);
+
+  const uint64_t total = prefix.size() + act_bytes + suffix.size();
+  char* buf = (char*)malloc(total ? total : 1);
+  if (!buf) return -1;
+  memset(buf, '#', total);
+  memcpy(buf, prefix.data(), prefix.size());
+  memcpy(buf + prefix.size() + act_bytes, suffix.data(), suffix.size());
+  char* act = buf + prefix.size();
+
+  // output-partitioned tiles
+  std::vector<char> tile(tile_bytes);
+  std::vector<CopyJob> jobs(64);
+  for (uint64_t lo = 0; lo < act_bytes; lo += tile_bytes) {
+    const uint64_t hi = std::min<uint64_t>(lo + tile_bytes, act_bytes);
+    // first record ending after lo, last record starting before hi
+    size_t r0 = std::upper_bound(offs.begin(), offs.end(), lo) - offs.begin() - 1;
+    size_t r1 = std::lower_bound(offs.begin(), offs.end(), hi) - offs.begin();  // exclusive
+    uint32_t nj = 0;
+    for (size_t r = r0; r < r1; ++r) {
+      TileWriter w;
+      w.buf = tile.data(); w.pos = (int32_t)((int64_t)offs[r] - (int64_t)lo); w.tile = (int32_t)(hi - lo);
+      w.jobs = jobs.data(); w.n_jobs = &nj; w.max_jobs = (uint32_t)jobs.size();
+      format_activity(w, mat[perm[r]], ctx);
+      if ((int64_t)w.pos != (int64_t)offs[r + 1] - (int64_t)lo) { free(buf); return -2; }
+    }
+    const uint32_t done = nj < jobs.size() ? nj : (uint32_t)jobs.size();
+    for (uint32_t j = 0; j < done; ++j) memcpy(tile.data() + jobs[j].dst, jobs[j].src, jobs[j].len);
+    memcpy(act + lo, tile.data(), hi - lo);
+  }
+  *out = buf;
+  *out_n = total;
+  return 0;
+}
+
+void ktjsim_free(char* p) { free(p); }
+
+}  // extern "C"
