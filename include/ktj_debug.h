@@ -1,0 +1,39 @@
+/*
+ * ktj_debug.h — read-back of the engine's intermediate device arrays, for stage-level tests.
+ * Not part of the drop-in surface; no counterpart in the reference.
+ */
+#ifndef KTJ_DEBUG_H_
+#define KTJ_DEBUG_H_
+
+#include "ktj.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  KTJ_DBG_COL_TS = 0,     /* int64[N]  timestamp() per arrival index            */
+  KTJ_DBG_COL_DUR = 1,    /* int64[N]  duration()                               */
+  KTJ_DBG_COL_DEV = 2,    /* int64[N]                                           */
+  KTJ_DBG_COL_RES = 3,    /* int64[N]  resourceId() after stream back-fill      */
+  KTJ_DBG_COL_META = 4,   /* uint32[N] bit 9 = inside the capture window        */
+  KTJ_DBG_COL_EXT = 5,    /* int32[N]  "External id" of runtime/device rows     */
+  KTJ_DBG_PERM = 6,       /* uint32[N] arrival index per sorted position        */
+  KTJ_DBG_LEN = 7,        /* uint32[N] byte length per sorted position          */
+  KTJ_DBG_OFFS = 8,       /* uint64[N+1] exclusive scan of the lengths          */
+  KTJ_DBG_MAT = 9,        /* 96-byte joined rows per arrival index              */
+  KTJ_DBG_SORT_KEYS = 10, /* uint64[N] sorted composite keys                    */
+  KTJ_DBG_NAME_VIEW = 11, /* bytes: all names after the name pipeline           */
+  KTJ_DBG_NAME_OFF = 12,  /* uint64[n_strings+1]                                */
+  KTJ_DBG_ARG_VIEW = 13,
+  KTJ_DBG_ARG_OFF = 14
+};
+
+/* Copies the array to dst (at most cap bytes) and reports its full size.  Valid after
+ * ktj_process. */
+int ktj_debug_fetch(ktj_engine* e, int what, void* dst, uint64_t cap, uint64_t* n_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

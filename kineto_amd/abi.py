@@ -222,6 +222,8 @@ def load_engine():
         lib.ktj_get_stats.argtypes = [vp, C.POINTER(Stats)]
         lib.ktj_version.restype = C.c_char_p
         lib.ktj_version.argtypes = []
+        lib.ktj_debug_fetch.restype = C.c_int
+        lib.ktj_debug_fetch.argtypes = [vp, C.c_int, C.c_void_p, C.c_uint64, C.POINTER(C.c_uint64)]
         _engine = lib
     return _engine
 

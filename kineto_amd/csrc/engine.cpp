@@ -1,0 +1,732 @@
+/*
+ * engine.cpp — host side of the trace post-processing engine behind the C ABI of include/ktj.h:
+ * owns device memory, accepts submissions, orders the kernel stages on one HIP stream, formats
+ * the handful of non-activity events and moves the finished document to the host / file.
+ *
+ * There is no CPU implementation of the activity path in this library: if a HIP call fails the
+ * entry point returns KTJ_ERR_HIP.
+ */
+#include <hip/hip_runtime_api.h>
+
+#include <cerrno>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <unistd.h>
+#include <vector>
+
+#include "../../include/ktj_debug.h"
+#include "gpu_stages.h"
+#include "host_events.h"
+
+using namespace ktj;
+using namespace ktj::gpu;
+
+namespace {
+
+struct DevBuf {
+  void* p = nullptr;
+  size_t cap = 0;
+  hipError_t ensure(size_t bytes) {
+    if (bytes <= cap) return hipSuccess;
+    if (p) { hipError_t e = hipFree(p); p = nullptr; cap = 0; if (e != hipSuccess) return e; }
+    size_t want = bytes + bytes / 8 + 256;
+    hipError_t e = hipMalloc(&p, want);
+    if (e != hipSuccess) { p = nullptr; return e; }
+    cap = want;
+    return hipSuccess;
+  }
+  void release() { if (p) (void)hipFree(p); p = nullptr; cap = 0; }
+  template <typename T> T* as() const { return reinterpret_cast<T*>(p); }
+};
+
+/* append-only device array fed from host memory */
+struct DevVec {
+  DevBuf buf;
+  size_t bytes = 0;
+  hipError_t append(const void* src, size_t n, hipStream_t st) {
+    if (n == 0) return hipSuccess;
+    if (bytes + n > buf.cap) {
+      DevBuf nb;
+      size_t want = (bytes + n) * 2;
+      hipError_t e = nb.ensure(want);
+      if (e != hipSuccess) return e;
+      if (bytes) { e = hipMemcpyAsync(nb.p, buf.p, bytes, hipMemcpyDeviceToDevice, st); if (e != hipSuccess) return e; }
+      e = hipStreamSynchronize(st);
+      if (e != hipSuccess) return e;
+      buf.release();
+      buf = nb;
+    }
+    hipError_t e = hipMemcpyAsync(static_cast<char*>(buf.p) + bytes, src, n, hipMemcpyHostToDevice, st);
+    if (e != hipSuccess) return e;
+    e = hipStreamSynchronize(st); /* caller may free src when we return */
+    if (e != hipSuccess) return e;
+    bytes += n;
+    return hipSuccess;
+  }
+  void release() { buf.release(); bytes = 0; }
+};
+
+struct RecordSet {
+  DevVec owned;
+  const void* external = nullptr; /* device pointer supplied by the caller */
+  uint64_t n = 0;
+  const void* ptr() const { return external ? external : owned.buf.p; }
+};
+
+enum { EV_START = 0, EV_DICT, EV_DECODE, EV_CONVERT, EV_JOIN, EV_SORT_A, EV_SORT_B, EV_SORT, EV_SIZE, EV_SCAN,
+       EV_EMIT_START, EV_EMIT, EV_COUNT };
+
+}  // namespace
+
+struct ktj_engine {
+  std::string out_path, tmp_path, last_error;
+  int64_t base_time_ns = 0;
+  int device = 0;
+  uint32_t flags = 0;
+  FILE* sink = nullptr;
+  bool bad_sink = false;
+  bool started = false;
+  bool processed = false;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev[EV_COUNT] = {};
+  hipEvent_t ev_d2h[2] = {};
+
+  /* inputs */
+  std::string txt_header, txt_dev, txt_res, txt_ovh, txt_span;
+  DevVec str_blob, str_off; /* str_off holds n_strings + 1 absolute offsets */
+  uint64_t n_strings = 0, blob_bytes = 0;
+  std::vector<ktj_field> fields;
+  std::vector<ktj_schema_desc> schemas;
+  DevBuf d_fields, d_schemas;
+  bool schemas_dirty = true;
+  DevVec args;
+  uint64_t n_args = 0;
+  std::vector<uint32_t> cid_names, flow_bits;
+  uint32_t malloc_cid = KTJ_NONE;
+  DevBuf d_cid_names, d_flow_bits;
+  bool api_dirty = true;
+  ktj_clock_model clock{};
+  int64_t win_start = INT64_MIN, win_end = INT64_MAX;
+  RecordSet generic, runtime, devrows, extcorr;
+
+  /* working buffers */
+  DevBuf d_scalars, d_name_len, d_arg_len, d_sflags, d_name_off, d_arg_off, d_name_blob, d_arg_blob;
+  DevBuf c_ts, c_dur, c_corr, c_dev, c_res, c_meta, c_ext;
+  DevBuf t_ext_k, t_ext_v, t_cpu_k, t_id_k, t_id_v0, t_id_v1, t_nr_k, t_nr_v0, t_nr_v1;
+  DevBuf q_keys, q_stream, q_amb, dn_hash, dn_first, dn_dev, dn_key, dn_rank;
+  DevBuf s_dev_k, s_dev_r, s_res_k, s_res_r;
+  DevBuf keys_a, keys_b, vals_a, vals_b, hist, scan_tmp;
+  DevBuf mat, len, len_sorted, offs, out;
+  void* pinned_small = nullptr; size_t pinned_small_cap = 0;
+  char* pinned_out = nullptr; size_t pinned_out_cap = 0;
+  bool host_copy_valid = false;
+
+  /* results */
+  uint64_t N = 0, prefix_len = 0, act_bytes = 0, total_bytes = 0;
+  uint32_t* perm = nullptr; uint64_t* sorted_keys = nullptr;
+  Scalars scalars{};
+  ktj_stats stats{};
+};
+
+namespace {
+
+int fail_hip(ktj_engine* e, hipError_t err, const char* what) {
+  e->last_error = std::string(what) + ": " + hipGetErrorString(err);
+  return KTJ_ERR_HIP;
+}
+#define HIPCHK(call)                                            \
+  do {                                                          \
+    hipError_t _e = (call);                                     \
+    if (_e != hipSuccess) return fail_hip(e, _e, #call);        \
+  } while (0)
+
+uint32_t pow2_at_least(uint64_t v) {
+  uint64_t c = 1024;
+  while (c < v) c <<= 1;
+  return (uint32_t)c;
+}
+
+std::string default_file_name() { /* output_json.cpp:65-70, 481-483 */
+  return "/tmp/libkineto_activities_" + std::to_string((long)getpid()) + ".json";
+}
+
+int upload_small(ktj_engine* e, DevBuf& dst, const void* src, size_t bytes) {
+  HIPCHK(dst.ensure(bytes ? bytes : 16));
+  if (bytes) HIPCHK(hipMemcpyAsync(dst.p, src, bytes, hipMemcpyHostToDevice, e->stream));
+  HIPCHK(hipStreamSynchronize(e->stream));
+  return KTJ_OK;
+}
+
+int bits_for(uint64_t max_value) { /* bits needed to hold values 0..max_value */
+  int b = 0;
+  while (b < 64 && (max_value >> b) != 0) ++b;
+  return b;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* ktj_version(void) { return "ktj 0.1 (gfx950)"; }
+
+int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int hip_device, uint32_t flags) {
+  if (!out) return KTJ_ERR_ARG;
+  *out = nullptr;
+  ktj_engine* e = new (std::nothrow) ktj_engine();
+  if (!e) return KTJ_ERR_NOMEM;
+  e->out_path = (out_path && out_path[0]) ? out_path : default_file_name();
+  e->tmp_path = e->out_path + ".tmp";
+  e->base_time_ns = base_time_ns;
+  e->device = hip_device;
+  e->flags = flags;
+  e->clock.scale = 1.0;
+  *out = e; /* from here on errors are reported through the handle */
+  if (!(flags & KTJ_CREATE_NO_FILE)) { /* openTraceFile, output_json.cpp:485-493 */
+    e->sink = fopen(e->tmp_path.c_str(), "w");
+    if (!e->sink) { e->bad_sink = true; e->last_error = "Failed to open '" + e->out_path + "': " + strerror(errno); }
+  }
+  HIPCHK(hipSetDevice(hip_device));
+  HIPCHK(hipStreamCreate(&e->stream));
+  for (auto& ev : e->ev) HIPCHK(hipEventCreate(&ev));
+  for (auto& ev : e->ev_d2h) HIPCHK(hipEventCreate(&ev));
+  HIPCHK(e->d_scalars.ensure(sizeof(Scalars)));
+  return KTJ_OK;
+}
+
+void ktj_destroy(ktj_engine* e) {
+  if (!e) return;
+  (void)hipSetDevice(e->device);
+  if (e->stream) (void)hipStreamSynchronize(e->stream);
+  DevBuf* bufs[] = {&e->d_fields, &e->d_schemas, &e->d_cid_names, &e->d_flow_bits, &e->d_scalars, &e->d_name_len,
+                    &e->d_arg_len, &e->d_sflags, &e->d_name_off, &e->d_arg_off, &e->d_name_blob, &e->d_arg_blob,
+                    &e->c_ts, &e->c_dur, &e->c_corr, &e->c_dev, &e->c_res, &e->c_meta, &e->c_ext, &e->t_ext_k,
+                    &e->t_ext_v, &e->t_cpu_k, &e->t_id_k, &e->t_id_v0, &e->t_id_v1, &e->t_nr_k, &e->t_nr_v0,
+                    &e->t_nr_v1, &e->q_keys, &e->q_stream, &e->q_amb, &e->dn_hash, &e->dn_first, &e->dn_dev,
+                    &e->dn_key, &e->dn_rank, &e->s_dev_k, &e->s_dev_r, &e->s_res_k, &e->s_res_r, &e->keys_a,
+                    &e->keys_b, &e->vals_a, &e->vals_b, &e->hist, &e->scan_tmp, &e->mat, &e->len, &e->len_sorted,
+                    &e->offs, &e->out};
+  for (DevBuf* b : bufs) b->release();
+  e->str_blob.release(); e->str_off.release(); e->args.release();
+  e->generic.owned.release(); e->runtime.owned.release(); e->devrows.owned.release(); e->extcorr.owned.release();
+  if (e->pinned_small) (void)hipHostFree(e->pinned_small);
+  if (e->pinned_out) (void)hipHostFree(e->pinned_out);
+  for (auto& ev : e->ev) if (ev) (void)hipEventDestroy(ev);
+  for (auto& ev : e->ev_d2h) if (ev) (void)hipEventDestroy(ev);
+  if (e->stream) (void)hipStreamDestroy(e->stream);
+  if (e->sink) { fclose(e->sink); remove(e->tmp_path.c_str()); }
+  delete e;
+}
+
+const char* ktj_last_error(const ktj_engine* e) { return e ? e->last_error.c_str() : "null engine"; }
+
+int ktj_trace_start(ktj_engine* e, const char* const* meta_kv, size_t n_kv, const char* device_properties) {
+  if (!e || (n_kv && !meta_kv)) return KTJ_ERR_ARG;
+  if (e->bad_sink) return KTJ_OK;
+  e->txt_header.clear();
+  append_trace_start(e->txt_header, meta_kv, n_kv, device_properties, e->base_time_ns);
+  e->started = true;
+  e->processed = false;
+  return KTJ_OK;
+}
+
+int ktj_intern_strings(ktj_engine* e, const char* blob, const uint64_t* offsets, size_t n, uint32_t* first_id) {
+  if (!e || (n && (!blob || !offsets))) return KTJ_ERR_ARG;
+  if (first_id) *first_id = (uint32_t)e->n_strings;
+  if (e->bad_sink || n == 0) return KTJ_OK;
+  if (e->n_strings + n >= KTJ_NONE) return KTJ_ERR_LIMIT;
+  HIPCHK(hipSetDevice(e->device));
+  const uint64_t src0 = offsets[0], nbytes = offsets[n] - offsets[0];
+  std::vector<uint64_t> abs_off(n + 1);
+  for (size_t i = 0; i <= n; ++i) {
+    if (offsets[i] < src0 || (i && offsets[i] < offsets[i - 1])) return KTJ_ERR_ARG;
+    abs_off[i] = e->blob_bytes + (offsets[i] - src0);
+  }
+  HIPCHK(e->str_blob.append(blob + src0, nbytes, e->stream));
+  if (e->n_strings == 0) HIPCHK(e->str_off.append(abs_off.data(), (n + 1) * 8, e->stream));
+  else HIPCHK(e->str_off.append(abs_off.data() + 1, n * 8, e->stream)); /* entry n_strings already equals blob_bytes */
+  e->n_strings += n;
+  e->blob_bytes += nbytes;
+  e->processed = false;
+  return KTJ_OK;
+}
+
+int ktj_register_schema(ktj_engine* e, const ktj_field* f, size_t n_fields, uint32_t* schema_id) {
+  if (!e || (n_fields && !f)) return KTJ_ERR_ARG;
+  if (n_fields > KTJ_MAX_SCHEMA_FIELDS) return KTJ_ERR_LIMIT;
+  for (size_t i = 0; i < n_fields; ++i)
+    if (f[i].type > KTJ_F_I64_ARRAY || f[i].count == 0 || (f[i].type != KTJ_F_I64_ARRAY && f[i].count != 1)) return KTJ_ERR_ARG;
+  ktj_schema_desc d;
+  d.first_field = (uint32_t)e->fields.size();
+  d.n_fields = (uint32_t)n_fields;
+  e->fields.insert(e->fields.end(), f, f + n_fields);
+  if (schema_id) *schema_id = (uint32_t)e->schemas.size();
+  e->schemas.push_back(d);
+  e->schemas_dirty = true;
+  e->processed = false;
+  return KTJ_OK;
+}
+
+int ktj_submit_args(ktj_engine* e, const uint64_t* slots, size_t n_slots, uint64_t* first_slot) {
+  if (!e || (n_slots && !slots)) return KTJ_ERR_ARG;
+  if (first_slot) *first_slot = e->n_args;
+  if (e->bad_sink || n_slots == 0) return KTJ_OK;
+  HIPCHK(hipSetDevice(e->device));
+  HIPCHK(e->args.append(slots, n_slots * 8, e->stream));
+  e->n_args += n_slots;
+  e->processed = false;
+  return KTJ_OK;
+}
+
+int ktj_set_api_table(ktj_engine* e, const uint32_t* cid_name_ids, size_t n_cids, const uint32_t* flow_start_cids,
+                      size_t n_flow_start, uint32_t malloc_cid) {
+  if (!e || (n_cids && !cid_name_ids) || (n_flow_start && !flow_start_cids)) return KTJ_ERR_ARG;
+  e->cid_names.assign(cid_name_ids, cid_name_ids + n_cids);
+  e->flow_bits.assign((n_cids + 31) / 32 + 1, 0u);
+  for (size_t i = 0; i < n_flow_start; ++i)
+    if (flow_start_cids[i] < n_cids) e->flow_bits[flow_start_cids[i] >> 5] |= 1u << (flow_start_cids[i] & 31u);
+  e->malloc_cid = malloc_cid;
+  e->api_dirty = true;
+  e->processed = false;
+  return KTJ_OK;
+}
+
+int ktj_set_clock_model(ktj_engine* e, const ktj_clock_model* m) {
+  if (!e || !m) return KTJ_ERR_ARG;
+  if (m->runtime_mode > KTJ_CLOCK_OFFSET || m->device_mode > KTJ_CLOCK_OFFSET) return KTJ_ERR_ARG;
+  e->clock = *m;
+  e->processed = false;
+  return KTJ_OK;
+}
+
+int ktj_set_window(ktj_engine* e, int64_t start_ns, int64_t end_ns) {
+  if (!e) return KTJ_ERR_ARG;
+  e->win_start = start_ns;
+  e->win_end = end_ns;
+  e->processed = false;
+  return KTJ_OK;
+}
+
+static RecordSet* record_set(ktj_engine* e, int rec_class, size_t* rec_size) {
+  switch (rec_class) {
+    case KTJ_REC_GENERIC: *rec_size = sizeof(ktj_generic_rec); return &e->generic;
+    case KTJ_REC_RUNTIME: *rec_size = sizeof(ktj_runtime_rec); return &e->runtime;
+    case KTJ_REC_DEVICE: *rec_size = sizeof(ktj_device_rec); return &e->devrows;
+    case KTJ_REC_EXTCORR: *rec_size = sizeof(ktj_extcorr_rec); return &e->extcorr;
+    default: return nullptr;
+  }
+}
+
+int ktj_submit_records(ktj_engine* e, int rec_class, const void* packed, size_t n_records) {
+  if (!e || (n_records && !packed)) return KTJ_ERR_ARG;
+  size_t rs = 0;
+  RecordSet* set = record_set(e, rec_class, &rs);
+  if (!set) return KTJ_ERR_ARG;
+  if (e->bad_sink || n_records == 0) return KTJ_OK;
+  if (set->external) return KTJ_ERR_STATE;
+  HIPCHK(hipSetDevice(e->device));
+  HIPCHK(set->owned.append(packed, n_records * rs, e->stream));
+  set->n += n_records;
+  e->processed = false;
+  return KTJ_OK;
+}
+
+int ktj_submit_records_device(ktj_engine* e, int rec_class, const void* device_ptr, size_t n_records) {
+  if (!e || (n_records && !device_ptr)) return KTJ_ERR_ARG;
+  size_t rs = 0;
+  RecordSet* set = record_set(e, rec_class, &rs);
+  if (!set) return KTJ_ERR_ARG;
+  if (((uintptr_t)device_ptr & 15u) != 0) return KTJ_ERR_ARG; /* kernels read 16-byte lanes */
+  if (e->bad_sink) return KTJ_OK;
+  if (set->owned.bytes != 0) return KTJ_ERR_STATE;
+  set->external = n_records ? device_ptr : nullptr;
+  set->n = n_records;
+  e->processed = false;
+  return KTJ_OK;
+}
+
+int ktj_submit_info(ktj_engine* e, int info_kind, const void* info) {
+  if (!e || !info) return KTJ_ERR_ARG;
+  if (e->bad_sink) return KTJ_OK;
+  switch (info_kind) {
+    case KTJ_INFO_DEVICE: append_device_info(e->txt_dev, *static_cast<const ktj_device_info*>(info), e->base_time_ns); break;
+    case KTJ_INFO_RESOURCE: append_resource_info(e->txt_res, *static_cast<const ktj_resource_info*>(info), e->base_time_ns); break;
+    case KTJ_INFO_OVERHEAD: append_overhead_info(e->txt_ovh, *static_cast<const ktj_overhead_info*>(info), e->base_time_ns); break;
+    case KTJ_INFO_SPAN: append_trace_span(e->txt_span, *static_cast<const ktj_trace_span*>(info), e->base_time_ns); break;
+    default: return KTJ_ERR_ARG;
+  }
+  e->processed = false;
+  return KTJ_OK;
+}
+
+int ktj_process(ktj_engine* e, int64_t end_time_ns) {
+  if (!e) return KTJ_ERR_ARG;
+  if (e->bad_sink) return KTJ_OK;
+  HIPCHK(hipSetDevice(e->device));
+  hipStream_t st = e->stream;
+  const uint64_t ng = e->generic.n, nr = e->runtime.n, nd = e->devrows.n, nx = e->extcorr.n;
+  const uint64_t N = ng + nr + nd;
+  if (N >= 0xFFFFFFF0ull) { e->last_error = "more than 2^32 - 16 records"; return KTJ_ERR_LIMIT; }
+  e->N = N;
+  e->host_copy_valid = false;
+  const uint64_t Na = N ? N : 1;
+
+  /* small tables */
+  if (e->schemas_dirty) {
+    int rc = upload_small(e, e->d_fields, e->fields.data(), e->fields.size() * sizeof(ktj_field));
+    if (rc) return rc;
+    rc = upload_small(e, e->d_schemas, e->schemas.data(), e->schemas.size() * sizeof(ktj_schema_desc));
+    if (rc) return rc;
+    e->schemas_dirty = false;
+  }
+  if (e->api_dirty) {
+    int rc = upload_small(e, e->d_cid_names, e->cid_names.data(), e->cid_names.size() * 4);
+    if (rc) return rc;
+    if (e->flow_bits.empty()) e->flow_bits.assign(1, 0u);
+    rc = upload_small(e, e->d_flow_bits, e->flow_bits.data(), e->flow_bits.size() * 4);
+    if (rc) return rc;
+    e->api_dirty = false;
+  }
+
+  /* working memory */
+  const uint32_t ns = (uint32_t)e->n_strings;
+  HIPCHK(e->d_name_len.ensure((ns + 1) * 4ull)); HIPCHK(e->d_arg_len.ensure((ns + 1) * 4ull));
+  HIPCHK(e->d_sflags.ensure((ns + 1) * 4ull));
+  HIPCHK(e->d_name_off.ensure((ns + 2) * 8ull)); HIPCHK(e->d_arg_off.ensure((ns + 2) * 8ull));
+  HIPCHK(e->d_name_blob.ensure(e->blob_bytes * 2 + 8ull * ns + 16)); HIPCHK(e->d_arg_blob.ensure(e->blob_bytes + 16));
+  HIPCHK(e->c_ts.ensure(Na * 8)); HIPCHK(e->c_dur.ensure(Na * 8)); HIPCHK(e->c_corr.ensure(Na * 8));
+  HIPCHK(e->c_dev.ensure(Na * 8)); HIPCHK(e->c_res.ensure(Na * 8)); HIPCHK(e->c_meta.ensure(Na * 4));
+  HIPCHK(e->c_ext.ensure(Na * 4));
+  const uint32_t cap_ext = pow2_at_least(2 * nx), cap_cpu = pow2_at_least(2 * ng);
+  const uint32_t cap_id = pow2_at_least(2 * (nr + nd)), cap_nr = pow2_at_least(2 * nr);
+  HIPCHK(e->t_ext_k.ensure((cap_ext + 1ull) * 8)); HIPCHK(e->t_ext_v.ensure((cap_ext + 1ull) * 4));
+  HIPCHK(e->t_cpu_k.ensure((cap_cpu + 1ull) * 8));
+  HIPCHK(e->t_id_k.ensure((cap_id + 1ull) * 8)); HIPCHK(e->t_id_v0.ensure((cap_id + 1ull) * 4));
+  HIPCHK(e->t_id_v1.ensure((cap_id + 1ull) * 4));
+  HIPCHK(e->t_nr_k.ensure((cap_nr + 1ull) * 8)); HIPCHK(e->t_nr_v0.ensure((cap_nr + 1ull) * 4));
+  HIPCHK(e->t_nr_v1.ensure((cap_nr + 1ull) * 4));
+  HIPCHK(e->q_keys.ensure((KTJ_QUEUE_CAP + 1ull) * 8)); HIPCHK(e->q_stream.ensure((KTJ_QUEUE_CAP + 1ull) * 8));
+  HIPCHK(e->q_amb.ensure((KTJ_QUEUE_CAP + 1ull) * 4));
+  HIPCHK(e->dn_hash.ensure((KTJ_DENSE_CAP + 1ull) * 8)); HIPCHK(e->dn_first.ensure((KTJ_DENSE_CAP + 1ull) * 4));
+  HIPCHK(e->dn_dev.ensure((KTJ_DENSE_CAP + 1ull) * 4)); HIPCHK(e->dn_key.ensure((KTJ_DENSE_CAP + 1ull) * 8));
+  HIPCHK(e->dn_rank.ensure((KTJ_DENSE_CAP + 1ull) * 4));
+  HIPCHK(e->s_dev_k.ensure((KTJ_SET_CAP + 1ull) * 8)); HIPCHK(e->s_dev_r.ensure((KTJ_SET_CAP + 1ull) * 4));
+  HIPCHK(e->s_res_k.ensure((KTJ_SET_CAP + 1ull) * 8)); HIPCHK(e->s_res_r.ensure((KTJ_SET_CAP + 1ull) * 4));
+  HIPCHK(e->keys_a.ensure(Na * 8)); HIPCHK(e->keys_b.ensure(Na * 8));
+  HIPCHK(e->vals_a.ensure(Na * 4)); HIPCHK(e->vals_b.ensure(Na * 4));
+  HIPCHK(e->hist.ensure(radix_tmp_elems(Na) * 4));
+  {
+    uint64_t m = scan_tmp_elems(radix_tmp_elems(Na));
+    const uint64_t m2 = scan_tmp_elems(Na), m3 = scan_tmp_elems(ns + 1ull);
+    if (m2 > m) m = m2;
+    if (m3 > m) m = m3;
+    HIPCHK(e->scan_tmp.ensure(m * 8));
+  }
+  HIPCHK(e->mat.ensure(Na * sizeof(MatRow))); HIPCHK(e->len.ensure(Na * 4)); HIPCHK(e->len_sorted.ensure(Na * 4));
+  HIPCHK(e->offs.ensure((Na + 1) * 8));
+
+  Scalars* sc = e->d_scalars.as<Scalars>();
+  Columns c;
+  c.ts = e->c_ts.as<int64_t>(); c.dur = e->c_dur.as<int64_t>(); c.corr = e->c_corr.as<uint64_t>();
+  c.dev = e->c_dev.as<int64_t>(); c.res = e->c_res.as<int64_t>(); c.meta = e->c_meta.as<uint32_t>();
+  c.ext = e->c_ext.as<int32_t>();
+  const ktj_generic_rec* g_recs = static_cast<const ktj_generic_rec*>(e->generic.ptr());
+  const ktj_runtime_rec* r_recs = static_cast<const ktj_runtime_rec*>(e->runtime.ptr());
+  const ktj_device_rec* d_recs = static_cast<const ktj_device_rec*>(e->devrows.ptr());
+  const ktj_extcorr_rec* x_recs = static_cast<const ktj_extcorr_rec*>(e->extcorr.ptr());
+
+  HIPCHK(hipEventRecord(e->ev[EV_START], st));
+  HIPCHK(init_scalars(sc, st));
+
+  /* ---- stage 0: dictionary ---- */
+  EmitCtx ctx;
+  ctx.dict.name_blob = e->d_name_blob.as<char>(); ctx.dict.name_off = e->d_name_off.as<uint64_t>();
+  ctx.dict.arg_blob = e->d_arg_blob.as<char>(); ctx.dict.arg_off = e->d_arg_off.as<uint64_t>();
+  ctx.dict.flags = e->d_sflags.as<uint32_t>(); ctx.dict.n = ns;
+  ctx.fields = e->d_fields.as<ktj_field>(); ctx.schemas = e->d_schemas.as<ktj_schema_desc>();
+  ctx.n_schemas = (uint32_t)e->schemas.size();
+  ctx.args = e->args.buf.as<uint64_t>(); ctx.n_args = e->n_args;
+  ctx.base_time_ns = e->base_time_ns;
+  if (ns) {
+    HIPCHK(dict_measure(e->str_blob.buf.as<char>(), e->str_off.buf.as<uint64_t>(), ns, e->d_name_len.as<uint32_t>(),
+                        e->d_arg_len.as<uint32_t>(), e->d_sflags.as<uint32_t>(), st));
+    HIPCHK(scan_u32_to_u64(e->d_name_len.as<uint32_t>(), e->d_name_off.as<uint64_t>(), ns, e->scan_tmp.as<uint64_t>(), st));
+    HIPCHK(scan_u32_to_u64(e->d_arg_len.as<uint32_t>(), e->d_arg_off.as<uint64_t>(), ns, e->scan_tmp.as<uint64_t>(), st));
+    HIPCHK(dict_write(e->str_blob.buf.as<char>(), e->str_off.buf.as<uint64_t>(), ns, e->d_name_off.as<uint64_t>(),
+                      e->d_arg_off.as<uint64_t>(), e->d_sflags.as<uint32_t>(), e->d_name_blob.as<char>(),
+                      e->d_arg_blob.as<char>(), st));
+  }
+  HIPCHK(hipEventRecord(e->ev[EV_DICT], st));
+
+  /* ---- stage 1: decode ---- */
+  HIPCHK(decode_generic(g_recs, ng, c, 0, st));
+  HIPCHK(decode_runtime(r_recs, nr, c, ng, st));
+  HIPCHK(decode_device(d_recs, nd, c, ng + nr, st));
+  HIPCHK(hipEventRecord(e->ev[EV_DECODE], st));
+
+  /* ---- stage 2a: clock + window ---- */
+  ClockDev clk;
+  clk.t0_approx = e->clock.t0_approx; clk.t0 = e->clock.t0;
+  memcpy(&clk.scale_bits, &e->clock.scale, 8);
+  clk.async_offset = e->clock.async_offset; clk.runtime_mode = e->clock.runtime_mode; clk.device_mode = e->clock.device_mode;
+  HIPCHK(convert_rows(c, ng, nr, nd, clk, e->win_start, e->win_end, sc, st));
+  HIPCHK(hipEventRecord(e->ev[EV_CONVERT], st));
+
+  /* ---- stage 2b: joins ---- */
+  Table t_ext{e->t_ext_k.as<uint64_t>(), e->t_ext_v.as<uint32_t>(), nullptr, cap_ext - 1};
+  Table t_cpu{e->t_cpu_k.as<uint64_t>(), nullptr, nullptr, cap_cpu - 1};
+  Table t_id{e->t_id_k.as<uint64_t>(), e->t_id_v0.as<uint32_t>(), e->t_id_v1.as<uint32_t>(), cap_id - 1};
+  Table t_nr{e->t_nr_k.as<uint64_t>(), e->t_nr_v0.as<uint32_t>(), e->t_nr_v1.as<uint32_t>(), cap_nr - 1};
+  HIPCHK(fill_u64(t_ext.keys, KTJ_EMPTY_KEY, cap_ext + 1ull, st)); HIPCHK(fill_u32(t_ext.v0, 0, cap_ext + 1ull, st));
+  HIPCHK(fill_u64(t_cpu.keys, KTJ_EMPTY_KEY, cap_cpu + 1ull, st));
+  HIPCHK(fill_u64(t_id.keys, KTJ_EMPTY_KEY, cap_id + 1ull, st)); HIPCHK(fill_u32(t_id.v0, 0, cap_id + 1ull, st));
+  HIPCHK(fill_u32(t_id.v1, 0xFFFFFFFFu, cap_id + 1ull, st));
+  HIPCHK(fill_u64(t_nr.keys, KTJ_EMPTY_KEY, cap_nr + 1ull, st)); HIPCHK(fill_u32(t_nr.v0, 0, cap_nr + 1ull, st));
+  HIPCHK(fill_u32(t_nr.v1, 0, cap_nr + 1ull, st));
+  StreamTables stt{e->q_keys.as<uint64_t>(), e->q_stream.as<uint64_t>(), e->q_amb.as<uint32_t>(), e->dn_hash.as<uint64_t>(),
+                   e->dn_first.as<uint32_t>(), e->dn_dev.as<int32_t>(), e->dn_key.as<uint64_t>(), e->dn_rank.as<uint32_t>()};
+  HIPCHK(fill_u64(stt.q_keys, KTJ_EMPTY_KEY, KTJ_QUEUE_CAP + 1ull, st)); HIPCHK(fill_u64(stt.q_stream, 0, KTJ_QUEUE_CAP + 1ull, st));
+  HIPCHK(fill_u32(stt.q_amb, 0, KTJ_QUEUE_CAP + 1ull, st));
+  HIPCHK(fill_u64(stt.d_hash, KTJ_EMPTY_KEY, KTJ_DENSE_CAP + 1ull, st)); HIPCHK(fill_u32(stt.d_first, 0xFFFFFFFFu, KTJ_DENSE_CAP + 1ull, st));
+  HIPCHK(fill_u32(stt.d_rank, 0, KTJ_DENSE_CAP + 1ull, st));
+  HIPCHK(build_extcorr(x_recs, nx, t_ext, sc, st));
+  HIPCHK(build_cpu_ids(g_recs, ng, t_cpu, sc, st));
+  HIPCHK(build_runtime(r_recs, nr, c, ng, t_id, t_nr, sc, st));
+  HIPCHK(insert_device_first(d_recs, nd, c, ng + nr, t_id, sc, st));
+  HIPCHK(probe_external(c, ng, nr + nd, x_recs, t_ext, t_cpu, sc, st));
+  HIPCHK(count_out_of_order(c, ng, nr, nd, t_id, sc, st));
+  HIPCHK(backfill_streams(d_recs, nd, r_recs, c, ng + nr, t_id, stt, sc, st));
+  HIPCHK(hipEventRecord(e->ev[EV_JOIN], st));
+
+  /* ---- stage 3: canonical order ---- */
+  SortSets sets{e->s_dev_k.as<uint64_t>(), e->s_dev_r.as<uint32_t>(), e->s_res_k.as<uint64_t>(), e->s_res_r.as<uint32_t>()};
+  HIPCHK(fill_u64(sets.dev_keys, KTJ_EMPTY_KEY, KTJ_SET_CAP + 1ull, st));
+  HIPCHK(fill_u64(sets.res_keys, KTJ_EMPTY_KEY, KTJ_SET_CAP + 1ull, st));
+  HIPCHK(collect_distinct(c, N, sets, sc, st));
+  HIPCHK(rank_distinct(sets, sc, st));
+  HIPCHK(hipEventRecord(e->ev[EV_SORT_A], st));
+  HIPCHK(hipMemcpyAsync(&e->scalars, sc, sizeof(Scalars), hipMemcpyDeviceToHost, st));
+  HIPCHK(hipStreamSynchronize(st));
+  if (e->scalars.error) {
+    e->last_error = "device-side limit hit before sort, error bits " + std::to_string(e->scalars.error);
+    return KTJ_ERR_LIMIT;
+  }
+  uint32_t ts_bits = 0, res_bits = 0, key_bits = 0;
+  if (e->scalars.n_valid) {
+    ts_bits = (uint32_t)bits_for(e->scalars.ts_max_biased - e->scalars.ts_min_biased);
+    res_bits = (uint32_t)bits_for(e->scalars.n_res_ranks ? e->scalars.n_res_ranks - 1 : 0);
+    const uint32_t dev_bits = (uint32_t)bits_for(e->scalars.n_dev_ranks ? e->scalars.n_dev_ranks - 1 : 0);
+    key_bits = ts_bits + res_bits + dev_bits;
+    if (key_bits > 62) {
+      e->last_error = "sort key needs " + std::to_string(key_bits) + " bits (timestamp span too wide)";
+      return KTJ_ERR_LIMIT;
+    }
+  }
+  HIPCHK(hipEventRecord(e->ev[EV_SORT_B], st));
+  HIPCHK(make_keys(c, N, sets, sc, ts_bits, res_bits, key_bits, e->keys_a.as<uint64_t>(), e->vals_a.as<uint32_t>(), st));
+  HIPCHK(radix_sort(e->keys_a.as<uint64_t>(), e->vals_a.as<uint32_t>(), e->keys_b.as<uint64_t>(), e->vals_b.as<uint32_t>(),
+                    N, key_bits + 1, e->hist.as<uint32_t>(), e->scan_tmp.as<uint64_t>(), &e->sorted_keys, &e->perm, st));
+  HIPCHK(hipEventRecord(e->ev[EV_SORT], st));
+
+  /* ---- stage 4a: joined rows + lengths ---- */
+  ApiTable api{e->d_cid_names.as<uint32_t>(), (uint32_t)e->cid_names.size(), e->d_flow_bits.as<uint32_t>(), e->malloc_cid};
+  MatRow* mat = e->mat.as<MatRow>();
+  HIPCHK(mat_generic_rows(g_recs, ng, ctx, mat, e->len.as<uint32_t>(), sc, st));
+  HIPCHK(mat_runtime_rows(r_recs, nr, c, ng, api, ctx, mat, e->len.as<uint32_t>(), sc, st));
+  HIPCHK(mat_device_rows(d_recs, nd, c, ng + nr, r_recs, t_nr, ctx, mat, e->len.as<uint32_t>(), sc, st));
+  HIPCHK(gather_len(e->perm, e->len.as<uint32_t>(), N, e->len_sorted.as<uint32_t>(), st));
+  HIPCHK(hipEventRecord(e->ev[EV_SIZE], st));
+
+  /* ---- scan ---- */
+  HIPCHK(scan_u32_to_u64(e->len_sorted.as<uint32_t>(), e->offs.as<uint64_t>(), N, e->scan_tmp.as<uint64_t>(), st));
+  HIPCHK(hipEventRecord(e->ev[EV_SCAN], st));
+  uint64_t act_bytes = 0;
+  HIPCHK(hipMemcpyAsync(&act_bytes, e->offs.as<uint64_t>() + N, 8, hipMemcpyDeviceToHost, st));
+  HIPCHK(hipMemcpyAsync(&e->scalars, sc, sizeof(Scalars), hipMemcpyDeviceToHost, st));
+  HIPCHK(hipStreamSynchronize(st));
+  if (e->scalars.error) {
+    e->last_error = "device-side limit hit, error bits " + std::to_string(e->scalars.error);
+    return KTJ_ERR_LIMIT;
+  }
+
+  /* ---- emit ---- */
+  std::string prefix = e->txt_header + e->txt_dev + e->txt_res + e->txt_ovh;
+  std::string suffix = e->txt_span;
+  append_trace_end(suffix, end_time_ns, e->base_time_ns, e->out_path);
+  e->prefix_len = prefix.size();
+  e->act_bytes = act_bytes;
+  e->total_bytes = prefix.size() + act_bytes + suffix.size();
+  HIPCHK(e->out.ensure(e->total_bytes + 64));
+  const size_t small = prefix.size() + suffix.size();
+  if (small > e->pinned_small_cap) {
+    if (e->pinned_small) HIPCHK(hipHostFree(e->pinned_small));
+    e->pinned_small = nullptr;
+    HIPCHK(hipHostMalloc(&e->pinned_small, small * 2 + 4096, hipHostMallocDefault));
+    e->pinned_small_cap = small * 2 + 4096;
+  }
+  memcpy(e->pinned_small, prefix.data(), prefix.size());
+  memcpy(static_cast<char*>(e->pinned_small) + prefix.size(), suffix.data(), suffix.size());
+  HIPCHK(hipMemcpyAsync(e->out.p, e->pinned_small, prefix.size(), hipMemcpyHostToDevice, st));
+  HIPCHK(hipMemcpyAsync(e->out.as<char>() + prefix.size() + act_bytes, static_cast<char*>(e->pinned_small) + prefix.size(),
+                        suffix.size(), hipMemcpyHostToDevice, st));
+  HIPCHK(hipEventRecord(e->ev[EV_EMIT_START], st));
+  HIPCHK(emit(mat, e->perm, e->offs.as<uint64_t>(), N, ctx, e->out.as<char>(), e->prefix_len, act_bytes, st));
+  HIPCHK(hipEventRecord(e->ev[EV_EMIT], st));
+  HIPCHK(hipStreamSynchronize(st));
+
+  /* ---- statistics ---- */
+  ktj_stats& s = e->stats;
+  memset(&s, 0, sizeof s);
+  s.n_generic = ng; s.n_runtime = nr; s.n_device = nd; s.n_extcorr = nx;
+  s.n_emitted = e->scalars.n_valid;
+  s.out_of_range_events = e->scalars.out_of_range;
+  s.gpu_and_cpu_op_out_of_order = e->scalars.out_of_order;
+  s.n_flow_events = e->scalars.n_flow;
+  s.n_linked = e->scalars.n_linked;
+  s.n_blank_names = e->scalars.n_blank_names;
+  s.output_bytes = e->total_bytes;
+  s.activity_bytes = act_bytes;
+  /* stage time = elapsed between the events that bracket it; the two host read-backs (after the
+   * distinct-value ranking and after the scan) are excluded from the per-stage figures but are
+   * part of KTJ_STAGE_TOTAL_GPU */
+  struct { int stage, from, to; } spans[] = {
+      {KTJ_STAGE_DICT, EV_START, EV_DICT},       {KTJ_STAGE_DECODE, EV_DICT, EV_DECODE},
+      {KTJ_STAGE_CONVERT, EV_DECODE, EV_CONVERT}, {KTJ_STAGE_JOIN, EV_CONVERT, EV_JOIN},
+      {KTJ_STAGE_SORT, EV_JOIN, EV_SORT_A},      {KTJ_STAGE_SORT, EV_SORT_B, EV_SORT},
+      {KTJ_STAGE_SIZE, EV_SORT, EV_SIZE},        {KTJ_STAGE_SCAN, EV_SIZE, EV_SCAN},
+      {KTJ_STAGE_EMIT, EV_EMIT_START, EV_EMIT}};
+  for (const auto& sp : spans) {
+    float ms = 0;
+    HIPCHK(hipEventElapsedTime(&ms, e->ev[sp.from], e->ev[sp.to]));
+    s.stage_ms[sp.stage] += ms;
+  }
+  {
+    float ms = 0;
+    HIPCHK(hipEventElapsedTime(&ms, e->ev[EV_START], e->ev[EV_EMIT]));
+    s.stage_ms[KTJ_STAGE_TOTAL_GPU] = ms;
+  }
+  const uint64_t raw_in = ng * sizeof(ktj_generic_rec) + nr * sizeof(ktj_runtime_rec) + nd * sizeof(ktj_device_rec);
+  s.stage_bytes[KTJ_STAGE_DICT] = e->blob_bytes * 3;
+  s.stage_bytes[KTJ_STAGE_DECODE] = raw_in + N * 48;
+  s.stage_bytes[KTJ_STAGE_CONVERT] = (nr + nd) * 32;
+  s.stage_bytes[KTJ_STAGE_JOIN] = nx * 12 + ng * 12 + nr * 12 + (nr + nd) * 12 * 2;
+  s.stage_bytes[KTJ_STAGE_SORT] = N * 56;
+  s.stage_bytes[KTJ_STAGE_SIZE] = raw_in + N * 48 + N * (sizeof(MatRow) + 4);
+  s.stage_bytes[KTJ_STAGE_SCAN] = N * 12;
+  s.stage_bytes[KTJ_STAGE_EMIT] = e->scalars.n_valid * (sizeof(MatRow) + 12) + act_bytes;
+  e->processed = true;
+  return KTJ_OK;
+}
+
+int ktj_output_device(ktj_engine* e, const void** device_ptr, uint64_t* n_bytes) {
+  if (!e || !device_ptr || !n_bytes) return KTJ_ERR_ARG;
+  if (!e->processed) return KTJ_ERR_STATE;
+  *device_ptr = e->out.p;
+  *n_bytes = e->total_bytes;
+  return KTJ_OK;
+}
+
+int ktj_output_host(ktj_engine* e, const char** host_ptr, uint64_t* n_bytes) {
+  if (!e || !host_ptr || !n_bytes) return KTJ_ERR_ARG;
+  if (!e->processed) return KTJ_ERR_STATE;
+  HIPCHK(hipSetDevice(e->device));
+  if (!e->host_copy_valid) {
+    if (e->total_bytes > e->pinned_out_cap) {
+      if (e->pinned_out) HIPCHK(hipHostFree(e->pinned_out));
+      e->pinned_out = nullptr; e->pinned_out_cap = 0;
+      void* p = nullptr;
+      HIPCHK(hipHostMalloc(&p, e->total_bytes + 4096, hipHostMallocDefault));
+      e->pinned_out = static_cast<char*>(p);
+      e->pinned_out_cap = e->total_bytes + 4096;
+    }
+    HIPCHK(hipEventRecord(e->ev_d2h[0], e->stream));
+    HIPCHK(hipMemcpyAsync(e->pinned_out, e->out.p, e->total_bytes, hipMemcpyDeviceToHost, e->stream));
+    HIPCHK(hipEventRecord(e->ev_d2h[1], e->stream));
+    HIPCHK(hipStreamSynchronize(e->stream));
+    float ms = 0;
+    HIPCHK(hipEventElapsedTime(&ms, e->ev_d2h[0], e->ev_d2h[1]));
+    e->stats.stage_ms[KTJ_STAGE_D2H] = ms;
+    e->stats.stage_bytes[KTJ_STAGE_D2H] = e->total_bytes;
+    e->host_copy_valid = true;
+  }
+  *host_ptr = e->pinned_out;
+  *n_bytes = e->total_bytes;
+  return KTJ_OK;
+}
+
+int ktj_finalize(ktj_engine* e, int64_t end_time_ns, uint64_t* bytes_written) {
+  if (!e) return KTJ_ERR_ARG;
+  if (bytes_written) *bytes_written = 0;
+  if (e->bad_sink) { /* output_json.cpp:1067-1070 */
+    e->last_error = "Failed to write to log file!";
+    return KTJ_ERR_IO;
+  }
+  int rc = ktj_process(e, end_time_ns);
+  if (rc != KTJ_OK) return rc;
+  if (e->flags & KTJ_CREATE_NO_FILE) {
+    if (bytes_written) *bytes_written = e->total_bytes;
+    return KTJ_OK;
+  }
+  const char* host = nullptr;
+  uint64_t n = 0;
+  rc = ktj_output_host(e, &host, &n);
+  if (rc != KTJ_OK) return rc;
+  struct timespec t0, t1;
+  clock_gettime(CLOCK_MONOTONIC, &t0);
+  if (!e->sink) return KTJ_ERR_STATE;
+  const size_t w = fwrite(host, 1, n, e->sink);
+  const int crc = fclose(e->sink);
+  e->sink = nullptr;
+  if (w != n || crc != 0) { e->last_error = "short write to " + e->tmp_path; return KTJ_ERR_IO; }
+  remove(e->out_path.c_str()); /* output_json.cpp:1100-1107 */
+  if (rename(e->tmp_path.c_str(), e->out_path.c_str()) != 0) {
+    e->last_error = "Failed to rename " + e->tmp_path + " to " + e->out_path + ": " + strerror(errno);
+    return KTJ_ERR_IO;
+  }
+  clock_gettime(CLOCK_MONOTONIC, &t1);
+  e->stats.stage_ms[KTJ_STAGE_FILE] = (float)((t1.tv_sec - t0.tv_sec) * 1e3 + (t1.tv_nsec - t0.tv_nsec) * 1e-6);
+  e->stats.stage_bytes[KTJ_STAGE_FILE] = n;
+  if (bytes_written) *bytes_written = n;
+  return KTJ_OK;
+}
+
+int ktj_get_stats(ktj_engine* e, ktj_stats* out) {
+  if (!e || !out) return KTJ_ERR_ARG;
+  *out = e->stats;
+  return KTJ_OK;
+}
+
+int ktj_debug_fetch(ktj_engine* e, int what, void* dst, uint64_t cap, uint64_t* n_bytes) {
+  if (!e || !n_bytes) return KTJ_ERR_ARG;
+  if (!e->processed) return KTJ_ERR_STATE;
+  const void* src = nullptr;
+  uint64_t n = 0;
+  const uint64_t N = e->N;
+  switch (what) {
+    case KTJ_DBG_COL_TS: src = e->c_ts.p; n = N * 8; break;
+    case KTJ_DBG_COL_DUR: src = e->c_dur.p; n = N * 8; break;
+    case KTJ_DBG_COL_DEV: src = e->c_dev.p; n = N * 8; break;
+    case KTJ_DBG_COL_RES: src = e->c_res.p; n = N * 8; break;
+    case KTJ_DBG_COL_META: src = e->c_meta.p; n = N * 4; break;
+    case KTJ_DBG_COL_EXT: src = e->c_ext.p; n = N * 4; break;
+    case KTJ_DBG_PERM: src = e->perm; n = N * 4; break;
+    case KTJ_DBG_LEN: src = e->len_sorted.p; n = N * 4; break;
+    case KTJ_DBG_OFFS: src = e->offs.p; n = (N + 1) * 8; break;
+    case KTJ_DBG_MAT: src = e->mat.p; n = N * sizeof(MatRow); break;
+    case KTJ_DBG_SORT_KEYS: src = e->sorted_keys; n = N * 8; break;
+    case KTJ_DBG_NAME_VIEW: src = e->d_name_blob.p; n = e->blob_bytes * 2 + 8ull * e->n_strings; break;
+    case KTJ_DBG_NAME_OFF: src = e->d_name_off.p; n = (e->n_strings + 1) * 8; break;
+    case KTJ_DBG_ARG_VIEW: src = e->d_arg_blob.p; n = e->blob_bytes; break;
+    case KTJ_DBG_ARG_OFF: src = e->d_arg_off.p; n = (e->n_strings + 1) * 8; break;
+    default: return KTJ_ERR_ARG;
+  }
+  *n_bytes = n;
+  if (dst && src && n) {
+    HIPCHK(hipSetDevice(e->device));
+    HIPCHK(hipMemcpy(dst, src, n < cap ? n : cap, hipMemcpyDeviceToHost));
+  }
+  return KTJ_OK;
+}
+
+}  // extern "C"

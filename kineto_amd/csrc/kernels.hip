@@ -1,0 +1,1075 @@
+/*
+ * kernels.hip — HIP kernels of the trace post-processing engine, written for gfx950 (CDNA4):
+ * 64-wide wavefronts, ballot/popcount based ranking, LDS-staged tiles, 16-byte lanes.
+ *
+ * Nothing here is a dense contraction, so there is no MFMA; every kernel is bound by HBM (or,
+ * for the hash joins, by random 64-byte sector access).  Stage by stage:
+ *   0  dictionary   strings → name view (logger's name pipeline) and arg view (sanitised)
+ *   1  decode       packed activity records → columns, through LDS so that global reads are
+ *                   lane-consecutive 16-byte loads
+ *   2  convert/join clock model, window filter, external-correlation join, runtime↔device join,
+ *                   stream back-fill with dense per-device stream indices
+ *   3  order        dense ranks of (device, resource), 64-bit composite keys, stable LSD radix sort
+ *   4  size/emit    exact byte length per activity, device-wide exclusive scan, output-partitioned
+ *                   tiles formatted in LDS and flushed with aligned 16-byte stores
+ */
+#include <hip/hip_runtime.h>
+
+#include "gpu_stages.h"
+
+namespace ktj {
+namespace gpu {
+
+#define KTJ_NOSLOT 0xFFFFFFFFu
+#define KTJ_BLOCK 256
+
+/* ------------------------------------------------------------------------------------------ */
+/* helpers                                                                                      */
+/* ------------------------------------------------------------------------------------------ */
+__device__ __forceinline__ uint64_t hash64(uint64_t x) {
+  x ^= x >> 33; x *= 0xff51afd7ed558ccdULL; x ^= x >> 33; x *= 0xc4ceb9fe1a85ec53ULL; x ^= x >> 33;
+  return x;
+}
+__device__ __forceinline__ uint32_t lane_id() { return threadIdx.x & 63u; }
+__device__ __forceinline__ uint64_t lanemask_lt() { return (1ULL << lane_id()) - 1ULL; }
+
+/* Returns the slot holding `key`, inserting it if absent; KTJ_NOSLOT when the table is full.
+ * The probe sequence is bounded by the table size, so every lane leaves the loop. */
+__device__ uint32_t table_insert(uint64_t* keys, uint32_t mask, uint64_t key) {
+  if (key == KTJ_EMPTY_KEY) { keys[mask + 1u] = 0; return mask + 1u; }
+  uint32_t slot = (uint32_t)hash64(key) & mask;
+  for (uint32_t probe = 0; probe <= mask; ++probe) {
+    uint64_t cur = keys[slot];
+    if (cur == key) return slot;
+    if (cur == KTJ_EMPTY_KEY) {
+      unsigned long long prev = atomicCAS((unsigned long long*)&keys[slot], (unsigned long long)KTJ_EMPTY_KEY,
+                                          (unsigned long long)key);
+      if (prev == KTJ_EMPTY_KEY || prev == key) return slot;
+    }
+    slot = (slot + 1u) & mask;
+  }
+  return KTJ_NOSLOT;
+}
+__device__ uint32_t table_find(const uint64_t* keys, uint32_t mask, uint64_t key) {
+  if (key == KTJ_EMPTY_KEY) return keys[mask + 1u] == 0 ? mask + 1u : KTJ_NOSLOT;
+  uint32_t slot = (uint32_t)hash64(key) & mask;
+  for (uint32_t probe = 0; probe <= mask; ++probe) {
+    uint64_t cur = keys[slot];
+    if (cur == key) return slot;
+    if (cur == KTJ_EMPTY_KEY) return KTJ_NOSLOT;
+    slot = (slot + 1u) & mask;
+  }
+  return KTJ_NOSLOT;
+}
+
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+/* one atomicAdd per wave */
+__device__ __forceinline__ void count_flag(unsigned long long* counter, bool flag) {
+  const uint64_t m = __ballot(flag ? 1 : 0);
+  if (m != 0 && lane_id() == (uint32_t)(__ffsll((long long)m) - 1)) atomicAdd(counter, (unsigned long long)__popcll(m));
+}
+
+__global__ void k_fill_u64(uint64_t* p, uint64_t v, uint64_t n) {
+  uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+__global__ void k_fill_u32(uint32_t* p, uint32_t v, uint64_t n) {
+  uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+__global__ void k_init_scalars(Scalars* s) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    s->ts_min_biased = ~0ULL; s->ts_max_biased = 0;
+    s->out_of_range = 0; s->out_of_order = 0; s->n_flow = 0; s->n_linked = 0; s->n_blank_names = 0; s->n_valid = 0;
+    s->error = 0; s->have_stream_src = 0; s->n_dev_ranks = 0; s->n_res_ranks = 0; s->n_dense = 0; s->pad = 0;
+  }
+}
+
+static inline unsigned grid_for(uint64_t n, unsigned per_block) { return (unsigned)((n + per_block - 1) / per_block); }
+#define KTJ_LAUNCH_CHECK() hipGetLastError()
+
+hipError_t fill_u64(uint64_t* p, uint64_t v, uint64_t n, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_fill_u64, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, p, v, n);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t fill_u32(uint32_t* p, uint32_t v, uint64_t n, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_fill_u32, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, p, v, n);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t init_scalars(Scalars* s, hipStream_t st) {
+  hipLaunchKernelGGL(k_init_scalars, dim3(1), dim3(64), 0, st, s);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* exclusive scan: per-block sums → scan of the sums (one block) → per-block scan               */
+/* ------------------------------------------------------------------------------------------ */
+#define SCAN_ITEMS 8
+#define SCAN_TILE (KTJ_BLOCK * SCAN_ITEMS)
+
+__device__ __forceinline__ uint64_t block_exclusive_scan_u64(uint64_t v, uint64_t* lds_wave /* 4 */, uint64_t* total) {
+  /* inclusive scan inside the wave */
+  unsigned long long x = v;
+  for (int o = 1; o < 64; o <<= 1) {
+    const unsigned long long y = __shfl_up(x, (unsigned)o);
+    if ((int)lane_id() >= o) x += y;
+  }
+  const uint32_t w = threadIdx.x >> 6;
+  if (lane_id() == 63) lds_wave[w] = x;
+  __syncthreads();
+  uint64_t base = 0, tot = 0;
+  for (uint32_t k = 0; k < (KTJ_BLOCK >> 6); ++k) {
+    const uint64_t s = lds_wave[k];
+    if (k < w) base += s;
+    tot += s;
+  }
+  __syncthreads();
+  *total = tot;
+  return base + x - v;
+}
+
+__global__ void k_scan_sums(const uint32_t* in, uint64_t n, uint64_t* sums) {
+  __shared__ uint64_t lds_wave[KTJ_BLOCK >> 6];
+  const uint64_t base = (uint64_t)blockIdx.x * SCAN_TILE + (uint64_t)threadIdx.x * SCAN_ITEMS;
+  uint64_t s = 0;
+  for (int k = 0; k < SCAN_ITEMS; ++k) if (base + k < n) s += in[base + k];
+  uint64_t tot;
+  block_exclusive_scan_u64(s, lds_wave, &tot);
+  if (threadIdx.x == 0) sums[blockIdx.x] = tot;
+}
+/* one block: sums[0..m) → exclusive prefix in place, grand total → sums[m] */
+__global__ void k_scan_of_sums(uint64_t* sums, uint64_t m) {
+  __shared__ uint64_t lds_wave[KTJ_BLOCK >> 6];
+  uint64_t carry = 0;
+  for (uint64_t base = 0; base < m; base += KTJ_BLOCK) {
+    const uint64_t i = base + threadIdx.x;
+    const uint64_t v = i < m ? sums[i] : 0;
+    uint64_t tot;
+    const uint64_t ex = block_exclusive_scan_u64(v, lds_wave, &tot);
+    if (i < m) sums[i] = carry + ex;
+    carry += tot;
+  }
+  if (threadIdx.x == 0) sums[m] = carry;
+}
+template <typename OutT>
+__global__ void k_scan_final(const uint32_t* in, uint64_t n, const uint64_t* sums, uint64_t m, OutT* out,
+                             bool write_total) {
+  __shared__ uint64_t lds_wave[KTJ_BLOCK >> 6];
+  const uint64_t base = (uint64_t)blockIdx.x * SCAN_TILE + (uint64_t)threadIdx.x * SCAN_ITEMS;
+  uint32_t v[SCAN_ITEMS];
+  uint64_t s = 0;
+  for (int k = 0; k < SCAN_ITEMS; ++k) { v[k] = base + k < n ? in[base + k] : 0u; s += v[k]; }
+  uint64_t tot;
+  uint64_t ex = block_exclusive_scan_u64(s, lds_wave, &tot) + sums[blockIdx.x];
+  for (int k = 0; k < SCAN_ITEMS; ++k) {
+    if (base + k < n) out[base + k] = (OutT)ex;
+    ex += v[k];
+  }
+  if (write_total && blockIdx.x == 0 && threadIdx.x == 0) out[n] = (OutT)sums[m];
+}
+
+uint64_t scan_tmp_elems(uint64_t n) { return (n + SCAN_TILE - 1) / SCAN_TILE + 2; }
+
+hipError_t scan_u32_to_u64(const uint32_t* in, uint64_t* out, uint64_t n, uint64_t* tmp, hipStream_t st) {
+  const uint64_t m = (n + SCAN_TILE - 1) / SCAN_TILE;
+  if (m > 0) hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st, in, n, tmp);
+  hipLaunchKernelGGL(k_scan_of_sums, dim3(1), dim3(KTJ_BLOCK), 0, st, tmp, m);
+  if (m > 0)
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(k_scan_final<uint64_t>), dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st, in, n,
+                       (const uint64_t*)tmp, m, out, true);
+  else
+    hipLaunchKernelGGL(k_fill_u64, dim3(1), dim3(64), 0, st, out, (uint64_t)0, (uint64_t)1);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t scan_u32_inplace(uint32_t* data, uint64_t n, uint64_t* tmp, hipStream_t st) {
+  const uint64_t m = (n + SCAN_TILE - 1) / SCAN_TILE;
+  if (m == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st, (const uint32_t*)data, n, tmp);
+  hipLaunchKernelGGL(k_scan_of_sums, dim3(1), dim3(KTJ_BLOCK), 0, st, tmp, m);
+  /* every block reads its tile completely before writing it, and tiles do not overlap */
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(k_scan_final<uint32_t>), dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st,
+                     (const uint32_t*)data, n, (const uint64_t*)tmp, m, data, false);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* stage 0: dictionary.  One wavefront per string.                                              */
+/*   arg view  = sanitizeStrForJSON            (libkineto/src/output_json.cpp:72-78)            */
+/*   name view = "kernel"→"Kernel", sanitize, non-printable → "unknown", quote escaping         */
+/*                                             (output_json.cpp:946-949, 86-112)                */
+/* ------------------------------------------------------------------------------------------ */
+#define KTJ_SF_NAME_KERNEL 4u
+
+__global__ void k_dict_measure(const char* blob, const uint64_t* off, uint32_t n, uint32_t* name_len,
+                               uint32_t* arg_len, uint32_t* flags) {
+  const uint32_t id = blockIdx.x * (KTJ_BLOCK >> 6) + (threadIdx.x >> 6);
+  if (id >= n) return;
+  const char* p = blob + off[id];
+  const uint64_t len = off[id + 1] - off[id];
+  uint32_t nl = 0, q = 0, bad = 0, nonblank = 0;
+  for (uint64_t k = lane_id(); k < len; k += 64) {
+    const unsigned char c = (unsigned char)p[k];
+    if (c == '\n') { ++nl; continue; }
+    if (c == '"') ++q;
+    if (c < 0x20 || c > 0x7e) ++bad;
+    if (!(c == ' ' || c == '\t' || c == '\v' || c == '\f' || c == '\r')) ++nonblank;
+  }
+  nl = wave_sum_u32(nl); q = wave_sum_u32(q); bad = wave_sum_u32(bad); nonblank = wave_sum_u32(nonblank);
+  if (lane_id() == 0) {
+    const bool is_kernel = len == 6 && p[0] == 'k' && p[1] == 'e' && p[2] == 'r' && p[3] == 'n' && p[4] == 'e' && p[5] == 'l';
+    uint32_t f = 0;
+    uint32_t nlen;
+    if (is_kernel) { f |= KTJ_SF_NAME_KERNEL; nlen = 6; }
+    else if (bad) { f |= KTJ_SF_NAME_UNKNOWN; nlen = 7; }
+    else nlen = (uint32_t)len - nl + q;
+    if (nonblank == 0) f |= KTJ_SF_ARG_BLANK;
+    name_len[id] = nlen;
+    arg_len[id] = (uint32_t)len - nl;
+    flags[id] = f;
+  }
+}
+
+__global__ void k_dict_write(const char* blob, const uint64_t* off, uint32_t n, const uint64_t* name_off,
+                             const uint64_t* arg_off, const uint32_t* flags, char* name_blob, char* arg_blob) {
+  const uint32_t id = blockIdx.x * (KTJ_BLOCK >> 6) + (threadIdx.x >> 6);
+  if (id >= n) return;
+  const char* p = blob + off[id];
+  const uint64_t len = off[id + 1] - off[id];
+  const uint32_t f = flags[id];
+  char* an = arg_blob + arg_off[id];
+  char* nn = name_blob + name_off[id];
+  const bool literal_name = (f & (KTJ_SF_NAME_KERNEL | KTJ_SF_NAME_UNKNOWN)) != 0;
+  if (literal_name) {
+    const char* lit = (f & KTJ_SF_NAME_KERNEL) ? "Kernel" : "unknown";
+    const uint32_t ll = (f & KTJ_SF_NAME_KERNEL) ? 6u : 7u;
+    if (lane_id() < ll) nn[lane_id()] = lit[lane_id()];
+  }
+  uint64_t aw = 0, nw = 0; /* bytes written so far (wave-uniform) */
+  const uint64_t lt = lanemask_lt();
+  for (uint64_t base = 0; base < len; base += 64) {
+    const uint64_t k = base + lane_id();
+    const bool in = k < len;
+    unsigned char c = in ? (unsigned char)p[k] : 0;
+    const bool keep = in && c != '\n';
+    if (c == '\\') c = '/';
+    const bool isq = keep && c == '"';
+    const uint64_t km = __ballot(keep ? 1 : 0);
+    const uint64_t qm = __ballot(isq ? 1 : 0);
+    const uint32_t kpos = (uint32_t)__popcll(km & lt);
+    if (keep) {
+      an[aw + kpos] = (char)c;
+      if (!literal_name) {
+        const uint64_t np = nw + kpos + (uint32_t)__popcll(qm & lt);
+        if (isq) { nn[np] = '\\'; nn[np + 1] = '"'; }
+        else nn[np] = (char)c;
+      }
+    }
+    aw += (uint32_t)__popcll(km);
+    nw += (uint32_t)__popcll(km) + (uint32_t)__popcll(qm);
+  }
+}
+
+hipError_t dict_measure(const char* blob, const uint64_t* off, uint32_t n, uint32_t* name_len, uint32_t* arg_len,
+                        uint32_t* flags, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_dict_measure, dim3(grid_for(n, KTJ_BLOCK >> 6)), dim3(KTJ_BLOCK), 0, st, blob, off, n,
+                     name_len, arg_len, flags);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t dict_write(const char* blob, const uint64_t* off, uint32_t n, const uint64_t* name_off,
+                      const uint64_t* arg_off, const uint32_t* flags, char* name_blob, char* arg_blob, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_dict_write, dim3(grid_for(n, KTJ_BLOCK >> 6)), dim3(KTJ_BLOCK), 0, st, blob, off, n, name_off,
+                     arg_off, flags, name_blob, arg_blob);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* stage 1: decode.  A workgroup pulls 256 packed records into LDS with lane-consecutive 16-byte */
+/* loads (fully coalesced), then each lane unpacks its own record into the columns.              */
+/* ------------------------------------------------------------------------------------------ */
+template <typename Rec>
+__device__ __forceinline__ const Rec* stage_records(const Rec* recs, uint64_t n, uint4* stage, uint32_t* n_here) {
+  constexpr uint32_t U = sizeof(Rec) / 16;
+  const uint64_t base = (uint64_t)blockIdx.x * KTJ_BLOCK;
+  const uint32_t cnt = (uint32_t)((n - base) < KTJ_BLOCK ? (n - base) : KTJ_BLOCK);
+  const uint4* g = reinterpret_cast<const uint4*>(recs + base);
+  for (uint32_t i = threadIdx.x; i < cnt * U; i += KTJ_BLOCK) stage[i] = g[i];
+  __syncthreads();
+  *n_here = cnt;
+  return reinterpret_cast<const Rec*>(stage);
+}
+
+__global__ void k_decode_generic(const ktj_generic_rec* recs, uint64_t n, Columns c, uint64_t first) {
+  __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_generic_rec) / 16];
+  uint32_t cnt;
+  const ktj_generic_rec* l = stage_records(recs, n, stage, &cnt);
+  if (threadIdx.x >= cnt) return;
+  const ktj_generic_rec g = l[threadIdx.x];
+  const uint64_t a = first + (uint64_t)blockIdx.x * KTJ_BLOCK + threadIdx.x;
+  c.ts[a] = g.start_ns;
+  c.dur[a] = g.end_ns - g.start_ns;               /* GenericTraceActivity.h:65-67 */
+  c.corr[a] = (uint64_t)(int64_t)g.id;
+  c.dev[a] = g.device;
+  c.res[a] = g.resource;
+  c.meta[a] = KTJ_M_VALID | (KTJ_CLASS_GENERIC << KTJ_M_CLASS_SHIFT);
+  c.ext[a] = 0;
+}
+__global__ void k_decode_runtime(const ktj_runtime_rec* recs, uint64_t n, Columns c, uint64_t first) {
+  __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_runtime_rec) / 16];
+  uint32_t cnt;
+  const ktj_runtime_rec* l = stage_records(recs, n, stage, &cnt);
+  if (threadIdx.x >= cnt) return;
+  const ktj_runtime_rec* r = &l[threadIdx.x];
+  const uint64_t a = first + (uint64_t)blockIdx.x * KTJ_BLOCK + threadIdx.x;
+  c.ts[a] = (int64_t)r->begin;
+  c.dur[a] = (int64_t)r->end;
+  c.corr[a] = r->id;
+  c.dev[a] = (int64_t)r->pid;
+  c.res[a] = (int64_t)r->tid;
+  c.meta[a] = (KTJ_CLASS_RUNTIME << KTJ_M_CLASS_SHIFT);
+  c.ext[a] = 0;
+}
+__global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns c, uint64_t first) {
+  __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_device_rec) / 16];
+  uint32_t cnt;
+  const ktj_device_rec* l = stage_records(recs, n, stage, &cnt);
+  if (threadIdx.x >= cnt) return;
+  const ktj_device_rec* d = &l[threadIdx.x];
+  const uint64_t a = first + (uint64_t)blockIdx.x * KTJ_BLOCK + threadIdx.x;
+  const uint32_t dom = d->domain <= KTJ_DOM_MEMSET ? d->domain : KTJ_DOM_KERNEL_DISPATCH;
+  c.ts[a] = (int64_t)d->begin;
+  c.dur[a] = (int64_t)d->end;
+  c.corr[a] = d->id;
+  c.dev[a] = (int64_t)d->device;
+  c.res[a] = (int64_t)d->stream;
+  c.meta[a] = (KTJ_CLASS_DEVICE << KTJ_M_CLASS_SHIFT) | (dom << KTJ_M_KIND_SHIFT);
+  c.ext[a] = 0;
+}
+
+hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_decode_generic, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_decode_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_decode_device, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* stage 2a: clock conversion and window filter                                                 */
+/*   RocprofActivityApi.cpp:166-175, ApproximateClock.cpp:83-90, RocprofActivity.h:122-127,      */
+/*   GenericActivityProfiler.cpp:329-340                                                        */
+/* ------------------------------------------------------------------------------------------ */
+__global__ void k_convert(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, ClockDev clk,
+                          int64_t win_start, int64_t win_end, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  bool oor = false;
+  if (i < n_runtime + n_device) {
+    const uint64_t a = first_runtime + i;
+    uint64_t b = (uint64_t)c.ts[a], e = (uint64_t)c.dur[a];
+    uint32_t meta = c.meta[a];
+    int64_t ts, dur;
+    if (i < n_runtime) {
+      convert_range(clk, clk.runtime_mode, &b, &e);
+      ts = (int64_t)b;                 /* RocprofActivity.h:42-47 */
+      dur = (int64_t)(e - b);
+    } else {
+      convert_range(clk, clk.device_mode, &b, &e);
+      device_times((meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT, b, e, &ts, &dur);
+    }
+    oor = out_of_range(ts, dur, win_start, win_end);
+    if (!oor) meta |= KTJ_M_VALID;
+    c.ts[a] = ts;
+    c.dur[a] = dur;
+    c.meta[a] = meta;
+  }
+  count_flag(&sc->out_of_range, oor);
+}
+hipError_t convert_rows(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, ClockDev clk,
+                        int64_t win_start, int64_t win_end, Scalars* sc, hipStream_t st) {
+  const uint64_t n = n_runtime + n_device;
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_convert, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first_runtime, n_runtime,
+                     n_device, clk, win_start, win_end, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* stage 2b: joins.  "Last writer wins" of the reference's sequential map updates becomes        */
+/* atomicMax over the source row index; "first seen" becomes atomicMin over the arrival index.   */
+/* ------------------------------------------------------------------------------------------ */
+__device__ __forceinline__ void flag_error(Scalars* sc, unsigned bit) { atomicOr(&sc->error, bit); }
+
+/* cpuCorrelationMap_[correlation] = externalId: RocmActivityProfiler.cpp:135-148 */
+__global__ void k_build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table t, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t slot = table_insert(t.keys, t.mask, e[i].correlation);
+  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
+  atomicMax(&t.v0[slot], (uint32_t)i + 1u);
+}
+/* activityMap_[act->correlationId()] = act: GenericActivityProfiler.cpp:262 */
+__global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table t, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t slot = table_insert(t.keys, t.mask, (uint64_t)(int64_t)g[i].id);
+  if (slot == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+}
+/* by_id  : full correlation id → v0 = last runtime row (index+1) that carries a stream
+ *          (RocmStreamQueue.h:47-54), v1 = first arrival index seen for checkTimestampOrder
+ *          (GenericActivityProfiler.cpp:363-395)
+ * by_narrow: int-narrowed id → v0 = last in-range kernel row, v1 = last in-range copy/malloc row
+ *          (thread_local correlationToGrid/Block/Size, RocprofActivity_inl.h:28-30, 221-223, 245, 267) */
+__global__ void k_build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, Table by_id,
+                                Table by_narrow, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint64_t a = first_runtime + i;
+  const uint64_t id = r[i].id;
+  const uint32_t kind = r[i].kind;
+  const uint32_t slot = table_insert(by_id.keys, by_id.mask, id);
+  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
+  atomicMin(&by_id.v1[slot], (uint32_t)a);
+  const uint64_t stream = kind == KTJ_RT_KERNEL ? r[i].u.kernel.stream : (kind == KTJ_RT_COPY ? r[i].u.copy.stream : 0);
+  if (stream != 0) {
+    atomicMax(&by_id.v0[slot], (uint32_t)i + 1u);
+    if (sc->have_stream_src == 0) sc->have_stream_src = 1;
+  }
+  if ((c.meta[a] & KTJ_M_VALID) && (kind == KTJ_RT_KERNEL || kind == KTJ_RT_COPY || kind == KTJ_RT_MALLOC)) {
+    const uint32_t ps = table_insert(by_narrow.keys, by_narrow.mask, narrow_corr_key(id));
+    if (ps == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
+    if (kind == KTJ_RT_KERNEL) atomicMax(&by_narrow.v0[ps], (uint32_t)i + 1u);
+    else atomicMax(&by_narrow.v1[ps], (uint32_t)i + 1u);
+  }
+}
+__global__ void k_insert_device_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device,
+                                      Table by_id, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint64_t a = first_device + i;
+  if (!(c.meta[a] & KTJ_M_VALID)) return;
+  const uint32_t slot = table_insert(by_id.keys, by_id.mask, d[i].id);
+  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
+  if (by_id.v1[slot] > (uint32_t)a) atomicMin(&by_id.v1[slot], (uint32_t)a);
+}
+/* linkedActivity(): GenericActivityProfiler.cpp:397-408; "External id": output_json.cpp:871-874 */
+__global__ void k_probe_external(Columns c, uint64_t first, uint64_t n, const ktj_extcorr_rec* e, Table ext,
+                                 Table cpu, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  bool linked = false;
+  if (i < n) {
+    const uint64_t a = first + i;
+    int32_t x = 0;
+    const uint32_t s1 = table_find(ext.keys, ext.mask, narrow_corr_key(c.corr[a]));
+    if (s1 != KTJ_NOSLOT) {
+      const uint32_t src = ext.v0[s1];
+      if (src != 0) {
+        const uint64_t ext_id = e[src - 1u].external_id;
+        if (table_find(cpu.keys, cpu.mask, ext_id) != KTJ_NOSLOT) {
+          x = (int32_t)(int64_t)ext_id;
+          linked = (c.meta[a] & KTJ_M_VALID) != 0;
+        }
+      }
+    }
+    c.ext[a] = x;
+  }
+  count_flag(&sc->n_linked, linked);
+}
+__global__ void k_count_out_of_order(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device,
+                                     Table by_id, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  bool bad = false;
+  if (i < n_runtime + n_device) {
+    const uint64_t a = first_runtime + i;
+    const bool me_runtime = i < n_runtime;
+    if (me_runtime || (c.meta[a] & KTJ_M_VALID)) {
+      const uint32_t slot = table_find(by_id.keys, by_id.mask, c.corr[a]);
+      if (slot != KTJ_NOSLOT) {
+        const uint64_t f = by_id.v1[slot];
+        if (f != a && f != 0xFFFFFFFFull) {
+          const bool first_runtime_row = f < first_runtime + n_runtime;
+          /* act1 = this row, act2 = first row; swapped when the first one is a runtime row */
+          const int64_t t1 = first_runtime_row ? c.ts[f] : c.ts[a];
+          const int64_t t2 = first_runtime_row ? c.ts[a] : c.ts[f];
+          bad = t2 != 0 && t1 > t2;
+        }
+      }
+    }
+  }
+  count_flag(&sc->out_of_order, bad);
+}
+
+hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table t, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_build_extcorr, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, t, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table t, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_build_cpu_ids, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, t, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, Table by_id,
+                         Table by_narrow, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_build_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first_runtime,
+                     by_id, by_narrow, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t insert_device_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, Table by_id,
+                               Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_insert_device_first, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, d, n, c,
+                     first_device, by_id, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t probe_external(Columns c, uint64_t first, uint64_t n, const ktj_extcorr_rec* e, Table ext, Table cpu,
+                          Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_probe_external, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first, n, e, ext, cpu, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t count_out_of_order(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, Table by_id,
+                              Scalars* sc, hipStream_t st) {
+  const uint64_t n = n_runtime + n_device;
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_count_out_of_order, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first_runtime,
+                     n_runtime, n_device, by_id, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* ---- stream back-fill: libkineto/src/RocmStreamQueue.h:42-136 ---- */
+__device__ __forceinline__ bool is_async_op(uint32_t domain) { return domain != KTJ_DOM_MEMSET; }
+
+/* pass 1: stream of the correlation-matched runtime row */
+__global__ void k_stream_by_corr(const ktj_device_rec* d, uint64_t n, const ktj_runtime_rec* r, Columns c,
+                                 uint64_t first_device, Table by_id, const Scalars* sc) {
+  if (sc->have_stream_src == 0) return;
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint64_t a = first_device + i;
+  if (!is_async_op(d[i].domain) || c.res[a] != 0) return;
+  const uint32_t slot = table_find(by_id.keys, by_id.mask, d[i].id);
+  if (slot == KTJ_NOSLOT) return;
+  const uint32_t src = by_id.v0[slot];
+  if (src == 0) return;
+  const ktj_runtime_rec* rr = &r[src - 1u];
+  c.res[a] = (int64_t)(rr->kind == KTJ_RT_KERNEL ? rr->u.kernel.stream : rr->u.copy.stream);
+}
+/* pass 2a: queue → stream, ambiguous when one queue shows two different streams */
+__global__ void k_queue_build(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+                              Scalars* sc) {
+  if (sc->have_stream_src == 0) return;
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint64_t stream = (uint64_t)c.res[first_device + i];
+  const uint64_t queue = d[i].queue;
+  if (!is_async_op(d[i].domain) || stream == 0 || queue == 0) return;
+  const uint32_t slot = table_insert(t.q_keys, KTJ_QUEUE_CAP - 1u, queue);
+  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
+  unsigned long long cur = t.q_stream[slot];
+  if (cur == 0) cur = atomicCAS((unsigned long long*)&t.q_stream[slot], 0ULL, (unsigned long long)stream);
+  if (cur != 0 && cur != stream) t.q_amb[slot] = 1u;
+}
+/* pass 2b: rows still without a stream take their queue's stream */
+__global__ void k_queue_fill(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+                             const Scalars* sc) {
+  if (sc->have_stream_src == 0) return;
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint64_t a = first_device + i;
+  if (!is_async_op(d[i].domain) || c.res[a] != 0) return;
+  const uint32_t slot = table_find(t.q_keys, KTJ_QUEUE_CAP - 1u, d[i].queue);
+  if (slot == KTJ_NOSLOT || t.q_amb[slot] != 0 || t.q_stream[slot] == 0) return;
+  c.res[a] = (int64_t)t.q_stream[slot];
+}
+__device__ __forceinline__ bool dense_key(const ktj_device_rec& d, uint64_t stream, uint64_t* key) {
+  if (!is_async_op(d.domain)) return false;
+  if (stream != 0) *key = stream;
+  else if (d.queue != 0) *key = d.queue | (1ULL << 63);
+  else return false;
+  return true;
+}
+__device__ __forceinline__ uint64_t dense_hash(int32_t device, uint64_t key) {
+  uint64_t h = hash64(key ^ hash64((uint64_t)(int64_t)device + 0x9E3779B97F4A7C15ULL));
+  return h == KTJ_EMPTY_KEY ? 0x5bd1e995ULL : h;
+}
+/* pass 3a: first arrival index per (device, stream key) */
+__global__ void k_dense_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+                              Scalars* sc) {
+  if (sc->have_stream_src == 0) return;
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  uint64_t key;
+  if (!dense_key(d[i], (uint64_t)c.res[first_device + i], &key)) return;
+  const uint32_t slot = table_insert(t.d_hash, KTJ_DENSE_CAP - 1u, dense_hash(d[i].device, key));
+  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT); return; }
+  if (t.d_first[slot] > (uint32_t)i) atomicMin(&t.d_first[slot], (uint32_t)i);
+}
+/* pass 3b: the first row of each pair records the pair itself (single writer per slot) */
+__global__ void k_dense_owner(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+                              const Scalars* sc) {
+  if (sc->have_stream_src == 0) return;
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  uint64_t key;
+  if (!dense_key(d[i], (uint64_t)c.res[first_device + i], &key)) return;
+  const uint32_t slot = table_find(t.d_hash, KTJ_DENSE_CAP - 1u, dense_hash(d[i].device, key));
+  if (slot == KTJ_NOSLOT) return;
+  if (t.d_first[slot] == (uint32_t)i) { t.d_dev[slot] = d[i].device; t.d_key[slot] = key; }
+}
+/* pass 3c (one workgroup): index = 1 + number of pairs of the same device seen earlier */
+#define KTJ_DENSE_MAX 4096
+__global__ void k_dense_rank(StreamTables t, Scalars* sc) {
+  __shared__ uint32_t slots[KTJ_DENSE_MAX];
+  __shared__ uint32_t count;
+  if (sc->have_stream_src == 0) return;
+  if (threadIdx.x == 0) count = 0;
+  __syncthreads();
+  for (uint32_t s = threadIdx.x; s <= KTJ_DENSE_CAP; s += blockDim.x) {
+    if (t.d_hash[s] != KTJ_EMPTY_KEY && t.d_first[s] != 0xFFFFFFFFu) {
+      const uint32_t k = atomicAdd(&count, 1u);
+      if (k < KTJ_DENSE_MAX) slots[k] = s;
+    }
+  }
+  __syncthreads();
+  const uint32_t m = count;
+  if (m > KTJ_DENSE_MAX) { if (threadIdx.x == 0) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT); return; }
+  if (threadIdx.x == 0) sc->n_dense = m;
+  for (uint32_t k = threadIdx.x; k < m; k += blockDim.x) {
+    const uint32_t s = slots[k];
+    const int32_t dev = t.d_dev[s];
+    const uint32_t first = t.d_first[s];
+    uint32_t rank = 1;
+    for (uint32_t j = 0; j < m; ++j) {
+      const uint32_t o = slots[j];
+      if (t.d_dev[o] == dev && t.d_first[o] < first) ++rank;
+    }
+    t.d_rank[s] = rank;
+  }
+}
+/* pass 3d: resourceId() = stream != 0 ? stream : queue (RocprofActivity.h:100-102) */
+__global__ void k_dense_assign(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+                               Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint64_t a = first_device + i;
+  if (!is_async_op(d[i].domain)) return;
+  uint64_t stream = (uint64_t)c.res[a];
+  if (sc->have_stream_src != 0) {
+    uint64_t key;
+    if (dense_key(d[i], stream, &key)) {
+      const uint32_t slot = table_find(t.d_hash, KTJ_DENSE_CAP - 1u, dense_hash(d[i].device, key));
+      if (slot == KTJ_NOSLOT || t.d_dev[slot] != d[i].device || t.d_key[slot] != key) {
+        flag_error(sc, KTJ_DEVERR_HASH_COLLISION);
+      } else stream = t.d_rank[slot];
+    }
+  }
+  c.res[a] = (int64_t)(stream != 0 ? stream : d[i].queue);
+}
+
+hipError_t backfill_streams(const ktj_device_rec* d, uint64_t n, const ktj_runtime_rec* r, Columns c,
+                            uint64_t first_device, Table by_id, StreamTables t, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  const dim3 g(grid_for(n, KTJ_BLOCK)), b(KTJ_BLOCK);
+  hipLaunchKernelGGL(k_stream_by_corr, g, b, 0, st, d, n, r, c, first_device, by_id, (const Scalars*)sc);
+  hipLaunchKernelGGL(k_queue_build, g, b, 0, st, d, n, c, first_device, t, sc);
+  hipLaunchKernelGGL(k_queue_fill, g, b, 0, st, d, n, c, first_device, t, (const Scalars*)sc);
+  hipLaunchKernelGGL(k_dense_first, g, b, 0, st, d, n, c, first_device, t, sc);
+  hipLaunchKernelGGL(k_dense_owner, g, b, 0, st, d, n, c, first_device, t, (const Scalars*)sc);
+  hipLaunchKernelGGL(k_dense_rank, dim3(1), dim3(1024), 0, st, t, sc);
+  hipLaunchKernelGGL(k_dense_assign, g, b, 0, st, d, n, c, first_device, t, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* stage 3: canonical order = stable sort by (deviceId, resourceId, timestamp), signed            */
+/* ------------------------------------------------------------------------------------------ */
+#define KTJ_SET_MAX 4096
+__global__ void k_collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* sc) {
+  const uint64_t a = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const bool valid = a < n && (c.meta[a] & KTJ_M_VALID);
+  uint64_t tb = 0;
+  if (valid) {
+    if (table_insert(s.dev_keys, KTJ_SET_CAP - 1u, (uint64_t)c.dev[a]) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT);
+    if (table_insert(s.res_keys, KTJ_SET_CAP - 1u, (uint64_t)c.res[a]) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT);
+    tb = (uint64_t)c.ts[a] ^ 0x8000000000000000ULL;
+  }
+  /* wave-level min/max, one atomic pair per wave */
+  uint64_t mn = valid ? tb : ~0ULL, mx = valid ? tb : 0ULL;
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint64_t on = __shfl_xor((unsigned long long)mn, o), ox = __shfl_xor((unsigned long long)mx, o);
+    mn = on < mn ? on : mn;
+    mx = ox > mx ? ox : mx;
+  }
+  const uint64_t vm = __ballot(valid ? 1 : 0);
+  if (vm != 0 && lane_id() == 0) {
+    atomicMin(&sc->ts_min_biased, (unsigned long long)mn);
+    atomicMax(&sc->ts_max_biased, (unsigned long long)mx);
+    atomicAdd(&sc->n_valid, (unsigned long long)__popcll(vm));
+  }
+}
+/* one workgroup per set: rank of each distinct value = number of smaller values (signed) */
+__global__ void k_rank_distinct(SortSets s, Scalars* sc) {
+  __shared__ int64_t vals[KTJ_SET_MAX];
+  __shared__ uint32_t slots[KTJ_SET_MAX];
+  __shared__ uint32_t count;
+  uint64_t* keys = blockIdx.x == 0 ? s.dev_keys : s.res_keys;
+  uint32_t* rank = blockIdx.x == 0 ? s.dev_rank : s.res_rank;
+  if (threadIdx.x == 0) count = 0;
+  __syncthreads();
+  for (uint32_t k = threadIdx.x; k <= KTJ_SET_CAP; k += blockDim.x) {
+    bool occupied = k < KTJ_SET_CAP ? keys[k] != KTJ_EMPTY_KEY : keys[k] == 0;
+    if (occupied) {
+      const uint32_t j = atomicAdd(&count, 1u);
+      if (j < KTJ_SET_MAX) { slots[j] = k; vals[j] = k < KTJ_SET_CAP ? (int64_t)keys[k] : (int64_t)-1; }
+    }
+  }
+  __syncthreads();
+  const uint32_t m = count;
+  if (m > KTJ_SET_MAX) { if (threadIdx.x == 0) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT); return; }
+  if (threadIdx.x == 0) { if (blockIdx.x == 0) sc->n_dev_ranks = m; else sc->n_res_ranks = m; }
+  for (uint32_t k = threadIdx.x; k < m; k += blockDim.x) {
+    const int64_t v = vals[k];
+    uint32_t r = 0;
+    for (uint32_t j = 0; j < m; ++j) r += vals[j] < v ? 1u : 0u;
+    rank[slots[k]] = r;
+  }
+}
+__global__ void k_make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits,
+                            uint32_t key_bits, uint64_t* keys, uint32_t* vals) {
+  const uint64_t a = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (a >= n) return;
+  uint64_t key = key_bits >= 64 ? ~0ULL : (1ULL << key_bits); /* dropped rows sort behind everything */
+  if (c.meta[a] & KTJ_M_VALID) {
+    const uint32_t sd = table_find(s.dev_keys, KTJ_SET_CAP - 1u, (uint64_t)c.dev[a]);
+    const uint32_t sr = table_find(s.res_keys, KTJ_SET_CAP - 1u, (uint64_t)c.res[a]);
+    const uint64_t rd = sd != KTJ_NOSLOT ? s.dev_rank[sd] : 0;
+    const uint64_t rr = sr != KTJ_NOSLOT ? s.res_rank[sr] : 0;
+    const uint64_t rel = ((uint64_t)c.ts[a] ^ 0x8000000000000000ULL) - sc->ts_min_biased;
+    uint64_t hi = (rd << res_bits) | rr;
+    key = ts_bits >= 64 ? rel : ((hi << ts_bits) | rel);
+  }
+  keys[a] = key;
+  vals[a] = (uint32_t)a;
+}
+
+hipError_t collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_collect_distinct, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, n, s, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t rank_distinct(SortSets s, Scalars* sc, hipStream_t st) {
+  hipLaunchKernelGGL(k_rank_distinct, dim3(2), dim3(1024), 0, st, s, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits,
+                     uint32_t key_bits, uint64_t* keys, uint32_t* vals, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_make_keys, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, n, s, sc, ts_bits,
+                     res_bits, key_bits, keys, vals);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* ---- stable LSD radix sort, 8 bits per pass ---- */
+#define RADIX_ITEMS 8
+#define RADIX_TILE (KTJ_BLOCK * RADIX_ITEMS)
+#define RADIX_WAVES (KTJ_BLOCK >> 6)
+
+__global__ void k_radix_hist(const uint64_t* keys, uint64_t n, uint32_t shift, uint32_t* hist, uint32_t n_blocks) {
+  __shared__ uint32_t h[256];
+  h[threadIdx.x] = 0;
+  __syncthreads();
+  const uint64_t base = (uint64_t)blockIdx.x * RADIX_TILE;
+  for (int r = 0; r < RADIX_ITEMS; ++r) {
+    const uint64_t i = base + (uint64_t)r * KTJ_BLOCK + threadIdx.x;
+    if (i < n) atomicAdd(&h[(uint32_t)(keys[i] >> shift) & 0xFFu], 1u);
+  }
+  __syncthreads();
+  hist[(uint64_t)threadIdx.x * n_blocks + blockIdx.x] = h[threadIdx.x]; /* digit-major */
+}
+__global__ void k_radix_scatter(const uint64_t* keys_in, const uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out,
+                                uint64_t n, uint32_t shift, const uint32_t* hist_scanned, uint32_t n_blocks) {
+  __shared__ uint32_t base_of[256];               /* global offset of this block's run per digit */
+  __shared__ uint32_t run[256];                   /* elements of each digit already placed        */
+  __shared__ uint32_t wave_cnt[RADIX_WAVES][256];
+  base_of[threadIdx.x] = hist_scanned[(uint64_t)threadIdx.x * n_blocks + blockIdx.x];
+  run[threadIdx.x] = 0;
+  for (int w = 0; w < RADIX_WAVES; ++w) wave_cnt[w][threadIdx.x] = 0;
+  __syncthreads();
+  const uint32_t w = threadIdx.x >> 6;
+  const uint64_t lt = lanemask_lt();
+  const uint64_t base = (uint64_t)blockIdx.x * RADIX_TILE;
+  for (int r = 0; r < RADIX_ITEMS; ++r) {
+    const uint64_t i = base + (uint64_t)r * KTJ_BLOCK + threadIdx.x;
+    const bool valid = i < n;
+    const uint64_t key = valid ? keys_in[i] : 0;
+    const uint32_t val = valid ? vals_in[i] : 0;
+    const uint32_t digit = (uint32_t)(key >> shift) & 0xFFu;
+    /* lanes of this wavefront holding the same digit */
+    uint64_t peers = __ballot(valid ? 1 : 0);
+    for (int b = 0; b < 8; ++b) {
+      const uint64_t bal = __ballot((digit >> b) & 1u);
+      peers &= ((digit >> b) & 1u) ? bal : ~bal;
+    }
+    const uint32_t rank_in_wave = (uint32_t)__popcll(peers & lt);
+    if (valid && rank_in_wave == 0) wave_cnt[w][digit] = (uint32_t)__popcll(peers);
+    __syncthreads();
+    if (valid) {
+      uint32_t off = run[digit] + rank_in_wave;
+      for (uint32_t k = 0; k < w; ++k) off += wave_cnt[k][digit];
+      const uint64_t dst = (uint64_t)base_of[digit] + off;
+      keys_out[dst] = key;
+      vals_out[dst] = val;
+    }
+    __syncthreads();
+    {
+      uint32_t s = 0;
+      for (int k = 0; k < RADIX_WAVES; ++k) { s += wave_cnt[k][threadIdx.x]; wave_cnt[k][threadIdx.x] = 0; }
+      run[threadIdx.x] += s;
+    }
+    __syncthreads();
+  }
+}
+
+uint64_t radix_tmp_elems(uint64_t n) { return 256ull * ((n + RADIX_TILE - 1) / RADIX_TILE) + 256; }
+
+hipError_t radix_sort(uint64_t* keys_a, uint32_t* vals_a, uint64_t* keys_b, uint32_t* vals_b, uint64_t n,
+                      uint32_t bits, uint32_t* hist, uint64_t* scan_tmp, uint64_t** res_keys, uint32_t** res_vals,
+                      hipStream_t st) {
+  *res_keys = keys_a;
+  *res_vals = vals_a;
+  if (n == 0) return hipSuccess;
+  const uint32_t n_blocks = (uint32_t)((n + RADIX_TILE - 1) / RADIX_TILE);
+  uint64_t* ki = keys_a; uint32_t* vi = vals_a; uint64_t* ko = keys_b; uint32_t* vo = vals_b;
+  for (uint32_t shift = 0; shift < bits; shift += 8) {
+    hipLaunchKernelGGL(k_radix_hist, dim3(n_blocks), dim3(KTJ_BLOCK), 0, st, (const uint64_t*)ki, n, shift, hist, n_blocks);
+    hipError_t e = scan_u32_inplace(hist, 256ull * n_blocks, scan_tmp, st);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(k_radix_scatter, dim3(n_blocks), dim3(KTJ_BLOCK), 0, st, (const uint64_t*)ki, (const uint32_t*)vi,
+                       ko, vo, n, shift, (const uint32_t*)hist, n_blocks);
+    uint64_t* tk = ki; ki = ko; ko = tk;
+    uint32_t* tv = vi; vi = vo; vo = tv;
+  }
+  *res_keys = ki;
+  *res_vals = vi;
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* stage 4a: joined rows and exact byte lengths, arrival order                                  */
+/* ------------------------------------------------------------------------------------------ */
+__device__ __forceinline__ void store_row(MatRow* dst, const MatRow& m) {
+  const uint4* s = reinterpret_cast<const uint4*>(&m);
+  uint4* d = reinterpret_cast<uint4*>(dst);
+  for (int k = 0; k < (int)(sizeof(MatRow) / 16); ++k) d[k] = s[k];
+}
+__device__ __forceinline__ uint32_t row_length(const MatRow& m, const EmitCtx& ctx, Scalars* sc) {
+  if (!(m.meta & KTJ_M_VALID)) return 0;
+  CountWriter cw;
+  format_activity(cw, m, ctx);
+  if (cw.n >= (1ull << 30)) { flag_error(sc, KTJ_DEVERR_RECORD_TOO_LONG); return 0; }
+  return (uint32_t)cw.n;
+}
+__device__ __forceinline__ void count_row_stats(const MatRow& m, bool in, const EmitCtx& ctx, Scalars* sc) {
+  const bool valid = in && (m.meta & KTJ_M_VALID);
+  count_flag(&sc->n_flow, valid && (m.meta & KTJ_M_FLOW));
+  const bool blank = valid && !(m.meta & KTJ_M_NAME_BUILTIN) && m.name_id < ctx.dict.n &&
+                     (ctx.dict.flags[m.name_id] & KTJ_SF_NAME_UNKNOWN);
+  count_flag(&sc->n_blank_names, blank);
+}
+
+__global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  MatRow m;
+  m.meta = 0; m.name_id = 0;
+  if (i < n) {
+    m = mat_generic(g[i]);
+    store_row(&mat[i], m);
+    len[i] = row_length(m, ctx, sc);
+  }
+  count_row_stats(m, i < n, ctx, sc);
+}
+__global__ void k_mat_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, EmitCtx ctx,
+                              MatRow* mat, uint32_t* len, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  MatRow m;
+  m.meta = 0; m.name_id = 0;
+  if (i < n) {
+    const uint64_t a = first + i;
+    const ktj_runtime_rec rec = r[i];
+    const bool known = rec.cid < api.n_cids;
+    const uint32_t name = known ? api.cid_name_ids[rec.cid] : KTJ_NONE;
+    const bool fs = known && ((api.flow_start_bits[rec.cid >> 5] >> (rec.cid & 31u)) & 1u);
+    m = mat_runtime(rec, c.ts[a], c.dur[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a], name, fs, rec.cid == api.malloc_cid);
+    store_row(&mat[a], m);
+    len[a] = row_length(m, ctx, sc);
+  }
+  count_row_stats(m, i < n, ctx, sc);
+}
+__global__ void k_mat_device(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const ktj_runtime_rec* r,
+                             Table by_narrow, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  MatRow m;
+  m.meta = 0; m.name_id = 0;
+  if (i < n) {
+    const uint64_t a = first + i;
+    const ktj_device_rec rec = d[i];
+    const ktj_runtime_rec* ksrc = nullptr;
+    bool has_size = false;
+    uint64_t size = 0;
+    if (rec.domain != KTJ_DOM_MEMSET && by_narrow.keys != nullptr) { /* RocprofActivity_inl.h:161-180 */
+      const uint32_t slot = table_find(by_narrow.keys, by_narrow.mask, narrow_corr_key(rec.id));
+      if (slot != KTJ_NOSLOT) {
+        const uint32_t ss = by_narrow.v1[slot], ks = by_narrow.v0[slot];
+        if (ss != 0) {
+          const ktj_runtime_rec* sr = &r[ss - 1u];
+          has_size = true;
+          size = sr->kind == KTJ_RT_COPY ? sr->u.copy.size : sr->u.malloc_.size;
+        } else if (ks != 0) ksrc = &r[ks - 1u];
+      }
+    }
+    m = mat_device(rec, c.ts[a], c.dur[a], c.res[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a], ksrc, has_size, size);
+    store_row(&mat[a], m);
+    len[a] = row_length(m, ctx, sc);
+  }
+  count_row_stats(m, i < n, ctx, sc);
+}
+__global__ void k_gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) len_sorted[i] = len[perm[i]];
+}
+
+hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc,
+                            hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_mat_generic, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, ctx, mat, len, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, EmitCtx ctx,
+                            MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_mat_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, ctx, mat,
+                     len, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const ktj_runtime_rec* r,
+                           Table by_narrow, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_mat_device, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, d, n, c, first, r, by_narrow,
+                     ctx, mat, len, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_gather_len, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, perm, len, n, len_sorted);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* stage 4b: emit.  Workgroup k owns the output bytes [k*TILE, (k+1)*TILE) of the whole document */
+/* (clipped to the activity section), so every global store is an aligned 16-byte store.  It     */
+/* finds the activities overlapping its range by binary search in the offsets, formats each one  */
+/* into LDS with clipping (an activity straddling a tile boundary is formatted by both tiles),   */
+/* copies dictionary strings with whole wavefronts, and flushes the tile.                        */
+/* ------------------------------------------------------------------------------------------ */
+#define EMIT_THREADS 128
+#define EMIT_MAX_JOBS 384
+
+__global__ void __launch_bounds__(EMIT_THREADS)
+k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n, EmitCtx ctx, char* out,
+       uint64_t prefix_len, uint64_t act_bytes) {
+  __shared__ __attribute__((aligned(16))) char tile[KTJ_EMIT_TILE];
+  __shared__ CopyJob jobs[EMIT_MAX_JOBS];
+  __shared__ uint32_t n_jobs;
+
+  const uint64_t t0 = ((prefix_len / KTJ_EMIT_TILE) + blockIdx.x) * (uint64_t)KTJ_EMIT_TILE; /* absolute */
+  const uint64_t abs_lo = t0 > prefix_len ? t0 : prefix_len;
+  const uint64_t abs_end = prefix_len + act_bytes;
+  const uint64_t abs_hi = t0 + KTJ_EMIT_TILE < abs_end ? t0 + KTJ_EMIT_TILE : abs_end;
+  if (abs_lo >= abs_hi) return;
+  const uint64_t lo = abs_lo - prefix_len, hi = abs_hi - prefix_len; /* activity-relative */
+  const uint32_t head = (uint32_t)(abs_lo - t0);                       /* tile[head] ↔ abs_lo */
+  const int32_t span = (int32_t)(hi - lo);
+
+  /* r0 = last record with offs[r0] <= lo; r1 = first record with offs[r1] >= hi */
+  uint64_t a = 0, b = n;
+  while (a < b) { const uint64_t m = (a + b) >> 1; if (offs[m + 1] > lo) b = m; else a = m + 1; }
+  const uint64_t r0 = a;
+  a = r0; b = n;
+  while (a < b) { const uint64_t m = (a + b) >> 1; if (offs[m] >= hi) b = m; else a = m + 1; }
+  const uint64_t r1 = a;
+
+  if (threadIdx.x == 0) n_jobs = 0;
+  __syncthreads();
+  for (uint64_t r = r0 + threadIdx.x; r < r1; r += EMIT_THREADS) {
+    const uint64_t o = offs[r];
+    if (offs[r + 1] == o) continue; /* dropped or empty */
+    MatRow m;
+    {
+      const uint4* s = reinterpret_cast<const uint4*>(&mat[perm[r]]);
+      uint4* d = reinterpret_cast<uint4*>(&m);
+      for (int k = 0; k < (int)(sizeof(MatRow) / 16); ++k) d[k] = s[k];
+    }
+    TileWriter w;
+    w.buf = tile + head;
+    w.pos = (int32_t)((int64_t)o - (int64_t)lo);
+    w.tile = span;
+    w.jobs = jobs;
+    w.n_jobs = &n_jobs;
+    w.max_jobs = EMIT_MAX_JOBS;
+    format_activity(w, m, ctx);
+  }
+  __syncthreads();
+  {
+    const uint32_t nj = n_jobs < EMIT_MAX_JOBS ? n_jobs : EMIT_MAX_JOBS;
+    const uint32_t wv = threadIdx.x >> 6, ln = threadIdx.x & 63u;
+    for (uint32_t j = wv; j < nj; j += (EMIT_THREADS >> 6)) {
+      const CopyJob job = jobs[j];
+      char* dst = tile + head + job.dst;
+      for (uint32_t k = ln; k < job.len; k += 64) dst[k] = job.src[k];
+    }
+  }
+  __syncthreads();
+  /* flush: unaligned head bytes (first tile only), 16-byte body, tail bytes */
+  char* g = out + abs_lo;
+  const char* s = tile + head;
+  const uint32_t nbytes = (uint32_t)span;
+  uint32_t pre = (uint32_t)((16u - (uint32_t)((uintptr_t)g & 15u)) & 15u);
+  if (pre > nbytes) pre = nbytes;
+  for (uint32_t k = threadIdx.x; k < pre; k += EMIT_THREADS) g[k] = s[k];
+  const uint32_t body = (nbytes - pre) / 16u;
+  {
+    uint4* gv = reinterpret_cast<uint4*>(g + pre);
+    const uint4* sv = reinterpret_cast<const uint4*>(s + pre);
+    for (uint32_t k = threadIdx.x; k < body; k += EMIT_THREADS) gv[k] = sv[k];
+  }
+  for (uint32_t k = pre + body * 16u + threadIdx.x; k < nbytes; k += EMIT_THREADS) g[k] = s[k];
+}
+
+hipError_t emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n, EmitCtx ctx, char* out,
+                uint64_t prefix_len, uint64_t act_bytes, hipStream_t st) {
+  if (act_bytes == 0) return hipSuccess;
+  const uint64_t first_tile = prefix_len / KTJ_EMIT_TILE;
+  const uint64_t last_tile = (prefix_len + act_bytes - 1) / KTJ_EMIT_TILE;
+  const uint64_t tiles = last_tile - first_tile + 1;
+  hipLaunchKernelGGL(k_emit, dim3((unsigned)tiles), dim3(EMIT_THREADS), 0, st, mat, perm, offs, n, ctx, out, prefix_len,
+                     act_bytes);
+  return KTJ_LAUNCH_CHECK();
+}
+
+}  // namespace gpu
+}  // namespace ktj
