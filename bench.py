@@ -1,0 +1,172 @@
+#!/usr/bin/env python3
+"""Benchmark of the records -> Chrome-trace JSON hot path on one MI355X.
+
+One "step" = one complete pass of the engine (dictionary, decode, clock conversion, joins, sort,
+size, scan, emit) over the 10M-record configuration (10M device rows + 10M runtime rows + 2M CPU
+ops, 128 streams), with the raw records already resident in HBM and the JSON document left in a
+device buffer.  Prints one JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--n-device N] [--config C]
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+FULL_SIZE = {1: 10000, 2: 1000000, 3: 10000000, 4: 11000000, 5: 5000000}
+WORKLOAD = {
+    1: "config1: 10k CPU ops + 10k launches + 10k kernels, 4 streams",
+    2: "config2: 1M device rows (70% kernel / 20% memcpy / 10% memset) + 1M runtime + 1M CPU ops, 32 streams, linear clock model",
+    3: "config3: 10M device + 10M runtime + 2M CPU-op records, 128 streams, block-shuffled arrival, ac2g flows",
+    4: "config4: graph launches with 100-1000 kernel fan-out (~11M kernels), 5% orphans each way",
+    5: "config5: 5M string-heavy generic kernel records with typed args",
+}
+
+
+def cpu_baseline(config, sample_device_rows):
+    """Times the single-threaded CPU restatement of the reference path (oracle/) on a bounded
+    sample of the same workload, and checks the engine against it on that sample."""
+    from kineto_amd import abi
+    from kineto_amd.engine import TraceEngine
+    import oracle_glue as og
+    sp, release = abi.synth_stream(config, sample_device_rows, host_name="bench")
+    s = sp.contents
+    n_records = s.n_generic + s.n_runtime + s.n_device
+    t0 = time.perf_counter()
+    ora = og.OracleRun(sp)
+    dt = time.perf_counter() - t0
+    want = ora.output()
+    with TraceEngine(s.trace_name.decode(), device=0) as eng:
+        eng.submit_stream(sp)
+        eng.process()
+        got = eng.output()
+    same = got == want
+    stages = ora.timings()
+    ora.close()
+    release()
+    return {
+        "value": n_records / dt, "unit": "records/s", "cores": 1, "kind": "port",
+        "sample": f"same workload scaled to {sample_device_rows} device rows ({n_records} records, "
+                  f"{len(want)} output bytes) in {dt:.2f} s on one host core "
+                  f"(join {stages[0]:.2f} s, sort {stages[1]:.2f} s, emit {stages[2]:.2f} s)",
+        "output_gb_per_s": len(want) / dt / 1e9,
+        "engine_output_identical_on_sample": bool(same),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--config", type=int, default=3)
+    ap.add_argument("--n-device", type=int, default=0, help="device rows (0 = the configuration's full size)")
+    ap.add_argument("--cpu-sample", type=int, default=0, help="device rows of the CPU-baseline sample (0 = auto)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path runs on exactly one GPU (no sharding, no collectives); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from kineto_amd import abi
+    from kineto_amd.engine import TraceEngine
+
+    cfg = args.config
+    n_dev = args.n_device or FULL_SIZE[cfg]
+    t0 = time.perf_counter()
+    sp, release = abi.synth_stream(cfg, n_dev, host_name="bench")
+    s = sp.contents
+    n_records = s.n_generic + s.n_runtime + s.n_device
+    gen_s = time.perf_counter() - t0
+    raw_bytes = s.n_generic * 64 + s.n_runtime * 96 + s.n_device * 64 + s.n_extcorr * 16 + s.n_args * 8
+
+    eng = TraceEngine(s.trace_name.decode(), device=0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    eng.submit_stream(sp)          # host -> HBM; not part of the timed steps
+    torch.cuda.synchronize()
+    h2d_s = time.perf_counter() - t0
+    release()
+
+    for _ in range(args.warmup):
+        eng.process()
+    torch.cuda.synchronize()
+    stage_sum = [0.0] * abi.N_STAGES
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        eng.process()
+        st = eng.stats()
+        for k in range(abi.N_STAGES):
+            stage_sum[k] += st.stage_ms[k]
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    st = eng.stats()
+    out_bytes = st.output_bytes
+    stage_ms = {abi.STAGE_NAMES[k]: stage_sum[k] / args.steps for k in range(abi.N_STAGES) if stage_sum[k] > 0}
+    stage_gbs = {abi.STAGE_NAMES[k]: st.stage_bytes[k] / (stage_sum[k] / args.steps * 1e-3) / 1e9
+                 for k in range(abi.N_STAGES) if stage_sum[k] > 0 and st.stage_bytes[k] > 0}
+
+    # PCIe-inclusive figure, reported on the side: one device -> pinned host copy of the document
+    t0 = time.perf_counter()
+    host_copy_ok = True
+    try:
+        p, n = C.c_void_p(), C.c_uint64()
+        rc = eng.lib.ktj_output_host(eng.h, C.byref(p), C.byref(n))
+        host_copy_ok = rc == 0
+    except Exception:
+        host_copy_ok = False
+    d2h_s = time.perf_counter() - t0
+    d2h_ms = eng.stats().stage_ms[8] if host_copy_ok else None
+    eng.close()
+
+    emit_ms = stage_ms.get("emit", 0.0)
+    emit_alg = int(st.stage_bytes[7])
+    achieved = emit_alg / (emit_ms * 1e-3) / 1e9 if emit_ms > 0 else 0.0
+    result = {
+        "metric": "trace_records_per_s",
+        "value": n_records / (ms_per_step * 1e-3),
+        "unit": "records/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8/int64",
+        "data": "synthetic",
+        "config": {"workload": WORKLOAD[cfg], "records": int(n_records), "device_rows": int(s.n_device) if False else int(n_dev),
+                   "output_bytes": int(out_bytes), "raw_input_bytes": int(raw_bytes),
+                   "output_placement": "device buffer (HBM)"},
+        "output_gb_per_s": out_bytes / (ms_per_step * 1e-3) / 1e9,
+        "output_frac_of_hbm_peak": out_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "stage_ms": stage_ms,
+        "stage_algorithmic_gb_per_s": stage_gbs,
+        "roofline": {"bound": "hbm", "kernel": "k_emit", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": emit_alg, "avg_launch_ms": emit_ms},
+        "pcie": {"h2d_submit_s": h2d_s, "d2h_document_ms": d2h_ms, "d2h_wall_s": d2h_s,
+                 "records_per_s_incl_d2h": (n_records / (ms_per_step * 1e-3 + (d2h_ms or 0) * 1e-3)) if d2h_ms else None},
+        "generate_s": gen_s,
+    }
+    if not args.no_cpu_baseline:
+        sample = args.cpu_sample or max(1000, min(n_dev, {1: 10000, 2: 400000, 3: 400000, 4: 800000, 5: 150000}[cfg]))
+        result["cpu_baseline"] = cpu_baseline(cfg, sample)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
