@@ -66,11 +66,22 @@ __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
   return v;
 }
-/* one atomicAdd per wave */
-__device__ __forceinline__ void count_flag(unsigned long long* counter, bool flag) {
-  const uint64_t m = __ballot(flag ? 1 : 0);
-  if (m != 0 && lane_id() == (uint32_t)(__ffsll((long long)m) - 1)) atomicAdd(counter, (unsigned long long)__popcll(m));
+/* Sums a per-thread count over the workgroup and adds it to a global counter with one atomic per
+ * workgroup (a single hot address serialises atomics in L2, so they must be rare).  Must be
+ * reached by every thread of the workgroup. */
+__device__ __forceinline__ void block_add(unsigned long long* counter, uint32_t mine) {
+  __shared__ uint32_t partial[KTJ_BLOCK >> 6];
+  const uint32_t w = wave_sum_u32(mine);
+  __syncthreads();
+  if (lane_id() == 0) partial[threadIdx.x >> 6] = w;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t t = 0;
+    for (uint32_t k = 0; k < (blockDim.x >> 6); ++k) t += partial[k];
+    if (t) atomicAdd(counter, (unsigned long long)t);
+  }
 }
+#define KTJ_MAX_GRID 4096u /* grid-stride kernels: enough workgroups to fill 256 CUs several times over */
 
 __global__ void k_fill_u64(uint64_t* p, uint64_t v, uint64_t n) {
   uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -89,6 +100,10 @@ __global__ void k_init_scalars(Scalars* s) {
 }
 
 static inline unsigned grid_for(uint64_t n, unsigned per_block) { return (unsigned)((n + per_block - 1) / per_block); }
+static inline unsigned grid_stride_for(uint64_t n, unsigned per_block) {
+  const uint64_t g = (n + per_block - 1) / per_block;
+  return (unsigned)(g < KTJ_MAX_GRID ? g : KTJ_MAX_GRID);
+}
 #define KTJ_LAUNCH_CHECK() hipGetLastError()
 
 hipError_t fill_u64(uint64_t* p, uint64_t v, uint64_t n, hipStream_t st) {
@@ -375,9 +390,9 @@ hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_
 /* ------------------------------------------------------------------------------------------ */
 __global__ void k_convert(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, ClockDev clk,
                           int64_t win_start, int64_t win_end, Scalars* sc) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  bool oor = false;
-  if (i < n_runtime + n_device) {
+  uint32_t n_oor = 0;
+  const uint64_t n = n_runtime + n_device;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t a = first_runtime + i;
     uint64_t b = (uint64_t)c.ts[a], e = (uint64_t)c.dur[a];
     uint32_t meta = c.meta[a];
@@ -390,19 +405,19 @@ __global__ void k_convert(Columns c, uint64_t first_runtime, uint64_t n_runtime,
       convert_range(clk, clk.device_mode, &b, &e);
       device_times((meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT, b, e, &ts, &dur);
     }
-    oor = out_of_range(ts, dur, win_start, win_end);
-    if (!oor) meta |= KTJ_M_VALID;
+    if (out_of_range(ts, dur, win_start, win_end)) ++n_oor;
+    else meta |= KTJ_M_VALID;
     c.ts[a] = ts;
     c.dur[a] = dur;
     c.meta[a] = meta;
   }
-  count_flag(&sc->out_of_range, oor);
+  block_add(&sc->out_of_range, n_oor);
 }
 hipError_t convert_rows(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, ClockDev clk,
                         int64_t win_start, int64_t win_end, Scalars* sc, hipStream_t st) {
   const uint64_t n = n_runtime + n_device;
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_convert, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first_runtime, n_runtime,
+  hipLaunchKernelGGL(k_convert, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first_runtime, n_runtime,
                      n_device, clk, win_start, win_end, sc);
   return KTJ_LAUNCH_CHECK();
 }
@@ -468,9 +483,8 @@ __global__ void k_insert_device_first(const ktj_device_rec* d, uint64_t n, Colum
 /* linkedActivity(): GenericActivityProfiler.cpp:397-408; "External id": output_json.cpp:871-874 */
 __global__ void k_probe_external(Columns c, uint64_t first, uint64_t n, const ktj_extcorr_rec* e, Table ext,
                                  Table cpu, Scalars* sc) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  bool linked = false;
-  if (i < n) {
+  uint32_t n_linked = 0;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t a = first + i;
     int32_t x = 0;
     const uint32_t s1 = table_find(ext.keys, ext.mask, narrow_corr_key(c.corr[a]));
@@ -480,36 +494,33 @@ __global__ void k_probe_external(Columns c, uint64_t first, uint64_t n, const kt
         const uint64_t ext_id = e[src - 1u].external_id;
         if (table_find(cpu.keys, cpu.mask, ext_id) != KTJ_NOSLOT) {
           x = (int32_t)(int64_t)ext_id;
-          linked = (c.meta[a] & KTJ_M_VALID) != 0;
+          if (c.meta[a] & KTJ_M_VALID) ++n_linked;
         }
       }
     }
     c.ext[a] = x;
   }
-  count_flag(&sc->n_linked, linked);
+  block_add(&sc->n_linked, n_linked);
 }
 __global__ void k_count_out_of_order(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device,
                                      Table by_id, Scalars* sc) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  bool bad = false;
-  if (i < n_runtime + n_device) {
+  uint32_t n_bad = 0;
+  const uint64_t n = n_runtime + n_device;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t a = first_runtime + i;
     const bool me_runtime = i < n_runtime;
-    if (me_runtime || (c.meta[a] & KTJ_M_VALID)) {
-      const uint32_t slot = table_find(by_id.keys, by_id.mask, c.corr[a]);
-      if (slot != KTJ_NOSLOT) {
-        const uint64_t f = by_id.v1[slot];
-        if (f != a && f != 0xFFFFFFFFull) {
-          const bool first_runtime_row = f < first_runtime + n_runtime;
-          /* act1 = this row, act2 = first row; swapped when the first one is a runtime row */
-          const int64_t t1 = first_runtime_row ? c.ts[f] : c.ts[a];
-          const int64_t t2 = first_runtime_row ? c.ts[a] : c.ts[f];
-          bad = t2 != 0 && t1 > t2;
-        }
-      }
-    }
+    if (!me_runtime && !(c.meta[a] & KTJ_M_VALID)) continue;
+    const uint32_t slot = table_find(by_id.keys, by_id.mask, c.corr[a]);
+    if (slot == KTJ_NOSLOT) continue;
+    const uint64_t f = by_id.v1[slot];
+    if (f == a || f == 0xFFFFFFFFull) continue;
+    const bool first_is_runtime = f < first_runtime + n_runtime;
+    /* act1 = this row, act2 = first row; swapped when the first one is a runtime row */
+    const int64_t t1 = first_is_runtime ? c.ts[f] : c.ts[a];
+    const int64_t t2 = first_is_runtime ? c.ts[a] : c.ts[f];
+    if (t2 != 0 && t1 > t2) ++n_bad;
   }
-  count_flag(&sc->out_of_order, bad);
+  block_add(&sc->out_of_order, n_bad);
 }
 
 hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table t, Scalars* sc, hipStream_t st) {
@@ -539,14 +550,14 @@ hipError_t insert_device_first(const ktj_device_rec* d, uint64_t n, Columns c, u
 hipError_t probe_external(Columns c, uint64_t first, uint64_t n, const ktj_extcorr_rec* e, Table ext, Table cpu,
                           Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_probe_external, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first, n, e, ext, cpu, sc);
+  hipLaunchKernelGGL(k_probe_external, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first, n, e, ext, cpu, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t count_out_of_order(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, Table by_id,
                               Scalars* sc, hipStream_t st) {
   const uint64_t n = n_runtime + n_device;
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_count_out_of_order, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first_runtime,
+  hipLaunchKernelGGL(k_count_out_of_order, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first_runtime,
                      n_runtime, n_device, by_id, sc);
   return KTJ_LAUNCH_CHECK();
 }
@@ -699,28 +710,65 @@ hipError_t backfill_streams(const ktj_device_rec* d, uint64_t n, const ktj_runti
 /* stage 3: canonical order = stable sort by (deviceId, resourceId, timestamp), signed            */
 /* ------------------------------------------------------------------------------------------ */
 #define KTJ_SET_MAX 4096
-__global__ void k_collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* sc) {
-  const uint64_t a = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const bool valid = a < n && (c.meta[a] & KTJ_M_VALID);
-  uint64_t tb = 0;
-  if (valid) {
-    if (table_insert(s.dev_keys, KTJ_SET_CAP - 1u, (uint64_t)c.dev[a]) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT);
-    if (table_insert(s.res_keys, KTJ_SET_CAP - 1u, (uint64_t)c.res[a]) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT);
-    tb = (uint64_t)c.ts[a] ^ 0x8000000000000000ULL;
+/* Workgroup-local set in LDS in front of the global set: a value reaches the global table once
+ * per workgroup instead of once per row.  (All rows share a handful of device/resource ids, and
+ * millions of probes of the same few global slots serialise in L2.)  Returns true when the
+ * caller is the first in its workgroup to see the key, or when the local set is full. */
+#define LOCAL_SET_SLOTS 1024u
+__device__ __forceinline__ bool local_set_first(unsigned long long* lds, uint64_t key) {
+  const uint32_t h = ((uint32_t)key ^ ((uint32_t)(key >> 32) * 0x9E3779B1u)) * 0x85EBCA6Bu;
+  uint32_t slot = h >> 22; /* 10 bits */
+  for (uint32_t probe = 0; probe < 16; ++probe) {
+    const unsigned long long cur = lds[slot];
+    if (cur == key) return false;
+    if (cur == KTJ_EMPTY_KEY) {
+      const unsigned long long prev = atomicCAS(&lds[slot], (unsigned long long)KTJ_EMPTY_KEY, (unsigned long long)key);
+      if (prev == KTJ_EMPTY_KEY) return true;
+      if (prev == key) return false;
+    }
+    slot = (slot + 1u) & (LOCAL_SET_SLOTS - 1u);
   }
-  /* wave-level min/max, one atomic pair per wave */
-  uint64_t mn = valid ? tb : ~0ULL, mx = valid ? tb : 0ULL;
+  return true;
+}
+__global__ void k_collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* sc) {
+  __shared__ uint64_t red_min[KTJ_BLOCK >> 6], red_max[KTJ_BLOCK >> 6];
+  __shared__ unsigned long long seen_dev[LOCAL_SET_SLOTS], seen_res[LOCAL_SET_SLOTS];
+  for (uint32_t k = threadIdx.x; k < LOCAL_SET_SLOTS; k += blockDim.x) { seen_dev[k] = KTJ_EMPTY_KEY; seen_res[k] = KTJ_EMPTY_KEY; }
+  __syncthreads();
+  uint64_t mn = ~0ULL, mx = 0ULL;
+  uint32_t n_valid = 0;
+  for (uint64_t a = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; a < n; a += (uint64_t)gridDim.x * blockDim.x) {
+    if (!(c.meta[a] & KTJ_M_VALID)) continue;
+    const uint64_t dev = (uint64_t)c.dev[a], res = (uint64_t)c.res[a];
+    if (dev == KTJ_EMPTY_KEY || local_set_first(seen_dev, dev)) {
+      if (table_insert(s.dev_keys, KTJ_SET_CAP - 1u, dev) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT);
+    }
+    if (res == KTJ_EMPTY_KEY || local_set_first(seen_res, res)) {
+      if (table_insert(s.res_keys, KTJ_SET_CAP - 1u, res) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT);
+    }
+    const uint64_t tb = (uint64_t)c.ts[a] ^ 0x8000000000000000ULL;
+    mn = tb < mn ? tb : mn;
+    mx = tb > mx ? tb : mx;
+    ++n_valid;
+  }
   for (int o = 32; o > 0; o >>= 1) {
     const uint64_t on = __shfl_xor((unsigned long long)mn, o), ox = __shfl_xor((unsigned long long)mx, o);
     mn = on < mn ? on : mn;
     mx = ox > mx ? ox : mx;
   }
-  const uint64_t vm = __ballot(valid ? 1 : 0);
-  if (vm != 0 && lane_id() == 0) {
-    atomicMin(&sc->ts_min_biased, (unsigned long long)mn);
-    atomicMax(&sc->ts_max_biased, (unsigned long long)mx);
-    atomicAdd(&sc->n_valid, (unsigned long long)__popcll(vm));
+  if (lane_id() == 0) { red_min[threadIdx.x >> 6] = mn; red_max[threadIdx.x >> 6] = mx; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (uint32_t k = 1; k < (blockDim.x >> 6); ++k) {
+      mn = red_min[k] < mn ? red_min[k] : mn;
+      mx = red_max[k] > mx ? red_max[k] : mx;
+    }
+    if (mn <= mx) {
+      atomicMin(&sc->ts_min_biased, (unsigned long long)mn);
+      atomicMax(&sc->ts_max_biased, (unsigned long long)mx);
+    }
   }
+  block_add(&sc->n_valid, n_valid);
 }
 /* one workgroup per set: rank of each distinct value = number of smaller values (signed) */
 __global__ void k_rank_distinct(SortSets s, Scalars* sc) {
@@ -769,7 +817,9 @@ __global__ void k_make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc
 
 hipError_t collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_collect_distinct, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, n, s, sc);
+  /* few, fat workgroups: each one pays for its own local set once */
+  const unsigned g = grid_stride_for(n, KTJ_BLOCK * 16);
+  hipLaunchKernelGGL(k_collect_distinct, dim3(g), dim3(KTJ_BLOCK), 0, st, c, n, s, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t rank_distinct(SortSets s, Scalars* sc, hipStream_t st) {
@@ -884,54 +934,55 @@ __device__ __forceinline__ uint32_t row_length(const MatRow& m, const EmitCtx& c
   if (cw.n >= (1ull << 30)) { flag_error(sc, KTJ_DEVERR_RECORD_TOO_LONG); return 0; }
   return (uint32_t)cw.n;
 }
-__device__ __forceinline__ void count_row_stats(const MatRow& m, bool in, const EmitCtx& ctx, Scalars* sc) {
-  const bool valid = in && (m.meta & KTJ_M_VALID);
-  count_flag(&sc->n_flow, valid && (m.meta & KTJ_M_FLOW));
-  const bool blank = valid && !(m.meta & KTJ_M_NAME_BUILTIN) && m.name_id < ctx.dict.n &&
-                     (ctx.dict.flags[m.name_id] & KTJ_SF_NAME_UNKNOWN);
-  count_flag(&sc->n_blank_names, blank);
+struct RowStats { uint32_t n_flow = 0, n_blank = 0; };
+__device__ __forceinline__ void count_row_stats(const MatRow& m, const EmitCtx& ctx, RowStats* rs) {
+  if (!(m.meta & KTJ_M_VALID)) return;
+  if (m.meta & KTJ_M_FLOW) ++rs->n_flow;
+  if (!(m.meta & KTJ_M_NAME_BUILTIN) && m.name_id < ctx.dict.n && (ctx.dict.flags[m.name_id] & KTJ_SF_NAME_UNKNOWN))
+    ++rs->n_blank;
+}
+__device__ __forceinline__ void flush_row_stats(const RowStats& rs, Scalars* sc) {
+  block_add(&sc->n_flow, rs.n_flow);
+  block_add(&sc->n_blank_names, rs.n_blank);
 }
 
 __global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  MatRow m;
-  m.meta = 0; m.name_id = 0;
-  if (i < n) {
-    m = mat_generic(g[i]);
+  RowStats rs;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const MatRow m = mat_generic(g[i]);
     store_row(&mat[i], m);
     len[i] = row_length(m, ctx, sc);
+    count_row_stats(m, ctx, &rs);
   }
-  count_row_stats(m, i < n, ctx, sc);
+  flush_row_stats(rs, sc);
 }
 __global__ void k_mat_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, EmitCtx ctx,
                               MatRow* mat, uint32_t* len, Scalars* sc) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  MatRow m;
-  m.meta = 0; m.name_id = 0;
-  if (i < n) {
+  RowStats rs;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t a = first + i;
     const ktj_runtime_rec rec = r[i];
     const bool known = rec.cid < api.n_cids;
     const uint32_t name = known ? api.cid_name_ids[rec.cid] : KTJ_NONE;
     const bool fs = known && ((api.flow_start_bits[rec.cid >> 5] >> (rec.cid & 31u)) & 1u);
-    m = mat_runtime(rec, c.ts[a], c.dur[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a], name, fs, rec.cid == api.malloc_cid);
+    const MatRow m = mat_runtime(rec, c.ts[a], c.dur[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a], name, fs,
+                                 rec.cid == api.malloc_cid);
     store_row(&mat[a], m);
     len[a] = row_length(m, ctx, sc);
+    count_row_stats(m, ctx, &rs);
   }
-  count_row_stats(m, i < n, ctx, sc);
+  flush_row_stats(rs, sc);
 }
 __global__ void k_mat_device(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const ktj_runtime_rec* r,
                              Table by_narrow, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  MatRow m;
-  m.meta = 0; m.name_id = 0;
-  if (i < n) {
+  RowStats rs;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t a = first + i;
     const ktj_device_rec rec = d[i];
     const ktj_runtime_rec* ksrc = nullptr;
     bool has_size = false;
     uint64_t size = 0;
-    if (rec.domain != KTJ_DOM_MEMSET && by_narrow.keys != nullptr) { /* RocprofActivity_inl.h:161-180 */
+    if (rec.domain != KTJ_DOM_MEMSET) { /* RocprofActivity_inl.h:161-180 */
       const uint32_t slot = table_find(by_narrow.keys, by_narrow.mask, narrow_corr_key(rec.id));
       if (slot != KTJ_NOSLOT) {
         const uint32_t ss = by_narrow.v1[slot], ks = by_narrow.v0[slot];
@@ -942,11 +993,13 @@ __global__ void k_mat_device(const ktj_device_rec* d, uint64_t n, Columns c, uin
         } else if (ks != 0) ksrc = &r[ks - 1u];
       }
     }
-    m = mat_device(rec, c.ts[a], c.dur[a], c.res[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a], ksrc, has_size, size);
+    const MatRow m = mat_device(rec, c.ts[a], c.dur[a], c.res[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a], ksrc,
+                                has_size, size);
     store_row(&mat[a], m);
     len[a] = row_length(m, ctx, sc);
+    count_row_stats(m, ctx, &rs);
   }
-  count_row_stats(m, i < n, ctx, sc);
+  flush_row_stats(rs, sc);
 }
 __global__ void k_gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -956,20 +1009,20 @@ __global__ void k_gather_len(const uint32_t* perm, const uint32_t* len, uint64_t
 hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc,
                             hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_mat_generic, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, ctx, mat, len, sc);
+  hipLaunchKernelGGL(k_mat_generic, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, ctx, mat, len, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, EmitCtx ctx,
                             MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_mat_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, ctx, mat,
+  hipLaunchKernelGGL(k_mat_runtime, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, ctx, mat,
                      len, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const ktj_runtime_rec* r,
                            Table by_narrow, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_mat_device, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, d, n, c, first, r, by_narrow,
+  hipLaunchKernelGGL(k_mat_device, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, d, n, c, first, r, by_narrow,
                      ctx, mat, len, sc);
   return KTJ_LAUNCH_CHECK();
 }

@@ -1,0 +1,144 @@
+"""Known-answer cases for the logger path.  Every expected string below was either observed from
+the real ChromeTraceLogger (built from the reference sources) or is a literal the reference's own
+tests assert; the source is named per case.  Used on the CPU against the oracle and on the GPU
+against the engine."""
+from kineto_amd import abi
+from stream_builder import B, StreamBuilder
+
+T = abi  # type constants live in abi as plain ints below
+CPU_OP, GPU_MEMCPY, KERNEL, RUNTIME = 0, 3, 5, 7
+
+
+def case_logger_events():
+    """Observed from the real logger: CPU op, linked runtime row with flow start, kernel with a name
+    that needs sanitising, orphan kernel with unprintable name, 'kernel' rename, blank metadata."""
+    b = StreamBuilder()
+    b.api([None] * 12 + ["hipLaunchKernel"], flow_start=[12])
+    b.add_generic("aten::mm", CPU_OP, B + 1234, B + 5678, 4242, 4243, id=7)
+    b.add_runtime(7, B + 2000, B + 3000, 12, 4242, 4243, kind=0)
+    b.add_extcorr(7, 7)
+    b.add_generic('void f<"q", a\\b>(int)\n', KERNEL, B + 4000, B + 4500, 0, 3, id=7, flow_id=7, flow_type=2)
+    b.add_generic("bad\x01name", KERNEL, B + 6000, B + 5997, 0, -5, id=99, flow_id=99, flow_type=2)
+    sch = b.schema([(None, abi.F_RAW, 1)])
+    b.add_generic("kernel", GPU_MEMCPY, B + 7000, B + 7100, 0, 3, id=0, schema=sch, values=[b.s("   ")])
+    expect = [
+        '"cat": "cpu_op",\n    "name": "aten::mm",\n    "pid": 4242,\n    "tid": 4243,\n    "ts": 1.234,\n    "dur": 4.444\n    ,\n    "args": {\n      "External id": 7\n    }',
+        '"External id": 7,"cid": 12, "correlation": 7',
+        '"ph": "s",\n    "id": 7,\n    "pid": 4242,\n    "tid": 4243,\n    "ts": 2.000,\n    "cat": "ac2g",\n    "name": "ac2g"\n    \n  },',
+        '"name": "void f<\\"q\\", a/b>(int)"',
+        '"name": "ac2g"\n    , "bp": "e"\n  },',
+        '"name": "unknown",\n    "pid": 0,\n    "tid": 5,\n    "ts": 6.000,\n    "dur": 0.000\n    \n  },\n  {\n    "ph": "f",\n    "id": 99,',
+        '"cat": "gpu_memcpy",\n    "name": "Kernel",\n    "pid": 0,\n    "tid": 3,\n    "ts": 7.000,\n    "dur": 0.100\n    \n  },',
+    ]
+    return b, expect
+
+
+def case_trace_span():
+    """Observed from the real logger (TraceSpan 'PyTorch Profiler', +1000..+900000, opCount 1, iter 0)."""
+    b = StreamBuilder(end_time=B + 900000)
+    b.add_span(B + 1000, B + 900000, 1, 0, "PyTorch Profiler")
+    expect = [
+        '"ph": "X",\n    "cat": "Trace",\n    "name": "PyTorch Profiler (0)",\n    "pid": "Spans",\n    "tid": "PyTorch Profiler",\n    "ts": 1.000,\n    "dur": 899.000\n    ,\n    "args": {\n      "Op count": 1\n    }\n  },',
+        '"ph": "M",\n    "name": "process_sort_index",\n    "ts": 1.000,\n    "pid": "Spans",\n    "tid": 0,\n    "args": {\n      "sort_index": 536870912\n    }',
+        '"s": "g",\n    "name": "Iteration Start: PyTorch Profiler",\n    "pid": "Traces",\n    "tid": "Trace PyTorch Profiler",\n    "ts": 1.000',
+        '"name": "Record Window End",\n    "pid": "",\n    "tid": "",\n    "ts": 900.000\n    \n  }\n  ],"traceName": "t.json" }',
+    ]
+    return b, expect
+
+
+def case_benchmark_cpu_op():
+    """benchmarks/json_output_benchmark.cpp:181-197 through the real logger: duplicate keys are
+    emitted as they are, the logger's own External id first."""
+    b = StreamBuilder()
+    sch = b.schema([("Sequence number", abi.F_I64, 1), ("Input Dims", abi.F_STR, 1), ("External id", abi.F_RAW, 1)])
+    b.add_generic("aten::conv2d", CPU_OP, B + 10, B + 20, 12345, 67890, id=2, schema=sch,
+                  values=[1, b.s("[[32, 64, 28, 28], [64, 64, 3, 3]]"), b.s("3")])
+    return b, ['"External id": 2,"Sequence number": 1, "Input Dims": "[[32, 64, 28, 28], [64, 64, 3, 3]]", "External id": 3']
+
+
+def case_typed_kernel_args():
+    """Observed from the real logger; key order is the reference's unordered_map order for keys
+    inserted as grid, block, registers per thread, shared memory, occupancy."""
+    b = StreamBuilder()
+    sch = b.schema([("occupancy", abi.F_F64, 1), ("registers per thread", abi.F_U64, 1), ("block", abi.F_I64_ARRAY, 3),
+                    ("shared memory", abi.F_I64, 1), ("grid", abi.F_I64_ARRAY, 3)])
+    b.add_generic("k1", KERNEL, B + 10, B + 20, 0, 1, id=1, schema=sch, values=[0.00003125, 64, 256, 1, 1, 163840, 128, 1, 1],
+                  flow_id=5, flow_type=2)
+    b.add_generic("k2", KERNEL, B + 30, B + 40, 0, 1, id=2, schema=sch, values=[0.4375, 64, 256, 1, 1, 163840, 128, 1, 1])
+    expect = [
+        '"occupancy": 3.125e-05, "registers per thread": 64, "block": [256, 1, 1], "shared memory": 163840, "grid": [128, 1, 1]',
+        '"occupancy": 0.4375, "registers per thread": 64',
+        '"ph": "f",\n    "id": 5,',
+    ]
+    return b, expect
+
+
+def case_typed_metadata_pins():
+    """Literals asserted by libkineto/test/TypedMetadataTest.cpp:164-178, 240 and
+    GenericTraceActivityMetadataTest.cpp:144-178 (strings pass through unescaped except for the
+    logger's later backslash/newline pass)."""
+    b = StreamBuilder()
+    sch = b.schema([("count", abi.F_I64, 1), ("ids", abi.F_I64_ARRAY, 2), ("label", abi.F_STR, 1), ("ratio", abi.F_F64, 1),
+                    ("enabled", abi.F_BOOL, 1), ("big", abi.F_U64, 1), ("raw", abi.F_RAW, 1), ("neg", abi.F_I64, 1),
+                    ("special", abi.F_STR, 1), ("nan", abi.F_F64, 1)])
+    b.add_generic("op", CPU_OP, B + 1, B + 2, 1, 2, id=0, schema=sch,
+                  values=[5, 1, 2, b.s("label"), 1.5, 1, 0xFFFFFFFFFFFFFFFF, b.s("[1, 2, 3]"), -7,
+                          b.s('quote " slash \\ newline\n'), float("nan")])
+    expect = ['"count": 5, "ids": [1, 2], "label": "label", "ratio": 1.5, "enabled": true, "big": 18446744073709551615, '
+              '"raw": [1, 2, 3], "neg": -7, "special": "quote " slash / newline", "nan": "nan"']
+    return b, expect
+
+
+def case_names():
+    """Observed from the real logger: UTF-8, TAB and DEL make the whole name 'unknown'; printable
+    punctuation is untouched; newlines vanish; quotes are escaped after backslashes became slashes."""
+    b = StreamBuilder()
+    names = [b"caf\xc3\xa9", b"tab\there", b"del\x7f", b"sp ace~!", b"nl\nonly\n", b'q""x\\\\']
+    for i, n in enumerate(names):
+        b.add_generic(n, CPU_OP, B + 10 * i, B + 10 * i + 5, 1, 1, id=0)
+    expect = ['"name": "unknown"', '"name": "sp ace~!"', '"name": "nlonly"', '"name": "q\\"\\"x//"']
+    return b, expect
+
+
+def case_resource_infos():
+    """libkineto/test/OutputJsonTest.cpp:154-179, 227-255: HOST_THREAD display name, escaping of quoted
+    resource names; RocmActivityProfilerTest.cpp:967-975: GPU labels and sort index."""
+    b = StreamBuilder()
+    b.add_resource_info(12345, 12345, 99, "worker", host_thread=True)
+    b.add_resource_info(-7, 3, 0, 'str"eam\\x')
+    b.add_device_info(3, 3 + 5000000, "python", "GPU 3")
+    b.add_overhead_info("CUPTI Overhead")
+    expect = ['"name": "thread_name",\n    "ts": 0.000,\n    "pid": 99,\n    "tid": 12345,\n    "args": {\n      "name": "thread 12345 (worker)"\n    }',
+              '"tid": 7,\n    "args": {\n      "name": "str\\"eam/x"\n    }',
+              '"name": "process_labels",\n    "ts": 0.000,\n    "pid": 3,\n    "tid": 0,\n    "args": {\n      "labels": "GPU 3"\n    }',
+              '"sort_index": 5000003', '"pid": -1,\n    "tid": 0,\n    "args": {\n      "sort_index": 16777226\n    }']
+    return b, expect
+
+
+def case_rocm_sync_trace():
+    """The 15-activity trace of libkineto/test/RocmActivityProfilerTest.cpp:315-397: names, counts and
+    resource ids (kernels on queue 1, copies on queue 2, no runtime row carries a stream)."""
+    b = StreamBuilder(window=(B, B + 300), end_time=B + 300)
+    b.api(["hipLaunchKernel", "hipMemcpy"], flow_start=[0, 1])
+    pid, tid = 4000, 4001
+    for i, (nm, s0, e0, cid) in enumerate([("op1", 20, 50, 1), ("op2", 30, 40, 2), ("op3", 100, 150, 3), ("op4", 160, 180, 4),
+                                           ("op5", 190, 210, 4)]):
+        b.add_generic(nm, CPU_OP, B + s0, B + e0, pid, tid, id=cid)
+    b.add_runtime(1, B + 33, B + 38, 0, pid, tid, kind=1)
+    b.add_runtime(2, B + 110, B + 120, 1, pid, tid, kind=2, size=1)
+    b.add_runtime(3, B + 130, B + 145, 0, pid, tid, kind=1)
+    b.add_runtime(4, B + 165, B + 175, 1, pid, tid, kind=2, size=1)
+    b.add_runtime(5, B + 195, B + 205, 0, pid, tid, kind=1)
+    b.add_device(1, B + 50, B + 70, domain=0, name="kernel", queue=1)
+    b.add_device(2, B + 140, B + 150, domain=1, op=2, queue=2)
+    b.add_device(3, B + 160, B + 220, domain=0, name="kernel", queue=1)
+    b.add_device(4, B + 230, B + 250, domain=1, op=3, queue=2)
+    b.add_device(5, B + 260, B + 280, domain=0, name="kernel", queue=1)
+    expect_counts = {'"name": "hipLaunchKernel"': 3, '"name": "Memcpy HtoD (Host -> Device)"': 1,
+                     '"name": "Memcpy DtoH (Device -> Host)"': 1, '"name": "Kernel"': 3, '"ph": "X"': 15,
+                     '"pid": 0,\n    "tid": 1,\n    "ts"': 6, '"pid": 0,\n    "tid": 2,\n    "ts"': 4}
+    return b, expect_counts
+
+
+SUBSTRING_CASES = [case_logger_events, case_trace_span, case_benchmark_cpu_op, case_typed_kernel_args,
+                   case_typed_metadata_pins, case_names, case_resource_infos]

@@ -1,0 +1,165 @@
+"""Hand-made ktj_stream objects for known-answer and edge-case tests (ctypes, no computation)."""
+import ctypes as C
+import struct
+
+from kineto_amd import abi
+
+B = abi.DEFAULT_BASE_TIME_NS
+
+
+class StreamBuilder:
+    def __init__(self, base=B, trace_name="t.json", host_name=None, window=(None, None), end_time=None):
+        self.base = base
+        self.trace_name = trace_name
+        self.meta = []
+        if host_name is not None:
+            self.meta.append(("host_name", '"%s"' % host_name))
+        self.strings = []
+        self.fields = []
+        self.schemas = []
+        self.args = []
+        self.cid_names = []
+        self.flow_start = []
+        self.malloc_cid = abi.KTJ_NONE
+        self.clock = abi.ClockModel(0, 0, 1.0, 0, 0, 0)
+        self.window = (base if window[0] is None else window[0], base + 10**12 if window[1] is None else window[1])
+        self.end_time = self.window[1] if end_time is None else end_time
+        self.generic, self.runtime, self.device, self.extcorr = [], [], [], []
+        self.device_infos, self.resource_infos, self.overhead_infos, self.spans = [], [], [], []
+        self._keep = []
+
+    # ---- dictionary / schemas ----
+    def s(self, text):
+        b = text if isinstance(text, bytes) else text.encode("latin1")
+        self.strings.append(b)
+        return len(self.strings) - 1
+
+    def schema(self, fields):
+        """fields: list of (key or None, type, count)"""
+        first = len(self.fields)
+        for key, typ, cnt in fields:
+            self.fields.append((abi.KTJ_NONE if key is None else self.s(key), typ, cnt))
+        self.schemas.append((first, len(fields)))
+        return len(self.schemas) - 1
+
+    def arg_slots(self, values):
+        off = len(self.args)
+        for v in values:
+            if isinstance(v, float):
+                v = struct.unpack("<Q", struct.pack("<d", v))[0]
+            self.args.append(v & 0xFFFFFFFFFFFFFFFF)
+        return off
+
+    def api(self, names, flow_start=(), malloc_cid=abi.KTJ_NONE):
+        self.cid_names = [abi.KTJ_NONE if n is None else self.s(n) for n in names]
+        self.flow_start = list(flow_start)
+        self.malloc_cid = malloc_cid
+
+    # ---- records ----
+    def add_generic(self, name, typ, start, end, device, resource, id=0, schema=None, values=(), flow_id=0,
+                    flow_type=0, flow_start=False, linked=None):
+        r = abi.GenericRec()
+        r.start_ns, r.end_ns, r.resource = start, end, resource
+        r.id, r.device = id, device
+        r.name_id = abi.KTJ_NONE if name is None else self.s(name)
+        r.type = typ
+        r.flow_id, r.flow_type = flow_id, flow_type
+        r.flags = (1 if flow_start else 0) | (2 if linked is not None else 0)
+        r.linked_corr = 0 if linked is None else linked
+        r.schema_id = abi.KTJ_NONE if schema is None else schema
+        r.args_off = self.arg_slots(values) if schema is not None else 0
+        self.generic.append(r)
+        return r
+
+    def add_runtime(self, id, begin, end, cid, pid, tid, kind=0, **kw):
+        r = abi.RuntimeRec()
+        r.id, r.begin, r.end, r.cid, r.pid, r.tid, r.kind = id, begin, end, cid, pid, tid, kind
+        if kind == 1:
+            g = kw.get("grid", (0, 0, 0)); w = kw.get("workgroup", (0, 0, 0))
+            for i in range(3):
+                r.u.kernel.grid[i] = g[i]; r.u.kernel.workgroup[i] = w[i]
+            r.u.kernel.group_segment_size = kw.get("lds", 0)
+            r.u.kernel.stream = kw.get("stream", 0)
+            r.u.kernel.kernel_name_id = abi.KTJ_NONE if kw.get("kernel_name") is None else self.s(kw["kernel_name"])
+        elif kind == 2:
+            r.u.copy.src, r.u.copy.dst = kw.get("src", 0), kw.get("dst", 0)
+            r.u.copy.size, r.u.copy.stream = kw.get("size", 0), kw.get("stream", 0)
+            r.u.copy.copy_kind = kw.get("copy_kind", 0)
+        elif kind == 3:
+            r.u.malloc_.ptr, r.u.malloc_.size = kw.get("ptr", 0), kw.get("size", 0)
+        self.runtime.append(r)
+        return r
+
+    def add_device(self, id, begin, end, domain=0, op=0, device=0, name=None, queue=0, stream=0, nbytes=0):
+        d = abi.DeviceRec()
+        d.id, d.begin, d.end, d.domain, d.op, d.device = id, begin, end, domain, op, device
+        d.name_id = abi.KTJ_NONE if name is None else self.s(name)
+        d.queue, d.stream, d.bytes = queue, stream, nbytes
+        self.device.append(d)
+        return d
+
+    def add_extcorr(self, corr, ext):
+        self.extcorr.append(abi.ExtCorrRec(corr, ext))
+
+    def add_device_info(self, id, sort_index, name, label, t=None):
+        self.device_infos.append(abi.DeviceInfo(id, sort_index, name.encode(), label.encode(), self.base if t is None else t))
+
+    def add_resource_info(self, id, sort_index, device_id, name, host_thread=False, t=None):
+        self.resource_infos.append(abi.ResourceInfo(id, sort_index, device_id, name.encode(), 1 if host_thread else 0, 0,
+                                                    self.base if t is None else t))
+
+    def add_overhead_info(self, name, t=None):
+        self.overhead_infos.append(abi.OverheadInfo(name.encode(), self.base if t is None else t))
+
+    def add_span(self, start, end, op_count, iteration, name, prefix=""):
+        self.spans.append(abi.TraceSpan(start, end, op_count, iteration, name.encode(), prefix.encode()))
+
+    # ---- assemble ----
+    def _arr(self, ctype, items):
+        a = (ctype * max(len(items), 1))(*items)
+        self._keep.append(a)
+        return a
+
+    def build(self):
+        st = abi.Stream()
+        st.base_time_ns = self.base
+        st.trace_name = self.trace_name.encode()
+        st.device_properties = b""
+        kv = []
+        for k, v in self.meta:
+            kv += [k.encode(), v.encode()]
+        st.meta_kv = self._arr(C.c_char_p, kv)
+        st.n_meta = len(self.meta)
+        blob = b"".join(self.strings)
+        offs = [0]
+        for x in self.strings:
+            offs.append(offs[-1] + len(x))
+        bb = C.create_string_buffer(blob, max(len(blob), 1))
+        self._keep.append(bb)
+        st.str_blob = C.cast(bb, C.c_void_p)
+        st.str_off = self._arr(C.c_uint64, offs)
+        st.n_strings = len(self.strings)
+        st.fields = self._arr(abi.Field, [abi.Field(*f) for f in self.fields])
+        st.n_fields = len(self.fields)
+        st.schemas = self._arr(abi.SchemaDesc, [abi.SchemaDesc(*x) for x in self.schemas])
+        st.n_schemas = len(self.schemas)
+        st.args = self._arr(C.c_uint64, self.args)
+        st.n_args = len(self.args)
+        st.cid_name_ids = self._arr(C.c_uint32, self.cid_names)
+        st.n_cids = len(self.cid_names)
+        st.flow_start_cids = self._arr(C.c_uint32, self.flow_start)
+        st.n_flow_start = len(self.flow_start)
+        st.malloc_cid = self.malloc_cid
+        st.clock = self.clock
+        st.window_start_ns, st.window_end_ns = self.window
+        st.end_time_ns = self.end_time
+        for name, ctype, items in (("generic", abi.GenericRec, self.generic), ("runtime", abi.RuntimeRec, self.runtime),
+                                   ("device", abi.DeviceRec, self.device), ("extcorr", abi.ExtCorrRec, self.extcorr),
+                                   ("device_infos", abi.DeviceInfo, self.device_infos),
+                                   ("resource_infos", abi.ResourceInfo, self.resource_infos),
+                                   ("overhead_infos", abi.OverheadInfo, self.overhead_infos),
+                                   ("spans", abi.TraceSpan, self.spans)):
+            setattr(st, name, self._arr(ctype, items))
+            setattr(st, "n_" + name, len(items))
+        self._keep.append(st)
+        return C.pointer(st)

@@ -67,3 +67,171 @@ def run_case(cfg, n, check_stages=True):
 def test_engine_matches_oracle(cfg, n):
     print(f"case config={cfg} n={n}", flush=True)
     run_case(cfg, n)
+
+
+def _engine_vs_oracle(sp, check_substrings=()):
+    import oracle_glue as og
+    from kineto_amd.engine import TraceEngine
+    ora = og.OracleRun(sp)
+    want = ora.output()
+    with TraceEngine(sp.contents.trace_name.decode(), device=0) as eng:
+        eng.submit_stream(sp)
+        eng.process()
+        got = eng.output()
+        st = eng.stats()
+    cnt = ora.counters()
+    ora.close()
+    if got != want:
+        i = _first_diff(got, want)
+        raise AssertionError(f"bytes differ at {i}:\nGOT : {got[max(0, i - 200):i + 120]!r}\nWANT: {want[max(0, i - 200):i + 120]!r}")
+    for sub in check_substrings:
+        assert sub.encode("latin1") in got
+    assert st.out_of_range_events == cnt["out_of_range"]
+    assert st.gpu_and_cpu_op_out_of_order == cnt["out_of_order"]
+    return got
+
+
+def test_known_answer_cases_on_gpu():
+    import kat_cases
+    for case in kat_cases.SUBSTRING_CASES:
+        print("case", case.__name__, flush=True)
+        b, expect = case()
+        _engine_vs_oracle(b.build(), expect)
+    b, counts = kat_cases.case_rocm_sync_trace()
+    got = _engine_vs_oracle(b.build()).decode("latin1")
+    for k, v in counts.items():
+        assert got.count(k) == v
+
+
+def test_join_edge_cases_on_gpu():
+    import test_join_bruteforce as tj
+    import inspect
+    # rebuild the hand-made stream of the CPU test and run it through the engine
+    src = inspect.getsource(tj.test_join_edge_cases).replace("compare(b.build())", "return b")
+    ns = {}
+    exec(src, {**tj.__dict__}, ns)
+    b = ns["test_join_edge_cases"]()
+    _engine_vs_oracle(b.build())
+
+
+def test_empty_and_tiny_streams_on_gpu():
+    from stream_builder import StreamBuilder, B
+    _engine_vs_oracle(StreamBuilder().build())
+    b = StreamBuilder()
+    b.add_generic(None, 0, B, B, 0, 0)          # no name, zero everything
+    _engine_vs_oracle(b.build())
+    b = StreamBuilder(window=(B + 10, B + 20))
+    b.api(["hipLaunchKernel"], flow_start=[0])
+    b.add_runtime(1, B, B + 5, 0, 1, 1, kind=1)  # everything filtered out by the window
+    b.add_device(1, B + 100, B + 200, name="k", queue=1)
+    _engine_vs_oracle(b.build())
+
+
+def test_process_is_repeatable_and_file_output(tmp_path):
+    import hashlib
+    import oracle_glue as og
+    from kineto_amd.engine import TraceEngine
+    path = str(tmp_path / "trace.json")
+    sp, release = abi.synth_stream(2, 5000, host_name="gpubox", trace_name=path)
+    ora = og.OracleRun(sp)
+    want = ora.output()
+    ora.close()
+    with TraceEngine(path, device=0, no_file=False) as eng:
+        eng.submit_stream(sp)
+        eng.process()
+        a = eng.output()
+        eng.process()
+        b = eng.output()
+        assert a == b == want
+        import os
+        assert os.path.exists(path + ".tmp") and not os.path.exists(path)
+        n = eng.finalize()
+        assert n == len(want)
+        assert not os.path.exists(path + ".tmp")
+        assert open(path, "rb").read() == want
+    release()
+
+
+def test_unwritable_sink_is_a_silent_noop():
+    """ChromeTraceLogger with a file it cannot open: every handler returns silently and only
+    finalizeTrace reports (output_json.cpp:485-505, 1067-1070)."""
+    from kineto_amd.engine import TraceEngine, EngineError
+    sp, release = abi.synth_stream(1, 100)
+    eng = TraceEngine("/nonexistent-dir/sub/trace.json", device=0, no_file=False)
+    eng.submit_stream(sp)        # no error
+    eng.process()                # no error, nothing done
+    with pytest.raises(EngineError) as ei:
+        eng.finalize()
+    assert "rc=-4" in str(ei.value)
+    eng.close()
+    release()
+
+
+def test_device_resident_submission():
+    """Records handed over as device pointers (zero copy) give the same document."""
+    import torch
+    import oracle_glue as og
+    from kineto_amd.engine import TraceEngine
+    sp, release = abi.synth_stream(3, 20000, host_name="gpubox")
+    s = sp.contents
+    ora = og.OracleRun(sp)
+    want = ora.output()
+    ora.close()
+    keep = []
+
+    def to_dev(ptr, n, size):
+        raw = C.string_at(C.cast(ptr, C.c_void_p), n * size)
+        t = torch.frombuffer(bytearray(raw), dtype=torch.uint8).cuda()
+        keep.append(t)
+        return t.data_ptr()
+
+    devptrs = {abi.REC_GENERIC: (to_dev(s.generic, s.n_generic, 64), s.n_generic),
+               abi.REC_RUNTIME: (to_dev(s.runtime, s.n_runtime, 96), s.n_runtime),
+               abi.REC_DEVICE: (to_dev(s.device, s.n_device, 64), s.n_device),
+               abi.REC_EXTCORR: (to_dev(s.extcorr, s.n_extcorr, 16), s.n_extcorr)}
+    torch.cuda.synchronize()
+    counts = (s.n_generic, s.n_runtime, s.n_device, s.n_extcorr)
+    s.n_generic = s.n_runtime = s.n_device = s.n_extcorr = 0   # submit_stream then sends no records
+    with TraceEngine(s.trace_name.decode(), device=0) as eng:
+        eng.submit_stream(sp)
+        for cls, (p, n) in devptrs.items():
+            assert eng.lib.ktj_submit_records_device(eng.h, cls, p, n) == 0
+        eng.process()
+        got = eng.output()
+    s.n_generic, s.n_runtime, s.n_device, s.n_extcorr = counts
+    release()
+    assert got == want
+
+
+@pytest.mark.parametrize("cfg", [3])
+def test_full_size_headline_config_digest(cfg):
+    """The headline configuration at its full size: the engine's document and the CPU checker's
+    must have the same length and the same BLAKE2 digest (hashed in place, chunk by chunk)."""
+    import hashlib
+    import oracle_glue as og
+    from kineto_amd.engine import TraceEngine
+    sp, release = abi.synth_stream(cfg, 0, host_name="gpubox")
+    with TraceEngine(sp.contents.trace_name.decode(), device=0) as eng:
+        eng.submit_stream(sp)
+        eng.process()
+        p, n = C.c_void_p(), C.c_uint64()
+        assert eng.lib.ktj_output_host(eng.h, C.byref(p), C.byref(n)) == 0
+        h1 = hashlib.blake2b()
+        view = (C.c_char * n.value).from_address(p.value)
+        mv = memoryview(view)
+        for off in range(0, n.value, 1 << 26):
+            h1.update(mv[off:off + (1 << 26)])
+        got_n = n.value
+    print("engine done", got_n, flush=True)
+    ora = og.OracleRun(sp)
+    p, n = C.c_void_p(), C.c_uint64()
+    ora.lib.ktj_oracle_output(ora.h, C.byref(p), C.byref(n))
+    h2 = hashlib.blake2b()
+    mv = memoryview((C.c_char * n.value).from_address(p.value))
+    for off in range(0, n.value, 1 << 26):
+        h2.update(mv[off:off + (1 << 26)])
+    want_n = n.value
+    ora.close()
+    release()
+    assert got_n == want_n
+    assert h1.hexdigest() == h2.hexdigest()
