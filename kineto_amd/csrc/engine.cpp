@@ -118,7 +118,7 @@ struct ktj_engine {
   DevBuf q_keys, q_stream, q_amb, dn_hash, dn_first, dn_dev, dn_key, dn_rank;
   DevBuf s_dev_k, s_dev_r, s_res_k, s_res_r;
   DevBuf keys_a, keys_b, vals_a, vals_b, hist, scan_tmp;
-  DevBuf mat, len, len_sorted, offs, out;
+  DevBuf mat, len, len_sorted, offs, out, tile_start;
   void* pinned_small = nullptr; size_t pinned_small_cap = 0;
   char* pinned_out = nullptr; size_t pinned_out_cap = 0;
   bool host_copy_valid = false;
@@ -206,7 +206,7 @@ void ktj_destroy(ktj_engine* e) {
                     &e->t_nr_v1, &e->q_keys, &e->q_stream, &e->q_amb, &e->dn_hash, &e->dn_first, &e->dn_dev,
                     &e->dn_key, &e->dn_rank, &e->s_dev_k, &e->s_dev_r, &e->s_res_k, &e->s_res_r, &e->keys_a,
                     &e->keys_b, &e->vals_a, &e->vals_b, &e->hist, &e->scan_tmp, &e->mat, &e->len, &e->len_sorted,
-                    &e->offs, &e->out};
+                    &e->offs, &e->out, &e->tile_start};
   for (DevBuf* b : bufs) b->release();
   e->str_blob.release(); e->str_off.release(); e->args.release();
   e->generic.owned.release(); e->runtime.owned.release(); e->devrows.owned.release(); e->extcorr.owned.release();
@@ -570,8 +570,11 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(hipMemcpyAsync(e->out.p, e->pinned_small, prefix.size(), hipMemcpyHostToDevice, st));
   HIPCHK(hipMemcpyAsync(e->out.as<char>() + prefix.size() + act_bytes, static_cast<char*>(e->pinned_small) + prefix.size(),
                         suffix.size(), hipMemcpyHostToDevice, st));
+  const uint32_t tile = emit_tile_bytes(act_bytes, e->scalars.n_valid);
+  HIPCHK(e->tile_start.ensure((emit_tile_count(e->prefix_len, act_bytes, tile) + 2) * 4));
   HIPCHK(hipEventRecord(e->ev[EV_EMIT_START], st));
-  HIPCHK(emit(mat, e->perm, e->offs.as<uint64_t>(), N, ctx, e->out.as<char>(), e->prefix_len, act_bytes, st));
+  HIPCHK(emit(mat, e->perm, e->offs.as<uint64_t>(), N, ctx, e->out.as<char>(), e->prefix_len, act_bytes, tile,
+              e->tile_start.as<uint32_t>(), st));
   HIPCHK(hipEventRecord(e->ev[EV_EMIT], st));
   HIPCHK(hipStreamSynchronize(st));
 

@@ -20,6 +20,14 @@
 
 #include "ktj_device.h"
 
+/* The writer must live in registers: everything that touches it is inlined into the kernel. */
+#define KTJ_FI __attribute__((always_inline))
+#if defined(__clang__)
+#define KTJ_NOUNROLL _Pragma("clang loop unroll(disable)")
+#else
+#define KTJ_NOUNROLL
+#endif
+
 #if defined(__HIP_DEVICE_COMPILE__)
 #define KTJ_POW10_QUALIFIER __device__
 #else
@@ -32,7 +40,7 @@ namespace ktj {
 /* ---------------------------------------------------------------------------------------- */
 /* integers                                                                                   */
 /* ---------------------------------------------------------------------------------------- */
-KTJ_HD inline int ndigits_u64(uint64_t v) {
+KTJ_HD KTJ_FI inline int ndigits_u64(uint64_t v) {
   int n = 1;
   if (v >= 10000000000ULL) { v /= 10000000000ULL; n += 10; }
   uint32_t x = (uint32_t)v; /* < 10^10 may exceed 32 bits */
@@ -43,7 +51,7 @@ KTJ_HD inline int ndigits_u64(uint64_t v) {
   return n;
 }
 
-KTJ_HD inline uint64_t mulhi64(uint64_t a, uint64_t b) {
+KTJ_HD KTJ_FI inline uint64_t mulhi64(uint64_t a, uint64_t b) {
 #if defined(__HIP_DEVICE_COMPILE__)
   return __umul64hi(a, b);
 #else
@@ -56,11 +64,11 @@ KTJ_HD inline uint64_t mulhi64(uint64_t a, uint64_t b) {
 /* returns digits (no trailing zeros) and decimal exponent so that v = digits * 10^exp10.     */
 /* Reproduces what fmt's "{}" (Dragonbox) prints: shortest, closest, ties to even.            */
 /* ---------------------------------------------------------------------------------------- */
-KTJ_HD inline int32_t floor_log2_pow10(int32_t e) { return (e * 1741647) >> 19; }
-KTJ_HD inline int32_t floor_log10_pow2(int32_t e) { return (e * 1262611) >> 22; }
-KTJ_HD inline int32_t floor_log10_3q_pow2(int32_t e) { return (e * 1262611 - 524031) >> 22; }
+KTJ_HD KTJ_FI inline int32_t floor_log2_pow10(int32_t e) { return (e * 1741647) >> 19; }
+KTJ_HD KTJ_FI inline int32_t floor_log10_pow2(int32_t e) { return (e * 1262611) >> 22; }
+KTJ_HD KTJ_FI inline int32_t floor_log10_3q_pow2(int32_t e) { return (e * 1262611 - 524031) >> 22; }
 
-KTJ_HD inline uint64_t round_to_odd(uint64_t ghi, uint64_t glo, uint64_t cp) {
+KTJ_HD KTJ_FI inline uint64_t round_to_odd(uint64_t ghi, uint64_t glo, uint64_t cp) {
   /* (cp * g) >> 128 with a sticky low bit; g = ghi:glo */
   uint64_t x_hi = mulhi64(cp, glo);
   uint64_t y_lo = cp * ghi;
@@ -71,7 +79,7 @@ KTJ_HD inline uint64_t round_to_odd(uint64_t ghi, uint64_t glo, uint64_t cp) {
   return y1 | (s_lo > 1 ? 1 : 0);
 }
 
-KTJ_HD inline void shortest_decimal(uint64_t bits, uint64_t* digits, int32_t* exp10) {
+KTJ_HD KTJ_FI inline void shortest_decimal(uint64_t bits, uint64_t* digits, int32_t* exp10) {
   const uint64_t frac = bits & 0x000FFFFFFFFFFFFFULL;
   const uint32_t bexp = (uint32_t)((bits >> 52) & 0x7FF);
   uint64_t c;
@@ -134,59 +142,13 @@ KTJ_HD inline void shortest_decimal(uint64_t bits, uint64_t* digits, int32_t* ex
   *exp10 = k;
 }
 
-/* fmt "{}" of a double into out (>= 32 bytes); returns the length.
- * Layout rule of fmt's write_float with default specs: fixed notation iff the scientific
- * exponent is in [-4, 16), else d[.ddd]e±XX with at least two exponent digits. */
-KTJ_HD inline int format_double(uint64_t bits, char* out) {
-  int n = 0;
-  const bool neg = (bits >> 63) != 0;
-  const uint64_t mag = bits & 0x7FFFFFFFFFFFFFFFULL;
-  if (neg) out[n++] = '-';
-  if (mag >= 0x7FF0000000000000ULL) { /* fmt prints "inf" / "nan" */
-    const bool is_nan = mag > 0x7FF0000000000000ULL;
-    out[n++] = is_nan ? 'n' : 'i';
-    out[n++] = is_nan ? 'a' : 'n';
-    out[n++] = is_nan ? 'n' : 'f';
-    return n;
-  }
-  if (mag == 0) { out[n++] = '0'; return n; }
-  uint64_t sig;
-  int32_t k;
-  shortest_decimal(mag, &sig, &k);
-  const int nd = ndigits_u64(sig);
-  const int E = k + nd - 1;
-  char d[20];
-  { uint64_t t = sig; for (int i = nd - 1; i >= 0; --i) { d[i] = (char)('0' + (int)(t % 10)); t /= 10; } }
-  if (E >= -4 && E < 16) {
-    if (E >= 0) {
-      int i = 0;
-      for (; i <= E; ++i) out[n++] = i < nd ? d[i] : '0';
-      if (nd > E + 1) { out[n++] = '.'; for (; i < nd; ++i) out[n++] = d[i]; }
-    } else {
-      out[n++] = '0'; out[n++] = '.';
-      for (int i = 0; i < -E - 1; ++i) out[n++] = '0';
-      for (int i = 0; i < nd; ++i) out[n++] = d[i];
-    }
-  } else {
-    out[n++] = d[0];
-    if (nd > 1) { out[n++] = '.'; for (int i = 1; i < nd; ++i) out[n++] = d[i]; }
-    out[n++] = 'e';
-    int a = E;
-    if (a < 0) { out[n++] = '-'; a = -a; } else out[n++] = '+';
-    if (a >= 100) { out[n++] = (char)('0' + a / 100); a %= 100; }
-    out[n++] = (char)('0' + a / 10);
-    out[n++] = (char)('0' + a % 10);
-  }
-  return n;
-}
-
 /* ---------------------------------------------------------------------------------------- */
 /* clock conversion: (int64)((double)(t - t0_approx) * (long double)scale) + t0, exactly as    */
 /* x87 extended precision computes it (libkineto/src/ApproximateClock.cpp:83-90): the exact    */
 /* 106-bit product of two 53-bit significands is rounded to 64 bits (nearest even) and the     */
 /* result truncated toward zero.                                                               */
 /* ---------------------------------------------------------------------------------------- */
-KTJ_HD inline int64_t convert_timestamp(uint64_t t, uint64_t t0_approx, int64_t t0, uint64_t scale_bits) {
+KTJ_HD KTJ_FI inline int64_t convert_timestamp(uint64_t t, uint64_t t0_approx, int64_t t0, uint64_t scale_bits) {
   const int64_t ta = (int64_t)t, t0a = (int64_t)t0_approx;
   if (!(ta > t0a)) return 0;
   const uint64_t dt = (uint64_t)(ta - t0a); /* > 0 */
@@ -225,65 +187,49 @@ KTJ_HD inline int64_t convert_timestamp(uint64_t t, uint64_t t0_approx, int64_t 
 }
 
 /* ---------------------------------------------------------------------------------------- */
-/* constant strings                                                                            */
+/* constant strings: packed at compile time into 8-byte little-endian words so that the emit   */
+/* kernel appends them as immediates (no loads) and the size pass adds a constant.             */
 /* ---------------------------------------------------------------------------------------- */
-struct Lit { const char* p; uint32_t n; };
-#define KTJ_LIT(s) ::ktj::Lit{s, (uint32_t)(sizeof(s) - 1)}
-
-/* libkineto/include/ActivityType.h:80-111 */
-KTJ_HD inline Lit category_name(uint32_t type) {
-  switch (type) {
-    case 0: return KTJ_LIT("cpu_op");
-    case 1: return KTJ_LIT("user_annotation");
-    case 2: return KTJ_LIT("gpu_user_annotation");
-    case 3: return KTJ_LIT("gpu_memcpy");
-    case 4: return KTJ_LIT("gpu_memset");
-    case 5: return KTJ_LIT("kernel");
-    case 6: return KTJ_LIT("external_correlation");
-    case 7: return KTJ_LIT("cuda_runtime");
-    case 8: return KTJ_LIT("cuda_driver");
-    case 9: return KTJ_LIT("cpu_instant_event");
-    case 10: return KTJ_LIT("python_function");
-    case 11: return KTJ_LIT("overhead");
-    case 12: return KTJ_LIT("mtia_runtime");
-    case 13: return KTJ_LIT("mtia_ccp_events");
-    case 14: return KTJ_LIT("mtia_insight");
-    case 15: return KTJ_LIT("cuda_sync");
-    case 16: return KTJ_LIT("cuda_event");
-    case 17: return KTJ_LIT("mtia_counters");
-    case 18: return KTJ_LIT("glow_runtime");
-    case 19: return KTJ_LIT("cuda_profiler_range");
-    case 20: return KTJ_LIT("hpu_op");
-    case 21: return KTJ_LIT("xpu_runtime");
-    case 22: return KTJ_LIT("xpu_driver");
-    case 23: return KTJ_LIT("collective_comm");
-    case 24: return KTJ_LIT("privateuse1_runtime");
-    case 25: return KTJ_LIT("privateuse1_driver");
-    case 26: return KTJ_LIT("xpu_scope_profiler");
-    case 27: return KTJ_LIT("xpu_sync");
-    case 28: return KTJ_LIT("hardware_counters");
-    default: return KTJ_LIT("ENUM_COUNT");
-  }
+template <unsigned N> struct PackedLit {
+  uint64_t w[(N + 7) / 8 ? (N + 7) / 8 : 1];
+};
+template <unsigned M> constexpr PackedLit<M - 1> pack_lit(const char (&s)[M]) {
+  PackedLit<M - 1> p{};
+  for (unsigned i = 0; i < (M - 1 + 7) / 8; ++i) p.w[i] = 0;
+  for (unsigned i = 0; i + 1 < M; ++i) p.w[i / 8] |= (uint64_t)(unsigned char)s[i] << (8 * (i % 8));
+  return p;
 }
+#define KTJ_PUT(w, s)                                   \
+  do {                                                  \
+    constexpr auto ktj_lit_ = ::ktj::pack_lit(s);       \
+    (w).lit(ktj_lit_);                                  \
+  } while (0)
 
-/* libkineto/src/RocprofActivity_inl.h:50-94, 98-127 */
-KTJ_HD inline Lit memcpy_name(uint32_t op) {
-  switch (op) {
-    case KTJ_COPY_H2H: return KTJ_LIT("Memcpy HtoH (Host -> Host)");
-    case KTJ_COPY_H2D: return KTJ_LIT("Memcpy HtoD (Host -> Device)");
-    case KTJ_COPY_D2H: return KTJ_LIT("Memcpy DtoH (Device -> Host)");
-    case KTJ_COPY_D2D: return KTJ_LIT("Memcpy DtoD (Device -> Device)");
-    default: return KTJ_LIT("Memcpy <unknown> (? -> ?)");
-  }
+/* ---------------------------------------------------------------------------------------- */
+/* decimal digits as packed ASCII                                                             */
+/* ---------------------------------------------------------------------------------------- */
+/* x < 10000 → its four digits as ASCII, most significant digit in the lowest byte */
+KTJ_HD KTJ_FI inline uint32_t ascii4(uint32_t x) {
+  const uint32_t hi = (x * 5243u) >> 19; /* x / 100 */
+  const uint32_t lo = x - hi * 100u;
+  const uint32_t h = (hi * 103u) >> 10, l = (lo * 103u) >> 10; /* / 10 */
+  return (h | ((hi - h * 10u) << 8) | (l << 16) | ((lo - l * 10u) << 24)) + 0x30303030u;
 }
-KTJ_HD inline Lit copy_kind_string(uint32_t op) {
-  switch (op) {
-    case KTJ_COPY_H2H: return KTJ_LIT("HtoH");
-    case KTJ_COPY_H2D: return KTJ_LIT("HtoD");
-    case KTJ_COPY_D2H: return KTJ_LIT("DtoH");
-    case KTJ_COPY_D2D: return KTJ_LIT("DtoD");
-    default: return KTJ_LIT("<unknown>");
-  }
+/* x < 10^8 → eight ASCII digits, most significant first (lowest byte) */
+KTJ_HD KTJ_FI inline uint64_t ascii8(uint32_t x) {
+  const uint32_t hi = x / 10000u;
+  const uint32_t lo = x - hi * 10000u;
+  return (uint64_t)ascii4(hi) | ((uint64_t)ascii4(lo) << 32);
+}
+/* number of leading '0' characters of an ascii8 word, at most 7 */
+KTJ_HD KTJ_FI inline uint32_t leading_zero_chars(uint64_t a) {
+  const uint64_t d = a ^ 0x3030303030303030ULL;
+  if (d == 0) return 7;
+#if defined(__HIP_DEVICE_COMPILE__)
+  return (uint32_t)(__ffsll((long long)d) - 1) >> 3;
+#else
+  return (uint32_t)__builtin_ctzll(d) >> 3;
+#endif
 }
 
 /* ---------------------------------------------------------------------------------------- */
@@ -292,66 +238,135 @@ KTJ_HD inline Lit copy_kind_string(uint32_t op) {
 /* Pass A: exact byte length. */
 struct CountWriter {
   uint64_t n = 0;
-  KTJ_HD void ch(char) { ++n; }
-  KTJ_HD void lit(Lit l) { n += l.n; }
-  KTJ_HD void local(const char*, int len) { n += (uint32_t)len; }
-  KTJ_HD void dec(uint64_t v) { n += (uint32_t)ndigits_u64(v); }
-  KTJ_HD void dec3(uint32_t) { n += 3; }
-  KTJ_HD void hex(uint64_t v) { int d = 1; while (v >>= 4) ++d; n += (uint32_t)d; }
-  KTJ_HD void str(const char*, uint64_t len) { n += len; }
+  KTJ_HD KTJ_FI void ch(char) { ++n; }
+  template <unsigned N> KTJ_HD KTJ_FI void lit(const PackedLit<N>&) { n += N; }
+  KTJ_HD KTJ_FI void dec(uint64_t v) { n += (uint32_t)ndigits_u64(v); }
+  KTJ_HD KTJ_FI void dec3(uint32_t) { n += 3; }
+  KTJ_HD KTJ_FI void str(const char*, uint64_t len) { n += len; }
+  /* a number that is printed more than once is prepared once */
+  typedef uint32_t Prepared;
+  KTJ_HD KTJ_FI static Prepared prepare(uint64_t v) { return (uint32_t)ndigits_u64(v); }
+  KTJ_HD KTJ_FI void num(Prepared len) { n += len; }
 };
 
-/* Pass B: bytes into one tile of the output.  `pos` is relative to the tile's first byte and may
- * lie outside [0, tile): everything is clipped.  Dictionary strings are not copied here but
- * queued as copy jobs that the whole workgroup executes afterwards with wide lanes. */
+/* A decimal number rendered once and appended several times (pid, tid and ts appear in the
+ * complete event and again in the flow event). */
+struct Num {
+  uint64_t word;  /* up to 8 ASCII digits, first digit in the lowest byte */
+  uint32_t len;   /* 1..8, or 0 when the value needs more than 8 digits */
+  uint64_t value;
+};
+KTJ_HD KTJ_FI inline Num make_num(uint64_t v) {
+  Num n;
+  n.value = v;
+  if (__builtin_expect(v < 100000000ULL, 1)) {
+    const uint64_t a = ascii8((uint32_t)v);
+    const uint32_t z = leading_zero_chars(a);
+    n.word = a >> (8 * z);
+    n.len = 8 - z;
+  } else { n.word = 0; n.len = 0; }
+  return n;
+}
+
+/* Pass B: bytes into one tile of the output, held in LDS.
+ *
+ * Coordinates are tile-local: byte L of the buffer is byte (tile origin + L) of the document and
+ * the buffer covers L in [0, size); an activity that straddles a tile boundary is formatted by
+ * both tiles and everything outside the buffer is dropped.  Bytes are gathered in a 64-bit
+ * accumulator and leave as aligned 8-byte OR operations into the zero-filled tile: neighbouring
+ * activities and strings share boundary words, and OR-ing zeros into their bytes leaves them
+ * alone, so the writer needs no ownership bookkeeping.  Dictionary strings are not copied here
+ * but queued as copy jobs that whole wavefronts execute afterwards. */
 struct CopyJob { const char* src; int32_t dst; uint32_t len; };
 
 struct TileWriter {
-  char* buf;
-  int32_t pos;
-  int32_t tile;
+  char* buf;          /* 8-byte aligned, zero-filled, `size` bytes */
+  uint32_t size;      /* multiple of 8 */
   CopyJob* jobs;
   uint32_t* n_jobs;
   uint32_t max_jobs;
+  /* accumulator */
+  uint64_t acc;
+  int32_t wpos;       /* tile-local position of acc's byte 0; multiple of 8 */
+  uint32_t fill;      /* bytes gathered in acc, 0..7 */
 
-  KTJ_HD void put(int32_t p, char c) { if ((uint32_t)p < (uint32_t)tile) buf[p] = c; }
-  KTJ_HD void ch(char c) { put(pos, c); ++pos; }
-  KTJ_HD void copy_clipped(const char* s, uint32_t n) {
-    int32_t b = pos < 0 ? -pos : 0;
-    int64_t room = (int64_t)tile - pos;
-    int32_t e = (int64_t)n < room ? (int32_t)n : (int32_t)(room < 0 ? 0 : room);
-    for (int32_t i = b; i < e; ++i) buf[pos + i] = s[i];
+  KTJ_HD KTJ_FI void begin(int32_t pos) {
+    wpos = pos & ~7;
+    fill = (uint32_t)(pos - wpos);
+    acc = 0;
   }
-  KTJ_HD void lit(Lit l) { copy_clipped(l.p, l.n); pos += (int32_t)l.n; }
-  KTJ_HD void local(const char* s, int len) { copy_clipped(s, (uint32_t)len); pos += len; }
-  KTJ_HD void dec(uint64_t v) {
-    const int nd = ndigits_u64(v);
-    int32_t p = pos + nd - 1;
-    if (v >> 32) {
-      for (int i = 0; i < nd; ++i, --p) { const uint64_t q = v / 10; put(p, (char)('0' + (int)(v - q * 10))); v = q; }
-    } else {
-      uint32_t x = (uint32_t)v;
-      for (int i = 0; i < nd; ++i, --p) { const uint32_t q = x / 10; put(p, (char)('0' + (int)(x - q * 10))); x = q; }
+  KTJ_HD KTJ_FI int32_t position() const { return wpos + (int32_t)fill; }
+  KTJ_HD KTJ_FI void or_word() {
+    if ((uint32_t)wpos < size) {
+#if defined(__HIP_DEVICE_COMPILE__)
+      __hip_atomic_fetch_or(reinterpret_cast<unsigned long long*>(buf + wpos), (unsigned long long)acc, __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_WORKGROUP);
+#else
+      *reinterpret_cast<uint64_t*>(buf + wpos) |= acc;
+#endif
     }
-    pos += nd;
   }
-  KTJ_HD void dec3(uint32_t x) { /* {:03} of 0..999 */
-    put(pos + 2, (char)('0' + x % 10)); x /= 10;
-    put(pos + 1, (char)('0' + x % 10)); x /= 10;
-    put(pos, (char)('0' + x));
-    pos += 3;
+  KTJ_HD KTJ_FI void end() { if (fill) or_word(); }
+  /* append the n (0..8) low bytes of v; bytes above n must be zero */
+  KTJ_HD KTJ_FI void append(uint64_t v, uint32_t n) {
+    acc |= v << (8 * fill);
+    const uint32_t total = fill + n;
+    if (total >= 8) {
+      or_word();
+      wpos += 8;
+      const uint32_t rest = total - 8;           /* bytes of v still unwritten: its top `rest` of n */
+      acc = rest ? v >> (8 * (n - rest)) : 0;
+      fill = rest;
+    } else fill = total;
   }
-  KTJ_HD void hex(uint64_t v) {
-    int nd = 1; { uint64_t t = v; while (t >>= 4) ++nd; }
-    int32_t p = pos + nd - 1;
-    for (int i = 0; i < nd; ++i, --p) { const uint32_t d = (uint32_t)(v & 15); put(p, (char)(d < 10 ? '0' + d : 'a' + d - 10)); v >>= 4; }
-    pos += nd;
+  KTJ_HD KTJ_FI void ch(char c) { append((uint64_t)(unsigned char)c, 1); }
+  template <unsigned N> KTJ_HD KTJ_FI void lit(const PackedLit<N>& l) {
+    for (unsigned i = 0; i < N / 8; ++i) append(l.w[i], 8);
+    if (N % 8) append(l.w[N / 8], N % 8);
   }
-  KTJ_HD void str(const char* src, uint64_t len) {
+  KTJ_HD KTJ_FI void dec_wide(uint64_t v) { /* more than 8 digits: up to three 8-digit groups */
+    const uint64_t top = v / 10000000000000000ULL;
+    const uint64_t rest = v - top * 10000000000000000ULL;
+    const uint64_t mid = rest / 100000000ULL;
+    const uint32_t low = (uint32_t)(rest - mid * 100000000ULL);
+    uint64_t a0 = 0, a1;
+    uint32_t n0 = 0, n1;
+    if (top) {
+      a0 = ascii8((uint32_t)top);
+      const uint32_t z = leading_zero_chars(a0);
+      a0 >>= 8 * z; n0 = 8 - z;
+      a1 = ascii8((uint32_t)mid); n1 = 8;
+    } else {
+      a1 = ascii8((uint32_t)mid);
+      const uint32_t z = leading_zero_chars(a1);
+      a1 >>= 8 * z; n1 = 8 - z;
+    }
+    append(a0, n0);
+    append(a1, n1);
+    append(ascii8(low), 8);
+  }
+  KTJ_HD KTJ_FI void dec(uint64_t v) {
+    if (__builtin_expect(v < 100000000ULL, 1)) {
+      const uint64_t a = ascii8((uint32_t)v);
+      const uint32_t z = leading_zero_chars(a);
+      append(a >> (8 * z), 8 - z);
+    } else dec_wide(v);
+  }
+  typedef Num Prepared;
+  KTJ_HD KTJ_FI static Prepared prepare(uint64_t v) { return make_num(v); }
+  KTJ_HD KTJ_FI void num(const Num& n) {
+    if (__builtin_expect(n.len != 0, 1)) append(n.word, n.len); else dec_wide(n.value);
+  }
+  KTJ_HD KTJ_FI void dec3(uint32_t x) { /* {:03} of 0..999 */
+    append((uint64_t)(ascii4(x) >> 8), 3);
+  }
+  KTJ_HD KTJ_FI void str(const char* src, uint64_t len) {
     if (len == 0) return;
-    int64_t b = pos < 0 ? -(int64_t)pos : 0;
-    int64_t room = (int64_t)tile - pos;
-    int64_t e = (int64_t)len < room ? (int64_t)len : (room < 0 ? 0 : room);
+    end(); /* bytes gathered so far */
+    const int64_t pos = position();
+    int64_t b = pos < 0 ? -pos : 0;
+    int64_t e = (int64_t)size - pos;
+    if (e > (int64_t)len) e = (int64_t)len;
     if (b < e) {
       uint32_t slot;
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -363,51 +378,195 @@ struct TileWriter {
         jobs[slot].src = src + b;
         jobs[slot].dst = (int32_t)(pos + b);
         jobs[slot].len = (uint32_t)(e - b);
-      } else { /* queue full: copy here */
+      } else { /* queue full: copy here (bytes of a zero-filled region nobody else writes) */
+        KTJ_NOUNROLL
         for (int64_t i = b; i < e; ++i) buf[pos + i] = src[i];
       }
     }
-    pos += (int32_t)len;
+    begin((int32_t)(pos + (int64_t)len));
   }
 };
 
 /* ---------------------------------------------------------------------------------------- */
 /* pieces                                                                                      */
 /* ---------------------------------------------------------------------------------------- */
-template <class W> KTJ_HD inline void put_i64(W& w, int64_t v) {
+template <class W> KTJ_HD KTJ_FI inline void put_i64(W& w, int64_t v) {
   if (v < 0) { w.ch('-'); w.dec(0ULL - (uint64_t)v); } else w.dec((uint64_t)v);
 }
 /* fmtTs: "{}.{:03}" of ns/1000, ns%1000 for ns >= 0 (libkineto/src/output_json.cpp:124-126) */
-template <class W> KTJ_HD inline void put_ts(W& w, int64_t ns) {
+template <class W> KTJ_HD KTJ_FI inline void put_ts(W& w, int64_t ns) {
   const uint64_t u = (uint64_t)ns;
-  const uint64_t us = u / 1000;
-  w.dec(us);
-  w.ch('.');
-  w.dec3((uint32_t)(u - us * 1000));
+  if ((u >> 32) == 0) {
+    const uint32_t x = (uint32_t)u, us = x / 1000u;
+    w.dec(us);
+    w.ch('.');
+    w.dec3(x - us * 1000u);
+  } else {
+    const uint64_t us = u / 1000;
+    w.dec(us);
+    w.ch('.');
+    w.dec3((uint32_t)(u - us * 1000));
+  }
 }
-template <class W> KTJ_HD inline void put_f64(W& w, uint64_t bits) { /* TypedMetadataJson.h:172-178 */
-  char tmp[32];
-  const int n = format_double(bits, tmp);
-  const bool finite = (bits & 0x7FF0000000000000ULL) != 0x7FF0000000000000ULL;
-  if (!finite) w.ch('"');
-  w.local(tmp, n);
-  if (!finite) w.ch('"');
+template <class W> KTJ_HD KTJ_FI inline void put_hex(W& w, uint64_t v) { /* fmt "{}" of a pointer, after "0x" */
+  int nd = 1;
+  { uint64_t t = v; while (t >>= 4) ++nd; }
+  KTJ_NOUNROLL
+  for (int i = nd - 1; i >= 0; --i) {
+    const uint32_t d = (uint32_t)(v >> (4 * i)) & 15u;
+    w.ch((char)(d < 10 ? '0' + d : 'a' + d - 10));
+  }
 }
-template <class W> KTJ_HD inline void put_arg_string(W& w, const DictViews& d, uint32_t id) {
+/* fmt "{}" of a double (TypedMetadataJson.h:172-178): shortest digits; fixed notation iff the
+ * scientific exponent is in [-4, 16), else d[.ddd]e±XX; non-finite values are quoted */
+KTJ_HD KTJ_FI inline char digit_of(uint64_t p0, uint64_t p1, uint64_t p2, int j) {
+  const uint64_t word = j < 8 ? p0 : (j < 16 ? p1 : p2);
+  return (char)(word >> (8 * (j & 7)));
+}
+template <class W> KTJ_HD KTJ_FI inline void put_f64(W& w, uint64_t bits) {
+  const bool neg = (bits >> 63) != 0;
+  const uint64_t mag = bits & 0x7FFFFFFFFFFFFFFFULL;
+  if (mag >= 0x7FF0000000000000ULL) {
+    w.ch('"');
+    if (neg) w.ch('-');
+    if (mag > 0x7FF0000000000000ULL) KTJ_PUT(w, "nan"); else KTJ_PUT(w, "inf");
+    w.ch('"');
+    return;
+  }
+  if (neg) w.ch('-');
+  if (mag == 0) { w.ch('0'); return; }
+  uint64_t sig;
+  int32_t k;
+  shortest_decimal(mag, &sig, &k);
+  const int nd = ndigits_u64(sig);
+  const int E = k + nd - 1;
+  /* digits as up to three ascii8 words, left-aligned: digit i (0 = most significant) */
+  uint64_t p0, p1, p2;
+  {
+    const uint64_t top = sig / 10000000000000000ULL;            /* digits 17.. */
+    const uint64_t rest = sig - top * 10000000000000000ULL;
+    const uint64_t mid = rest / 100000000ULL;
+    p0 = ascii8((uint32_t)top); p1 = ascii8((uint32_t)mid); p2 = ascii8((uint32_t)(rest - mid * 100000000ULL));
+  }
+  const int lead = 24 - nd; /* leading zero characters of the 24-character string p0 p1 p2 */
+#define digit(i) ::ktj::digit_of(p0, p1, p2, (i) + lead)
+  if (E >= -4 && E < 16) {
+    if (E >= 0) {
+      int i = 0;
+      KTJ_NOUNROLL
+      for (; i <= E; ++i) w.ch(i < nd ? digit(i) : '0');
+      if (nd > E + 1) {
+        w.ch('.');
+        KTJ_NOUNROLL
+        for (; i < nd; ++i) w.ch(digit(i));
+      }
+    } else {
+      w.ch('0'); w.ch('.');
+      KTJ_NOUNROLL
+      for (int i = 0; i < -E - 1; ++i) w.ch('0');
+      KTJ_NOUNROLL
+      for (int i = 0; i < nd; ++i) w.ch(digit(i));
+    }
+  } else {
+    w.ch(digit(0));
+    if (nd > 1) {
+      w.ch('.');
+      KTJ_NOUNROLL
+      for (int i = 1; i < nd; ++i) w.ch(digit(i));
+    }
+    w.ch('e');
+    int a = E;
+    if (a < 0) { w.ch('-'); a = -a; } else w.ch('+');
+    if (a >= 100) { w.ch((char)('0' + a / 100)); a %= 100; }
+    w.ch((char)('0' + a / 10));
+    w.ch((char)('0' + a % 10));
+  }
+#undef digit
+}
+/* same text into a caller buffer (>= 32 bytes); used by host-side checks */
+struct BufferWriter {
+  char* p; int n = 0;
+  KTJ_HD KTJ_FI void ch(char c) { p[n++] = c; }
+  template <unsigned N> KTJ_HD KTJ_FI void lit(const PackedLit<N>& l) { for (unsigned i = 0; i < N; ++i) p[n++] = (char)(l.w[i / 8] >> (8 * (i % 8))); }
+};
+KTJ_HD KTJ_FI inline int format_double(uint64_t bits, char* out) {
+  BufferWriter b{out};
+  put_f64(b, bits);
+  /* put_f64 quotes non-finite values; the bare text is wanted here */
+  if (b.n && out[0] == '"') { for (int i = 1; i + 1 < b.n; ++i) out[i - 1] = out[i]; b.n -= 2; }
+  return b.n;
+}
+
+template <class W> KTJ_HD KTJ_FI inline void put_arg_string(W& w, const DictViews& d, uint32_t id) {
   if (id < d.n) w.str(d.arg_blob + d.arg_off[id], d.arg_off[id + 1] - d.arg_off[id]);
 }
-template <class W> KTJ_HD inline void put_array3(W& w, uint64_t a, uint64_t b, uint64_t c) {
-  w.ch('['); put_i64(w, (int64_t)a); w.lit(KTJ_LIT(", ")); put_i64(w, (int64_t)b); w.lit(KTJ_LIT(", "));
+template <class W> KTJ_HD KTJ_FI inline void put_array3(W& w, uint64_t a, uint64_t b, uint64_t c) {
+  w.ch('['); put_i64(w, (int64_t)a); KTJ_PUT(w, ", "); put_i64(w, (int64_t)b); KTJ_PUT(w, ", ");
   put_i64(w, (int64_t)c); w.ch(']');
 }
 
-KTJ_HD inline int64_t sanitize_tid(int64_t tid) { /* output_json.cpp:114-121 */
+KTJ_HD KTJ_FI inline int64_t sanitize_tid(int64_t tid) { /* output_json.cpp:114-121 */
   if (tid == (int64_t)0x8000000000000000ULL) return 0;
   return tid < 0 ? -tid : tid;
 }
 
+/* libkineto/include/ActivityType.h:80-111 */
+template <class W> KTJ_HD KTJ_FI inline void put_category(W& w, uint32_t type) {
+  switch (type) {
+    case 0: KTJ_PUT(w, "cpu_op"); break;
+    case 1: KTJ_PUT(w, "user_annotation"); break;
+    case 2: KTJ_PUT(w, "gpu_user_annotation"); break;
+    case 3: KTJ_PUT(w, "gpu_memcpy"); break;
+    case 4: KTJ_PUT(w, "gpu_memset"); break;
+    case 5: KTJ_PUT(w, "kernel"); break;
+    case 6: KTJ_PUT(w, "external_correlation"); break;
+    case 7: KTJ_PUT(w, "cuda_runtime"); break;
+    case 8: KTJ_PUT(w, "cuda_driver"); break;
+    case 9: KTJ_PUT(w, "cpu_instant_event"); break;
+    case 10: KTJ_PUT(w, "python_function"); break;
+    case 11: KTJ_PUT(w, "overhead"); break;
+    case 12: KTJ_PUT(w, "mtia_runtime"); break;
+    case 13: KTJ_PUT(w, "mtia_ccp_events"); break;
+    case 14: KTJ_PUT(w, "mtia_insight"); break;
+    case 15: KTJ_PUT(w, "cuda_sync"); break;
+    case 16: KTJ_PUT(w, "cuda_event"); break;
+    case 17: KTJ_PUT(w, "mtia_counters"); break;
+    case 18: KTJ_PUT(w, "glow_runtime"); break;
+    case 19: KTJ_PUT(w, "cuda_profiler_range"); break;
+    case 20: KTJ_PUT(w, "hpu_op"); break;
+    case 21: KTJ_PUT(w, "xpu_runtime"); break;
+    case 22: KTJ_PUT(w, "xpu_driver"); break;
+    case 23: KTJ_PUT(w, "collective_comm"); break;
+    case 24: KTJ_PUT(w, "privateuse1_runtime"); break;
+    case 25: KTJ_PUT(w, "privateuse1_driver"); break;
+    case 26: KTJ_PUT(w, "xpu_scope_profiler"); break;
+    case 27: KTJ_PUT(w, "xpu_sync"); break;
+    case 28: KTJ_PUT(w, "hardware_counters"); break;
+    default: KTJ_PUT(w, "ENUM_COUNT"); break;
+  }
+}
+/* libkineto/src/RocprofActivity_inl.h:50-94, 98-127 */
+template <class W> KTJ_HD KTJ_FI inline void put_memcpy_name(W& w, uint32_t op) {
+  switch (op) {
+    case KTJ_COPY_H2H: KTJ_PUT(w, "Memcpy HtoH (Host -> Host)"); break;
+    case KTJ_COPY_H2D: KTJ_PUT(w, "Memcpy HtoD (Host -> Device)"); break;
+    case KTJ_COPY_D2H: KTJ_PUT(w, "Memcpy DtoH (Device -> Host)"); break;
+    case KTJ_COPY_D2D: KTJ_PUT(w, "Memcpy DtoD (Device -> Device)"); break;
+    default: KTJ_PUT(w, "Memcpy <unknown> (? -> ?)"); break;
+  }
+}
+template <class W> KTJ_HD KTJ_FI inline void put_copy_kind(W& w, uint32_t op) {
+  switch (op) {
+    case KTJ_COPY_H2H: KTJ_PUT(w, "HtoH"); break;
+    case KTJ_COPY_H2D: KTJ_PUT(w, "HtoD"); break;
+    case KTJ_COPY_D2H: KTJ_PUT(w, "DtoH"); break;
+    case KTJ_COPY_D2D: KTJ_PUT(w, "DtoD"); break;
+    default: KTJ_PUT(w, "<unknown>"); break;
+  }
+}
+
 /* does this row print a metadata fragment?  (ArgsBuilder::appendFragment, output_json.cpp:173-181) */
-KTJ_HD inline bool has_fragment(const MatRow& r, const EmitCtx& c) {
+KTJ_HD KTJ_FI inline bool has_fragment(const MatRow& r, const EmitCtx& c) {
   const uint32_t cls = (r.meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT;
   if (cls != KTJ_CLASS_GENERIC) return true;
   if (r.aux >= c.n_schemas) return false;
@@ -423,7 +582,7 @@ KTJ_HD inline bool has_fragment(const MatRow& r, const EmitCtx& c) {
 }
 
 /* the metadataJson() fragment, after sanitizeStrForJSON */
-template <class W> KTJ_HD inline void put_fragment(W& w, const MatRow& r, const EmitCtx& c) {
+template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r, const EmitCtx& c) {
   const uint32_t cls = (r.meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT;
   const uint32_t kind = (r.meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
   if (cls == KTJ_CLASS_GENERIC) { /* GenericTraceActivity.cpp:60-64 + TypedMetadataJson.h */
@@ -433,22 +592,22 @@ template <class W> KTJ_HD inline void put_fragment(W& w, const MatRow& r, const 
     for (uint32_t f = 0; f < sd.n_fields; ++f) {
       const ktj_field fd = c.fields[sd.first_field + f];
       if (fd.key_id != KTJ_NONE) {
-        if (!first) w.lit(KTJ_LIT(", "));
+        if (!first) KTJ_PUT(w, ", ");
         first = false;
-        w.ch('"'); put_arg_string(w, c.dict, fd.key_id); w.lit(KTJ_LIT("\": "));
+        w.ch('"'); put_arg_string(w, c.dict, fd.key_id); KTJ_PUT(w, "\": ");
       }
       const uint64_t v = slot < c.n_args ? c.args[slot] : 0;
       switch (fd.type) {
         case KTJ_F_I64: put_i64(w, (int64_t)v); break;
         case KTJ_F_U64: w.dec(v); break;
         case KTJ_F_F64: put_f64(w, v); break;
-        case KTJ_F_BOOL: if (v) w.lit(KTJ_LIT("true")); else w.lit(KTJ_LIT("false")); break;
+        case KTJ_F_BOOL: if (v) KTJ_PUT(w, "true"); else KTJ_PUT(w, "false"); break;
         case KTJ_F_STR: w.ch('"'); put_arg_string(w, c.dict, (uint32_t)v); w.ch('"'); break;
         case KTJ_F_RAW: put_arg_string(w, c.dict, (uint32_t)v); break;
         case KTJ_F_I64_ARRAY:
           w.ch('[');
           for (uint32_t k = 0; k < fd.count; ++k) {
-            if (k) w.lit(KTJ_LIT(", "));
+            if (k) KTJ_PUT(w, ", ");
             put_i64(w, (int64_t)(slot + k < c.n_args ? c.args[slot + k] : 0));
           }
           w.ch(']');
@@ -463,77 +622,76 @@ template <class W> KTJ_HD inline void put_fragment(W& w, const MatRow& r, const 
     switch (kind) {
       case KTJ_RT_KERNEL: /* RocprofActivity_inl.h:208-232 */
         if (r.meta & KTJ_M_HAS_KERNEL_ARG) {
-          w.lit(KTJ_LIT("\"kernel\": \"")); put_arg_string(w, c.dict, (uint32_t)r.p[4]); w.lit(KTJ_LIT("\", "));
+          KTJ_PUT(w, "\"kernel\": \""); put_arg_string(w, c.dict, (uint32_t)r.p[4]); KTJ_PUT(w, "\", ");
         }
-        w.lit(KTJ_LIT("\"cid\": ")); w.dec(r.aux);
-        w.lit(KTJ_LIT(", \"correlation\": ")); w.dec((uint64_t)r.flow_id);
-        w.lit(KTJ_LIT(", \"grid\": ")); put_array3(w, r.p[0] & 0xFFFFFFFFu, r.p[0] >> 32, r.p[1] & 0xFFFFFFFFu);
-        w.lit(KTJ_LIT(", \"block\": ")); put_array3(w, r.p[1] >> 32, r.p[2] & 0xFFFFFFFFu, r.p[2] >> 32);
-        w.lit(KTJ_LIT(", \"shared memory\": ")); w.dec(r.p[3]);
+        KTJ_PUT(w, "\"cid\": "); w.dec(r.aux);
+        KTJ_PUT(w, ", \"correlation\": "); w.dec((uint64_t)r.flow_id);
+        KTJ_PUT(w, ", \"grid\": "); put_array3(w, r.p[0] & 0xFFFFFFFFu, r.p[0] >> 32, r.p[1] & 0xFFFFFFFFu);
+        KTJ_PUT(w, ", \"block\": "); put_array3(w, r.p[1] >> 32, r.p[2] & 0xFFFFFFFFu, r.p[2] >> 32);
+        KTJ_PUT(w, ", \"shared memory\": "); w.dec(r.p[3]);
         break;
       case KTJ_RT_COPY: /* RocprofActivity_inl.h:243-255 */
-        w.lit(KTJ_LIT("\"cid\": ")); w.dec(r.aux);
-        w.lit(KTJ_LIT(", \"correlation\": ")); w.dec((uint64_t)r.flow_id);
-        w.lit(KTJ_LIT(", \"src\": \"0x")); w.hex(r.p[0]);
-        w.lit(KTJ_LIT("\", \"dst\": \"0x")); w.hex(r.p[1]);
-        w.lit(KTJ_LIT("\", \"bytes\": ")); w.dec(r.p[2]);
-        w.lit(KTJ_LIT(", \"kind\": \"")); put_i64(w, (int64_t)(int32_t)(uint32_t)r.p[3]); w.ch('"');
+        KTJ_PUT(w, "\"cid\": "); w.dec(r.aux);
+        KTJ_PUT(w, ", \"correlation\": "); w.dec((uint64_t)r.flow_id);
+        KTJ_PUT(w, ", \"src\": \"0x"); put_hex(w, r.p[0]);
+        KTJ_PUT(w, "\", \"dst\": \"0x"); put_hex(w, r.p[1]);
+        KTJ_PUT(w, "\", \"bytes\": "); w.dec(r.p[2]);
+        KTJ_PUT(w, ", \"kind\": \""); put_i64(w, (int64_t)(int32_t)(uint32_t)r.p[3]); w.ch('"');
         break;
       case KTJ_RT_MALLOC: /* RocprofActivity_inl.h:265-277 */
-        if (r.meta & KTJ_M_MALLOC_BYTES) { w.lit(KTJ_LIT("\"bytes\": ")); w.dec(r.p[1]); w.lit(KTJ_LIT(", ")); }
-        w.lit(KTJ_LIT("\"cid\": ")); w.dec(r.aux);
-        w.lit(KTJ_LIT(", \"correlation\": ")); w.dec((uint64_t)r.flow_id);
-        w.lit(KTJ_LIT(", \"ptr\": \"0x")); w.hex(r.p[0]); w.ch('"');
+        if (r.meta & KTJ_M_MALLOC_BYTES) { KTJ_PUT(w, "\"bytes\": "); w.dec(r.p[1]); KTJ_PUT(w, ", "); }
+        KTJ_PUT(w, "\"cid\": "); w.dec(r.aux);
+        KTJ_PUT(w, ", \"correlation\": "); w.dec((uint64_t)r.flow_id);
+        KTJ_PUT(w, ", \"ptr\": \"0x"); put_hex(w, r.p[0]); w.ch('"');
         break;
       default: /* RocprofActivity_inl.h:294-299 */
-        w.lit(KTJ_LIT("\"cid\": ")); w.dec(r.aux);
-        w.lit(KTJ_LIT(", \"correlation\": ")); w.dec((uint64_t)r.flow_id);
+        KTJ_PUT(w, "\"cid\": "); w.dec(r.aux);
+        KTJ_PUT(w, ", \"correlation\": "); w.dec((uint64_t)r.flow_id);
         break;
     }
     return;
   }
   /* device rows */
   if (kind == KTJ_DOM_MEMSET) { /* CuptiActivity.h:682-713, 460-470 */
-    w.lit(KTJ_LIT("\"device\": ")); put_i64(w, r.dev);
-    w.lit(KTJ_LIT(", \"context\": ")); w.dec(r.p[3]);
-    w.lit(KTJ_LIT(", \"stream\": ")); put_i64(w, r.res);
-    w.lit(KTJ_LIT(", \"correlation\": ")); w.dec((uint64_t)r.flow_id);
-    w.lit(KTJ_LIT(", \"bytes\": ")); w.dec(r.p[0]);
+    KTJ_PUT(w, "\"device\": "); put_i64(w, r.dev);
+    KTJ_PUT(w, ", \"context\": "); w.dec(r.p[3]);
+    KTJ_PUT(w, ", \"stream\": "); put_i64(w, r.res);
+    KTJ_PUT(w, ", \"correlation\": "); w.dec((uint64_t)r.flow_id);
+    KTJ_PUT(w, ", \"bytes\": "); w.dec(r.p[0]);
     if (r.dur != 0) {
       const double bw = (double)r.p[0] / (double)r.dur;
       uint64_t bits; __builtin_memcpy(&bits, &bw, 8);
-      w.lit(KTJ_LIT(", \"memory bandwidth (GB/s)\": ")); put_f64(w, bits);
+      KTJ_PUT(w, ", \"memory bandwidth (GB/s)\": "); put_f64(w, bits);
     }
     return;
   }
   /* GpuActivity::visitTypedMetadata: RocprofActivity_inl.h:147-180 */
-  w.lit(KTJ_LIT("\"device\": ")); put_i64(w, r.dev);
-  w.lit(KTJ_LIT(", \"stream\": ")); put_i64(w, r.res);
-  w.lit(KTJ_LIT(", \"hsa_queue\": ")); w.dec(r.p[3]);
-  w.lit(KTJ_LIT(", \"correlation\": ")); w.dec((uint64_t)r.flow_id);
-  w.lit(KTJ_LIT(", \"kind\": \""));
-  if (kind == KTJ_DOM_MEMORY_COPY) w.lit(copy_kind_string(r.aux)); else w.lit(KTJ_LIT("Dispatch Kernel"));
-  w.ch('"');
+  KTJ_PUT(w, "\"device\": "); put_i64(w, r.dev);
+  KTJ_PUT(w, ", \"stream\": "); put_i64(w, r.res);
+  KTJ_PUT(w, ", \"hsa_queue\": "); w.dec(r.p[3]);
+  KTJ_PUT(w, ", \"correlation\": "); w.dec((uint64_t)r.flow_id);
+  if (kind == KTJ_DOM_MEMORY_COPY) { KTJ_PUT(w, ", \"kind\": \""); put_copy_kind(w, r.aux); w.ch('"'); }
+  else KTJ_PUT(w, ", \"kind\": \"Dispatch Kernel\"");
   if (r.meta & KTJ_M_HAS_SIZE) {
-    w.lit(KTJ_LIT(", \"bytes\": ")); w.dec(r.p[0]);
+    KTJ_PUT(w, ", \"bytes\": "); w.dec(r.p[0]);
     const uint64_t raw_dur = (uint64_t)r.dur + 1; /* end - begin; duration() is end - (begin + 1) */
     if (raw_dur != 0) { /* RocprofActivity_inl.h:129-139 */
       const double bw = (double)r.p[0] / (double)raw_dur;
       uint64_t bits; __builtin_memcpy(&bits, &bw, 8);
-      w.lit(KTJ_LIT(", \"memory bandwidth (GB/s)\": ")); put_f64(w, bits);
+      KTJ_PUT(w, ", \"memory bandwidth (GB/s)\": "); put_f64(w, bits);
     }
   } else if (r.meta & KTJ_M_HAS_GRID) {
-    w.lit(KTJ_LIT(", \"grid\": ")); put_array3(w, r.p[0] & 0xFFFFFFFFu, r.p[0] >> 32, r.p[1] & 0xFFFFFFFFu);
-    w.lit(KTJ_LIT(", \"block\": ")); put_array3(w, r.p[1] >> 32, r.p[2] & 0xFFFFFFFFu, r.p[2] >> 32);
+    KTJ_PUT(w, ", \"grid\": "); put_array3(w, r.p[0] & 0xFFFFFFFFu, r.p[0] >> 32, r.p[1] & 0xFFFFFFFFu);
+    KTJ_PUT(w, ", \"block\": "); put_array3(w, r.p[1] >> 32, r.p[2] & 0xFFFFFFFFu, r.p[2] >> 32);
   }
 }
 
 /* name after the logger's pipeline (output_json.cpp:946-949) */
-template <class W> KTJ_HD inline void put_name(W& w, const MatRow& r, const EmitCtx& c) {
+template <class W> KTJ_HD KTJ_FI inline void put_name(W& w, const MatRow& r, const EmitCtx& c) {
   if (r.meta & KTJ_M_NAME_BUILTIN) {
-    if (r.name_id <= 4) w.lit(memcpy_name(r.name_id));
-    else if (r.name_id == KTJ_NAME_MEMSET) w.lit(KTJ_LIT("Memset (Device)"));
-    else if (r.name_id == KTJ_NAME_UNKNOWN_OP) { w.lit(KTJ_LIT("<unknown operation:")); w.dec(r.aux); w.ch('>'); }
+    if (r.name_id <= 4) put_memcpy_name(w, r.name_id);
+    else if (r.name_id == KTJ_NAME_MEMSET) KTJ_PUT(w, "Memset (Device)");
+    else if (r.name_id == KTJ_NAME_UNKNOWN_OP) { KTJ_PUT(w, "<unknown operation:"); w.dec(r.aux); w.ch('>'); }
     return;
   }
   if (r.name_id < c.dict.n)
@@ -541,7 +699,7 @@ template <class W> KTJ_HD inline void put_name(W& w, const MatRow& r, const Emit
 }
 
 /* One activity: the complete event and, if it takes part in a flow, the flow event after it. */
-template <class W> KTJ_HD inline void format_activity(W& w, const MatRow& r, const EmitCtx& c) {
+template <class W> KTJ_HD KTJ_FI inline void format_activity(W& w, const MatRow& r, const EmitCtx& c) {
   const uint32_t type = r.meta & KTJ_M_TYPE_MASK;
   int64_t ts = r.ts;
   int64_t dur = r.dur < 0 ? 0 : r.dur;                       /* output_json.cpp:860 */
@@ -549,35 +707,38 @@ template <class W> KTJ_HD inline void format_activity(W& w, const MatRow& r, con
   int64_t rel = ts - c.base_time_ns;                         /* transToRelativeTime :144-153 */
   if (rel < 0) rel = 0;
   const int64_t tid = sanitize_tid(r.res);
-  w.lit(KTJ_LIT("\n  {\n    \"ph\": \"X\",\n    \"cat\": \""));
-  w.lit(category_name(type));
-  w.lit(KTJ_LIT("\",\n    \"name\": \""));
+  const bool flow = (r.meta & KTJ_M_FLOW) != 0;
+  /* pid and tid are printed again by the flow event */
+  const bool pid_neg = r.dev < 0;
+  const typename W::Prepared pid = W::prepare(pid_neg ? 0ULL - (uint64_t)r.dev : (uint64_t)r.dev);
+  const typename W::Prepared tidn = W::prepare((uint64_t)tid);
+  KTJ_PUT(w, "\n  {\n    \"ph\": \"X\",\n    \"cat\": \"");
+  put_category(w, type);
+  KTJ_PUT(w, "\",\n    \"name\": \"");
   put_name(w, r, c);
-  w.lit(KTJ_LIT("\",\n    \"pid\": ")); put_i64(w, r.dev);
-  w.lit(KTJ_LIT(",\n    \"tid\": ")); put_i64(w, tid);
-  w.lit(KTJ_LIT(",\n    \"ts\": ")); put_ts(w, rel);
-  w.lit(KTJ_LIT(",\n    \"dur\": ")); put_ts(w, dur);
-  w.lit(KTJ_LIT("\n    "));
+  KTJ_PUT(w, "\",\n    \"pid\": "); if (pid_neg) w.ch('-'); w.num(pid);
+  KTJ_PUT(w, ",\n    \"tid\": "); w.num(tidn);
+  KTJ_PUT(w, ",\n    \"ts\": "); put_ts(w, rel);
+  KTJ_PUT(w, ",\n    \"dur\": "); put_ts(w, dur);
   const bool frag = has_fragment(r, c);
   if (r.ext != 0 || frag) {                                  /* ArgsBuilder :157-212 */
-    w.lit(KTJ_LIT(",\n    \"args\": {\n      "));
-    if (r.ext != 0) { w.lit(KTJ_LIT("\"External id\": ")); put_i64(w, r.ext); }
+    KTJ_PUT(w, "\n    ,\n    \"args\": {\n      ");
+    if (r.ext != 0) { KTJ_PUT(w, "\"External id\": "); put_i64(w, r.ext); }
     if (frag) { if (r.ext != 0) w.ch(','); put_fragment(w, r, c); }
-    w.lit(KTJ_LIT("\n    }"));
-  }
-  w.lit(KTJ_LIT("\n  },"));
-  if (r.meta & KTJ_M_FLOW) {                                 /* :960-1021, writeFlowEvent :318-345 */
+    KTJ_PUT(w, "\n    }\n  },");
+  } else KTJ_PUT(w, "\n    \n  },");
+  if (flow) {                                                /* :960-1021, writeFlowEvent :318-345 */
     int64_t frel = r.ts - c.base_time_ns;
     if (frel < 0) frel = 0;
-    w.lit(KTJ_LIT("\n  {\n    \"ph\": \"")); w.ch((r.meta & KTJ_M_FLOW_START) ? 's' : 'f');
-    w.lit(KTJ_LIT("\",\n    \"id\": ")); put_i64(w, r.flow_id);
-    w.lit(KTJ_LIT(",\n    \"pid\": ")); put_i64(w, r.dev);
-    w.lit(KTJ_LIT(",\n    \"tid\": ")); put_i64(w, tid);
-    w.lit(KTJ_LIT(",\n    \"ts\": ")); put_ts(w, frel);
-    if (r.meta & KTJ_M_FLOW_FWDBWD) w.lit(KTJ_LIT(",\n    \"cat\": \"fwdbwd\",\n    \"name\": \"fwdbwd\"\n    "));
-    else w.lit(KTJ_LIT(",\n    \"cat\": \"ac2g\",\n    \"name\": \"ac2g\"\n    "));
-    if (!(r.meta & KTJ_M_FLOW_START)) w.lit(KTJ_LIT(", \"bp\": \"e\""));
-    w.lit(KTJ_LIT("\n  },"));
+    if (r.meta & KTJ_M_FLOW_START) KTJ_PUT(w, "\n  {\n    \"ph\": \"s\",\n    \"id\": ");
+    else KTJ_PUT(w, "\n  {\n    \"ph\": \"f\",\n    \"id\": ");
+    put_i64(w, r.flow_id);
+    KTJ_PUT(w, ",\n    \"pid\": "); if (pid_neg) w.ch('-'); w.num(pid);
+    KTJ_PUT(w, ",\n    \"tid\": "); w.num(tidn);
+    KTJ_PUT(w, ",\n    \"ts\": "); put_ts(w, frel);
+    if (r.meta & KTJ_M_FLOW_FWDBWD) KTJ_PUT(w, ",\n    \"cat\": \"fwdbwd\",\n    \"name\": \"fwdbwd\"\n    ");
+    else KTJ_PUT(w, ",\n    \"cat\": \"ac2g\",\n    \"name\": \"ac2g\"\n    ");
+    if (r.meta & KTJ_M_FLOW_START) KTJ_PUT(w, "\n  },"); else KTJ_PUT(w, ", \"bp\": \"e\"\n  },");
   }
 }
 

@@ -147,9 +147,13 @@ hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint6
 hipError_t gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted, hipStream_t st);
 
 /* ---- stage 4b: emit ---- */
-#define KTJ_EMIT_TILE 16384
+/* tile size (bytes of output per workgroup) for a document whose activity section has act_bytes
+ * bytes in n_rows activities, and the number of tiles / entries of tile_start (tiles + 1) */
+uint32_t emit_tile_bytes(uint64_t act_bytes, uint64_t n_rows);
+uint64_t emit_tile_count(uint64_t prefix_len, uint64_t act_bytes, uint32_t tile);
 hipError_t emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs /* n+1 */, uint64_t n,
-                EmitCtx ctx, char* out, uint64_t prefix_len, uint64_t act_bytes, hipStream_t st);
+                EmitCtx ctx, char* out, uint64_t prefix_len, uint64_t act_bytes, uint32_t tile,
+                uint32_t* tile_start /* tiles + 1 */, hipStream_t st);
 
 }  // namespace gpu
 }  // namespace ktj

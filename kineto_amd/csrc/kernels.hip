@@ -15,6 +15,8 @@
  */
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "gpu_stages.h"
 
 namespace ktj {
@@ -1033,74 +1035,97 @@ hipError_t gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uin
 }
 
 /* ------------------------------------------------------------------------------------------ */
-/* stage 4b: emit.  Workgroup k owns the output bytes [k*TILE, (k+1)*TILE) of the whole document */
-/* (clipped to the activity section), so every global store is an aligned 16-byte store.  It     */
-/* finds the activities overlapping its range by binary search in the offsets, formats each one  */
-/* into LDS with clipping (an activity straddling a tile boundary is formatted by both tiles),   */
-/* copies dictionary strings with whole wavefronts, and flushes the tile.                        */
+/* stage 4b: emit.  Workgroup k owns the output bytes [k*T, (k+1)*T) of the whole document      */
+/* (clipped to the activity section), so every global store is an aligned 16-byte store.  The    */
+/* first activity of every tile is found once by k_tile_starts (binary search in the offsets);   */
+/* the emit workgroup formats one activity per lane into LDS through a 64-bit accumulator        */
+/* (literals are immediates, digits are packed arithmetically, no per-byte loads), with clipping */
+/* (an activity straddling a tile boundary is formatted by both tiles), copies dictionary        */
+/* strings with whole wavefronts, and flushes the tile.  T is chosen by the host so that a tile  */
+/* holds about as many activities as the workgroup has lanes.                                    */
 /* ------------------------------------------------------------------------------------------ */
 #define EMIT_THREADS 128
-#define EMIT_MAX_JOBS 384
+#define EMIT_MAX_JOBS 512
+
+__global__ void k_tile_starts(const uint64_t* offs, uint64_t n, uint64_t prefix_len, uint32_t tile, uint64_t first_tile,
+                              uint32_t n_tiles, uint32_t* start) {
+  const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t > n_tiles) return;
+  if (t == n_tiles) { start[t] = (uint32_t)n; return; }
+  const uint64_t t0 = (first_tile + t) * (uint64_t)tile;
+  const uint64_t lo = (t0 > prefix_len ? t0 : prefix_len) - prefix_len;
+  uint64_t a = 0, b = n; /* first record with offs[r + 1] > lo */
+  while (a < b) { const uint64_t m = (a + b) >> 1; if (offs[m + 1] > lo) b = m; else a = m + 1; }
+  start[t] = (uint32_t)a;
+}
 
 __global__ void __launch_bounds__(EMIT_THREADS)
 k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n, EmitCtx ctx, char* out,
-       uint64_t prefix_len, uint64_t act_bytes) {
-  __shared__ __attribute__((aligned(16))) char tile[KTJ_EMIT_TILE];
-  __shared__ CopyJob jobs[EMIT_MAX_JOBS];
-  __shared__ uint32_t n_jobs;
+       uint64_t prefix_len, uint64_t act_bytes, uint32_t tile, uint64_t first_tile, const uint32_t* start, int dbg) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  char* buf = smem;                                                   /* tile bytes */
+  CopyJob* jobs = reinterpret_cast<CopyJob*>(smem + tile);            /* EMIT_MAX_JOBS */
+  uint32_t* n_jobs = reinterpret_cast<uint32_t*>(smem + tile + EMIT_MAX_JOBS * sizeof(CopyJob));
 
-  const uint64_t t0 = ((prefix_len / KTJ_EMIT_TILE) + blockIdx.x) * (uint64_t)KTJ_EMIT_TILE; /* absolute */
+  const uint64_t t0 = (first_tile + blockIdx.x) * (uint64_t)tile;     /* absolute, multiple of the tile size */
   const uint64_t abs_lo = t0 > prefix_len ? t0 : prefix_len;
   const uint64_t abs_end = prefix_len + act_bytes;
-  const uint64_t abs_hi = t0 + KTJ_EMIT_TILE < abs_end ? t0 + KTJ_EMIT_TILE : abs_end;
+  const uint64_t abs_hi = t0 + tile < abs_end ? t0 + tile : abs_end;
   if (abs_lo >= abs_hi) return;
-  const uint64_t lo = abs_lo - prefix_len, hi = abs_hi - prefix_len; /* activity-relative */
-  const uint32_t head = (uint32_t)(abs_lo - t0);                       /* tile[head] ↔ abs_lo */
-  const int32_t span = (int32_t)(hi - lo);
+  const int32_t lo = (int32_t)(abs_lo - t0), hi = (int32_t)(abs_hi - t0); /* tile-local */
 
-  /* r0 = last record with offs[r0] <= lo; r1 = first record with offs[r1] >= hi */
-  uint64_t a = 0, b = n;
-  while (a < b) { const uint64_t m = (a + b) >> 1; if (offs[m + 1] > lo) b = m; else a = m + 1; }
-  const uint64_t r0 = a;
-  a = r0; b = n;
-  while (a < b) { const uint64_t m = (a + b) >> 1; if (offs[m] >= hi) b = m; else a = m + 1; }
-  const uint64_t r1 = a;
+  const uint64_t r0 = start[blockIdx.x];
+  uint64_t r1 = start[blockIdx.x + 1];
+  if (r1 < n && offs[r1] + prefix_len < abs_hi) ++r1;                  /* the straddler at the upper edge */
 
-  if (threadIdx.x == 0) n_jobs = 0;
+  if (threadIdx.x == 0) *n_jobs = 0;
+  {
+    uint4* z = reinterpret_cast<uint4*>(buf);
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    for (uint32_t k = threadIdx.x; k < tile / 16u; k += EMIT_THREADS) z[k] = zero;
+  }
   __syncthreads();
   for (uint64_t r = r0 + threadIdx.x; r < r1; r += EMIT_THREADS) {
     const uint64_t o = offs[r];
     if (offs[r + 1] == o) continue; /* dropped or empty */
-    MatRow m;
-    {
-      const uint4* s = reinterpret_cast<const uint4*>(&mat[perm[r]]);
-      uint4* d = reinterpret_cast<uint4*>(&m);
-      for (int k = 0; k < (int)(sizeof(MatRow) / 16); ++k) d[k] = s[k];
-    }
+    const MatRow m = mat[perm[r]];
     TileWriter w;
-    w.buf = tile + head;
-    w.pos = (int32_t)((int64_t)o - (int64_t)lo);
-    w.tile = span;
-    w.jobs = jobs;
-    w.n_jobs = &n_jobs;
-    w.max_jobs = EMIT_MAX_JOBS;
-    format_activity(w, m, ctx);
+    w.buf = buf; w.size = tile;
+    w.jobs = jobs; w.n_jobs = n_jobs; w.max_jobs = EMIT_MAX_JOBS;
+    w.begin((int32_t)((int64_t)(o + prefix_len) - (int64_t)t0));
+    if (!(dbg & 1)) format_activity(w, m, ctx);
+    w.end();
   }
   __syncthreads();
-  {
-    const uint32_t nj = n_jobs < EMIT_MAX_JOBS ? n_jobs : EMIT_MAX_JOBS;
-    const uint32_t wv = threadIdx.x >> 6, ln = threadIdx.x & 63u;
-    for (uint32_t j = wv; j < nj; j += (EMIT_THREADS >> 6)) {
+  if (!(dbg & 2)) {
+    /* string copies: one job per 16-lane group; aligned 8-byte words in the middle (two aligned
+     * global loads funnel-shifted into one aligned LDS store), single bytes at both ends */
+    const uint32_t nj = *n_jobs < EMIT_MAX_JOBS ? *n_jobs : EMIT_MAX_JOBS;
+    const uint32_t group = threadIdx.x >> 4, gl = threadIdx.x & 15u;
+    for (uint32_t j = group; j < nj; j += (EMIT_THREADS >> 4)) {
       const CopyJob job = jobs[j];
-      char* dst = tile + head + job.dst;
-      for (uint32_t k = ln; k < job.len; k += 64) dst[k] = job.src[k];
+      uint32_t headb = (8u - ((uint32_t)job.dst & 7u)) & 7u;
+      if (headb > job.len) headb = job.len;
+      if (gl < headb) buf[job.dst + (int32_t)gl] = job.src[gl];
+      const uint32_t words = (job.len - headb) >> 3;
+      const uintptr_t sa = (uintptr_t)(job.src + headb);
+      const uint32_t sh = (uint32_t)(sa & 7u) * 8u;
+      const uint64_t* sp = reinterpret_cast<const uint64_t*>(sa & ~(uintptr_t)7);
+      uint64_t* dp = reinterpret_cast<uint64_t*>(buf + job.dst + (int32_t)headb);
+      for (uint32_t k = gl; k < words; k += 16u) {
+        uint64_t v = sp[k];
+        if (sh) v = (v >> sh) | (sp[k + 1] << (64u - sh));
+        dp[k] = v;
+      }
+      const uint32_t done = headb + words * 8u;
+      if (gl < job.len - done) buf[job.dst + (int32_t)(done + gl)] = job.src[done + gl];
     }
   }
   __syncthreads();
   /* flush: unaligned head bytes (first tile only), 16-byte body, tail bytes */
   char* g = out + abs_lo;
-  const char* s = tile + head;
-  const uint32_t nbytes = (uint32_t)span;
+  const char* s = buf + lo;
+  const uint32_t nbytes = (uint32_t)(hi - lo);
   uint32_t pre = (uint32_t)((16u - (uint32_t)((uintptr_t)g & 15u)) & 15u);
   if (pre > nbytes) pre = nbytes;
   for (uint32_t k = threadIdx.x; k < pre; k += EMIT_THREADS) g[k] = s[k];
@@ -1113,14 +1138,31 @@ k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n
   for (uint32_t k = pre + body * 16u + threadIdx.x; k < nbytes; k += EMIT_THREADS) g[k] = s[k];
 }
 
+static int dbg_flags() { const char* e = getenv("KTJ_DBG"); return e ? atoi(e) : 0; }
+uint32_t emit_tile_bytes(uint64_t act_bytes, uint64_t n_rows) {
+  if (const char* e = getenv("KTJ_EMIT_TILE")) return (uint32_t)atoi(e);
+  /* about 0.85 activities per lane, in steps of 4 KiB, between 8 and 40 KiB */
+  const uint64_t avg = n_rows ? act_bytes / n_rows : 512;
+  uint64_t t = (avg * EMIT_THREADS * 85 / 100 + 4095) / 4096 * 4096;
+  if (t < 8192) t = 8192;
+  if (t > 40960) t = 40960;
+  return (uint32_t)t;
+}
+uint64_t emit_tile_count(uint64_t prefix_len, uint64_t act_bytes, uint32_t tile) {
+  if (act_bytes == 0) return 0;
+  return (prefix_len + act_bytes - 1) / tile - prefix_len / tile + 1;
+}
+
 hipError_t emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n, EmitCtx ctx, char* out,
-                uint64_t prefix_len, uint64_t act_bytes, hipStream_t st) {
+                uint64_t prefix_len, uint64_t act_bytes, uint32_t tile, uint32_t* tile_start, hipStream_t st) {
   if (act_bytes == 0) return hipSuccess;
-  const uint64_t first_tile = prefix_len / KTJ_EMIT_TILE;
-  const uint64_t last_tile = (prefix_len + act_bytes - 1) / KTJ_EMIT_TILE;
-  const uint64_t tiles = last_tile - first_tile + 1;
-  hipLaunchKernelGGL(k_emit, dim3((unsigned)tiles), dim3(EMIT_THREADS), 0, st, mat, perm, offs, n, ctx, out, prefix_len,
-                     act_bytes);
+  const uint64_t first_tile = prefix_len / tile;
+  const uint32_t tiles = (uint32_t)emit_tile_count(prefix_len, act_bytes, tile);
+  hipLaunchKernelGGL(k_tile_starts, dim3(grid_for((uint64_t)tiles + 1, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, offs, n,
+                     prefix_len, tile, first_tile, tiles, tile_start);
+  const size_t lds = (size_t)tile + EMIT_MAX_JOBS * sizeof(CopyJob) + 16;
+  hipLaunchKernelGGL(k_emit, dim3(tiles), dim3(EMIT_THREADS), lds, st, mat, perm, offs, n, ctx, out, prefix_len,
+                     act_bytes, tile, first_tile, (const uint32_t*)tile_start, dbg_flags());
   return KTJ_LAUNCH_CHECK();
 }
 

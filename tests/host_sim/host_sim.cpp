@@ -222,27 +222,40 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   memset(buf, '#', total);
   memcpy(buf, prefix.data(), prefix.size());
   memcpy(buf + prefix.size() + act_bytes, suffix.data(), suffix.size());
-  char* act = buf + prefix.size();
 
-  // output-partitioned tiles
-  std::vector<char> tile(tile_bytes);
+  // output-partitioned tiles, exactly as the emit kernel lays them out: tile k owns the
+  // document bytes [k*T, (k+1)*T) clipped to the activity section; tile-local coordinate
+  // L = absolute offset - k*T
+  const uint64_t T = tile_bytes;
+  if (T % 8) { free(buf); return -3; }
+  std::vector<uint64_t> tile_store(T / 8 + 1);
+  char* tile = reinterpret_cast<char*>(tile_store.data());
   std::vector<CopyJob> jobs(64);
-  for (uint64_t lo = 0; lo < act_bytes; lo += tile_bytes) {
-    const uint64_t hi = std::min<uint64_t>(lo + tile_bytes, act_bytes);
-    // first record ending after lo, last record starting before hi
-    size_t r0 = std::upper_bound(offs.begin(), offs.end(), lo) - offs.begin() - 1;
-    size_t r1 = std::lower_bound(offs.begin(), offs.end(), hi) - offs.begin();  // exclusive
-    uint32_t nj = 0;
-    for (size_t r = r0; r < r1; ++r) {
-      TileWriter w;
-      w.buf = tile.data(); w.pos = (int32_t)((int64_t)offs[r] - (int64_t)lo); w.tile = (int32_t)(hi - lo);
-      w.jobs = jobs.data(); w.n_jobs = &nj; w.max_jobs = (uint32_t)jobs.size();
-      format_activity(w, mat[perm[r]], ctx);
-      if ((int64_t)w.pos != (int64_t)offs[r + 1] - (int64_t)lo) { free(buf); return -2; }
+  const uint64_t P = prefix.size();
+  if (act_bytes) {
+    for (uint64_t k = P / T; k * T < P + act_bytes; ++k) {
+      const uint64_t t0 = k * T;
+      const uint64_t abs_lo = t0 > P ? t0 : P;
+      const uint64_t abs_hi = std::min<uint64_t>(t0 + T, P + act_bytes);
+      const uint64_t lo = abs_lo - P, hi = abs_hi - P;  // activity-relative
+      size_t r0 = std::upper_bound(offs.begin(), offs.end(), lo) - offs.begin() - 1;
+      size_t r1 = std::lower_bound(offs.begin(), offs.end(), hi) - offs.begin();  // exclusive
+      uint32_t nj = 0;
+      memset(tile, 0, T);
+      for (size_t r = r0; r < r1; ++r) {
+        if (offs[r + 1] == offs[r]) continue;
+        TileWriter w;
+        w.buf = tile; w.size = (uint32_t)T;
+        w.jobs = jobs.data(); w.n_jobs = &nj; w.max_jobs = (uint32_t)jobs.size();
+        w.begin((int32_t)((int64_t)(offs[r] + P) - (int64_t)t0));
+        format_activity(w, mat[perm[r]], ctx);
+        w.end();
+        if ((int64_t)w.position() != (int64_t)(offs[r + 1] + P) - (int64_t)t0) { free(buf); return -2; }
+      }
+      const uint32_t done = nj < jobs.size() ? nj : (uint32_t)jobs.size();
+      for (uint32_t j = 0; j < done; ++j) memcpy(tile + jobs[j].dst, jobs[j].src, jobs[j].len);
+      memcpy(buf + abs_lo, tile + (abs_lo - t0), abs_hi - abs_lo);
     }
-    const uint32_t done = nj < jobs.size() ? nj : (uint32_t)jobs.size();
-    for (uint32_t j = 0; j < done; ++j) memcpy(tile.data() + jobs[j].dst, jobs[j].src, jobs[j].len);
-    memcpy(act + lo, tile.data(), hi - lo);
   }
   *out = buf;
   *out_n = total;
