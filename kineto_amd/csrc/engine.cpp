@@ -573,8 +573,15 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   const uint32_t tile = emit_tile_bytes(act_bytes, e->scalars.n_valid);
   HIPCHK(e->tile_start.ensure((emit_tile_count(e->prefix_len, act_bytes, tile) + 2) * 4));
   HIPCHK(hipEventRecord(e->ev[EV_EMIT_START], st));
-  HIPCHK(emit(mat, e->perm, e->offs.as<uint64_t>(), N, ctx, e->out.as<char>(), e->prefix_len, act_bytes, tile,
-              e->tile_start.as<uint32_t>(), st));
+  {
+    const char* mode = getenv("KTJ_EMIT_MODE"); /* "tile" selects the LDS-staged variant */
+    if (mode && strcmp(mode, "tile") == 0)
+      HIPCHK(emit(mat, e->perm, e->offs.as<uint64_t>(), N, ctx, e->out.as<char>(), e->prefix_len, act_bytes, tile,
+                  e->tile_start.as<uint32_t>(), st));
+    else
+      HIPCHK(emit_direct(mat, e->perm, e->offs.as<uint64_t>(), e->len.as<uint32_t>(), e->scalars.n_valid, ctx,
+                         e->out.as<char>(), e->prefix_len, st));
+  }
   HIPCHK(hipEventRecord(e->ev[EV_EMIT], st));
   HIPCHK(hipStreamSynchronize(st));
 

@@ -387,6 +387,110 @@ struct TileWriter {
   }
 };
 
+/* Pass B, direct variant: one lane formats one activity straight into the document in device
+ * memory.  Bytes are gathered in a 64-bit accumulator and leave as aligned 8-byte stores.  An
+ * activity's first word also holds the last bytes of its predecessor; those are one of three
+ * fixed strings (see tail_kind), so the successor writes the whole shared word and the
+ * predecessor never writes its trailing partial word.  Dictionary strings are appended inline,
+ * eight bytes at a time, through a funnel shift over aligned loads (dictionary blobs are padded
+ * by 16 bytes so that the last load stays inside the allocation). */
+struct GlobalWriter {
+  uint64_t* wptr;     /* aligned address of the word being gathered */
+  uint64_t acc;
+  uint32_t fill;      /* bytes gathered in acc, 0..7 */
+
+  KTJ_HD KTJ_FI void begin(char* doc, uint64_t pos, uint64_t low_bytes) {
+    wptr = reinterpret_cast<uint64_t*>(doc + (pos & ~7ULL));
+    fill = (uint32_t)(pos & 7ULL);
+    acc = low_bytes; /* the `fill` bytes that precede this activity in its first word */
+  }
+  KTJ_HD KTJ_FI void append(uint64_t v, uint32_t n) {
+    acc |= v << (8 * fill);
+    const uint32_t total = fill + n;
+    if (total >= 8) {
+      *wptr++ = acc;
+      const uint32_t rest = total - 8;
+      acc = rest ? v >> (8 * (n - rest)) : 0;
+      fill = rest;
+    } else fill = total;
+  }
+  KTJ_HD KTJ_FI void ch(char c) { append((uint64_t)(unsigned char)c, 1); }
+  template <unsigned N> KTJ_HD KTJ_FI void lit(const PackedLit<N>& l) {
+    for (unsigned i = 0; i < N / 8; ++i) append(l.w[i], 8);
+    if (N % 8) append(l.w[N / 8], N % 8);
+  }
+  KTJ_HD KTJ_FI void dec_wide(uint64_t v) {
+    const uint64_t top = v / 10000000000000000ULL;
+    const uint64_t rest = v - top * 10000000000000000ULL;
+    const uint64_t mid = rest / 100000000ULL;
+    const uint32_t low = (uint32_t)(rest - mid * 100000000ULL);
+    uint64_t a0 = 0, a1;
+    uint32_t n0 = 0, n1;
+    if (top) {
+      a0 = ascii8((uint32_t)top);
+      const uint32_t z = leading_zero_chars(a0);
+      a0 >>= 8 * z; n0 = 8 - z;
+      a1 = ascii8((uint32_t)mid); n1 = 8;
+    } else {
+      a1 = ascii8((uint32_t)mid);
+      const uint32_t z = leading_zero_chars(a1);
+      a1 >>= 8 * z; n1 = 8 - z;
+    }
+    append(a0, n0);
+    append(a1, n1);
+    append(ascii8(low), 8);
+  }
+  KTJ_HD KTJ_FI void dec(uint64_t v) {
+    if (__builtin_expect(v < 100000000ULL, 1)) {
+      const uint64_t a = ascii8((uint32_t)v);
+      const uint32_t z = leading_zero_chars(a);
+      append(a >> (8 * z), 8 - z);
+    } else dec_wide(v);
+  }
+  typedef Num Prepared;
+  KTJ_HD KTJ_FI static Prepared prepare(uint64_t v) { return make_num(v); }
+  KTJ_HD KTJ_FI void num(const Num& n) {
+    if (__builtin_expect(n.len != 0, 1)) append(n.word, n.len); else dec_wide(n.value);
+  }
+  KTJ_HD KTJ_FI void dec3(uint32_t x) { append((uint64_t)(ascii4(x) >> 8), 3); }
+  KTJ_HD KTJ_FI void str(const char* src, uint64_t len) {
+    if (len == 0) return;
+    const uintptr_t sa = (uintptr_t)src;
+    const uint32_t sh = (uint32_t)(sa & 7u) * 8u;
+    const uint64_t* sp = reinterpret_cast<const uint64_t*>(sa & ~(uintptr_t)7);
+    uint64_t cur = sp[0];
+    const uint64_t full = len >> 3;
+    KTJ_NOUNROLL
+    for (uint64_t k = 0; k < full; ++k) {
+      const uint64_t next = sp[k + 1];
+      append(sh ? (cur >> sh) | (next << (64u - sh)) : cur, 8);
+      cur = next;
+    }
+    const uint32_t rem = (uint32_t)(len & 7u);
+    if (rem) {
+      uint64_t v = cur >> sh;
+      if (sh && rem * 8u > 64u - sh) v |= sp[full + 1] << (64u - sh);
+      append(v & ((1ULL << (8 * rem)) - 1ULL), rem);
+    }
+  }
+};
+
+/* The last seven bytes of a formatted activity, by kind (see format_activity):
+ *   0: `  \n  },`   complete event without args, or a flow-start event
+ *   1: ` }\n  },`   complete event with args and no flow event
+ *   2: `e"\n  },`   flow-end event */
+KTJ_HD KTJ_FI inline uint32_t tail_kind(const MatRow& r, bool has_args) {
+  if (r.meta & KTJ_M_FLOW) return (r.meta & KTJ_M_FLOW_START) ? 0u : 2u;
+  return has_args ? 1u : 0u;
+}
+KTJ_HD KTJ_FI inline uint64_t tail_bytes(uint32_t kind, uint32_t count) { /* last `count` (0..7) bytes, low-aligned */
+  constexpr auto t0 = pack_lit("  \n  },");
+  constexpr auto t1 = pack_lit(" }\n  },");
+  constexpr auto t2 = pack_lit("e\"\n  },");
+  const uint64_t t = kind == 0 ? t0.w[0] : (kind == 1 ? t1.w[0] : t2.w[0]);
+  return t >> (8 * (7 - count));
+}
+
 /* ---------------------------------------------------------------------------------------- */
 /* pieces                                                                                      */
 /* ---------------------------------------------------------------------------------------- */

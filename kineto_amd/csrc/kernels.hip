@@ -929,12 +929,13 @@ __device__ __forceinline__ void store_row(MatRow* dst, const MatRow& m) {
   uint4* d = reinterpret_cast<uint4*>(dst);
   for (int k = 0; k < (int)(sizeof(MatRow) / 16); ++k) d[k] = s[k];
 }
+/* exact byte length in the low 30 bits, tail kind (see tail_kind) in the top two */
 __device__ __forceinline__ uint32_t row_length(const MatRow& m, const EmitCtx& ctx, Scalars* sc) {
   if (!(m.meta & KTJ_M_VALID)) return 0;
   CountWriter cw;
   format_activity(cw, m, ctx);
   if (cw.n >= (1ull << 30)) { flag_error(sc, KTJ_DEVERR_RECORD_TOO_LONG); return 0; }
-  return (uint32_t)cw.n;
+  return (uint32_t)cw.n | (tail_kind(m, m.ext != 0 || has_fragment(m, ctx)) << 30);
 }
 struct RowStats { uint32_t n_flow = 0, n_blank = 0; };
 __device__ __forceinline__ void count_row_stats(const MatRow& m, const EmitCtx& ctx, RowStats* rs) {
@@ -1005,7 +1006,7 @@ __global__ void k_mat_device(const ktj_device_rec* d, uint64_t n, Columns c, uin
 }
 __global__ void k_gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) len_sorted[i] = len[perm[i]];
+  if (i < n) len_sorted[i] = len[perm[i]] & 0x3FFFFFFFu;
 }
 
 hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc,
@@ -1139,6 +1140,43 @@ k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n
 }
 
 static int dbg_flags() { const char* e = getenv("KTJ_DBG"); return e ? atoi(e) : 0; }
+/* Direct variant: one lane per activity, aligned 8-byte stores straight into the document, no
+ * LDS.  Lane i owns every word that starts inside its activity, including the one it shares
+ * with activity i+1's predecessor bytes... i.e. the first word of an activity is written by that
+ * activity's lane together with the (fixed) last bytes of its predecessor.  The document's
+ * prefix and suffix are already in place when this kernel runs; the first and the last activity
+ * merge with them. */
+__global__ void __launch_bounds__(KTJ_BLOCK)
+k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint32_t* len_kind, uint64_t n_rows,
+              EmitCtx ctx, char* out, uint64_t prefix_len) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_rows) return;
+  const uint64_t o = offs[i];
+  if (offs[i + 1] == o) return;
+  const MatRow m = mat[perm[i]];
+  const uint64_t pos = prefix_len + o;
+  const uint32_t fill = (uint32_t)(pos & 7ULL);
+  uint64_t low = 0;
+  if (fill) {
+    if (i == 0) low = *reinterpret_cast<const uint64_t*>(out + (pos & ~7ULL)) & ((1ULL << (8 * fill)) - 1ULL);
+    else low = tail_bytes(len_kind[perm[i - 1]] >> 30, fill);
+  }
+  GlobalWriter w;
+  w.begin(out, pos, low);
+  format_activity(w, m, ctx);
+  if (w.fill && i + 1 == n_rows) { /* last activity: merge with the suffix bytes behind it */
+    const uint64_t mask = (1ULL << (8 * w.fill)) - 1ULL;
+    *w.wptr = (*w.wptr & ~mask) | (w.acc & mask);
+  }
+}
+hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint32_t* len_kind,
+                       uint64_t n_rows, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st) {
+  if (n_rows == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_emit_direct, dim3(grid_for(n_rows, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, mat, perm, offs, len_kind,
+                     n_rows, ctx, out, prefix_len);
+  return KTJ_LAUNCH_CHECK();
+}
+
 uint32_t emit_tile_bytes(uint64_t act_bytes, uint64_t n_rows) {
   if (const char* e = getenv("KTJ_EMIT_TILE")) return (uint32_t)atoi(e);
   /* about 0.85 activities per lane, in steps of 4 KiB, between 8 and 40 KiB */

@@ -217,7 +217,7 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   append_trace_end(suffix, s->end_time_ns, s->base_time_ns, s->trace_name);
 
   const uint64_t total = prefix.size() + act_bytes + suffix.size();
-  char* buf = (char*)malloc(total ? total : 1);
+  char* buf = (char*)aligned_alloc(64, (total + 64 + 63) / 64 * 64);
   if (!buf) return -1;
   memset(buf, '#', total);
   memcpy(buf, prefix.data(), prefix.size());
@@ -226,6 +226,36 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   // output-partitioned tiles, exactly as the emit kernel lays them out: tile k owns the
   // document bytes [k*T, (k+1)*T) clipped to the activity section; tile-local coordinate
   // L = absolute offset - k*T
+  if (tile_bytes == 0) {
+    // direct variant: one "lane" per activity, aligned 8-byte stores; the buffer is over-allocated
+    // so that aligned accesses at the end stay inside it
+    std::vector<uint32_t> kinds(perm.size());
+    for (size_t i = 0; i < perm.size(); ++i) {
+      const MatRow& m = mat[perm[i]];
+      kinds[i] = tail_kind(m, m.ext != 0 || has_fragment(m, ctx));
+    }
+    const uint64_t P = prefix.size();
+    for (size_t i = 0; i < perm.size(); ++i) {
+      const uint64_t pos = P + offs[i];
+      const uint32_t fill = (uint32_t)(pos & 7);
+      uint64_t low = 0;
+      if (fill) {
+        if (i == 0) { uint64_t cur; memcpy(&cur, buf + (pos & ~7ULL), 8); low = cur & ((1ULL << (8 * fill)) - 1); }
+        else low = tail_bytes(kinds[i - 1], fill);
+      }
+      GlobalWriter w;
+      w.begin(buf, pos, low);
+      format_activity(w, mat[perm[i]], ctx);
+      if ((uint64_t)((char*)w.wptr - buf) + w.fill != P + offs[i + 1]) { free(buf); return -2; }
+      if (w.fill && i + 1 == perm.size()) {
+        const uint64_t mask = (1ULL << (8 * w.fill)) - 1;
+        *w.wptr = (*w.wptr & ~mask) | (w.acc & mask);
+      }
+    }
+    *out = buf;
+    *out_n = total;
+    return 0;
+  }
   const uint64_t T = tile_bytes;
   if (T % 8) { free(buf); return -3; }
   std::vector<uint64_t> tile_store(T / 8 + 1);

@@ -61,7 +61,7 @@ def sim():
 
 
 @pytest.mark.parametrize("cfg,n,tile", [(1, 5000, 16384), (2, 9000, 16384), (3, 12000, 4096), (4, 12000, 16384),
-                                        (5, 1500, 16384), (5, 700, 336), (1, 300, 24)])
+                                        (5, 1500, 16384), (5, 700, 336), (1, 300, 24), (3, 9000, 0), (5, 900, 0), (2, 7000, 0), (4, 9000, 0)])
 def test_formatting_core_host_build_matches_oracle(sim, cfg, n, tile):
     sp, release = abi.synth_stream(cfg, n, host_name="box")
     o = og.OracleRun(sp)
