@@ -20,6 +20,11 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per k_emit_direct launch, from two separate `rocprofv3 --pmc` runs of this script
+# (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter reads for the 1 GiB
+# k_copy_reference launch at the end of the run (2048 and 1024 bytes per unit).  Keyed by
+# (configuration, device rows); a counter run cannot share a process with the timed run.
+MEASURED_EMIT_TRAFFIC = {(3, 10000000): 5.05e9 + 20.95e9}
 FULL_SIZE = {1: 10000, 2: 1000000, 3: 10000000, 4: 11000000, 5: 5000000}
 WORKLOAD = {
     1: "config1: 10k CPU ops + 10k launches + 10k kernels, 4 streams",
@@ -70,6 +75,8 @@ def main():
     ap.add_argument("--n-device", type=int, default=0, help="device rows (0 = the configuration's full size)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="device rows of the CPU-baseline sample (0 = auto)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-bytes", type=int, default=1 << 30, help="size of the reference copy kernel run (0 = skip)")
+    ap.add_argument("--traffic", type=str, default="", help="JSON file with measured HBM bytes per emit launch (from rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path runs on exactly one GPU (no sharding, no collectives); use --gpus 1",
@@ -130,6 +137,11 @@ def main():
         host_copy_ok = False
     d2h_s = time.perf_counter() - t0
     d2h_ms = eng.stats().stage_ms[8] if host_copy_ok else None
+    copy_gbs = None
+    if args.copy_bytes:
+        ms = C.c_float()
+        if eng.lib.ktj_debug_copy_reference(eng.h, args.copy_bytes, C.byref(ms)) == 0 and ms.value > 0:
+            copy_gbs = 2 * args.copy_bytes / (ms.value * 1e-3) / 1e9   # read + write
     eng.close()
 
     emit_ms = stage_ms.get("emit", 0.0)
@@ -148,22 +160,28 @@ def main():
         "vs_baseline": None,
         "dtype": "u8/int64",
         "data": "synthetic",
-        "config": {"workload": WORKLOAD[cfg], "records": int(n_records), "device_rows": int(s.n_device) if False else int(n_dev),
+        "config": {"workload": WORKLOAD[cfg], "records": int(n_records), "device_rows": int(n_dev),
                    "output_bytes": int(out_bytes), "raw_input_bytes": int(raw_bytes),
                    "output_placement": "device buffer (HBM)"},
         "output_gb_per_s": out_bytes / (ms_per_step * 1e-3) / 1e9,
         "output_frac_of_hbm_peak": out_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "stage_ms": stage_ms,
         "stage_algorithmic_gb_per_s": stage_gbs,
-        "roofline": {"bound": "hbm", "kernel": "k_emit", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "roofline": {"bound": "hbm", "kernel": "k_emit_direct", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": emit_alg, "avg_launch_ms": emit_ms},
         "pcie": {"h2d_submit_s": h2d_s, "d2h_document_ms": d2h_ms, "d2h_wall_s": d2h_s,
                  "records_per_s_incl_d2h": (n_records / (ms_per_step * 1e-3 + (d2h_ms or 0) * 1e-3)) if d2h_ms else None},
         "generate_s": gen_s,
+        "copy_kernel_gb_per_s": copy_gbs,
     }
+    if copy_gbs:
+        result["roofline"]["frac_of_copy_kernel"] = achieved / copy_gbs
+    result["roofline"]["traffic"] = MEASURED_EMIT_TRAFFIC.get((cfg, n_dev))
+    if args.traffic and os.path.exists(args.traffic):
+        result["roofline"]["traffic"] = json.load(open(args.traffic)).get("emit_hbm_bytes_per_launch")
     if not args.no_cpu_baseline:
-        sample = args.cpu_sample or max(1000, min(n_dev, {1: 10000, 2: 400000, 3: 400000, 4: 800000, 5: 150000}[cfg]))
+        sample = args.cpu_sample or max(1000, min(n_dev, {1: 10000, 2: 1000000, 3: 2500000, 4: 4000000, 5: 1000000}[cfg]))
         result["cpu_baseline"] = cpu_baseline(cfg, sample)
     print(json.dumps(result))
 

@@ -325,8 +325,12 @@ typedef struct ktj_engine ktj_engine;
  * `if (!traceOf_) return;`; ktj_finalize then returns KTJ_ERR_IO.
  * With KTJ_CREATE_NO_FILE no file is opened or written: the document stays in the engine's
  * buffers (ktj_output_device / ktj_output_host) and out_path is only the "traceName".
+ * KTJ_CREATE_TILE_EMIT selects the output-partitioned emit kernel (one workgroup per tile of
+ * output bytes, staged in LDS) instead of the default one-lane-per-activity kernel; both produce
+ * the same bytes.
  * ---------------------------------------------------------------------------------------- */
 #define KTJ_CREATE_NO_FILE 0x1u
+#define KTJ_CREATE_TILE_EMIT 0x2u
 int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int hip_device,
                uint32_t flags);
 void ktj_destroy(ktj_engine* e);

@@ -33,6 +33,10 @@ enum {
  * ktj_process. */
 int ktj_debug_fetch(ktj_engine* e, int what, void* dst, uint64_t cap, uint64_t* n_bytes);
 
+/* Runs a plain device-to-device copy kernel of n_bytes (16 bytes per lane) twice and reports the
+ * second run's time: the achievable-bandwidth yardstick and the scale for the HBM counters. */
+int ktj_debug_copy_reference(ktj_engine* e, uint64_t n_bytes, float* ms);
+
 #ifdef __cplusplus
 }
 #endif

@@ -10,6 +10,7 @@ LIB_DIR = os.path.join(_HERE, "lib")
 
 KTJ_NONE = 0xFFFFFFFF
 KTJ_CREATE_NO_FILE = 0x1
+KTJ_CREATE_TILE_EMIT = 0x2
 
 REC_GENERIC, REC_RUNTIME, REC_DEVICE, REC_EXTCORR = 0, 1, 2, 3
 INFO_DEVICE, INFO_RESOURCE, INFO_OVERHEAD, INFO_SPAN = 0, 1, 2, 3
@@ -224,6 +225,8 @@ def load_engine():
         lib.ktj_version.argtypes = []
         lib.ktj_debug_fetch.restype = C.c_int
         lib.ktj_debug_fetch.argtypes = [vp, C.c_int, C.c_void_p, C.c_uint64, C.POINTER(C.c_uint64)]
+        lib.ktj_debug_copy_reference.restype = C.c_int
+        lib.ktj_debug_copy_reference.argtypes = [vp, C.c_uint64, C.POINTER(C.c_float)]
         _engine = lib
     return _engine
 

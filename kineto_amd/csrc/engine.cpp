@@ -574,8 +574,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(e->tile_start.ensure((emit_tile_count(e->prefix_len, act_bytes, tile) + 2) * 4));
   HIPCHK(hipEventRecord(e->ev[EV_EMIT_START], st));
   {
-    const char* mode = getenv("KTJ_EMIT_MODE"); /* "tile" selects the LDS-staged variant */
-    if (mode && strcmp(mode, "tile") == 0)
+    if (e->flags & KTJ_CREATE_TILE_EMIT)
       HIPCHK(emit(mat, e->perm, e->offs.as<uint64_t>(), N, ctx, e->out.as<char>(), e->prefix_len, act_bytes, tile,
                   e->tile_start.as<uint32_t>(), st));
     else
@@ -704,6 +703,24 @@ int ktj_finalize(ktj_engine* e, int64_t end_time_ns, uint64_t* bytes_written) {
 int ktj_get_stats(ktj_engine* e, ktj_stats* out) {
   if (!e || !out) return KTJ_ERR_ARG;
   *out = e->stats;
+  return KTJ_OK;
+}
+
+int ktj_debug_copy_reference(ktj_engine* e, uint64_t n_bytes, float* ms) {
+  if (!e || !ms) return KTJ_ERR_ARG;
+  HIPCHK(hipSetDevice(e->device));
+  DevBuf a, b;
+  HIPCHK(a.ensure(n_bytes));
+  HIPCHK(b.ensure(n_bytes));
+  HIPCHK(hipMemsetAsync(a.p, 1, n_bytes, e->stream));
+  HIPCHK(copy_reference(a.p, b.p, n_bytes, e->stream)); /* warm-up */
+  HIPCHK(hipEventRecord(e->ev_d2h[0], e->stream));
+  HIPCHK(copy_reference(a.p, b.p, n_bytes, e->stream));
+  HIPCHK(hipEventRecord(e->ev_d2h[1], e->stream));
+  HIPCHK(hipStreamSynchronize(e->stream));
+  HIPCHK(hipEventElapsedTime(ms, e->ev_d2h[0], e->ev_d2h[1]));
+  a.release();
+  b.release();
   return KTJ_OK;
 }
 

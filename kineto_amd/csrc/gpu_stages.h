@@ -71,6 +71,7 @@ struct ApiTable {
 hipError_t fill_u64(uint64_t* p, uint64_t v, uint64_t n, hipStream_t st);
 hipError_t fill_u32(uint32_t* p, uint32_t v, uint64_t n, hipStream_t st);
 hipError_t init_scalars(Scalars* s, hipStream_t st);
+hipError_t copy_reference(const void* src, void* dst, uint64_t bytes, hipStream_t st);
 
 /* exclusive scans; tmp must hold scan_tmp_elems(n) uint64 values */
 uint64_t scan_tmp_elems(uint64_t n);

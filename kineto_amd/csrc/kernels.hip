@@ -1062,7 +1062,7 @@ __global__ void k_tile_starts(const uint64_t* offs, uint64_t n, uint64_t prefix_
 
 __global__ void __launch_bounds__(EMIT_THREADS)
 k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n, EmitCtx ctx, char* out,
-       uint64_t prefix_len, uint64_t act_bytes, uint32_t tile, uint64_t first_tile, const uint32_t* start, int dbg) {
+       uint64_t prefix_len, uint64_t act_bytes, uint32_t tile, uint64_t first_tile, const uint32_t* start) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   char* buf = smem;                                                   /* tile bytes */
   CopyJob* jobs = reinterpret_cast<CopyJob*>(smem + tile);            /* EMIT_MAX_JOBS */
@@ -1094,11 +1094,11 @@ k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n
     w.buf = buf; w.size = tile;
     w.jobs = jobs; w.n_jobs = n_jobs; w.max_jobs = EMIT_MAX_JOBS;
     w.begin((int32_t)((int64_t)(o + prefix_len) - (int64_t)t0));
-    if (!(dbg & 1)) format_activity(w, m, ctx);
+    format_activity(w, m, ctx);
     w.end();
   }
   __syncthreads();
-  if (!(dbg & 2)) {
+  {
     /* string copies: one job per 16-lane group; aligned 8-byte words in the middle (two aligned
      * global loads funnel-shifted into one aligned LDS store), single bytes at both ends */
     const uint32_t nj = *n_jobs < EMIT_MAX_JOBS ? *n_jobs : EMIT_MAX_JOBS;
@@ -1139,7 +1139,6 @@ k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n
   for (uint32_t k = pre + body * 16u + threadIdx.x; k < nbytes; k += EMIT_THREADS) g[k] = s[k];
 }
 
-static int dbg_flags() { const char* e = getenv("KTJ_DBG"); return e ? atoi(e) : 0; }
 /* Direct variant: one lane per activity, aligned 8-byte stores straight into the document, no
  * LDS.  Lane i owns every word that starts inside its activity, including the one it shares
  * with activity i+1's predecessor bytes... i.e. the first word of an activity is written by that
@@ -1172,13 +1171,24 @@ k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, con
 hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint32_t* len_kind,
                        uint64_t n_rows, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st) {
   if (n_rows == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_emit_direct, dim3(grid_for(n_rows, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, mat, perm, offs, len_kind,
-                     n_rows, ctx, out, prefix_len);
+  hipLaunchKernelGGL(k_emit_direct, dim3(grid_for(n_rows, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, mat, perm, offs,
+                     len_kind, n_rows, ctx, out, prefix_len);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* plain 16-byte-per-lane copy of known size: the yardstick for the HBM counters */
+__global__ void k_copy_reference(const uint4* src, uint4* dst, uint64_t n16) {
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+hipError_t copy_reference(const void* src, void* dst, uint64_t bytes, hipStream_t st) {
+  const uint64_t n16 = bytes / 16;
+  if (n16 == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_copy_reference, dim3(grid_stride_for(n16, KTJ_BLOCK * 4)), dim3(KTJ_BLOCK), 0, st,
+                     static_cast<const uint4*>(src), static_cast<uint4*>(dst), n16);
   return KTJ_LAUNCH_CHECK();
 }
 
 uint32_t emit_tile_bytes(uint64_t act_bytes, uint64_t n_rows) {
-  if (const char* e = getenv("KTJ_EMIT_TILE")) return (uint32_t)atoi(e);
   /* about 0.85 activities per lane, in steps of 4 KiB, between 8 and 40 KiB */
   const uint64_t avg = n_rows ? act_bytes / n_rows : 512;
   uint64_t t = (avg * EMIT_THREADS * 85 / 100 + 4095) / 4096 * 4096;
@@ -1200,7 +1210,7 @@ hipError_t emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, u
                      prefix_len, tile, first_tile, tiles, tile_start);
   const size_t lds = (size_t)tile + EMIT_MAX_JOBS * sizeof(CopyJob) + 16;
   hipLaunchKernelGGL(k_emit, dim3(tiles), dim3(EMIT_THREADS), lds, st, mat, perm, offs, n, ctx, out, prefix_len,
-                     act_bytes, tile, first_tile, (const uint32_t*)tile_start, dbg_flags());
+                     act_bytes, tile, first_tile, (const uint32_t*)tile_start);
   return KTJ_LAUNCH_CHECK();
 }
 
