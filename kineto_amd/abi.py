@@ -9,6 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_DIR = os.path.join(_HERE, "lib")
 
 KTJ_NONE = 0xFFFFFFFF
+KTJ_OK, KTJ_ERR_ARG, KTJ_ERR_STATE, KTJ_ERR_HIP, KTJ_ERR_IO, KTJ_ERR_NOMEM, KTJ_ERR_LIMIT = 0, -1, -2, -3, -4, -5, -6
 KTJ_CREATE_NO_FILE = 0x1
 KTJ_CREATE_TILE_EMIT = 0x2
 

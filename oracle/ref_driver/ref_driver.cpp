@@ -28,101 +28,11 @@
 
 using namespace libkineto;
 
+#include "mat_activity.h"
+
+using namespace ktj_ref_driver;
+
 namespace {
-
-typedef void (*string_fn)(const void* ctx, uint32_t id, const char** p, uint64_t* n);
-
-struct StringTable {
-  string_fn fn;
-  const void* ctx;
-  std::string get(uint32_t id) const {
-    const char* p = nullptr;
-    uint64_t n = 0;
-    fn(ctx, id, &p, &n);
-    return std::string(p, n);
-  }
-};
-
-// ITraceActivity over one materialised activity.  metadataJson() feeds the typed values, in
-// visit order, through the reference's JsonTypedMetadataVisitor.
-struct MatActivity : public ITraceActivity {
-  const ktj_mat_activity* a;
-  const StringTable* st;
-  mutable GenericTraceActivity linkedStub;  // only correlationId()/name() are read from it
-  bool hasLinked;
-
-  MatActivity(const ktj_mat_activity* act, const StringTable* s) : a(act), st(s), hasLinked(act->has_linked != 0) {
-    linkedStub.id = static_cast<int32_t>(act->linked_corr);
-    linkedStub.activityName = "linked_op";
-  }
-  int64_t deviceId() const override { return a->device; }
-  int64_t resourceId() const override { return a->resource; }
-  int32_t getThreadId() const override { return 0; }
-  int64_t timestamp() const override { return a->ts; }
-  int64_t duration() const override { return a->dur; }
-  int64_t correlationId() const override { return a->corr; }
-  int flowType() const override { return a->flow_type; }
-  int64_t flowId() const override { return a->flow_id; }
-  bool flowStart() const override { return a->flow_start != 0; }
-  ActivityType type() const override { return static_cast<ActivityType>(a->type); }
-  const std::string name() const override { return st->get(a->name_id); }
-  const ITraceActivity* linkedActivity() const override { return hasLinked ? &linkedStub : nullptr; }
-  const TraceSpan* traceSpan() const override { return nullptr; }
-  void log(ActivityLogger& logger) const override { logger.handleActivity(*this); }
-
-  void visitTypedMetadata(ITypedMetadataVisitor& visitor) const override {
-    const uint64_t* slot = a->slots;
-    std::vector<std::string> keep;  // MetadataField holds a string_view
-    keep.reserve(a->n_fields);
-    for (uint32_t f = 0; f < a->n_fields; ++f) {
-      const ktj_field& fd = a->fields[f];
-      keep.push_back(fd.key_id == KTJ_NONE ? std::string() : st->get(fd.key_id));
-      const std::string& key = keep.back();
-      switch (fd.type) {
-        case KTJ_F_I64:
-          visitor.visit(MetadataField<int64_t>{key}, static_cast<int64_t>(slot[0]));
-          break;
-        case KTJ_F_U64:
-          visitor.visit(MetadataField<uint64_t>{key}, static_cast<uint64_t>(slot[0]));
-          break;
-        case KTJ_F_F64: {
-          double d;
-          std::memcpy(&d, &slot[0], 8);
-          visitor.visit(MetadataField<double>{key}, d);
-          break;
-        }
-        case KTJ_F_BOOL:
-          visitor.visit(MetadataField<bool>{key}, slot[0] != 0);
-          break;
-        case KTJ_F_STR:
-          visitor.visit(MetadataField<std::string>{key}, st->get(static_cast<uint32_t>(slot[0])));
-          break;
-        case KTJ_F_RAW:
-          visitor.visit(MetadataField<RawJson>{key}, RawJson{st->get(static_cast<uint32_t>(slot[0]))});
-          break;
-        case KTJ_F_I64_ARRAY: {
-          std::vector<int64_t> v(fd.count);
-          for (uint32_t k = 0; k < fd.count; ++k) v[k] = static_cast<int64_t>(slot[k]);
-          visitor.visit(MetadataField<std::vector<int64_t>>{key}, v);
-          break;
-        }
-        default:
-          break;
-      }
-      slot += fd.count;
-    }
-  }
-  const std::string metadataJson() const override {
-    // A field without a key stands for a whole pre-rendered fragment (what an activity's own
-    // metadataJson() returned); it is passed through untouched.
-    if (a->n_fields == 1 && a->fields[0].key_id == KTJ_NONE) {
-      return st->get(static_cast<uint32_t>(a->slots[0]));
-    }
-    libkineto::internal::JsonTypedMetadataVisitor visitor;
-    visitTypedMetadata(visitor);
-    return std::move(visitor).json();
-  }
-};
 
 // Exposes the protected finalizeTrace(int64_t) so that no Config object is needed.
 struct RefLogger : public ChromeTraceLogger {
@@ -143,42 +53,8 @@ int ktj_ref_render(const ktj_stream* s, const ktj_mat_activity* acts, uint64_t n
                    const void* ctx, const char* out_path) {
   SET_LOG_SEVERITY_LEVEL(3);  // ERROR: silence per-name WARNING lines
   if (s->base_time_ns != ChromeTraceBaseTime::singleton().get()) return -2;
-  StringTable st{fn, ctx};
-  std::vector<MatActivity> wrapped;
-  wrapped.reserve(n_acts);
-  for (uint64_t i = 0; i < n_acts; ++i) wrapped.emplace_back(&acts[i], &st);
-  std::vector<const MatActivity*> order(n_acts);
-  for (uint64_t i = 0; i < n_acts; ++i) order[i] = &wrapped[i];
-  std::stable_sort(order.begin(), order.end(), [](const MatActivity* x, const MatActivity* y) {
-    return std::make_tuple(x->deviceId(), x->resourceId(), x->timestamp()) <
-        std::make_tuple(y->deviceId(), y->resourceId(), y->timestamp());
-  });
-
   RefLogger logger{std::string(out_path)};
-  std::unordered_map<std::string, std::string> metadata;  // env metadata (host_name) is added by the logger
-  logger.handleTraceStart(metadata, s->device_properties ? s->device_properties : "");
-  for (uint64_t i = 0; i < s->n_device_infos; ++i) {
-    const ktj_device_info& d = s->device_infos[i];
-    logger.handleDeviceInfo({d.id, d.sort_index, d.name, d.label}, d.time_ns);
-  }
-  for (uint64_t i = 0; i < s->n_resource_infos; ++i) {
-    const ktj_resource_info& r = s->resource_infos[i];
-    logger.handleResourceInfo(
-        {r.id, r.sort_index, r.device_id, r.name, r.host_thread ? ResourceType::HOST_THREAD : ResourceType::UNKNOWN},
-        r.time_ns);
-  }
-  for (uint64_t i = 0; i < s->n_overhead_infos; ++i) {
-    logger.handleOverheadInfo(ActivityLogger::OverheadInfo(s->overhead_infos[i].name), s->overhead_infos[i].time_ns);
-  }
-  for (const MatActivity* a : order) a->log(logger);
-  for (uint64_t i = 0; i < s->n_spans; ++i) {
-    const ktj_trace_span& sp = s->spans[i];
-    TraceSpan span(sp.op_count, sp.iteration, sp.name, sp.prefix);
-    span.startTime = sp.start_ns;
-    span.endTime = sp.end_ns;
-    logger.handleTraceSpan(span);
-  }
-  logger.finalizeTrace(s->end_time_ns);
+  replay_stream(logger, s, acts, n_acts, fn, ctx);
   return 0;
 }
 

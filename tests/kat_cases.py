@@ -142,3 +142,29 @@ def case_rocm_sync_trace():
 
 SUBSTRING_CASES = [case_logger_events, case_trace_span, case_benchmark_cpu_op, case_typed_kernel_args,
                    case_typed_metadata_pins, case_names, case_resource_infos]
+
+
+def build_for_real_logger(case, ref_args):
+    """Builds a hand-made case so that the real logger can render it: every absolute time is
+    shifted by the difference between the real logger's base time (wall clock, `ref_args` from
+    oracle_glue.ref_stream_args()) and the default one, and the header carries this machine's
+    host name."""
+    import stream_builder
+    delta = ref_args["base_time_ns"] - stream_builder.B
+    b, _ = case()
+    b.base += delta
+    b.window = (b.window[0] + delta, b.window[1] + delta)
+    b.end_time += delta
+    for r in b.generic:
+        r.start_ns += delta; r.end_ns += delta
+    for r in b.runtime:
+        r.begin += delta; r.end += delta
+    for r in b.device:
+        r.begin += delta; r.end += delta
+    for lst in (b.device_infos, b.resource_infos, b.overhead_infos):
+        for x in lst:
+            x.time_ns += delta
+    for x in b.spans:
+        x.start_ns += delta; x.end_ns += delta
+    b.meta = [("host_name", '"%s"' % ref_args["host_name"])]
+    return b.build()

@@ -10,6 +10,7 @@ from kineto_amd import abi
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_SO = os.path.join(ROOT, "oracle", "libktj_oracle.so")
 REF_SO = os.path.join(ROOT, "oracle", "_ref", "libktj_ref.so")
+SHIM_SO = os.path.join(ROOT, "oracle", "_ref", "libktj_shim_test.so")
 
 
 class MatActivity(C.Structure):
@@ -23,6 +24,7 @@ class MatActivity(C.Structure):
 
 _oracle = None
 _ref = None
+_shim = None
 
 
 def load_oracle():
@@ -88,6 +90,25 @@ def load_ref():
     return _ref
 
 
+def have_shim():
+    return os.path.exists(SHIM_SO)
+
+
+def load_shim():
+    """The ActivityLogger shim (kineto_amd/shim) built against the reference's headers, plus its
+    replay driver.  Links the engine library, so it is only loaded where a GPU is present."""
+    global _shim
+    if _shim is None:
+        abi.load_engine()
+        lib = C.CDLL(SHIM_SO)
+        lib.ktj_shim_base_time.restype = C.c_int64
+        lib.ktj_shim_render.restype = C.c_int
+        lib.ktj_shim_render.argtypes = [C.POINTER(abi.Stream), C.POINTER(MatActivity), C.c_uint64,
+                                        C.c_void_p, C.c_void_p, C.c_char_p, C.c_int, C.POINTER(C.c_uint64)]
+        _shim = lib
+    return _shim
+
+
 class OracleRun:
     """Runs the oracle on a stream; exposes output bytes, activities and counters."""
 
@@ -149,6 +170,26 @@ def ref_render(stream_ptr, oracle_run):
             data = f.read()
     # The real logger prints the path it was given as "traceName"; the stream carries the bare name.
     return data.replace(path.encode(), stream_ptr.contents.trace_name)
+
+
+def shim_render(stream_ptr, oracle_run, protocol="gpujson", directory=None):
+    """Renders the stream through the GpuChromeTraceLogger shim obtained from a logger factory by
+    URL, fed with the same activities as ref_render.  Returns (status, bytes or None, dropped)."""
+    shim = load_shim()
+    acts, n = oracle_run.activities()
+    fn = C.cast(load_oracle().ktj_oracle_string, C.c_void_p)
+    dropped = C.c_uint64()
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(directory or d, stream_ptr.contents.trace_name.decode())
+        url = f"{protocol}://{path}"
+        rc = shim.ktj_shim_render(stream_ptr, acts, n, fn, oracle_run.h, url.encode(), 0, C.byref(dropped))
+        data = None
+        if rc == 0:
+            with open(path, "rb") as f:
+                data = f.read()
+            assert not os.path.exists(path + ".tmp")
+            data = data.replace(path.encode(), stream_ptr.contents.trace_name)
+    return rc, data, dropped.value
 
 
 def ref_stream_args():

@@ -1,0 +1,67 @@
+"""GPU: the libkineto ActivityLogger shim (kineto_amd/shim/GpuChromeTraceLogger) against the
+reference's own ChromeTraceLogger.  Both loggers are fed the same libkineto::ITraceActivity objects
+through the same calls (handleTraceStart, handle*Info, handleActivity, handleTraceSpan,
+finalizeTrace); the shim is obtained from an ActivityLoggerFactory by URL.  The two files must be
+byte-identical.  Needs oracle/_ref (built where the reference sources are available)."""
+import pytest
+
+import kat_cases
+import oracle_glue as og
+from kineto_amd import abi
+
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skipif(not (og.have_ref() and og.have_shim()), reason="oracle/_ref not built")]
+
+
+def _first_diff(a, b):
+    n = min(len(a), len(b))
+    for i in range(0, n, 4096):
+        if a[i:i + 4096] != b[i:i + 4096]:
+            for k in range(i, min(i + 4096, n)):
+                if a[k] != b[k]:
+                    return k
+    return n
+
+
+def _compare(sp):
+    o = og.OracleRun(sp)
+    try:
+        theirs = og.ref_render(sp, o)
+        rc, mine, dropped = og.shim_render(sp, o)
+        mixed_case_rc, mixed, _ = og.shim_render(sp, o, protocol="GPUJSON")
+    finally:
+        o.close()
+    assert rc == 0 and dropped == 0
+    if mine != theirs:
+        i = _first_diff(mine, theirs)
+        raise AssertionError(f"byte {i} of {len(theirs)}: shim {mine[max(0, i - 80):i + 80]!r} "
+                             f"reference {theirs[max(0, i - 80):i + 80]!r}")
+    assert mixed_case_rc == 0 and mixed == theirs  # protocol lookup is case-insensitive
+
+
+@pytest.mark.parametrize("cfg,n", [(1, 10000), (2, 20000), (3, 30000), (4, 30000), (5, 4000), (1, 1), (2, 7)])
+def test_shim_matches_reference_logger(cfg, n):
+    sp, release = abi.synth_stream(cfg, n, **og.ref_stream_args())
+    try:
+        _compare(sp)
+    finally:
+        release()
+
+
+@pytest.mark.parametrize("case", kat_cases.SUBSTRING_CASES + [kat_cases.case_rocm_sync_trace], ids=lambda c: c.__name__)
+def test_shim_hand_made_cases(case):
+    sp = kat_cases.build_for_real_logger(case, og.ref_stream_args())
+    _compare(sp)
+
+
+def test_shim_unknown_protocol_and_bad_sink():
+    sp, release = abi.synth_stream(1, 50, **og.ref_stream_args())
+    o = og.OracleRun(sp)
+    try:
+        rc, data, _ = og.shim_render(sp, o, protocol="nosuch")
+        assert rc == -3 and data is None          # factory: no logger for that prefix
+        rc, data, _ = og.shim_render(sp, o, directory="/nonexistent-dir/sub")
+        assert rc == abi.KTJ_ERR_IO and data is None  # bad sink: handlers are no-ops, finalize reports
+    finally:
+        o.close()
+        release()

@@ -28,29 +28,7 @@ def test_synthetic_configs_byte_identical(cfg, n):
 
 @pytest.mark.parametrize("case", kat_cases.SUBSTRING_CASES + [kat_cases.case_rocm_sync_trace], ids=lambda c: c.__name__)
 def test_hand_made_cases_byte_identical(case):
-    import socket
-    import stream_builder
-    args = og.ref_stream_args()
-    old_b = stream_builder.B
-    delta = args["base_time_ns"] - old_b
-    b, _ = case()
-    # shift every absolute time by the difference between the real logger's base and the default one
-    b.base += delta
-    b.window = (b.window[0] + delta, b.window[1] + delta)
-    b.end_time += delta
-    for r in b.generic:
-        r.start_ns += delta; r.end_ns += delta
-    for r in b.runtime:
-        r.begin += delta; r.end += delta
-    for r in b.device:
-        r.begin += delta; r.end += delta
-    for lst in (b.device_infos, b.resource_infos, b.overhead_infos):
-        for x in lst:
-            x.time_ns += delta
-    for x in b.spans:
-        x.start_ns += delta; x.end_ns += delta
-    b.meta = [("host_name", '"%s"' % socket.gethostname())]
-    sp = b.build()
+    sp = kat_cases.build_for_real_logger(case, og.ref_stream_args())
     o = og.OracleRun(sp)
     mine = o.output()
     theirs = og.ref_render(sp, o)
