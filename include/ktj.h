@@ -328,9 +328,12 @@ typedef struct ktj_engine ktj_engine;
  * KTJ_CREATE_TILE_EMIT selects the output-partitioned emit kernel (one workgroup per tile of
  * output bytes, staged in LDS) instead of the default one-lane-per-activity kernel; both produce
  * the same bytes.
+ * KTJ_CREATE_HASH_JOIN keeps the join tables in hash mode even when the correlation ids are dense
+ * enough for direct addressing (the engine chooses per table otherwise); same results, slower.
  * ---------------------------------------------------------------------------------------- */
 #define KTJ_CREATE_NO_FILE 0x1u
 #define KTJ_CREATE_TILE_EMIT 0x2u
+#define KTJ_CREATE_HASH_JOIN 0x4u
 int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int hip_device,
                uint32_t flags);
 void ktj_destroy(ktj_engine* e);

@@ -12,6 +12,7 @@ KTJ_NONE = 0xFFFFFFFF
 KTJ_OK, KTJ_ERR_ARG, KTJ_ERR_STATE, KTJ_ERR_HIP, KTJ_ERR_IO, KTJ_ERR_NOMEM, KTJ_ERR_LIMIT = 0, -1, -2, -3, -4, -5, -6
 KTJ_CREATE_NO_FILE = 0x1
 KTJ_CREATE_TILE_EMIT = 0x2
+KTJ_CREATE_HASH_JOIN = 0x4
 
 REC_GENERIC, REC_RUNTIME, REC_DEVICE, REC_EXTCORR = 0, 1, 2, 3
 INFO_DEVICE, INFO_RESOURCE, INFO_OVERHEAD, INFO_SPAN = 0, 1, 2, 3

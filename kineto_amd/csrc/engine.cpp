@@ -114,7 +114,7 @@ struct ktj_engine {
   /* working buffers */
   DevBuf d_scalars, d_name_len, d_arg_len, d_sflags, d_name_off, d_arg_off, d_name_blob, d_arg_blob;
   DevBuf c_ts, c_dur, c_corr, c_dev, c_res, c_meta, c_ext;
-  DevBuf t_ext_k, t_ext_v, t_cpu_k, t_id_k, t_id_v0, t_id_v1, t_nr_k, t_nr_v0, t_nr_v1;
+  DevBuf t_full, t_narrow, t_cpu, slot_ext, slot_f, slot_n, slot_f_dev, dev_link, dev_brief;
   DevBuf q_keys, q_stream, q_amb, dn_hash, dn_first, dn_dev, dn_key, dn_rank;
   DevBuf s_dev_k, s_dev_r, s_res_k, s_res_r;
   DevBuf keys_a, keys_b, vals_a, vals_b, hist, scan_tmp;
@@ -201,9 +201,8 @@ void ktj_destroy(ktj_engine* e) {
   if (e->stream) (void)hipStreamSynchronize(e->stream);
   DevBuf* bufs[] = {&e->d_fields, &e->d_schemas, &e->d_cid_names, &e->d_flow_bits, &e->d_scalars, &e->d_name_len,
                     &e->d_arg_len, &e->d_sflags, &e->d_name_off, &e->d_arg_off, &e->d_name_blob, &e->d_arg_blob,
-                    &e->c_ts, &e->c_dur, &e->c_corr, &e->c_dev, &e->c_res, &e->c_meta, &e->c_ext, &e->t_ext_k,
-                    &e->t_ext_v, &e->t_cpu_k, &e->t_id_k, &e->t_id_v0, &e->t_id_v1, &e->t_nr_k, &e->t_nr_v0,
-                    &e->t_nr_v1, &e->q_keys, &e->q_stream, &e->q_amb, &e->dn_hash, &e->dn_first, &e->dn_dev,
+                    &e->c_ts, &e->c_dur, &e->c_corr, &e->c_dev, &e->c_res, &e->c_meta, &e->c_ext, &e->t_full,
+                    &e->t_narrow, &e->t_cpu, &e->slot_ext, &e->slot_f, &e->slot_n, &e->slot_f_dev, &e->dev_link, &e->dev_brief, &e->q_keys, &e->q_stream, &e->q_amb, &e->dn_hash, &e->dn_first, &e->dn_dev,
                     &e->dn_key, &e->dn_rank, &e->s_dev_k, &e->s_dev_r, &e->s_res_k, &e->s_res_r, &e->keys_a,
                     &e->keys_b, &e->vals_a, &e->vals_b, &e->hist, &e->scan_tmp, &e->mat, &e->len, &e->len_sorted,
                     &e->offs, &e->out, &e->tile_start};
@@ -398,14 +397,15 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(e->c_ts.ensure(Na * 8)); HIPCHK(e->c_dur.ensure(Na * 8)); HIPCHK(e->c_corr.ensure(Na * 8));
   HIPCHK(e->c_dev.ensure(Na * 8)); HIPCHK(e->c_res.ensure(Na * 8)); HIPCHK(e->c_meta.ensure(Na * 4));
   HIPCHK(e->c_ext.ensure(Na * 4));
-  const uint32_t cap_ext = pow2_at_least(2 * nx), cap_cpu = pow2_at_least(2 * ng);
-  const uint32_t cap_id = pow2_at_least(2 * (nr + nd)), cap_nr = pow2_at_least(2 * nr);
-  HIPCHK(e->t_ext_k.ensure((cap_ext + 1ull) * 8)); HIPCHK(e->t_ext_v.ensure((cap_ext + 1ull) * 4));
-  HIPCHK(e->t_cpu_k.ensure((cap_cpu + 1ull) * 8));
-  HIPCHK(e->t_id_k.ensure((cap_id + 1ull) * 8)); HIPCHK(e->t_id_v0.ensure((cap_id + 1ull) * 4));
-  HIPCHK(e->t_id_v1.ensure((cap_id + 1ull) * 4));
-  HIPCHK(e->t_nr_k.ensure((cap_nr + 1ull) * 8)); HIPCHK(e->t_nr_v0.ensure((cap_nr + 1ull) * 4));
-  HIPCHK(e->t_nr_v1.ensure((cap_nr + 1ull) * 4));
+  /* capacities for the hash mode (load <= 2/3); the direct mode uses a prefix of the same buffers */
+  const uint32_t cap_full = pow2_at_least((nr + nd) + (nr + nd) / 2);
+  const uint32_t cap_narrow = pow2_at_least((nx + nr) + (nx + nr) / 2), cap_cpu = pow2_at_least(2 * ng);
+  HIPCHK(e->t_full.ensure((cap_full + 1ull) * sizeof(FullSlot)));
+  HIPCHK(e->t_narrow.ensure((cap_narrow + 1ull) * sizeof(NarrowSlot)));
+  HIPCHK(e->t_cpu.ensure((cap_cpu + 1ull) * sizeof(KeySlot)));
+  HIPCHK(e->slot_ext.ensure(nx * 4 + 16)); HIPCHK(e->slot_f.ensure(nr * 4 + 16)); HIPCHK(e->slot_n.ensure(nr * 4 + 16));
+  HIPCHK(e->slot_f_dev.ensure(nd * 4 + 16)); HIPCHK(e->dev_link.ensure(nd * sizeof(DevLink) + 16));
+  HIPCHK(e->dev_brief.ensure(nd * sizeof(DevBrief) + 16));
   HIPCHK(e->q_keys.ensure((KTJ_QUEUE_CAP + 1ull) * 8)); HIPCHK(e->q_stream.ensure((KTJ_QUEUE_CAP + 1ull) * 8));
   HIPCHK(e->q_amb.ensure((KTJ_QUEUE_CAP + 1ull) * 4));
   HIPCHK(e->dn_hash.ensure((KTJ_DENSE_CAP + 1ull) * 8)); HIPCHK(e->dn_first.ensure((KTJ_DENSE_CAP + 1ull) * 4));
@@ -474,29 +474,30 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(hipEventRecord(e->ev[EV_CONVERT], st));
 
   /* ---- stage 2b: joins ---- */
-  Table t_ext{e->t_ext_k.as<uint64_t>(), e->t_ext_v.as<uint32_t>(), nullptr, cap_ext - 1};
-  Table t_cpu{e->t_cpu_k.as<uint64_t>(), nullptr, nullptr, cap_cpu - 1};
-  Table t_id{e->t_id_k.as<uint64_t>(), e->t_id_v0.as<uint32_t>(), e->t_id_v1.as<uint32_t>(), cap_id - 1};
-  Table t_nr{e->t_nr_k.as<uint64_t>(), e->t_nr_v0.as<uint32_t>(), e->t_nr_v1.as<uint32_t>(), cap_nr - 1};
-  HIPCHK(fill_u64(t_ext.keys, KTJ_EMPTY_KEY, cap_ext + 1ull, st)); HIPCHK(fill_u32(t_ext.v0, 0, cap_ext + 1ull, st));
-  HIPCHK(fill_u64(t_cpu.keys, KTJ_EMPTY_KEY, cap_cpu + 1ull, st));
-  HIPCHK(fill_u64(t_id.keys, KTJ_EMPTY_KEY, cap_id + 1ull, st)); HIPCHK(fill_u32(t_id.v0, 0, cap_id + 1ull, st));
-  HIPCHK(fill_u32(t_id.v1, 0xFFFFFFFFu, cap_id + 1ull, st));
-  HIPCHK(fill_u64(t_nr.keys, KTJ_EMPTY_KEY, cap_nr + 1ull, st)); HIPCHK(fill_u32(t_nr.v0, 0, cap_nr + 1ull, st));
-  HIPCHK(fill_u32(t_nr.v1, 0, cap_nr + 1ull, st));
+  FullTable tf{e->t_full.as<FullSlot>(), cap_full - 1, &sc->plan.ctl[KTJ_TBL_FULL]};
+  NarrowTable tn{e->t_narrow.as<NarrowSlot>(), cap_narrow - 1, &sc->plan.ctl[KTJ_TBL_NARROW]};
+  KeyTable t_cpu{e->t_cpu.as<KeySlot>(), cap_cpu - 1, &sc->plan.ctl[KTJ_TBL_CPU]};
+  HIPCHK(plan_tables(c, ng, nr, nd, x_recs, nx, cap_full, cap_narrow, cap_cpu, (e->flags & KTJ_CREATE_HASH_JOIN) != 0, sc, st));
+  HIPCHK(clear_tables(tf, tn, t_cpu, st));
   StreamTables stt{e->q_keys.as<uint64_t>(), e->q_stream.as<uint64_t>(), e->q_amb.as<uint32_t>(), e->dn_hash.as<uint64_t>(),
                    e->dn_first.as<uint32_t>(), e->dn_dev.as<int32_t>(), e->dn_key.as<uint64_t>(), e->dn_rank.as<uint32_t>()};
   HIPCHK(fill_u64(stt.q_keys, KTJ_EMPTY_KEY, KTJ_QUEUE_CAP + 1ull, st)); HIPCHK(fill_u64(stt.q_stream, 0, KTJ_QUEUE_CAP + 1ull, st));
   HIPCHK(fill_u32(stt.q_amb, 0, KTJ_QUEUE_CAP + 1ull, st));
   HIPCHK(fill_u64(stt.d_hash, KTJ_EMPTY_KEY, KTJ_DENSE_CAP + 1ull, st)); HIPCHK(fill_u32(stt.d_first, 0xFFFFFFFFu, KTJ_DENSE_CAP + 1ull, st));
   HIPCHK(fill_u32(stt.d_rank, 0, KTJ_DENSE_CAP + 1ull, st));
-  HIPCHK(build_extcorr(x_recs, nx, t_ext, sc, st));
+  ApiTable api{e->d_cid_names.as<uint32_t>(), (uint32_t)e->cid_names.size(), e->d_flow_bits.as<uint32_t>(), e->malloc_cid};
+  MatRow* mat = e->mat.as<MatRow>();
+  HIPCHK(build_extcorr(x_recs, nx, tn, e->slot_ext.as<uint32_t>(), sc, st));
   HIPCHK(build_cpu_ids(g_recs, ng, t_cpu, sc, st));
-  HIPCHK(build_runtime(r_recs, nr, c, ng, t_id, t_nr, sc, st));
-  HIPCHK(insert_device_first(d_recs, nd, c, ng + nr, t_id, sc, st));
-  HIPCHK(probe_external(c, ng, nr + nd, x_recs, t_ext, t_cpu, sc, st));
-  HIPCHK(count_out_of_order(c, ng, nr, nd, t_id, sc, st));
-  HIPCHK(backfill_streams(d_recs, nd, r_recs, c, ng + nr, t_id, stt, sc, st));
+  HIPCHK(build_runtime(r_recs, nr, c, ng, tf, tn, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), sc, st));
+  HIPCHK(insert_device_first(d_recs, nd, c, ng + nr, tf, e->slot_f_dev.as<uint32_t>(), sc, st));
+  HIPCHK(resolve_external(x_recs, nx, tn, e->slot_ext.as<uint32_t>(), t_cpu, st));
+  /* second pass over the runtime rows: publishes into the tables and writes the joined rows */
+  HIPCHK(mat_runtime_rows(r_recs, nr, c, ng, api, tf, tn, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), ctx, mat,
+                          e->len.as<uint32_t>(), sc, st));
+  HIPCHK(link_device_rows(d_recs, nd, c, ng + nr, tf, tn, e->slot_f_dev.as<uint32_t>(), e->dev_link.as<DevLink>(),
+                          e->dev_brief.as<DevBrief>(), sc, st));
+  HIPCHK(backfill_streams(e->dev_brief.as<DevBrief>(), nd, c, ng + nr, stt, sc, st));
   HIPCHK(hipEventRecord(e->ev[EV_JOIN], st));
 
   /* ---- stage 3: canonical order ---- */
@@ -530,11 +531,8 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(hipEventRecord(e->ev[EV_SORT], st));
 
   /* ---- stage 4a: joined rows + lengths ---- */
-  ApiTable api{e->d_cid_names.as<uint32_t>(), (uint32_t)e->cid_names.size(), e->d_flow_bits.as<uint32_t>(), e->malloc_cid};
-  MatRow* mat = e->mat.as<MatRow>();
   HIPCHK(mat_generic_rows(g_recs, ng, ctx, mat, e->len.as<uint32_t>(), sc, st));
-  HIPCHK(mat_runtime_rows(r_recs, nr, c, ng, api, ctx, mat, e->len.as<uint32_t>(), sc, st));
-  HIPCHK(mat_device_rows(d_recs, nd, c, ng + nr, r_recs, t_nr, ctx, mat, e->len.as<uint32_t>(), sc, st));
+  HIPCHK(mat_device_rows(d_recs, nd, c, ng + nr, e->dev_link.as<DevLink>(), ctx, mat, e->len.as<uint32_t>(), sc, st));
   HIPCHK(gather_len(e->perm, e->len.as<uint32_t>(), N, e->len_sorted.as<uint32_t>(), st));
   HIPCHK(hipEventRecord(e->ev[EV_SIZE], st));
 
@@ -619,9 +617,11 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   s.stage_bytes[KTJ_STAGE_DICT] = e->blob_bytes * 3;
   s.stage_bytes[KTJ_STAGE_DECODE] = raw_in + N * 48;
   s.stage_bytes[KTJ_STAGE_CONVERT] = (nr + nd) * 32;
-  s.stage_bytes[KTJ_STAGE_JOIN] = nx * 12 + ng * 12 + nr * 12 + (nr + nd) * 12 * 2;
+  s.stage_bytes[KTJ_STAGE_JOIN] = nx * 12 + ng * 12 + nr * 12 + (nr + nd) * 12 * 2 +
+                                   nr * (sizeof(ktj_runtime_rec) + 48 + sizeof(MatRow) + 4); /* incl. the runtime rows' joined rows */
   s.stage_bytes[KTJ_STAGE_SORT] = N * 56;
-  s.stage_bytes[KTJ_STAGE_SIZE] = raw_in + N * 48 + N * (sizeof(MatRow) + 4);
+  s.stage_bytes[KTJ_STAGE_SIZE] = (ng * sizeof(ktj_generic_rec) + nd * sizeof(ktj_device_rec)) + (ng + nd) * 48 +
+                                   (ng + nd) * (sizeof(MatRow) + 4) + N * 8;
   s.stage_bytes[KTJ_STAGE_SCAN] = N * 12;
   s.stage_bytes[KTJ_STAGE_EMIT] = e->scalars.n_valid * (sizeof(MatRow) + 12) + act_bytes;
   e->processed = true;

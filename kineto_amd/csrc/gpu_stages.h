@@ -13,15 +13,76 @@
 namespace ktj {
 namespace gpu {
 
-/* open-addressing hash table in device memory; keys hold KTJ_EMPTY_KEY when free.  Slot `cap` (one
- * past the power-of-two range) is reserved for the key whose value equals KTJ_EMPTY_KEY. */
+/* Join tables in device memory.  A table is either direct-addressed (slot = key - base, chosen on
+ * the GPU when the keys that will be inserted span less than the capacity: correlation ids are
+ * dense counters in practice, so rows that arrive in id order touch consecutive slots and no slot
+ * is ever probed twice) or an open-addressing hash table (any other key set).  A slot is free
+ * while its key is KTJ_EMPTY_KEY; slot `cap` (one past the power-of-two range) is reserved for
+ * the key whose value equals KTJ_EMPTY_KEY.  The mode lives in device memory (TableCtl) so that
+ * no host round trip is needed to choose it. */
 #define KTJ_EMPTY_KEY 0xFFFFFFFFFFFFFFFFULL
-struct Table {
-  uint64_t* keys;
-  uint32_t* v0;
-  uint32_t* v1;
-  uint32_t mask; /* cap - 1 */
+struct KeyRange {          /* over the keys that will be inserted; empty while lo > hi */
+  unsigned long long lo, hi;
 };
+struct TableCtl {
+  uint64_t base;           /* direct mode: smallest key */
+  uint64_t span;           /* direct mode: largest key - base */
+  uint32_t direct;
+  uint32_t pad;
+};
+/* keyed by the full correlation id */
+struct FullSlot {
+  uint64_t key;
+  uint32_t stream_src;     /* last runtime row (index + 1) that carries a stream, 0 = none     */
+  uint32_t first;          /* smallest arrival index seen with this id, 0xFFFFFFFF = none      */
+  int64_t first_ts;        /* timestamp of row `first` when that is a runtime row              */
+  uint64_t stream;         /* stream of row stream_src                                          */
+};                         /* 32 bytes */
+/* keyed by the int-narrowed correlation id (and by the external-correlation records' full id) */
+struct NarrowSlot {
+  uint64_t key;
+  uint32_t ext_src;        /* last external-correlation record (index + 1), 0 = none           */
+  int32_t ext_val;         /* its external id if a CPU op with that id exists, else 0           */
+  uint32_t kern_src;       /* last in-window kernel-launch row (index + 1)                     */
+  uint32_t copy_src;       /* last in-window copy / malloc row (index + 1)                     */
+  uint64_t size;           /* bytes of row copy_src                                             */
+  uint64_t grid[3];        /* packed grid / workgroup of row kern_src (see pack_grid)           */
+  uint32_t linked;         /* 1 when ext_val names an existing CPU op                           */
+  uint32_t pad;
+};                         /* 64 bytes */
+struct KeySlot {           /* plain set */
+  uint64_t key;
+};
+template <typename S>
+struct TableT {
+  S* s;
+  uint32_t mask;           /* cap - 1, cap a power of two >= 16 */
+  const TableCtl* ctl;
+};
+typedef TableT<FullSlot> FullTable;
+typedef TableT<NarrowSlot> NarrowTable;
+typedef TableT<KeySlot> KeyTable;
+#define KTJ_TBL_FULL 0
+#define KTJ_TBL_NARROW 1
+#define KTJ_TBL_CPU 2
+struct JoinPlan {
+  KeyRange range[3];
+  TableCtl ctl[3];
+};
+/* what a device row takes over from the runtime row(s) with its correlation id */
+struct DevLink {
+  uint64_t p[3];           /* size in p[0], or packed grid / workgroup */
+  uint32_t flags;          /* KTJ_DL_* */
+  uint32_t pad;
+};                         /* 32 bytes */
+/* the fields of a device row that the stream back-fill passes read */
+struct DevBrief {
+  uint64_t queue;
+  int32_t device;
+  uint32_t domain;
+};                         /* 16 bytes */
+#define KTJ_DL_HAS_SIZE 1u
+#define KTJ_DL_HAS_GRID 2u
 
 /* columns in arrival order: generic rows, then runtime rows, then device rows */
 struct Columns {
@@ -44,12 +105,14 @@ struct Scalars {
   unsigned long long n_linked;
   unsigned long long n_blank_names;
   unsigned long long n_valid;
+  unsigned long long n_unresolved;    /* device rows still without a stream after the correlation pass */
   unsigned int error;                 /* KTJ_DEVERR_* bits */
   unsigned int have_stream_src;       /* some runtime row carries a stream */
   unsigned int n_dev_ranks;           /* distinct deviceId values */
   unsigned int n_res_ranks;           /* distinct resourceId values */
   unsigned int n_dense;               /* distinct (device, stream key) pairs */
   unsigned int pad;
+  JoinPlan plan;                      /* key ranges and modes of the join tables */
 };
 #define KTJ_DEVERR_TABLE_FULL 1u
 #define KTJ_DEVERR_TOO_MANY_DISTINCT 2u
@@ -94,16 +157,25 @@ hipError_t convert_rows(Columns c, uint64_t first_runtime, uint64_t n_runtime, u
                         int64_t win_start, int64_t win_end, Scalars* sc, hipStream_t st);
 
 /* ---- stage 2b: joins ---- */
-hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table t, Scalars* sc, hipStream_t st);
-hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table t, Scalars* sc, hipStream_t st);
-hipError_t build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, Table by_id,
-                         Table by_narrow, Scalars* sc, hipStream_t st);
-hipError_t insert_device_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, Table by_id,
-                               Scalars* sc, hipStream_t st);
-hipError_t probe_external(Columns c, uint64_t first, uint64_t n, const ktj_extcorr_rec* e, Table ext, Table cpu,
-                          Scalars* sc, hipStream_t st);
-hipError_t count_out_of_order(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, Table by_id,
-                              Scalars* sc, hipStream_t st);
+/* key ranges of the three tables, then their modes (direct unless force_hash or the span is too wide) */
+hipError_t plan_tables(Columns c, uint64_t n_generic, uint64_t n_runtime, uint64_t n_device, const ktj_extcorr_rec* e,
+                       uint64_t n_ext, uint32_t cap_full, uint32_t cap_narrow, uint32_t cap_cpu, bool force_hash,
+                       Scalars* sc, hipStream_t st);
+hipError_t clear_tables(FullTable tf, NarrowTable tn, KeyTable cpu, hipStream_t st);
+hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, uint32_t* slot_ext, Scalars* sc,
+                         hipStream_t st);
+hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, KeyTable cpu, Scalars* sc, hipStream_t st);
+hipError_t build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, FullTable tf,
+                         NarrowTable tn, uint32_t* slot_f, uint32_t* slot_n, Scalars* sc, hipStream_t st);
+hipError_t insert_device_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, FullTable tf,
+                               uint32_t* slot_f_dev, Scalars* sc, hipStream_t st);
+hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, const uint32_t* slot_ext, KeyTable cpu,
+                            hipStream_t st);
+/* per device row: "External id", timestamp-order check, stream of the launching row, and the
+ * size / grid hand-over (into link[]) */
+hipError_t link_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, FullTable tf,
+                            NarrowTable tn, const uint32_t* slot_f_dev, DevLink* link, DevBrief* brief, Scalars* sc,
+                            hipStream_t st);
 /* stream back-fill: queue table (keys/vals/ambiguous) and dense table are caller-provided, zeroed */
 struct StreamTables {
   uint64_t* q_keys;   /* KTJ_QUEUE_CAP + 1, filled with KTJ_EMPTY_KEY */
@@ -115,8 +187,8 @@ struct StreamTables {
   uint64_t* d_key;
   uint32_t* d_rank;
 };
-hipError_t backfill_streams(const ktj_device_rec* d, uint64_t n, const ktj_runtime_rec* r, Columns c,
-                            uint64_t first_device, Table by_id, StreamTables t, Scalars* sc, hipStream_t st);
+hipError_t backfill_streams(const DevBrief* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+                            Scalars* sc, hipStream_t st);
 
 /* ---- stage 3: canonical order ---- */
 struct SortSets {
@@ -140,11 +212,14 @@ hipError_t radix_sort(uint64_t* keys_a, uint32_t* vals_a, uint64_t* keys_b, uint
 /* ---- stage 4a: joined rows + exact byte length (arrival order) ---- */
 hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, MatRow* mat, uint32_t* len,
                             Scalars* sc, hipStream_t st);
-hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api,
-                            EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st);
-hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first,
-                           const ktj_runtime_rec* r, Table by_narrow, EmitCtx ctx, MatRow* mat, uint32_t* len,
-                           Scalars* sc, hipStream_t st);
+/* runtime rows: also publishes what device rows take over (first timestamp, stream, grid, size)
+ * into the tables, reads the "External id" and counts timestamp-order violations; runs after
+ * resolve_external and before link_device_rows */
+hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullTable tf,
+                            NarrowTable tn, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
+                            uint32_t* len, Scalars* sc, hipStream_t st);
+hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const DevLink* link,
+                           EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st);
 hipError_t gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted, hipStream_t st);
 
 /* ---- stage 4b: emit ---- */

@@ -64,6 +64,65 @@ __device__ uint32_t table_find(const uint64_t* keys, uint32_t mask, uint64_t key
   return KTJ_NOSLOT;
 }
 
+/* Join tables (TableT).  Direct mode: slot = key - base.  Hash mode: slots are grouped in runs of
+ * sixteen; a key lives at position (key + rotation) & 15 of a run, where the rotation and the
+ * probe sequence over runs (double hashing) depend only on the remaining key bits.  Sixteen
+ * consecutive ids therefore share one run, while strided or clustered ids still spread like under
+ * a full hash and a collision costs one probe in another run rather than a walk through a full one. */
+struct ProbeSeq {
+  uint32_t run, step, low;
+  __device__ __forceinline__ ProbeSeq(uint64_t key) {
+    const uint64_t h = hash64(key >> 4);
+    run = (uint32_t)h;
+    step = (uint32_t)(h >> 32) | 1u; /* odd: visits every run of a power-of-two table */
+    low = ((uint32_t)key + (uint32_t)((h * 0x9E3779B97F4A7C15ULL) >> 60)) & 15u; /* ids sharing low bits still use all positions */
+  }
+  __device__ __forceinline__ uint32_t slot(uint32_t mask) const { return ((run << 4) | low) & mask; }
+  __device__ __forceinline__ void next() { run += step; }
+};
+/* Returns the slot holding `key`, inserting it if absent; KTJ_NOSLOT when the table is full (hash
+ * mode) or the key lies outside the planned range (direct mode; cannot happen for keys that were
+ * part of the range computation). */
+template <typename S>
+__device__ uint32_t slot_insert(const TableT<S>& t, uint64_t key) {
+  if (key == KTJ_EMPTY_KEY) { t.s[t.mask + 1u].key = 0; return t.mask + 1u; }
+  if (t.ctl->direct) {
+    const uint64_t idx = key - t.ctl->base;
+    if (idx > t.ctl->span) return KTJ_NOSLOT;
+    if (t.s[idx].key != key) t.s[idx].key = key; /* every writer stores the same value */
+    return (uint32_t)idx;
+  }
+  ProbeSeq p(key);
+  for (uint32_t probe = 0; probe <= (t.mask >> 4); ++probe, p.next()) {
+    const uint32_t slot = p.slot(t.mask);
+    uint64_t cur = t.s[slot].key;
+    if (cur == key) return slot;
+    if (cur == KTJ_EMPTY_KEY) {
+      unsigned long long prev = atomicCAS((unsigned long long*)&t.s[slot].key, (unsigned long long)KTJ_EMPTY_KEY,
+                                          (unsigned long long)key);
+      if (prev == KTJ_EMPTY_KEY || prev == key) return slot;
+    }
+  }
+  return KTJ_NOSLOT;
+}
+template <typename S>
+__device__ uint32_t slot_find(const TableT<S>& t, uint64_t key) {
+  if (key == KTJ_EMPTY_KEY) return t.s[t.mask + 1u].key == 0 ? t.mask + 1u : KTJ_NOSLOT;
+  if (t.ctl->direct) {
+    const uint64_t idx = key - t.ctl->base;
+    if (idx > t.ctl->span) return KTJ_NOSLOT;
+    return t.s[idx].key == key ? (uint32_t)idx : KTJ_NOSLOT;
+  }
+  ProbeSeq p(key);
+  for (uint32_t probe = 0; probe <= (t.mask >> 4); ++probe, p.next()) {
+    const uint32_t slot = p.slot(t.mask);
+    uint64_t cur = t.s[slot].key;
+    if (cur == key) return slot;
+    if (cur == KTJ_EMPTY_KEY) return KTJ_NOSLOT;
+  }
+  return KTJ_NOSLOT;
+}
+
 __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
   return v;
@@ -97,7 +156,11 @@ __global__ void k_init_scalars(Scalars* s) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     s->ts_min_biased = ~0ULL; s->ts_max_biased = 0;
     s->out_of_range = 0; s->out_of_order = 0; s->n_flow = 0; s->n_linked = 0; s->n_blank_names = 0; s->n_valid = 0;
-    s->error = 0; s->have_stream_src = 0; s->n_dev_ranks = 0; s->n_res_ranks = 0; s->n_dense = 0; s->pad = 0;
+    s->n_unresolved = 0; s->error = 0; s->have_stream_src = 0; s->n_dev_ranks = 0; s->n_res_ranks = 0; s->n_dense = 0; s->pad = 0;
+    for (int k = 0; k < 3; ++k) {
+      s->plan.range[k].lo = ~0ULL; s->plan.range[k].hi = 0;
+      s->plan.ctl[k].base = 0; s->plan.ctl[k].span = 0; s->plan.ctl[k].direct = 0; s->plan.ctl[k].pad = 0;
+    }
   }
 }
 
@@ -427,165 +490,277 @@ hipError_t convert_rows(Columns c, uint64_t first_runtime, uint64_t n_runtime, u
 /* ------------------------------------------------------------------------------------------ */
 /* stage 2b: joins.  "Last writer wins" of the reference's sequential map updates becomes        */
 /* atomicMax over the source row index; "first seen" becomes atomicMin over the arrival index.   */
+/* What a device row takes over from "its" runtime row is then published into the table slot by  */
+/* the winning row, so that a device row needs one slot of each table and no other row.          */
 /* ------------------------------------------------------------------------------------------ */
 __device__ __forceinline__ void flag_error(Scalars* sc, unsigned bit) { atomicOr(&sc->error, bit); }
 
+/* min / max of p[i * stride] (optionally int-narrowed) into *out: one atomic pair per workgroup */
+__global__ void k_key_range(const uint64_t* p, uint32_t stride, uint64_t n, int narrow, KeyRange* out) {
+  __shared__ unsigned long long s_lo[KTJ_BLOCK >> 6], s_hi[KTJ_BLOCK >> 6];
+  unsigned long long lo = ~0ULL, hi = 0;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    uint64_t k = p[i * stride];
+    if (narrow) k = narrow_corr_key(k);
+    lo = k < lo ? k : lo;
+    hi = k > hi ? k : hi;
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    const unsigned long long l2 = __shfl_xor(lo, o), h2 = __shfl_xor(hi, o);
+    lo = l2 < lo ? l2 : lo;
+    hi = h2 > hi ? h2 : hi;
+  }
+  if (lane_id() == 0) { s_lo[threadIdx.x >> 6] = lo; s_hi[threadIdx.x >> 6] = hi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (uint32_t k = 1; k < (blockDim.x >> 6); ++k) { lo = s_lo[k] < lo ? s_lo[k] : lo; hi = s_hi[k] > hi ? s_hi[k] : hi; }
+    if (lo <= hi) { atomicMin(&out->lo, lo); atomicMax(&out->hi, hi); }
+  }
+}
+__global__ void k_plan_tables(Scalars* sc, uint32_t cap_full, uint32_t cap_narrow, uint32_t cap_cpu, int force_hash) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  const uint32_t cap[3] = {cap_full, cap_narrow, cap_cpu};
+  for (int k = 0; k < 3; ++k) {
+    const KeyRange r = sc->plan.range[k];
+    TableCtl c;
+    c.base = 0; c.span = 0; c.direct = 0; c.pad = 0;
+    /* the reserved key never takes part in direct addressing (it has its own slot) */
+    if (!force_hash && r.lo <= r.hi && r.hi - r.lo < (unsigned long long)cap[k]) { c.base = r.lo; c.span = r.hi - r.lo; c.direct = 1; }
+    sc->plan.ctl[k] = c;
+  }
+}
+/* frees every slot that can be reached: the planned span in direct mode, the whole table otherwise */
+template <typename S>
+__global__ void k_clear_table(TableT<S> t, S init) {
+  const uint64_t n = t.ctl->direct ? t.ctl->span + 1ull : (uint64_t)t.mask + 1ull;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) t.s[i] = init;
+  if (blockIdx.x == 0 && threadIdx.x == 0) t.s[t.mask + 1ull] = init;
+}
+
+hipError_t plan_tables(Columns c, uint64_t n_generic, uint64_t n_runtime, uint64_t n_device, const ktj_extcorr_rec* e,
+                       uint64_t n_ext, uint32_t cap_full, uint32_t cap_narrow, uint32_t cap_cpu, bool force_hash,
+                       Scalars* sc, hipStream_t st) {
+  const dim3 b(KTJ_BLOCK);
+  auto grid = [](uint64_t n) { const uint64_t g = (n + KTJ_BLOCK * 8 - 1) / (KTJ_BLOCK * 8); return dim3((unsigned)(g < 1024 ? (g ? g : 1) : 1024)); };
+  if (n_runtime + n_device)
+    hipLaunchKernelGGL(k_key_range, grid(n_runtime + n_device), b, 0, st, c.corr + n_generic, 1u, n_runtime + n_device, 0,
+                       &sc->plan.range[KTJ_TBL_FULL]);
+  if (n_runtime)
+    hipLaunchKernelGGL(k_key_range, grid(n_runtime), b, 0, st, c.corr + n_generic, 1u, n_runtime, 1,
+                       &sc->plan.range[KTJ_TBL_NARROW]);
+  if (n_ext)
+    hipLaunchKernelGGL(k_key_range, grid(n_ext), b, 0, st, reinterpret_cast<const uint64_t*>(e), 2u, n_ext, 0,
+                       &sc->plan.range[KTJ_TBL_NARROW]);
+  if (n_generic)
+    hipLaunchKernelGGL(k_key_range, grid(n_generic), b, 0, st, c.corr, 1u, n_generic, 0, &sc->plan.range[KTJ_TBL_CPU]);
+  hipLaunchKernelGGL(k_plan_tables, dim3(1), dim3(64), 0, st, sc, cap_full, cap_narrow, cap_cpu, force_hash ? 1 : 0);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t clear_tables(FullTable tf, NarrowTable tn, KeyTable cpu, hipStream_t st) {
+  FullSlot f;
+  f.key = KTJ_EMPTY_KEY; f.stream_src = 0; f.first = 0xFFFFFFFFu; f.first_ts = 0; f.stream = 0;
+  NarrowSlot nn;
+  nn.key = KTJ_EMPTY_KEY; nn.ext_src = 0; nn.ext_val = 0; nn.kern_src = 0; nn.copy_src = 0; nn.size = 0;
+  nn.grid[0] = nn.grid[1] = nn.grid[2] = 0; nn.linked = 0; nn.pad = 0;
+  KeySlot k;
+  k.key = KTJ_EMPTY_KEY;
+  hipLaunchKernelGGL(k_clear_table<FullSlot>, dim3(grid_stride_for((uint64_t)tf.mask + 1, KTJ_BLOCK * 4)), dim3(KTJ_BLOCK), 0, st, tf, f);
+  hipLaunchKernelGGL(k_clear_table<NarrowSlot>, dim3(grid_stride_for((uint64_t)tn.mask + 1, KTJ_BLOCK * 4)), dim3(KTJ_BLOCK), 0, st, tn, nn);
+  hipLaunchKernelGGL(k_clear_table<KeySlot>, dim3(grid_stride_for((uint64_t)cpu.mask + 1, KTJ_BLOCK * 4)), dim3(KTJ_BLOCK), 0, st, cpu, k);
+  return KTJ_LAUNCH_CHECK();
+}
+
 /* cpuCorrelationMap_[correlation] = externalId: RocmActivityProfiler.cpp:135-148 */
-__global__ void k_build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table t, Scalars* sc) {
+__global__ void k_build_extcorr(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, uint32_t* slot_ext, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const uint32_t slot = table_insert(t.keys, t.mask, e[i].correlation);
+  const uint32_t slot = slot_insert(tn, e[i].correlation);
+  slot_ext[i] = slot;
   if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
-  atomicMax(&t.v0[slot], (uint32_t)i + 1u);
+  atomicMax(&tn.s[slot].ext_src, (uint32_t)i + 1u);
 }
 /* activityMap_[act->correlationId()] = act: GenericActivityProfiler.cpp:262 */
-__global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table t, Scalars* sc) {
+__global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, KeyTable cpu, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const uint32_t slot = table_insert(t.keys, t.mask, (uint64_t)(int64_t)g[i].id);
-  if (slot == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+  if (slot_insert(cpu, (uint64_t)(int64_t)g[i].id) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
 }
-/* by_id  : full correlation id → v0 = last runtime row (index+1) that carries a stream
- *          (RocmStreamQueue.h:47-54), v1 = first arrival index seen for checkTimestampOrder
- *          (GenericActivityProfiler.cpp:363-395)
- * by_narrow: int-narrowed id → v0 = last in-range kernel row, v1 = last in-range copy/malloc row
- *          (thread_local correlationToGrid/Block/Size, RocprofActivity_inl.h:28-30, 221-223, 245, 267) */
-__global__ void k_build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, Table by_id,
-                                Table by_narrow, Scalars* sc) {
+/* full table : correlation id → stream_src = last runtime row that carries a stream
+ *              (RocmStreamQueue.h:47-54), first = first arrival index seen, for checkTimestampOrder
+ *              (GenericActivityProfiler.cpp:363-395)
+ * narrow table: int-narrowed id → kern_src = last in-range kernel row, copy_src = last in-range
+ *              copy/malloc row (thread_local correlationToGrid/Block/Size,
+ *              RocprofActivity_inl.h:28-30, 221-223, 245, 267)
+ * The slots are remembered per row (slot_f, slot_n) for the second pass over the runtime rows;
+ * slot_n also serves the "External id" lookup, so rows that insert nothing look their key up. */
+__global__ void k_build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, FullTable tf,
+                                NarrowTable tn, uint32_t* slot_f, uint32_t* slot_n, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint64_t a = first_runtime + i;
   const uint64_t id = r[i].id;
   const uint32_t kind = r[i].kind;
-  const uint32_t slot = table_insert(by_id.keys, by_id.mask, id);
-  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
-  atomicMin(&by_id.v1[slot], (uint32_t)a);
-  const uint64_t stream = kind == KTJ_RT_KERNEL ? r[i].u.kernel.stream : (kind == KTJ_RT_COPY ? r[i].u.copy.stream : 0);
-  if (stream != 0) {
-    atomicMax(&by_id.v0[slot], (uint32_t)i + 1u);
-    if (sc->have_stream_src == 0) sc->have_stream_src = 1;
+  const uint32_t sf = slot_insert(tf, id);
+  slot_f[i] = sf;
+  if (sf == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+  else {
+    if (tf.s[sf].first > (uint32_t)a) atomicMin(&tf.s[sf].first, (uint32_t)a);
+    const uint64_t stream = kind == KTJ_RT_KERNEL ? r[i].u.kernel.stream : (kind == KTJ_RT_COPY ? r[i].u.copy.stream : 0);
+    if (stream != 0) {
+      atomicMax(&tf.s[sf].stream_src, (uint32_t)i + 1u);
+      if (sc->have_stream_src == 0) sc->have_stream_src = 1;
+    }
   }
-  if ((c.meta[a] & KTJ_M_VALID) && (kind == KTJ_RT_KERNEL || kind == KTJ_RT_COPY || kind == KTJ_RT_MALLOC)) {
-    const uint32_t ps = table_insert(by_narrow.keys, by_narrow.mask, narrow_corr_key(id));
-    if (ps == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
-    if (kind == KTJ_RT_KERNEL) atomicMax(&by_narrow.v0[ps], (uint32_t)i + 1u);
-    else atomicMax(&by_narrow.v1[ps], (uint32_t)i + 1u);
+  const bool publishes = (c.meta[a] & KTJ_M_VALID) && (kind == KTJ_RT_KERNEL || kind == KTJ_RT_COPY || kind == KTJ_RT_MALLOC);
+  uint32_t sn;
+  if (publishes) {
+    sn = slot_insert(tn, narrow_corr_key(id));
+    if (sn == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+    else if (kind == KTJ_RT_KERNEL) atomicMax(&tn.s[sn].kern_src, (uint32_t)i + 1u);
+    else atomicMax(&tn.s[sn].copy_src, (uint32_t)i + 1u);
+  } else {
+    /* every slot that carries an external id exists already (k_build_extcorr ran before) */
+    sn = slot_find(tn, narrow_corr_key(id));
   }
+  slot_n[i] = sn;
 }
+/* Device rows take part in "first seen" only when they are inside the window; every device row
+ * remembers its slot (rows outside the window still take a stream from it). */
 __global__ void k_insert_device_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device,
-                                      Table by_id, Scalars* sc) {
+                                      FullTable tf, uint32_t* slot_f_dev, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint64_t a = first_device + i;
-  if (!(c.meta[a] & KTJ_M_VALID)) return;
-  const uint32_t slot = table_insert(by_id.keys, by_id.mask, d[i].id);
-  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
-  if (by_id.v1[slot] > (uint32_t)a) atomicMin(&by_id.v1[slot], (uint32_t)a);
-}
-/* linkedActivity(): GenericActivityProfiler.cpp:397-408; "External id": output_json.cpp:871-874 */
-__global__ void k_probe_external(Columns c, uint64_t first, uint64_t n, const ktj_extcorr_rec* e, Table ext,
-                                 Table cpu, Scalars* sc) {
-  uint32_t n_linked = 0;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    const uint64_t a = first + i;
-    int32_t x = 0;
-    const uint32_t s1 = table_find(ext.keys, ext.mask, narrow_corr_key(c.corr[a]));
-    if (s1 != KTJ_NOSLOT) {
-      const uint32_t src = ext.v0[s1];
-      if (src != 0) {
-        const uint64_t ext_id = e[src - 1u].external_id;
-        if (table_find(cpu.keys, cpu.mask, ext_id) != KTJ_NOSLOT) {
-          x = (int32_t)(int64_t)ext_id;
-          if (c.meta[a] & KTJ_M_VALID) ++n_linked;
-        }
-      }
-    }
-    c.ext[a] = x;
+  uint32_t slot;
+  if (c.meta[a] & KTJ_M_VALID) {
+    slot = slot_insert(tf, d[i].id);
+    if (slot == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+    else if (tf.s[slot].first > (uint32_t)a) atomicMin(&tf.s[slot].first, (uint32_t)a);
+  } else {
+    /* slots with a stream come from runtime rows and exist already */
+    slot = slot_find(tf, d[i].id);
   }
-  block_add(&sc->n_linked, n_linked);
+  slot_f_dev[i] = slot;
 }
-__global__ void k_count_out_of_order(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device,
-                                     Table by_id, Scalars* sc) {
-  uint32_t n_bad = 0;
-  const uint64_t n = n_runtime + n_device;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    const uint64_t a = first_runtime + i;
-    const bool me_runtime = i < n_runtime;
-    if (!me_runtime && !(c.meta[a] & KTJ_M_VALID)) continue;
-    const uint32_t slot = table_find(by_id.keys, by_id.mask, c.corr[a]);
-    if (slot == KTJ_NOSLOT) continue;
-    const uint64_t f = by_id.v1[slot];
-    if (f == a || f == 0xFFFFFFFFull) continue;
-    const bool first_is_runtime = f < first_runtime + n_runtime;
-    /* act1 = this row, act2 = first row; swapped when the first one is a runtime row */
-    const int64_t t1 = first_is_runtime ? c.ts[f] : c.ts[a];
-    const int64_t t2 = first_is_runtime ? c.ts[a] : c.ts[f];
-    if (t2 != 0 && t1 > t2) ++n_bad;
+/* linkedActivity(): GenericActivityProfiler.cpp:397-408.  The record that won the slot resolves
+ * its external id against the CPU-op ids once, for every row that will read the slot. */
+__global__ void k_resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, const uint32_t* slot_ext, KeyTable cpu) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t slot = slot_ext[i];
+  if (slot == KTJ_NOSLOT || tn.s[slot].ext_src != (uint32_t)i + 1u) return;
+  const uint64_t ext_id = e[i].external_id;
+  if (slot_find(cpu, ext_id) != KTJ_NOSLOT) {
+    tn.s[slot].ext_val = (int32_t)(int64_t)ext_id;
+    tn.s[slot].linked = 1u;
   }
-  block_add(&sc->out_of_order, n_bad);
 }
-
-hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table t, Scalars* sc, hipStream_t st) {
-  if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_build_extcorr, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, t, sc);
-  return KTJ_LAUNCH_CHECK();
-}
-hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table t, Scalars* sc, hipStream_t st) {
-  if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_build_cpu_ids, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, t, sc);
-  return KTJ_LAUNCH_CHECK();
-}
-hipError_t build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, Table by_id,
-                         Table by_narrow, Scalars* sc, hipStream_t st) {
-  if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_build_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first_runtime,
-                     by_id, by_narrow, sc);
-  return KTJ_LAUNCH_CHECK();
-}
-hipError_t insert_device_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, Table by_id,
-                               Scalars* sc, hipStream_t st) {
-  if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_insert_device_first, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, d, n, c,
-                     first_device, by_id, sc);
-  return KTJ_LAUNCH_CHECK();
-}
-hipError_t probe_external(Columns c, uint64_t first, uint64_t n, const ktj_extcorr_rec* e, Table ext, Table cpu,
-                          Scalars* sc, hipStream_t st) {
-  if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_probe_external, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first, n, e, ext, cpu, sc);
-  return KTJ_LAUNCH_CHECK();
-}
-hipError_t count_out_of_order(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, Table by_id,
-                              Scalars* sc, hipStream_t st) {
-  const uint64_t n = n_runtime + n_device;
-  if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_count_out_of_order, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first_runtime,
-                     n_runtime, n_device, by_id, sc);
-  return KTJ_LAUNCH_CHECK();
-}
-
-/* ---- stream back-fill: libkineto/src/RocmStreamQueue.h:42-136 ---- */
 __device__ __forceinline__ bool is_async_op(uint32_t domain) { return domain != KTJ_DOM_MEMSET; }
 
-/* pass 1: stream of the correlation-matched runtime row */
-__global__ void k_stream_by_corr(const ktj_device_rec* d, uint64_t n, const ktj_runtime_rec* r, Columns c,
-                                 uint64_t first_device, Table by_id, const Scalars* sc) {
-  if (sc->have_stream_src == 0) return;
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const uint64_t a = first_device + i;
-  if (!is_async_op(d[i].domain) || c.res[a] != 0) return;
-  const uint32_t slot = table_find(by_id.keys, by_id.mask, d[i].id);
-  if (slot == KTJ_NOSLOT) return;
-  const uint32_t src = by_id.v0[slot];
-  if (src == 0) return;
-  const ktj_runtime_rec* rr = &r[src - 1u];
-  c.res[a] = (int64_t)(rr->kind == KTJ_RT_KERNEL ? rr->u.kernel.stream : rr->u.copy.stream);
+/* One pass over the device rows with one slot of each table:
+ *  - "External id" (output_json.cpp:871-874) from the narrow slot,
+ *  - checkTimestampOrder (GenericActivityProfiler.cpp:363-395) against the first row of the id,
+ *  - the stream of the correlation-matched runtime row (RocmStreamQueue.h:56-75, first pass),
+ *  - the size or grid/block the launching row hands over (RocprofActivity_inl.h:161-180). */
+__global__ void k_link_device(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, FullTable tf,
+                              NarrowTable tn, const uint32_t* slot_f_dev, DevLink* link, DevBrief* brief, Scalars* sc) {
+  uint32_t n_linked = 0, n_bad = 0, n_unresolved = 0;
+  const bool have_stream_src = sc->have_stream_src != 0;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t a = first_device + i;
+    const uint64_t id = d[i].id;
+    const uint32_t domain = d[i].domain;
+    const bool valid = (c.meta[a] & KTJ_M_VALID) != 0;
+    DevLink l;
+    l.p[0] = l.p[1] = l.p[2] = 0; l.flags = 0; l.pad = 0;
+    int32_t ext = 0;
+    const uint32_t sn = slot_find(tn, narrow_corr_key(id));
+    if (sn != KTJ_NOSLOT) {
+      const NarrowSlot ns = tn.s[sn];
+      ext = ns.ext_val;
+      if (ns.linked && valid) ++n_linked;
+      if (domain != KTJ_DOM_MEMSET) {
+        if (ns.copy_src != 0) { l.flags = KTJ_DL_HAS_SIZE; l.p[0] = ns.size; }
+        else if (ns.kern_src != 0) { l.flags = KTJ_DL_HAS_GRID; l.p[0] = ns.grid[0]; l.p[1] = ns.grid[1]; l.p[2] = ns.grid[2]; }
+      }
+    }
+    c.ext[a] = ext;
+    link[i] = l;
+    int64_t res = c.res[a];
+    const uint32_t sf = slot_f_dev[i];
+    if (sf != KTJ_NOSLOT) {
+      const FullSlot fs = tf.s[sf];
+      if (valid) {
+        const uint64_t f = fs.first;
+        if (f != a && f != 0xFFFFFFFFull) {
+          /* act1 = this row, act2 = first row; swapped when the first one is a runtime row */
+          const bool first_is_runtime = f < first_device;
+          const int64_t tf_ts = first_is_runtime ? fs.first_ts : c.ts[f];
+          const int64_t t1 = first_is_runtime ? tf_ts : c.ts[a];
+          const int64_t t2 = first_is_runtime ? c.ts[a] : tf_ts;
+          if (t2 != 0 && t1 > t2) ++n_bad;
+        }
+      }
+      if (have_stream_src && is_async_op(domain) && res == 0 && fs.stream_src != 0) { res = (int64_t)fs.stream; c.res[a] = res; }
+    }
+    if (is_async_op(domain) && res == 0) ++n_unresolved;
+    DevBrief b;
+    b.queue = d[i].queue; b.device = d[i].device; b.domain = domain;
+    brief[i] = b;
+  }
+  block_add(&sc->n_linked, n_linked);
+  block_add(&sc->out_of_order, n_bad);
+  block_add(&sc->n_unresolved, n_unresolved);
 }
-/* pass 2a: queue → stream, ambiguous when one queue shows two different streams */
-__global__ void k_queue_build(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+
+hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, uint32_t* slot_ext, Scalars* sc,
+                         hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_build_extcorr, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, tn, slot_ext, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, KeyTable cpu, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_build_cpu_ids, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, cpu, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, FullTable tf,
+                         NarrowTable tn, uint32_t* slot_f, uint32_t* slot_n, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_build_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first_runtime, tf, tn,
+                     slot_f, slot_n, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t insert_device_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, FullTable tf,
+                               uint32_t* slot_f_dev, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_insert_device_first, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, d, n, c, first_device, tf,
+                     slot_f_dev, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, const uint32_t* slot_ext, KeyTable cpu,
+                            hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_resolve_external, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, tn, slot_ext, cpu);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t link_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, FullTable tf,
+                            NarrowTable tn, const uint32_t* slot_f_dev, DevLink* link, DevBrief* brief, Scalars* sc,
+                            hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_link_device, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, d, n, c, first_device, tf,
+                     tn, slot_f_dev, link, brief, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* ---- stream back-fill: libkineto/src/RocmStreamQueue.h:42-136 (its first pass, the stream of
+ * the correlation-matched runtime row, is part of k_link_device) ---- */
+/* pass 2a: queue → stream, ambiguous when one queue shows two different streams.  Passes 2a/2b
+ * have no effect when the first pass left no row without a stream (the usual case: every device
+ * row has a launching runtime row), and return at once then. */
+__global__ void k_queue_build(const DevBrief* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
                               Scalars* sc) {
-  if (sc->have_stream_src == 0) return;
+  if (sc->have_stream_src == 0 || sc->n_unresolved == 0) return;
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint64_t stream = (uint64_t)c.res[first_device + i];
@@ -598,9 +773,9 @@ __global__ void k_queue_build(const ktj_device_rec* d, uint64_t n, Columns c, ui
   if (cur != 0 && cur != stream) t.q_amb[slot] = 1u;
 }
 /* pass 2b: rows still without a stream take their queue's stream */
-__global__ void k_queue_fill(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+__global__ void k_queue_fill(const DevBrief* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
                              const Scalars* sc) {
-  if (sc->have_stream_src == 0) return;
+  if (sc->have_stream_src == 0 || sc->n_unresolved == 0) return;
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint64_t a = first_device + i;
@@ -609,7 +784,7 @@ __global__ void k_queue_fill(const ktj_device_rec* d, uint64_t n, Columns c, uin
   if (slot == KTJ_NOSLOT || t.q_amb[slot] != 0 || t.q_stream[slot] == 0) return;
   c.res[a] = (int64_t)t.q_stream[slot];
 }
-__device__ __forceinline__ bool dense_key(const ktj_device_rec& d, uint64_t stream, uint64_t* key) {
+__device__ __forceinline__ bool dense_key(const DevBrief& d, uint64_t stream, uint64_t* key) {
   if (!is_async_op(d.domain)) return false;
   if (stream != 0) *key = stream;
   else if (d.queue != 0) *key = d.queue | (1ULL << 63);
@@ -620,20 +795,46 @@ __device__ __forceinline__ uint64_t dense_hash(int32_t device, uint64_t key) {
   uint64_t h = hash64(key ^ hash64((uint64_t)(int64_t)device + 0x9E3779B97F4A7C15ULL));
   return h == KTJ_EMPTY_KEY ? 0x5bd1e995ULL : h;
 }
-/* pass 3a: first arrival index per (device, stream key) */
-__global__ void k_dense_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+/* pass 3a: first arrival index per (device, stream key).  Millions of rows share a few hundred
+ * pairs, so each workgroup first reduces its rows in an LDS table and touches the global table
+ * once per pair. */
+#define DENSE_LOCAL_SLOTS 1024u
+__global__ void k_dense_first(const DevBrief* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
                               Scalars* sc) {
+  __shared__ unsigned long long l_key[DENSE_LOCAL_SLOTS];
+  __shared__ uint32_t l_min[DENSE_LOCAL_SLOTS];
   if (sc->have_stream_src == 0) return;
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  uint64_t key;
-  if (!dense_key(d[i], (uint64_t)c.res[first_device + i], &key)) return;
-  const uint32_t slot = table_insert(t.d_hash, KTJ_DENSE_CAP - 1u, dense_hash(d[i].device, key));
-  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT); return; }
-  if (t.d_first[slot] > (uint32_t)i) atomicMin(&t.d_first[slot], (uint32_t)i);
+  for (uint32_t k = threadIdx.x; k < DENSE_LOCAL_SLOTS; k += blockDim.x) { l_key[k] = KTJ_EMPTY_KEY; l_min[k] = 0xFFFFFFFFu; }
+  __syncthreads();
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    uint64_t key;
+    if (!dense_key(d[i], (uint64_t)c.res[first_device + i], &key)) continue;
+    const uint64_t h = dense_hash(d[i].device, key);
+    uint32_t slot = (uint32_t)(h >> 20) & (DENSE_LOCAL_SLOTS - 1u);
+    bool placed = false;
+    for (uint32_t probe = 0; probe < 16 && !placed; ++probe) {
+      unsigned long long cur = l_key[slot];
+      if (cur == KTJ_EMPTY_KEY) cur = atomicCAS(&l_key[slot], (unsigned long long)KTJ_EMPTY_KEY, (unsigned long long)h);
+      if (cur == KTJ_EMPTY_KEY || cur == h) { atomicMin(&l_min[slot], (uint32_t)i); placed = true; }
+      else slot = (slot + 1u) & (DENSE_LOCAL_SLOTS - 1u);
+    }
+    if (!placed) { /* local table crowded: straight to the global one */
+      const uint32_t g = table_insert(t.d_hash, KTJ_DENSE_CAP - 1u, h);
+      if (g == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT);
+      else if (t.d_first[g] > (uint32_t)i) atomicMin(&t.d_first[g], (uint32_t)i);
+    }
+  }
+  __syncthreads();
+  for (uint32_t k = threadIdx.x; k < DENSE_LOCAL_SLOTS; k += blockDim.x) {
+    const unsigned long long h = l_key[k];
+    if (h == KTJ_EMPTY_KEY) continue;
+    const uint32_t g = table_insert(t.d_hash, KTJ_DENSE_CAP - 1u, h);
+    if (g == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT); continue; }
+    if (t.d_first[g] > l_min[k]) atomicMin(&t.d_first[g], l_min[k]);
+  }
 }
 /* pass 3b: the first row of each pair records the pair itself (single writer per slot) */
-__global__ void k_dense_owner(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+__global__ void k_dense_owner(const DevBrief* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
                               const Scalars* sc) {
   if (sc->have_stream_src == 0) return;
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -675,33 +876,33 @@ __global__ void k_dense_rank(StreamTables t, Scalars* sc) {
   }
 }
 /* pass 3d: resourceId() = stream != 0 ? stream : queue (RocprofActivity.h:100-102) */
-__global__ void k_dense_assign(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+__global__ void k_dense_assign(const DevBrief* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
                                Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint64_t a = first_device + i;
-  if (!is_async_op(d[i].domain)) return;
+  const DevBrief b = d[i];
+  if (!is_async_op(b.domain)) return;
   uint64_t stream = (uint64_t)c.res[a];
   if (sc->have_stream_src != 0) {
     uint64_t key;
-    if (dense_key(d[i], stream, &key)) {
-      const uint32_t slot = table_find(t.d_hash, KTJ_DENSE_CAP - 1u, dense_hash(d[i].device, key));
-      if (slot == KTJ_NOSLOT || t.d_dev[slot] != d[i].device || t.d_key[slot] != key) {
+    if (dense_key(b, stream, &key)) {
+      const uint32_t slot = table_find(t.d_hash, KTJ_DENSE_CAP - 1u, dense_hash(b.device, key));
+      if (slot == KTJ_NOSLOT || t.d_dev[slot] != b.device || t.d_key[slot] != key) {
         flag_error(sc, KTJ_DEVERR_HASH_COLLISION);
       } else stream = t.d_rank[slot];
     }
   }
-  c.res[a] = (int64_t)(stream != 0 ? stream : d[i].queue);
+  c.res[a] = (int64_t)(stream != 0 ? stream : b.queue);
 }
 
-hipError_t backfill_streams(const ktj_device_rec* d, uint64_t n, const ktj_runtime_rec* r, Columns c,
-                            uint64_t first_device, Table by_id, StreamTables t, Scalars* sc, hipStream_t st) {
+hipError_t backfill_streams(const DevBrief* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
+                            Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
   const dim3 g(grid_for(n, KTJ_BLOCK)), b(KTJ_BLOCK);
-  hipLaunchKernelGGL(k_stream_by_corr, g, b, 0, st, d, n, r, c, first_device, by_id, (const Scalars*)sc);
   hipLaunchKernelGGL(k_queue_build, g, b, 0, st, d, n, c, first_device, t, sc);
   hipLaunchKernelGGL(k_queue_fill, g, b, 0, st, d, n, c, first_device, t, (const Scalars*)sc);
-  hipLaunchKernelGGL(k_dense_first, g, b, 0, st, d, n, c, first_device, t, sc);
+  hipLaunchKernelGGL(k_dense_first, dim3(grid_stride_for(n, KTJ_BLOCK * 8)), b, 0, st, d, n, c, first_device, t, sc);
   hipLaunchKernelGGL(k_dense_owner, g, b, 0, st, d, n, c, first_device, t, (const Scalars*)sc);
   hipLaunchKernelGGL(k_dense_rank, dim3(1), dim3(1024), 0, st, t, sc);
   hipLaunchKernelGGL(k_dense_assign, g, b, 0, st, d, n, c, first_device, t, sc);
@@ -959,45 +1160,61 @@ __global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx,
   }
   flush_row_stats(rs, sc);
 }
-__global__ void k_mat_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, EmitCtx ctx,
-                              MatRow* mat, uint32_t* len, Scalars* sc) {
+/* Second pass over the runtime rows.  The row that won a slot field publishes what device rows
+ * take over (timestamp of the first row, stream, grid/block, size); every row reads its
+ * "External id" from the narrow slot and is checked against the first row of its id. */
+__global__ void k_mat_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullTable tf,
+                              NarrowTable tn, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
+                              uint32_t* len, Scalars* sc) {
   RowStats rs;
+  uint32_t n_linked = 0, n_bad = 0;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t a = first + i;
     const ktj_runtime_rec rec = r[i];
+    const int64_t ts = c.ts[a];
+    const bool valid = (c.meta[a] & KTJ_M_VALID) != 0;
+    const uint32_t sf = slot_f[i], sn = slot_n[i];
+    if (sf != KTJ_NOSLOT) {
+      FullSlot* fs = &tf.s[sf];
+      const uint64_t f = fs->first;
+      if (f == a) fs->first_ts = ts;
+      else if (f != 0xFFFFFFFFull) { /* an earlier runtime row has this id: checkTimestampOrder, swapped */
+        const int64_t t1 = c.ts[f];
+        if (ts != 0 && t1 > ts) ++n_bad;
+      }
+      if (fs->stream_src == (uint32_t)i + 1u)
+        fs->stream = rec.kind == KTJ_RT_KERNEL ? rec.u.kernel.stream : rec.u.copy.stream;
+    }
+    int32_t ext = 0;
+    if (sn != KTJ_NOSLOT) {
+      NarrowSlot* ns = &tn.s[sn];
+      ext = ns->ext_val;
+      if (ns->linked && valid) ++n_linked;
+      if (ns->kern_src == (uint32_t)i + 1u) pack_grid(rec, ns->grid);
+      if (ns->copy_src == (uint32_t)i + 1u) ns->size = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
+    }
+    c.ext[a] = ext;
     const bool known = rec.cid < api.n_cids;
     const uint32_t name = known ? api.cid_name_ids[rec.cid] : KTJ_NONE;
-    const bool fs = known && ((api.flow_start_bits[rec.cid >> 5] >> (rec.cid & 31u)) & 1u);
-    const MatRow m = mat_runtime(rec, c.ts[a], c.dur[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a], name, fs,
-                                 rec.cid == api.malloc_cid);
+    const bool fstart = known && ((api.flow_start_bits[rec.cid >> 5] >> (rec.cid & 31u)) & 1u);
+    const MatRow m = mat_runtime(rec, ts, c.dur[a], valid, ext, name, fstart, rec.cid == api.malloc_cid);
     store_row(&mat[a], m);
     len[a] = row_length(m, ctx, sc);
     count_row_stats(m, ctx, &rs);
   }
   flush_row_stats(rs, sc);
+  block_add(&sc->n_linked, n_linked);
+  block_add(&sc->out_of_order, n_bad);
 }
-__global__ void k_mat_device(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const ktj_runtime_rec* r,
-                             Table by_narrow, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc) {
+__global__ void k_mat_device(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const DevLink* link,
+                             EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc) {
   RowStats rs;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t a = first + i;
     const ktj_device_rec rec = d[i];
-    const ktj_runtime_rec* ksrc = nullptr;
-    bool has_size = false;
-    uint64_t size = 0;
-    if (rec.domain != KTJ_DOM_MEMSET) { /* RocprofActivity_inl.h:161-180 */
-      const uint32_t slot = table_find(by_narrow.keys, by_narrow.mask, narrow_corr_key(rec.id));
-      if (slot != KTJ_NOSLOT) {
-        const uint32_t ss = by_narrow.v1[slot], ks = by_narrow.v0[slot];
-        if (ss != 0) {
-          const ktj_runtime_rec* sr = &r[ss - 1u];
-          has_size = true;
-          size = sr->kind == KTJ_RT_COPY ? sr->u.copy.size : sr->u.malloc_.size;
-        } else if (ks != 0) ksrc = &r[ks - 1u];
-      }
-    }
-    const MatRow m = mat_device(rec, c.ts[a], c.dur[a], c.res[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a], ksrc,
-                                has_size, size);
+    const DevLink l = link[i];
+    const MatRow m = mat_device(rec, c.ts[a], c.dur[a], c.res[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a],
+                                (l.flags & KTJ_DL_HAS_GRID) ? l.p : nullptr, (l.flags & KTJ_DL_HAS_SIZE) != 0, l.p[0]);
     store_row(&mat[a], m);
     len[a] = row_length(m, ctx, sc);
     count_row_stats(m, ctx, &rs);
@@ -1015,18 +1232,19 @@ hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, M
   hipLaunchKernelGGL(k_mat_generic, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, ctx, mat, len, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, EmitCtx ctx,
-                            MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st) {
+hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullTable tf,
+                            NarrowTable tn, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
+                            uint32_t* len, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_mat_runtime, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, ctx, mat,
-                     len, sc);
+  hipLaunchKernelGGL(k_mat_runtime, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, tf, tn,
+                     slot_f, slot_n, ctx, mat, len, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const ktj_runtime_rec* r,
-                           Table by_narrow, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st) {
+hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const DevLink* link,
+                           EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_mat_device, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, d, n, c, first, r, by_narrow,
-                     ctx, mat, len, sc);
+  hipLaunchKernelGGL(k_mat_device, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, d, n, c, first, link, ctx,
+                     mat, len, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted, hipStream_t st) {
@@ -1171,7 +1389,13 @@ k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, con
 hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint32_t* len_kind,
                        uint64_t n_rows, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st) {
   if (n_rows == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_emit_direct, dim3(grid_for(n_rows, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, mat, perm, offs,
+  /* Every lane keeps one partially written 128-byte line open at a time.  At full occupancy
+   * (2048 lanes per CU, 256 CUs) those lines exceed the L2 capacity and are evicted half-filled,
+   * which doubles the HBM writes.  Unused dynamic LDS caps residency at two workgroups per CU
+   * (8 waves), so the open lines stay in L2 until complete; measured 15-20% faster on every
+   * configuration than unrestricted residency. */
+  const size_t residency_lds = 60000;
+  hipLaunchKernelGGL(k_emit_direct, dim3(grid_for(n_rows, KTJ_BLOCK)), dim3(KTJ_BLOCK), residency_lds, st, mat, perm, offs,
                      len_kind, n_rows, ctx, out, prefix_len);
   return KTJ_LAUNCH_CHECK();
 }

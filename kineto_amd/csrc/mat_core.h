@@ -87,6 +87,13 @@ KTJ_HD inline MatRow mat_generic(const ktj_generic_rec& g) {
   return m;
 }
 
+/* grid[0..2] and workgroup[0..2] of a kernel-launch row as three 64-bit words */
+KTJ_HD inline void pack_grid(const ktj_runtime_rec& r, uint64_t g[3]) {
+  g[0] = (uint64_t)r.u.kernel.grid[0] | ((uint64_t)r.u.kernel.grid[1] << 32);
+  g[1] = (uint64_t)r.u.kernel.grid[2] | ((uint64_t)r.u.kernel.workgroup[0] << 32);
+  g[2] = (uint64_t)r.u.kernel.workgroup[1] | ((uint64_t)r.u.kernel.workgroup[2] << 32);
+}
+
 /* name_id: dictionary id of the API name, KTJ_NONE when the cid is outside the API table */
 KTJ_HD inline MatRow mat_runtime(const ktj_runtime_rec& r, int64_t ts, int64_t dur, bool valid, int32_t ext,
                                  uint32_t name_id, bool flow_start, bool is_malloc_cid) {
@@ -104,9 +111,7 @@ KTJ_HD inline MatRow mat_runtime(const ktj_runtime_rec& r, int64_t ts, int64_t d
   m.aux = r.cid;
   m.p[0] = m.p[1] = m.p[2] = m.p[3] = m.p[4] = 0;
   if (kind == KTJ_RT_KERNEL) {
-    m.p[0] = (uint64_t)r.u.kernel.grid[0] | ((uint64_t)r.u.kernel.grid[1] << 32);
-    m.p[1] = (uint64_t)r.u.kernel.grid[2] | ((uint64_t)r.u.kernel.workgroup[0] << 32);
-    m.p[2] = (uint64_t)r.u.kernel.workgroup[1] | ((uint64_t)r.u.kernel.workgroup[2] << 32);
+    pack_grid(r, m.p);
     m.p[3] = r.u.kernel.group_segment_size;
     m.p[4] = r.u.kernel.kernel_name_id;
     if (r.u.kernel.kernel_name_id != KTJ_NONE) meta |= KTJ_M_HAS_KERNEL_ARG;
@@ -120,10 +125,10 @@ KTJ_HD inline MatRow mat_runtime(const ktj_runtime_rec& r, int64_t ts, int64_t d
   return m;
 }
 
-/* res: resourceId() after stream back-fill.  kernel_src: the launching kernel row whose grid and
- * block the reference hands over (may be null); size: bytes handed over by a copy/malloc row. */
+/* res: resourceId() after stream back-fill.  grid: packed grid and block of the launching kernel
+ * row that the reference hands over (null = none); size: bytes handed over by a copy/malloc row. */
 KTJ_HD inline MatRow mat_device(const ktj_device_rec& d, int64_t ts, int64_t dur, int64_t res, bool valid,
-                                int32_t ext, const ktj_runtime_rec* kernel_src, bool has_size, uint64_t size) {
+                                int32_t ext, const uint64_t* grid, bool has_size, uint64_t size) {
   MatRow m;
   m.ts = ts; m.dur = dur; m.dev = (int64_t)d.device; m.res = res;
   m.flow_id = (int64_t)d.id;
@@ -147,11 +152,9 @@ KTJ_HD inline MatRow mat_device(const ktj_device_rec& d, int64_t ts, int64_t dur
     } else if (d.name_id == KTJ_NONE) { meta |= KTJ_M_NAME_BUILTIN; m.name_id = KTJ_NAME_UNKNOWN_OP; }
     else m.name_id = d.name_id;
     if (has_size) { meta |= KTJ_M_HAS_SIZE; m.p[0] = size; }
-    else if (kernel_src) {
+    else if (grid) {
       meta |= KTJ_M_HAS_GRID;
-      m.p[0] = (uint64_t)kernel_src->u.kernel.grid[0] | ((uint64_t)kernel_src->u.kernel.grid[1] << 32);
-      m.p[1] = (uint64_t)kernel_src->u.kernel.grid[2] | ((uint64_t)kernel_src->u.kernel.workgroup[0] << 32);
-      m.p[2] = (uint64_t)kernel_src->u.kernel.workgroup[1] | ((uint64_t)kernel_src->u.kernel.workgroup[2] << 32);
+      m.p[0] = grid[0]; m.p[1] = grid[1]; m.p[2] = grid[2];
     }
   }
   m.meta = meta;

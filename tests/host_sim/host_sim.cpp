@@ -188,7 +188,9 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
         if (ki != kernel_src.end()) ksrc = &s->runtime[ki->second];
       }
     }
-    mat[ng + nr + i] = mat_device(d, ts, dur, res, valid, ext_of(d.id), ksrc, has_size, size);
+    uint64_t grid[3];
+    if (ksrc) pack_grid(*ksrc, grid);
+    mat[ng + nr + i] = mat_device(d, ts, dur, res, valid, ext_of(d.id), ksrc ? grid : nullptr, has_size, size);
   }
 
   // canonical order over valid rows

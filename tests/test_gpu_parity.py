@@ -54,16 +54,19 @@ def run_case(cfg, n, check_stages=True):
             assert st.n_flow_events == cnt["n_flow_events"]
             assert st.n_linked == cnt["n_linked"]
         got = eng.output()
-    # the output-partitioned emit kernel must produce the same document
-    with TraceEngine(sp.contents.trace_name.decode(), device=0, tile_emit=True) as eng:
+    # the output-partitioned emit kernel and hash-mode join tables must produce the same document
+    with TraceEngine(sp.contents.trace_name.decode(), device=0, tile_emit=True, hash_join=True) as eng:
         eng.submit_stream(sp)
         eng.process()
+        st_hash = eng.stats()
         got_tile = eng.output()
+    if check_stages:  # hash-mode join tables: same counters as the direct-addressed ones
+        assert st_hash.gpu_and_cpu_op_out_of_order == st.gpu_and_cpu_op_out_of_order and st_hash.n_linked == st.n_linked
     ora.close()
     release()
     if got_tile != want:
         i = _first_diff(got_tile, want)
-        raise AssertionError(f"tile emit: byte {i} of {len(want)}: got {got_tile[max(0, i - 60):i + 60]!r} want {want[max(0, i - 60):i + 60]!r}")
+        raise AssertionError(f"tile emit + hash join: byte {i} of {len(want)}: got {got_tile[max(0, i - 60):i + 60]!r} want {want[max(0, i - 60):i + 60]!r}")
     if got != want:
         i = _first_diff(got, want)
         raise AssertionError(f"config {cfg} n={n}: bytes differ at {i} (got {len(got)} bytes, want {len(want)}):\n"
