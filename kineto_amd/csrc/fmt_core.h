@@ -387,20 +387,31 @@ struct TileWriter {
   }
 };
 
-/* Pass B, direct variant: one lane formats one activity straight into the document in device
- * memory.  Bytes are gathered in a 64-bit accumulator and leave as aligned 8-byte stores.  An
+/* Pass B: one lane formats one activity straight into the document in device memory.  Bytes are
+ * gathered in a 64-bit accumulator and leave as aligned 8-byte words through a sink.  An
  * activity's first word also holds the last bytes of its predecessor; those are one of three
  * fixed strings (see tail_kind), so the successor writes the whole shared word and the
  * predecessor never writes its trailing partial word.  Dictionary strings are appended inline,
  * eight bytes at a time, through a funnel shift over aligned loads (dictionary blobs are padded
  * by 16 bytes so that the last load stays inside the allocation). */
-struct GlobalWriter {
+
+/* every finished word is stored at once by the lane that gathered it */
+struct DirectSink {
   uint64_t* wptr;     /* aligned address of the word being gathered */
+  KTJ_HD KTJ_FI void open(uint64_t* first_word) { wptr = first_word; }
+  KTJ_HD KTJ_FI void put(uint64_t w) { *wptr++ = w; }
+  KTJ_HD KTJ_FI void close() {}
+  KTJ_HD KTJ_FI uint64_t* next_word() const { return wptr; }
+};
+
+template <class Sink>
+struct WordWriter {
+  Sink sink;
   uint64_t acc;
   uint32_t fill;      /* bytes gathered in acc, 0..7 */
 
   KTJ_HD KTJ_FI void begin(char* doc, uint64_t pos, uint64_t low_bytes) {
-    wptr = reinterpret_cast<uint64_t*>(doc + (pos & ~7ULL));
+    sink.open(reinterpret_cast<uint64_t*>(doc + (pos & ~7ULL)));
     fill = (uint32_t)(pos & 7ULL);
     acc = low_bytes; /* the `fill` bytes that precede this activity in its first word */
   }
@@ -408,7 +419,7 @@ struct GlobalWriter {
     acc |= v << (8 * fill);
     const uint32_t total = fill + n;
     if (total >= 8) {
-      *wptr++ = acc;
+      sink.put(acc);
       const uint32_t rest = total - 8;
       acc = rest ? v >> (8 * (n - rest)) : 0;
       fill = rest;
@@ -474,6 +485,7 @@ struct GlobalWriter {
     }
   }
 };
+typedef WordWriter<DirectSink> GlobalWriter;
 
 /* The last seven bytes of a formatted activity, by kind (see format_activity):
  *   0: `  \n  },`   complete event without args, or a flow-start event

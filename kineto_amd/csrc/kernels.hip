@@ -1383,7 +1383,8 @@ k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, con
   format_activity(w, m, ctx);
   if (w.fill && i + 1 == n_rows) { /* last activity: merge with the suffix bytes behind it */
     const uint64_t mask = (1ULL << (8 * w.fill)) - 1ULL;
-    *w.wptr = (*w.wptr & ~mask) | (w.acc & mask);
+    uint64_t* last = w.sink.next_word();
+    *last = (*last & ~mask) | (w.acc & mask);
   }
 }
 hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint32_t* len_kind,

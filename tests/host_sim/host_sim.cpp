@@ -248,10 +248,11 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
       GlobalWriter w;
       w.begin(buf, pos, low);
       format_activity(w, mat[perm[i]], ctx);
-      if ((uint64_t)((char*)w.wptr - buf) + w.fill != P + offs[i + 1]) { free(buf); return -2; }
+      if ((uint64_t)((char*)w.sink.next_word() - buf) + w.fill != P + offs[i + 1]) { free(buf); return -2; }
       if (w.fill && i + 1 == perm.size()) {
         const uint64_t mask = (1ULL << (8 * w.fill)) - 1;
-        *w.wptr = (*w.wptr & ~mask) | (w.acc & mask);
+        uint64_t* last = w.sink.next_word();
+        *last = (*last & ~mask) | (w.acc & mask);
       }
     }
     *out = buf;
