@@ -462,7 +462,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   /* ---- stage 1: decode ---- */
   HIPCHK(decode_generic(g_recs, ng, c, 0, st));
   HIPCHK(decode_runtime(r_recs, nr, c, ng, st));
-  HIPCHK(decode_device(d_recs, nd, c, ng + nr, st));
+  HIPCHK(decode_device(d_recs, nd, c, ng + nr, e->dev_brief.as<DevBrief>(), st));
   HIPCHK(hipEventRecord(e->ev[EV_DECODE], st));
 
   /* ---- stage 2a: clock + window ---- */
@@ -489,14 +489,13 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   MatRow* mat = e->mat.as<MatRow>();
   HIPCHK(build_extcorr(x_recs, nx, tn, e->slot_ext.as<uint32_t>(), sc, st));
   HIPCHK(build_cpu_ids(g_recs, ng, t_cpu, sc, st));
-  HIPCHK(build_runtime(r_recs, nr, c, ng, tf, tn, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), sc, st));
-  HIPCHK(insert_device_first(d_recs, nd, c, ng + nr, tf, e->slot_f_dev.as<uint32_t>(), sc, st));
+  HIPCHK(build_runtime(nr, c, ng, tf, tn, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), sc, st));
+  HIPCHK(insert_device_first(nd, c, ng + nr, tf, e->slot_f_dev.as<uint32_t>(), sc, st));
   HIPCHK(resolve_external(x_recs, nx, tn, e->slot_ext.as<uint32_t>(), t_cpu, st));
   /* second pass over the runtime rows: publishes into the tables and writes the joined rows */
   HIPCHK(mat_runtime_rows(r_recs, nr, c, ng, api, tf, tn, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), ctx, mat,
                           e->len.as<uint32_t>(), sc, st));
-  HIPCHK(link_device_rows(d_recs, nd, c, ng + nr, tf, tn, e->slot_f_dev.as<uint32_t>(), e->dev_link.as<DevLink>(),
-                          e->dev_brief.as<DevBrief>(), sc, st));
+  HIPCHK(link_device_rows(nd, c, ng + nr, tf, tn, e->slot_f_dev.as<uint32_t>(), e->dev_link.as<DevLink>(), sc, st));
   HIPCHK(backfill_streams(e->dev_brief.as<DevBrief>(), nd, c, ng + nr, stt, sc, st));
   HIPCHK(hipEventRecord(e->ev[EV_JOIN], st));
 

@@ -150,7 +150,7 @@ hipError_t dict_write(const char* blob, const uint64_t* off, uint32_t n, const u
 /* ---- stage 1: decode ---- */
 hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st);
 hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st);
-hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st);
+hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, DevBrief* brief, hipStream_t st);
 
 /* ---- stage 2a: clock conversion + window filter (runtime and device rows) ---- */
 hipError_t convert_rows(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, ClockDev clk,
@@ -165,17 +165,17 @@ hipError_t clear_tables(FullTable tf, NarrowTable tn, KeyTable cpu, hipStream_t 
 hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, uint32_t* slot_ext, Scalars* sc,
                          hipStream_t st);
 hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, KeyTable cpu, Scalars* sc, hipStream_t st);
-hipError_t build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, FullTable tf,
-                         NarrowTable tn, uint32_t* slot_f, uint32_t* slot_n, Scalars* sc, hipStream_t st);
-hipError_t insert_device_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, FullTable tf,
-                               uint32_t* slot_f_dev, Scalars* sc, hipStream_t st);
+/* the build passes read the columns only (correlation id, kind and has-stream bits of meta) */
+hipError_t build_runtime(uint64_t n, Columns c, uint64_t first_runtime, FullTable tf, NarrowTable tn, uint32_t* slot_f,
+                         uint32_t* slot_n, Scalars* sc, hipStream_t st);
+hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, FullTable tf, uint32_t* slot_f_dev,
+                               Scalars* sc, hipStream_t st);
 hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, const uint32_t* slot_ext, KeyTable cpu,
                             hipStream_t st);
 /* per device row: "External id", timestamp-order check, stream of the launching row, and the
  * size / grid hand-over (into link[]) */
-hipError_t link_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, FullTable tf,
-                            NarrowTable tn, const uint32_t* slot_f_dev, DevLink* link, DevBrief* brief, Scalars* sc,
-                            hipStream_t st);
+hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, FullTable tf, NarrowTable tn,
+                            const uint32_t* slot_f_dev, DevLink* link, Scalars* sc, hipStream_t st);
 /* stream back-fill: queue table (keys/vals/ambiguous) and dense table are caller-provided, zeroed */
 struct StreamTables {
   uint64_t* q_keys;   /* KTJ_QUEUE_CAP + 1, filled with KTJ_EMPTY_KEY */

@@ -412,10 +412,12 @@ __global__ void k_decode_runtime(const ktj_runtime_rec* recs, uint64_t n, Column
   c.corr[a] = r->id;
   c.dev[a] = (int64_t)r->pid;
   c.res[a] = (int64_t)r->tid;
-  c.meta[a] = (KTJ_CLASS_RUNTIME << KTJ_M_CLASS_SHIFT);
+  const uint32_t kind = r->kind <= KTJ_RT_MALLOC ? r->kind : KTJ_RT_DEFAULT;
+  const uint64_t stream = kind == KTJ_RT_KERNEL ? r->u.kernel.stream : (kind == KTJ_RT_COPY ? r->u.copy.stream : 0);
+  c.meta[a] = (KTJ_CLASS_RUNTIME << KTJ_M_CLASS_SHIFT) | (kind << KTJ_M_KIND_SHIFT) | (stream != 0 ? KTJ_M_HAS_STREAM : 0u);
   c.ext[a] = 0;
 }
-__global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns c, uint64_t first) {
+__global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns c, uint64_t first, DevBrief* brief) {
   __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_device_rec) / 16];
   uint32_t cnt;
   const ktj_device_rec* l = stage_records(recs, n, stage, &cnt);
@@ -430,6 +432,9 @@ __global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns 
   c.res[a] = (int64_t)d->stream;
   c.meta[a] = (KTJ_CLASS_DEVICE << KTJ_M_CLASS_SHIFT) | (dom << KTJ_M_KIND_SHIFT);
   c.ext[a] = 0;
+  DevBrief b;
+  b.queue = d->queue; b.device = d->device; b.domain = d->domain;
+  brief[a - first] = b;
 }
 
 hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st) {
@@ -442,9 +447,9 @@ hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint6
   hipLaunchKernelGGL(k_decode_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st) {
+hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, DevBrief* brief, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_decode_device, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first);
+  hipLaunchKernelGGL(k_decode_device, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, brief);
   return KTJ_LAUNCH_CHECK();
 }
 
@@ -593,25 +598,25 @@ __global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, KeyTable c
  *              RocprofActivity_inl.h:28-30, 221-223, 245, 267)
  * The slots are remembered per row (slot_f, slot_n) for the second pass over the runtime rows;
  * slot_n also serves the "External id" lookup, so rows that insert nothing look their key up. */
-__global__ void k_build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, FullTable tf,
-                                NarrowTable tn, uint32_t* slot_f, uint32_t* slot_n, Scalars* sc) {
+__global__ void k_build_runtime(uint64_t n, Columns c, uint64_t first_runtime, FullTable tf, NarrowTable tn,
+                                uint32_t* slot_f, uint32_t* slot_n, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint64_t a = first_runtime + i;
-  const uint64_t id = r[i].id;
-  const uint32_t kind = r[i].kind;
+  const uint64_t id = c.corr[a];
+  const uint32_t meta = c.meta[a];
+  const uint32_t kind = (meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
   const uint32_t sf = slot_insert(tf, id);
   slot_f[i] = sf;
   if (sf == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
   else {
     if (tf.s[sf].first > (uint32_t)a) atomicMin(&tf.s[sf].first, (uint32_t)a);
-    const uint64_t stream = kind == KTJ_RT_KERNEL ? r[i].u.kernel.stream : (kind == KTJ_RT_COPY ? r[i].u.copy.stream : 0);
-    if (stream != 0) {
+    if (meta & KTJ_M_HAS_STREAM) {
       atomicMax(&tf.s[sf].stream_src, (uint32_t)i + 1u);
       if (sc->have_stream_src == 0) sc->have_stream_src = 1;
     }
   }
-  const bool publishes = (c.meta[a] & KTJ_M_VALID) && (kind == KTJ_RT_KERNEL || kind == KTJ_RT_COPY || kind == KTJ_RT_MALLOC);
+  const bool publishes = (meta & KTJ_M_VALID) && kind != KTJ_RT_DEFAULT;
   uint32_t sn;
   if (publishes) {
     sn = slot_insert(tn, narrow_corr_key(id));
@@ -626,19 +631,20 @@ __global__ void k_build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c,
 }
 /* Device rows take part in "first seen" only when they are inside the window; every device row
  * remembers its slot (rows outside the window still take a stream from it). */
-__global__ void k_insert_device_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device,
-                                      FullTable tf, uint32_t* slot_f_dev, Scalars* sc) {
+__global__ void k_insert_device_first(uint64_t n, Columns c, uint64_t first_device, FullTable tf, uint32_t* slot_f_dev,
+                                      Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint64_t a = first_device + i;
+  const uint64_t id = c.corr[a];
   uint32_t slot;
   if (c.meta[a] & KTJ_M_VALID) {
-    slot = slot_insert(tf, d[i].id);
+    slot = slot_insert(tf, id);
     if (slot == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
     else if (tf.s[slot].first > (uint32_t)a) atomicMin(&tf.s[slot].first, (uint32_t)a);
   } else {
     /* slots with a stream come from runtime rows and exist already */
-    slot = slot_find(tf, d[i].id);
+    slot = slot_find(tf, id);
   }
   slot_f_dev[i] = slot;
 }
@@ -662,15 +668,16 @@ __device__ __forceinline__ bool is_async_op(uint32_t domain) { return domain != 
  *  - checkTimestampOrder (GenericActivityProfiler.cpp:363-395) against the first row of the id,
  *  - the stream of the correlation-matched runtime row (RocmStreamQueue.h:56-75, first pass),
  *  - the size or grid/block the launching row hands over (RocprofActivity_inl.h:161-180). */
-__global__ void k_link_device(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, FullTable tf,
-                              NarrowTable tn, const uint32_t* slot_f_dev, DevLink* link, DevBrief* brief, Scalars* sc) {
+__global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, FullTable tf, NarrowTable tn,
+                              const uint32_t* slot_f_dev, DevLink* link, Scalars* sc) {
   uint32_t n_linked = 0, n_bad = 0, n_unresolved = 0;
   const bool have_stream_src = sc->have_stream_src != 0;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t a = first_device + i;
-    const uint64_t id = d[i].id;
-    const uint32_t domain = d[i].domain;
-    const bool valid = (c.meta[a] & KTJ_M_VALID) != 0;
+    const uint64_t id = c.corr[a];
+    const uint32_t meta = c.meta[a];
+    const uint32_t domain = (meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
+    const bool valid = (meta & KTJ_M_VALID) != 0;
     DevLink l;
     l.p[0] = l.p[1] = l.p[2] = 0; l.flags = 0; l.pad = 0;
     int32_t ext = 0;
@@ -704,9 +711,6 @@ __global__ void k_link_device(const ktj_device_rec* d, uint64_t n, Columns c, ui
       if (have_stream_src && is_async_op(domain) && res == 0 && fs.stream_src != 0) { res = (int64_t)fs.stream; c.res[a] = res; }
     }
     if (is_async_op(domain) && res == 0) ++n_unresolved;
-    DevBrief b;
-    b.queue = d[i].queue; b.device = d[i].device; b.domain = domain;
-    brief[i] = b;
   }
   block_add(&sc->n_linked, n_linked);
   block_add(&sc->out_of_order, n_bad);
@@ -724,17 +728,17 @@ hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, KeyTable cpu, Sca
   hipLaunchKernelGGL(k_build_cpu_ids, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, cpu, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t build_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, FullTable tf,
-                         NarrowTable tn, uint32_t* slot_f, uint32_t* slot_n, Scalars* sc, hipStream_t st) {
+hipError_t build_runtime(uint64_t n, Columns c, uint64_t first_runtime, FullTable tf, NarrowTable tn, uint32_t* slot_f,
+                         uint32_t* slot_n, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_build_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first_runtime, tf, tn,
+  hipLaunchKernelGGL(k_build_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_runtime, tf, tn,
                      slot_f, slot_n, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t insert_device_first(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, FullTable tf,
-                               uint32_t* slot_f_dev, Scalars* sc, hipStream_t st) {
+hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, FullTable tf, uint32_t* slot_f_dev,
+                               Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_insert_device_first, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, d, n, c, first_device, tf,
+  hipLaunchKernelGGL(k_insert_device_first, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_device, tf,
                      slot_f_dev, sc);
   return KTJ_LAUNCH_CHECK();
 }
@@ -744,12 +748,11 @@ hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn
   hipLaunchKernelGGL(k_resolve_external, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, tn, slot_ext, cpu);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t link_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first_device, FullTable tf,
-                            NarrowTable tn, const uint32_t* slot_f_dev, DevLink* link, DevBrief* brief, Scalars* sc,
-                            hipStream_t st) {
+hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, FullTable tf, NarrowTable tn,
+                            const uint32_t* slot_f_dev, DevLink* link, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_link_device, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, d, n, c, first_device, tf,
-                     tn, slot_f_dev, link, brief, sc);
+  hipLaunchKernelGGL(k_link_device, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_device, tf, tn,
+                     slot_f_dev, link, sc);
   return KTJ_LAUNCH_CHECK();
 }
 
@@ -1037,12 +1040,18 @@ hipError_t make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint3
   return KTJ_LAUNCH_CHECK();
 }
 
-/* ---- stable LSD radix sort, 8 bits per pass ---- */
-#define RADIX_ITEMS 8
+/* ---- stable LSD radix sort, 8 bits per pass ----
+ * A workgroup owns a tile of 4096 consecutive keys, one quarter per wavefront.  Ranks within the
+ * tile come from wavefront match (ballots) plus per-wavefront running counts; the tile is then
+ * laid out in LDS in digit order and written from there, so that neighbouring lanes store
+ * neighbouring elements of a digit's run (whole lines instead of single 8-byte stores). */
+#define RADIX_ITEMS 16
 #define RADIX_TILE (KTJ_BLOCK * RADIX_ITEMS)
 #define RADIX_WAVES (KTJ_BLOCK >> 6)
+#define RADIX_WAVE_KEYS (64 * RADIX_ITEMS)
 
-__global__ void k_radix_hist(const uint64_t* keys, uint64_t n, uint32_t shift, uint32_t* hist, uint32_t n_blocks) {
+__global__ void __launch_bounds__(KTJ_BLOCK)
+k_radix_hist(const uint64_t* keys, uint64_t n, uint32_t shift, uint32_t* hist, uint32_t n_blocks) {
   __shared__ uint32_t h[256];
   h[threadIdx.x] = 0;
   __syncthreads();
@@ -1054,47 +1063,79 @@ __global__ void k_radix_hist(const uint64_t* keys, uint64_t n, uint32_t shift, u
   __syncthreads();
   hist[(uint64_t)threadIdx.x * n_blocks + blockIdx.x] = h[threadIdx.x]; /* digit-major */
 }
-__global__ void k_radix_scatter(const uint64_t* keys_in, const uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out,
-                                uint64_t n, uint32_t shift, const uint32_t* hist_scanned, uint32_t n_blocks) {
-  __shared__ uint32_t base_of[256];               /* global offset of this block's run per digit */
-  __shared__ uint32_t run[256];                   /* elements of each digit already placed        */
-  __shared__ uint32_t wave_cnt[RADIX_WAVES][256];
+__global__ void __launch_bounds__(KTJ_BLOCK)
+k_radix_scatter(const uint64_t* keys_in, const uint32_t* vals_in, uint64_t* keys_out, uint32_t* vals_out, uint64_t n,
+                uint32_t shift, const uint32_t* hist_scanned, uint32_t n_blocks) {
+  __shared__ uint64_t s_key[RADIX_TILE];
+  __shared__ uint32_t s_val[RADIX_TILE];
+  __shared__ uint32_t wave_run[RADIX_WAVES][256]; /* count per (wavefront, digit), then its start inside the digit's run */
+  __shared__ uint32_t digit_start[256];           /* start of the digit's run inside the tile     */
+  __shared__ uint32_t base_of[256];               /* global offset of this tile's run per digit   */
+  __shared__ uint32_t wave_tot[RADIX_WAVES];
   base_of[threadIdx.x] = hist_scanned[(uint64_t)threadIdx.x * n_blocks + blockIdx.x];
-  run[threadIdx.x] = 0;
-  for (int w = 0; w < RADIX_WAVES; ++w) wave_cnt[w][threadIdx.x] = 0;
+  for (int k = 0; k < RADIX_WAVES; ++k) wave_run[k][threadIdx.x] = 0;
   __syncthreads();
-  const uint32_t w = threadIdx.x >> 6;
+  const uint32_t w = threadIdx.x >> 6, lane = lane_id();
   const uint64_t lt = lanemask_lt();
-  const uint64_t base = (uint64_t)blockIdx.x * RADIX_TILE;
+  const uint64_t tile_base = (uint64_t)blockIdx.x * RADIX_TILE;
+  const uint64_t chunk = tile_base + (uint64_t)w * RADIX_WAVE_KEYS;
+  volatile uint32_t* my_run = wave_run[w];
+  uint64_t key[RADIX_ITEMS];
+  uint32_t val[RADIX_ITEMS], rank[RADIX_ITEMS];
+#pragma unroll
   for (int r = 0; r < RADIX_ITEMS; ++r) {
-    const uint64_t i = base + (uint64_t)r * KTJ_BLOCK + threadIdx.x;
+    const uint64_t i = chunk + (uint64_t)r * 64u + lane;
     const bool valid = i < n;
-    const uint64_t key = valid ? keys_in[i] : 0;
-    const uint32_t val = valid ? vals_in[i] : 0;
-    const uint32_t digit = (uint32_t)(key >> shift) & 0xFFu;
+    key[r] = valid ? keys_in[i] : ~0ULL;
+    val[r] = valid ? vals_in[i] : 0u;
+  }
+#pragma unroll
+  for (int r = 0; r < RADIX_ITEMS; ++r) {
+    const bool valid = chunk + (uint64_t)r * 64u + lane < n;
+    const uint32_t digit = (uint32_t)(key[r] >> shift) & 0xFFu;
     /* lanes of this wavefront holding the same digit */
     uint64_t peers = __ballot(valid ? 1 : 0);
+#pragma unroll
     for (int b = 0; b < 8; ++b) {
       const uint64_t bal = __ballot((digit >> b) & 1u);
       peers &= ((digit >> b) & 1u) ? bal : ~bal;
     }
     const uint32_t rank_in_wave = (uint32_t)__popcll(peers & lt);
-    if (valid && rank_in_wave == 0) wave_cnt[w][digit] = (uint32_t)__popcll(peers);
+    const uint32_t before = my_run[digit];   /* same digit in earlier rounds of this wavefront */
+    rank[r] = before + rank_in_wave;
+    if (valid && rank_in_wave == 0) my_run[digit] = before + (uint32_t)__popcll(peers);
+  }
+  __syncthreads();
+  {
+    /* per digit: wavefront counts -> starts inside the digit's run; digit totals -> exclusive scan */
+    uint32_t tot = 0;
+    for (int k = 0; k < RADIX_WAVES; ++k) { const uint32_t cnt = wave_run[k][threadIdx.x]; wave_run[k][threadIdx.x] = tot; tot += cnt; }
+    uint32_t inc = tot;
+    for (int o = 1; o < 64; o <<= 1) { const uint32_t t = __shfl_up(inc, o); if (lane >= (uint32_t)o) inc += t; }
+    if (lane == 63) wave_tot[w] = inc;
     __syncthreads();
-    if (valid) {
-      uint32_t off = run[digit] + rank_in_wave;
-      for (uint32_t k = 0; k < w; ++k) off += wave_cnt[k][digit];
-      const uint64_t dst = (uint64_t)base_of[digit] + off;
-      keys_out[dst] = key;
-      vals_out[dst] = val;
+    uint32_t add = 0;
+    for (uint32_t k = 0; k < w; ++k) add += wave_tot[k];
+    digit_start[threadIdx.x] = add + inc - tot;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < RADIX_ITEMS; ++r) {
+    if (chunk + (uint64_t)r * 64u + lane < n) {
+      const uint32_t digit = (uint32_t)(key[r] >> shift) & 0xFFu;
+      const uint32_t p = digit_start[digit] + wave_run[w][digit] + rank[r];
+      s_key[p] = key[r];
+      s_val[p] = val[r];
     }
-    __syncthreads();
-    {
-      uint32_t s = 0;
-      for (int k = 0; k < RADIX_WAVES; ++k) { s += wave_cnt[k][threadIdx.x]; wave_cnt[k][threadIdx.x] = 0; }
-      run[threadIdx.x] += s;
-    }
-    __syncthreads();
+  }
+  __syncthreads();
+  const uint32_t cnt = (uint32_t)(n - tile_base < RADIX_TILE ? n - tile_base : RADIX_TILE);
+  for (uint32_t p = threadIdx.x; p < cnt; p += KTJ_BLOCK) {
+    const uint64_t k = s_key[p];
+    const uint32_t digit = (uint32_t)(k >> shift) & 0xFFu;
+    const uint64_t dst = (uint64_t)base_of[digit] + (p - digit_start[digit]);
+    keys_out[dst] = k;
+    vals_out[dst] = s_val[p];
   }
 }
 

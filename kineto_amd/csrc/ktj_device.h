@@ -53,6 +53,7 @@ struct MatRow {
 #define KTJ_M_HAS_KERNEL_ARG (1u << 15)
 #define KTJ_M_MALLOC_BYTES (1u << 16)
 #define KTJ_M_NAME_BUILTIN (1u << 17)
+#define KTJ_M_HAS_STREAM (1u << 18) /* meta column of runtime rows only: the row carries a stream */
 
 #define KTJ_CLASS_GENERIC 0u
 #define KTJ_CLASS_RUNTIME 1u
