@@ -397,6 +397,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(e->c_ts.ensure(Na * 8)); HIPCHK(e->c_dur.ensure(Na * 8)); HIPCHK(e->c_corr.ensure(Na * 8));
   HIPCHK(e->c_dev.ensure(Na * 8)); HIPCHK(e->c_res.ensure(Na * 8)); HIPCHK(e->c_meta.ensure(Na * 4));
   HIPCHK(e->c_ext.ensure(Na * 4));
+  if (nx >= 0x7FFFFFFFull || nr >= 0x7FFFFFFFull) { e->last_error = "more than 2^31 - 2 records of one class"; return KTJ_ERR_LIMIT; }
   /* capacities for the hash mode (load <= 2/3); the direct mode uses a prefix of the same buffers */
   const uint32_t cap_full = pow2_at_least((nr + nd) + (nr + nd) / 2);
   const uint32_t cap_narrow = pow2_at_least((nx + nr) + (nx + nr) / 2), cap_cpu = pow2_at_least(2 * ng);

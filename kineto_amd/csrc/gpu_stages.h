@@ -41,15 +41,15 @@ struct FullSlot {
 /* keyed by the int-narrowed correlation id (and by the external-correlation records' full id) */
 struct NarrowSlot {
   uint64_t key;
-  uint32_t ext_src;        /* last external-correlation record (index + 1), 0 = none           */
+  uint32_t ext_src;        /* last external-correlation record (index + 1), 0 = none; bit 31 is
+                              set once ext_val names an existing CPU op                          */
   int32_t ext_val;         /* its external id if a CPU op with that id exists, else 0           */
   uint32_t kern_src;       /* last in-window kernel-launch row (index + 1)                     */
   uint32_t copy_src;       /* last in-window copy / malloc row (index + 1)                     */
-  uint64_t size;           /* bytes of row copy_src                                             */
-  uint64_t grid[3];        /* packed grid / workgroup of row kern_src (see pack_grid)           */
-  uint32_t linked;         /* 1 when ext_val names an existing CPU op                           */
-  uint32_t pad;
-};                         /* 64 bytes */
+  uint64_t pay[3];         /* copy_src != 0: bytes of that row in pay[0]; else packed grid /
+                              workgroup of row kern_src (see pack_grid)                         */
+};                         /* 48 bytes */
+#define KTJ_EXT_LINKED 0x80000000u
 struct KeySlot {           /* plain set */
   uint64_t key;
 };

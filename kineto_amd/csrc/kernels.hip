@@ -565,8 +565,8 @@ hipError_t clear_tables(FullTable tf, NarrowTable tn, KeyTable cpu, hipStream_t 
   FullSlot f;
   f.key = KTJ_EMPTY_KEY; f.stream_src = 0; f.first = 0xFFFFFFFFu; f.first_ts = 0; f.stream = 0;
   NarrowSlot nn;
-  nn.key = KTJ_EMPTY_KEY; nn.ext_src = 0; nn.ext_val = 0; nn.kern_src = 0; nn.copy_src = 0; nn.size = 0;
-  nn.grid[0] = nn.grid[1] = nn.grid[2] = 0; nn.linked = 0; nn.pad = 0;
+  nn.key = KTJ_EMPTY_KEY; nn.ext_src = 0; nn.ext_val = 0; nn.kern_src = 0; nn.copy_src = 0;
+  nn.pay[0] = nn.pay[1] = nn.pay[2] = 0;
   KeySlot k;
   k.key = KTJ_EMPTY_KEY;
   hipLaunchKernelGGL(k_clear_table<FullSlot>, dim3(grid_stride_for((uint64_t)tf.mask + 1, KTJ_BLOCK * 4)), dim3(KTJ_BLOCK), 0, st, tf, f);
@@ -654,11 +654,11 @@ __global__ void k_resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowT
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint32_t slot = slot_ext[i];
-  if (slot == KTJ_NOSLOT || tn.s[slot].ext_src != (uint32_t)i + 1u) return;
+  if (slot == KTJ_NOSLOT || (tn.s[slot].ext_src & ~KTJ_EXT_LINKED) != (uint32_t)i + 1u) return;
   const uint64_t ext_id = e[i].external_id;
   if (slot_find(cpu, ext_id) != KTJ_NOSLOT) {
     tn.s[slot].ext_val = (int32_t)(int64_t)ext_id;
-    tn.s[slot].linked = 1u;
+    tn.s[slot].ext_src = ((uint32_t)i + 1u) | KTJ_EXT_LINKED; /* only the winner writes here */
   }
 }
 __device__ __forceinline__ bool is_async_op(uint32_t domain) { return domain != KTJ_DOM_MEMSET; }
@@ -685,10 +685,10 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Full
     if (sn != KTJ_NOSLOT) {
       const NarrowSlot ns = tn.s[sn];
       ext = ns.ext_val;
-      if (ns.linked && valid) ++n_linked;
+      if ((ns.ext_src & KTJ_EXT_LINKED) && valid) ++n_linked;
       if (domain != KTJ_DOM_MEMSET) {
-        if (ns.copy_src != 0) { l.flags = KTJ_DL_HAS_SIZE; l.p[0] = ns.size; }
-        else if (ns.kern_src != 0) { l.flags = KTJ_DL_HAS_GRID; l.p[0] = ns.grid[0]; l.p[1] = ns.grid[1]; l.p[2] = ns.grid[2]; }
+        if (ns.copy_src != 0) { l.flags = KTJ_DL_HAS_SIZE; l.p[0] = ns.pay[0]; }
+        else if (ns.kern_src != 0) { l.flags = KTJ_DL_HAS_GRID; l.p[0] = ns.pay[0]; l.p[1] = ns.pay[1]; l.p[2] = ns.pay[2]; }
       }
     }
     c.ext[a] = ext;
@@ -1230,9 +1230,10 @@ __global__ void k_mat_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, u
     if (sn != KTJ_NOSLOT) {
       NarrowSlot* ns = &tn.s[sn];
       ext = ns->ext_val;
-      if (ns->linked && valid) ++n_linked;
-      if (ns->kern_src == (uint32_t)i + 1u) pack_grid(rec, ns->grid);
-      if (ns->copy_src == (uint32_t)i + 1u) ns->size = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
+      if ((ns->ext_src & KTJ_EXT_LINKED) && valid) ++n_linked;
+      const uint32_t copy_src = ns->copy_src; /* final: the build pass has ended */
+      if (copy_src == (uint32_t)i + 1u) ns->pay[0] = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
+      else if (copy_src == 0 && ns->kern_src == (uint32_t)i + 1u) pack_grid(rec, ns->pay);
     }
     c.ext[a] = ext;
     const bool known = rec.cid < api.n_cids;

@@ -82,6 +82,15 @@ class TraceEngine:
         self._chk(self.lib.ktj_output_host(self.h, C.byref(p), C.byref(n)), "ktj_output_host")
         return C.string_at(p, n.value)
 
+    def output_view(self):
+        """The finished document as a uint8 numpy view of the engine's pinned host copy (no copy;
+        valid until the next process() or close(); works beyond 2 GiB)."""
+        p, n = C.c_void_p(), C.c_uint64()
+        self._chk(self.lib.ktj_output_host(self.h, C.byref(p), C.byref(n)), "ktj_output_host")
+        if n.value == 0:
+            return np.zeros(0, dtype=np.uint8)
+        return np.ctypeslib.as_array((C.c_ubyte * n.value).from_address(p.value))
+
     def output_size(self):
         p, n = C.c_void_p(), C.c_uint64()
         self._chk(self.lib.ktj_output_device(self.h, C.byref(p), C.byref(n)), "ktj_output_device")

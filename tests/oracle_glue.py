@@ -123,6 +123,15 @@ class OracleRun:
         self.lib.ktj_oracle_output(self.h, C.byref(p), C.byref(n))
         return C.string_at(p, n.value)
 
+    def output_view(self):
+        """uint8 numpy view of the oracle's document (no copy; works beyond 2 GiB)."""
+        import numpy as np
+        p, n = C.c_void_p(), C.c_uint64()
+        self.lib.ktj_oracle_output(self.h, C.byref(p), C.byref(n))
+        if n.value == 0:
+            return np.zeros(0, dtype=np.uint8)
+        return np.ctypeslib.as_array((C.c_ubyte * n.value).from_address(p.value))
+
     def activities(self):
         p, n = C.POINTER(MatActivity)(), C.c_uint64()
         self.lib.ktj_oracle_activities(self.h, C.byref(p), C.byref(n))
