@@ -47,9 +47,9 @@ struct DevVec {
   size_t bytes = 0;
   hipError_t append(const void* src, size_t n, hipStream_t st) {
     if (n == 0) return hipSuccess;
-    if (bytes + n > buf.cap) {
+    if (bytes + n + 16 > buf.cap) { /* 16 spare bytes: string copies load whole aligned words */
       DevBuf nb;
-      size_t want = (bytes + n) * 2;
+      size_t want = (bytes + n) * 2 + 16;
       hipError_t e = nb.ensure(want);
       if (e != hipSuccess) return e;
       if (bytes) { e = hipMemcpyAsync(nb.p, buf.p, bytes, hipMemcpyDeviceToDevice, st); if (e != hipSuccess) return e; }
@@ -114,7 +114,7 @@ struct ktj_engine {
   /* working buffers */
   DevBuf d_scalars, d_name_len, d_arg_len, d_sflags, d_name_off, d_arg_off, d_name_blob, d_arg_blob;
   DevBuf c_ts, c_dur, c_corr, c_dev, c_res, c_meta, c_ext;
-  DevBuf t_full, t_narrow, t_cpu, slot_ext, slot_f, slot_n, slot_f_dev, dev_link, dev_brief;
+  DevBuf t_full, t_narrow, t_cpu, slot_ext, slot_f, slot_n, slot_f_dev, dev_link, dev_brief, sync_keys, sync_pos, sync_first;
   DevBuf q_keys, q_stream, q_amb, dn_hash, dn_first, dn_dev, dn_key, dn_rank;
   DevBuf s_dev_k, s_dev_r, s_res_k, s_res_r;
   DevBuf keys_a, keys_b, vals_a, vals_b, hist, scan_tmp;
@@ -202,7 +202,7 @@ void ktj_destroy(ktj_engine* e) {
   DevBuf* bufs[] = {&e->d_fields, &e->d_schemas, &e->d_cid_names, &e->d_flow_bits, &e->d_scalars, &e->d_name_len,
                     &e->d_arg_len, &e->d_sflags, &e->d_name_off, &e->d_arg_off, &e->d_name_blob, &e->d_arg_blob,
                     &e->c_ts, &e->c_dur, &e->c_corr, &e->c_dev, &e->c_res, &e->c_meta, &e->c_ext, &e->t_full,
-                    &e->t_narrow, &e->t_cpu, &e->slot_ext, &e->slot_f, &e->slot_n, &e->slot_f_dev, &e->dev_link, &e->dev_brief, &e->q_keys, &e->q_stream, &e->q_amb, &e->dn_hash, &e->dn_first, &e->dn_dev,
+                    &e->t_narrow, &e->t_cpu, &e->slot_ext, &e->slot_f, &e->slot_n, &e->slot_f_dev, &e->dev_link, &e->dev_brief, &e->sync_keys, &e->sync_pos, &e->sync_first, &e->q_keys, &e->q_stream, &e->q_amb, &e->dn_hash, &e->dn_first, &e->dn_dev,
                     &e->dn_key, &e->dn_rank, &e->s_dev_k, &e->s_dev_r, &e->s_res_k, &e->s_res_r, &e->keys_a,
                     &e->keys_b, &e->vals_a, &e->vals_b, &e->hist, &e->scan_tmp, &e->mat, &e->len, &e->len_sorted,
                     &e->offs, &e->out, &e->tile_start};
@@ -444,6 +444,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   EmitCtx ctx;
   ctx.dict.name_blob = e->d_name_blob.as<char>(); ctx.dict.name_off = e->d_name_off.as<uint64_t>();
   ctx.dict.arg_blob = e->d_arg_blob.as<char>(); ctx.dict.arg_off = e->d_arg_off.as<uint64_t>();
+  ctx.dict.raw_blob = e->str_blob.buf.as<char>(); ctx.dict.raw_off = e->str_off.buf.as<uint64_t>();
   ctx.dict.flags = e->d_sflags.as<uint32_t>(); ctx.dict.n = ns;
   ctx.fields = e->d_fields.as<ktj_field>(); ctx.schemas = e->d_schemas.as<ktj_schema_desc>();
   ctx.n_schemas = (uint32_t)e->schemas.size();
@@ -461,7 +462,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(hipEventRecord(e->ev[EV_DICT], st));
 
   /* ---- stage 1: decode ---- */
-  HIPCHK(decode_generic(g_recs, ng, c, 0, st));
+  HIPCHK(decode_generic(g_recs, ng, c, 0, sc, st));
   HIPCHK(decode_runtime(r_recs, nr, c, ng, st));
   HIPCHK(decode_device(d_recs, nd, c, ng + nr, e->dev_brief.as<DevBrief>(), st));
   HIPCHK(hipEventRecord(e->ev[EV_DECODE], st));
@@ -531,7 +532,15 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(hipEventRecord(e->ev[EV_SORT], st));
 
   /* ---- stage 4a: joined rows + lengths ---- */
-  HIPCHK(mat_generic_rows(g_recs, ng, ctx, mat, e->len.as<uint32_t>(), sc, st));
+  const uint32_t* sync_first = nullptr;
+  if (e->scalars.n_sync_typed != 0) { /* known since the read-back before the sort */
+    HIPCHK(e->sync_keys.ensure((KTJ_SYNC_CAP + 1ull) * 8)); HIPCHK(e->sync_pos.ensure((KTJ_SYNC_CAP + 1ull) * 4));
+    HIPCHK(e->sync_first.ensure(ng * 4 + 16));
+    HIPCHK(stream_sync_first(e->perm, e->scalars.n_valid, g_recs, ng, ctx.dict, e->sync_keys.as<uint64_t>(),
+                             e->sync_pos.as<uint32_t>(), e->sync_first.as<uint32_t>(), sc, st));
+    sync_first = e->sync_first.as<uint32_t>();
+  }
+  HIPCHK(mat_generic_rows(g_recs, ng, ctx, sync_first, mat, e->len.as<uint32_t>(), sc, st));
   HIPCHK(mat_device_rows(d_recs, nd, c, ng + nr, e->dev_link.as<DevLink>(), ctx, mat, e->len.as<uint32_t>(), sc, st));
   HIPCHK(gather_len(e->perm, e->len.as<uint32_t>(), N, e->len_sorted.as<uint32_t>(), st));
   HIPCHK(hipEventRecord(e->ev[EV_SIZE], st));

@@ -613,8 +613,10 @@ KTJ_HD KTJ_FI inline int format_double(uint64_t bits, char* out) {
   return b.n;
 }
 
-template <class W> KTJ_HD KTJ_FI inline void put_arg_string(W& w, const DictViews& d, uint32_t id) {
-  if (id < d.n) w.str(d.arg_blob + d.arg_off[id], d.arg_off[id + 1] - d.arg_off[id]);
+template <class W> KTJ_HD KTJ_FI inline void put_arg_string(W& w, const DictViews& d, uint32_t id, bool raw = false) {
+  if (id >= d.n) return;
+  if (raw) w.str(d.raw_blob + d.raw_off[id], d.raw_off[id + 1] - d.raw_off[id]);
+  else w.str(d.arg_blob + d.arg_off[id], d.arg_off[id + 1] - d.arg_off[id]);
 }
 template <class W> KTJ_HD KTJ_FI inline void put_array3(W& w, uint64_t a, uint64_t b, uint64_t c) {
   w.ch('['); put_i64(w, (int64_t)a); KTJ_PUT(w, ", "); put_i64(w, (int64_t)b); KTJ_PUT(w, ", ");
@@ -697,8 +699,8 @@ KTJ_HD KTJ_FI inline bool has_fragment(const MatRow& r, const EmitCtx& c) {
   return true;
 }
 
-/* the metadataJson() fragment, after sanitizeStrForJSON */
-template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r, const EmitCtx& c) {
+/* the metadataJson() fragment, after sanitizeStrForJSON (raw: as metadataJson() returned it) */
+template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r, const EmitCtx& c, bool raw = false) {
   const uint32_t cls = (r.meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT;
   const uint32_t kind = (r.meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
   if (cls == KTJ_CLASS_GENERIC) { /* GenericTraceActivity.cpp:60-64 + TypedMetadataJson.h */
@@ -710,7 +712,7 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
       if (fd.key_id != KTJ_NONE) {
         if (!first) KTJ_PUT(w, ", ");
         first = false;
-        w.ch('"'); put_arg_string(w, c.dict, fd.key_id); KTJ_PUT(w, "\": ");
+        w.ch('"'); put_arg_string(w, c.dict, fd.key_id, raw); KTJ_PUT(w, "\": ");
       }
       const uint64_t v = slot < c.n_args ? c.args[slot] : 0;
       switch (fd.type) {
@@ -718,8 +720,8 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
         case KTJ_F_U64: w.dec(v); break;
         case KTJ_F_F64: put_f64(w, v); break;
         case KTJ_F_BOOL: if (v) KTJ_PUT(w, "true"); else KTJ_PUT(w, "false"); break;
-        case KTJ_F_STR: w.ch('"'); put_arg_string(w, c.dict, (uint32_t)v); w.ch('"'); break;
-        case KTJ_F_RAW: put_arg_string(w, c.dict, (uint32_t)v); break;
+        case KTJ_F_STR: w.ch('"'); put_arg_string(w, c.dict, (uint32_t)v, raw); w.ch('"'); break;
+        case KTJ_F_RAW: put_arg_string(w, c.dict, (uint32_t)v, raw); break;
         case KTJ_F_I64_ARRAY:
           w.ch('[');
           for (uint32_t k = 0; k < fd.count; ++k) {
@@ -814,20 +816,63 @@ template <class W> KTJ_HD KTJ_FI inline void put_name(W& w, const MatRow& r, con
     w.str(c.dict.name_blob + c.dict.name_off[r.name_id], c.dict.name_off[r.name_id + 1] - c.dict.name_off[r.name_id]);
 }
 
+/* Generic rows only: marks a CUDA_SYNC activity named "Stream Sync" (output_json.cpp:915) and
+ * whether it is the first of its (device, row) in emission order. */
+KTJ_HD KTJ_FI inline void mark_stream_sync(MatRow& m, const EmitCtx& c, bool first_of_row) {
+  if ((m.meta & KTJ_M_TYPE_MASK) != KTJ_TYPE_CUDA_SYNC || (m.meta & KTJ_M_NAME_BUILTIN) || m.name_id >= c.dict.n) return;
+  if (!(c.dict.flags[m.name_id] & KTJ_SF_STREAM_SYNC)) return;
+  m.meta |= KTJ_M_SYNC;
+  if (first_of_row) m.meta |= KTJ_M_SYNC_FIRST;
+}
+/* (device << 32) | virtual tid, the key of syncStreamMetadataEmitted_ (output_json.cpp:917) */
+KTJ_HD KTJ_FI inline uint64_t stream_sync_key(int64_t device, int64_t resource) {
+  return ((uint64_t)device << 32) | (uint64_t)(resource + KTJ_SYNC_TID_OFFSET);
+}
+
+/* handleGenericInstantEvent + writeInstantEvent (output_json.cpp:660-677, 261-292): name and
+ * metadata are printed as they were handed over, no flow event follows. */
+template <class W> KTJ_HD KTJ_FI inline void format_instant(W& w, const MatRow& r, const EmitCtx& c) {
+  int64_t rel = r.ts - c.base_time_ns;
+  if (rel < 0) rel = 0;
+  KTJ_PUT(w, "\n  {\n    \"ph\": \"i\",\n    \n    \"cat\": \"cpu_instant_event\",\n    \"s\": \"t\",\n    \"name\": \"");
+  if (!(r.meta & KTJ_M_NAME_BUILTIN)) put_arg_string(w, c.dict, r.name_id, true);
+  KTJ_PUT(w, "\",\n    \"pid\": "); put_i64(w, r.dev);
+  KTJ_PUT(w, ",\n    \"tid\": "); w.dec((uint64_t)sanitize_tid(r.res));
+  KTJ_PUT(w, ",\n    \"ts\": "); put_ts(w, rel);
+  if (has_fragment(r, c)) {
+    KTJ_PUT(w, "\n    ,\n    \"args\": {\n      ");
+    put_fragment(w, r, c, true);
+    KTJ_PUT(w, "\n    }\n  },");
+  } else KTJ_PUT(w, "\n    \n  },");
+}
+
 /* One activity: the complete event and, if it takes part in a flow, the flow event after it. */
 template <class W> KTJ_HD KTJ_FI inline void format_activity(W& w, const MatRow& r, const EmitCtx& c) {
   const uint32_t type = r.meta & KTJ_M_TYPE_MASK;
+  if (type == KTJ_TYPE_CPU_INSTANT_EVENT && ((r.meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT) == KTJ_CLASS_GENERIC) {
+    format_instant(w, r, c);
+    return;
+  }
   int64_t ts = r.ts;
   int64_t dur = r.dur < 0 ? 0 : r.dur;                       /* output_json.cpp:860 */
   if (type == KTJ_TYPE_GPU_USER_ANNOTATION) { ts -= 1; dur += 2; } /* :862-869 */
   int64_t rel = ts - c.base_time_ns;                         /* transToRelativeTime :144-153 */
   if (rel < 0) rel = 0;
-  const int64_t tid = sanitize_tid(r.res);
+  /* Stream Sync activities sit on a row of their own (output_json.cpp:913-943, 1008-1013) */
+  const int64_t tid = sanitize_tid((r.meta & KTJ_M_SYNC) ? r.res + KTJ_SYNC_TID_OFFSET : r.res);
   const bool flow = (r.meta & KTJ_M_FLOW) != 0;
   /* pid and tid are printed again by the flow event */
   const bool pid_neg = r.dev < 0;
   const typename W::Prepared pid = W::prepare(pid_neg ? 0ULL - (uint64_t)r.dev : (uint64_t)r.dev);
   const typename W::Prepared tidn = W::prepare((uint64_t)tid);
+  if (r.meta & KTJ_M_SYNC_FIRST) { /* the row is announced once, before its first activity */
+    KTJ_PUT(w, "\n  {\n    \"name\": \"thread_name\", \"ph\": \"M\", \"ts\": "); put_ts(w, rel);
+    KTJ_PUT(w, ", \"pid\": "); put_i64(w, r.dev); KTJ_PUT(w, ", \"tid\": "); put_i64(w, r.res + KTJ_SYNC_TID_OFFSET);
+    KTJ_PUT(w, ",\n    \"args\": {\n      \"name\": \"stream "); put_i64(w, r.res); KTJ_PUT(w, " (sync)\"\n    }\n  },");
+    KTJ_PUT(w, "\n  {\n    \"name\": \"thread_sort_index\", \"ph\": \"M\", \"ts\": "); put_ts(w, rel);
+    KTJ_PUT(w, ", \"pid\": "); put_i64(w, r.dev); KTJ_PUT(w, ", \"tid\": "); put_i64(w, r.res + KTJ_SYNC_TID_OFFSET);
+    KTJ_PUT(w, ",\n    \"args\": {\n      \"sort_index\": "); put_i64(w, r.res); KTJ_PUT(w, "\n    }\n  },");
+  }
   KTJ_PUT(w, "\n  {\n    \"ph\": \"X\",\n    \"cat\": \"");
   put_category(w, type);
   KTJ_PUT(w, "\",\n    \"name\": \"");

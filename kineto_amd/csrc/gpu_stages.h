@@ -106,6 +106,7 @@ struct Scalars {
   unsigned long long n_blank_names;
   unsigned long long n_valid;
   unsigned long long n_unresolved;    /* device rows still without a stream after the correlation pass */
+  unsigned long long n_sync_typed;    /* generic rows of type CUDA_SYNC */
   unsigned int error;                 /* KTJ_DEVERR_* bits */
   unsigned int have_stream_src;       /* some runtime row carries a stream */
   unsigned int n_dev_ranks;           /* distinct deviceId values */
@@ -122,6 +123,7 @@ struct Scalars {
 #define KTJ_SET_CAP 16384u     /* slots of the distinct-value sets (at most half may be used) */
 #define KTJ_DENSE_CAP 8192u    /* slots of the (device, stream) table */
 #define KTJ_QUEUE_CAP 65536u   /* slots of the queue -> stream table */
+#define KTJ_SYNC_CAP 65536u    /* slots of the Stream Sync (device, row) table */
 
 struct ApiTable {
   const uint32_t* cid_name_ids;
@@ -148,7 +150,7 @@ hipError_t dict_write(const char* blob, const uint64_t* off, uint32_t n, const u
                       const uint64_t* arg_off, const uint32_t* flags, char* name_blob, char* arg_blob, hipStream_t st);
 
 /* ---- stage 1: decode ---- */
-hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st);
+hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, Scalars* sc, hipStream_t st);
 hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st);
 hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, DevBrief* brief, hipStream_t st);
 
@@ -210,8 +212,13 @@ hipError_t radix_sort(uint64_t* keys_a, uint32_t* vals_a, uint64_t* keys_b, uint
                       uint64_t** res_keys, uint32_t** res_vals, hipStream_t st);
 
 /* ---- stage 4a: joined rows + exact byte length (arrival order) ---- */
-hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, MatRow* mat, uint32_t* len,
-                            Scalars* sc, hipStream_t st);
+/* keys: KTJ_SYNC_CAP + 1, first_pos: KTJ_SYNC_CAP + 1, is_first: n_generic (all caller-provided) */
+hipError_t stream_sync_first(const uint32_t* perm, uint64_t n_sorted, const ktj_generic_rec* g, uint64_t n_generic,
+                             DictViews d, uint64_t* keys, uint32_t* first_pos, uint32_t* is_first, Scalars* sc,
+                             hipStream_t st);
+/* sync_first: per generic row, from stream_sync_first, or null when there are no such rows */
+hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, const uint32_t* sync_first, MatRow* mat,
+                            uint32_t* len, Scalars* sc, hipStream_t st);
 /* runtime rows: also publishes what device rows take over (first timestamp, stream, grid, size)
  * into the tables, reads the "External id" and counts timestamp-order violations; runs after
  * resolve_external and before link_device_rows */

@@ -156,7 +156,7 @@ __global__ void k_init_scalars(Scalars* s) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     s->ts_min_biased = ~0ULL; s->ts_max_biased = 0;
     s->out_of_range = 0; s->out_of_order = 0; s->n_flow = 0; s->n_linked = 0; s->n_blank_names = 0; s->n_valid = 0;
-    s->n_unresolved = 0; s->error = 0; s->have_stream_src = 0; s->n_dev_ranks = 0; s->n_res_ranks = 0; s->n_dense = 0; s->pad = 0;
+    s->n_unresolved = 0; s->n_sync_typed = 0; s->error = 0; s->have_stream_src = 0; s->n_dev_ranks = 0; s->n_res_ranks = 0; s->n_dense = 0; s->pad = 0;
     for (int k = 0; k < 3; ++k) {
       s->plan.range[k].lo = ~0ULL; s->plan.range[k].hi = 0;
       s->plan.ctl[k].base = 0; s->plan.ctl[k].span = 0; s->plan.ctl[k].direct = 0; s->plan.ctl[k].pad = 0;
@@ -283,8 +283,6 @@ hipError_t scan_u32_inplace(uint32_t* data, uint64_t n, uint64_t* tmp, hipStream
 /*   name view = "kernel"→"Kernel", sanitize, non-printable → "unknown", quote escaping         */
 /*                                             (output_json.cpp:946-949, 86-112)                */
 /* ------------------------------------------------------------------------------------------ */
-#define KTJ_SF_NAME_KERNEL 4u
-
 __global__ void k_dict_measure(const char* blob, const uint64_t* off, uint32_t n, uint32_t* name_len,
                                uint32_t* arg_len, uint32_t* flags) {
   const uint32_t id = blockIdx.x * (KTJ_BLOCK >> 6) + (threadIdx.x >> 6);
@@ -308,6 +306,12 @@ __global__ void k_dict_measure(const char* blob, const uint64_t* off, uint32_t n
     else if (bad) { f |= KTJ_SF_NAME_UNKNOWN; nlen = 7; }
     else nlen = (uint32_t)len - nl + q;
     if (nonblank == 0) f |= KTJ_SF_ARG_BLANK;
+    if (len == 11) {
+      const char* want = "Stream Sync";
+      bool same = true;
+      for (int k = 0; k < 11; ++k) same = same && p[k] == want[k];
+      if (same) f |= KTJ_SF_STREAM_SYNC;
+    }
     name_len[id] = nlen;
     arg_len[id] = (uint32_t)len - nl;
     flags[id] = f;
@@ -385,10 +389,13 @@ __device__ __forceinline__ const Rec* stage_records(const Rec* recs, uint64_t n,
   return reinterpret_cast<const Rec*>(stage);
 }
 
-__global__ void k_decode_generic(const ktj_generic_rec* recs, uint64_t n, Columns c, uint64_t first) {
+__global__ void k_decode_generic(const ktj_generic_rec* recs, uint64_t n, Columns c, uint64_t first, Scalars* sc) {
   __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_generic_rec) / 16];
   uint32_t cnt;
   const ktj_generic_rec* l = stage_records(recs, n, stage, &cnt);
+  /* rows that may need a Stream Sync row of their own are rare: the extra passes run only if any */
+  const bool sync_typed = threadIdx.x < cnt && l[threadIdx.x].type == KTJ_TYPE_CUDA_SYNC;
+  if (__syncthreads_or(sync_typed ? 1 : 0)) block_add(&sc->n_sync_typed, sync_typed ? 1u : 0u);
   if (threadIdx.x >= cnt) return;
   const ktj_generic_rec g = l[threadIdx.x];
   const uint64_t a = first + (uint64_t)blockIdx.x * KTJ_BLOCK + threadIdx.x;
@@ -437,9 +444,9 @@ __global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns 
   brief[a - first] = b;
 }
 
-hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st) {
+hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_decode_generic, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first);
+  hipLaunchKernelGGL(k_decode_generic, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st) {
@@ -1191,10 +1198,59 @@ __device__ __forceinline__ void flush_row_stats(const RowStats& rs, Scalars* sc)
   block_add(&sc->n_blank_names, rs.n_blank);
 }
 
-__global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc) {
+/* Stream Sync rows (output_json.cpp:913-943): which activity is the first of its (device, row) key
+ * in emission order.  Pass a: smallest sorted position per key; pass b: the activity at that
+ * position is marked.  Both run over the sorted positions of generic rows only when the stream
+ * holds CUDA_SYNC activities at all. */
+__device__ __forceinline__ bool is_stream_sync(const ktj_generic_rec& g, const DictViews& d) {
+  return g.type == KTJ_TYPE_CUDA_SYNC && g.name_id < d.n && (d.flags[g.name_id] & KTJ_SF_STREAM_SYNC);
+}
+__global__ void k_sync_first_a(const uint32_t* perm, uint64_t n_sorted, const ktj_generic_rec* g, uint64_t n_generic,
+                               DictViews d, uint64_t* keys, uint32_t* first_pos, Scalars* sc) {
+  const uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n_sorted) return;
+  const uint64_t a = perm[p];
+  if (a >= n_generic || !is_stream_sync(g[a], d)) return;
+  const uint32_t slot = table_insert(keys, KTJ_SYNC_CAP - 1u, stream_sync_key(g[a].device, g[a].resource));
+  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT); return; }
+  atomicMin(&first_pos[slot], (uint32_t)p);
+}
+__global__ void k_sync_first_b(const uint32_t* perm, uint64_t n_sorted, const ktj_generic_rec* g, uint64_t n_generic,
+                               DictViews d, const uint64_t* keys, const uint32_t* first_pos, uint32_t* is_first) {
+  const uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n_sorted) return;
+  const uint64_t a = perm[p];
+  if (a >= n_generic) return;
+  uint32_t first = 0;
+  if (is_stream_sync(g[a], d)) {
+    const uint32_t slot = table_find(keys, KTJ_SYNC_CAP - 1u, stream_sync_key(g[a].device, g[a].resource));
+    first = slot != KTJ_NOSLOT && first_pos[slot] == (uint32_t)p;
+  }
+  is_first[a] = first;
+}
+hipError_t stream_sync_first(const uint32_t* perm, uint64_t n_sorted, const ktj_generic_rec* g, uint64_t n_generic,
+                             DictViews d, uint64_t* keys, uint32_t* first_pos, uint32_t* is_first, Scalars* sc,
+                             hipStream_t st) {
+  if (n_sorted == 0 || n_generic == 0) return hipSuccess;
+  hipError_t e = fill_u64(keys, KTJ_EMPTY_KEY, KTJ_SYNC_CAP + 1ull, st);
+  if (e != hipSuccess) return e;
+  e = fill_u32(first_pos, 0xFFFFFFFFu, KTJ_SYNC_CAP + 1ull, st);
+  if (e != hipSuccess) return e;
+  e = fill_u32(is_first, 0u, n_generic, st);
+  if (e != hipSuccess) return e;
+  const dim3 grid(grid_for(n_sorted, KTJ_BLOCK)), b(KTJ_BLOCK);
+  hipLaunchKernelGGL(k_sync_first_a, grid, b, 0, st, perm, n_sorted, g, n_generic, d, keys, first_pos, sc);
+  hipLaunchKernelGGL(k_sync_first_b, grid, b, 0, st, perm, n_sorted, g, n_generic, d, (const uint64_t*)keys,
+                     (const uint32_t*)first_pos, is_first);
+  return KTJ_LAUNCH_CHECK();
+}
+
+__global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, const uint32_t* sync_first, MatRow* mat,
+                              uint32_t* len, Scalars* sc) {
   RowStats rs;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    const MatRow m = mat_generic(g[i]);
+    MatRow m = mat_generic(g[i]);
+    mark_stream_sync(m, ctx, sync_first != nullptr && sync_first[i] != 0);
     store_row(&mat[i], m);
     len[i] = row_length(m, ctx, sc);
     count_row_stats(m, ctx, &rs);
@@ -1268,10 +1324,11 @@ __global__ void k_gather_len(const uint32_t* perm, const uint32_t* len, uint64_t
   if (i < n) len_sorted[i] = len[perm[i]] & 0x3FFFFFFFu;
 }
 
-hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc,
-                            hipStream_t st) {
+hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, const uint32_t* sync_first, MatRow* mat,
+                            uint32_t* len, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_mat_generic, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, ctx, mat, len, sc);
+  hipLaunchKernelGGL(k_mat_generic, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, ctx, sync_first, mat,
+                     len, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullTable tf,

@@ -54,6 +54,8 @@ struct MatRow {
 #define KTJ_M_MALLOC_BYTES (1u << 16)
 #define KTJ_M_NAME_BUILTIN (1u << 17)
 #define KTJ_M_HAS_STREAM (1u << 18) /* meta column of runtime rows only: the row carries a stream */
+#define KTJ_M_SYNC (1u << 19)       /* CUDA_SYNC activity named "Stream Sync": own row at tid + 1000000 */
+#define KTJ_M_SYNC_FIRST (1u << 20) /* first such activity of its (device, row) in emission order  */
 
 #define KTJ_CLASS_GENERIC 0u
 #define KTJ_CLASS_RUNTIME 1u
@@ -71,11 +73,16 @@ struct DictViews {
   const uint64_t* name_off;  /* n + 1                                                          */
   const char* arg_blob;      /* strings after sanitizeStrForJSON                               */
   const uint64_t* arg_off;   /* n + 1                                                          */
+  const char* raw_blob;      /* strings as interned (instant events print them untouched)      */
+  const uint64_t* raw_off;   /* n + 1                                                          */
   const uint32_t* flags;     /* KTJ_SF_*                                                       */
   uint32_t n;
 };
 #define KTJ_SF_ARG_BLANK 1u  /* arg view is empty or whitespace only                           */
 #define KTJ_SF_NAME_UNKNOWN 2u /* name view was replaced by "unknown"                          */
+#define KTJ_SF_NAME_KERNEL 4u  /* the string is "kernel" (printed as "Kernel")                  */
+#define KTJ_SF_STREAM_SYNC 8u  /* the string is "Stream Sync"                                    */
+#define KTJ_SYNC_TID_OFFSET 1000000 /* libkineto/src/output_json.h: kSyncStreamTidOffset          */
 
 /* everything format_activity needs besides the row itself */
 struct EmitCtx {

@@ -132,11 +132,10 @@ void GpuChromeTraceLogger::handleActivity(const ITraceActivity& op) {
   const ITraceActivity* linked = op.linkedActivity();
   const int64_t device = op.deviceId();
   const int64_t flowId = op.flowId();
-  /* kinds ChromeTraceLogger::handleActivity renders through other templates
-   * (output_json.cpp:842-856, 899-943) and values the packed record cannot hold */
-  bool unsupported = type == ActivityType::CPU_INSTANT_EVENT || type == ActivityType::HARDWARE_COUNTERS ||
-      type == ActivityType::MTIA_COUNTERS || type == ActivityType::XPU_SCOPE_PROFILER ||
-      (type == ActivityType::CUDA_SYNC && name == "Stream Sync");
+  /* counter events (output_json.cpp:847-856, 679-716) need counterValues(), collective metadata
+   * (:899-908) the linked op's own metadata: neither fits the packed record */
+  bool unsupported = type == ActivityType::HARDWARE_COUNTERS || type == ActivityType::MTIA_COUNTERS ||
+      type == ActivityType::XPU_SCOPE_PROFILER;
   if (linked != nullptr && linked->name() == kParamCommsName) {
     unsupported = unsupported || type == ActivityType::CONCURRENT_KERNEL ||
         (type == ActivityType::MTIA_CCP_EVENTS && name.rfind("hccl::", 0) == 0);

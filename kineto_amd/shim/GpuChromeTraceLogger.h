@@ -52,8 +52,8 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
                      int64_t endTime) override;
 
   std::string traceFileName() const { return fileName_; }
-  /* activities of kinds the engine does not render (instant and counter events, Stream Sync
-   * rows, collective metadata of record_param_comms): they are dropped and counted here */
+  /* activities of kinds the engine does not render (counter events, collective metadata of
+   * record_param_comms): they are dropped and counted here */
   uint64_t unsupportedActivities() const { return unsupported_; }
   /* ktj status of the first failed engine call, 0 if none */
   int engineStatus() const { return status_; }

@@ -24,6 +24,9 @@
  *       The reference's own join code (RocmActivityProfiler / RocprofActivityApi) needs a live
  *       rocprofiler-sdk context and is not part of oracle/_ref.
  *   - canonical order: stable merge sort here; std::stable_sort on tuples inside oracle/_ref.
+ *   - instant events and the Stream Sync row remap: byte-compared with the real logger on a
+ *       hand-made case (tests/kat_cases.py: case_instant_and_stream_sync).
+ * Not restated: counter events (output_json.cpp:679-716) and collective metadata (:718-835, 899-908).
  */
 #define _GNU_SOURCE
 #include "ktj_oracle.h"
@@ -318,6 +321,9 @@ struct ktj_oracle {
   /* output */
   sbuf out;
   uint64_t out_of_range, out_of_order, n_flow, n_linked, n_blank;
+  /* (device << 32 | virtual tid) keys whose Stream-Sync row header was written: output_json.h
+   * syncStreamMetadataEmitted_ */
+  int64_t* sync_seen; uint64_t n_sync_seen, cap_sync_seen;
   double t_join, t_sort, t_emit;
   int64_t win_start, win_end;
 };
@@ -1013,10 +1019,36 @@ static int is_whitespace(const char* p, size_t n) { /* output_json.cpp:128-131 *
   return 1;
 }
 
-/* handleActivity (complete events only) + handleGenericLink + handleLink:
- * output_json.cpp:837-1021.  Instant/counter event kinds and the Stream-Sync row remap are not
- * part of the accelerated path and are not restated here. */
+#define SYNC_STREAM_TID_OFFSET 1000000 /* output_json.h: kSyncStreamTidOffset */
+static int is_stream_sync(const ktj_oracle* o, const ktj_mat_activity* a) { /* :915, :1011 */
+  if (a->type != KTJ_TYPE_CUDA_SYNC) return 0;
+  const char* nm; uint64_t nl;
+  ktj_oracle_string(o, a->name_id, &nm, &nl);
+  return nl == 11 && memcmp(nm, "Stream Sync", 11) == 0;
+}
+/* handleGenericInstantEvent: output_json.cpp:660-677.  Name and metadata are printed as they are. */
+static void handle_instant_event(ktj_oracle* o, const ktj_mat_activity* a) {
+  sbuf args = {0}, meta = {0};
+  render_metadata(o, a, &meta);
+  if (meta.n && !is_whitespace(meta.p, meta.n)) sb_put(&args, meta.p, meta.n);
+  const char* nm; uint64_t nl;
+  ktj_oracle_string(o, a->name_id, &nm, &nl);
+  char* name = (char*)malloc(nl + 1);
+  if (!name) abort();
+  memcpy(name, nm, nl);
+  name[nl] = 0;
+  char pid[24], tid[24];
+  fmt_i64(a->device, pid);
+  fmt_i64(sanitize_tid(a->resource), tid);
+  write_instant_event(o, ktj_oracle_type_name(a->type), "t", name, pid, tid, rel_time(o, a->ts), &args, 0);
+  free(name); free(args.p); free(meta.p);
+}
+
+/* handleActivity + handleGenericLink + handleLink: output_json.cpp:837-1021.  Counter event kinds
+ * (handleCounterEvent, :679-716) and the collective metadata of record_param_comms (:899-908) are
+ * not restated here. */
 static void handle_activity(ktj_oracle* o, const ktj_mat_activity* a) {
+  if (a->type == KTJ_TYPE_CPU_INSTANT_EVENT) { handle_instant_event(o, a); return; } /* :842-845 */
   int64_t ts = a->ts;
   int64_t duration = a->dur < 0 ? 0 : a->dur;              /* :860 */
   if (a->type == KTJ_TYPE_GPU_USER_ANNOTATION) { ts -= 1; duration += 2; } /* :862-869 */
@@ -1053,14 +1085,45 @@ static void handle_activity(ktj_oracle* o, const ktj_mat_activity* a) {
     o->n_blank++;
   char pid[24], tid[24];
   fmt_i64(a->device, pid);
-  fmt_i64(sanitize_tid(a->resource), tid);
+  int64_t resource = a->resource;
+  const int sync = is_stream_sync(o, a);
+  if (sync) { /* :913-943: own row per stream, announced once per (device, row) */
+    const int64_t sync_tid = resource + SYNC_STREAM_TID_OFFSET;
+    const int64_t key = (int64_t)(((uint64_t)a->device << 32) | (uint64_t)sync_tid);
+    int seen = 0;
+    for (uint64_t k = 0; k < o->n_sync_seen && !seen; ++k) seen = o->sync_seen[k] == key;
+    if (!seen) {
+      if (o->n_sync_seen == o->cap_sync_seen) {
+        o->cap_sync_seen = o->cap_sync_seen ? o->cap_sync_seen * 2 : 64;
+        o->sync_seen = (int64_t*)realloc(o->sync_seen, o->cap_sync_seen * 8);
+        if (!o->sync_seen) abort();
+      }
+      o->sync_seen[o->n_sync_seen++] = key;
+      char t[40], st[24], rs[24];
+      ktj_oracle_fmt_ts(rel_time(o, ts), t);
+      fmt_i64(sync_tid, st);
+      fmt_i64(resource, rs);
+      sbuf* b = &o->out;
+      sb_puts(b, "\n  {\n    \"name\": \"thread_name\", \"ph\": \"M\", \"ts\": "); sb_puts(b, t);
+      sb_puts(b, ", \"pid\": "); sb_puts(b, pid); sb_puts(b, ", \"tid\": "); sb_puts(b, st);
+      sb_puts(b, ",\n    \"args\": {\n      \"name\": \"stream "); sb_puts(b, rs);
+      sb_puts(b, " (sync)\"\n    }\n  },");
+      sb_puts(b, "\n  {\n    \"name\": \"thread_sort_index\", \"ph\": \"M\", \"ts\": "); sb_puts(b, t);
+      sb_puts(b, ", \"pid\": "); sb_puts(b, pid); sb_puts(b, ", \"tid\": "); sb_puts(b, st);
+      sb_puts(b, ",\n    \"args\": {\n      \"sort_index\": "); sb_puts(b, rs);
+      sb_puts(b, "\n    }\n  },");
+    }
+    resource = sync_tid;
+  }
+  fmt_i64(sanitize_tid(resource), tid);
   write_complete_event(o, ktj_oracle_type_name(a->type), name, name_n, pid, tid, rel_time(o, ts),
                        duration, &args);
   if (a->flow_id > 0) {                                     /* :960-962, 973-995 */
     const char* fname = a->flow_type == (int)KTJ_LINK_FWDBWD ? "fwdbwd"
                       : a->flow_type == (int)KTJ_LINK_ASYNC_CPU_GPU ? "ac2g" : NULL;
     if (fname) {
-      write_flow_event(o, a->flow_start ? 's' : 'f', a->flow_id, a->device, sanitize_tid(a->resource),
+      write_flow_event(o, a->flow_start ? 's' : 'f', a->flow_id, a->device,
+                       sanitize_tid(sync ? a->resource + SYNC_STREAM_TID_OFFSET : a->resource),
                        rel_time(o, a->ts), fname);          /* handleLink :997-1021 */
       o->n_flow++;
     }
@@ -1119,7 +1182,7 @@ ktj_oracle* ktj_oracle_run(const ktj_stream* s) {
 void ktj_oracle_free(ktj_oracle* o) {
   if (!o) return;
   free(o->xblob.p); free(o->xoff); free(o->acts); free(o->order); free(o->fpool); free(o->spool);
-  free(o->act_f0); free(o->act_s0); free(o->out.p);
+  free(o->act_f0); free(o->act_s0); free(o->out.p); free(o->sync_seen);
   free(o);
 }
 void ktj_oracle_output(const ktj_oracle* o, const char** bytes, uint64_t* n) { *bytes = o->out.p; *n = o->out.n; }

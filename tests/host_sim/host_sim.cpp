@@ -9,6 +9,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <set>
 #include <string>
 #include <unordered_map>
 #include <unordered_set>
@@ -22,7 +23,7 @@ using namespace ktj;
 namespace {
 
 struct Views {
-  std::string name_blob, arg_blob;
+  std::string name_blob, arg_blob, raw_blob;
   std::vector<uint64_t> name_off, arg_off;
   std::vector<uint32_t> flags;
 };
@@ -50,6 +51,7 @@ void build_views(const ktj_stream* s, Views& v) {
     if (n == 6 && memcmp(p, "kernel", 6) == 0) name = "Kernel";
     else if (unknown) { name = "unknown"; fl |= KTJ_SF_NAME_UNKNOWN; }
     if (blank) fl |= KTJ_SF_ARG_BLANK;
+    if (n == 11 && memcmp(p, "Stream Sync", 11) == 0) fl |= KTJ_SF_STREAM_SYNC;
     v.name_blob += name; v.name_off.push_back(v.name_blob.size());
     v.arg_blob += arg; v.arg_off.push_back(v.arg_blob.size());
     v.flags.push_back(fl);
@@ -67,6 +69,9 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   EmitCtx ctx;
   ctx.dict.name_blob = v.name_blob.data(); ctx.dict.name_off = v.name_off.data();
   ctx.dict.arg_blob = v.arg_blob.data(); ctx.dict.arg_off = v.arg_off.data();
+  v.raw_blob.assign(s->str_blob ? s->str_blob : "", s->n_strings ? s->str_off[s->n_strings] : 0);
+  v.raw_blob.append(16, '\0'); /* string copies load whole aligned words */
+  ctx.dict.raw_blob = v.raw_blob.data(); ctx.dict.raw_off = s->str_off;
   ctx.dict.flags = v.flags.data(); ctx.dict.n = (uint32_t)s->n_strings;
   ctx.fields = s->fields; ctx.schemas = s->schemas; ctx.n_schemas = (uint32_t)s->n_schemas;
   ctx.args = s->args; ctx.n_args = s->n_args; ctx.base_time_ns = s->base_time_ns;
@@ -202,6 +207,18 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
     if (a.res != b.res) return a.res < b.res;
     return a.ts < b.ts;
   });
+  {
+    // Stream Sync rows: the first activity of each (device, row) key in emission order announces the row
+    std::set<uint64_t> announced;
+    for (uint64_t a : perm) {
+      if (a >= ng) continue;
+      MatRow probe = mat[a];
+      mark_stream_sync(probe, ctx, false);
+      if (!(probe.meta & KTJ_M_SYNC)) continue;
+      const bool first = announced.insert(stream_sync_key(mat[a].dev, mat[a].res)).second;
+      mark_stream_sync(mat[a], ctx, first);
+    }
+  }
   std::vector<uint64_t> offs(perm.size() + 1, 0);
   for (size_t i = 0; i < perm.size(); ++i) {
     CountWriter cw;

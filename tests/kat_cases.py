@@ -140,7 +140,35 @@ def case_rocm_sync_trace():
     return b, expect_counts
 
 
-SUBSTRING_CASES = [case_logger_events, case_trace_span, case_benchmark_cpu_op, case_typed_kernel_args,
+def case_instant_and_stream_sync():
+    """Instant events (handleGenericInstantEvent, output_json.cpp:660-677: name and metadata printed
+    as they are) and Stream Sync rows (output_json.cpp:913-943, 1008-1013: own row at tid + 1000000,
+    announced once per (device, row), flow events on the same row).  Expected strings follow the
+    reference's templates; the whole document is compared with the real logger where it is built."""
+    CPU_INSTANT_EVENT, CUDA_SYNC = 9, 15
+    b = StreamBuilder()
+    frag = b.schema([(None, abi.F_RAW, 1)])
+    b.add_generic('mark "a"\\b', CPU_INSTANT_EVENT, B + 100, B + 100, 7, 8, id=3, schema=frag,
+                  values=[b.s('"note": "x\\y"')])
+    b.add_generic("plain mark", CPU_INSTANT_EVENT, B + 150, B + 150, 7, 8)
+    b.add_generic("Stream Sync", CUDA_SYNC, B + 2000, B + 2500, 0, 5, id=11, flow_id=11, flow_type=2)
+    b.add_generic("Stream Sync", CUDA_SYNC, B + 1000, B + 1200, 0, 5, id=12)        # earlier in time: this one announces the row
+    b.add_generic("Stream Sync", CUDA_SYNC, B + 3000, B + 3100, 1, 5, id=13)        # other device: own announcement
+    b.add_generic("Event Sync", CUDA_SYNC, B + 4000, B + 4100, 0, 5, id=14)         # other name: stays on the stream's row
+    b.add_generic("Stream Sync", KERNEL, B + 5000, B + 5100, 0, 5, id=15)           # other type: stays too
+    expect = [
+        '"ph": "i",\n    \n    "cat": "cpu_instant_event",\n    "s": "t",\n    "name": "mark "a"\\b",\n    "pid": 7,\n    "tid": 8,\n    "ts": 0.100\n    ,\n    "args": {\n      "note": "x\\y"\n    }\n  },',
+        '"name": "plain mark",\n    "pid": 7,\n    "tid": 8,\n    "ts": 0.150\n    \n  },',
+        '"name": "thread_name", "ph": "M", "ts": 1.000, "pid": 0, "tid": 1000005,\n    "args": {\n      "name": "stream 5 (sync)"\n    }\n  },\n  {\n    "name": "thread_sort_index", "ph": "M", "ts": 1.000, "pid": 0, "tid": 1000005,\n    "args": {\n      "sort_index": 5\n    }\n  },\n  {\n    "ph": "X",\n    "cat": "cuda_sync",\n    "name": "Stream Sync",\n    "pid": 0,\n    "tid": 1000005,\n    "ts": 1.000,',
+        '"ph": "f",\n    "id": 11,\n    "pid": 0,\n    "tid": 1000005,\n    "ts": 2.000,',
+        '"ts": 3.000, "pid": 1, "tid": 1000005,',
+        '"name": "Event Sync",\n    "pid": 0,\n    "tid": 5,',
+        '"cat": "kernel",\n    "name": "Stream Sync",\n    "pid": 0,\n    "tid": 5,',
+    ]
+    return b, expect
+
+
+SUBSTRING_CASES = [case_instant_and_stream_sync, case_logger_events, case_trace_span, case_benchmark_cpu_op, case_typed_kernel_args,
                    case_typed_metadata_pins, case_names, case_resource_infos]
 
 
