@@ -585,7 +585,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
       HIPCHK(emit(mat, e->perm, e->offs.as<uint64_t>(), N, ctx, e->out.as<char>(), e->prefix_len, act_bytes, tile,
                   e->tile_start.as<uint32_t>(), st));
     else
-      HIPCHK(emit_direct(mat, e->perm, e->offs.as<uint64_t>(), e->len.as<uint32_t>(), e->scalars.n_valid, ctx,
+      HIPCHK(emit_direct(mat, e->perm, e->offs.as<uint64_t>(), e->len.as<uint32_t>(), e->scalars.n_valid, act_bytes, ctx,
                          e->out.as<char>(), e->prefix_len, st));
   }
   HIPCHK(hipEventRecord(e->ev[EV_EMIT], st));

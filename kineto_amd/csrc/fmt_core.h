@@ -395,6 +395,38 @@ struct TileWriter {
  * eight bytes at a time, through a funnel shift over aligned loads (dictionary blobs are padded
  * by 16 bytes so that the last load stays inside the allocation). */
 
+/* Long dictionary strings (templated C++ kernel names run to kilobytes) are not copied by the lane
+ * that owns the activity but by all lanes that are active with it: for one owner at a time,
+ * neighbouring lanes move neighbouring 8-byte words, so loads and stores are whole lines.  The
+ * owner has already brought its output to a word boundary; `src` is the first byte that lands on
+ * that boundary (any alignment: two aligned loads are funnel-shifted), `dst` the word, `n_words`
+ * the whole words (0 for lanes that only help).  Works under any set of active lanes. */
+#define KTJ_COOP_MIN_BYTES 256u
+#if defined(__HIP_DEVICE_COMPILE__)
+static __device__ __attribute__((noinline)) void cooperative_word_copy(const char* src, uint64_t* dst, uint32_t n_words) {
+  const uint64_t active = __ballot(1);
+  const uint32_t lane = (uint32_t)(threadIdx.x & 63u);
+  const uint32_t n_active = (uint32_t)__popcll(active);
+  const uint32_t rank = (uint32_t)__popcll(active & ((1ULL << lane) - 1ULL));
+  uint64_t todo = __ballot(n_words != 0);
+  while (todo) {
+    const int owner = __ffsll((unsigned long long)todo) - 1;
+    todo &= todo - 1;
+    const uint32_t n = (uint32_t)__shfl((int)n_words, owner);
+    const uintptr_t sa = (uintptr_t)__shfl((unsigned long long)(uintptr_t)src, owner);
+    uint64_t* d = reinterpret_cast<uint64_t*>((uintptr_t)__shfl((unsigned long long)(uintptr_t)dst, owner));
+    const uint32_t sh = (uint32_t)(sa & 7u) * 8u;
+    const uint64_t* sp = reinterpret_cast<const uint64_t*>(sa & ~(uintptr_t)7);
+    KTJ_NOUNROLL
+    for (uint32_t k = rank; k < n; k += n_active) {
+      uint64_t v = sp[k];
+      if (sh) v = (v >> sh) | (sp[k + 1] << (64u - sh));
+      d[k] = v;
+    }
+  }
+}
+#endif
+
 /* every finished word is stored at once by the lane that gathered it */
 struct DirectSink {
   uint64_t* wptr;     /* aligned address of the word being gathered */
@@ -402,6 +434,8 @@ struct DirectSink {
   KTJ_HD KTJ_FI void put(uint64_t w) { *wptr++ = w; }
   KTJ_HD KTJ_FI void close() {}
   KTJ_HD KTJ_FI uint64_t* next_word() const { return wptr; }
+  /* hands out `n` whole words that somebody else fills */
+  KTJ_HD KTJ_FI uint64_t* reserve(uint32_t n) { uint64_t* p = wptr; wptr += n; return p; }
 };
 
 template <class Sink>
@@ -464,7 +498,7 @@ struct WordWriter {
     if (__builtin_expect(n.len != 0, 1)) append(n.word, n.len); else dec_wide(n.value);
   }
   KTJ_HD KTJ_FI void dec3(uint32_t x) { append((uint64_t)(ascii4(x) >> 8), 3); }
-  KTJ_HD KTJ_FI void str(const char* src, uint64_t len) {
+  KTJ_HD KTJ_FI void str_own(const char* src, uint64_t len) {
     if (len == 0) return;
     const uintptr_t sa = (uintptr_t)src;
     const uint32_t sh = (uint32_t)(sa & 7u) * 8u;
@@ -483,6 +517,29 @@ struct WordWriter {
       if (sh && rem * 8u > 64u - sh) v |= sp[full + 1] << (64u - sh);
       append(v & ((1ULL << (8 * rem)) - 1ULL), rem);
     }
+  }
+  KTJ_HD KTJ_FI void str(const char* src, uint64_t len) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const bool big = len >= KTJ_COOP_MIN_BYTES;
+    if (__any(big)) { /* see cooperative_word_copy */
+      const char* body = src;
+      uint64_t* dst = nullptr;
+      uint32_t n_words = 0;
+      uint64_t tail = 0;
+      if (big) {
+        const uint32_t head = (8u - fill) & 7u;     /* bytes that complete the word being gathered */
+        str_own(src, head);                          /* now fill == 0 and acc == 0 */
+        body = src + head;
+        n_words = (uint32_t)((len - head) >> 3);
+        tail = (len - head) & 7u;
+        dst = sink.reserve(n_words);
+      } else str_own(src, len);
+      cooperative_word_copy(body, dst, n_words);
+      if (big) str_own(body + (uint64_t)n_words * 8u, tail);
+      return;
+    }
+#endif
+    str_own(src, len);
   }
 };
 typedef WordWriter<DirectSink> GlobalWriter;

@@ -241,7 +241,7 @@ hipError_t emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs /*
 /* direct variant: one lane per activity, no LDS staging; len_kind is the arrival-order length
  * array whose top two bits carry the tail kind; n_rows = number of activities that are written */
 hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint32_t* len_kind,
-                       uint64_t n_rows, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st);
+                       uint64_t n_rows, uint64_t act_bytes, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st);
 
 }  // namespace gpu
 }  // namespace ktj

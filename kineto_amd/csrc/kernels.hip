@@ -1487,14 +1487,16 @@ k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, con
   }
 }
 hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint32_t* len_kind,
-                       uint64_t n_rows, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st) {
+                       uint64_t n_rows, uint64_t act_bytes, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st) {
   if (n_rows == 0) return hipSuccess;
   /* Every lane keeps one partially written 128-byte line open at a time.  At full occupancy
    * (2048 lanes per CU, 256 CUs) those lines exceed the L2 capacity and are evicted half-filled,
    * which doubles the HBM writes.  Unused dynamic LDS caps residency at two workgroups per CU
-   * (8 waves), so the open lines stay in L2 until complete; measured 15-20% faster on every
-   * configuration than unrestricted residency. */
-  const size_t residency_lds = 60000;
+   * (8 waves), so the open lines stay in L2 until complete; measured 15-20% faster than
+   * unrestricted residency where activities are short.  Where most bytes are long dictionary
+   * strings, which the lanes copy together as whole lines, the cap only costs parallelism
+   * (measured 13% slower at 1.4 KB per activity), so it is applied below 768 bytes per activity. */
+  const size_t residency_lds = act_bytes / n_rows < 768 ? 60000 : 0;
   hipLaunchKernelGGL(k_emit_direct, dim3(grid_for(n_rows, KTJ_BLOCK)), dim3(KTJ_BLOCK), residency_lds, st, mat, perm, offs,
                      len_kind, n_rows, ctx, out, prefix_len);
   return KTJ_LAUNCH_CHECK();
