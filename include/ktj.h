@@ -98,12 +98,15 @@ typedef struct ktj_generic_rec {
   int64_t start_ns;      /* startTime (absolute ns)                                            */
   int64_t end_ns;        /* endTime; duration() = end_ns - start_ns                            */
   int64_t resource;      /* resourceId(): thread id or stream id                               */
-  int64_t linked_corr;   /* linkedActivity()->correlationId(); read only if KTJ_GF_LINKED      */
+  int64_t flow_id;       /* flowId(): flow.id of a GenericTraceActivity, the correlation id of
+                            runtime / device wrappers; a flow event follows when it is > 0     */
   uint64_t args_off;     /* first 8-byte slot of this record's values in the args blob         */
-  int32_t id;            /* correlationId() — GenericTraceActivity::id is int32                */
+  int32_t id;            /* correlationId() as the logger reads it: `int external_id`
+                            (output_json.cpp:871-893); GenericTraceActivity::id is int32       */
   int32_t device;        /* deviceId() — process id for CPU ops                                */
   uint32_t name_id;      /* string id of name()                                                */
-  uint32_t flow_id;      /* flow.id (uint32)                                                   */
+  int32_t linked_id;     /* linkedActivity()->correlationId(), int-truncated like the logger's
+                            `int external_id`; read only if KTJ_GF_LINKED                      */
   uint32_t schema_id;    /* args schema, KTJ_NONE = no metadata                                */
   uint8_t type;          /* KTJ_TYPE_*                                                         */
   uint8_t flow_type;     /* flow.type (4 bits)                                                 */

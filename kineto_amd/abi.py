@@ -24,9 +24,9 @@ STAGE_NAMES = ["dict", "decode", "convert", "join", "sort", "size", "scan", "emi
 
 class GenericRec(C.Structure):
     _fields_ = [("start_ns", C.c_int64), ("end_ns", C.c_int64), ("resource", C.c_int64),
-                ("linked_corr", C.c_int64), ("args_off", C.c_uint64), ("id", C.c_int32),
+                ("flow_id", C.c_int64), ("args_off", C.c_uint64), ("id", C.c_int32),
                 ("device", C.c_int32), ("name_id", C.c_uint32),
-                ("flow_id", C.c_uint32), ("schema_id", C.c_uint32), ("type", C.c_uint8),
+                ("linked_id", C.c_int32), ("schema_id", C.c_uint32), ("type", C.c_uint8),
                 ("flow_type", C.c_uint8), ("flags", C.c_uint8), ("pad0", C.c_uint8)]
 
 

@@ -514,21 +514,37 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
     e->last_error = "device-side limit hit before sort, error bits " + std::to_string(e->scalars.error);
     return KTJ_ERR_LIMIT;
   }
-  uint32_t ts_bits = 0, res_bits = 0, key_bits = 0;
+  uint32_t ts_bits = 0, res_bits = 0, key_bits = 0, rank_bits = 0;
   if (e->scalars.n_valid) {
     ts_bits = (uint32_t)bits_for(e->scalars.ts_max_biased - e->scalars.ts_min_biased);
     res_bits = (uint32_t)bits_for(e->scalars.n_res_ranks ? e->scalars.n_res_ranks - 1 : 0);
     const uint32_t dev_bits = (uint32_t)bits_for(e->scalars.n_dev_ranks ? e->scalars.n_dev_ranks - 1 : 0);
     key_bits = ts_bits + res_bits + dev_bits;
-    if (key_bits > 62) {
-      e->last_error = "sort key needs " + std::to_string(key_bits) + " bits (timestamp span too wide)";
-      return KTJ_ERR_LIMIT;
-    }
+    rank_bits = res_bits + dev_bits;
   }
   HIPCHK(hipEventRecord(e->ev[EV_SORT_B], st));
-  HIPCHK(make_keys(c, N, sets, sc, ts_bits, res_bits, key_bits, e->keys_a.as<uint64_t>(), e->vals_a.as<uint32_t>(), st));
-  HIPCHK(radix_sort(e->keys_a.as<uint64_t>(), e->vals_a.as<uint32_t>(), e->keys_b.as<uint64_t>(), e->vals_b.as<uint32_t>(),
-                    N, key_bits + 1, e->hist.as<uint32_t>(), e->scan_tmp.as<uint64_t>(), &e->sorted_keys, &e->perm, st));
+  if (key_bits <= 62) {
+    HIPCHK(make_keys(c, N, sets, sc, ts_bits, res_bits, key_bits, e->keys_a.as<uint64_t>(), e->vals_a.as<uint32_t>(), st));
+    HIPCHK(radix_sort(e->keys_a.as<uint64_t>(), e->vals_a.as<uint32_t>(), e->keys_b.as<uint64_t>(), e->vals_b.as<uint32_t>(),
+                      N, key_bits + 1, e->hist.as<uint32_t>(), e->scan_tmp.as<uint64_t>(), &e->sorted_keys, &e->perm, st));
+  } else {
+    /* timestamp span too wide for one composite key: stable sort by timestamp, then by ranks */
+    if (rank_bits > 62) {
+      e->last_error = "sort key needs " + std::to_string(rank_bits) + " bits for device and resource ranks";
+      return KTJ_ERR_LIMIT;
+    }
+    uint64_t* ka = e->keys_a.as<uint64_t>(); uint32_t* va = e->vals_a.as<uint32_t>();
+    uint64_t* kb = e->keys_b.as<uint64_t>(); uint32_t* vb = e->vals_b.as<uint32_t>();
+    HIPCHK(make_ts_keys(c, N, sc, ka, va, st));
+    HIPCHK(radix_sort(ka, va, kb, vb, N, ts_bits, e->hist.as<uint32_t>(), e->scan_tmp.as<uint64_t>(), &e->sorted_keys, &e->perm, st));
+    if (e->perm == va) { /* result in the first pair: rank keys go into the second */
+      HIPCHK(make_rank_keys(c, va, N, sets, res_bits, rank_bits, kb, vb, st));
+      HIPCHK(radix_sort(kb, vb, ka, va, N, rank_bits + 1, e->hist.as<uint32_t>(), e->scan_tmp.as<uint64_t>(), &e->sorted_keys, &e->perm, st));
+    } else {
+      HIPCHK(make_rank_keys(c, vb, N, sets, res_bits, rank_bits, ka, va, st));
+      HIPCHK(radix_sort(ka, va, kb, vb, N, rank_bits + 1, e->hist.as<uint32_t>(), e->scan_tmp.as<uint64_t>(), &e->sorted_keys, &e->perm, st));
+    }
+  }
   HIPCHK(hipEventRecord(e->ev[EV_SORT], st));
 
   /* ---- stage 4a: joined rows + lengths ---- */

@@ -204,6 +204,12 @@ hipError_t rank_distinct(SortSets s, Scalars* sc, hipStream_t st);
 /* key = ((rank(dev) << res_bits | rank(res)) << ts_bits) | (ts - ts_min); dropped rows get 1 << key_bits */
 hipError_t make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits,
                      uint32_t key_bits, uint64_t* keys, uint32_t* vals, hipStream_t st);
+/* for timestamp spans too wide for one composite key: keys = ts - ts_min with vals = arrival
+ * index, then keys = composite rank of row order[p] with vals = order[p] (dropped rows get
+ * 1 << rank_bits) */
+hipError_t make_ts_keys(Columns c, uint64_t n, const Scalars* sc, uint64_t* keys, uint32_t* vals, hipStream_t st);
+hipError_t make_rank_keys(Columns c, const uint32_t* order, uint64_t n, SortSets s, uint32_t res_bits, uint32_t rank_bits,
+                          uint64_t* keys, uint32_t* vals, hipStream_t st);
 /* stable LSD radix sort of (key, val) pairs on the low `bits` bits; result ends in keys_out/vals_out
  * pointers returned through *res_keys / *res_vals (one of the two buffer pairs) */
 uint64_t radix_tmp_elems(uint64_t n);

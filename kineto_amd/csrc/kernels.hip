@@ -1028,6 +1028,44 @@ __global__ void k_make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc
   vals[a] = (uint32_t)a;
 }
 
+/* Wide timestamp spans (a row at time 0 next to rows at wall-clock time) do not fit one 64-bit
+ * composite key.  The order is then built in two stable sorts: by timestamp, then by the
+ * (device, resource) ranks of the rows in that order. */
+__global__ void k_make_ts_keys(Columns c, uint64_t n, const Scalars* sc, uint64_t* keys, uint32_t* vals) {
+  const uint64_t a = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (a >= n) return;
+  keys[a] = (c.meta[a] & KTJ_M_VALID) ? (((uint64_t)c.ts[a] ^ 0x8000000000000000ULL) - sc->ts_min_biased) : 0;
+  vals[a] = (uint32_t)a;
+}
+__global__ void k_make_rank_keys(Columns c, const uint32_t* order, uint64_t n, SortSets s, uint32_t res_bits,
+                                 uint32_t rank_bits, uint64_t* keys, uint32_t* vals) {
+  const uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n) return;
+  const uint32_t a = order[p];
+  uint64_t key = 1ULL << rank_bits; /* dropped rows sort behind everything */
+  if (c.meta[a] & KTJ_M_VALID) {
+    const uint32_t sd = table_find(s.dev_keys, KTJ_SET_CAP - 1u, (uint64_t)c.dev[a]);
+    const uint32_t sr = table_find(s.res_keys, KTJ_SET_CAP - 1u, (uint64_t)c.res[a]);
+    const uint64_t rd = sd != KTJ_NOSLOT ? s.dev_rank[sd] : 0;
+    const uint64_t rr = sr != KTJ_NOSLOT ? s.res_rank[sr] : 0;
+    key = (rd << res_bits) | rr;
+  }
+  keys[p] = key;
+  vals[p] = a;
+}
+hipError_t make_ts_keys(Columns c, uint64_t n, const Scalars* sc, uint64_t* keys, uint32_t* vals, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_make_ts_keys, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, n, sc, keys, vals);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t make_rank_keys(Columns c, const uint32_t* order, uint64_t n, SortSets s, uint32_t res_bits, uint32_t rank_bits,
+                          uint64_t* keys, uint32_t* vals, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_make_rank_keys, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, order, n, s, res_bits,
+                     rank_bits, keys, vals);
+  return KTJ_LAUNCH_CHECK();
+}
+
 hipError_t collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
   /* few, fat workgroups: each one pays for its own local set once */

@@ -70,7 +70,7 @@ KTJ_HD inline MatRow mat_generic(const ktj_generic_rec& g) {
   m.dur = g.end_ns - g.start_ns;
   m.dev = g.device;
   m.res = g.resource;
-  m.flow_id = (int64_t)g.flow_id;
+  m.flow_id = g.flow_id;
   uint32_t meta = (g.type & KTJ_M_TYPE_MASK) | (KTJ_CLASS_GENERIC << KTJ_M_CLASS_SHIFT) | KTJ_M_VALID;
   const bool instant = g.type == KTJ_TYPE_CPU_INSTANT_EVENT; /* output_json.cpp:842-845, 660-677: no flow, no External id */
   if (!instant && g.flow_id > 0 && (g.flow_type == KTJ_LINK_FWDBWD || g.flow_type == KTJ_LINK_ASYNC_CPU_GPU)) {
@@ -82,7 +82,7 @@ KTJ_HD inline MatRow mat_generic(const ktj_generic_rec& g) {
   else m.name_id = g.name_id;
   m.meta = meta;
   if (instant) m.ext = 0;
-  else if (g.flags & KTJ_GF_LINKED) m.ext = (int32_t)g.linked_corr;
+  else if (g.flags & KTJ_GF_LINKED) m.ext = g.linked_id;
   else m.ext = type_hides_own_external_id(g.type) ? 0 : g.id;
   m.aux = g.schema_id;
   m.p[0] = g.args_off; m.p[1] = 0; m.p[2] = 0; m.p[3] = 0; m.p[4] = 0;

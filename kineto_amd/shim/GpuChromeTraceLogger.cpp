@@ -140,9 +140,7 @@ void GpuChromeTraceLogger::handleActivity(const ITraceActivity& op) {
     unsupported = unsupported || type == ActivityType::CONCURRENT_KERNEL ||
         (type == ActivityType::MTIA_CCP_EVENTS && name.rfind("hccl::", 0) == 0);
   }
-  unsupported = unsupported || device < std::numeric_limits<int32_t>::min() ||
-      device > std::numeric_limits<int32_t>::max() || flowId > std::numeric_limits<uint32_t>::max() ||
-      static_cast<unsigned>(op.flowType()) > 15u;
+  unsupported = unsupported || device < std::numeric_limits<int32_t>::min() || device > std::numeric_limits<int32_t>::max();
   if (unsupported) {
     if (unsupported_++ == 0) {
       LOG(WARNING) << "GpuChromeTraceLogger: activity '" << name << "' of type " << toString(type)
@@ -159,12 +157,13 @@ void GpuChromeTraceLogger::handleActivity(const ITraceActivity& op) {
   r.id = static_cast<int32_t>(op.correlationId()); /* `int external_id = op.correlationId()`, :893 */
   r.type = static_cast<uint8_t>(type);
   r.name_id = intern(names_, name);
-  r.flow_id = flowId > 0 ? static_cast<uint32_t>(flowId) : 0u;
-  r.flow_type = static_cast<uint8_t>(op.flowType());
+  r.flow_id = flowId;
+  const int flowType = op.flowType(); /* anything but the two known kinds prints no flow event (:979-994) */
+  r.flow_type = (flowType == static_cast<int>(KTJ_LINK_FWDBWD) || flowType == static_cast<int>(KTJ_LINK_ASYNC_CPU_GPU)) ? static_cast<uint8_t>(flowType) : 0;
   r.flags = op.flowStart() ? KTJ_GF_FLOW_START : 0;
   if (linked != nullptr) {
     r.flags |= KTJ_GF_LINKED;
-    r.linked_corr = linked->correlationId();
+    r.linked_id = static_cast<int32_t>(linked->correlationId()); /* `int external_id = …`, :873 */
   }
   const std::string metadata = op.metadataJson();
   if (metadata.empty()) {

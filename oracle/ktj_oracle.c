@@ -483,7 +483,7 @@ static int stage_join(ktj_oracle* o) {
     a->flow_start = (r->flags & KTJ_GF_FLOW_START) ? 1 : 0;
     a->type = r->type;
     a->has_linked = (r->flags & KTJ_GF_LINKED) ? 1 : 0;
-    a->linked_corr = r->linked_corr;
+    a->linked_corr = r->linked_id;
     a->name_id = r->name_id == KTJ_NONE ? o->builtin0 + BS_EMPTY : r->name_id;
     a->arrival = i;
     if (r->schema_id != KTJ_NONE && r->schema_id < s->n_schemas) {

@@ -1,0 +1,121 @@
+"""Seeded random ktj_stream objects that mix every record class, type and edge value the engine
+accepts: used for differential tests (host build of the formatting core, and the GPU engine,
+against the oracle)."""
+import random
+import struct
+
+from kineto_amd import abi
+from stream_builder import B, StreamBuilder
+
+# every ActivityType except the counter kinds, which the engine does not render
+TYPES = [t for t in range(29) if t not in (17, 26, 28)]
+I64_MIN, I64_MAX = -(1 << 63), (1 << 63) - 1
+
+
+def _name(rng):
+    r = rng.random()
+    if r < 0.08:
+        return rng.choice(["kernel", "Stream Sync", "", "unknown", "Kernel", " ", "\n"])
+    alphabet = "abcXYZ019_:<>(), *&[]"
+    if r < 0.35:
+        alphabet += '"\\\n\t'
+    if r < 0.15:
+        alphabet += "\x01\x7f\xe9"
+    n = rng.choice([1, 3, 7, 8, 9, 15, 16, 17, 31, 40, 63, 64, 65, 120, 300, 700])
+    return "".join(rng.choice(alphabet) for _ in range(n))
+
+
+def _i64(rng):
+    return rng.choice([0, 1, -1, 7, 999, 1000, 1001, 99999999, 100000000, 10**16 - 1, 10**16, I64_MAX, I64_MIN,
+                       rng.randrange(-10**6, 10**6), rng.randrange(I64_MIN, I64_MAX)])
+
+
+def _f64(rng):
+    v = rng.choice([0.0, -0.0, 1.5, 2.5, 0.1, 1e-5, 1e-4, 123456.789, 1e15, 1e16, 1e22, 5e-324, 1.7976931348623157e308,
+                    float("inf"), float("-inf"), float("nan"), rng.random(), rng.uniform(-1e9, 1e9),
+                    struct.unpack("<d", struct.pack("<Q", rng.getrandbits(64)))[0]])
+    return v
+
+
+def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False):
+    rng = random.Random(seed)
+    lo, hi = B + 1000, B + 10**7
+    window = (lo, hi) if rng.random() < 0.7 else (B + 3 * 10**6, B + 6 * 10**6)
+    b = StreamBuilder(window=window, host_name="rnd", end_time=hi + 5)
+    if rng.random() < 0.5:
+        b.clock = abi.ClockModel(rng.randrange(0, 1000), rng.randrange(-500, 500), rng.choice([1.0, 1.000001, 0.999]), rng.randrange(-50, 50),
+                                 rng.choice([0, 1]), rng.choice([0, 1, 2]))
+    apis = ["hipLaunchKernel", "hipMemcpyAsync", "hipMalloc", "hipGraphLaunch", None, "hipFree", 'odd "api"\\name']
+    b.api(apis, flow_start=rng.sample(range(len(apis)), 4), malloc_cid=rng.choice([2, abi.KTJ_NONE]))
+    names = [_name(rng) for _ in range(12)]
+
+    def t():
+        return rng.choice([rng.randrange(lo - 500, hi + 500), rng.randrange(lo, hi), 0, lo, hi])
+
+    # schemas
+    schemas = [None, b.schema([(None, abi.F_RAW, 1)])]
+    for _ in range(4):
+        fields = []
+        for _k in range(rng.randrange(0, 6)):
+            typ = rng.randrange(7)
+            fields.append((_name(rng)[:12] or "k", typ, rng.randrange(1, 5) if typ == abi.F_I64_ARRAY else 1))
+        schemas.append((b.schema(fields), fields))
+    pids, tids = [0, 1, 7, -3, 4242], [0, 5, -5, 4243, I64_MIN, I64_MAX, 10**12]
+    ids = list(range(1, 30))
+    if wide_ids:
+        ids += [(1 << 32) + 3, (1 << 31) + 1, 0xFFFFFFFFFFFFFFFF, 0xFFFFFFFF00000001, 1 << 40]
+    for _ in range(n_generic):
+        sch = rng.choice(schemas)
+        values, sid = (), None
+        if isinstance(sch, int):
+            sid = sch
+            values = [b.s(rng.choice(['"k": 1', "   ", "", "\n", '"a": "b\\c"', _name(rng)]))]
+        elif sch is not None:
+            sid, fields = sch
+            values = []
+            for _key, typ, cnt in fields:
+                if typ == abi.F_F64:
+                    values.append(_f64(rng))
+                elif typ in (abi.F_STR, abi.F_RAW):
+                    values.append(b.s(_name(rng)))
+                elif typ == abi.F_BOOL:
+                    values.append(rng.randrange(3))
+                elif typ == abi.F_I64_ARRAY:
+                    values += [_i64(rng) for _ in range(cnt)]
+                else:
+                    values.append(_i64(rng))
+        s0 = t()
+        b.add_generic(rng.choice(names + [None]), rng.choice(TYPES + [0, 0, 0, 9, 15]), s0, s0 + rng.choice([0, 1, 999, 1000, -3, 10**5]),
+                      rng.choice(pids), rng.choice(tids), id=rng.choice([0, -2, 5, 6, 7, 8, 2**31 - 1, -(2**31)] + ids[:8]),
+                      schema=sid, values=values, flow_id=rng.choice([0, 0, 1, 77, 2**32 - 1, 2**40 + 3, -4]), flow_type=rng.choice([0, 1, 2, 3]),
+                      flow_start=rng.random() < 0.5, linked=rng.choice([None, None, 5, -9, 2**40 + 1]))
+    for _ in range(n_runtime):
+        kind = rng.randrange(4)
+        s0 = t()
+        kw = {}
+        if kind == 1:
+            kw = dict(grid=[rng.choice([0, 1, 7, 2**32 - 1]) for _ in range(3)], workgroup=[rng.choice([1, 64, 1024]) for _ in range(3)],
+                      lds=rng.choice([0, 65536, 2**40]), stream=rng.choice([0, 0x7000, 0x8000, 0x9000]),
+                      kernel_name=rng.choice([None, None, _name(rng)]))
+        elif kind == 2:
+            kw = dict(src=rng.getrandbits(48), dst=rng.choice([0, rng.getrandbits(64)]), size=rng.choice([0, 4096, 2**35]),
+                      stream=rng.choice([0, 0x7000, 0xA000]), copy_kind=rng.choice([0, 1, 2, 3, 4, 0xFFFFFFFF]))
+        elif kind == 3:
+            kw = dict(ptr=rng.getrandbits(47), size=rng.choice([0, 777, 2**33]))
+        b.add_runtime(rng.choice(ids), s0, s0 + rng.choice([0, 5, 5000, -7]), rng.choice([0, 1, 2, 3, 4, 5, 6, 9, 10**6]),
+                      rng.choice([10, 11]), rng.choice([20, 21, 22]), kind=kind, **kw)
+    for _ in range(n_device):
+        dom = rng.choice([0, 0, 0, 1, 1, 2, 7])
+        s0 = t()
+        b.add_device(rng.choice(ids + [100, 101, 0]), s0, s0 + rng.choice([0, 1, 2, 900, 10**5]), domain=dom,
+                     op=rng.choice([0, 1, 2, 3, 4, 9]), device=rng.choice([0, 0, 1, -1]), name=rng.choice(names + [None]),
+                     queue=rng.choice([0, 1, 2, 3, 2**63 + 5]), stream=rng.choice([0, 0, 0, 5, 0x7000]), nbytes=rng.choice([0, 1000, 2**40]))
+    for _ in range(rng.randrange(0, 40)):
+        b.add_extcorr(rng.choice(ids + [0xFFFFFFFFFFFFFFFF]), rng.choice([5, 6, 7, 8, 0, 2**31 - 1, 0xFFFFFFFF80000000, 2**40, 12345]))
+    if rng.random() < 0.5:
+        b.add_device_info(0, 5000000, 'GPU "zero"', "GPU 0", B + 10)
+        b.add_resource_info(5, 5, 0, 'stream "5"', False, B + 10)
+        b.add_resource_info(4243, 4243, 4242, "worker", True, B + 11)
+        b.add_overhead_info("CUPTI overhead", B + 12)
+        b.add_span(lo, hi, 3, 1, "PyTorch Profiler", "pfx")
+    return b

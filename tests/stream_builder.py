@@ -65,7 +65,7 @@ class StreamBuilder:
         r.type = typ
         r.flow_id, r.flow_type = flow_id, flow_type
         r.flags = (1 if flow_start else 0) | (2 if linked is not None else 0)
-        r.linked_corr = 0 if linked is None else linked
+        r.linked_id = 0 if linked is None else C.c_int32(linked & 0xFFFFFFFF).value
         r.schema_id = abi.KTJ_NONE if schema is None else schema
         r.args_off = self.arg_slots(values) if schema is not None else 0
         self.generic.append(r)

@@ -80,12 +80,12 @@ def test_engine_matches_oracle(cfg, n):
     run_case(cfg, n)
 
 
-def _engine_vs_oracle(sp, check_substrings=()):
+def _engine_vs_oracle(sp, check_substrings=(), **engine_options):
     import oracle_glue as og
     from kineto_amd.engine import TraceEngine
     ora = og.OracleRun(sp)
     want = ora.output()
-    with TraceEngine(sp.contents.trace_name.decode(), device=0) as eng:
+    with TraceEngine(sp.contents.trace_name.decode(), device=0, **engine_options) as eng:
         eng.submit_stream(sp)
         eng.process()
         got = eng.output()
@@ -112,6 +112,17 @@ def test_known_answer_cases_on_gpu():
     got = _engine_vs_oracle(b.build()).decode("latin1")
     for k, v in counts.items():
         assert got.count(k) == v
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_streams_on_gpu(seed):
+    """Every record class, activity type and edge value, mixed at random (tests/random_streams.py),
+    with direct-addressed and with hash-mode join tables and both emit kernels."""
+    import random_streams
+    print(f"random stream seed={seed}", flush=True)
+    sp = random_streams.random_stream(seed, wide_ids=seed % 2 == 1).build()
+    _engine_vs_oracle(sp)
+    _engine_vs_oracle(sp, hash_join=True, tile_emit=True)
 
 
 def test_join_edge_cases_on_gpu():

@@ -54,6 +54,14 @@ def test_shim_hand_made_cases(case):
     _compare(sp)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_shim_random_streams(seed):
+    import random_streams
+    sp = kat_cases.build_for_real_logger(lambda: (random_streams.random_stream(seed, wide_ids=seed % 2 == 1), None),
+                                         og.ref_stream_args())
+    _compare(sp)
+
+
 def test_shim_unknown_protocol_and_bad_sink():
     sp, release = abi.synth_stream(1, 50, **og.ref_stream_args())
     o = og.OracleRun(sp)

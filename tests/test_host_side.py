@@ -76,6 +76,36 @@ def test_formatting_core_host_build_matches_oracle(sim, cfg, n, tile):
     assert got == want
 
 
+def _sim_vs_oracle(sim, sp, tile):
+    o = og.OracleRun(sp)
+    want = o.output()
+    o.close()
+    p, nb = C.c_void_p(), C.c_uint64()
+    rc = sim.ktjsim_render(sp, tile, C.byref(p), C.byref(nb))
+    assert rc == 0
+    got = C.string_at(p, nb.value)
+    sim.ktjsim_free(p)
+    if got != want:
+        i = next((k for k in range(min(len(got), len(want))) if got[k] != want[k]), min(len(got), len(want)))
+        raise AssertionError(f"byte {i}: got {got[max(0, i - 80):i + 60]!r} want {want[max(0, i - 80):i + 60]!r}")
+
+
+def test_hand_made_cases_host_build_matches_oracle(sim):
+    import kat_cases
+    for case in kat_cases.SUBSTRING_CASES + [kat_cases.case_rocm_sync_trace]:
+        b, _ = case()
+        sp = b.build()
+        for tile in (0, 4096):
+            _sim_vs_oracle(sim, sp, tile)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_streams_host_build_matches_oracle(sim, seed):
+    import random_streams
+    sp = random_streams.random_stream(seed, wide_ids=seed % 2 == 1).build()
+    _sim_vs_oracle(sim, sp, 0 if seed % 3 else 4096)
+
+
 def test_device_double_and_clock_code_matches_oracle(sim):
     import math
     import random

@@ -36,6 +36,22 @@ def test_hand_made_cases_byte_identical(case):
     assert mine == theirs
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_streams_byte_identical(seed):
+    """Every record class, activity type and edge value the engine accepts, mixed at random: the
+    oracle's document against the real logger's."""
+    import random_streams
+    sp = kat_cases.build_for_real_logger(lambda: (random_streams.random_stream(seed, wide_ids=seed % 2 == 1), None),
+                                         og.ref_stream_args())
+    o = og.OracleRun(sp)
+    mine = o.output()
+    theirs = og.ref_render(sp, o)
+    o.close()
+    if mine != theirs:
+        i = next((k for k in range(min(len(mine), len(theirs))) if mine[k] != theirs[k]), min(len(mine), len(theirs)))
+        raise AssertionError(f"byte {i}: oracle {mine[max(0, i - 80):i + 60]!r} reference {theirs[max(0, i - 80):i + 60]!r}")
+
+
 def test_double_formatting_matches_fmt():
     ref, ora = og.load_ref(), og.load_oracle()
     b1, b2 = C.create_string_buffer(64), C.create_string_buffer(64)
