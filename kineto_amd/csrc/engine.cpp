@@ -114,7 +114,7 @@ struct ktj_engine {
   /* working buffers */
   DevBuf d_scalars, d_name_len, d_arg_len, d_sflags, d_name_off, d_arg_off, d_name_blob, d_arg_blob;
   DevBuf c_ts, c_dur, c_corr, c_dev, c_res, c_meta, c_ext;
-  DevBuf t_full, t_narrow, t_cpu, slot_ext, slot_f, slot_n, slot_f_dev, dev_link, dev_brief, sync_keys, sync_pos, sync_first;
+  DevBuf t_full, t_narrow, t_cpu, f_first, f_stream_src, f_pay, n_ext_src, n_kern_src, n_copy_src, n_pay, slot_ext, slot_f, slot_n, slot_f_dev, dev_link, dev_brief, sync_keys, sync_pos, sync_first;
   DevBuf q_keys, q_stream, q_amb, dn_hash, dn_first, dn_dev, dn_key, dn_rank;
   DevBuf s_dev_k, s_dev_r, s_res_k, s_res_r;
   DevBuf keys_a, keys_b, vals_a, vals_b, hist, scan_tmp;
@@ -202,7 +202,8 @@ void ktj_destroy(ktj_engine* e) {
   DevBuf* bufs[] = {&e->d_fields, &e->d_schemas, &e->d_cid_names, &e->d_flow_bits, &e->d_scalars, &e->d_name_len,
                     &e->d_arg_len, &e->d_sflags, &e->d_name_off, &e->d_arg_off, &e->d_name_blob, &e->d_arg_blob,
                     &e->c_ts, &e->c_dur, &e->c_corr, &e->c_dev, &e->c_res, &e->c_meta, &e->c_ext, &e->t_full,
-                    &e->t_narrow, &e->t_cpu, &e->slot_ext, &e->slot_f, &e->slot_n, &e->slot_f_dev, &e->dev_link, &e->dev_brief, &e->sync_keys, &e->sync_pos, &e->sync_first, &e->q_keys, &e->q_stream, &e->q_amb, &e->dn_hash, &e->dn_first, &e->dn_dev,
+                    &e->t_narrow, &e->t_cpu, &e->f_first, &e->f_stream_src, &e->f_pay, &e->n_ext_src, &e->n_kern_src,
+                    &e->n_copy_src, &e->n_pay, &e->slot_ext, &e->slot_f, &e->slot_n, &e->slot_f_dev, &e->dev_link, &e->dev_brief, &e->sync_keys, &e->sync_pos, &e->sync_first, &e->q_keys, &e->q_stream, &e->q_amb, &e->dn_hash, &e->dn_first, &e->dn_dev,
                     &e->dn_key, &e->dn_rank, &e->s_dev_k, &e->s_dev_r, &e->s_res_k, &e->s_res_r, &e->keys_a,
                     &e->keys_b, &e->vals_a, &e->vals_b, &e->hist, &e->scan_tmp, &e->mat, &e->len, &e->len_sorted,
                     &e->offs, &e->out, &e->tile_start};
@@ -401,9 +402,12 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   /* capacities for the hash mode (load <= 2/3); the direct mode uses a prefix of the same buffers */
   const uint32_t cap_full = pow2_at_least((nr + nd) + (nr + nd) / 2);
   const uint32_t cap_narrow = pow2_at_least((nx + nr) + (nx + nr) / 2), cap_cpu = pow2_at_least(2 * ng);
-  HIPCHK(e->t_full.ensure((cap_full + 1ull) * sizeof(FullSlot)));
-  HIPCHK(e->t_narrow.ensure((cap_narrow + 1ull) * sizeof(NarrowSlot)));
-  HIPCHK(e->t_cpu.ensure((cap_cpu + 1ull) * sizeof(KeySlot)));
+  HIPCHK(e->t_full.ensure((cap_full + 1ull) * 8)); HIPCHK(e->t_narrow.ensure((cap_narrow + 1ull) * 8));
+  HIPCHK(e->t_cpu.ensure((cap_cpu + 1ull) * 8));
+  HIPCHK(e->f_first.ensure((cap_full + 1ull) * 4)); HIPCHK(e->f_stream_src.ensure((cap_full + 1ull) * 4));
+  HIPCHK(e->f_pay.ensure((cap_full + 1ull) * sizeof(FullPay)));
+  HIPCHK(e->n_ext_src.ensure((cap_narrow + 1ull) * 4)); HIPCHK(e->n_kern_src.ensure((cap_narrow + 1ull) * 4));
+  HIPCHK(e->n_copy_src.ensure((cap_narrow + 1ull) * 4)); HIPCHK(e->n_pay.ensure((cap_narrow + 1ull) * sizeof(NarrowPay)));
   HIPCHK(e->slot_ext.ensure(nx * 4 + 16)); HIPCHK(e->slot_f.ensure(nr * 4 + 16)); HIPCHK(e->slot_n.ensure(nr * 4 + 16));
   HIPCHK(e->slot_f_dev.ensure(nd * 4 + 16)); HIPCHK(e->dev_link.ensure(nd * sizeof(DevLink) + 16));
   HIPCHK(e->dev_brief.ensure(nd * sizeof(DevBrief) + 16));
@@ -476,11 +480,13 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(hipEventRecord(e->ev[EV_CONVERT], st));
 
   /* ---- stage 2b: joins ---- */
-  FullTable tf{e->t_full.as<FullSlot>(), cap_full - 1, &sc->plan.ctl[KTJ_TBL_FULL]};
-  NarrowTable tn{e->t_narrow.as<NarrowSlot>(), cap_narrow - 1, &sc->plan.ctl[KTJ_TBL_NARROW]};
-  KeyTable t_cpu{e->t_cpu.as<KeySlot>(), cap_cpu - 1, &sc->plan.ctl[KTJ_TBL_CPU]};
+  Table tf{e->t_full.as<uint64_t>(), cap_full - 1, 0u, &sc->plan.ctl[KTJ_TBL_FULL]};
+  Table tn{e->t_narrow.as<uint64_t>(), cap_narrow - 1, 0u, &sc->plan.ctl[KTJ_TBL_NARROW]};
+  Table t_cpu{e->t_cpu.as<uint64_t>(), cap_cpu - 1, 1u, &sc->plan.ctl[KTJ_TBL_CPU]};
+  FullCols fc{e->f_first.as<uint32_t>(), e->f_stream_src.as<uint32_t>(), e->f_pay.as<FullPay>()};
+  NarrowCols nc{e->n_ext_src.as<uint32_t>(), e->n_kern_src.as<uint32_t>(), e->n_copy_src.as<uint32_t>(), e->n_pay.as<NarrowPay>()};
   HIPCHK(plan_tables(c, ng, nr, nd, x_recs, nx, cap_full, cap_narrow, cap_cpu, (e->flags & KTJ_CREATE_HASH_JOIN) != 0, sc, st));
-  HIPCHK(clear_tables(tf, tn, t_cpu, st));
+  HIPCHK(clear_tables(tf, fc, tn, nc, t_cpu, st));
   StreamTables stt{e->q_keys.as<uint64_t>(), e->q_stream.as<uint64_t>(), e->q_amb.as<uint32_t>(), e->dn_hash.as<uint64_t>(),
                    e->dn_first.as<uint32_t>(), e->dn_dev.as<int32_t>(), e->dn_key.as<uint64_t>(), e->dn_rank.as<uint32_t>()};
   HIPCHK(fill_u64(stt.q_keys, KTJ_EMPTY_KEY, KTJ_QUEUE_CAP + 1ull, st)); HIPCHK(fill_u64(stt.q_stream, 0, KTJ_QUEUE_CAP + 1ull, st));
@@ -489,15 +495,15 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(fill_u32(stt.d_rank, 0, KTJ_DENSE_CAP + 1ull, st));
   ApiTable api{e->d_cid_names.as<uint32_t>(), (uint32_t)e->cid_names.size(), e->d_flow_bits.as<uint32_t>(), e->malloc_cid};
   MatRow* mat = e->mat.as<MatRow>();
-  HIPCHK(build_extcorr(x_recs, nx, tn, e->slot_ext.as<uint32_t>(), sc, st));
+  HIPCHK(build_extcorr(x_recs, nx, tn, nc, e->slot_ext.as<uint32_t>(), sc, st));
   HIPCHK(build_cpu_ids(g_recs, ng, t_cpu, sc, st));
-  HIPCHK(build_runtime(nr, c, ng, tf, tn, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), sc, st));
-  HIPCHK(insert_device_first(nd, c, ng + nr, tf, e->slot_f_dev.as<uint32_t>(), sc, st));
-  HIPCHK(resolve_external(x_recs, nx, tn, e->slot_ext.as<uint32_t>(), t_cpu, st));
+  HIPCHK(build_runtime(nr, c, ng, tf, fc, tn, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), sc, st));
+  HIPCHK(insert_device_first(nd, c, ng + nr, tf, fc, e->slot_f_dev.as<uint32_t>(), sc, st));
+  HIPCHK(resolve_external(x_recs, nx, nc, e->slot_ext.as<uint32_t>(), t_cpu, st));
   /* second pass over the runtime rows: publishes into the tables and writes the joined rows */
-  HIPCHK(mat_runtime_rows(r_recs, nr, c, ng, api, tf, tn, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), ctx, mat,
+  HIPCHK(mat_runtime_rows(r_recs, nr, c, ng, api, fc, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), ctx, mat,
                           e->len.as<uint32_t>(), sc, st));
-  HIPCHK(link_device_rows(nd, c, ng + nr, tf, tn, e->slot_f_dev.as<uint32_t>(), e->dev_link.as<DevLink>(), sc, st));
+  HIPCHK(link_device_rows(nd, c, ng + nr, fc, tn, nc, e->slot_f_dev.as<uint32_t>(), e->dev_link.as<DevLink>(), sc, st));
   HIPCHK(backfill_streams(e->dev_brief.as<DevBrief>(), nd, c, ng + nr, stt, sc, st));
   HIPCHK(hipEventRecord(e->ev[EV_JOIN], st));
 

@@ -13,13 +13,19 @@
 namespace ktj {
 namespace gpu {
 
-/* Join tables in device memory.  A table is either direct-addressed (slot = key - base, chosen on
- * the GPU when the keys that will be inserted span less than the capacity: correlation ids are
- * dense counters in practice, so rows that arrive in id order touch consecutive slots and no slot
- * is ever probed twice) or an open-addressing hash table (any other key set).  A slot is free
- * while its key is KTJ_EMPTY_KEY; slot `cap` (one past the power-of-two range) is reserved for
- * the key whose value equals KTJ_EMPTY_KEY.  The mode lives in device memory (TableCtl) so that
- * no host round trip is needed to choose it. */
+/* Join tables in device memory.  A table maps a 64-bit key to a slot index; what is stored per
+ * slot lives in separate arrays indexed by it: compact 4-byte arrays for the "winner" indices that
+ * are updated with atomics (atomics on neighbouring addresses coalesce; on 48-byte strides they
+ * were measured 20 times slower), and payload arrays that the winners fill with plain stores.
+ * A table is either direct-addressed (slot = key - base, chosen on the GPU when the keys that
+ * will be inserted span less than the capacity: correlation ids are dense counters in practice,
+ * so rows that arrive in id order touch consecutive slots and nothing is probed) or an
+ * open-addressing hash table over `keys` (any other key set).  A hash slot is free while its key
+ * is KTJ_EMPTY_KEY; slot `cap` (one past the power-of-two range) is reserved for the key whose
+ * value equals KTJ_EMPTY_KEY.  The mode lives in device memory (TableCtl) so that no host round
+ * trip is needed to choose it.  In direct mode a table with keyed_direct == 0 does not touch
+ * `keys` at all: an id inside the range that was never inserted simply has empty per-slot
+ * values. */
 #define KTJ_EMPTY_KEY 0xFFFFFFFFFFFFFFFFULL
 struct KeyRange {          /* over the keys that will be inserted; empty while lo > hi */
   unsigned long long lo, hi;
@@ -30,38 +36,38 @@ struct TableCtl {
   uint32_t direct;
   uint32_t pad;
 };
-/* keyed by the full correlation id */
-struct FullSlot {
-  uint64_t key;
-  uint32_t stream_src;     /* last runtime row (index + 1) that carries a stream, 0 = none     */
-  uint32_t first;          /* smallest arrival index seen with this id, 0xFFFFFFFF = none      */
-  int64_t first_ts;        /* timestamp of row `first` when that is a runtime row              */
-  uint64_t stream;         /* stream of row stream_src                                          */
-};                         /* 32 bytes */
-/* keyed by the int-narrowed correlation id (and by the external-correlation records' full id) */
-struct NarrowSlot {
-  uint64_t key;
-  uint32_t ext_src;        /* last external-correlation record (index + 1), 0 = none; bit 31 is
-                              set once ext_val names an existing CPU op                          */
-  int32_t ext_val;         /* its external id if a CPU op with that id exists, else 0           */
-  uint32_t kern_src;       /* last in-window kernel-launch row (index + 1)                     */
-  uint32_t copy_src;       /* last in-window copy / malloc row (index + 1)                     */
-  uint64_t pay[3];         /* copy_src != 0: bytes of that row in pay[0]; else packed grid /
-                              workgroup of row kern_src (see pack_grid)                         */
-};                         /* 48 bytes */
-#define KTJ_EXT_LINKED 0x80000000u
-struct KeySlot {           /* plain set */
-  uint64_t key;
-};
-template <typename S>
-struct TableT {
-  S* s;
+struct Table {
+  uint64_t* keys;          /* cap + 1 */
   uint32_t mask;           /* cap - 1, cap a power of two >= 16 */
+  uint32_t keyed_direct;   /* 1: a plain set, membership is told by the stored key in both modes */
   const TableCtl* ctl;
 };
-typedef TableT<FullSlot> FullTable;
-typedef TableT<NarrowSlot> NarrowTable;
-typedef TableT<KeySlot> KeyTable;
+/* per slot of the table keyed by the full correlation id */
+struct FullPay {           /* published by the winning runtime row, read by device rows */
+  int64_t first_ts;        /* timestamp of row first[slot] when that is a runtime row          */
+  uint64_t stream;         /* stream of row stream_src[slot]; 0 = no row carries one            */
+};                         /* 16 bytes */
+struct FullCols {
+  uint32_t* first;         /* smallest arrival index seen with this id, 0xFFFFFFFF = none (atomicMin) */
+  uint32_t* stream_src;    /* last runtime row (index + 1) that carries a stream (atomicMax)    */
+  FullPay* pay;
+};
+/* per slot of the table keyed by the int-narrowed correlation id (and by the external-correlation
+ * records' full id) */
+struct NarrowPay {         /* two writers, each with whole 8-byte words of its own */
+  int32_t ext_val;         /* external id if a CPU op with that id exists, else 0               */
+  uint32_t linked;         /* 1 when ext_val names an existing CPU op                           */
+  uint32_t kind;           /* KTJ_DL_*: what pay[] holds                                        */
+  uint32_t pad;
+  uint64_t pay[3];         /* bytes of the winning copy / malloc row in pay[0], or packed grid /
+                              workgroup of the winning kernel-launch row (see pack_grid)        */
+};                         /* 40 bytes */
+struct NarrowCols {
+  uint32_t* ext_src;       /* last external-correlation record (index + 1), 0 = none            */
+  uint32_t* kern_src;      /* last in-window kernel-launch row (index + 1)                     */
+  uint32_t* copy_src;      /* last in-window copy / malloc row (index + 1)                     */
+  NarrowPay* pay;
+};
 #define KTJ_TBL_FULL 0
 #define KTJ_TBL_NARROW 1
 #define KTJ_TBL_CPU 2
@@ -163,20 +169,20 @@ hipError_t convert_rows(Columns c, uint64_t first_runtime, uint64_t n_runtime, u
 hipError_t plan_tables(Columns c, uint64_t n_generic, uint64_t n_runtime, uint64_t n_device, const ktj_extcorr_rec* e,
                        uint64_t n_ext, uint32_t cap_full, uint32_t cap_narrow, uint32_t cap_cpu, bool force_hash,
                        Scalars* sc, hipStream_t st);
-hipError_t clear_tables(FullTable tf, NarrowTable tn, KeyTable cpu, hipStream_t st);
-hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, uint32_t* slot_ext, Scalars* sc,
+hipError_t clear_tables(Table tf, FullCols fc, Table tn, NarrowCols nc, Table cpu, hipStream_t st);
+hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, uint32_t* slot_ext, Scalars* sc,
                          hipStream_t st);
-hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, KeyTable cpu, Scalars* sc, hipStream_t st);
+hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, Scalars* sc, hipStream_t st);
 /* the build passes read the columns only (correlation id, kind and has-stream bits of meta) */
-hipError_t build_runtime(uint64_t n, Columns c, uint64_t first_runtime, FullTable tf, NarrowTable tn, uint32_t* slot_f,
-                         uint32_t* slot_n, Scalars* sc, hipStream_t st);
-hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, FullTable tf, uint32_t* slot_f_dev,
+hipError_t build_runtime(uint64_t n, Columns c, uint64_t first_runtime, Table tf, FullCols fc, Table tn, NarrowCols nc,
+                         uint32_t* slot_f, uint32_t* slot_n, Scalars* sc, hipStream_t st);
+hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, uint32_t* slot_f_dev,
                                Scalars* sc, hipStream_t st);
-hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, const uint32_t* slot_ext, KeyTable cpu,
+hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
                             hipStream_t st);
 /* per device row: "External id", timestamp-order check, stream of the launching row, and the
  * size / grid hand-over (into link[]) */
-hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, FullTable tf, NarrowTable tn,
+hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, FullCols fc, Table tn, NarrowCols nc,
                             const uint32_t* slot_f_dev, DevLink* link, Scalars* sc, hipStream_t st);
 /* stream back-fill: queue table (keys/vals/ambiguous) and dense table are caller-provided, zeroed */
 struct StreamTables {
@@ -228,8 +234,8 @@ hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, c
 /* runtime rows: also publishes what device rows take over (first timestamp, stream, grid, size)
  * into the tables, reads the "External id" and counts timestamp-order violations; runs after
  * resolve_external and before link_device_rows */
-hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullTable tf,
-                            NarrowTable tn, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
+hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullCols fc,
+                            NarrowCols nc, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
                             uint32_t* len, Scalars* sc, hipStream_t st);
 hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const DevLink* link,
                            EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st);

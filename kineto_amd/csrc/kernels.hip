@@ -64,7 +64,7 @@ __device__ uint32_t table_find(const uint64_t* keys, uint32_t mask, uint64_t key
   return KTJ_NOSLOT;
 }
 
-/* Join tables (TableT).  Direct mode: slot = key - base.  Hash mode: slots are grouped in runs of
+/* Join tables (Table).  Direct mode: slot = key - base.  Hash mode: slots are grouped in runs of
  * sixteen; a key lives at position (key + rotation) & 15 of a run, where the rotation and the
  * probe sequence over runs (double hashing) depend only on the remaining key bits.  Sixteen
  * consecutive ids therefore share one run, while strided or clustered ids still spread like under
@@ -80,43 +80,46 @@ struct ProbeSeq {
   __device__ __forceinline__ uint32_t slot(uint32_t mask) const { return ((run << 4) | low) & mask; }
   __device__ __forceinline__ void next() { run += step; }
 };
-/* Returns the slot holding `key`, inserting it if absent; KTJ_NOSLOT when the table is full (hash
+/* Returns the slot of `key`, inserting it if absent; KTJ_NOSLOT when the table is full (hash
  * mode) or the key lies outside the planned range (direct mode; cannot happen for keys that were
  * part of the range computation). */
-template <typename S>
-__device__ uint32_t slot_insert(const TableT<S>& t, uint64_t key) {
-  if (key == KTJ_EMPTY_KEY) { t.s[t.mask + 1u].key = 0; return t.mask + 1u; }
+__device__ uint32_t slot_insert(const Table& t, uint64_t key) {
   if (t.ctl->direct) {
+    if (t.keyed_direct && key == KTJ_EMPTY_KEY) { t.keys[t.mask + 1u] = 0; return t.mask + 1u; }
     const uint64_t idx = key - t.ctl->base;
     if (idx > t.ctl->span) return KTJ_NOSLOT;
-    if (t.s[idx].key != key) t.s[idx].key = key; /* every writer stores the same value */
+    if (t.keyed_direct && t.keys[idx] != key) t.keys[idx] = key; /* every writer stores the same value */
     return (uint32_t)idx;
   }
+  if (key == KTJ_EMPTY_KEY) { t.keys[t.mask + 1u] = 0; return t.mask + 1u; }
   ProbeSeq p(key);
   for (uint32_t probe = 0; probe <= (t.mask >> 4); ++probe, p.next()) {
     const uint32_t slot = p.slot(t.mask);
-    uint64_t cur = t.s[slot].key;
+    uint64_t cur = t.keys[slot];
     if (cur == key) return slot;
     if (cur == KTJ_EMPTY_KEY) {
-      unsigned long long prev = atomicCAS((unsigned long long*)&t.s[slot].key, (unsigned long long)KTJ_EMPTY_KEY,
+      unsigned long long prev = atomicCAS((unsigned long long*)&t.keys[slot], (unsigned long long)KTJ_EMPTY_KEY,
                                           (unsigned long long)key);
       if (prev == KTJ_EMPTY_KEY || prev == key) return slot;
     }
   }
   return KTJ_NOSLOT;
 }
-template <typename S>
-__device__ uint32_t slot_find(const TableT<S>& t, uint64_t key) {
-  if (key == KTJ_EMPTY_KEY) return t.s[t.mask + 1u].key == 0 ? t.mask + 1u : KTJ_NOSLOT;
+/* In direct mode without stored keys every id inside the range has a slot; one that was never
+ * inserted reads as empty per-slot values. */
+__device__ uint32_t slot_find(const Table& t, uint64_t key) {
   if (t.ctl->direct) {
+    if (t.keyed_direct && key == KTJ_EMPTY_KEY) return t.keys[t.mask + 1u] == 0 ? t.mask + 1u : KTJ_NOSLOT;
     const uint64_t idx = key - t.ctl->base;
     if (idx > t.ctl->span) return KTJ_NOSLOT;
-    return t.s[idx].key == key ? (uint32_t)idx : KTJ_NOSLOT;
+    if (t.keyed_direct && t.keys[idx] != key) return KTJ_NOSLOT;
+    return (uint32_t)idx;
   }
+  if (key == KTJ_EMPTY_KEY) return t.keys[t.mask + 1u] == 0 ? t.mask + 1u : KTJ_NOSLOT;
   ProbeSeq p(key);
   for (uint32_t probe = 0; probe <= (t.mask >> 4); ++probe, p.next()) {
     const uint32_t slot = p.slot(t.mask);
-    uint64_t cur = t.s[slot].key;
+    uint64_t cur = t.keys[slot];
     if (cur == key) return slot;
     if (cur == KTJ_EMPTY_KEY) return KTJ_NOSLOT;
   }
@@ -541,12 +544,31 @@ __global__ void k_plan_tables(Scalars* sc, uint32_t cap_full, uint32_t cap_narro
     sc->plan.ctl[k] = c;
   }
 }
-/* frees every slot that can be reached: the planned span in direct mode, the whole table otherwise */
-template <typename S>
-__global__ void k_clear_table(TableT<S> t, S init) {
-  const uint64_t n = t.ctl->direct ? t.ctl->span + 1ull : (uint64_t)t.mask + 1ull;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) t.s[i] = init;
-  if (blockIdx.x == 0 && threadIdx.x == 0) t.s[t.mask + 1ull] = init;
+/* frees what can be reached: the planned span in direct mode, the whole table otherwise */
+__device__ __forceinline__ uint64_t table_extent(const Table& t) {
+  return t.ctl->direct ? t.ctl->span + 1ull : (uint64_t)t.mask + 1ull;
+}
+__global__ void k_clear_keys(Table t) {
+  if (t.ctl->direct && !t.keyed_direct) return; /* keys are not used at all */
+  const uint64_t n = table_extent(t);
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) t.keys[i] = KTJ_EMPTY_KEY;
+  if (blockIdx.x == 0 && threadIdx.x == 0) t.keys[t.mask + 1ull] = KTJ_EMPTY_KEY;
+}
+__global__ void k_clear_full(Table t, FullCols c) {
+  const uint64_t n = table_extent(t);
+  FullPay z; z.first_ts = 0; z.stream = 0;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i <= n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t k = i < n ? i : t.mask + 1ull; /* the last iteration clears the reserved slot */
+    c.first[k] = 0xFFFFFFFFu; c.stream_src[k] = 0; c.pay[k] = z;
+  }
+}
+__global__ void k_clear_narrow(Table t, NarrowCols c) {
+  const uint64_t n = table_extent(t);
+  NarrowPay z; z.ext_val = 0; z.linked = 0; z.kind = 0; z.pad = 0; z.pay[0] = z.pay[1] = z.pay[2] = 0;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i <= n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t k = i < n ? i : t.mask + 1ull;
+    c.ext_src[k] = 0; c.kern_src[k] = 0; c.copy_src[k] = 0; c.pay[k] = z;
+  }
 }
 
 hipError_t plan_tables(Columns c, uint64_t n_generic, uint64_t n_runtime, uint64_t n_device, const ktj_extcorr_rec* e,
@@ -568,31 +590,27 @@ hipError_t plan_tables(Columns c, uint64_t n_generic, uint64_t n_runtime, uint64
   hipLaunchKernelGGL(k_plan_tables, dim3(1), dim3(64), 0, st, sc, cap_full, cap_narrow, cap_cpu, force_hash ? 1 : 0);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t clear_tables(FullTable tf, NarrowTable tn, KeyTable cpu, hipStream_t st) {
-  FullSlot f;
-  f.key = KTJ_EMPTY_KEY; f.stream_src = 0; f.first = 0xFFFFFFFFu; f.first_ts = 0; f.stream = 0;
-  NarrowSlot nn;
-  nn.key = KTJ_EMPTY_KEY; nn.ext_src = 0; nn.ext_val = 0; nn.kern_src = 0; nn.copy_src = 0;
-  nn.pay[0] = nn.pay[1] = nn.pay[2] = 0;
-  KeySlot k;
-  k.key = KTJ_EMPTY_KEY;
-  hipLaunchKernelGGL(k_clear_table<FullSlot>, dim3(grid_stride_for((uint64_t)tf.mask + 1, KTJ_BLOCK * 4)), dim3(KTJ_BLOCK), 0, st, tf, f);
-  hipLaunchKernelGGL(k_clear_table<NarrowSlot>, dim3(grid_stride_for((uint64_t)tn.mask + 1, KTJ_BLOCK * 4)), dim3(KTJ_BLOCK), 0, st, tn, nn);
-  hipLaunchKernelGGL(k_clear_table<KeySlot>, dim3(grid_stride_for((uint64_t)cpu.mask + 1, KTJ_BLOCK * 4)), dim3(KTJ_BLOCK), 0, st, cpu, k);
+hipError_t clear_tables(Table tf, FullCols fc, Table tn, NarrowCols nc, Table cpu, hipStream_t st) {
+  const dim3 b(KTJ_BLOCK);
+  hipLaunchKernelGGL(k_clear_keys, dim3(grid_stride_for((uint64_t)tf.mask + 1, KTJ_BLOCK * 4)), b, 0, st, tf);
+  hipLaunchKernelGGL(k_clear_keys, dim3(grid_stride_for((uint64_t)tn.mask + 1, KTJ_BLOCK * 4)), b, 0, st, tn);
+  hipLaunchKernelGGL(k_clear_keys, dim3(grid_stride_for((uint64_t)cpu.mask + 1, KTJ_BLOCK * 4)), b, 0, st, cpu);
+  hipLaunchKernelGGL(k_clear_full, dim3(grid_stride_for((uint64_t)tf.mask + 1, KTJ_BLOCK * 4)), b, 0, st, tf, fc);
+  hipLaunchKernelGGL(k_clear_narrow, dim3(grid_stride_for((uint64_t)tn.mask + 1, KTJ_BLOCK * 4)), b, 0, st, tn, nc);
   return KTJ_LAUNCH_CHECK();
 }
 
 /* cpuCorrelationMap_[correlation] = externalId: RocmActivityProfiler.cpp:135-148 */
-__global__ void k_build_extcorr(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, uint32_t* slot_ext, Scalars* sc) {
+__global__ void k_build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, uint32_t* slot_ext, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint32_t slot = slot_insert(tn, e[i].correlation);
   slot_ext[i] = slot;
   if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
-  atomicMax(&tn.s[slot].ext_src, (uint32_t)i + 1u);
+  atomicMax(&nc.ext_src[slot], (uint32_t)i + 1u);
 }
 /* activityMap_[act->correlationId()] = act: GenericActivityProfiler.cpp:262 */
-__global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, KeyTable cpu, Scalars* sc) {
+__global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   if (slot_insert(cpu, (uint64_t)(int64_t)g[i].id) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
@@ -605,9 +623,12 @@ __global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, KeyTable c
  *              RocprofActivity_inl.h:28-30, 221-223, 245, 267)
  * The slots are remembered per row (slot_f, slot_n) for the second pass over the runtime rows;
  * slot_n also serves the "External id" lookup, so rows that insert nothing look their key up. */
-__global__ void k_build_runtime(uint64_t n, Columns c, uint64_t first_runtime, FullTable tf, NarrowTable tn,
-                                uint32_t* slot_f, uint32_t* slot_n, Scalars* sc) {
+__global__ void k_build_runtime(uint64_t n, Columns c, uint64_t first_runtime, Table tf, FullCols fc, Table tn,
+                                NarrowCols nc, uint32_t* slot_f, uint32_t* slot_n, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  /* one store per workgroup at most: every lane storing the same flag would queue up in L2 */
+  const bool carries_stream = i < n && (c.meta[first_runtime + i] & KTJ_M_HAS_STREAM);
+  if (__syncthreads_or(carries_stream ? 1 : 0) && threadIdx.x == 0) sc->have_stream_src = 1;
   if (i >= n) return;
   const uint64_t a = first_runtime + i;
   const uint64_t id = c.corr[a];
@@ -617,19 +638,16 @@ __global__ void k_build_runtime(uint64_t n, Columns c, uint64_t first_runtime, F
   slot_f[i] = sf;
   if (sf == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
   else {
-    if (tf.s[sf].first > (uint32_t)a) atomicMin(&tf.s[sf].first, (uint32_t)a);
-    if (meta & KTJ_M_HAS_STREAM) {
-      atomicMax(&tf.s[sf].stream_src, (uint32_t)i + 1u);
-      if (sc->have_stream_src == 0) sc->have_stream_src = 1;
-    }
+    if (fc.first[sf] > (uint32_t)a) atomicMin(&fc.first[sf], (uint32_t)a);
+    if (meta & KTJ_M_HAS_STREAM) atomicMax(&fc.stream_src[sf], (uint32_t)i + 1u);
   }
   const bool publishes = (meta & KTJ_M_VALID) && kind != KTJ_RT_DEFAULT;
   uint32_t sn;
   if (publishes) {
     sn = slot_insert(tn, narrow_corr_key(id));
     if (sn == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
-    else if (kind == KTJ_RT_KERNEL) atomicMax(&tn.s[sn].kern_src, (uint32_t)i + 1u);
-    else atomicMax(&tn.s[sn].copy_src, (uint32_t)i + 1u);
+    else if (kind == KTJ_RT_KERNEL) atomicMax(&nc.kern_src[sn], (uint32_t)i + 1u);
+    else atomicMax(&nc.copy_src[sn], (uint32_t)i + 1u);
   } else {
     /* every slot that carries an external id exists already (k_build_extcorr ran before) */
     sn = slot_find(tn, narrow_corr_key(id));
@@ -638,8 +656,8 @@ __global__ void k_build_runtime(uint64_t n, Columns c, uint64_t first_runtime, F
 }
 /* Device rows take part in "first seen" only when they are inside the window; every device row
  * remembers its slot (rows outside the window still take a stream from it). */
-__global__ void k_insert_device_first(uint64_t n, Columns c, uint64_t first_device, FullTable tf, uint32_t* slot_f_dev,
-                                      Scalars* sc) {
+__global__ void k_insert_device_first(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc,
+                                      uint32_t* slot_f_dev, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint64_t a = first_device + i;
@@ -648,7 +666,7 @@ __global__ void k_insert_device_first(uint64_t n, Columns c, uint64_t first_devi
   if (c.meta[a] & KTJ_M_VALID) {
     slot = slot_insert(tf, id);
     if (slot == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
-    else if (tf.s[slot].first > (uint32_t)a) atomicMin(&tf.s[slot].first, (uint32_t)a);
+    else if (fc.first[slot] > (uint32_t)a) atomicMin(&fc.first[slot], (uint32_t)a);
   } else {
     /* slots with a stream come from runtime rows and exist already */
     slot = slot_find(tf, id);
@@ -657,15 +675,15 @@ __global__ void k_insert_device_first(uint64_t n, Columns c, uint64_t first_devi
 }
 /* linkedActivity(): GenericActivityProfiler.cpp:397-408.  The record that won the slot resolves
  * its external id against the CPU-op ids once, for every row that will read the slot. */
-__global__ void k_resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, const uint32_t* slot_ext, KeyTable cpu) {
+__global__ void k_resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint32_t slot = slot_ext[i];
-  if (slot == KTJ_NOSLOT || (tn.s[slot].ext_src & ~KTJ_EXT_LINKED) != (uint32_t)i + 1u) return;
+  if (slot == KTJ_NOSLOT || nc.ext_src[slot] != (uint32_t)i + 1u) return;
   const uint64_t ext_id = e[i].external_id;
   if (slot_find(cpu, ext_id) != KTJ_NOSLOT) {
-    tn.s[slot].ext_val = (int32_t)(int64_t)ext_id;
-    tn.s[slot].ext_src = ((uint32_t)i + 1u) | KTJ_EXT_LINKED; /* only the winner writes here */
+    nc.pay[slot].ext_val = (int32_t)(int64_t)ext_id;
+    nc.pay[slot].linked = 1u;
   }
 }
 __device__ __forceinline__ bool is_async_op(uint32_t domain) { return domain != KTJ_DOM_MEMSET; }
@@ -675,7 +693,7 @@ __device__ __forceinline__ bool is_async_op(uint32_t domain) { return domain != 
  *  - checkTimestampOrder (GenericActivityProfiler.cpp:363-395) against the first row of the id,
  *  - the stream of the correlation-matched runtime row (RocmStreamQueue.h:56-75, first pass),
  *  - the size or grid/block the launching row hands over (RocprofActivity_inl.h:161-180). */
-__global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, FullTable tf, NarrowTable tn,
+__global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, FullCols fc, Table tn, NarrowCols nc,
                               const uint32_t* slot_f_dev, DevLink* link, Scalars* sc) {
   uint32_t n_linked = 0, n_bad = 0, n_unresolved = 0;
   const bool have_stream_src = sc->have_stream_src != 0;
@@ -690,12 +708,12 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Full
     int32_t ext = 0;
     const uint32_t sn = slot_find(tn, narrow_corr_key(id));
     if (sn != KTJ_NOSLOT) {
-      const NarrowSlot ns = tn.s[sn];
-      ext = ns.ext_val;
-      if ((ns.ext_src & KTJ_EXT_LINKED) && valid) ++n_linked;
-      if (domain != KTJ_DOM_MEMSET) {
-        if (ns.copy_src != 0) { l.flags = KTJ_DL_HAS_SIZE; l.p[0] = ns.pay[0]; }
-        else if (ns.kern_src != 0) { l.flags = KTJ_DL_HAS_GRID; l.p[0] = ns.pay[0]; l.p[1] = ns.pay[1]; l.p[2] = ns.pay[2]; }
+      const NarrowPay np = nc.pay[sn];
+      ext = np.ext_val;
+      if (np.linked && valid) ++n_linked;
+      if (domain != KTJ_DOM_MEMSET && np.kind != 0) {
+        l.flags = np.kind;
+        l.p[0] = np.pay[0]; l.p[1] = np.pay[1]; l.p[2] = np.pay[2];
       }
     }
     c.ext[a] = ext;
@@ -703,19 +721,19 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Full
     int64_t res = c.res[a];
     const uint32_t sf = slot_f_dev[i];
     if (sf != KTJ_NOSLOT) {
-      const FullSlot fs = tf.s[sf];
+      const FullPay fp = fc.pay[sf];
       if (valid) {
-        const uint64_t f = fs.first;
+        const uint64_t f = fc.first[sf];
         if (f != a && f != 0xFFFFFFFFull) {
           /* act1 = this row, act2 = first row; swapped when the first one is a runtime row */
           const bool first_is_runtime = f < first_device;
-          const int64_t tf_ts = first_is_runtime ? fs.first_ts : c.ts[f];
+          const int64_t tf_ts = first_is_runtime ? fp.first_ts : c.ts[f];
           const int64_t t1 = first_is_runtime ? tf_ts : c.ts[a];
           const int64_t t2 = first_is_runtime ? c.ts[a] : tf_ts;
           if (t2 != 0 && t1 > t2) ++n_bad;
         }
       }
-      if (have_stream_src && is_async_op(domain) && res == 0 && fs.stream_src != 0) { res = (int64_t)fs.stream; c.res[a] = res; }
+      if (have_stream_src && is_async_op(domain) && res == 0 && fp.stream != 0) { res = (int64_t)fp.stream; c.res[a] = res; }
     }
     if (is_async_op(domain) && res == 0) ++n_unresolved;
   }
@@ -724,42 +742,42 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Full
   block_add(&sc->n_unresolved, n_unresolved);
 }
 
-hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, uint32_t* slot_ext, Scalars* sc,
+hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, uint32_t* slot_ext, Scalars* sc,
                          hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_build_extcorr, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, tn, slot_ext, sc);
+  hipLaunchKernelGGL(k_build_extcorr, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, tn, nc, slot_ext, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, KeyTable cpu, Scalars* sc, hipStream_t st) {
+hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
   hipLaunchKernelGGL(k_build_cpu_ids, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, cpu, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t build_runtime(uint64_t n, Columns c, uint64_t first_runtime, FullTable tf, NarrowTable tn, uint32_t* slot_f,
-                         uint32_t* slot_n, Scalars* sc, hipStream_t st) {
+hipError_t build_runtime(uint64_t n, Columns c, uint64_t first_runtime, Table tf, FullCols fc, Table tn, NarrowCols nc,
+                         uint32_t* slot_f, uint32_t* slot_n, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_build_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_runtime, tf, tn,
-                     slot_f, slot_n, sc);
+  hipLaunchKernelGGL(k_build_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_runtime, tf, fc, tn,
+                     nc, slot_f, slot_n, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, FullTable tf, uint32_t* slot_f_dev,
+hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, uint32_t* slot_f_dev,
                                Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_insert_device_first, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_device, tf,
+  hipLaunchKernelGGL(k_insert_device_first, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_device, tf, fc,
                      slot_f_dev, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowTable tn, const uint32_t* slot_ext, KeyTable cpu,
+hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
                             hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_resolve_external, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, tn, slot_ext, cpu);
+  hipLaunchKernelGGL(k_resolve_external, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, nc, slot_ext, cpu);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, FullTable tf, NarrowTable tn,
+hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, FullCols fc, Table tn, NarrowCols nc,
                             const uint32_t* slot_f_dev, DevLink* link, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_link_device, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_device, tf, tn,
-                     slot_f_dev, link, sc);
+  hipLaunchKernelGGL(k_link_device, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_device, fc, tn,
+                     nc, slot_f_dev, link, sc);
   return KTJ_LAUNCH_CHECK();
 }
 
@@ -1298,8 +1316,8 @@ __global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx,
 /* Second pass over the runtime rows.  The row that won a slot field publishes what device rows
  * take over (timestamp of the first row, stream, grid/block, size); every row reads its
  * "External id" from the narrow slot and is checked against the first row of its id. */
-__global__ void k_mat_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullTable tf,
-                              NarrowTable tn, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
+__global__ void k_mat_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullCols fc,
+                              NarrowCols nc, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
                               uint32_t* len, Scalars* sc) {
   RowStats rs;
   uint32_t n_linked = 0, n_bad = 0;
@@ -1310,24 +1328,28 @@ __global__ void k_mat_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, u
     const bool valid = (c.meta[a] & KTJ_M_VALID) != 0;
     const uint32_t sf = slot_f[i], sn = slot_n[i];
     if (sf != KTJ_NOSLOT) {
-      FullSlot* fs = &tf.s[sf];
-      const uint64_t f = fs->first;
-      if (f == a) fs->first_ts = ts;
+      const uint64_t f = fc.first[sf];
+      if (f == a) fc.pay[sf].first_ts = ts;
       else if (f != 0xFFFFFFFFull) { /* an earlier runtime row has this id: checkTimestampOrder, swapped */
         const int64_t t1 = c.ts[f];
         if (ts != 0 && t1 > ts) ++n_bad;
       }
-      if (fs->stream_src == (uint32_t)i + 1u)
-        fs->stream = rec.kind == KTJ_RT_KERNEL ? rec.u.kernel.stream : rec.u.copy.stream;
+      if (fc.stream_src[sf] == (uint32_t)i + 1u)
+        fc.pay[sf].stream = rec.kind == KTJ_RT_KERNEL ? rec.u.kernel.stream : rec.u.copy.stream;
     }
     int32_t ext = 0;
     if (sn != KTJ_NOSLOT) {
-      NarrowSlot* ns = &tn.s[sn];
-      ext = ns->ext_val;
-      if ((ns->ext_src & KTJ_EXT_LINKED) && valid) ++n_linked;
-      const uint32_t copy_src = ns->copy_src; /* final: the build pass has ended */
-      if (copy_src == (uint32_t)i + 1u) ns->pay[0] = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
-      else if (copy_src == 0 && ns->kern_src == (uint32_t)i + 1u) pack_grid(rec, ns->pay);
+      NarrowPay* np = &nc.pay[sn];
+      ext = np->ext_val;
+      if (np->linked && valid) ++n_linked;
+      const uint32_t copy_src = nc.copy_src[sn]; /* final: the build pass has ended */
+      if (copy_src == (uint32_t)i + 1u) {
+        np->pay[0] = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
+        np->kind = KTJ_DL_HAS_SIZE;
+      } else if (copy_src == 0 && nc.kern_src[sn] == (uint32_t)i + 1u) {
+        pack_grid(rec, np->pay);
+        np->kind = KTJ_DL_HAS_GRID;
+      }
     }
     c.ext[a] = ext;
     const bool known = rec.cid < api.n_cids;
@@ -1369,11 +1391,11 @@ hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, c
                      len, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullTable tf,
-                            NarrowTable tn, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
+hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullCols fc,
+                            NarrowCols nc, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
                             uint32_t* len, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_mat_runtime, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, tf, tn,
+  hipLaunchKernelGGL(k_mat_runtime, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, fc, nc,
                      slot_f, slot_n, ctx, mat, len, sc);
   return KTJ_LAUNCH_CHECK();
 }
