@@ -93,6 +93,12 @@ enum {
  * linked activity (libkineto/src/output_json.cpp:871-874).  CPU-op spans submitted by a
  * profiler client and every activity that arrives through ActivityLogger::handleActivity use
  * this shape.
+ *
+ * Two kinds are not complete events.  KTJ_TYPE_CPU_INSTANT_EVENT prints an instant event
+ * (output_json.cpp:660-677).  KTJ_TYPE_HARDWARE_COUNTERS, KTJ_TYPE_MTIA_COUNTERS and
+ * KTJ_TYPE_XPU_SCOPE_PROFILER print counter events (output_json.cpp:679-716): the record's
+ * counterValues() are the keyed KTJ_F_F64 fields of its schema in schema order, its other fields
+ * are not printed.  Neither kind prints an External id or a flow event.
  */
 typedef struct ktj_generic_rec {
   int64_t start_ns;      /* startTime (absolute ns)                                            */
@@ -226,7 +232,7 @@ typedef struct ktj_field {
   uint16_t count;  /* slots consumed (1 except for arrays)                                    */
 } ktj_field;
 
-#define KTJ_MAX_SCHEMA_FIELDS 32
+#define KTJ_MAX_SCHEMA_FIELDS 1024
 
 /* ------------------------------------------------------------------------------------------
  * Small host-side events (formatted by the host part of the library; O(#devices + #streams)).

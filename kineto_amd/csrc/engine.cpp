@@ -466,7 +466,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(hipEventRecord(e->ev[EV_DICT], st));
 
   /* ---- stage 1: decode ---- */
-  HIPCHK(decode_generic(g_recs, ng, c, 0, sc, st));
+  HIPCHK(decode_generic(g_recs, ng, c, 0, sc, ctx, st));
   HIPCHK(decode_runtime(r_recs, nr, c, ng, st));
   HIPCHK(decode_device(d_recs, nd, c, ng + nr, e->dev_brief.as<DevBrief>(), st));
   HIPCHK(hipEventRecord(e->ev[EV_DECODE], st));

@@ -546,10 +546,14 @@ typedef WordWriter<DirectSink> GlobalWriter;
 
 /* The last seven bytes of a formatted activity, by kind (see format_activity):
  *   0: `  \n  },`   complete event without args, or a flow-start event
- *   1: ` }\n  },`   complete event with args and no flow event
+ *   1: ` }\n  },`   complete or instant event with args and no flow event, or a counter event
  *   2: `e"\n  },`   flow-end event */
 KTJ_HD KTJ_FI inline uint32_t tail_kind(const MatRow& r, bool has_args) {
   if (r.meta & KTJ_M_FLOW) return (r.meta & KTJ_M_FLOW_START) ? 0u : 2u;
+  if (((r.meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT) == KTJ_CLASS_GENERIC) { /* counter events always close an args object */
+    const uint32_t type = r.meta & KTJ_M_TYPE_MASK;
+    if (type == KTJ_TYPE_HARDWARE_COUNTERS || type == KTJ_TYPE_MTIA_COUNTERS || type == KTJ_TYPE_XPU_SCOPE_PROFILER) return 1u;
+  }
   return has_args ? 1u : 0u;
 }
 KTJ_HD KTJ_FI inline uint64_t tail_bytes(uint32_t kind, uint32_t count) { /* last `count` (0..7) bytes, low-aligned */
@@ -596,14 +600,14 @@ KTJ_HD KTJ_FI inline char digit_of(uint64_t p0, uint64_t p1, uint64_t p2, int j)
   const uint64_t word = j < 8 ? p0 : (j < 16 ? p1 : p2);
   return (char)(word >> (8 * (j & 7)));
 }
-template <class W> KTJ_HD KTJ_FI inline void put_f64(W& w, uint64_t bits) {
+template <class W> KTJ_HD KTJ_FI inline void put_f64(W& w, uint64_t bits, bool quote_non_finite = true) {
   const bool neg = (bits >> 63) != 0;
   const uint64_t mag = bits & 0x7FFFFFFFFFFFFFFFULL;
   if (mag >= 0x7FF0000000000000ULL) {
-    w.ch('"');
+    if (quote_non_finite) w.ch('"');
     if (neg) w.ch('-');
     if (mag > 0x7FF0000000000000ULL) KTJ_PUT(w, "nan"); else KTJ_PUT(w, "inf");
-    w.ch('"');
+    if (quote_non_finite) w.ch('"');
     return;
   }
   if (neg) w.ch('-');
@@ -664,9 +668,7 @@ struct BufferWriter {
 };
 KTJ_HD KTJ_FI inline int format_double(uint64_t bits, char* out) {
   BufferWriter b{out};
-  put_f64(b, bits);
-  /* put_f64 quotes non-finite values; the bare text is wanted here */
-  if (b.n && out[0] == '"') { for (int i = 1; i + 1 < b.n; ++i) out[i - 1] = out[i]; b.n -= 2; }
+  put_f64(b, bits, false);
   return b.n;
 }
 
@@ -903,12 +905,76 @@ template <class W> KTJ_HD KTJ_FI inline void format_instant(W& w, const MatRow& 
   } else KTJ_PUT(w, "\n    \n  },");
 }
 
+KTJ_HD KTJ_FI inline bool is_counter_type(uint32_t type) { /* output_json.cpp:847-856 */
+  return type == KTJ_TYPE_HARDWARE_COUNTERS || type == KTJ_TYPE_MTIA_COUNTERS || type == KTJ_TYPE_XPU_SCOPE_PROFILER;
+}
+/* A hardware-counter record prints one event per value (output_json.cpp:687-701): without values
+ * it prints nothing and takes no place in the document.  Every other record prints something. */
+KTJ_HD KTJ_FI inline bool generic_record_prints(const ktj_generic_rec& g, const EmitCtx& c) {
+  if (g.type != KTJ_TYPE_HARDWARE_COUNTERS) return true;
+  if (g.schema_id >= c.n_schemas) return false;
+  const ktj_schema_desc sd = c.schemas[g.schema_id];
+  for (uint32_t f = 0; f < sd.n_fields; ++f) {
+    const ktj_field fd = c.fields[sd.first_field + f];
+    if (fd.type == KTJ_F_F64 && fd.key_id != KTJ_NONE) return true;
+  }
+  return false;
+}
+/* handleCounterEvent + writeCounterEvent (output_json.cpp:679-716, 294-316).  The counter values
+ * of a record are the keyed double fields of its schema.  Hardware counters give one event per
+ * value on the device's "GPU <n> Counters" track; the other kinds one event holding all values.
+ * Names are printed as they were handed over, non-finite values bare; no flow event follows. */
+template <class W> KTJ_HD KTJ_FI inline void put_counter_head(W& w, uint32_t type) {
+  KTJ_PUT(w, "\n  {\n    \"ph\": \"C\",\n    \"cat\": \""); put_category(w, type); KTJ_PUT(w, "\",\n    \"name\": \"");
+}
+template <class W> KTJ_HD KTJ_FI inline void format_counter(W& w, const MatRow& r, const EmitCtx& c) {
+  const uint32_t type = r.meta & KTJ_M_TYPE_MASK;
+  const bool hw = type == KTJ_TYPE_HARDWARE_COUNTERS;
+  int64_t rel = r.ts - c.base_time_ns;
+  if (rel < 0) rel = 0;
+  const uint64_t tid = (uint64_t)sanitize_tid(r.res);
+  ktj_schema_desc sd;
+  sd.first_field = 0; sd.n_fields = 0;
+  if (r.aux < c.n_schemas) sd = c.schemas[r.aux];
+  if (!hw) {
+    put_counter_head(w, type);
+    if (!(r.meta & KTJ_M_NAME_BUILTIN)) put_arg_string(w, c.dict, r.name_id, true);
+    KTJ_PUT(w, "\",\n    \"pid\": "); put_i64(w, r.dev);
+    KTJ_PUT(w, ",\n    \"tid\": "); w.dec(tid);
+    KTJ_PUT(w, ",\n    \"ts\": "); put_ts(w, rel);
+    KTJ_PUT(w, ",\n    \"args\": {\n      ");
+  }
+  uint64_t slot = r.p[0];
+  bool first = true;
+  for (uint32_t f = 0; f < sd.n_fields; ++f) {
+    const ktj_field fd = c.fields[sd.first_field + f];
+    if (fd.type == KTJ_F_F64 && fd.key_id != KTJ_NONE) {
+      const uint64_t v = slot < c.n_args ? c.args[slot] : 0;
+      if (hw) {
+        put_counter_head(w, type);
+        put_arg_string(w, c.dict, fd.key_id, true);
+        KTJ_PUT(w, "\",\n    \"pid\": \"GPU "); put_i64(w, r.dev); KTJ_PUT(w, " Counters\"");
+        KTJ_PUT(w, ",\n    \"tid\": "); w.dec(tid);
+        KTJ_PUT(w, ",\n    \"ts\": "); put_ts(w, rel);
+        KTJ_PUT(w, ",\n    \"args\": {\n      \"\": "); put_f64(w, v, false);
+        KTJ_PUT(w, "\n    }\n  },");
+      } else {
+        if (!first) w.ch(',');
+        first = false;
+        w.ch('"'); put_arg_string(w, c.dict, fd.key_id, true); KTJ_PUT(w, "\": "); put_f64(w, v, false);
+      }
+    }
+    slot += fd.count;
+  }
+  if (!hw) KTJ_PUT(w, "\n    }\n  },");
+}
+
 /* One activity: the complete event and, if it takes part in a flow, the flow event after it. */
 template <class W> KTJ_HD KTJ_FI inline void format_activity(W& w, const MatRow& r, const EmitCtx& c) {
   const uint32_t type = r.meta & KTJ_M_TYPE_MASK;
-  if (type == KTJ_TYPE_CPU_INSTANT_EVENT && ((r.meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT) == KTJ_CLASS_GENERIC) {
-    format_instant(w, r, c);
-    return;
+  if (((r.meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT) == KTJ_CLASS_GENERIC) {
+    if (type == KTJ_TYPE_CPU_INSTANT_EVENT) { format_instant(w, r, c); return; }
+    if (is_counter_type(type)) { format_counter(w, r, c); return; }
   }
   int64_t ts = r.ts;
   int64_t dur = r.dur < 0 ? 0 : r.dur;                       /* output_json.cpp:860 */

@@ -156,7 +156,8 @@ hipError_t dict_write(const char* blob, const uint64_t* off, uint32_t n, const u
                       const uint64_t* arg_off, const uint32_t* flags, char* name_blob, char* arg_blob, hipStream_t st);
 
 /* ---- stage 1: decode ---- */
-hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, Scalars* sc, hipStream_t st);
+hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, Scalars* sc, EmitCtx ctx,
+                          hipStream_t st);
 hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st);
 hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, DevBrief* brief, hipStream_t st);
 

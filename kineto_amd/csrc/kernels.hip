@@ -392,7 +392,8 @@ __device__ __forceinline__ const Rec* stage_records(const Rec* recs, uint64_t n,
   return reinterpret_cast<const Rec*>(stage);
 }
 
-__global__ void k_decode_generic(const ktj_generic_rec* recs, uint64_t n, Columns c, uint64_t first, Scalars* sc) {
+__global__ void k_decode_generic(const ktj_generic_rec* recs, uint64_t n, Columns c, uint64_t first, Scalars* sc,
+                                 EmitCtx ctx) {
   __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_generic_rec) / 16];
   uint32_t cnt;
   const ktj_generic_rec* l = stage_records(recs, n, stage, &cnt);
@@ -407,7 +408,7 @@ __global__ void k_decode_generic(const ktj_generic_rec* recs, uint64_t n, Column
   c.corr[a] = (uint64_t)(int64_t)g.id;
   c.dev[a] = g.device;
   c.res[a] = g.resource;
-  c.meta[a] = KTJ_M_VALID | (KTJ_CLASS_GENERIC << KTJ_M_CLASS_SHIFT);
+  c.meta[a] = (generic_record_prints(g, ctx) ? KTJ_M_VALID : 0u) | (KTJ_CLASS_GENERIC << KTJ_M_CLASS_SHIFT);
   c.ext[a] = 0;
 }
 __global__ void k_decode_runtime(const ktj_runtime_rec* recs, uint64_t n, Columns c, uint64_t first) {
@@ -447,9 +448,10 @@ __global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns 
   brief[a - first] = b;
 }
 
-hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, Scalars* sc, hipStream_t st) {
+hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, Scalars* sc, EmitCtx ctx,
+                          hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_decode_generic, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, sc);
+  hipLaunchKernelGGL(k_decode_generic, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, sc, ctx);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st) {
@@ -1305,7 +1307,9 @@ __global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx,
                               uint32_t* len, Scalars* sc) {
   RowStats rs;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    MatRow m = mat_generic(g[i]);
+    const ktj_generic_rec rec = g[i];
+    MatRow m = mat_generic(rec);
+    if (!generic_record_prints(rec, ctx)) m.meta &= ~KTJ_M_VALID;
     mark_stream_sync(m, ctx, sync_first != nullptr && sync_first[i] != 0);
     store_row(&mat[i], m);
     len[i] = row_length(m, ctx, sc);

@@ -72,7 +72,9 @@ KTJ_HD inline MatRow mat_generic(const ktj_generic_rec& g) {
   m.res = g.resource;
   m.flow_id = g.flow_id;
   uint32_t meta = (g.type & KTJ_M_TYPE_MASK) | (KTJ_CLASS_GENERIC << KTJ_M_CLASS_SHIFT) | KTJ_M_VALID;
-  const bool instant = g.type == KTJ_TYPE_CPU_INSTANT_EVENT; /* output_json.cpp:842-845, 660-677: no flow, no External id */
+  /* instant and counter events (output_json.cpp:842-856, 660-716): no flow, no External id */
+  const bool instant = g.type == KTJ_TYPE_CPU_INSTANT_EVENT || g.type == KTJ_TYPE_HARDWARE_COUNTERS ||
+                       g.type == KTJ_TYPE_MTIA_COUNTERS || g.type == KTJ_TYPE_XPU_SCOPE_PROFILER;
   if (!instant && g.flow_id > 0 && (g.flow_type == KTJ_LINK_FWDBWD || g.flow_type == KTJ_LINK_ASYNC_CPU_GPU)) {
     meta |= KTJ_M_FLOW;
     if (g.flags & KTJ_GF_FLOW_START) meta |= KTJ_M_FLOW_START;

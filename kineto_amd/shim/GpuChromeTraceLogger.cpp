@@ -7,6 +7,7 @@
  */
 #include "GpuChromeTraceLogger.h"
 
+#include <cstring>
 #include <limits>
 
 #include "EnvMetadata.h"
@@ -60,6 +61,25 @@ uint32_t GpuChromeTraceLogger::intern(std::unordered_map<std::string, uint32_t>&
   pendingOffsets_.push_back(pendingBlob_.size());
   if (pendingBlob_.size() >= kStringBatchBytes) flushStrings();
   return id;
+}
+
+/* One schema per distinct list of counter names: a keyed double field for each. */
+uint32_t GpuChromeTraceLogger::counterSchema(const std::vector<std::pair<std::string, double>>& values) {
+  if (values.empty()) return KTJ_NONE;
+  std::string key;
+  std::vector<ktj_field> fields;
+  fields.reserve(values.size());
+  for (const auto& kv : values) {
+    const uint32_t id = intern(names_, kv.first);
+    fields.push_back(ktj_field{id, KTJ_F_F64, 1});
+    key.append(reinterpret_cast<const char*>(&id), sizeof(id));
+  }
+  auto it = counterSchemas_.find(key);
+  if (it != counterSchemas_.end()) return it->second;
+  uint32_t sid = KTJ_NONE;
+  note(ktj_register_schema(engine_, fields.data(), fields.size(), &sid), "ktj_register_schema");
+  counterSchemas_.emplace(std::move(key), sid);
+  return sid;
 }
 
 void GpuChromeTraceLogger::flushStrings() {
@@ -132,12 +152,13 @@ void GpuChromeTraceLogger::handleActivity(const ITraceActivity& op) {
   const ITraceActivity* linked = op.linkedActivity();
   const int64_t device = op.deviceId();
   const int64_t flowId = op.flowId();
-  /* counter events (output_json.cpp:847-856, 679-716) need counterValues(), collective metadata
-   * (:899-908) the linked op's own metadata: neither fits the packed record */
-  bool unsupported = type == ActivityType::HARDWARE_COUNTERS || type == ActivityType::MTIA_COUNTERS ||
-      type == ActivityType::XPU_SCOPE_PROFILER;
-  if (linked != nullptr && linked->name() == kParamCommsName) {
-    unsupported = unsupported || type == ActivityType::CONCURRENT_KERNEL ||
+  const bool counter = type == ActivityType::HARDWARE_COUNTERS || type == ActivityType::MTIA_COUNTERS ||
+      type == ActivityType::XPU_SCOPE_PROFILER; /* output_json.cpp:847-856 */
+  /* collective metadata (output_json.cpp:899-908) needs the linked op's own metadata, which does
+   * not fit the packed record */
+  bool unsupported = false;
+  if (!counter && linked != nullptr && linked->name() == kParamCommsName) {
+    unsupported = type == ActivityType::CONCURRENT_KERNEL ||
         (type == ActivityType::MTIA_CCP_EVENTS && name.rfind("hccl::", 0) == 0);
   }
   unsupported = unsupported || device < std::numeric_limits<int32_t>::min() || device > std::numeric_limits<int32_t>::max();
@@ -164,6 +185,21 @@ void GpuChromeTraceLogger::handleActivity(const ITraceActivity& op) {
   if (linked != nullptr) {
     r.flags |= KTJ_GF_LINKED;
     r.linked_id = static_cast<int32_t>(linked->correlationId()); /* `int external_id = …`, :873 */
+  }
+  if (counter) { /* handleCounterEvent (:679-716) prints counterValues() and nothing else */
+    const auto& values = op.counterValues();
+    r.schema_id = counterSchema(values);
+    r.args_off = nextSlot_;
+    nextSlot_ += values.size();
+    for (const auto& kv : values) {
+      uint64_t bits;
+      static_assert(sizeof(bits) == sizeof(kv.second), "double is 64 bits");
+      std::memcpy(&bits, &kv.second, sizeof(bits));
+      slots_.push_back(bits);
+    }
+    records_.push_back(r);
+    if (records_.size() >= kRecordBatch) flushRecords();
+    return;
   }
   const std::string metadata = op.metadataJson();
   if (metadata.empty()) {

@@ -52,8 +52,8 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
                      int64_t endTime) override;
 
   std::string traceFileName() const { return fileName_; }
-  /* activities of kinds the engine does not render (counter events, collective metadata of
-   * record_param_comms): they are dropped and counted here */
+  /* activities the engine does not render (kernels that would carry the collective metadata of
+   * a linked record_param_comms op): they are dropped and counted here */
   uint64_t unsupportedActivities() const { return unsupported_; }
   /* ktj status of the first failed engine call, 0 if none */
   int engineStatus() const { return status_; }
@@ -63,6 +63,7 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
 
  private:
   uint32_t intern(std::unordered_map<std::string, uint32_t>& index, const std::string& s);
+  uint32_t counterSchema(const std::vector<std::pair<std::string, double>>& values);
   void flushStrings();
   void flushRecords();
   bool ok() const { return engine_ != nullptr && status_ == 0; }
@@ -77,6 +78,7 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
   /* strings not yet handed to the engine: blob + offsets, ids are consecutive from nextStringId_ */
   std::unordered_map<std::string, uint32_t> names_;
   std::unordered_map<std::string, uint32_t> fragments_;
+  std::unordered_map<std::string, uint32_t> counterSchemas_; /* key: the name ids, 4 bytes each */
   std::string pendingBlob_;
   std::vector<uint64_t> pendingOffsets_;
   uint32_t nextStringId_ = 0;

@@ -26,7 +26,9 @@
  *   - canonical order: stable merge sort here; std::stable_sort on tuples inside oracle/_ref.
  *   - instant events and the Stream Sync row remap: byte-compared with the real logger on a
  *       hand-made case (tests/kat_cases.py: case_instant_and_stream_sync).
- * Not restated: counter events (output_json.cpp:679-716) and collective metadata (:718-835, 899-908).
+ *   - counter events: byte-compared with the real logger on a hand-made case
+ *       (tests/kat_cases.py: case_counter_events) and inside the seeded random streams.
+ * Not restated: collective metadata (output_json.cpp:718-835, 899-908).
  */
 #define _GNU_SOURCE
 #include "ktj_oracle.h"
@@ -1044,11 +1046,67 @@ static void handle_instant_event(ktj_oracle* o, const ktj_mat_activity* a) {
   free(name); free(args.p); free(meta.p);
 }
 
-/* handleActivity + handleGenericLink + handleLink: output_json.cpp:837-1021.  Counter event kinds
- * (handleCounterEvent, :679-716) and the collective metadata of record_param_comms (:899-908) are
- * not restated here. */
+/* writeCounterEvent: output_json.cpp:294-316.  The args object is printed even when empty. */
+static void write_counter_event(ktj_oracle* o, const char* cat, const char* name, size_t name_n,
+                                const char* pid, const char* tid, int64_t ts, const sbuf* args) {
+  char t[40];
+  ktj_oracle_fmt_ts(ts, t);
+  sbuf* b = &o->out;
+  sb_puts(b, "\n  {\n    \"ph\": \"C\",\n    \"cat\": \""); sb_puts(b, cat);
+  sb_puts(b, "\",\n    \"name\": \""); sb_put(b, name, name_n);
+  sb_puts(b, "\",\n    \"pid\": "); sb_puts(b, pid);
+  sb_puts(b, ",\n    \"tid\": "); sb_puts(b, tid);
+  sb_puts(b, ",\n    \"ts\": "); sb_puts(b, t);
+  sb_puts(b, ",\n    \"args\": {\n      "); sb_put(b, args->p, args->n);
+  sb_puts(b, "\n    }\n  },");
+}
+
+static int is_counter_type(int type) { /* output_json.cpp:847-856 */
+  return type == KTJ_TYPE_HARDWARE_COUNTERS || type == KTJ_TYPE_MTIA_COUNTERS || type == KTJ_TYPE_XPU_SCOPE_PROFILER;
+}
+/* handleCounterEvent: output_json.cpp:679-716.  counterValues() of a record are the keyed
+ * double fields of its schema, in schema order; its other fields are never printed.  Names are
+ * printed as they are, values by fmt "{}" (non-finite ones bare). */
+static void handle_counter_event(ktj_oracle* o, const ktj_mat_activity* a) {
+  const int64_t ts = rel_time(o, a->ts);
+  const char* cat = ktj_oracle_type_name(a->type);
+  char pid[48], tid[24], n[48];
+  fmt_i64(sanitize_tid(a->resource), tid);
+  const int hw = a->type == KTJ_TYPE_HARDWARE_COUNTERS;
+  if (hw) sprintf(pid, "\"GPU %lld Counters\"", (long long)a->device); /* :688 */
+  else fmt_i64(a->device, pid);
+  sbuf args = {0};
+  const uint64_t* slot = a->slots;
+  for (uint32_t f = 0; f < a->n_fields; slot += a->fields[f].count, ++f) {
+    const ktj_field* fd = &a->fields[f];
+    if (fd->type != KTJ_F_F64 || fd->key_id == KTJ_NONE) continue;
+    const char* kp; uint64_t kl;
+    ktj_oracle_string(o, fd->key_id, &kp, &kl);
+    double d; memcpy(&d, &slot[0], 8);
+    const size_t vn = ktj_oracle_fmt_double(d, n);
+    if (hw) { /* one event per counter on the device's counter track: :687-701 */
+      sbuf one = {0};
+      sb_puts(&one, "\"\": "); sb_put(&one, n, vn);
+      write_counter_event(o, cat, kp, kl, pid, tid, ts, &one);
+      free(one.p);
+    } else {  /* ArgsBuilder::addRaw :161-164 */
+      if (args.n) sb_putc(&args, ',');
+      sb_putc(&args, '"'); sb_put(&args, kp, kl); sb_puts(&args, "\": "); sb_put(&args, n, vn);
+    }
+  }
+  if (!hw) {
+    const char* nm; uint64_t nl;
+    ktj_oracle_string(o, a->name_id, &nm, &nl);
+    write_counter_event(o, cat, nm, nl, pid, tid, ts, &args);
+  }
+  free(args.p);
+}
+
+/* handleActivity + handleGenericLink + handleLink: output_json.cpp:837-1021.  The collective
+ * metadata of record_param_comms (:899-908) is not restated here. */
 static void handle_activity(ktj_oracle* o, const ktj_mat_activity* a) {
   if (a->type == KTJ_TYPE_CPU_INSTANT_EVENT) { handle_instant_event(o, a); return; } /* :842-845 */
+  if (is_counter_type(a->type)) { handle_counter_event(o, a); return; }               /* :847-856 */
   int64_t ts = a->ts;
   int64_t duration = a->dur < 0 ? 0 : a->dur;              /* :860 */
   if (a->type == KTJ_TYPE_GPU_USER_ANNOTATION) { ts -= 1; duration += 2; } /* :862-869 */

@@ -106,6 +106,23 @@ struct MatActivity : public ITraceActivity {
       slot += fd.count;
     }
   }
+  // The keyed double fields are the activity's counter values (read for counter kinds only).
+  mutable std::vector<std::pair<std::string, double>> counters;
+  mutable bool countersBuilt = false;
+  const std::vector<std::pair<std::string, double>>& counterValues() const override {
+    if (!countersBuilt) {
+      countersBuilt = true;
+      const uint64_t* slot = a->slots;
+      for (uint32_t f = 0; f < a->n_fields; slot += a->fields[f].count, ++f) {
+        const ktj_field& fd = a->fields[f];
+        if (fd.type != KTJ_F_F64 || fd.key_id == KTJ_NONE) continue;
+        double d;
+        std::memcpy(&d, &slot[0], 8);
+        counters.emplace_back(st->get(fd.key_id), d);
+      }
+    }
+    return counters;
+  }
   const std::string metadataJson() const override {
     // A field without a key stands for a whole pre-rendered fragment (what an activity's own
     // metadataJson() returned); it is passed through untouched.

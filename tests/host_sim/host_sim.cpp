@@ -97,7 +97,10 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   std::vector<uint8_t> flow_start(s->n_cids ? s->n_cids : 1, 0);
   for (uint64_t i = 0; i < s->n_flow_start; ++i) if (s->flow_start_cids[i] < s->n_cids) flow_start[s->flow_start_cids[i]] = 1;
 
-  for (uint64_t i = 0; i < ng; ++i) mat[i] = mat_generic(s->generic[i]);
+  for (uint64_t i = 0; i < ng; ++i) {
+    mat[i] = mat_generic(s->generic[i]);
+    if (!generic_record_prints(s->generic[i], ctx)) mat[i].meta &= ~KTJ_M_VALID;
+  }
 
   std::unordered_map<uint64_t, uint64_t> stream_src;       // full id -> runtime idx (last wins)
   std::unordered_map<uint64_t, uint64_t> kernel_src, size_src;  // int-truncated id -> runtime idx (in range, last wins)

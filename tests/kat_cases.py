@@ -168,7 +168,39 @@ def case_instant_and_stream_sync():
     return b, expect
 
 
-SUBSTRING_CASES = [case_instant_and_stream_sync, case_logger_events, case_trace_span, case_benchmark_cpu_op, case_typed_kernel_args,
+def case_counter_events():
+    """Counter events (handleCounterEvent + writeCounterEvent, output_json.cpp:679-716, 294-316).
+    Hardware counters print one event per value on the device's counter track, the other counter
+    kinds one event with every value; values go through fmt "{}" and non-finite ones stay bare;
+    names are printed as they are; neither an External id nor a flow event follows.  Expected
+    strings follow the reference's templates; the whole document is compared with the real
+    logger where it is built."""
+    MTIA_COUNTERS, XPU_SCOPE_PROFILER, HARDWARE_COUNTERS = 17, 26, 28
+    b = StreamBuilder()
+    two = b.schema([("sm__cycles", abi.F_F64, 1), ('odd "name"\\x', abi.F_F64, 1)])
+    mixed = b.schema([("skipped int", abi.F_I64, 1), ("busy", abi.F_F64, 1), (None, abi.F_RAW, 1), ("idle", abi.F_F64, 1)])
+    specials = b.schema([("a", abi.F_F64, 1), ("b", abi.F_F64, 1), ("c", abi.F_F64, 1), ("d", abi.F_F64, 1), ("e", abi.F_F64, 1)])
+    b.add_generic("ignored name", HARDWARE_COUNTERS, B + 1000, B + 1000, 3, -9, id=5, schema=two, values=[1.5, 2e-7],
+                  flow_id=5, flow_type=2)
+    b.add_generic('mtia "c"\\n', MTIA_COUNTERS, B + 2000, B + 2500, 1, 4, id=6, schema=mixed,
+                  values=[12, 0.25, b.s('"x": 1'), 1e21], flow_id=6, flow_type=2, flow_start=True)
+    b.add_generic("scope", XPU_SCOPE_PROFILER, B + 3000, B + 3000, 2, 2, schema=specials,
+                  values=[float("inf"), float("-inf"), float("nan"), -0.0, 123456789012345680.0])
+    b.add_generic("no values", MTIA_COUNTERS, B + 4000, B + 4000, 1, 4)
+    b.add_generic("no values hw", HARDWARE_COUNTERS, B + 4500, B + 4500, 1, 4)
+    b.add_generic("before base", XPU_SCOPE_PROFILER, B - 50, B - 50, 2, 2, schema=two, values=[3.0, 4.0])
+    expect = [
+        '\n  {\n    "ph": "C",\n    "cat": "hardware_counters",\n    "name": "sm__cycles",\n    "pid": "GPU 3 Counters",\n    "tid": 9,\n    "ts": 1.000,\n    "args": {\n      "": 1.5\n    }\n  },'
+        '\n  {\n    "ph": "C",\n    "cat": "hardware_counters",\n    "name": "odd "name"\\x",\n    "pid": "GPU 3 Counters",\n    "tid": 9,\n    "ts": 1.000,\n    "args": {\n      "": 2e-07\n    }\n  },',
+        '\n  {\n    "ph": "C",\n    "cat": "mtia_counters",\n    "name": "mtia "c"\\n",\n    "pid": 1,\n    "tid": 4,\n    "ts": 2.000,\n    "args": {\n      "busy": 0.25,"idle": 1e+21\n    }\n  },',
+        '"name": "scope",\n    "pid": 2,\n    "tid": 2,\n    "ts": 3.000,\n    "args": {\n      "a": inf,"b": -inf,"c": nan,"d": -0,"e": 1.2345678901234568e+17\n    }\n  },',
+        '"name": "no values",\n    "pid": 1,\n    "tid": 4,\n    "ts": 4.000,\n    "args": {\n      \n    }\n  },',
+        '"name": "before base",\n    "pid": 2,\n    "tid": 2,\n    "ts": 0.000,\n    "args": {\n      "sm__cycles": 3,"odd "name"\\x": 4\n    }\n  },',
+    ]
+    return b, expect
+
+
+SUBSTRING_CASES = [case_counter_events, case_instant_and_stream_sync, case_logger_events, case_trace_span, case_benchmark_cpu_op, case_typed_kernel_args,
                    case_typed_metadata_pins, case_names, case_resource_infos]
 
 

@@ -7,8 +7,7 @@ import struct
 from kineto_amd import abi
 from stream_builder import B, StreamBuilder
 
-# every ActivityType except the counter kinds, which the engine does not render
-TYPES = [t for t in range(29) if t not in (17, 26, 28)]
+TYPES = list(range(29))  # every ActivityType
 I64_MIN, I64_MAX = -(1 << 63), (1 << 63) - 1
 
 
@@ -85,7 +84,7 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False)
                 else:
                     values.append(_i64(rng))
         s0 = t()
-        b.add_generic(rng.choice(names + [None]), rng.choice(TYPES + [0, 0, 0, 9, 15]), s0, s0 + rng.choice([0, 1, 999, 1000, -3, 10**5]),
+        b.add_generic(rng.choice(names + [None]), rng.choice(TYPES + [0, 0, 0, 9, 15, 17, 28, 28]), s0, s0 + rng.choice([0, 1, 999, 1000, -3, 10**5]),
                       rng.choice(pids), rng.choice(tids), id=rng.choice([0, -2, 5, 6, 7, 8, 2**31 - 1, -(2**31)] + ids[:8]),
                       schema=sid, values=values, flow_id=rng.choice([0, 0, 1, 77, 2**32 - 1, 2**40 + 3, -4]), flow_type=rng.choice([0, 1, 2, 3]),
                       flow_start=rng.random() < 0.5, linked=rng.choice([None, None, 5, -9, 2**40 + 1]))
