@@ -223,7 +223,9 @@ enum {
   KTJ_F_BOOL = 3,  /* true / false                                        (1 slot)            */
   KTJ_F_STR = 4,   /* slot = string id, emitted in double quotes          (1 slot)            */
   KTJ_F_RAW = 5,   /* slot = string id, emitted verbatim (RawJson)        (1 slot)            */
-  KTJ_F_I64_ARRAY = 6 /* [a, b, c] with `count` int64 elements            (count slots)       */
+  KTJ_F_I64_ARRAY = 6, /* [a, b, c] with `count` int64 elements           (count slots)       */
+  KTJ_F_COLLECTIVE = 7 /* slot = index from ktj_add_collective; keyless, recognised only as the
+                          first field of a schema; prints nothing in the fragment (1 slot)    */
 };
 
 typedef struct ktj_field {
@@ -233,6 +235,40 @@ typedef struct ktj_field {
 } ktj_field;
 
 #define KTJ_MAX_SCHEMA_FIELDS 1024
+
+/* ------------------------------------------------------------------------------------------
+ * Collective metadata (ChromeTraceLogger::appendCollectiveMetadata, output_json.cpp:718-835,
+ * 899-908, and the "distributedInfo" entry of the footer, :1030-1064).  The logger copies it from
+ * the `record_param_comms` CPU op an activity is linked to; here the caller hands the op's
+ * values over once (ktj_add_collective) and refers to them from records by index, through a
+ * leading KTJ_F_COLLECTIVE field:
+ *   - on a generic record of type KTJ_TYPE_CONCURRENT_KERNEL or KTJ_TYPE_MTIA_CCP_EVENTS
+ *     (backends "nccl" / "hccl"): the record prints the collective arguments after its own
+ *     metadata — the case of an activity that arrives with its linked op resolved;
+ *   - on any other generic record (the record_param_comms CPU op itself): kernel rows of
+ *     KTJ_REC_DEVICE that the join links to this record print them (backend "nccl").
+ * Every value is the text getMetadataValue() returns for the key (strings may keep their
+ * surrounding quotes); NULL or "" = the op does not carry the key.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct ktj_collective_meta {
+  const char* collective_name;   /* "Collective name"            */
+  const char* in_msg_nelems;     /* "In msg nelems"              */
+  const char* out_msg_nelems;    /* "Out msg nelems"             */
+  const char* group_size;        /* "Group size"                 */
+  const char* dtype;             /* "dtype"                      */
+  const char* in_tensors_start;  /* "Input Tensors start"        */
+  const char* out_tensors_start; /* "Output Tensors start"       */
+  const char* in_split;          /* "In split size"              */
+  const char* out_split;         /* "Out split size"             */
+  const char* pg_name;           /* "Process Group Name"         */
+  const char* pg_desc;           /* "Process Group Description"  */
+  const char* group_ranks;       /* "Process Group Ranks"        */
+  const char* dst_rank;          /* "Dst Rank"                   */
+  const char* src_rank;          /* "Src Rank"                   */
+  const char* seq;               /* "Seq"                        */
+  const char* comms_id;          /* "Comms Id"                   */
+  const char* rank;              /* "Rank" (distributedInfo only) */
+} ktj_collective_meta;
 
 /* ------------------------------------------------------------------------------------------
  * Small host-side events (formatted by the host part of the library; O(#devices + #streams)).
@@ -362,6 +398,10 @@ int ktj_intern_strings(ktj_engine* e, const char* blob, const uint64_t* offsets,
 /* Args schema registration (fields in emission order). */
 int ktj_register_schema(ktj_engine* e, const ktj_field* fields, size_t n_fields,
                         uint32_t* schema_id);
+
+/* One record_param_comms op's collective metadata; *index receives the value for the slot of a
+ * KTJ_F_COLLECTIVE field.  The strings are copied. */
+int ktj_add_collective(ktj_engine* e, const ktj_collective_meta* meta, uint32_t* index);
 
 /* Args blob (8-byte slots) referenced by ktj_generic_rec::args_off.  Appends; *first_slot
  * receives the slot index of the first appended value. */

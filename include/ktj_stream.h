@@ -72,6 +72,10 @@ typedef struct ktj_stream {
   uint64_t n_overhead_infos;
   const ktj_trace_span* spans;
   uint64_t n_spans;
+
+  /* collective metadata, indexed by the slots of KTJ_F_COLLECTIVE fields */
+  const ktj_collective_meta* collectives;
+  uint64_t n_collectives;
 } ktj_stream;
 
 /* ------------------------------------------------------------------------------------------

@@ -16,7 +16,7 @@ KTJ_CREATE_HASH_JOIN = 0x4
 
 REC_GENERIC, REC_RUNTIME, REC_DEVICE, REC_EXTCORR = 0, 1, 2, 3
 INFO_DEVICE, INFO_RESOURCE, INFO_OVERHEAD, INFO_SPAN = 0, 1, 2, 3
-F_I64, F_U64, F_F64, F_BOOL, F_STR, F_RAW, F_I64_ARRAY = range(7)
+F_I64, F_U64, F_F64, F_BOOL, F_STR, F_RAW, F_I64_ARRAY, F_COLLECTIVE = range(8)
 N_STAGES = 12
 STAGE_NAMES = ["dict", "decode", "convert", "join", "sort", "size", "scan", "emit", "d2h", "file",
                "total_gpu", "reserved"]
@@ -95,6 +95,15 @@ class TraceSpan(C.Structure):
                 ("iteration", C.c_int32), ("name", C.c_char_p), ("prefix", C.c_char_p)]
 
 
+COLLECTIVE_KEYS = ("collective_name", "in_msg_nelems", "out_msg_nelems", "group_size", "dtype", "in_tensors_start",
+                   "out_tensors_start", "in_split", "out_split", "pg_name", "pg_desc", "group_ranks", "dst_rank",
+                   "src_rank", "seq", "comms_id", "rank")
+
+
+class CollectiveMeta(C.Structure):
+    _fields_ = [(k, C.c_char_p) for k in COLLECTIVE_KEYS]
+
+
 class ClockModel(C.Structure):
     _fields_ = [("t0_approx", C.c_uint64), ("t0", C.c_int64), ("scale", C.c_double),
                 ("async_offset", C.c_int64), ("runtime_mode", C.c_uint32),
@@ -131,7 +140,8 @@ class Stream(C.Structure):
                 ("device_infos", C.POINTER(DeviceInfo)), ("n_device_infos", C.c_uint64),
                 ("resource_infos", C.POINTER(ResourceInfo)), ("n_resource_infos", C.c_uint64),
                 ("overhead_infos", C.POINTER(OverheadInfo)), ("n_overhead_infos", C.c_uint64),
-                ("spans", C.POINTER(TraceSpan)), ("n_spans", C.c_uint64)]
+                ("spans", C.POINTER(TraceSpan)), ("n_spans", C.c_uint64),
+                ("collectives", C.POINTER(CollectiveMeta)), ("n_collectives", C.c_uint64)]
 
 
 class SynthParams(C.Structure):
@@ -169,7 +179,7 @@ def load_synth():
 
 ENGINE_SYMBOLS = [
     "ktj_create", "ktj_destroy", "ktj_last_error", "ktj_trace_start", "ktj_intern_strings",
-    "ktj_register_schema", "ktj_submit_args", "ktj_set_api_table", "ktj_set_clock_model",
+    "ktj_register_schema", "ktj_add_collective", "ktj_submit_args", "ktj_set_api_table", "ktj_set_clock_model",
     "ktj_set_window", "ktj_submit_records", "ktj_submit_records_device", "ktj_submit_info",
     "ktj_process", "ktj_output_device", "ktj_output_host", "ktj_finalize", "ktj_get_stats",
     "ktj_version",
@@ -196,6 +206,8 @@ def load_engine():
         lib.ktj_intern_strings.restype = C.c_int
         lib.ktj_intern_strings.argtypes = [vp, C.c_void_p, C.POINTER(C.c_uint64), C.c_size_t,
                                            C.POINTER(C.c_uint32)]
+        lib.ktj_add_collective.restype = C.c_int
+        lib.ktj_add_collective.argtypes = [vp, C.POINTER(CollectiveMeta), C.POINTER(C.c_uint32)]
         lib.ktj_register_schema.restype = C.c_int
         lib.ktj_register_schema.argtypes = [vp, C.POINTER(Field), C.c_size_t, C.POINTER(C.c_uint32)]
         lib.ktj_submit_args.restype = C.c_int

@@ -8,12 +8,14 @@
  */
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cerrno>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <string>
 #include <unistd.h>
+#include <utility>
 #include <vector>
 
 #include "../../include/ktj_debug.h"
@@ -103,6 +105,11 @@ struct ktj_engine {
   bool schemas_dirty = true;
   DevVec args;
   uint64_t n_args = 0;
+  std::vector<CollectiveInfo> collectives; /* ktj_add_collective entries */
+  bool coll_schemas = false;               /* a schema with a leading KTJ_F_COLLECTIVE field exists */
+  bool coll_dirty = true;
+  DevBuf d_coll_blob, d_coll_off, d_coll_first, cpu_row;
+  std::vector<uint32_t> coll_first;        /* read back: first use of each entry per backend */
   std::vector<uint32_t> cid_names, flow_bits;
   uint32_t malloc_cid = KTJ_NONE;
   DevBuf d_cid_names, d_flow_bits;
@@ -256,7 +263,8 @@ int ktj_register_schema(ktj_engine* e, const ktj_field* f, size_t n_fields, uint
   if (!e || (n_fields && !f)) return KTJ_ERR_ARG;
   if (n_fields > KTJ_MAX_SCHEMA_FIELDS) return KTJ_ERR_LIMIT;
   for (size_t i = 0; i < n_fields; ++i)
-    if (f[i].type > KTJ_F_I64_ARRAY || f[i].count == 0 || (f[i].type != KTJ_F_I64_ARRAY && f[i].count != 1)) return KTJ_ERR_ARG;
+    if (f[i].type > KTJ_F_COLLECTIVE || f[i].count == 0 || (f[i].type != KTJ_F_I64_ARRAY && f[i].count != 1)) return KTJ_ERR_ARG;
+  if (n_fields && f[0].type == KTJ_F_COLLECTIVE) e->coll_schemas = true;
   ktj_schema_desc d;
   d.first_field = (uint32_t)e->fields.size();
   d.n_fields = (uint32_t)n_fields;
@@ -264,6 +272,16 @@ int ktj_register_schema(ktj_engine* e, const ktj_field* f, size_t n_fields, uint
   if (schema_id) *schema_id = (uint32_t)e->schemas.size();
   e->schemas.push_back(d);
   e->schemas_dirty = true;
+  e->processed = false;
+  return KTJ_OK;
+}
+
+int ktj_add_collective(ktj_engine* e, const ktj_collective_meta* meta, uint32_t* index) {
+  if (!e || !meta) return KTJ_ERR_ARG;
+  if (e->collectives.size() >= 0x7FFFFFFEull) return KTJ_ERR_LIMIT;
+  if (index) *index = (uint32_t)e->collectives.size();
+  e->collectives.push_back(make_collective(*meta));
+  e->coll_dirty = true;
   e->processed = false;
   return KTJ_OK;
 }
@@ -454,6 +472,25 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   ctx.n_schemas = (uint32_t)e->schemas.size();
   ctx.args = e->args.buf.as<uint64_t>(); ctx.n_args = e->n_args;
   ctx.base_time_ns = e->base_time_ns;
+  /* collective metadata is looked at only if both entries and a schema that refers to them exist */
+  const uint32_t n_coll = e->coll_schemas ? (uint32_t)e->collectives.size() : 0u;
+  if (n_coll && e->coll_dirty) {
+    std::string blob;
+    std::vector<uint64_t> off(e->collectives.size() + 1, 0);
+    for (size_t k = 0; k < e->collectives.size(); ++k) { blob += e->collectives[k].args; off[k + 1] = blob.size(); }
+    blob.append(16, '\0'); /* string copies load whole aligned words */
+    int rc = upload_small(e, e->d_coll_blob, blob.data(), blob.size());
+    if (rc == KTJ_OK) rc = upload_small(e, e->d_coll_off, off.data(), off.size() * 8);
+    if (rc != KTJ_OK) return rc;
+    e->coll_dirty = false;
+  }
+  ctx.coll_blob = e->d_coll_blob.as<char>(); ctx.coll_off = e->d_coll_off.as<uint64_t>(); ctx.n_coll = n_coll;
+  uint32_t* cpu_row = nullptr;
+  if (n_coll) {
+    HIPCHK(e->cpu_row.ensure((cap_cpu + 1ull) * 4)); HIPCHK(e->d_coll_first.ensure(2ull * n_coll * 4));
+    cpu_row = e->cpu_row.as<uint32_t>();
+    HIPCHK(fill_u32(cpu_row, 0, cap_cpu + 1ull, st));
+  }
   if (ns) {
     HIPCHK(dict_measure(e->str_blob.buf.as<char>(), e->str_off.buf.as<uint64_t>(), ns, e->d_name_len.as<uint32_t>(),
                         e->d_arg_len.as<uint32_t>(), e->d_sflags.as<uint32_t>(), st));
@@ -496,10 +533,10 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   ApiTable api{e->d_cid_names.as<uint32_t>(), (uint32_t)e->cid_names.size(), e->d_flow_bits.as<uint32_t>(), e->malloc_cid};
   MatRow* mat = e->mat.as<MatRow>();
   HIPCHK(build_extcorr(x_recs, nx, tn, nc, e->slot_ext.as<uint32_t>(), sc, st));
-  HIPCHK(build_cpu_ids(g_recs, ng, t_cpu, sc, st));
+  HIPCHK(build_cpu_ids(g_recs, ng, t_cpu, cpu_row, sc, st));
   HIPCHK(build_runtime(nr, c, ng, tf, fc, tn, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), sc, st));
   HIPCHK(insert_device_first(nd, c, ng + nr, tf, fc, e->slot_f_dev.as<uint32_t>(), sc, st));
-  HIPCHK(resolve_external(x_recs, nx, nc, e->slot_ext.as<uint32_t>(), t_cpu, st));
+  HIPCHK(resolve_external(x_recs, nx, nc, e->slot_ext.as<uint32_t>(), t_cpu, cpu_row, g_recs, ctx, st));
   /* second pass over the runtime rows: publishes into the tables and writes the joined rows */
   HIPCHK(mat_runtime_rows(r_recs, nr, c, ng, api, fc, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), ctx, mat,
                           e->len.as<uint32_t>(), sc, st));
@@ -565,6 +602,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(mat_generic_rows(g_recs, ng, ctx, sync_first, mat, e->len.as<uint32_t>(), sc, st));
   HIPCHK(mat_device_rows(d_recs, nd, c, ng + nr, e->dev_link.as<DevLink>(), ctx, mat, e->len.as<uint32_t>(), sc, st));
   HIPCHK(gather_len(e->perm, e->len.as<uint32_t>(), N, e->len_sorted.as<uint32_t>(), st));
+  if (n_coll) HIPCHK(collective_first(mat, e->perm, e->scalars.n_valid, n_coll, e->d_coll_first.as<uint32_t>(), st));
   HIPCHK(hipEventRecord(e->ev[EV_SIZE], st));
 
   /* ---- scan ---- */
@@ -573,16 +611,28 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   uint64_t act_bytes = 0;
   HIPCHK(hipMemcpyAsync(&act_bytes, e->offs.as<uint64_t>() + N, 8, hipMemcpyDeviceToHost, st));
   HIPCHK(hipMemcpyAsync(&e->scalars, sc, sizeof(Scalars), hipMemcpyDeviceToHost, st));
+  e->coll_first.assign(2ull * n_coll, 0xFFFFFFFFu);
+  if (n_coll) HIPCHK(hipMemcpyAsync(e->coll_first.data(), e->d_coll_first.p, 2ull * n_coll * 4, hipMemcpyDeviceToHost, st));
   HIPCHK(hipStreamSynchronize(st));
   if (e->scalars.error) {
     e->last_error = "device-side limit hit, error bits " + std::to_string(e->scalars.error);
     return KTJ_ERR_LIMIT;
   }
+  std::string distributed_info;
+  if (n_coll) { /* the uses in emission order: one per entry and backend is enough, later ones repeat it */
+    std::vector<std::pair<uint32_t, uint32_t>> firsts; /* (position, 2 * index + hccl) */
+    for (uint32_t k = 0; k < 2u * n_coll; ++k)
+      if (e->coll_first[k] != 0xFFFFFFFFu) firsts.emplace_back(e->coll_first[k], k);
+    std::sort(firsts.begin(), firsts.end());
+    std::vector<CollectiveUse> uses;
+    for (const auto& f : firsts) uses.push_back(CollectiveUse{f.second >> 1, (f.second & 1u) != 0});
+    distributed_info = distributed_info_text(e->collectives, uses);
+  }
 
   /* ---- emit ---- */
   std::string prefix = e->txt_header + e->txt_dev + e->txt_res + e->txt_ovh;
   std::string suffix = e->txt_span;
-  append_trace_end(suffix, end_time_ns, e->base_time_ns, e->out_path);
+  append_trace_end(suffix, end_time_ns, e->base_time_ns, e->out_path, distributed_info);
   e->prefix_len = prefix.size();
   e->act_bytes = act_bytes;
   e->total_bytes = prefix.size() + act_bytes + suffix.size();

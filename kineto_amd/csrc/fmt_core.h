@@ -742,20 +742,63 @@ template <class W> KTJ_HD KTJ_FI inline void put_copy_kind(W& w, uint32_t op) {
   }
 }
 
+/* a leading KTJ_F_COLLECTIVE field refers to collective metadata and is no part of the fragment */
+KTJ_HD KTJ_FI inline uint32_t leading_collective(const ktj_schema_desc& sd, const EmitCtx& c) {
+  return sd.n_fields != 0 && c.fields[sd.first_field].type == KTJ_F_COLLECTIVE ? 1u : 0u;
+}
 /* does this row print a metadata fragment?  (ArgsBuilder::appendFragment, output_json.cpp:173-181) */
 KTJ_HD KTJ_FI inline bool has_fragment(const MatRow& r, const EmitCtx& c) {
   const uint32_t cls = (r.meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT;
   if (cls != KTJ_CLASS_GENERIC) return true;
   if (r.aux >= c.n_schemas) return false;
   const ktj_schema_desc sd = c.schemas[r.aux];
-  if (sd.n_fields == 0) return false;
-  if (sd.n_fields == 1 && c.fields[sd.first_field].key_id == KTJ_NONE &&
-      c.fields[sd.first_field].type == KTJ_F_RAW) { /* a whole pre-rendered fragment */
-    if (r.p[0] >= c.n_args) return false;
-    const uint32_t id = (uint32_t)c.args[r.p[0]];
+  const uint32_t skip = leading_collective(sd, c);
+  if (sd.n_fields == skip) return false;
+  if (sd.n_fields == skip + 1 && c.fields[sd.first_field + skip].key_id == KTJ_NONE &&
+      c.fields[sd.first_field + skip].type == KTJ_F_RAW) { /* a whole pre-rendered fragment */
+    if (r.p[0] + skip >= c.n_args) return false;
+    const uint32_t id = (uint32_t)c.args[r.p[0] + skip];
     return id < c.dict.n && (c.dict.flags[id] & KTJ_SF_ARG_BLANK) == 0;
   }
   return true;
+}
+/* 1 + index of the collective metadata this row carries (appendCollectiveMetadata,
+ * output_json.cpp:899-908), 0 = none */
+KTJ_HD KTJ_FI inline uint32_t collective_of(const MatRow& r) {
+  const uint32_t cls = (r.meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT;
+  if (cls == KTJ_CLASS_GENERIC) return (uint32_t)r.p[1];
+  if (cls == KTJ_CLASS_DEVICE && (r.meta & KTJ_M_TYPE_MASK) == KTJ_TYPE_CONCURRENT_KERNEL) return (uint32_t)r.p[4];
+  return 0;
+}
+/* does the row append collective arguments?  An op without any of the keys appends nothing. */
+KTJ_HD KTJ_FI inline bool has_collective_args(const MatRow& r, const EmitCtx& c) {
+  const uint32_t k = collective_of(r);
+  return k != 0 && k <= c.n_coll && c.coll_off[k] != c.coll_off[k - 1];
+}
+/* does the complete event of this row print an args object? */
+KTJ_HD KTJ_FI inline bool has_args(const MatRow& r, const EmitCtx& c) {
+  return r.ext != 0 || has_fragment(r, c) || has_collective_args(r, c);
+}
+/* Generic rows: a record with a linked op and a leading KTJ_F_COLLECTIVE field prints that
+ * collective metadata itself if it is a kernel, or an MTIA event named "hccl::..."
+ * (output_json.cpp:899-908). */
+KTJ_HD KTJ_FI inline void attach_own_collective(MatRow& m, const ktj_generic_rec& g, const EmitCtx& c) {
+  if (c.n_coll == 0 || !(g.flags & KTJ_GF_LINKED)) return;
+  if (g.type == KTJ_TYPE_MTIA_CCP_EVENTS) {
+    if (g.name_id >= c.dict.n || c.dict.raw_off[g.name_id + 1] - c.dict.raw_off[g.name_id] < 6) return;
+    const char* nm = c.dict.raw_blob + c.dict.raw_off[g.name_id];
+    if (nm[0] != 'h' || nm[1] != 'c' || nm[2] != 'c' || nm[3] != 'l' || nm[4] != ':' || nm[5] != ':') return;
+  } else if (g.type != KTJ_TYPE_CONCURRENT_KERNEL) return;
+  if (g.schema_id >= c.n_schemas || !leading_collective(c.schemas[g.schema_id], c) || g.args_off >= c.n_args) return;
+  const uint64_t k = c.args[g.args_off];
+  if (k < c.n_coll) m.p[1] = k + 1;
+}
+/* Generic rows other than those: the collective metadata handed to the kernels linked to them. */
+KTJ_HD KTJ_FI inline uint32_t collective_for_linked(const ktj_generic_rec& g, const EmitCtx& c) {
+  if (c.n_coll == 0 || g.type == KTJ_TYPE_CONCURRENT_KERNEL || g.type == KTJ_TYPE_MTIA_CCP_EVENTS) return 0;
+  if (g.schema_id >= c.n_schemas || !leading_collective(c.schemas[g.schema_id], c) || g.args_off >= c.n_args) return 0;
+  const uint64_t k = c.args[g.args_off];
+  return k < c.n_coll ? (uint32_t)k + 1u : 0u;
 }
 
 /* the metadataJson() fragment, after sanitizeStrForJSON (raw: as metadataJson() returned it) */
@@ -768,6 +811,7 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
     bool first = true;
     for (uint32_t f = 0; f < sd.n_fields; ++f) {
       const ktj_field fd = c.fields[sd.first_field + f];
+      if (fd.type == KTJ_F_COLLECTIVE) { slot += fd.count; continue; }
       if (fd.key_id != KTJ_NONE) {
         if (!first) KTJ_PUT(w, ", ");
         first = false;
@@ -883,9 +927,14 @@ KTJ_HD KTJ_FI inline void mark_stream_sync(MatRow& m, const EmitCtx& c, bool fir
   m.meta |= KTJ_M_SYNC;
   if (first_of_row) m.meta |= KTJ_M_SYNC_FIRST;
 }
+/* resource + kSyncStreamTidOffset (output_json.cpp:916); a resource id near INT64_MAX wraps, as the
+ * logger's own addition does on the machines it runs on */
+KTJ_HD KTJ_FI inline int64_t sync_row_tid(int64_t resource) {
+  return (int64_t)((uint64_t)resource + (uint64_t)KTJ_SYNC_TID_OFFSET);
+}
 /* (device << 32) | virtual tid, the key of syncStreamMetadataEmitted_ (output_json.cpp:917) */
 KTJ_HD KTJ_FI inline uint64_t stream_sync_key(int64_t device, int64_t resource) {
-  return ((uint64_t)device << 32) | (uint64_t)(resource + KTJ_SYNC_TID_OFFSET);
+  return ((uint64_t)device << 32) | (uint64_t)sync_row_tid(resource);
 }
 
 /* handleGenericInstantEvent + writeInstantEvent (output_json.cpp:660-677, 261-292): name and
@@ -982,7 +1031,7 @@ template <class W> KTJ_HD KTJ_FI inline void format_activity(W& w, const MatRow&
   int64_t rel = ts - c.base_time_ns;                         /* transToRelativeTime :144-153 */
   if (rel < 0) rel = 0;
   /* Stream Sync activities sit on a row of their own (output_json.cpp:913-943, 1008-1013) */
-  const int64_t tid = sanitize_tid((r.meta & KTJ_M_SYNC) ? r.res + KTJ_SYNC_TID_OFFSET : r.res);
+  const int64_t tid = sanitize_tid((r.meta & KTJ_M_SYNC) ? sync_row_tid(r.res) : r.res);
   const bool flow = (r.meta & KTJ_M_FLOW) != 0;
   /* pid and tid are printed again by the flow event */
   const bool pid_neg = r.dev < 0;
@@ -990,10 +1039,10 @@ template <class W> KTJ_HD KTJ_FI inline void format_activity(W& w, const MatRow&
   const typename W::Prepared tidn = W::prepare((uint64_t)tid);
   if (r.meta & KTJ_M_SYNC_FIRST) { /* the row is announced once, before its first activity */
     KTJ_PUT(w, "\n  {\n    \"name\": \"thread_name\", \"ph\": \"M\", \"ts\": "); put_ts(w, rel);
-    KTJ_PUT(w, ", \"pid\": "); put_i64(w, r.dev); KTJ_PUT(w, ", \"tid\": "); put_i64(w, r.res + KTJ_SYNC_TID_OFFSET);
+    KTJ_PUT(w, ", \"pid\": "); put_i64(w, r.dev); KTJ_PUT(w, ", \"tid\": "); put_i64(w, sync_row_tid(r.res));
     KTJ_PUT(w, ",\n    \"args\": {\n      \"name\": \"stream "); put_i64(w, r.res); KTJ_PUT(w, " (sync)\"\n    }\n  },");
     KTJ_PUT(w, "\n  {\n    \"name\": \"thread_sort_index\", \"ph\": \"M\", \"ts\": "); put_ts(w, rel);
-    KTJ_PUT(w, ", \"pid\": "); put_i64(w, r.dev); KTJ_PUT(w, ", \"tid\": "); put_i64(w, r.res + KTJ_SYNC_TID_OFFSET);
+    KTJ_PUT(w, ", \"pid\": "); put_i64(w, r.dev); KTJ_PUT(w, ", \"tid\": "); put_i64(w, sync_row_tid(r.res));
     KTJ_PUT(w, ",\n    \"args\": {\n      \"sort_index\": "); put_i64(w, r.res); KTJ_PUT(w, "\n    }\n  },");
   }
   KTJ_PUT(w, "\n  {\n    \"ph\": \"X\",\n    \"cat\": \"");
@@ -1005,10 +1054,16 @@ template <class W> KTJ_HD KTJ_FI inline void format_activity(W& w, const MatRow&
   KTJ_PUT(w, ",\n    \"ts\": "); put_ts(w, rel);
   KTJ_PUT(w, ",\n    \"dur\": "); put_ts(w, dur);
   const bool frag = has_fragment(r, c);
-  if (r.ext != 0 || frag) {                                  /* ArgsBuilder :157-212 */
+  const bool coll = has_collective_args(r, c);
+  if (r.ext != 0 || frag || coll) {                          /* ArgsBuilder :157-212 */
     KTJ_PUT(w, "\n    ,\n    \"args\": {\n      ");
     if (r.ext != 0) { KTJ_PUT(w, "\"External id\": "); put_i64(w, r.ext); }
     if (frag) { if (r.ext != 0) w.ch(','); put_fragment(w, r, c); }
+    if (coll) { /* appendCollectiveMetadata :899-908: printed as the op's values were handed over */
+      if (r.ext != 0 || frag) w.ch(',');
+      const uint32_t k = collective_of(r);
+      w.str(c.coll_blob + c.coll_off[k - 1], c.coll_off[k] - c.coll_off[k - 1]);
+    }
     KTJ_PUT(w, "\n    }\n  },");
   } else KTJ_PUT(w, "\n    \n  },");
   if (flow) {                                                /* :960-1021, writeFlowEvent :318-345 */

@@ -58,7 +58,7 @@ struct NarrowPay {         /* two writers, each with whole 8-byte words of its o
   int32_t ext_val;         /* external id if a CPU op with that id exists, else 0               */
   uint32_t linked;         /* 1 when ext_val names an existing CPU op                           */
   uint32_t kind;           /* KTJ_DL_*: what pay[] holds                                        */
-  uint32_t pad;
+  uint32_t coll;           /* 1 + index of the collective metadata of the linked CPU op, 0 = none */
   uint64_t pay[3];         /* bytes of the winning copy / malloc row in pay[0], or packed grid /
                               workgroup of the winning kernel-launch row (see pack_grid)        */
 };                         /* 40 bytes */
@@ -79,7 +79,7 @@ struct JoinPlan {
 struct DevLink {
   uint64_t p[3];           /* size in p[0], or packed grid / workgroup */
   uint32_t flags;          /* KTJ_DL_* */
-  uint32_t pad;
+  uint32_t coll;           /* 1 + index of the collective metadata of the linked CPU op (kernels) */
 };                         /* 32 bytes */
 /* the fields of a device row that the stream back-fill passes read */
 struct DevBrief {
@@ -173,13 +173,15 @@ hipError_t plan_tables(Columns c, uint64_t n_generic, uint64_t n_runtime, uint64
 hipError_t clear_tables(Table tf, FullCols fc, Table tn, NarrowCols nc, Table cpu, hipStream_t st);
 hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, uint32_t* slot_ext, Scalars* sc,
                          hipStream_t st);
-hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, Scalars* sc, hipStream_t st);
+hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, uint32_t* cpu_row, Scalars* sc, hipStream_t st);
 /* the build passes read the columns only (correlation id, kind and has-stream bits of meta) */
 hipError_t build_runtime(uint64_t n, Columns c, uint64_t first_runtime, Table tf, FullCols fc, Table tn, NarrowCols nc,
                          uint32_t* slot_f, uint32_t* slot_n, Scalars* sc, hipStream_t st);
 hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, uint32_t* slot_f_dev,
                                Scalars* sc, hipStream_t st);
 hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
+                            const uint32_t* cpu_row, const ktj_generic_rec* g, EmitCtx ctx, hipStream_t st);
+hipError_t collective_first(const MatRow* mat, const uint32_t* perm, uint64_t n_rows, uint32_t n_coll, uint32_t* first,
                             hipStream_t st);
 /* per device row: "External id", timestamp-order check, stream of the launching row, and the
  * size / grid hand-over (into link[]) */

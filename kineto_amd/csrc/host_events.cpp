@@ -1,6 +1,8 @@
 /* host_events.cpp — see host_events.h.  Plain host C++; one std::string append per piece. */
 #include "host_events.h"
 
+#include <unordered_map>
+
 #include <cstdint>
 #include <cstdlib>
 
@@ -135,12 +137,98 @@ void append_trace_span(std::string& out, const ktj_trace_span& sp, int64_t base)
   out += "\n    \n  },";
 }
 
-void append_trace_end(std::string& out, int64_t end_time_ns, int64_t base, const std::string& file_name) {
+void append_trace_end(std::string& out, int64_t end_time_ns, int64_t base, const std::string& file_name,
+                      const std::string& distributed_info) {
   out += "\n  {\n    \"ph\": \"i\",\n    \n    \"s\": \"g\",\n    \"name\": \"Record Window End\",\n    \"pid\": \"\",\n    \"tid\": \"\",\n    \"ts\": ";
   out += fmt_ts(rel_time(end_time_ns, base));
   out += "\n    \n  }";
   out += "\n  ],";
+  out += distributed_info;
   out += "\"traceName\": \"" + sanitize_only(file_name.c_str()) + "\" }";
+}
+
+namespace {
+std::string value_of(const char* p) { return p ? std::string(p) : std::string(); }
+/* stripQuotes (output_json.cpp:57-63): one surrounding pair of double quotes goes */
+std::string unquoted(const char* p) {
+  std::string v = value_of(p);
+  if (v.size() >= 2 && v.front() == '"' && v.back() == '"') v = v.substr(1, v.size() - 2);
+  return v;
+}
+struct ArgList { /* ArgsBuilder (output_json.cpp:157-212): entries joined by a bare comma */
+  std::string text;
+  void raw(const char* key, const std::string& v) {
+    if (!text.empty()) text += ',';
+    text += '"'; text += key; text += "\": "; text += v;
+  }
+  void quoted(const char* key, const std::string& v) { raw(key, '"' + v + '"'); }
+};
+}  // namespace
+
+CollectiveInfo make_collective(const ktj_collective_meta& m) {
+  CollectiveInfo c;
+  ArgList a;
+  const std::string name = unquoted(m.collective_name), dtype = unquoted(m.dtype);
+  const std::string in_n = value_of(m.in_msg_nelems), out_n = value_of(m.out_msg_nelems), group = value_of(m.group_size);
+  if (!name.empty() && !in_n.empty() && !out_n.empty() && !group.empty() && !dtype.empty()) { /* all five or none: :731-738 */
+    a.quoted("Collective name", name);
+    a.raw("In msg nelems", in_n);
+    a.raw("Out msg nelems", out_n);
+    a.raw("Group size", group);
+    a.quoted("dtype", dtype);
+  }
+  const std::string in_start = unquoted(m.in_tensors_start), out_start = unquoted(m.out_tensors_start);
+  if (!in_start.empty()) a.quoted("Input Tensors start", in_start);
+  if (!out_start.empty()) a.quoted("Output Tensors start", out_start);
+  const std::string in_split = unquoted(m.in_split), out_split = unquoted(m.out_split);
+  if (!in_split.empty() && !out_split.empty()) { /* all_to_all only, both or none: :752-759 */
+    a.quoted("In split size", in_split);
+    a.quoted("Out split size", out_split);
+  }
+  c.pg_name = unquoted(m.pg_name);
+  c.pg_desc = unquoted(m.pg_desc);
+  c.ranks = unquoted(m.group_ranks);
+  c.group_size = group;
+  c.rank = value_of(m.rank);
+  if (!c.pg_name.empty()) a.quoted("Process Group Name", c.pg_name);
+  if (!c.pg_desc.empty()) a.quoted("Process Group Description", c.pg_desc);
+  if (!c.ranks.empty()) a.quoted("Process Group Ranks", c.ranks);
+  const std::string dst = value_of(m.dst_rank), src = value_of(m.src_rank), seq = value_of(m.seq), comms = value_of(m.comms_id);
+  if (!dst.empty()) a.raw("Dst Rank", dst);
+  if (!src.empty()) a.raw("Src Rank", src);
+  if (!seq.empty()) a.raw("Seq", seq);
+  if (!comms.empty()) a.raw("Comms Id", comms);
+  c.args = std::move(a.text);
+  return c;
+}
+
+std::string distributed_info_text(const std::vector<CollectiveInfo>& collectives, const std::vector<CollectiveUse>& uses) {
+  struct Group { std::string desc, backend_config, size, ranks; };
+  std::unordered_map<std::string, Group> groups; /* pgMap_ (output_json.h:233): the first entry of a name stays */
+  std::string backend, rank, world_size, nccl_version;
+  for (const CollectiveUse& u : uses) {
+    if (u.index >= collectives.size()) continue;
+    const CollectiveInfo& c = collectives[u.index];
+    if (backend.empty() && c.pg_desc == "default_pg") { /* :807-817 */
+      backend = u.hccl ? "hccl" : "nccl";
+      rank = c.rank;
+      world_size = c.group_size;
+      nccl_version = u.hccl ? "" : "unknown";
+    }
+    groups.insert({c.pg_name, Group{c.pg_desc, u.hccl ? "mtia:hccl" : "cuda:nccl", c.group_size, c.ranks}});
+  }
+  if (backend.empty()) return std::string();
+  std::string out = "\n  \"distributedInfo\": {\"backend\": \"" + backend + "\", \"rank\": " + rank + ", \"world_size\": " +
+                    world_size + ", \"pg_count\": " + std::to_string(groups.size()) + ", \"pg_config\": [";
+  bool first = true;
+  for (const auto& g : groups) {
+    if (!first) out += ',';
+    first = false;
+    out += "{\"pg_name\": \"" + g.first + "\", \"pg_desc\": \"" + g.second.desc + "\", \"backend_config\": \"" +
+           g.second.backend_config + "\", \"pg_size\": " + g.second.size + ", \"ranks\": \"" + g.second.ranks + "\"}";
+  }
+  out += "], \"nccl_version\": \"" + nccl_version + "\"},";
+  return out;
 }
 
 }  // namespace ktj

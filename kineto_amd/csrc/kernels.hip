@@ -566,7 +566,7 @@ __global__ void k_clear_full(Table t, FullCols c) {
 }
 __global__ void k_clear_narrow(Table t, NarrowCols c) {
   const uint64_t n = table_extent(t);
-  NarrowPay z; z.ext_val = 0; z.linked = 0; z.kind = 0; z.pad = 0; z.pay[0] = z.pay[1] = z.pay[2] = 0;
+  NarrowPay z; z.ext_val = 0; z.linked = 0; z.kind = 0; z.coll = 0; z.pay[0] = z.pay[1] = z.pay[2] = 0;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i <= n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t k = i < n ? i : t.mask + 1ull;
     c.ext_src[k] = 0; c.kern_src[k] = 0; c.copy_src[k] = 0; c.pay[k] = z;
@@ -612,10 +612,14 @@ __global__ void k_build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, 
   atomicMax(&nc.ext_src[slot], (uint32_t)i + 1u);
 }
 /* activityMap_[act->correlationId()] = act: GenericActivityProfiler.cpp:262 */
-__global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, Scalars* sc) {
+/* cpu_row (optional): per slot, 1 + index of the last record with that id, for the traces whose
+ * CPU ops hand collective metadata to the kernels linked to them */
+__global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, uint32_t* cpu_row, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  if (slot_insert(cpu, (uint64_t)(int64_t)g[i].id) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+  const uint32_t slot = slot_insert(cpu, (uint64_t)(int64_t)g[i].id);
+  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
+  if (cpu_row) atomicMax(&cpu_row[slot], (uint32_t)i + 1u);
 }
 /* full table : correlation id → stream_src = last runtime row that carries a stream
  *              (RocmStreamQueue.h:47-54), first = first arrival index seen, for checkTimestampOrder
@@ -677,15 +681,21 @@ __global__ void k_insert_device_first(uint64_t n, Columns c, uint64_t first_devi
 }
 /* linkedActivity(): GenericActivityProfiler.cpp:397-408.  The record that won the slot resolves
  * its external id against the CPU-op ids once, for every row that will read the slot. */
-__global__ void k_resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu) {
+__global__ void k_resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
+                                   const uint32_t* cpu_row, const ktj_generic_rec* g, EmitCtx ctx) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const uint32_t slot = slot_ext[i];
   if (slot == KTJ_NOSLOT || nc.ext_src[slot] != (uint32_t)i + 1u) return;
   const uint64_t ext_id = e[i].external_id;
-  if (slot_find(cpu, ext_id) != KTJ_NOSLOT) {
+  const uint32_t cs = slot_find(cpu, ext_id);
+  if (cs != KTJ_NOSLOT) {
     nc.pay[slot].ext_val = (int32_t)(int64_t)ext_id;
     nc.pay[slot].linked = 1u;
+    if (cpu_row) { /* the linked op is the last record with that id (activityMap_, GenericActivityProfiler.cpp:262) */
+      const uint32_t row = cpu_row[cs];
+      if (row) nc.pay[slot].coll = collective_for_linked(g[row - 1], ctx);
+    }
   }
 }
 __device__ __forceinline__ bool is_async_op(uint32_t domain) { return domain != KTJ_DOM_MEMSET; }
@@ -706,7 +716,7 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Full
     const uint32_t domain = (meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
     const bool valid = (meta & KTJ_M_VALID) != 0;
     DevLink l;
-    l.p[0] = l.p[1] = l.p[2] = 0; l.flags = 0; l.pad = 0;
+    l.p[0] = l.p[1] = l.p[2] = 0; l.flags = 0; l.coll = 0;
     int32_t ext = 0;
     const uint32_t sn = slot_find(tn, narrow_corr_key(id));
     if (sn != KTJ_NOSLOT) {
@@ -717,6 +727,7 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Full
         l.flags = np.kind;
         l.p[0] = np.pay[0]; l.p[1] = np.pay[1]; l.p[2] = np.pay[2];
       }
+      l.coll = np.coll;
     }
     c.ext[a] = ext;
     link[i] = l;
@@ -750,9 +761,9 @@ hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowC
   hipLaunchKernelGGL(k_build_extcorr, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, tn, nc, slot_ext, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, Scalars* sc, hipStream_t st) {
+hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, uint32_t* cpu_row, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_build_cpu_ids, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, cpu, sc);
+  hipLaunchKernelGGL(k_build_cpu_ids, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, cpu, cpu_row, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t build_runtime(uint64_t n, Columns c, uint64_t first_runtime, Table tf, FullCols fc, Table tn, NarrowCols nc,
@@ -770,9 +781,10 @@ hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, Tab
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
-                            hipStream_t st) {
+                            const uint32_t* cpu_row, const ktj_generic_rec* g, EmitCtx ctx, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_resolve_external, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, nc, slot_ext, cpu);
+  hipLaunchKernelGGL(k_resolve_external, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, nc, slot_ext, cpu, cpu_row,
+                     g, ctx);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, FullCols fc, Table tn, NarrowCols nc,
@@ -1242,7 +1254,7 @@ __device__ __forceinline__ uint32_t row_length(const MatRow& m, const EmitCtx& c
   CountWriter cw;
   format_activity(cw, m, ctx);
   if (cw.n >= (1ull << 30)) { flag_error(sc, KTJ_DEVERR_RECORD_TOO_LONG); return 0; }
-  return (uint32_t)cw.n | (tail_kind(m, m.ext != 0 || has_fragment(m, ctx)) << 30);
+  return (uint32_t)cw.n | (tail_kind(m, has_args(m, ctx)) << 30);
 }
 struct RowStats { uint32_t n_flow = 0, n_blank = 0; };
 __device__ __forceinline__ void count_row_stats(const MatRow& m, const EmitCtx& ctx, RowStats* rs) {
@@ -1310,6 +1322,7 @@ __global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx,
     const ktj_generic_rec rec = g[i];
     MatRow m = mat_generic(rec);
     if (!generic_record_prints(rec, ctx)) m.meta &= ~KTJ_M_VALID;
+    attach_own_collective(m, rec, ctx);
     mark_stream_sync(m, ctx, sync_first != nullptr && sync_first[i] != 0);
     store_row(&mat[i], m);
     len[i] = row_length(m, ctx, sc);
@@ -1376,12 +1389,36 @@ __global__ void k_mat_device(const ktj_device_rec* d, uint64_t n, Columns c, uin
     const ktj_device_rec rec = d[i];
     const DevLink l = link[i];
     const MatRow m = mat_device(rec, c.ts[a], c.dur[a], c.res[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a],
-                                (l.flags & KTJ_DL_HAS_GRID) ? l.p : nullptr, (l.flags & KTJ_DL_HAS_SIZE) != 0, l.p[0]);
+                                (l.flags & KTJ_DL_HAS_GRID) ? l.p : nullptr, (l.flags & KTJ_DL_HAS_SIZE) != 0, l.p[0], l.coll);
     store_row(&mat[a], m);
     len[a] = row_length(m, ctx, sc);
     count_row_stats(m, ctx, &rs);
   }
   flush_row_stats(rs, sc);
+}
+/* Collective metadata: the first activity, in emission order, that prints each entry, per
+ * backend (first[2k] nccl, first[2k + 1] hccl).  The host replays appendCollectiveMetadata's
+ * bookkeeping (output_json.cpp:799-835) over these.  Runs only for traces that carry any. */
+__global__ void k_collective_first(const MatRow* mat, const uint32_t* perm, uint64_t n_rows, uint32_t n_coll, uint32_t* first) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_rows) return;
+  const MatRow* m = &mat[perm[i]];
+  const uint32_t meta = m->meta;
+  const uint32_t cls = (meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT;
+  uint32_t k = 0;
+  if (cls == KTJ_CLASS_GENERIC) k = (uint32_t)m->p[1];
+  else if (cls == KTJ_CLASS_DEVICE && (meta & KTJ_M_TYPE_MASK) == KTJ_TYPE_CONCURRENT_KERNEL) k = (uint32_t)m->p[4];
+  if (k == 0 || k > n_coll) return;
+  const uint32_t hccl = cls == KTJ_CLASS_GENERIC && (meta & KTJ_M_TYPE_MASK) == KTJ_TYPE_MTIA_CCP_EVENTS ? 1u : 0u;
+  atomicMin(&first[2u * (k - 1u) + hccl], (uint32_t)i);
+}
+hipError_t collective_first(const MatRow* mat, const uint32_t* perm, uint64_t n_rows, uint32_t n_coll, uint32_t* first,
+                            hipStream_t st) {
+  hipError_t e = fill_u32(first, 0xFFFFFFFFu, 2ull * n_coll, st);
+  if (e != hipSuccess || n_rows == 0) return e;
+  hipLaunchKernelGGL(k_collective_first, dim3(grid_for(n_rows, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, mat, perm, n_rows, n_coll,
+                     first);
+  return KTJ_LAUNCH_CHECK();
 }
 __global__ void k_gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;

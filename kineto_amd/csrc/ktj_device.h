@@ -29,12 +29,13 @@ struct MatRow {
   uint64_t p[5];     /* payload, see below                                                      */
 };
 /* payload by class:
- *   generic          p0 = args_off
+ *   generic          p0 = args_off, p1 = 1 + index of the collective metadata the row prints (0 = none)
  *   runtime KERNEL   p0 = grid0 | grid1<<32, p1 = grid2 | wg0<<32, p2 = wg1 | wg2<<32, p3 = group
  *                    segment size, p4 = kernel_name_id
  *   runtime COPY     p0 = src, p1 = dst, p2 = size, p3 = copy_kind
  *   runtime MALLOC   p0 = ptr, p1 = size
- *   device kernel    p0..p2 = grid/block of the launching row (if KTJ_M_HAS_GRID), p3 = queue
+ *   device kernel    p0..p2 = grid/block of the launching row (if KTJ_M_HAS_GRID), p3 = queue,
+ *                    p4 = 1 + index of the collective metadata of the linked CPU op (0 = none)
  *   device copy      p0 = bytes of the launching row (if KTJ_M_HAS_SIZE), p3 = queue
  *   device memset    p0 = bytes, p3 = context id
  */
@@ -93,6 +94,9 @@ struct EmitCtx {
   const uint64_t* args;             /* 8-byte slots                                            */
   uint64_t n_args;
   int64_t base_time_ns;
+  const char* coll_blob;            /* collective arguments of each ktj_add_collective entry   */
+  const uint64_t* coll_off;         /* n_coll + 1                                              */
+  uint32_t n_coll;
 };
 
 #endif

@@ -131,8 +131,9 @@ KTJ_HD inline MatRow mat_runtime(const ktj_runtime_rec& r, int64_t ts, int64_t d
 
 /* res: resourceId() after stream back-fill.  grid: packed grid and block of the launching kernel
  * row that the reference hands over (null = none); size: bytes handed over by a copy/malloc row. */
+/* coll: 1 + index of the collective metadata of the linked CPU op, 0 = none (kernels only) */
 KTJ_HD inline MatRow mat_device(const ktj_device_rec& d, int64_t ts, int64_t dur, int64_t res, bool valid,
-                                int32_t ext, const uint64_t* grid, bool has_size, uint64_t size) {
+                                int32_t ext, const uint64_t* grid, bool has_size, uint64_t size, uint32_t coll = 0) {
   MatRow m;
   m.ts = ts; m.dur = dur; m.dev = (int64_t)d.device; m.res = res;
   m.flow_id = (int64_t)d.id;
@@ -160,6 +161,7 @@ KTJ_HD inline MatRow mat_device(const ktj_device_rec& d, int64_t ts, int64_t dur
       meta |= KTJ_M_HAS_GRID;
       m.p[0] = grid[0]; m.p[1] = grid[1]; m.p[2] = grid[2];
     }
+    if (dom == KTJ_DOM_KERNEL_DISPATCH) m.p[4] = coll;
   }
   m.meta = meta;
   return m;

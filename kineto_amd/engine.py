@@ -50,6 +50,8 @@ class TraceEngine:
             sid = C.c_uint32()
             fptr = C.cast(C.addressof(s.fields.contents) + d.first_field * C.sizeof(abi.Field), C.POINTER(abi.Field))
             self._chk(lib.ktj_register_schema(h, fptr, d.n_fields, C.byref(sid)), "ktj_register_schema")
+        for i in range(s.n_collectives):
+            self._chk(lib.ktj_add_collective(h, C.byref(s.collectives[i]), None), "ktj_add_collective")
         slot0 = C.c_uint64()
         self._chk(lib.ktj_submit_args(h, s.args, s.n_args, C.byref(slot0)), "ktj_submit_args")
         self._chk(lib.ktj_set_api_table(h, s.cid_name_ids, s.n_cids, s.flow_start_cids, s.n_flow_start, s.malloc_cid),

@@ -39,6 +39,9 @@ GpuChromeTraceLogger::GpuChromeTraceLogger(const std::string& traceFileName, int
   }
   const ktj_field fragment = {KTJ_NONE, KTJ_F_RAW, 1}; /* one slot: string id of a whole args fragment */
   note(ktj_register_schema(engine_, &fragment, 1, &fragmentSchema_), "ktj_register_schema");
+  const ktj_field withCollective[2] = {{KTJ_NONE, KTJ_F_COLLECTIVE, 1}, fragment};
+  note(ktj_register_schema(engine_, withCollective, 1, &collectiveSchema_), "ktj_register_schema");
+  note(ktj_register_schema(engine_, withCollective, 2, &collectiveFragmentSchema_), "ktj_register_schema");
   pendingOffsets_.push_back(0);
 }
 
@@ -61,6 +64,34 @@ uint32_t GpuChromeTraceLogger::intern(std::unordered_map<std::string, uint32_t>&
   pendingOffsets_.push_back(pendingBlob_.size());
   if (pendingBlob_.size() >= kStringBatchBytes) flushStrings();
   return id;
+}
+
+/* The values ChromeTraceLogger::appendCollectiveMetadata reads from a record_param_comms op
+ * (output_json.cpp:718-835), handed to the engine once per distinct set of values. */
+uint32_t GpuChromeTraceLogger::collectiveIndex(const ITraceActivity& op) {
+  static const char* const kKeys[] = {"Collective name", "In msg nelems", "Out msg nelems", "Group size", "dtype",
+                                      "Input Tensors start", "Output Tensors start", "In split size", "Out split size",
+                                      "Process Group Name", "Process Group Description", "Process Group Ranks",
+                                      "Dst Rank", "Src Rank", "Seq", "Comms Id", "Rank"};
+  constexpr size_t kCount = sizeof(kKeys) / sizeof(kKeys[0]);
+  static_assert(kCount * sizeof(const char*) == sizeof(ktj_collective_meta), "one key per field of ktj_collective_meta");
+  std::string values[kCount];
+  std::string key;
+  for (size_t i = 0; i < kCount; ++i) {
+    values[i] = op.getMetadataValue(kKeys[i]);
+    key += values[i];
+    key += '\0';
+  }
+  auto it = collectives_.find(key);
+  if (it != collectives_.end()) return it->second;
+  const ktj_collective_meta meta = {
+      values[0].c_str(),  values[1].c_str(),  values[2].c_str(),  values[3].c_str(),  values[4].c_str(),  values[5].c_str(),
+      values[6].c_str(),  values[7].c_str(),  values[8].c_str(),  values[9].c_str(),  values[10].c_str(), values[11].c_str(),
+      values[12].c_str(), values[13].c_str(), values[14].c_str(), values[15].c_str(), values[16].c_str()}; /* kKeys order */
+  uint32_t index = 0;
+  note(ktj_add_collective(engine_, &meta, &index), "ktj_add_collective");
+  collectives_.emplace(std::move(key), index);
+  return index;
 }
 
 /* One schema per distinct list of counter names: a keyed double field for each. */
@@ -154,14 +185,11 @@ void GpuChromeTraceLogger::handleActivity(const ITraceActivity& op) {
   const int64_t flowId = op.flowId();
   const bool counter = type == ActivityType::HARDWARE_COUNTERS || type == ActivityType::MTIA_COUNTERS ||
       type == ActivityType::XPU_SCOPE_PROFILER; /* output_json.cpp:847-856 */
-  /* collective metadata (output_json.cpp:899-908) needs the linked op's own metadata, which does
-   * not fit the packed record */
-  bool unsupported = false;
-  if (!counter && linked != nullptr && linked->name() == kParamCommsName) {
-    unsupported = type == ActivityType::CONCURRENT_KERNEL ||
-        (type == ActivityType::MTIA_CCP_EVENTS && name.rfind("hccl::", 0) == 0);
-  }
-  unsupported = unsupported || device < std::numeric_limits<int32_t>::min() || device > std::numeric_limits<int32_t>::max();
+  /* collective metadata comes from a linked record_param_comms op (output_json.cpp:899-908) */
+  const bool collective = !counter && linked != nullptr &&
+      (type == ActivityType::CONCURRENT_KERNEL || (type == ActivityType::MTIA_CCP_EVENTS && name.rfind("hccl::", 0) == 0)) &&
+      linked->name() == kParamCommsName;
+  const bool unsupported = device < std::numeric_limits<int32_t>::min() || device > std::numeric_limits<int32_t>::max();
   if (unsupported) {
     if (unsupported_++ == 0) {
       LOG(WARNING) << "GpuChromeTraceLogger: activity '" << name << "' of type " << toString(type)
@@ -202,7 +230,15 @@ void GpuChromeTraceLogger::handleActivity(const ITraceActivity& op) {
     return;
   }
   const std::string metadata = op.metadataJson();
-  if (metadata.empty()) {
+  if (collective) { /* the first slot names the linked op's collective metadata */
+    r.schema_id = metadata.empty() ? collectiveSchema_ : collectiveFragmentSchema_;
+    r.args_off = nextSlot_++;
+    slots_.push_back(collectiveIndex(*linked));
+    if (!metadata.empty()) {
+      ++nextSlot_;
+      slots_.push_back(intern(fragments_, metadata));
+    }
+  } else if (metadata.empty()) {
     r.schema_id = KTJ_NONE;
   } else {
     r.schema_id = fragmentSchema_;

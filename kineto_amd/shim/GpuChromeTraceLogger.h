@@ -52,8 +52,7 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
                      int64_t endTime) override;
 
   std::string traceFileName() const { return fileName_; }
-  /* activities the engine does not render (kernels that would carry the collective metadata of
-   * a linked record_param_comms op): they are dropped and counted here */
+  /* activities the engine cannot take (a deviceId outside 32 bits): dropped and counted here */
   uint64_t unsupportedActivities() const { return unsupported_; }
   /* ktj status of the first failed engine call, 0 if none */
   int engineStatus() const { return status_; }
@@ -63,6 +62,7 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
 
  private:
   uint32_t intern(std::unordered_map<std::string, uint32_t>& index, const std::string& s);
+  uint32_t collectiveIndex(const libkineto::ITraceActivity& op);
   uint32_t counterSchema(const std::vector<std::pair<std::string, double>>& values);
   void flushStrings();
   void flushRecords();
@@ -74,10 +74,13 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
   int status_ = 0;
   uint64_t unsupported_ = 0;
   uint32_t fragmentSchema_ = KTJ_NONE;
+  uint32_t collectiveSchema_ = KTJ_NONE;         /* collective metadata only        */
+  uint32_t collectiveFragmentSchema_ = KTJ_NONE; /* collective metadata + fragment  */
 
   /* strings not yet handed to the engine: blob + offsets, ids are consecutive from nextStringId_ */
   std::unordered_map<std::string, uint32_t> names_;
   std::unordered_map<std::string, uint32_t> fragments_;
+  std::unordered_map<std::string, uint32_t> collectives_;    /* key: the 17 values, NUL-separated */
   std::unordered_map<std::string, uint32_t> counterSchemas_; /* key: the name ids, 4 bytes each */
   std::string pendingBlob_;
   std::vector<uint64_t> pendingOffsets_;

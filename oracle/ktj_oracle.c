@@ -28,7 +28,11 @@
  *       hand-made case (tests/kat_cases.py: case_instant_and_stream_sync).
  *   - counter events: byte-compared with the real logger on a hand-made case
  *       (tests/kat_cases.py: case_counter_events) and inside the seeded random streams.
- * Not restated: collective metadata (output_json.cpp:718-835, 899-908).
+ *   - collective metadata and the "distributedInfo" footer entry: the inputs and expected
+ *       values of test/OutputJsonTest.cpp:81-225, and byte-compared with the real logger on
+ *       hand-made cases (tests/kat_cases.py: case_collective_*).  The order of the process groups
+ *       is the iteration order of a std::unordered_map and is taken from the C++ library
+ *       (map_order.cpp), as the logger takes it.
  */
 #define _GNU_SOURCE
 #include "ktj_oracle.h"
@@ -326,6 +330,10 @@ struct ktj_oracle {
   /* (device << 32 | virtual tid) keys whose Stream-Sync row header was written: output_json.h
    * syncStreamMetadataEmitted_ */
   int64_t* sync_seen; uint64_t n_sync_seen, cap_sync_seen;
+  /* distInfo_ and pgMap_ (output_json.h:229-233); process groups in insertion order */
+  char *dist_backend, *dist_rank, *dist_world_size, *dist_nccl_version;
+  struct pg_entry { char *name, *desc, *backend_config, *size, *ranks; } *pgs;
+  uint64_t n_pgs, cap_pgs;
   double t_join, t_sort, t_emit;
   int64_t win_start, win_end;
 };
@@ -446,6 +454,15 @@ static int64_t linked_activity(const umap* cpu_corr, const umap* activity_map, u
   return act ? (int64_t)*act : -1;
 }
 
+/* 1 + the slot value of a record's leading KTJ_F_COLLECTIVE field, 0 if it has none */
+static uint32_t collective_index(const ktj_stream* s, const ktj_generic_rec* r) {
+  if (r->schema_id == KTJ_NONE || r->schema_id >= s->n_schemas) return 0;
+  const ktj_schema_desc* d = &s->schemas[r->schema_id];
+  if (d->n_fields == 0 || s->fields[d->first_field].type != KTJ_F_COLLECTIVE || r->args_off >= s->n_args) return 0;
+  const uint64_t k = s->args[r->args_off];
+  return k < s->n_collectives ? (uint32_t)k + 1u : 0u;
+}
+
 static uint32_t ptr_string(ktj_oracle* o, uint64_t p) { /* fmt "{}" of const void* */
   char b[32];
   int n = sprintf(b, "0x%llx", (unsigned long long)p);
@@ -493,10 +510,13 @@ static int stage_join(ktj_oracle* o) {
       uint64_t slot = r->args_off;
       for (uint32_t f = 0; f < d->n_fields; ++f) {
         const ktj_field* fd = &s->fields[d->first_field + f];
-        visit(o, a, fd->key_id, fd->type, fd->count, s->args + slot);
+        if (fd->type != KTJ_F_COLLECTIVE) visit(o, a, fd->key_id, fd->type, fd->count, s->args + slot);
         slot += fd->count;
       }
     }
+    /* an activity that arrives with its record_param_comms op resolved (output_json.cpp:899-908) */
+    if (a->has_linked && (r->type == KTJ_TYPE_CONCURRENT_KERNEL || r->type == KTJ_TYPE_MTIA_CCP_EVENTS))
+      a->collective = collective_index(s, r);
     *umap_slot(&activity_map, (uint64_t)(int64_t)r->id, NULL) = i;
   }
   for (uint64_t i = 0; i < s->n_extcorr; ++i)
@@ -670,7 +690,13 @@ static int stage_join(ktj_oracle* o) {
     a->flow_type = KTJ_LINK_ASYNC_CPU_GPU;
     a->flow_start = 0;
     a->arrival = s->n_generic + s->n_runtime + i;
-    if (linked >= 0) { a->has_linked = 1; a->linked_corr = s->generic[linked].id; o->n_linked++; }
+    if (linked >= 0) {
+      a->has_linked = 1; a->linked_corr = s->generic[linked].id; o->n_linked++;
+      const ktj_generic_rec* op = &s->generic[linked]; /* the op hands its collective metadata to kernels */
+      if (d->domain != KTJ_DOM_MEMSET && d->domain != KTJ_DOM_MEMORY_COPY && op->type != KTJ_TYPE_CONCURRENT_KERNEL &&
+          op->type != KTJ_TYPE_MTIA_CCP_EVENTS)
+        a->collective = collective_index(s, op);
+    }
     int key = (int)(uint32_t)d->id;
     if (d->domain == KTJ_DOM_MEMSET) { /* CuptiActivity.h:682-713 */
       a->type = KTJ_TYPE_GPU_MEMSET;
@@ -1102,8 +1128,124 @@ static void handle_counter_event(ktj_oracle* o, const ktj_mat_activity* a) {
   free(args.p);
 }
 
-/* handleActivity + handleGenericLink + handleLink: output_json.cpp:837-1021.  The collective
- * metadata of record_param_comms (:899-908) is not restated here. */
+/* ---- collective metadata: output_json.cpp:718-835 ---- */
+void ktj_oracle_string_map_order(const char* const* keys, uint64_t n, uint64_t* order); /* map_order.cpp */
+
+static char* dup_value(const char* p) { return strdup(p ? p : ""); }
+/* stripQuotes: output_json.cpp:57-63 */
+static char* strip_quotes(const char* p) {
+  if (!p) p = "";
+  size_t n = strlen(p);
+  if (n >= 2 && p[0] == '"' && p[n - 1] == '"') { p += 1; n -= 2; }
+  char* r = (char*)malloc(n + 1);
+  if (!r) abort();
+  memcpy(r, p, n);
+  r[n] = 0;
+  return r;
+}
+static void args_add_raw(sbuf* args, const char* key, const char* value) { /* ArgsBuilder::addRaw :161-164 */
+  if (args->n) sb_putc(args, ',');
+  sb_putc(args, '"'); sb_puts(args, key); sb_puts(args, "\": "); sb_puts(args, value);
+}
+static void args_add_quoted(sbuf* args, const char* key, const char* value) { /* ArgsBuilder::addQuoted :167-170 */
+  if (args->n) sb_putc(args, ',');
+  sb_putc(args, '"'); sb_puts(args, key); sb_puts(args, "\": \""); sb_puts(args, value); sb_putc(args, '"');
+}
+/* appendCollectiveArgs: output_json.cpp:718-797 */
+static void append_collective_args(sbuf* args, const ktj_collective_meta* m) {
+  char* name = strip_quotes(m->collective_name);
+  char* in_n = dup_value(m->in_msg_nelems);
+  char* out_n = dup_value(m->out_msg_nelems);
+  char* group = dup_value(m->group_size);
+  char* dtype = strip_quotes(m->dtype);
+  if (name[0] && in_n[0] && out_n[0] && group[0] && dtype[0]) {
+    args_add_quoted(args, "Collective name", name);
+    args_add_raw(args, "In msg nelems", in_n);
+    args_add_raw(args, "Out msg nelems", out_n);
+    args_add_raw(args, "Group size", group);
+    args_add_quoted(args, "dtype", dtype);
+  }
+  char* in_start = strip_quotes(m->in_tensors_start);
+  char* out_start = strip_quotes(m->out_tensors_start);
+  if (in_start[0]) args_add_quoted(args, "Input Tensors start", in_start);
+  if (out_start[0]) args_add_quoted(args, "Output Tensors start", out_start);
+  char* in_split = strip_quotes(m->in_split);
+  char* out_split = strip_quotes(m->out_split);
+  if (in_split[0] && out_split[0]) {
+    args_add_quoted(args, "In split size", in_split);
+    args_add_quoted(args, "Out split size", out_split);
+  }
+  char* pg_name = strip_quotes(m->pg_name);
+  if (pg_name[0]) args_add_quoted(args, "Process Group Name", pg_name);
+  char* pg_desc = strip_quotes(m->pg_desc);
+  if (pg_desc[0]) args_add_quoted(args, "Process Group Description", pg_desc);
+  char* ranks = strip_quotes(m->group_ranks);
+  if (ranks[0]) args_add_quoted(args, "Process Group Ranks", ranks);
+  if (m->dst_rank && m->dst_rank[0]) args_add_raw(args, "Dst Rank", m->dst_rank);
+  if (m->src_rank && m->src_rank[0]) args_add_raw(args, "Src Rank", m->src_rank);
+  if (m->seq && m->seq[0]) args_add_raw(args, "Seq", m->seq);
+  if (m->comms_id && m->comms_id[0]) args_add_raw(args, "Comms Id", m->comms_id);
+  free(name); free(in_n); free(out_n); free(group); free(dtype); free(in_start); free(out_start);
+  free(in_split); free(out_split); free(pg_name); free(pg_desc); free(ranks);
+}
+/* appendCollectiveMetadata: output_json.cpp:799-835 */
+static void append_collective_metadata(ktj_oracle* o, sbuf* args, const ktj_collective_meta* m, const char* backend,
+                                       const char* backend_config) {
+  append_collective_args(args, m);
+  char* pg_name = strip_quotes(m->pg_name);
+  char* pg_desc = strip_quotes(m->pg_desc);
+  if (!o->dist_backend && strcmp(pg_desc, "default_pg") == 0) { /* :807-817 */
+    o->dist_backend = dup_value(backend);
+    o->dist_rank = dup_value(m->rank);
+    o->dist_world_size = dup_value(m->group_size);
+    o->dist_nccl_version = dup_value(strcmp(backend, "nccl") == 0 ? "unknown" : "");
+  }
+  int known = 0; /* pgMap_.insert: the first entry of a name stays */
+  for (uint64_t k = 0; k < o->n_pgs && !known; ++k) known = strcmp(o->pgs[k].name, pg_name) == 0;
+  if (!known) {
+    if (o->n_pgs == o->cap_pgs) {
+      o->cap_pgs = o->cap_pgs ? o->cap_pgs * 2 : 8;
+      o->pgs = (struct pg_entry*)realloc(o->pgs, o->cap_pgs * sizeof *o->pgs);
+      if (!o->pgs) abort();
+    }
+    struct pg_entry* e = &o->pgs[o->n_pgs++];
+    e->name = pg_name; pg_name = NULL;
+    e->desc = pg_desc; pg_desc = NULL;
+    e->backend_config = dup_value(backend_config);
+    e->size = dup_value(m->group_size);
+    e->ranks = strip_quotes(m->group_ranks);
+  }
+  free(pg_name); free(pg_desc);
+}
+/* addOnDemandDistMetadata: output_json.cpp:1030-1064 */
+static void add_dist_metadata(ktj_oracle* o) {
+  if (!o->dist_backend) return;
+  sbuf* b = &o->out;
+  char n[24];
+  sb_puts(b, "\n  \"distributedInfo\": {\"backend\": \""); sb_puts(b, o->dist_backend);
+  sb_puts(b, "\", \"rank\": "); sb_puts(b, o->dist_rank);
+  sb_puts(b, ", \"world_size\": "); sb_puts(b, o->dist_world_size);
+  sb_puts(b, ", \"pg_count\": "); sb_put(b, n, fmt_u64(o->n_pgs, n));
+  sb_puts(b, ", \"pg_config\": [");
+  const char** names = (const char**)malloc(sizeof(char*) * (o->n_pgs ? o->n_pgs : 1));
+  uint64_t* order = (uint64_t*)malloc(8 * (o->n_pgs ? o->n_pgs : 1));
+  if (!names || !order) abort();
+  for (uint64_t k = 0; k < o->n_pgs; ++k) names[k] = o->pgs[k].name;
+  ktj_oracle_string_map_order(names, o->n_pgs, order);
+  for (uint64_t k = 0; k < o->n_pgs; ++k) {
+    const struct pg_entry* e = &o->pgs[order[k]];
+    if (k) sb_putc(b, ',');
+    sb_puts(b, "{\"pg_name\": \""); sb_puts(b, e->name);
+    sb_puts(b, "\", \"pg_desc\": \""); sb_puts(b, e->desc);
+    sb_puts(b, "\", \"backend_config\": \""); sb_puts(b, e->backend_config);
+    sb_puts(b, "\", \"pg_size\": "); sb_puts(b, e->size);
+    sb_puts(b, ", \"ranks\": \""); sb_puts(b, e->ranks); sb_puts(b, "\"}");
+  }
+  sb_puts(b, "], \"nccl_version\": \""); sb_puts(b, o->dist_nccl_version); sb_puts(b, "\"},");
+  free(names); free(order);
+}
+
+/* handleActivity + handleGenericLink + handleLink: output_json.cpp:837-1021. */
 static void handle_activity(ktj_oracle* o, const ktj_mat_activity* a) {
   if (a->type == KTJ_TYPE_CPU_INSTANT_EVENT) { handle_instant_event(o, a); return; } /* :842-845 */
   if (is_counter_type(a->type)) { handle_counter_event(o, a); return; }               /* :847-856 */
@@ -1136,6 +1278,12 @@ static void handle_activity(ktj_oracle* o, const ktj_mat_activity* a) {
   }
   const char* nm; uint64_t nl;
   ktj_oracle_string(o, a->name_id, &nm, &nl);
+  if (a->has_linked && a->collective) {                     /* :899-908: the linked op is a record_param_comms */
+    const ktj_collective_meta* m = &o->s->collectives[a->collective - 1];
+    if (a->type == KTJ_TYPE_CONCURRENT_KERNEL) append_collective_metadata(o, &args, m, "nccl", "cuda:nccl");
+    else if (a->type == KTJ_TYPE_MTIA_CCP_EVENTS && nl >= 6 && memcmp(nm, "hccl::", 6) == 0)
+      append_collective_metadata(o, &args, m, "hccl", "mtia:hccl");
+  }
   char* name = (char*)malloc(nl * 2 + 8);
   if (!name) abort();
   size_t name_n = ktj_oracle_sanitize_name(nm, nl, name);   /* :946-949 */
@@ -1146,7 +1294,7 @@ static void handle_activity(ktj_oracle* o, const ktj_mat_activity* a) {
   int64_t resource = a->resource;
   const int sync = is_stream_sync(o, a);
   if (sync) { /* :913-943: own row per stream, announced once per (device, row) */
-    const int64_t sync_tid = resource + SYNC_STREAM_TID_OFFSET;
+    const int64_t sync_tid = (int64_t)((uint64_t)resource + SYNC_STREAM_TID_OFFSET); /* wraps like the logger's own sum */
     const int64_t key = (int64_t)(((uint64_t)a->device << 32) | (uint64_t)sync_tid);
     int seen = 0;
     for (uint64_t k = 0; k < o->n_sync_seen && !seen; ++k) seen = o->sync_seen[k] == key;
@@ -1181,7 +1329,7 @@ static void handle_activity(ktj_oracle* o, const ktj_mat_activity* a) {
                       : a->flow_type == (int)KTJ_LINK_ASYNC_CPU_GPU ? "ac2g" : NULL;
     if (fname) {
       write_flow_event(o, a->flow_start ? 's' : 'f', a->flow_id, a->device,
-                       sanitize_tid(sync ? a->resource + SYNC_STREAM_TID_OFFSET : a->resource),
+                       sanitize_tid(sync ? (int64_t)((uint64_t)a->resource + SYNC_STREAM_TID_OFFSET) : a->resource),
                        rel_time(o, a->ts), fname);          /* handleLink :997-1021 */
       o->n_flow++;
     }
@@ -1195,6 +1343,7 @@ static void finalize_trace(ktj_oracle* o) {
   sbuf none = {0};
   write_instant_event(o, "", "g", "Record Window End", "\"\"", "\"\"", rel_time(o, s->end_time_ns), &none, 1);
   sb_puts(&o->out, "\n  ],");
+  add_dist_metadata(o);                                     /* :1094-1096 */
   sb_puts(&o->out, "\"traceName\": \"");
   size_t n = strlen(s->trace_name);
   char* t = (char*)malloc(n + 1);
@@ -1241,6 +1390,11 @@ void ktj_oracle_free(ktj_oracle* o) {
   if (!o) return;
   free(o->xblob.p); free(o->xoff); free(o->acts); free(o->order); free(o->fpool); free(o->spool);
   free(o->act_f0); free(o->act_s0); free(o->out.p); free(o->sync_seen);
+  free(o->dist_backend); free(o->dist_rank); free(o->dist_world_size); free(o->dist_nccl_version);
+  for (uint64_t k = 0; k < o->n_pgs; ++k) {
+    free(o->pgs[k].name); free(o->pgs[k].desc); free(o->pgs[k].backend_config); free(o->pgs[k].size); free(o->pgs[k].ranks);
+  }
+  free(o->pgs);
   free(o);
 }
 void ktj_oracle_output(const ktj_oracle* o, const char** bytes, uint64_t* n) { *bytes = o->out.p; *n = o->out.n; }

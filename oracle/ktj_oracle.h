@@ -35,6 +35,9 @@ typedef struct ktj_mat_activity {
   int32_t flow_type;    /* flowType()                                                          */
   int32_t flow_start;   /* flowStart()                                                         */
   int32_t has_linked;
+  uint32_t collective;  /* 1 + index (ktj_stream::collectives) of the metadata of the linked
+                           record_param_comms op, 0 = the linked op is no such op                */
+  uint32_t pad;
 } ktj_mat_activity;
 
 typedef struct ktj_oracle ktj_oracle;

@@ -45,9 +45,25 @@ struct MatActivity : public ITraceActivity {
   mutable GenericTraceActivity linkedStub;  // only correlationId()/name() are read from it
   bool hasLinked;
 
-  MatActivity(const ktj_mat_activity* act, const StringTable* s) : a(act), st(s), hasLinked(act->has_linked != 0) {
+  // collectives: ktj_stream::collectives; an activity whose linked op carries collective metadata
+  // gets a record_param_comms op with those values as its linked activity
+  MatActivity(const ktj_mat_activity* act, const StringTable* s, const ktj_collective_meta* collectives = nullptr)
+      : a(act), st(s), hasLinked(act->has_linked != 0) {
     linkedStub.id = static_cast<int32_t>(act->linked_corr);
     linkedStub.activityName = "linked_op";
+    if (act->collective != 0 && collectives != nullptr) {
+      const ktj_collective_meta& m = collectives[act->collective - 1];
+      linkedStub.activityName = "record_param_comms";
+      const std::pair<const char*, const char*> kv[] = {
+          {"Collective name", m.collective_name}, {"In msg nelems", m.in_msg_nelems}, {"Out msg nelems", m.out_msg_nelems},
+          {"Group size", m.group_size}, {"dtype", m.dtype}, {"Input Tensors start", m.in_tensors_start},
+          {"Output Tensors start", m.out_tensors_start}, {"In split size", m.in_split}, {"Out split size", m.out_split},
+          {"Process Group Name", m.pg_name}, {"Process Group Description", m.pg_desc},
+          {"Process Group Ranks", m.group_ranks}, {"Dst Rank", m.dst_rank}, {"Src Rank", m.src_rank}, {"Seq", m.seq},
+          {"Comms Id", m.comms_id}, {"Rank", m.rank}};
+      for (const auto& e : kv)
+        if (e.second != nullptr && e.second[0] != 0) linkedStub.addMetadata(std::string(e.first), std::string(e.second));
+    }
   }
   int64_t deviceId() const override { return a->device; }
   int64_t resourceId() const override { return a->resource; }
@@ -145,7 +161,7 @@ void replay_stream(L& logger, const ktj_stream* s, const ktj_mat_activity* acts,
   StringTable st{fn, ctx};
   std::vector<MatActivity> wrapped;
   wrapped.reserve(n_acts);
-  for (uint64_t i = 0; i < n_acts; ++i) wrapped.emplace_back(&acts[i], &st);
+  for (uint64_t i = 0; i < n_acts; ++i) wrapped.emplace_back(&acts[i], &st, s->collectives);
   std::vector<const MatActivity*> order(n_acts);
   for (uint64_t i = 0; i < n_acts; ++i) order[i] = &wrapped[i];
   std::stable_sort(order.begin(), order.end(), [](const MatActivity* x, const MatActivity* y) {

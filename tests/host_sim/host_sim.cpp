@@ -75,6 +75,17 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   ctx.dict.flags = v.flags.data(); ctx.dict.n = (uint32_t)s->n_strings;
   ctx.fields = s->fields; ctx.schemas = s->schemas; ctx.n_schemas = (uint32_t)s->n_schemas;
   ctx.args = s->args; ctx.n_args = s->n_args; ctx.base_time_ns = s->base_time_ns;
+  // collective metadata: the arguments of every entry in one blob
+  std::vector<ktj::CollectiveInfo> collectives;
+  std::string coll_blob;
+  std::vector<uint64_t> coll_off(1, 0);
+  for (uint64_t k = 0; k < s->n_collectives; ++k) {
+    collectives.push_back(ktj::make_collective(s->collectives[k]));
+    coll_blob += collectives.back().args;
+    coll_off.push_back(coll_blob.size());
+  }
+  coll_blob.append(16, '\0');
+  ctx.coll_blob = coll_blob.data(); ctx.coll_off = coll_off.data(); ctx.n_coll = (uint32_t)s->n_collectives;
 
   ClockDev clk;
   clk.t0_approx = s->clock.t0_approx; clk.t0 = s->clock.t0; memcpy(&clk.scale_bits, &s->clock.scale, 8);
@@ -86,8 +97,14 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   // tables (value = winning source index)
   std::unordered_map<uint64_t, uint64_t> extcorr;          // correlation -> external id (last wins)
   for (uint64_t i = 0; i < s->n_extcorr; ++i) extcorr[s->extcorr[i].correlation] = s->extcorr[i].external_id;
-  std::unordered_set<uint64_t> cpu_ids;
-  for (uint64_t i = 0; i < ng; ++i) cpu_ids.insert((uint64_t)(int64_t)s->generic[i].id);
+  std::unordered_map<uint64_t, uint64_t> cpu_ids;          // CPU op id -> generic idx (last wins)
+  for (uint64_t i = 0; i < ng; ++i) cpu_ids[(uint64_t)(int64_t)s->generic[i].id] = i;
+  auto coll_of = [&](uint64_t id) -> uint32_t {            // collective metadata of the linked CPU op
+    auto it = extcorr.find(narrow_corr_key(id));
+    if (it == extcorr.end()) return 0;
+    auto ci = cpu_ids.find(it->second);
+    return ci == cpu_ids.end() ? 0 : collective_for_linked(s->generic[ci->second], ctx);
+  };
   auto ext_of = [&](uint64_t id) -> int32_t {
     auto it = extcorr.find(narrow_corr_key(id));
     if (it == extcorr.end()) return 0;
@@ -100,6 +117,7 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   for (uint64_t i = 0; i < ng; ++i) {
     mat[i] = mat_generic(s->generic[i]);
     if (!generic_record_prints(s->generic[i], ctx)) mat[i].meta &= ~KTJ_M_VALID;
+    attach_own_collective(mat[i], s->generic[i], ctx);
   }
 
   std::unordered_map<uint64_t, uint64_t> stream_src;       // full id -> runtime idx (last wins)
@@ -198,7 +216,7 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
     }
     uint64_t grid[3];
     if (ksrc) pack_grid(*ksrc, grid);
-    mat[ng + nr + i] = mat_device(d, ts, dur, res, valid, ext_of(d.id), ksrc ? grid : nullptr, has_size, size);
+    mat[ng + nr + i] = mat_device(d, ts, dur, res, valid, ext_of(d.id), ksrc ? grid : nullptr, has_size, size, coll_of(d.id));
   }
 
   // canonical order over valid rows
@@ -236,7 +254,13 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   for (uint64_t i = 0; i < s->n_resource_infos; ++i) append_resource_info(prefix, s->resource_infos[i], s->base_time_ns);
   for (uint64_t i = 0; i < s->n_overhead_infos; ++i) append_overhead_info(prefix, s->overhead_infos[i], s->base_time_ns);
   for (uint64_t i = 0; i < s->n_spans; ++i) append_trace_span(suffix, s->spans[i], s->base_time_ns);
-  append_trace_end(suffix, s->end_time_ns, s->base_time_ns, s->trace_name);
+  std::vector<ktj::CollectiveUse> uses; // every activity that prints collective metadata, in emission order
+  for (uint64_t a : perm) {
+    const uint32_t k = collective_of(mat[a]);
+    const uint32_t cls = (mat[a].meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT;
+    if (k) uses.push_back(ktj::CollectiveUse{k - 1, cls == KTJ_CLASS_GENERIC && (mat[a].meta & KTJ_M_TYPE_MASK) == KTJ_TYPE_MTIA_CCP_EVENTS});
+  }
+  append_trace_end(suffix, s->end_time_ns, s->base_time_ns, s->trace_name, ktj::distributed_info_text(collectives, uses));
 
   const uint64_t total = prefix.size() + act_bytes + suffix.size();
   char* buf = (char*)aligned_alloc(64, (total + 64 + 63) / 64 * 64);
@@ -254,7 +278,7 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
     std::vector<uint32_t> kinds(perm.size());
     for (size_t i = 0; i < perm.size(); ++i) {
       const MatRow& m = mat[perm[i]];
-      kinds[i] = tail_kind(m, m.ext != 0 || has_fragment(m, ctx));
+      kinds[i] = tail_kind(m, has_args(m, ctx));
     }
     const uint64_t P = prefix.size();
     for (size_t i = 0; i < perm.size(); ++i) {

@@ -200,7 +200,129 @@ def case_counter_events():
     return b, expect
 
 
-SUBSTRING_CASES = [case_counter_events, case_instant_and_stream_sync, case_logger_events, case_trace_span, case_benchmark_cpu_op, case_typed_kernel_args,
+COLLECTIVE_REF_VALUES = dict(collective_name="allreduce", dtype="Float", pg_name="0", pg_desc="default_pg", in_split="[1, 2]",
+                             out_split="[3, 4]", group_ranks="[0, 1, 2, 3, 4, 5, 6, 7]", in_tensors_start="[[4096, 8192]]",
+                             out_tensors_start="[[12288]]")
+COLLECTIVE_REF_NUMBERS = dict(in_msg_nelems="1024", out_msg_nelems="512", group_size="8", rank="0", src_rank="1", dst_rank="2",
+                              seq="3", comms_id="4")
+# expectedArgs / expectedDistInfo of libkineto/test/OutputJsonTest.cpp:188-219
+COLLECTIVE_REF_ARGS = {"Collective name": "allreduce", "In msg nelems": 1024, "Out msg nelems": 512, "Group size": 8,
+                       "dtype": "Float", "Input Tensors start": "[[4096, 8192]]", "Output Tensors start": "[[12288]]",
+                       "In split size": "[1, 2]", "Out split size": "[3, 4]", "Process Group Name": "0",
+                       "Process Group Description": "default_pg", "Process Group Ranks": "[0, 1, 2, 3, 4, 5, 6, 7]",
+                       "Src Rank": 1, "Dst Rank": 2, "Seq": 3, "Comms Id": 4}
+COLLECTIVE_REF_DIST = {"backend": "nccl", "rank": 0, "world_size": 8, "pg_count": 1,
+                       "pg_config": [{"pg_name": "0", "pg_desc": "default_pg", "backend_config": "cuda:nccl", "pg_size": 8,
+                                      "ranks": "[0, 1, 2, 3, 4, 5, 6, 7]"}],
+                       "nccl_version": "unknown"}
+
+
+def case_collective_reference_test(quoted=False):
+    """The trace of libkineto/test/OutputJsonTest.cpp:81-130: one CONCURRENT_KERNEL activity linked to
+    a record_param_comms op; string values arrive with surrounding quotes (`quoted`) or bare.  The
+    activity arrives with its linked op resolved, so the record itself carries the collective
+    metadata."""
+    b = StreamBuilder(end_time=B + 300)
+    q = (lambda v: '"%s"' % v) if quoted else (lambda v: v)
+    k = b.add_collective(**{key: q(v) for key, v in COLLECTIVE_REF_VALUES.items()}, **COLLECTIVE_REF_NUMBERS)
+    own = b.schema([(None, abi.F_COLLECTIVE, 1)])
+    b.add_generic("nccl:all_reduce", KERNEL, B + 100, B + 200, 0, 0, schema=own, values=[k], linked=0)
+    expect = [
+        '"name": "nccl:all_reduce",\n    "pid": 0,\n    "tid": 0,\n    "ts": 0.100,\n    "dur": 0.100\n    ,\n    "args": {\n      '
+        '"Collective name": "allreduce","In msg nelems": 1024,"Out msg nelems": 512,"Group size": 8,"dtype": "Float",'
+        '"Input Tensors start": "[[4096, 8192]]","Output Tensors start": "[[12288]]","In split size": "[1, 2]",'
+        '"Out split size": "[3, 4]","Process Group Name": "0","Process Group Description": "default_pg",'
+        '"Process Group Ranks": "[0, 1, 2, 3, 4, 5, 6, 7]","Dst Rank": 2,"Src Rank": 1,"Seq": 3,"Comms Id": 4\n    }\n  },',
+        '\n  ],\n  "distributedInfo": {"backend": "nccl", "rank": 0, "world_size": 8, "pg_count": 1, "pg_config": ['
+        '{"pg_name": "0", "pg_desc": "default_pg", "backend_config": "cuda:nccl", "pg_size": 8, '
+        '"ranks": "[0, 1, 2, 3, 4, 5, 6, 7]"}], "nccl_version": "unknown"},"traceName": "t.json" }',
+    ]
+    return b, expect
+
+
+def case_collective_reference_test_quoted():
+    return case_collective_reference_test(quoted=True)
+
+
+def case_collective_joined():
+    """Collective metadata through the join (output_json.cpp:718-835, 899-908, 1030-1064): kernel rows
+    print the values of the record_param_comms op their correlation id leads to; copies and kernels
+    linked to other ops do not; the first kernel in emission order that names the default process
+    group fills "distributedInfo", every group is listed once (first entry of a name stays); an
+    MTIA event named hccl::... reports backend "hccl"; a kernel outside the window counts for
+    nothing.  Expected strings follow the reference's templates; the whole document is compared
+    with the real logger where it is built."""
+    MTIA_CCP_EVENTS = 13
+    b = StreamBuilder(window=(B, B + 10**6), end_time=B + 10**6)
+    b.api(["hipLaunchKernel", "hipMemcpyAsync"], flow_start=[0, 1])
+    typed = [(None, abi.F_COLLECTIVE, 1), ("Collective name", abi.F_STR, 1), ("Seq", abi.F_I64, 1)]
+    sch = b.schema(typed)
+    bare = b.schema([(None, abi.F_COLLECTIVE, 1)])
+    plain = b.schema([("Seq", abi.F_I64, 1)])
+    groups = [("7", "tp_group", "4", "[0, 1, 2, 3]"), ("0", "default_pg", "8", "[0, 1, 2, 3, 4, 5, 6, 7]"),
+              ("12", "pp", "2", "[0, 4]"), ("3", 'dp "x"', "2", "[0, 1]"), ("0", "shadowed", "9", "[9]")]
+    colls = []
+    for i, (name, desc, size, ranks) in enumerate(groups):
+        colls.append(b.add_collective(collective_name='"allgather"' if i % 2 else "allgather", in_msg_nelems=str(100 + i),
+                                      out_msg_nelems=str(200 + i), group_size=size, dtype="Half", pg_name=name, pg_desc=desc,
+                                      group_ranks=ranks, rank=str(5), seq=str(i), comms_id=str(1 << 40)))
+    partial = b.add_collective(collective_name="broadcast", in_msg_nelems="1", pg_name="21", pg_desc="default_pg",
+                               in_split="[1]", src_rank="3", rank="6")   # no dtype: none of the five; no out split: no splits
+    empty = b.add_collective()                                            # nothing at all: group "" is still listed
+    ops = colls + [partial, empty]
+    pid, tid = 500, 501
+    for i, k in enumerate(ops):                                           # CPU ops, ids 1..7
+        b.add_generic("record_param_comms", CPU_OP, B + 1000 * i, B + 1000 * i + 500, pid, tid, id=i + 1, schema=sch if i < 5 else bare,
+                      values=[k, b.s("allgather"), i] if i < 5 else [k])
+    b.add_generic("aten::add", CPU_OP, B + 9000, B + 9500, pid, tid, id=8, schema=plain, values=[77])
+    for corr in range(1, 11):
+        b.add_extcorr(100 + corr, min(corr, 8))
+        b.add_runtime(100 + corr, B + 20000 + corr, B + 20010 + corr, 0, pid, tid, kind=1, grid=[1, 1, 1], workgroup=[64, 1, 1], stream=0x7000)
+    # kernels: emission order is by (device, stream index, start); arrival order is deliberately different
+    b.add_device(104, B + 50000, B + 50100, domain=0, name="ncclDevKernel_dp", queue=1)          # group 3
+    b.add_device(101, B + 40000, B + 40100, domain=0, name="ncclDevKernel_tp", queue=1)          # group 7: first in time on its stream
+    b.add_device(102, B + 60000, B + 60100, domain=0, name="ncclDevKernel_default", queue=1)     # group 0 default_pg
+    b.add_device(105, B + 30000, B + 30100, domain=0, name="ncclDevKernel_shadow", queue=1)      # group 0 again, other description: seen first
+    b.add_device(103, B + 70000, B + 70100, domain=0, name="ncclDevKernel_pp", queue=1)
+    b.add_device(106, B + 80000, B + 80100, domain=0, name="ncclDevKernel_partial", queue=1)
+    b.add_device(107, B + 90000, B + 90100, domain=0, name="ncclDevKernel_empty", queue=1)
+    b.add_device(108, B + 95000, B + 95100, domain=0, name="vector_add", queue=1)                # linked to aten::add
+    b.add_device(102, B + 96000, B + 96100, domain=1, op=2, queue=1)                               # a copy linked to a collective op
+    b.add_device(103, B + 2 * 10**6, B + 2 * 10**6 + 5, domain=0, name="late", queue=1)           # outside the window
+    b.add_device(109, B + 97000, B + 97100, domain=0, name="vector_mul", queue=1)                # ids above 108 lead to aten::add too
+    k_h = b.add_collective(collective_name="all_reduce", in_msg_nelems="4", out_msg_nelems="4", group_size="2", dtype="Int",
+                           pg_name="h0", pg_desc="hccl_pg", group_ranks="[0, 1]", rank="1")
+    own = b.schema([(None, abi.F_COLLECTIVE, 1), (None, abi.F_RAW, 1)])
+    b.add_generic("hccl::all_reduce", MTIA_CCP_EVENTS, B + 100, B + 200, 0, 1, id=40, schema=own, values=[k_h, b.s('"x": 1')], linked=3)
+    b.add_generic("not_hccl", MTIA_CCP_EVENTS, B + 300, B + 400, 0, 1, id=41, schema=own, values=[k_h, b.s('"y": 2')], linked=3)
+    b.add_generic("hccl::unlinked", MTIA_CCP_EVENTS, B + 500, B + 600, 0, 1, id=42, schema=own, values=[k_h, b.s('"z": 3')])
+    expect = [
+        '"name": "hccl::all_reduce",\n    "pid": 0,\n    "tid": 1,\n    "ts": 0.100,\n    "dur": 0.100\n    ,\n    "args": {\n      "External id": 3,"x": 1,'
+        '"Collective name": "all_reduce","In msg nelems": 4,"Out msg nelems": 4,"Group size": 2,"dtype": "Int","Process Group Name": "h0",'
+        '"Process Group Description": "hccl_pg","Process Group Ranks": "[0, 1]"\n    }\n  },',
+        '"name": "not_hccl",\n    "pid": 0,\n    "tid": 1,\n    "ts": 0.300,\n    "dur": 0.100\n    ,\n    "args": {\n      "External id": 3,"y": 2\n    }\n  },',
+        '"args": {\n      "External id": 42,"z": 3\n    }\n  },',
+        '"name": "ncclDevKernel_shadow",',
+        '"correlation": 105, "kind": "Dispatch Kernel", "grid": [1, 1, 1], "block": [64, 1, 1],"Collective name": "allgather","In msg nelems": 104,'
+        '"Out msg nelems": 204,"Group size": 9,"dtype": "Half","Process Group Name": "0","Process Group Description": "shadowed",'
+        '"Process Group Ranks": "[9]","Seq": 4,"Comms Id": 1099511627776\n    }\n  },',
+        '"correlation": 106, "kind": "Dispatch Kernel", "grid": [1, 1, 1], "block": [64, 1, 1],"In msg nelems"',
+        '"correlation": 106, "kind": "Dispatch Kernel", "grid": [1, 1, 1], "block": [64, 1, 1],"Process Group Name": "21","Process Group Description": "default_pg","Src Rank": 3\n    }',
+        '"correlation": 107, "kind": "Dispatch Kernel", "grid": [1, 1, 1], "block": [64, 1, 1]\n    }',
+        '"correlation": 108, "kind": "Dispatch Kernel", "grid": [1, 1, 1], "block": [64, 1, 1]\n    }',
+        '"distributedInfo": {"backend": "nccl", "rank": 5, "world_size": 8, "pg_count": 7, "pg_config": [',
+        '{"pg_name": "0", "pg_desc": "shadowed", "backend_config": "cuda:nccl", "pg_size": 9, "ranks": "[9]"}',
+        '{"pg_name": "h0", "pg_desc": "hccl_pg", "backend_config": "mtia:hccl", "pg_size": 2, "ranks": "[0, 1]"}',
+        '{"pg_name": "", "pg_desc": "", "backend_config": "cuda:nccl", "pg_size": , "ranks": ""}',
+        '{"pg_name": "3", "pg_desc": "dp "x"", "backend_config": "cuda:nccl", "pg_size": 2, "ranks": "[0, 1]"}',
+        '], "nccl_version": "unknown"},"traceName": "t.json" }',
+    ]
+    absent = ['"correlation": 106, "kind": "Dispatch Kernel", "grid": [1, 1, 1], "block": [64, 1, 1],"In msg nelems"']
+    expect = [e for e in expect if e not in absent]
+    return b, expect
+
+
+SUBSTRING_CASES = [case_collective_reference_test, case_collective_reference_test_quoted, case_collective_joined, case_counter_events, case_instant_and_stream_sync, case_logger_events, case_trace_span, case_benchmark_cpu_op, case_typed_kernel_args,
                    case_typed_metadata_pins, case_names, case_resource_infos]
 
 

@@ -19,7 +19,7 @@ class MatActivity(C.Structure):
                 ("arrival", C.c_uint64), ("slots", C.POINTER(C.c_uint64)),
                 ("fields", C.POINTER(abi.Field)), ("n_fields", C.c_uint32), ("name_id", C.c_uint32),
                 ("type", C.c_int32), ("flow_type", C.c_int32), ("flow_start", C.c_int32),
-                ("has_linked", C.c_int32)]
+                ("has_linked", C.c_int32), ("collective", C.c_uint32), ("pad", C.c_uint32)]
 
 
 _oracle = None

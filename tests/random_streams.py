@@ -46,7 +46,7 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False)
                                  rng.choice([0, 1]), rng.choice([0, 1, 2]))
     apis = ["hipLaunchKernel", "hipMemcpyAsync", "hipMalloc", "hipGraphLaunch", None, "hipFree", 'odd "api"\\name']
     b.api(apis, flow_start=rng.sample(range(len(apis)), 4), malloc_cid=rng.choice([2, abi.KTJ_NONE]))
-    names = [_name(rng) for _ in range(12)]
+    names = [_name(rng) for _ in range(12)] + ["hccl::all_reduce", "record_param_comms"]
 
     def t():
         return rng.choice([rng.randrange(lo - 500, hi + 500), rng.randrange(lo, hi), 0, lo, hi])
@@ -59,6 +59,27 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False)
             typ = rng.randrange(7)
             fields.append((_name(rng)[:12] or "k", typ, rng.randrange(1, 5) if typ == abi.F_I64_ARRAY else 1))
         schemas.append((b.schema(fields), fields))
+    # collective metadata: entries with random subsets of the keys, schemas that start with a reference to one
+    n_coll = rng.choice([0, 0, 1, 5])
+    for _ in range(n_coll):
+        vals = {}
+        for key in abi.COLLECTIVE_KEYS:
+            if rng.random() < 0.6:
+                v = rng.choice(["0", "8", "default_pg", '"default_pg"', "[0, 1]", '"x"', '"', '""', "a\\b", "tp", "allreduce", "Float"])
+                if key == "pg_desc" and rng.random() < 0.5:
+                    v = rng.choice(["default_pg", '"default_pg"'])
+                if key == "pg_name":
+                    v = rng.choice(["0", "1", "2", '"3"', "4", "5", "group six", ""])
+                vals[key] = v
+        b.add_collective(**vals)
+    if n_coll:
+        for _ in range(3):
+            fields = [(None, abi.F_COLLECTIVE, 1)]
+            for _k in range(rng.randrange(0, 3)):
+                typ = rng.randrange(7)
+                fields.append((_name(rng)[:12] or "k", typ, rng.randrange(1, 5) if typ == abi.F_I64_ARRAY else 1))
+            schemas.append((b.schema(fields), fields))
+        schemas.append((b.schema([(None, abi.F_COLLECTIVE, 1), (None, abi.F_RAW, 1)]), [(None, abi.F_COLLECTIVE, 1), (None, abi.F_RAW, 1)]))
     pids, tids = [0, 1, 7, -3, 4242], [0, 5, -5, 4243, I64_MIN, I64_MAX, 10**12]
     ids = list(range(1, 30))
     if wide_ids:
@@ -73,7 +94,9 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False)
             sid, fields = sch
             values = []
             for _key, typ, cnt in fields:
-                if typ == abi.F_F64:
+                if typ == abi.F_COLLECTIVE:
+                    values.append(rng.choice(list(range(n_coll)) + [n_coll, 2**40]))
+                elif typ == abi.F_F64:
                     values.append(_f64(rng))
                 elif typ in (abi.F_STR, abi.F_RAW):
                     values.append(b.s(_name(rng)))
@@ -84,7 +107,7 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False)
                 else:
                     values.append(_i64(rng))
         s0 = t()
-        b.add_generic(rng.choice(names + [None]), rng.choice(TYPES + [0, 0, 0, 9, 15, 17, 28, 28]), s0, s0 + rng.choice([0, 1, 999, 1000, -3, 10**5]),
+        b.add_generic(rng.choice(names + [None]), rng.choice(TYPES + [0, 0, 0, 9, 15, 17, 28, 28, 5, 5, 13, 13]), s0, s0 + rng.choice([0, 1, 999, 1000, -3, 10**5]),
                       rng.choice(pids), rng.choice(tids), id=rng.choice([0, -2, 5, 6, 7, 8, 2**31 - 1, -(2**31)] + ids[:8]),
                       schema=sid, values=values, flow_id=rng.choice([0, 0, 1, 77, 2**32 - 1, 2**40 + 3, -4]), flow_type=rng.choice([0, 1, 2, 3]),
                       flow_start=rng.random() < 0.5, linked=rng.choice([None, None, 5, -9, 2**40 + 1]))

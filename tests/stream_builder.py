@@ -26,6 +26,7 @@ class StreamBuilder:
         self.end_time = self.window[1] if end_time is None else end_time
         self.generic, self.runtime, self.device, self.extcorr = [], [], [], []
         self.device_infos, self.resource_infos, self.overhead_infos, self.spans = [], [], [], []
+        self.collectives = []
         self._keep = []
 
     # ---- dictionary / schemas ----
@@ -41,6 +42,16 @@ class StreamBuilder:
             self.fields.append((abi.KTJ_NONE if key is None else self.s(key), typ, cnt))
         self.schemas.append((first, len(fields)))
         return len(self.schemas) - 1
+
+    def add_collective(self, **values):
+        """One record_param_comms op's metadata values (abi.COLLECTIVE_KEYS, as getMetadataValue()
+        returns them); returns the index for the slot of a leading F_COLLECTIVE field."""
+        m = abi.CollectiveMeta()
+        for k, v in values.items():
+            assert k in abi.COLLECTIVE_KEYS, k
+            setattr(m, k, v.encode("latin1") if isinstance(v, str) else v)
+        self.collectives.append(m)
+        return len(self.collectives) - 1
 
     def arg_slots(self, values):
         off = len(self.args)
@@ -158,7 +169,7 @@ class StreamBuilder:
                                    ("device_infos", abi.DeviceInfo, self.device_infos),
                                    ("resource_infos", abi.ResourceInfo, self.resource_infos),
                                    ("overhead_infos", abi.OverheadInfo, self.overhead_infos),
-                                   ("spans", abi.TraceSpan, self.spans)):
+                                   ("spans", abi.TraceSpan, self.spans), ("collectives", abi.CollectiveMeta, self.collectives)):
             setattr(st, name, self._arr(ctype, items))
             setattr(st, "n_" + name, len(items))
         self._keep.append(st)

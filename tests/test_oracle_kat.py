@@ -16,6 +16,20 @@ def test_known_answers(case):
         assert e in out, f"missing {e!r} in\n{out}"
 
 
+@pytest.mark.parametrize("quoted", [False, True])
+def test_collective_metadata_expectations_of_the_reference_test(quoted):
+    """libkineto/test/OutputJsonTest.cpp:186-225: the document parses as JSON and the kernel's args
+    and "distributedInfo" equal the expected objects, for quoted and bare string values alike."""
+    import json
+    b, _ = kat_cases.case_collective_reference_test(quoted)
+    o = og.OracleRun(b.build())
+    trace = json.loads(o.output().decode())
+    o.close()
+    args = [e["args"] for e in trace["traceEvents"] if e.get("name") == "nccl:all_reduce"]
+    assert args == [kat_cases.COLLECTIVE_REF_ARGS]
+    assert trace["distributedInfo"] == kat_cases.COLLECTIVE_REF_DIST
+
+
 def test_rocm_sync_trace_counts():
     b, counts = kat_cases.case_rocm_sync_trace()
     o = og.OracleRun(b.build())
