@@ -2,15 +2,18 @@
  * GpuChromeTraceLogger.cpp — see GpuChromeTraceLogger.h.
  *
  * Per-record work on the host is limited to reading the activity's accessors once, interning
- * its name and its metadataJson() text in a string dictionary, and appending one 64-byte packed
- * record; sorting, sizing and all formatting happen on the GPU in ktj_finalize.
+ * its name in a string dictionary, appending its metadataJson() text to a blob, and appending one
+ * 64-byte packed record; sorting, sizing and all formatting happen on the GPU in ktj_finalize.
  */
 #include "GpuChromeTraceLogger.h"
 
+#include <algorithm>
 #include <cstring>
 #include <limits>
+#include <thread>
 
 #include "EnvMetadata.h"
+#include "GenericTraceActivity.h"
 #include "ITraceActivity.h"
 #include "Logger.h"
 #include "TraceSpan.h"
@@ -26,7 +29,65 @@ constexpr size_t kStringBatchBytes = 16u << 20; /* dictionary bytes per ktj_inte
 constexpr const char* kParamCommsName = "record_param_comms"; /* output_json.cpp: kParamCommsCallName */
 }  // namespace
 
-GpuChromeTraceLogger::GpuChromeTraceLogger(const std::string& traceFileName, int hipDevice) : fileName_(traceFileName) {
+/* ---- packing: activity -> 64-byte record, with ids local to the packer ---- */
+
+namespace {
+const char* const kCollectiveKeys[] = {"Collective name", "In msg nelems", "Out msg nelems", "Group size", "dtype",
+                                       "Input Tensors start", "Output Tensors start", "In split size", "Out split size",
+                                       "Process Group Name", "Process Group Description", "Process Group Ranks",
+                                       "Dst Rank", "Src Rank", "Seq", "Comms Id", "Rank"};
+constexpr size_t kCollectiveKeyCount = sizeof(kCollectiveKeys) / sizeof(kCollectiveKeys[0]);
+static_assert(kCollectiveKeyCount * sizeof(const char*) == sizeof(ktj_collective_meta), "one key per field of ktj_collective_meta");
+
+/* schema codes inside a Packed (KTJ_NONE = no metadata) */
+constexpr uint32_t kLocalFragment = 0, kLocalCollective = 1, kLocalCollectiveFragment = 2, kLocalCounterBase = 3;
+/* what a slot holds, for the translation to engine ids */
+constexpr uint8_t kSlotPlain = 0, kSlotFragment = 1, kSlotCollective = 2;
+}  // namespace
+
+/* The output of one packer: records whose string ids, schema ids, collective indices and slot
+ * offsets are local to it, plus the local dictionaries.  A packer touches no logger state, so
+ * several can run at once on disjoint activities; merge() translates to engine ids. */
+struct GpuChromeTraceLogger::Packed {
+  std::vector<ktj_generic_rec> records;
+  std::vector<uint64_t> origin;    /* position of each record in the caller's sequence */
+  std::vector<uint64_t> slots;
+  std::vector<uint8_t> slotKind;
+  std::vector<std::string> names; /* activity and counter names: few distinct ones, kept once */
+  std::unordered_map<std::string, uint32_t> nameIndex;
+  std::string fragmentBlob;       /* metadataJson() texts: nearly all distinct (sequence numbers, */
+  std::vector<uint64_t> fragmentEnd; /* correlation ids), so they are stored as they come         */
+  std::vector<std::string> collectives; /* the 17 values of an op, each followed by NUL */
+  std::unordered_map<std::string, uint32_t> collectiveIndex;
+  std::vector<std::vector<uint32_t>> counterSchemas; /* local ids of the counter names */
+  std::unordered_map<std::string, uint32_t> counterIndex;
+  uint64_t unsupported = 0;
+  std::string firstUnsupported;
+  /* engine ids of the local entries translated so far (merge) */
+  std::vector<uint32_t> nameGlobal, collectiveGlobal, counterGlobal;
+  uint32_t fragmentBase = 0; /* engine id of local fragment 0 */
+
+  uint32_t name(const std::string& s) {
+    auto it = nameIndex.find(s);
+    if (it != nameIndex.end()) return it->second;
+    const uint32_t id = static_cast<uint32_t>(names.size());
+    nameIndex.emplace(s, id);
+    names.push_back(s);
+    return id;
+  }
+  uint32_t fragment(const std::string& s) {
+    fragmentBlob.append(s);
+    fragmentEnd.push_back(fragmentBlob.size());
+    return static_cast<uint32_t>(fragmentEnd.size() - 1);
+  }
+  void slot(uint64_t v, uint8_t kind) { slots.push_back(v); slotKind.push_back(kind); }
+  void clearRecords() {
+    records.clear(); origin.clear(); slots.clear(); slotKind.clear(); fragmentBlob.clear(); fragmentEnd.clear();
+  }
+};
+
+GpuChromeTraceLogger::GpuChromeTraceLogger(const std::string& traceFileName, int hipDevice)
+    : fileName_(traceFileName), staging_(new Packed) {
   /* the engine applies the default-file-name rule (output_json.cpp:481-483) for an empty name */
   const int rc = ktj_create(&engine_, traceFileName.c_str(), ChromeTraceBaseTime::singleton().get(), hipDevice, 0);
   if (rc != KTJ_OK) {
@@ -55,62 +116,186 @@ void GpuChromeTraceLogger::note(int rc, const char* what) {
   LOG(ERROR) << what << " failed (rc=" << rc << "): " << (engine_ ? ktj_last_error(engine_) : "");
 }
 
-uint32_t GpuChromeTraceLogger::intern(std::unordered_map<std::string, uint32_t>& index, const std::string& s) {
-  auto it = index.find(s);
-  if (it != index.end()) return it->second;
+/* ---- packing: one activity -> one record in a Packed ---- */
+
+/* Reads the activity's accessors once and appends one record (what ChromeTraceLogger::handleActivity
+ * reads, output_json.cpp:837-963). */
+void GpuChromeTraceLogger::pack(const ITraceActivity& op, uint64_t origin, Packed& out) {
+  const ActivityType type = op.type();
+  const std::string name = op.name();
+  const ITraceActivity* linked = op.linkedActivity();
+  const int64_t device = op.deviceId();
+  const bool counter = type == ActivityType::HARDWARE_COUNTERS || type == ActivityType::MTIA_COUNTERS ||
+      type == ActivityType::XPU_SCOPE_PROFILER; /* output_json.cpp:847-856 */
+  /* collective metadata comes from a linked record_param_comms op (output_json.cpp:899-908) */
+  const bool collective = !counter && linked != nullptr &&
+      (type == ActivityType::CONCURRENT_KERNEL || (type == ActivityType::MTIA_CCP_EVENTS && name.rfind("hccl::", 0) == 0)) &&
+      linked->name() == kParamCommsName;
+  if (device < std::numeric_limits<int32_t>::min() || device > std::numeric_limits<int32_t>::max()) {
+    if (out.unsupported++ == 0) out.firstUnsupported = name;
+    return;
+  }
+  ktj_generic_rec r{};
+  r.start_ns = op.timestamp();
+  r.end_ns = r.start_ns + op.duration();
+  r.resource = op.resourceId();
+  r.device = static_cast<int32_t>(device);
+  r.id = static_cast<int32_t>(op.correlationId()); /* `int external_id = op.correlationId()`, :893 */
+  r.type = static_cast<uint8_t>(type);
+  r.name_id = out.name(name);
+  r.flow_id = op.flowId();
+  const int flowType = op.flowType(); /* anything but the two known kinds prints no flow event (:979-994) */
+  r.flow_type = (flowType == static_cast<int>(KTJ_LINK_FWDBWD) || flowType == static_cast<int>(KTJ_LINK_ASYNC_CPU_GPU)) ? static_cast<uint8_t>(flowType) : 0;
+  r.flags = op.flowStart() ? KTJ_GF_FLOW_START : 0;
+  if (linked != nullptr) {
+    r.flags |= KTJ_GF_LINKED;
+    r.linked_id = static_cast<int32_t>(linked->correlationId()); /* `int external_id = …`, :873 */
+  }
+  r.schema_id = KTJ_NONE;
+  r.args_off = out.slots.size();
+  if (counter) { /* handleCounterEvent (:679-716) prints counterValues() and nothing else */
+    const auto& values = op.counterValues();
+    if (!values.empty()) { /* one schema per distinct list of counter names: a keyed double field for each */
+      std::vector<uint32_t> names;
+      names.reserve(values.size());
+      for (const auto& kv : values) names.push_back(out.name(kv.first));
+      const std::string key(reinterpret_cast<const char*>(names.data()), names.size() * sizeof(uint32_t));
+      auto it = out.counterIndex.find(key);
+      if (it == out.counterIndex.end()) {
+        it = out.counterIndex.emplace(key, static_cast<uint32_t>(out.counterSchemas.size())).first;
+        out.counterSchemas.push_back(std::move(names));
+      }
+      r.schema_id = kLocalCounterBase + it->second;
+      for (const auto& kv : values) {
+        uint64_t bits;
+        static_assert(sizeof(bits) == sizeof(kv.second), "double is 64 bits");
+        std::memcpy(&bits, &kv.second, sizeof(bits));
+        out.slot(bits, kSlotPlain);
+      }
+    }
+  } else {
+    const std::string metadata = op.metadataJson();
+    if (collective) { /* the first slot names the linked op's collective metadata */
+      std::string key;
+      for (size_t i = 0; i < kCollectiveKeyCount; ++i) {
+        key += linked->getMetadataValue(kCollectiveKeys[i]);
+        key += '\0';
+      }
+      auto it = out.collectiveIndex.find(key);
+      if (it == out.collectiveIndex.end()) {
+        it = out.collectiveIndex.emplace(key, static_cast<uint32_t>(out.collectives.size())).first;
+        out.collectives.push_back(key);
+      }
+      r.schema_id = metadata.empty() ? kLocalCollective : kLocalCollectiveFragment;
+      out.slot(it->second, kSlotCollective);
+    } else if (!metadata.empty()) {
+      r.schema_id = kLocalFragment;
+    }
+    if (!metadata.empty()) out.slot(out.fragment(metadata), kSlotFragment);
+  }
+  out.records.push_back(r);
+  out.origin.push_back(origin);
+}
+
+/* ---- merging: local ids -> engine ids ---- */
+
+uint32_t GpuChromeTraceLogger::intern(const std::string& s) {
+  auto it = strings_.find(s);
+  if (it != strings_.end()) return it->second;
   const uint32_t id = nextStringId_++;
-  index.emplace(s, id);
+  strings_.emplace(s, id);
   pendingBlob_.append(s);
   pendingOffsets_.push_back(pendingBlob_.size());
   if (pendingBlob_.size() >= kStringBatchBytes) flushStrings();
   return id;
 }
 
-/* The values ChromeTraceLogger::appendCollectiveMetadata reads from a record_param_comms op
- * (output_json.cpp:718-835), handed to the engine once per distinct set of values. */
-uint32_t GpuChromeTraceLogger::collectiveIndex(const ITraceActivity& op) {
-  static const char* const kKeys[] = {"Collective name", "In msg nelems", "Out msg nelems", "Group size", "dtype",
-                                      "Input Tensors start", "Output Tensors start", "In split size", "Out split size",
-                                      "Process Group Name", "Process Group Description", "Process Group Ranks",
-                                      "Dst Rank", "Src Rank", "Seq", "Comms Id", "Rank"};
-  constexpr size_t kCount = sizeof(kKeys) / sizeof(kKeys[0]);
-  static_assert(kCount * sizeof(const char*) == sizeof(ktj_collective_meta), "one key per field of ktj_collective_meta");
-  std::string values[kCount];
-  std::string key;
-  for (size_t i = 0; i < kCount; ++i) {
-    values[i] = op.getMetadataValue(kKeys[i]);
-    key += values[i];
-    key += '\0';
+/* Brings the packer's dictionaries up to date with the engine's: every local string, collective
+ * entry and counter schema that has no engine id yet gets one. */
+void GpuChromeTraceLogger::translate(Packed& p) {
+  if (p.unsupported != 0) {
+    if (unsupported_ == 0) {
+      LOG(WARNING) << "GpuChromeTraceLogger: activity '" << p.firstUnsupported
+                   << "' has a deviceId outside 32 bits; such activities are dropped";
+    }
+    unsupported_ += p.unsupported;
+    p.unsupported = 0;
   }
-  auto it = collectives_.find(key);
-  if (it != collectives_.end()) return it->second;
-  const ktj_collective_meta meta = {
-      values[0].c_str(),  values[1].c_str(),  values[2].c_str(),  values[3].c_str(),  values[4].c_str(),  values[5].c_str(),
-      values[6].c_str(),  values[7].c_str(),  values[8].c_str(),  values[9].c_str(),  values[10].c_str(), values[11].c_str(),
-      values[12].c_str(), values[13].c_str(), values[14].c_str(), values[15].c_str(), values[16].c_str()}; /* kKeys order */
-  uint32_t index = 0;
-  note(ktj_add_collective(engine_, &meta, &index), "ktj_add_collective");
-  collectives_.emplace(std::move(key), index);
-  return index;
+  for (size_t i = p.nameGlobal.size(); i < p.names.size(); ++i) p.nameGlobal.push_back(intern(p.names[i]));
+  /* the fragments of this batch get consecutive ids */
+  p.fragmentBase = nextStringId_;
+  if (!p.fragmentEnd.empty()) {
+    const uint64_t at = pendingBlob_.size();
+    pendingBlob_.append(p.fragmentBlob);
+    pendingOffsets_.reserve(pendingOffsets_.size() + p.fragmentEnd.size());
+    for (uint64_t end : p.fragmentEnd) pendingOffsets_.push_back(at + end);
+    nextStringId_ += static_cast<uint32_t>(p.fragmentEnd.size());
+    if (pendingBlob_.size() >= kStringBatchBytes) flushStrings();
+  }
+  for (size_t i = p.collectiveGlobal.size(); i < p.collectives.size(); ++i) {
+    const std::string& key = p.collectives[i];
+    auto it = collectives_.find(key);
+    if (it == collectives_.end()) {
+      /* the values ChromeTraceLogger::appendCollectiveMetadata reads (output_json.cpp:718-835), handed
+       * to the engine once per distinct set */
+      const char* v[kCollectiveKeyCount];
+      const char* q = key.c_str();
+      for (size_t k = 0; k < kCollectiveKeyCount; ++k) { v[k] = q; q += std::strlen(q) + 1; }
+      const ktj_collective_meta meta = {v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8],
+                                        v[9], v[10], v[11], v[12], v[13], v[14], v[15], v[16]}; /* kCollectiveKeys order */
+      uint32_t index = 0;
+      note(ktj_add_collective(engine_, &meta, &index), "ktj_add_collective");
+      it = collectives_.emplace(key, index).first;
+    }
+    p.collectiveGlobal.push_back(it->second);
+  }
+  for (size_t i = p.counterGlobal.size(); i < p.counterSchemas.size(); ++i) {
+    std::vector<ktj_field> fields;
+    fields.reserve(p.counterSchemas[i].size());
+    for (uint32_t local : p.counterSchemas[i]) fields.push_back(ktj_field{p.nameGlobal[local], KTJ_F_F64, 1});
+    const std::string key(reinterpret_cast<const char*>(fields.data()), fields.size() * sizeof(ktj_field));
+    auto it = counterSchemas_.find(key);
+    if (it == counterSchemas_.end()) {
+      uint32_t sid = KTJ_NONE;
+      note(ktj_register_schema(engine_, fields.data(), fields.size(), &sid), "ktj_register_schema");
+      it = counterSchemas_.emplace(key, sid).first;
+    }
+    p.counterGlobal.push_back(it->second);
+  }
 }
 
-/* One schema per distinct list of counter names: a keyed double field for each. */
-uint32_t GpuChromeTraceLogger::counterSchema(const std::vector<std::pair<std::string, double>>& values) {
-  if (values.empty()) return KTJ_NONE;
-  std::string key;
-  std::vector<ktj_field> fields;
-  fields.reserve(values.size());
-  for (const auto& kv : values) {
-    const uint32_t id = intern(names_, kv.first);
-    fields.push_back(ktj_field{id, KTJ_F_F64, 1});
-    key.append(reinterpret_cast<const char*>(&id), sizeof(id));
+/* Appends the packer's slots to the pending args and returns where they start. */
+uint64_t GpuChromeTraceLogger::appendSlots(const Packed& p) {
+  const uint64_t base = nextSlot_;
+  slots_.reserve(slots_.size() + p.slots.size());
+  for (size_t i = 0; i < p.slots.size(); ++i) {
+    const uint64_t v = p.slots[i];
+    slots_.push_back(p.slotKind[i] == kSlotFragment ? p.fragmentBase + v : p.slotKind[i] == kSlotCollective ? p.collectiveGlobal[v] : v);
   }
-  auto it = counterSchemas_.find(key);
-  if (it != counterSchemas_.end()) return it->second;
-  uint32_t sid = KTJ_NONE;
-  note(ktj_register_schema(engine_, fields.data(), fields.size(), &sid), "ktj_register_schema");
-  counterSchemas_.emplace(std::move(key), sid);
-  return sid;
+  nextSlot_ += p.slots.size();
+  return base;
+}
+
+ktj_generic_rec GpuChromeTraceLogger::translated(const Packed& p, size_t i, uint64_t slotBase) const {
+  ktj_generic_rec r = p.records[i];
+  r.name_id = p.nameGlobal[r.name_id];
+  r.args_off += slotBase;
+  if (r.schema_id == kLocalFragment) r.schema_id = fragmentSchema_;
+  else if (r.schema_id == kLocalCollective) r.schema_id = collectiveSchema_;
+  else if (r.schema_id == kLocalCollectiveFragment) r.schema_id = collectiveFragmentSchema_;
+  else if (r.schema_id != KTJ_NONE) r.schema_id = p.counterGlobal[r.schema_id - kLocalCounterBase];
+  return r;
+}
+
+/* One packer whose records are already in arrival order. */
+void GpuChromeTraceLogger::mergeInOrder(Packed& p) {
+  translate(p);
+  const uint64_t base = appendSlots(p);
+  records_.reserve(records_.size() + p.records.size());
+  for (size_t i = 0; i < p.records.size(); ++i) records_.push_back(translated(p, i, base));
+  p.clearRecords();
+  flushStrings();
+  flushRecords();
 }
 
 void GpuChromeTraceLogger::flushStrings() {
@@ -178,75 +363,55 @@ void GpuChromeTraceLogger::handleTraceSpan(const TraceSpan& span) {
 
 void GpuChromeTraceLogger::handleActivity(const ITraceActivity& op) {
   if (!ok()) return;
-  const ActivityType type = op.type();
-  const std::string name = op.name();
-  const ITraceActivity* linked = op.linkedActivity();
-  const int64_t device = op.deviceId();
-  const int64_t flowId = op.flowId();
-  const bool counter = type == ActivityType::HARDWARE_COUNTERS || type == ActivityType::MTIA_COUNTERS ||
-      type == ActivityType::XPU_SCOPE_PROFILER; /* output_json.cpp:847-856 */
-  /* collective metadata comes from a linked record_param_comms op (output_json.cpp:899-908) */
-  const bool collective = !counter && linked != nullptr &&
-      (type == ActivityType::CONCURRENT_KERNEL || (type == ActivityType::MTIA_CCP_EVENTS && name.rfind("hccl::", 0) == 0)) &&
-      linked->name() == kParamCommsName;
-  const bool unsupported = device < std::numeric_limits<int32_t>::min() || device > std::numeric_limits<int32_t>::max();
-  if (unsupported) {
-    if (unsupported_++ == 0) {
-      LOG(WARNING) << "GpuChromeTraceLogger: activity '" << name << "' of type " << toString(type)
-                   << " is of a kind the GPU engine does not render; such activities are dropped";
-    }
-    return;
-  }
+  pack(op, 0, *staging_);
+  if (staging_->records.size() >= kRecordBatch) mergeInOrder(*staging_);
+}
 
-  ktj_generic_rec r{};
-  r.start_ns = op.timestamp();
-  r.end_ns = r.start_ns + op.duration();
-  r.resource = op.resourceId();
-  r.device = static_cast<int32_t>(device);
-  r.id = static_cast<int32_t>(op.correlationId()); /* `int external_id = op.correlationId()`, :893 */
-  r.type = static_cast<uint8_t>(type);
-  r.name_id = intern(names_, name);
-  r.flow_id = flowId;
-  const int flowType = op.flowType(); /* anything but the two known kinds prints no flow event (:979-994) */
-  r.flow_type = (flowType == static_cast<int>(KTJ_LINK_FWDBWD) || flowType == static_cast<int>(KTJ_LINK_ASYNC_CPU_GPU)) ? static_cast<uint8_t>(flowType) : 0;
-  r.flags = op.flowStart() ? KTJ_GF_FLOW_START : 0;
-  if (linked != nullptr) {
-    r.flags |= KTJ_GF_LINKED;
-    r.linked_id = static_cast<int32_t>(linked->correlationId()); /* `int external_id = …`, :873 */
-  }
-  if (counter) { /* handleCounterEvent (:679-716) prints counterValues() and nothing else */
-    const auto& values = op.counterValues();
-    r.schema_id = counterSchema(values);
-    r.args_off = nextSlot_;
-    nextSlot_ += values.size();
-    for (const auto& kv : values) {
-      uint64_t bits;
-      static_assert(sizeof(bits) == sizeof(kv.second), "double is 64 bits");
-      std::memcpy(&bits, &kv.second, sizeof(bits));
-      slots_.push_back(bits);
+/* The replay loop of a buffering logger (MemoryTraceLogger::log, libkineto/src/output_membuf.h:91-107:
+ * `for (auto& activity : activities_) activity->log(logger)`) as one call.  The host gather runs
+ * on `threads` workers: each packs the GenericTraceActivity objects of one contiguous slice.  Every
+ * other kind of activity is packed by the calling thread, in order: the ROCm wrappers hand grid,
+ * block and size from the runtime row to the device row through thread_local maps inside
+ * metadataJson() (libkineto/src/RocprofActivity_inl.h:28-30, 163-180, 221-232), so they must stay on
+ * one thread and in sequence.  The records reach the engine in the order of `activities`. */
+void GpuChromeTraceLogger::handleActivities(const std::vector<const ITraceActivity*>& activities, unsigned threads) {
+  if (!ok() || activities.empty()) return;
+  mergeInOrder(*staging_); /* what single calls left behind comes first */
+  const size_t n = activities.size();
+  if (threads == 0) threads = std::max(1u, std::thread::hardware_concurrency());
+  threads = static_cast<unsigned>(std::min<size_t>(threads, (n + 4095) / 4096));
+  std::vector<uint8_t> generic(n);
+  for (size_t i = 0; i < n; ++i) generic[i] = dynamic_cast<const GenericTraceActivity*>(activities[i]) != nullptr;
+  std::vector<Packed> parts(threads + 1); /* parts[threads]: the calling thread's, everything that is not generic */
+  auto work = [&](unsigned w) {
+    const size_t lo = n * w / threads, hi = n * (w + 1) / threads;
+    for (size_t i = lo; i < hi; ++i)
+      if (generic[i]) pack(*activities[i], i, parts[w]);
+  };
+  std::vector<std::thread> pool;
+  for (unsigned w = 1; w < threads; ++w) pool.emplace_back(work, w);
+  for (size_t i = 0; i < n; ++i)
+    if (!generic[i]) pack(*activities[i], i, parts[threads]);
+  work(0);
+  for (auto& t : pool) t.join();
+
+  /* merge: which packer holds position i, and where */
+  constexpr uint32_t kNobody = 0xFFFFFFFFu;
+  std::vector<uint32_t> owner(n, kNobody), at(n, 0);
+  std::vector<uint64_t> base(parts.size());
+  for (size_t w = 0; w < parts.size(); ++w) {
+    translate(parts[w]);
+    base[w] = appendSlots(parts[w]);
+    for (size_t j = 0; j < parts[w].records.size(); ++j) {
+      owner[parts[w].origin[j]] = static_cast<uint32_t>(w);
+      at[parts[w].origin[j]] = static_cast<uint32_t>(j);
     }
-    records_.push_back(r);
-    if (records_.size() >= kRecordBatch) flushRecords();
-    return;
   }
-  const std::string metadata = op.metadataJson();
-  if (collective) { /* the first slot names the linked op's collective metadata */
-    r.schema_id = metadata.empty() ? collectiveSchema_ : collectiveFragmentSchema_;
-    r.args_off = nextSlot_++;
-    slots_.push_back(collectiveIndex(*linked));
-    if (!metadata.empty()) {
-      ++nextSlot_;
-      slots_.push_back(intern(fragments_, metadata));
-    }
-  } else if (metadata.empty()) {
-    r.schema_id = KTJ_NONE;
-  } else {
-    r.schema_id = fragmentSchema_;
-    r.args_off = nextSlot_++;
-    slots_.push_back(intern(fragments_, metadata));
-  }
-  records_.push_back(r);
-  if (records_.size() >= kRecordBatch) flushRecords();
+  records_.reserve(n);
+  for (size_t i = 0; i < n; ++i)
+    if (owner[i] != kNobody) records_.push_back(translated(parts[owner[i]], at[i], base[owner[i]]));
+  flushStrings();
+  flushRecords();
 }
 
 void GpuChromeTraceLogger::handleGenericActivity(const GenericTraceActivity& op) {
@@ -267,8 +432,7 @@ void GpuChromeTraceLogger::finalizeTrace(int64_t endTime) {
     LOG(ERROR) << "Failed to write to log file!";
     return;
   }
-  flushStrings();
-  flushRecords();
+  mergeInOrder(*staging_);
   uint64_t written = 0;
   if (status_ == 0) note(ktj_finalize(engine_, endTime, &written), "ktj_finalize");
   if (status_ != 0) {

@@ -45,6 +45,10 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
   void handleTraceSpan(const libkineto::TraceSpan& span) override;
   void handleActivity(const libkineto::ITraceActivity& activity) override;
   void handleGenericActivity(const libkineto::GenericTraceActivity& activity) override;
+  /* Every activity of a buffering logger's replay loop (libkineto/src/output_membuf.h:91-107) in
+   * one call, equivalent to handleActivity() on each in turn; the host-side packing of
+   * GenericTraceActivity objects is spread over `threads` workers (0 = one per core). */
+  void handleActivities(const std::vector<const libkineto::ITraceActivity*>& activities, unsigned threads = 0);
   void handleTraceStart(const std::unordered_map<std::string, std::string>& metadata,
                         const std::string& device_properties) override;
   void finalizeMemoryTrace(const std::string&, const libkineto::Config&) override;
@@ -61,9 +65,13 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
   void finalizeTrace(int64_t endTime); /* output_json.h: protected finalizeTrace(int64_t) */
 
  private:
-  uint32_t intern(std::unordered_map<std::string, uint32_t>& index, const std::string& s);
-  uint32_t collectiveIndex(const libkineto::ITraceActivity& op);
-  uint32_t counterSchema(const std::vector<std::pair<std::string, double>>& values);
+  struct Packed;
+  static void pack(const libkineto::ITraceActivity& op, uint64_t origin, Packed& out);
+  uint32_t intern(const std::string& s);
+  void translate(Packed& p);
+  uint64_t appendSlots(const Packed& p);
+  ktj_generic_rec translated(const Packed& p, size_t i, uint64_t slotBase) const;
+  void mergeInOrder(Packed& p);
   void flushStrings();
   void flushRecords();
   bool ok() const { return engine_ != nullptr && status_ == 0; }
@@ -78,10 +86,10 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
   uint32_t collectiveFragmentSchema_ = KTJ_NONE; /* collective metadata + fragment  */
 
   /* strings not yet handed to the engine: blob + offsets, ids are consecutive from nextStringId_ */
-  std::unordered_map<std::string, uint32_t> names_;
-  std::unordered_map<std::string, uint32_t> fragments_;
-  std::unordered_map<std::string, uint32_t> collectives_;    /* key: the 17 values, NUL-separated */
-  std::unordered_map<std::string, uint32_t> counterSchemas_; /* key: the name ids, 4 bytes each */
+  std::unordered_map<std::string, uint32_t> strings_;        /* activity and counter names */
+  std::unordered_map<std::string, uint32_t> collectives_;    /* key: the 17 values, each followed by NUL */
+  std::unordered_map<std::string, uint32_t> counterSchemas_; /* key: the fields' bytes */
+  std::unique_ptr<Packed> staging_;                          /* packer of the single-activity calls */
   std::string pendingBlob_;
   std::vector<uint64_t> pendingOffsets_;
   uint32_t nextStringId_ = 0;

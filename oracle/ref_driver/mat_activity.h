@@ -151,13 +151,37 @@ struct MatActivity : public ITraceActivity {
   }
 };
 
+// The same activity as a GenericTraceActivity (what a buffering logger's replay loop mostly holds):
+// every accessor forwards to the MatActivity.
+struct GenericMatActivity : public GenericTraceActivity {
+  const MatActivity* m;
+  explicit GenericMatActivity(const MatActivity* mat) : m(mat) {}
+  int64_t deviceId() const override { return m->deviceId(); }
+  int64_t resourceId() const override { return m->resourceId(); }
+  int32_t getThreadId() const override { return m->getThreadId(); }
+  int64_t timestamp() const override { return m->timestamp(); }
+  int64_t duration() const override { return m->duration(); }
+  int64_t correlationId() const override { return m->correlationId(); }
+  int flowType() const override { return m->flowType(); }
+  int64_t flowId() const override { return m->flowId(); }
+  bool flowStart() const override { return m->flowStart(); }
+  ActivityType type() const override { return m->type(); }
+  const std::string name() const override { return m->name(); }
+  const ITraceActivity* linkedActivity() const override { return m->linkedActivity(); }
+  const TraceSpan* traceSpan() const override { return nullptr; }
+  void log(ActivityLogger& logger) const override { logger.handleActivity(*this); }
+  const std::string metadataJson() const override { return m->metadataJson(); }
+  const std::vector<std::pair<std::string, double>>& counterValues() const override { return m->counterValues(); }
+};
+
 // Replays one stream into a logger in the order of the reference's buffering logger
 // (src/output_membuf.h:91-107): trace start, device / resource / overhead infos, the activities
 // stable-sorted by (deviceId, resourceId, timestamp), spans, finalizeTrace(endTime).  L must
-// expose finalizeTrace(int64_t).
-template <class L>
+// expose finalizeTrace(int64_t).  `log_all` hands the sorted activities to the logger; the default
+// is the replay loop of src/output_membuf.h:101-103, one log() call each.
+template <class L, class LogAll>
 void replay_stream(L& logger, const ktj_stream* s, const ktj_mat_activity* acts, uint64_t n_acts, string_fn fn,
-                   const void* ctx) {
+                   const void* ctx, LogAll log_all) {
   StringTable st{fn, ctx};
   std::vector<MatActivity> wrapped;
   wrapped.reserve(n_acts);
@@ -184,7 +208,7 @@ void replay_stream(L& logger, const ktj_stream* s, const ktj_mat_activity* acts,
   for (uint64_t i = 0; i < s->n_overhead_infos; ++i) {
     logger.handleOverheadInfo(ActivityLogger::OverheadInfo(s->overhead_infos[i].name), s->overhead_infos[i].time_ns);
   }
-  for (const MatActivity* a : order) a->log(logger);
+  log_all(logger, order);
   for (uint64_t i = 0; i < s->n_spans; ++i) {
     const ktj_trace_span& sp = s->spans[i];
     TraceSpan span(sp.op_count, sp.iteration, sp.name, sp.prefix);
@@ -193,6 +217,14 @@ void replay_stream(L& logger, const ktj_stream* s, const ktj_mat_activity* acts,
     logger.handleTraceSpan(span);
   }
   logger.finalizeTrace(s->end_time_ns);
+}
+
+template <class L>
+void replay_stream(L& logger, const ktj_stream* s, const ktj_mat_activity* acts, uint64_t n_acts, string_fn fn,
+                   const void* ctx) {
+  replay_stream(logger, s, acts, n_acts, fn, ctx, [](L& l, const std::vector<const MatActivity*>& order) {
+    for (const MatActivity* a : order) a->log(l);
+  });
 }
 
 }  // namespace ktj_ref_driver

@@ -7,9 +7,11 @@
  *
  * TEST INFRASTRUCTURE ONLY; this repository's own code.
  */
+#include <chrono>
 #include <memory>
 #include <stdexcept>
 #include <string>
+#include <vector>
 
 #include "ActivityLoggerFactory.h"
 #include "Logger.h"
@@ -34,8 +36,10 @@ int64_t ktj_shim_base_time(void) { return ChromeTraceBaseTime::singleton().get()
 // url is "<protocol>://<path>"; the protocol is registered here with a factory that builds the
 // shim.  Returns 0, -2 for a base-time mismatch, -3 if the factory did not produce the shim,
 // else the shim's engine status.  *unsupported receives the number of dropped activities.
+// bulk_threads > 0: the activities are handed over in one handleActivities() call with that many
+// workers, as GenericTraceActivity objects (so that the workers pack them).
 int ktj_shim_render(const ktj_stream* s, const ktj_mat_activity* acts, uint64_t n_acts, string_fn fn,
-                    const void* ctx, const char* url, int hip_device, uint64_t* unsupported) {
+                    const void* ctx, const char* url, int hip_device, uint64_t* unsupported, int bulk_threads) {
   SET_LOG_SEVERITY_LEVEL(3);
   if (s->base_time_ns != ChromeTraceBaseTime::singleton().get()) return -2;
   ActivityLoggerFactory factory;
@@ -50,9 +54,57 @@ int ktj_shim_render(const ktj_stream* s, const ktj_mat_activity* acts, uint64_t 
   }
   auto* shim = dynamic_cast<ShimLogger*>(logger.get());
   if (shim == nullptr) return -3;
-  replay_stream(*shim, s, acts, n_acts, fn, ctx);
+  if (bulk_threads > 0) {
+    replay_stream(*shim, s, acts, n_acts, fn, ctx, [bulk_threads](ShimLogger& l, const std::vector<const MatActivity*>& order) {
+      std::vector<GenericMatActivity> generic;
+      generic.reserve(order.size());
+      std::vector<const ITraceActivity*> all;
+      all.reserve(order.size());
+      for (size_t i = 0; i < order.size(); ++i) {
+        if (i % 7 == 3) all.push_back(order[i]); /* some stay plain ITraceActivity: packed by the calling thread */
+        else { generic.emplace_back(order[i]); all.push_back(&generic.back()); }
+      }
+      l.handleActivities(all, static_cast<unsigned>(bulk_threads));
+    });
+  } else {
+    replay_stream(*shim, s, acts, n_acts, fn, ctx);
+  }
   if (unsupported) *unsupported = shim->unsupportedActivities();
   return shim->engineStatus();
+}
+
+// Times handleActivities() alone (host-side packing, merge and hand-over to the engine; no
+// finalizeTrace) on n CPU-op activities with typed metadata, as a profiler's CpuTraceBuffer holds
+// them.  Returns the engine status; *seconds receives the wall time of the call.
+int ktj_shim_time_bulk(uint64_t n, int threads, const char* path, int hip_device, double* seconds) {
+  SET_LOG_SEVERITY_LEVEL(3);
+  ShimLogger shim(path, hip_device);
+  shim.handleTraceStart({}, "");
+  TraceSpan span(0, 0, "bench");
+  std::vector<GenericTraceActivity> acts;
+  acts.reserve(n);
+  const int64_t base = ChromeTraceBaseTime::singleton().get();
+  for (uint64_t i = 0; i < n; ++i) {
+    acts.emplace_back(span, ActivityType::CPU_OP, "aten::op_" + std::to_string(i % 997));
+    GenericTraceActivity& a = acts.back();
+    a.startTime = base + static_cast<int64_t>(i) * 1000;
+    a.endTime = a.startTime + 500;
+    a.device = 4000;
+    a.resource = 4001 + static_cast<int32_t>(i % 8);
+    a.id = static_cast<int32_t>(i + 1);
+    a.addMetadata("Sequence number", static_cast<int64_t>(i));
+    a.addMetadata("Fwd thread id", 0);
+    a.addMetadataQuoted("Input type", "float");
+  }
+  std::vector<const ITraceActivity*> all;
+  all.reserve(n);
+  for (const auto& a : acts) all.push_back(&a);
+  const auto t0 = std::chrono::steady_clock::now();
+  shim.handleActivities(all, static_cast<unsigned>(threads));
+  const auto t1 = std::chrono::steady_clock::now();
+  if (seconds) *seconds = std::chrono::duration<double>(t1 - t0).count();
+  shim.finalizeTrace(base + static_cast<int64_t>(n) * 1000 + 1000);
+  return shim.engineStatus();
 }
 
 }  // extern "C"

@@ -104,7 +104,7 @@ def load_shim():
         lib.ktj_shim_base_time.restype = C.c_int64
         lib.ktj_shim_render.restype = C.c_int
         lib.ktj_shim_render.argtypes = [C.POINTER(abi.Stream), C.POINTER(MatActivity), C.c_uint64,
-                                        C.c_void_p, C.c_void_p, C.c_char_p, C.c_int, C.POINTER(C.c_uint64)]
+                                        C.c_void_p, C.c_void_p, C.c_char_p, C.c_int, C.POINTER(C.c_uint64), C.c_int]
         _shim = lib
     return _shim
 
@@ -181,9 +181,10 @@ def ref_render(stream_ptr, oracle_run):
     return data.replace(path.encode(), stream_ptr.contents.trace_name)
 
 
-def shim_render(stream_ptr, oracle_run, protocol="gpujson", directory=None):
+def shim_render(stream_ptr, oracle_run, protocol="gpujson", directory=None, bulk_threads=0):
     """Renders the stream through the GpuChromeTraceLogger shim obtained from a logger factory by
-    URL, fed with the same activities as ref_render.  Returns (status, bytes or None, dropped)."""
+    URL, fed with the same activities as ref_render, one handleActivity() call each or, with
+    bulk_threads > 0, in one handleActivities() call.  Returns (status, bytes or None, dropped)."""
     shim = load_shim()
     acts, n = oracle_run.activities()
     fn = C.cast(load_oracle().ktj_oracle_string, C.c_void_p)
@@ -191,7 +192,7 @@ def shim_render(stream_ptr, oracle_run, protocol="gpujson", directory=None):
     with tempfile.TemporaryDirectory() as d:
         path = os.path.join(directory or d, stream_ptr.contents.trace_name.decode())
         url = f"{protocol}://{path}"
-        rc = shim.ktj_shim_render(stream_ptr, acts, n, fn, oracle_run.h, url.encode(), 0, C.byref(dropped))
+        rc = shim.ktj_shim_render(stream_ptr, acts, n, fn, oracle_run.h, url.encode(), 0, C.byref(dropped), bulk_threads)
         data = None
         if rc == 0:
             with open(path, "rb") as f:

@@ -23,12 +23,13 @@ def _first_diff(a, b):
     return n
 
 
-def _compare(sp):
+def _compare(sp, bulk_threads=3):
     o = og.OracleRun(sp)
     try:
         theirs = og.ref_render(sp, o)
         rc, mine, dropped = og.shim_render(sp, o)
         mixed_case_rc, mixed, _ = og.shim_render(sp, o, protocol="GPUJSON")
+        bulk_rc, bulk, bulk_dropped = og.shim_render(sp, o, bulk_threads=bulk_threads)
     finally:
         o.close()
     assert rc == 0 and dropped == 0
@@ -37,6 +38,12 @@ def _compare(sp):
         raise AssertionError(f"byte {i} of {len(theirs)}: shim {mine[max(0, i - 80):i + 80]!r} "
                              f"reference {theirs[max(0, i - 80):i + 80]!r}")
     assert mixed_case_rc == 0 and mixed == theirs  # protocol lookup is case-insensitive
+    # all activities in one handleActivities() call, packed by several workers
+    assert bulk_rc == 0 and bulk_dropped == 0
+    if bulk != theirs:
+        i = _first_diff(bulk, theirs)
+        raise AssertionError(f"bulk: byte {i} of {len(theirs)}: shim {bulk[max(0, i - 80):i + 80]!r} "
+                             f"reference {theirs[max(0, i - 80):i + 80]!r}")
 
 
 @pytest.mark.parametrize("cfg,n", [(1, 10000), (2, 20000), (3, 30000), (4, 30000), (5, 4000), (1, 1), (2, 7)])
@@ -60,6 +67,21 @@ def test_shim_random_streams(seed):
     sp = kat_cases.build_for_real_logger(lambda: (random_streams.random_stream(seed, wide_ids=seed % 2 == 1), None),
                                          og.ref_stream_args())
     _compare(sp)
+
+
+def test_shim_bulk_packing_is_independent_of_the_worker_count():
+    """handleActivities() with 1, 2, 5 and 16 workers writes the same file as the reference."""
+    sp, release = abi.synth_stream(3, 40000, **og.ref_stream_args())
+    o = og.OracleRun(sp)
+    try:
+        theirs = og.ref_render(sp, o)
+        for threads in (1, 2, 5, 16):
+            rc, mine, dropped = og.shim_render(sp, o, bulk_threads=threads)
+            assert rc == 0 and dropped == 0
+            assert mine == theirs, threads
+    finally:
+        o.close()
+        release()
 
 
 def test_shim_unknown_protocol_and_bad_sink():
