@@ -1,0 +1,44 @@
+/*
+ * ktj_rocprofiler.h — rocprofiler-sdk buffer records straight into the engine.
+ *
+ * Replaces the body of RocprofLogger::buffer_callback (libkineto/src/RocprofLogger.cpp:681-749),
+ * which turns every kernel-dispatch and memory-copy record of an SDK buffer into a heap-allocated
+ * rocprofAsyncRow with a copied kernel-name string.  Here the same fields go into packed device
+ * rows (ktj_device_rec) in one pass over the headers, and from there to the GPU; the two lookups of
+ * that function (agent handle -> device index, kernel id -> kernel name) use tables the caller
+ * keeps up to date from the SDK's agent query and code-object callbacks
+ * (RocprofLogger.cpp: globalContext.agents, globalContext.kernel_names).
+ *
+ * The header does not include the SDK's: `headers` is the `rocprofiler_record_header_t**` the
+ * SDK passes to its buffer callback.
+ */
+#ifndef KTJ_ROCPROFILER_H_
+#define KTJ_ROCPROFILER_H_
+
+#include "ktj.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* globalContext.agents: agent handle -> logical_node_type_id.  An agent that is not listed gives
+ * device -1 (RocprofLogger.cpp:703-707).  Replaces the table. */
+int ktj_set_sdk_agents(ktj_engine* e, const uint64_t* agent_handles, const int32_t* device_ids, size_t n);
+
+/* globalContext.kernel_names: kernel id -> string id of the kernel's name.  A kernel that is not
+ * listed gets unknown_name_id, the string id of "<unknown kernel>" (RocprofLogger.cpp:709-714).
+ * Adds to the table; a kernel id given again takes the new name. */
+int ktj_set_sdk_kernel_names(ktj_engine* e, const uint64_t* kernel_ids, const uint32_t* name_ids, size_t n,
+                             uint32_t unknown_name_id);
+
+/* One call of the SDK's buffer callback.  Records of category ROCPROFILER_BUFFER_CATEGORY_TRACING
+ * and kind ROCPROFILER_BUFFER_TRACING_KERNEL_DISPATCH or ROCPROFILER_BUFFER_TRACING_MEMORY_COPY
+ * become device rows, in header order, after the rows submitted so far; every other record is
+ * skipped, as the reference skips it.  *n_rows receives the number of rows taken.  The SDK's
+ * buffer may be released when the call returns. */
+int ktj_submit_sdk_buffer(ktj_engine* e, void* const* headers, size_t num_headers, uint64_t* n_rows);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KTJ_ROCPROFILER_H_ */

@@ -183,6 +183,8 @@ ENGINE_SYMBOLS = [
     "ktj_set_window", "ktj_submit_records", "ktj_submit_records_device", "ktj_submit_info",
     "ktj_process", "ktj_output_device", "ktj_output_host", "ktj_finalize", "ktj_get_stats",
     "ktj_version",
+    # include/ktj_rocprofiler.h
+    "ktj_set_sdk_agents", "ktj_set_sdk_kernel_names", "ktj_submit_sdk_buffer",
 ]
 
 
@@ -225,6 +227,12 @@ def load_engine():
         lib.ktj_submit_records_device.argtypes = [vp, C.c_int, C.c_void_p, C.c_size_t]
         lib.ktj_submit_info.restype = C.c_int
         lib.ktj_submit_info.argtypes = [vp, C.c_int, C.c_void_p]
+        lib.ktj_set_sdk_agents.restype = C.c_int
+        lib.ktj_set_sdk_agents.argtypes = [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_int32), C.c_size_t]
+        lib.ktj_set_sdk_kernel_names.restype = C.c_int
+        lib.ktj_set_sdk_kernel_names.argtypes = [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), C.c_size_t, C.c_uint32]
+        lib.ktj_submit_sdk_buffer.restype = C.c_int
+        lib.ktj_submit_sdk_buffer.argtypes = [vp, C.POINTER(C.c_void_p), C.c_size_t, C.POINTER(C.c_uint64)]
         lib.ktj_process.restype = C.c_int
         lib.ktj_process.argtypes = [vp, C.c_int64]
         lib.ktj_output_device.restype = C.c_int

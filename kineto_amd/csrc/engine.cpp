@@ -15,10 +15,14 @@
 #include <cstring>
 #include <string>
 #include <unistd.h>
+#include <unordered_map>
 #include <utility>
 #include <vector>
 
+#include <rocprofiler-sdk/buffer_tracing.h>
+
 #include "../../include/ktj_debug.h"
+#include "../../include/ktj_rocprofiler.h"
 #include "gpu_stages.h"
 #include "host_events.h"
 
@@ -110,6 +114,10 @@ struct ktj_engine {
   bool coll_dirty = true;
   DevBuf d_coll_blob, d_coll_off, d_coll_first, cpu_row;
   std::vector<uint32_t> coll_first;        /* read back: first use of each entry per backend */
+  std::unordered_map<uint64_t, int32_t> sdk_agents;        /* agent handle -> device index */
+  std::unordered_map<uint64_t, uint32_t> sdk_kernel_names; /* kernel id -> string id of its name */
+  uint32_t sdk_unknown_name = KTJ_NONE;
+  std::vector<ktj_device_rec> sdk_rows;                    /* conversion buffer, reused */
   std::vector<uint32_t> cid_names, flow_bits;
   uint32_t malloc_cid = KTJ_NONE;
   DevBuf d_cid_names, d_flow_bits;
@@ -362,6 +370,69 @@ int ktj_submit_records_device(ktj_engine* e, int rec_class, const void* device_p
   set->n = n_records;
   e->processed = false;
   return KTJ_OK;
+}
+
+/* ---- rocprofiler-sdk buffer records (include/ktj_rocprofiler.h) ---- */
+
+int ktj_set_sdk_agents(ktj_engine* e, const uint64_t* agent_handles, const int32_t* device_ids, size_t n) {
+  if (!e || (n && (!agent_handles || !device_ids))) return KTJ_ERR_ARG;
+  e->sdk_agents.clear();
+  for (size_t i = 0; i < n; ++i) e->sdk_agents[agent_handles[i]] = device_ids[i];
+  return KTJ_OK;
+}
+
+int ktj_set_sdk_kernel_names(ktj_engine* e, const uint64_t* kernel_ids, const uint32_t* name_ids, size_t n,
+                             uint32_t unknown_name_id) {
+  if (!e || (n && (!kernel_ids || !name_ids))) return KTJ_ERR_ARG;
+  for (size_t i = 0; i < n; ++i) e->sdk_kernel_names[kernel_ids[i]] = name_ids[i];
+  e->sdk_unknown_name = unknown_name_id;
+  return KTJ_OK;
+}
+
+/* RocprofLogger::buffer_callback (libkineto/src/RocprofLogger.cpp:681-749): the fields of a
+ * rocprofAsyncRow (src/RocLogger.h:216-240) from a kernel-dispatch or memory-copy record. */
+int ktj_submit_sdk_buffer(ktj_engine* e, void* const* headers, size_t num_headers, uint64_t* n_rows) {
+  if (n_rows) *n_rows = 0;
+  if (!e || (num_headers && !headers)) return KTJ_ERR_ARG;
+  std::vector<ktj_device_rec>& rows = e->sdk_rows;
+  rows.clear();
+  rows.reserve(num_headers);
+  auto device_of = [e](uint64_t agent_handle) {
+    const auto it = e->sdk_agents.find(agent_handle);
+    return it != e->sdk_agents.end() ? it->second : -1;
+  };
+  for (size_t i = 0; i < num_headers; ++i) {
+    const rocprofiler_record_header_t* h = static_cast<const rocprofiler_record_header_t*>(headers[i]);
+    if (!h || h->category != ROCPROFILER_BUFFER_CATEGORY_TRACING || !h->payload) continue;
+    ktj_device_rec r{};
+    if (h->kind == ROCPROFILER_BUFFER_TRACING_KERNEL_DISPATCH) {
+      const auto& rec = *static_cast<const rocprofiler_buffer_tracing_kernel_dispatch_record_t*>(h->payload);
+      const auto name = e->sdk_kernel_names.find(rec.dispatch_info.kernel_id);
+      r.id = rec.correlation_id.internal;
+      r.begin = rec.start_timestamp;
+      r.end = rec.end_timestamp;
+      r.domain = KTJ_DOM_KERNEL_DISPATCH;
+      r.op = static_cast<uint32_t>(rec.operation);
+      r.device = device_of(rec.dispatch_info.agent_id.handle);
+      r.name_id = name != e->sdk_kernel_names.end() ? name->second : e->sdk_unknown_name;
+      r.queue = rec.dispatch_info.queue_id.handle;
+    } else if (h->kind == ROCPROFILER_BUFFER_TRACING_MEMORY_COPY) {
+      const auto& rec = *static_cast<const rocprofiler_buffer_tracing_memory_copy_record_t*>(h->payload);
+      r.id = rec.correlation_id.internal;
+      r.begin = rec.start_timestamp;
+      r.end = rec.end_timestamp;
+      r.domain = KTJ_DOM_MEMORY_COPY;
+      r.op = static_cast<uint32_t>(rec.operation);
+      r.device = device_of(rec.dst_agent_id.handle);
+      r.name_id = KTJ_NONE; /* the row's name is empty; the copy direction names the activity */
+      r.queue = 0;
+    } else {
+      continue;
+    }
+    rows.push_back(r);
+  }
+  if (n_rows) *n_rows = rows.size();
+  return ktj_submit_records(e, KTJ_REC_DEVICE, rows.data(), rows.size());
 }
 
 int ktj_submit_info(ktj_engine* e, int info_kind, const void* info) {

@@ -33,6 +33,8 @@
  *       hand-made cases (tests/kat_cases.py: case_collective_*).  The order of the process groups
  *       is the iteration order of a std::unordered_map and is taken from the C++ library
  *       (map_order.cpp), as the logger takes it.
+ *   - rocprofiler-sdk buffer records -> device rows (sdk_rows.c): PARITY UNPINNED by the reference
+ *       (its buffer callback needs a live profiling session); hand-written expectations only.
  */
 #define _GNU_SOURCE
 #include "ktj_oracle.h"

@@ -17,7 +17,7 @@ SIM_SO = os.path.join(ROOT, "tests", "host_sim", "libktjsim.so")
 
 def test_engine_library_exports_every_declared_symbol():
     decl = set()
-    for hdr in ("ktj.h", "ktj_debug.h"):
+    for hdr in ("ktj.h", "ktj_debug.h", "ktj_rocprofiler.h"):
         text = open(os.path.join(ROOT, "include", hdr)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         decl |= set(re.findall(r"\b(ktj_[a-z_]+)\s*\(", text))

@@ -1,0 +1,159 @@
+"""rocprofiler-sdk buffer records as device rows (include/ktj_rocprofiler.h).
+
+The record structs come from the SDK's own header (tests/host_sim/sdk_records.cpp builds them).
+CPU: the checker's restatement of RocprofLogger::buffer_callback (oracle/sdk_rows.c) against
+hand-written expectations.  GPU: ktj_submit_sdk_buffer against the checker, end to end.  The
+reference's buffer_callback needs a live profiling session and is not built, so these
+expectations are this repository's reading of libkineto/src/RocprofLogger.cpp:681-749."""
+import ctypes as C
+import os
+
+import pytest
+
+import oracle_glue as og
+from kineto_amd import abi
+from stream_builder import B, StreamBuilder
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+AGENT_BASE, KERNEL_BASE = 0xA0000, 0x5000
+
+
+def _sim():
+    lib = C.CDLL(os.path.join(ROOT, "tests", "host_sim", "libktjsim.so"))
+    lib.ktjsim_sdk_buffer_create.restype = C.c_void_p
+    lib.ktjsim_sdk_buffer_create.argtypes = [C.POINTER(abi.DeviceRec), C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint32, C.c_int]
+    lib.ktjsim_sdk_buffer_headers.restype = C.POINTER(C.c_void_p)
+    lib.ktjsim_sdk_buffer_headers.argtypes = [C.c_void_p]
+    lib.ktjsim_sdk_buffer_count.restype = C.c_uint64
+    lib.ktjsim_sdk_buffer_count.argtypes = [C.c_void_p]
+    lib.ktjsim_sdk_buffer_free.argtypes = [C.c_void_p]
+    return lib
+
+
+def _oracle_rows(headers, n_headers, agents, kernels, unknown):
+    lib = og.load_oracle()
+    lib.ktj_oracle_sdk_rows.restype = C.c_uint64
+    lib.ktj_oracle_sdk_rows.argtypes = [C.POINTER(C.c_void_p), C.c_uint64, C.POINTER(C.c_uint64), C.POINTER(C.c_int32), C.c_uint64,
+                                        C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), C.c_uint64, C.c_uint32, C.POINTER(abi.DeviceRec)]
+    ah = (C.c_uint64 * max(len(agents), 1))(*[a for a, _ in agents])
+    ad = (C.c_int32 * max(len(agents), 1))(*[d for _, d in agents])
+    ki = (C.c_uint64 * max(len(kernels), 1))(*[k for k, _ in kernels])
+    kn = (C.c_uint32 * max(len(kernels), 1))(*[v for _, v in kernels])
+    out = (abi.DeviceRec * max(n_headers, 1))()
+    n = lib.ktj_oracle_sdk_rows(headers, n_headers, ah, ad, len(agents), ki, kn, len(kernels), unknown, out)
+    return out, n
+
+
+def _tables(rows, unknown):
+    """Agent and kernel-name tables for rows built by ktjsim_sdk_buffer_create: devices >= 0 are
+    listed (device -1 stands for an agent the logger does not know), every name but `unknown` too."""
+    agents = sorted({(AGENT_BASE + r.device + 1, r.device) for r in rows if r.device >= 0})
+    kernels = sorted({(KERNEL_BASE + r.name_id, r.name_id) for r in rows if r.domain == 0 and r.name_id != unknown})
+    return agents, kernels
+
+
+def _row(**kw):
+    r = abi.DeviceRec()
+    for k, v in kw.items():
+        setattr(r, k, v)
+    return r
+
+
+def test_checker_restatement_on_hand_written_records():
+    sim = _sim()
+    unknown = 900
+    rows = [_row(id=11, begin=1000, end=2000, domain=0, op=1, device=0, name_id=5, queue=77),
+            _row(id=12, begin=3000, end=3500, domain=1, op=2, device=1, name_id=123, queue=99, stream=7, bytes=4096),
+            _row(id=(1 << 40) + 3, begin=5000, end=5001, domain=0, op=1, device=-1, name_id=unknown, queue=(1 << 63) + 2),
+            _row(id=14, begin=0, end=0, domain=1, op=4, device=-1)]
+    arr = (abi.DeviceRec * len(rows))(*rows)
+    buf = sim.ktjsim_sdk_buffer_create(arr, len(rows), AGENT_BASE, KERNEL_BASE, unknown, 1)
+    n_headers = sim.ktjsim_sdk_buffer_count(buf)
+    assert n_headers > len(rows)  # records of other kinds and categories are mixed in
+    agents, kernels = _tables(rows, unknown)
+    out, n = _oracle_rows(sim.ktjsim_sdk_buffer_headers(buf), n_headers, agents, kernels, unknown)
+    sim.ktjsim_sdk_buffer_free(buf)
+    assert n == 4
+    got = [(r.id, r.begin, r.end, r.domain, r.op, r.device, r.name_id, r.queue, r.stream, r.bytes) for r in out[:n]]
+    assert got == [
+        (11, 1000, 2000, 0, 1, 0, 5, 77, 0, 0),                       # kernel: every field of the dispatch record
+        (12, 3000, 3500, 1, 2, 1, abi.KTJ_NONE, 0, 0, 0),             # copy: no name, queue 0, destination agent, no byte count
+        ((1 << 40) + 3, 5000, 5001, 0, 1, -1, unknown, (1 << 63) + 2, 0, 0),  # unknown agent and kernel
+        (14, 0, 0, 1, 4, -1, abi.KTJ_NONE, 0, 0, 0),
+    ]
+
+
+def _sdk_case(cfg, n):
+    """A synthetic stream whose kernel and copy rows went through SDK records: returns the stream
+    with its device rows replaced by the checker's reading of those records, and what the engine
+    needs to submit them."""
+    sp, release = abi.synth_stream(cfg, n, host_name="box")
+    s = sp.contents
+    unknown = s.n_strings  # one more string: "<unknown kernel>"
+    rows = [s.device[i] for i in range(s.n_device) if s.device[i].domain != 2]
+    for k, r in enumerate(rows):
+        if k % 11 == 3:
+            r.device = -1
+        if k % 13 == 5 and r.domain == 0:
+            r.name_id = unknown
+    return sp, release, rows, unknown
+
+
+def _with_extra_string(sp, text, keep):
+    s = sp.contents
+    blob = C.string_at(s.str_blob, s.str_off[s.n_strings]) + text
+    offs = (C.c_uint64 * (s.n_strings + 2))(*([s.str_off[i] for i in range(s.n_strings + 1)] + [len(blob)]))
+    bb = C.create_string_buffer(blob, len(blob))
+    keep += [bb, offs]
+    s.str_blob = C.cast(bb, C.c_void_p)
+    s.str_off = offs
+    s.n_strings += 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cfg,n", [(1, 3000), (2, 5000), (3, 20000), (4, 8000)])
+def test_sdk_buffer_ingestion_matches_checker(cfg, n):
+    from kineto_amd.engine import TraceEngine
+    sim = _sim()
+    sp, release, rows, unknown = _sdk_case(cfg, n)
+    keep = []
+    try:
+        s = sp.contents
+        _with_extra_string(sp, b"<unknown kernel>", keep)
+        arr = (abi.DeviceRec * max(len(rows), 1))(*rows)
+        buf = sim.ktjsim_sdk_buffer_create(arr, len(rows), AGENT_BASE, KERNEL_BASE, unknown, 1)
+        headers, n_headers = sim.ktjsim_sdk_buffer_headers(buf), sim.ktjsim_sdk_buffer_count(buf)
+        agents, kernels = _tables(rows, unknown)
+        expect_rows, n_rows = _oracle_rows(headers, n_headers, agents, kernels, unknown)
+        assert n_rows == len(rows)
+        # the checker renders the stream with exactly these device rows
+        s.device, s.n_device = C.cast(expect_rows, C.POINTER(abi.DeviceRec)), n_rows
+        ora = og.OracleRun(sp)
+        want = ora.output()
+        ora.close()
+        # the engine gets the same stream, but its device rows arrive as SDK buffers (three calls)
+        with TraceEngine(s.trace_name.decode(), device=0) as eng:
+            s.n_device = 0
+            eng.submit_stream(sp)
+            s.n_device = n_rows
+            lib, h = eng.lib, eng.h
+            ah = (C.c_uint64 * max(len(agents), 1))(*[a for a, _ in agents])
+            ad = (C.c_int32 * max(len(agents), 1))(*[d for _, d in agents])
+            ki = (C.c_uint64 * max(len(kernels), 1))(*[k for k, _ in kernels])
+            kn = (C.c_uint32 * max(len(kernels), 1))(*[v for _, v in kernels])
+            assert lib.ktj_set_sdk_agents(h, ah, ad, len(agents)) == 0
+            assert lib.ktj_set_sdk_kernel_names(h, ki, kn, len(kernels), unknown) == 0
+            taken_total, cut = 0, [0, n_headers // 3, n_headers // 2, n_headers]
+            for lo, hi in zip(cut, cut[1:]):
+                taken = C.c_uint64()
+                part = C.cast(C.addressof(headers.contents) + 8 * lo, C.POINTER(C.c_void_p))
+                assert lib.ktj_submit_sdk_buffer(h, part, hi - lo, C.byref(taken)) == 0
+                taken_total += taken.value
+            assert taken_total == n_rows
+            eng.process()
+            got = eng.output()
+        sim.ktjsim_sdk_buffer_free(buf)
+        assert got == want
+        assert b"<unknown kernel>" in want and b'"pid": -1,' in want
+    finally:
+        release()
