@@ -84,7 +84,8 @@ enum {
   KTJ_REC_GENERIC = 0,  /* ktj_generic_rec  */
   KTJ_REC_RUNTIME = 1,  /* ktj_runtime_rec  */
   KTJ_REC_DEVICE = 2,   /* ktj_device_rec   */
-  KTJ_REC_EXTCORR = 3   /* ktj_extcorr_rec  */
+  KTJ_REC_EXTCORR = 3,  /* ktj_extcorr_rec, domain 0: correlation id -> CPU op              */
+  KTJ_REC_USERCORR = 4  /* ktj_extcorr_rec, domain 1: correlation id -> user annotation     */
 };
 
 /*
@@ -204,8 +205,11 @@ typedef struct ktj_device_rec {
   uint64_t bytes;    /* KTJ_DOM_MEMSET only                                                   */
 } ktj_device_rec;    /* 64 bytes */
 
-/* External-correlation pair, domain 0: (correlation id → CPU-op id)
- * (libkineto/src/RocmActivityProfiler.cpp:135-148). */
+/* External-correlation pair (libkineto/src/RocmActivityProfiler.cpp:135-148).  Domain 0
+ * (KTJ_REC_EXTCORR, cpuCorrelationMap_): correlation id -> CPU-op id, the "External id" link.
+ * Domain 1 (KTJ_REC_USERCORR, userCorrelationMap_): correlation id -> id of a user annotation; when
+ * any are submitted, every (device, stream) on which device rows of one annotation ran gets a
+ * GPU_USER_ANNOTATION activity that spans them (GenericActivityProfiler.cpp:277-327, 425-433, 726). */
 typedef struct ktj_extcorr_rec {
   uint64_t correlation;
   uint64_t external_id;

@@ -76,6 +76,10 @@ typedef struct ktj_stream {
   /* collective metadata, indexed by the slots of KTJ_F_COLLECTIVE fields */
   const ktj_collective_meta* collectives;
   uint64_t n_collectives;
+
+  /* external correlation of the user domain (KTJ_REC_USERCORR), arrival order */
+  const ktj_extcorr_rec* usercorr;
+  uint64_t n_usercorr;
 } ktj_stream;
 
 /* ------------------------------------------------------------------------------------------

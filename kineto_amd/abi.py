@@ -14,7 +14,7 @@ KTJ_CREATE_NO_FILE = 0x1
 KTJ_CREATE_TILE_EMIT = 0x2
 KTJ_CREATE_HASH_JOIN = 0x4
 
-REC_GENERIC, REC_RUNTIME, REC_DEVICE, REC_EXTCORR = 0, 1, 2, 3
+REC_GENERIC, REC_RUNTIME, REC_DEVICE, REC_EXTCORR, REC_USERCORR = 0, 1, 2, 3, 4
 INFO_DEVICE, INFO_RESOURCE, INFO_OVERHEAD, INFO_SPAN = 0, 1, 2, 3
 F_I64, F_U64, F_F64, F_BOOL, F_STR, F_RAW, F_I64_ARRAY, F_COLLECTIVE = range(8)
 N_STAGES = 12
@@ -141,7 +141,8 @@ class Stream(C.Structure):
                 ("resource_infos", C.POINTER(ResourceInfo)), ("n_resource_infos", C.c_uint64),
                 ("overhead_infos", C.POINTER(OverheadInfo)), ("n_overhead_infos", C.c_uint64),
                 ("spans", C.POINTER(TraceSpan)), ("n_spans", C.c_uint64),
-                ("collectives", C.POINTER(CollectiveMeta)), ("n_collectives", C.c_uint64)]
+                ("collectives", C.POINTER(CollectiveMeta)), ("n_collectives", C.c_uint64),
+                ("usercorr", C.POINTER(ExtCorrRec)), ("n_usercorr", C.c_uint64)]
 
 
 class SynthParams(C.Structure):

@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <string>
 #include <unistd.h>
 #include <unordered_map>
@@ -113,6 +114,10 @@ struct ktj_engine {
   bool coll_schemas = false;               /* a schema with a leading KTJ_F_COLLECTIVE field exists */
   bool coll_dirty = true;
   DevBuf d_coll_blob, d_coll_off, d_coll_first, cpu_row;
+  /* GPU user annotations: correlation table, span table, finished spans, synthesised records */
+  DevBuf u_keys, u_src, sp_hash, sp_first, sp_lo, sp_hi, sp_zero, sp_dev, sp_res, sp_ext, sp_name, sp_out, sp_count, sp_members,
+      synth_recs;
+  uint64_t n_spans = 0;
   std::vector<uint32_t> coll_first;        /* read back: first use of each entry per backend */
   std::unordered_map<uint64_t, int32_t> sdk_agents;        /* agent handle -> device index */
   std::unordered_map<uint64_t, uint32_t> sdk_kernel_names; /* kernel id -> string id of its name */
@@ -124,7 +129,7 @@ struct ktj_engine {
   bool api_dirty = true;
   ktj_clock_model clock{};
   int64_t win_start = INT64_MIN, win_end = INT64_MAX;
-  RecordSet generic, runtime, devrows, extcorr;
+  RecordSet generic, runtime, devrows, extcorr, usercorr;
 
   /* working buffers */
   DevBuf d_scalars, d_name_len, d_arg_len, d_sflags, d_name_off, d_arg_off, d_name_blob, d_arg_blob;
@@ -178,6 +183,102 @@ int bits_for(uint64_t max_value) { /* bits needed to hold values 0..max_value */
   int b = 0;
   while (b < 64 && (max_value >> b) != 0) ++b;
   return b;
+}
+
+/* GPU user annotations (GenericActivityProfiler.cpp:277-327, 423-433, 726).  The device groups the
+ * in-window device rows by (device, resource, annotation) and reduces each group to its extent;
+ * the host puts the finished spans into the order the profiler logs them in — stream by stream
+ * (std::map), inside a stream the iteration order of a std::unordered_map keyed by the
+ * annotation's id, both filled in the order of the spans' first rows — and hands them back as
+ * generic records of type GPU_USER_ANNOTATION whose rows follow the device rows. */
+int synthesise_user_spans(ktj_engine* e, Columns c, const EmitCtx& ctx, Table t_cpu, const uint32_t* cpu_row, Scalars* sc,
+                          uint64_t first_row) {
+  hipStream_t st = e->stream;
+  const uint64_t ng = e->generic.n, nr = e->runtime.n, nd = e->devrows.n, nu = e->usercorr.n;
+  const ktj_generic_rec* g_recs = static_cast<const ktj_generic_rec*>(e->generic.ptr());
+  const ktj_extcorr_rec* u_recs = static_cast<const ktj_extcorr_rec*>(e->usercorr.ptr());
+  const uint32_t cap_user = pow2_at_least(2 * nu), cap_span = pow2_at_least(2 * nd);
+  HIPCHK(e->u_keys.ensure((cap_user + 1ull) * 8)); HIPCHK(e->u_src.ensure((cap_user + 1ull) * 4));
+  HIPCHK(e->sp_hash.ensure((cap_span + 1ull) * 8)); HIPCHK(e->sp_first.ensure((cap_span + 1ull) * 4));
+  HIPCHK(e->sp_lo.ensure((cap_span + 1ull) * 8)); HIPCHK(e->sp_hi.ensure((cap_span + 1ull) * 8));
+  HIPCHK(e->sp_zero.ensure((cap_span + 1ull) * 4)); HIPCHK(e->sp_dev.ensure((cap_span + 1ull) * 4));
+  HIPCHK(e->sp_res.ensure((cap_span + 1ull) * 8)); HIPCHK(e->sp_ext.ensure((cap_span + 1ull) * 8));
+  HIPCHK(e->sp_name.ensure((cap_span + 1ull) * 4)); HIPCHK(e->sp_out.ensure((nd + 1ull) * sizeof(SpanOut)));
+  HIPCHK(e->sp_count.ensure(16));
+  SpanTables t{e->u_keys.as<uint64_t>(), e->u_src.as<uint32_t>(), cap_user - 1,
+               e->sp_hash.as<uint64_t>(), e->sp_first.as<uint32_t>(), e->sp_lo.as<uint64_t>(), e->sp_hi.as<uint64_t>(),
+               e->sp_zero.as<uint32_t>(), cap_span - 1,
+               e->sp_dev.as<int32_t>(), e->sp_res.as<int64_t>(), e->sp_ext.as<uint64_t>(), e->sp_name.as<uint32_t>()};
+  HIPCHK(fill_u64(t.u_keys, KTJ_EMPTY_KEY, cap_user + 1ull, st)); HIPCHK(fill_u32(t.u_src, 0, cap_user + 1ull, st));
+  HIPCHK(fill_u64(t.hash, KTJ_EMPTY_KEY, cap_span + 1ull, st)); HIPCHK(fill_u32(t.first, 0xFFFFFFFFu, cap_span + 1ull, st));
+  HIPCHK(fill_u64(t.lo, ~0ull, cap_span + 1ull, st)); HIPCHK(fill_u64(t.hi, 0, cap_span + 1ull, st));
+  HIPCHK(fill_u32(t.zero, 0, cap_span + 1ull, st));
+  HIPCHK(build_usercorr(u_recs, nu, t, sc, st));
+  HIPCHK(group_spans(u_recs, g_recs, nd, c, ng + nr, t_cpu, cpu_row, t, e->sp_out.as<SpanOut>(), e->sp_count.as<uint32_t>(), sc, st));
+  uint32_t n_out = 0;
+  HIPCHK(hipMemcpyAsync(&n_out, e->sp_count.p, 4, hipMemcpyDeviceToHost, st));
+  HIPCHK(hipStreamSynchronize(st));
+  if (n_out == 0) return KTJ_OK;
+  std::vector<SpanOut> spans(n_out);
+  HIPCHK(hipMemcpyAsync(spans.data(), e->sp_out.p, n_out * sizeof(SpanOut), hipMemcpyDeviceToHost, st));
+  HIPCHK(hipStreamSynchronize(st));
+  std::sort(spans.begin(), spans.end(), [](const SpanOut& a, const SpanOut& b) { return a.first < b.first; });
+
+  /* insertOrExtendEvent's start rule is `if (ts < start || start == 0) start = ts` (:304-306): the
+   * plain minimum unless a row of the span starts at time 0, after which the next row's time is
+   * taken whatever it is.  Those spans (rare) are replayed row by row here. */
+  bool any_zero = false;
+  for (const SpanOut& sp : spans) any_zero = any_zero || sp.zero != 0;
+  if (any_zero) {
+    HIPCHK(e->sp_members.ensure((nd + 1ull) * sizeof(SpanMember)));
+    HIPCHK(span_members(u_recs, nd, c, ng + nr, t_cpu, t, e->sp_members.as<SpanMember>(), (uint32_t)nd, e->sp_count.as<uint32_t>(), st));
+    uint32_t n_members = 0;
+    HIPCHK(hipMemcpyAsync(&n_members, e->sp_count.p, 4, hipMemcpyDeviceToHost, st));
+    HIPCHK(hipStreamSynchronize(st));
+    std::vector<SpanMember> members(n_members);
+    if (n_members) HIPCHK(hipMemcpyAsync(members.data(), e->sp_members.p, n_members * sizeof(SpanMember), hipMemcpyDeviceToHost, st));
+    HIPCHK(hipStreamSynchronize(st));
+    std::sort(members.begin(), members.end(), [](const SpanMember& a, const SpanMember& b) { return a.row < b.row; });
+    std::unordered_map<uint32_t, size_t> by_slot;
+    for (size_t k = 0; k < spans.size(); ++k)
+      if (spans[k].zero) by_slot[spans[k].zero] = k;
+    std::vector<uint8_t> started(spans.size(), 0);
+    for (const SpanMember& m : members) {
+      const auto it = by_slot.find(m.slot);
+      if (it == by_slot.end()) continue;
+      SpanOut& sp = spans[it->second];
+      if (!started[it->second]) { started[it->second] = 1; sp.start = m.ts; }
+      if (m.ts < sp.start || sp.start == 0) sp.start = m.ts;
+    }
+  }
+
+  /* logEvents order (:313-319) */
+  std::map<std::pair<int64_t, int64_t>, std::unordered_map<int64_t, size_t>> streams;
+  for (size_t k = 0; k < spans.size(); ++k)
+    streams[{(int64_t)spans[k].dev, spans[k].res}].insert({(int64_t)spans[k].ext, k});
+  std::vector<ktj_generic_rec> recs;
+  recs.reserve(spans.size());
+  for (const auto& stream : streams) {
+    for (const auto& entry : stream.second) {
+      const SpanOut& sp = spans[entry.second];
+      ktj_generic_rec r{}; /* createUserGpuSpan (:277-290): no metadata, no flow, no linked activity */
+      r.start_ns = sp.start;
+      r.end_ns = sp.end;
+      r.resource = sp.res;
+      r.device = sp.dev;
+      r.id = (int32_t)(int64_t)sp.ext;
+      r.name_id = sp.name;
+      r.schema_id = KTJ_NONE;
+      r.type = KTJ_TYPE_GPU_USER_ANNOTATION;
+      recs.push_back(r);
+    }
+  }
+  HIPCHK(e->synth_recs.ensure(recs.size() * sizeof(ktj_generic_rec) + 16));
+  HIPCHK(hipMemcpyAsync(e->synth_recs.p, recs.data(), recs.size() * sizeof(ktj_generic_rec), hipMemcpyHostToDevice, st));
+  HIPCHK(hipStreamSynchronize(st));
+  HIPCHK(decode_generic(e->synth_recs.as<ktj_generic_rec>(), recs.size(), c, first_row, sc, ctx, st));
+  e->n_spans = recs.size();
+  return KTJ_OK;
 }
 
 }  // namespace
@@ -340,6 +441,7 @@ static RecordSet* record_set(ktj_engine* e, int rec_class, size_t* rec_size) {
     case KTJ_REC_RUNTIME: *rec_size = sizeof(ktj_runtime_rec); return &e->runtime;
     case KTJ_REC_DEVICE: *rec_size = sizeof(ktj_device_rec); return &e->devrows;
     case KTJ_REC_EXTCORR: *rec_size = sizeof(ktj_extcorr_rec); return &e->extcorr;
+    case KTJ_REC_USERCORR: *rec_size = sizeof(ktj_extcorr_rec); return &e->usercorr;
     default: return nullptr;
   }
 }
@@ -454,12 +556,14 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   if (e->bad_sink) return KTJ_OK;
   HIPCHK(hipSetDevice(e->device));
   hipStream_t st = e->stream;
-  const uint64_t ng = e->generic.n, nr = e->runtime.n, nd = e->devrows.n, nx = e->extcorr.n;
-  const uint64_t N = ng + nr + nd;
-  if (N >= 0xFFFFFFF0ull) { e->last_error = "more than 2^32 - 16 records"; return KTJ_ERR_LIMIT; }
+  const uint64_t ng = e->generic.n, nr = e->runtime.n, nd = e->devrows.n, nx = e->extcorr.n, nu = e->usercorr.n;
+  uint64_t N = ng + nr + nd; /* grows by the synthesised GPU user-annotation spans, at most one per device row */
+  const uint64_t max_spans = nu ? nd : 0;
+  if (N + max_spans >= 0xFFFFFFF0ull) { e->last_error = "more than 2^32 - 16 records"; return KTJ_ERR_LIMIT; }
   e->N = N;
+  e->n_spans = 0;
   e->host_copy_valid = false;
-  const uint64_t Na = N ? N : 1;
+  const uint64_t Na = N + max_spans ? N + max_spans : 1;
 
   /* small tables */
   if (e->schemas_dirty) {
@@ -556,12 +660,13 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
     e->coll_dirty = false;
   }
   ctx.coll_blob = e->d_coll_blob.as<char>(); ctx.coll_off = e->d_coll_off.as<uint64_t>(); ctx.n_coll = n_coll;
-  uint32_t* cpu_row = nullptr;
-  if (n_coll) {
-    HIPCHK(e->cpu_row.ensure((cap_cpu + 1ull) * 4)); HIPCHK(e->d_coll_first.ensure(2ull * n_coll * 4));
+  uint32_t* cpu_row = nullptr; /* last CPU op per id: only where something is read from that op */
+  if (n_coll || max_spans) {
+    HIPCHK(e->cpu_row.ensure((cap_cpu + 1ull) * 4));
     cpu_row = e->cpu_row.as<uint32_t>();
     HIPCHK(fill_u32(cpu_row, 0, cap_cpu + 1ull, st));
   }
+  if (n_coll) HIPCHK(e->d_coll_first.ensure(2ull * n_coll * 4));
   if (ns) {
     HIPCHK(dict_measure(e->str_blob.buf.as<char>(), e->str_off.buf.as<uint64_t>(), ns, e->d_name_len.as<uint32_t>(),
                         e->d_arg_len.as<uint32_t>(), e->d_sflags.as<uint32_t>(), st));
@@ -613,6 +718,12 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
                           e->len.as<uint32_t>(), sc, st));
   HIPCHK(link_device_rows(nd, c, ng + nr, fc, tn, nc, e->slot_f_dev.as<uint32_t>(), e->dev_link.as<DevLink>(), sc, st));
   HIPCHK(backfill_streams(e->dev_brief.as<DevBrief>(), nd, c, ng + nr, stt, sc, st));
+  if (max_spans) {
+    const int rc = synthesise_user_spans(e, c, ctx, t_cpu, cpu_row, sc, N);
+    if (rc != KTJ_OK) return rc;
+    N += e->n_spans;
+    e->N = N;
+  }
   HIPCHK(hipEventRecord(e->ev[EV_JOIN], st));
 
   /* ---- stage 3: canonical order ---- */
@@ -670,7 +781,9 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
                              e->sync_pos.as<uint32_t>(), e->sync_first.as<uint32_t>(), sc, st));
     sync_first = e->sync_first.as<uint32_t>();
   }
-  HIPCHK(mat_generic_rows(g_recs, ng, ctx, sync_first, mat, e->len.as<uint32_t>(), sc, st));
+  HIPCHK(mat_generic_rows(g_recs, ng, 0, ctx, sync_first, mat, e->len.as<uint32_t>(), sc, st));
+  HIPCHK(mat_generic_rows(e->synth_recs.as<ktj_generic_rec>(), e->n_spans, ng + nr + nd, ctx, nullptr, mat, e->len.as<uint32_t>(),
+                          sc, st));
   HIPCHK(mat_device_rows(d_recs, nd, c, ng + nr, e->dev_link.as<DevLink>(), ctx, mat, e->len.as<uint32_t>(), sc, st));
   HIPCHK(gather_len(e->perm, e->len.as<uint32_t>(), N, e->len_sorted.as<uint32_t>(), st));
   if (n_coll) HIPCHK(collective_first(mat, e->perm, e->scalars.n_valid, n_coll, e->d_coll_first.as<uint32_t>(), st));

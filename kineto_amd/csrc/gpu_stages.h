@@ -201,6 +201,33 @@ struct StreamTables {
 hipError_t backfill_streams(const DevBrief* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
                             Scalars* sc, hipStream_t st);
 
+/* ---- GPU user annotations (GenericActivityProfiler.cpp:277-327, 423-433): one span per
+ * (device, resource, annotation id) over the device rows that the user-domain correlation
+ * records lead to.  Tables are caller-provided: u_keys (cap_user + 1, KTJ_EMPTY_KEY), u_src (0),
+ * and the span table of cap_span + 1 slots: hash (KTJ_EMPTY_KEY), first (0xFFFFFFFF), lo/hi
+ * (biased timestamps: lo ~0, hi 0), zero (0). ---- */
+struct SpanTables {
+  uint64_t* u_keys; uint32_t* u_src; uint32_t u_mask;   /* correlation id -> last user record (index + 1) */
+  uint64_t* hash; uint32_t* first; uint64_t* lo; uint64_t* hi; uint32_t* zero; uint32_t mask;
+  int32_t* dev; int64_t* res; uint64_t* ext; uint32_t* name;  /* written by the first row of a span */
+};
+struct SpanOut {            /* one finished span, read back by the host */
+  int64_t res;
+  uint64_t ext;             /* the annotation's id (key of the CPU-op table) */
+  int64_t start, end;       /* min timestamp, max end over the span's rows */
+  int32_t dev;
+  uint32_t name;            /* string id of the annotation's name */
+  uint32_t first;           /* index of the first device row of the span: insertion order */
+  uint32_t zero;            /* some row starts at time 0: the start needs the sequential rule */
+};                          /* 48 bytes */
+struct SpanMember { uint32_t slot, row; int64_t ts; };  /* rows of spans with `zero` set */
+hipError_t build_usercorr(const ktj_extcorr_rec* u, uint64_t n, SpanTables t, Scalars* sc, hipStream_t st);
+hipError_t group_spans(const ktj_extcorr_rec* u, const ktj_generic_rec* g, uint64_t n_device, Columns c, uint64_t first_device,
+                       Table cpu, const uint32_t* cpu_row, SpanTables t, SpanOut* out, uint32_t* n_out, Scalars* sc,
+                       hipStream_t st);
+hipError_t span_members(const ktj_extcorr_rec* u, uint64_t n_device, Columns c, uint64_t first_device, Table cpu,
+                        SpanTables t, SpanMember* out, uint32_t cap_out, uint32_t* n_out, hipStream_t st);
+
 /* ---- stage 3: canonical order ---- */
 struct SortSets {
   uint64_t* dev_keys;  /* KTJ_SET_CAP + 1, KTJ_EMPTY_KEY filled */
@@ -232,8 +259,9 @@ hipError_t stream_sync_first(const uint32_t* perm, uint64_t n_sorted, const ktj_
                              DictViews d, uint64_t* keys, uint32_t* first_pos, uint32_t* is_first, Scalars* sc,
                              hipStream_t st);
 /* sync_first: per generic row, from stream_sync_first, or null when there are no such rows */
-hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, const uint32_t* sync_first, MatRow* mat,
-                            uint32_t* len, Scalars* sc, hipStream_t st);
+/* generic records whose rows start at arrival index `first` */
+hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, uint64_t first, EmitCtx ctx, const uint32_t* sync_first,
+                            MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st);
 /* runtime rows: also publishes what device rows take over (first timestamp, stream, grid, size)
  * into the tables, reads the "External id" and counts timestamp-order violations; runs after
  * resolve_external and before link_device_rows */

@@ -795,6 +795,108 @@ hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, FullCo
   return KTJ_LAUNCH_CHECK();
 }
 
+/* ---- GPU user annotations: GenericActivityProfiler.cpp:277-327, 423-433 ---- */
+/* userCorrelationMap_[correlation] = externalId, the last record of an id stays */
+__global__ void k_build_usercorr(const ktj_extcorr_rec* u, uint64_t n, SpanTables t, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t slot = table_insert(t.u_keys, t.u_mask, u[i].correlation);
+  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
+  atomicMax(&t.u_src[slot], (uint32_t)i + 1u);
+}
+__device__ __forceinline__ uint64_t span_hash(int64_t device, int64_t resource, uint64_t ext) {
+  uint64_t h = hash64(ext ^ hash64((uint64_t)resource + 0x9E3779B97F4A7C15ULL) ^ hash64((uint64_t)device * 0xC2B2AE3D27D4EB4FULL + 1ULL));
+  return h == KTJ_EMPTY_KEY ? 0x5bd1e995ULL : h;
+}
+/* the annotation a device row belongs to: its id and the slot of that id in the CPU-op table */
+__device__ __forceinline__ bool span_of_row(const ktj_extcorr_rec* u, const SpanTables& t, const Table& cpu, uint64_t corr,
+                                            uint64_t* ext, uint32_t* cpu_slot) {
+  const uint32_t us = table_find(t.u_keys, t.u_mask, corr);
+  if (us == KTJ_NOSLOT || t.u_src[us] == 0) return false;
+  *ext = u[t.u_src[us] - 1u].external_id;
+  *cpu_slot = slot_find(cpu, *ext);
+  return *cpu_slot != KTJ_NOSLOT;
+}
+/* insertOrExtendEvent for every in-window device row: extent of the span, its first row */
+__global__ void k_span_extend(const ktj_extcorr_rec* u, uint64_t n, Columns c, uint64_t first_device, Table cpu, SpanTables t,
+                              Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint64_t a = first_device + i;
+  if (!(c.meta[a] & KTJ_M_VALID)) return;
+  uint64_t ext; uint32_t cs;
+  if (!span_of_row(u, t, cpu, c.corr[a], &ext, &cs)) return;
+  const uint32_t slot = table_insert(t.hash, t.mask, span_hash(c.dev[a], c.res[a], ext));
+  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
+  const int64_t ts = c.ts[a];
+  atomicMin(&t.first[slot], (uint32_t)i);
+  atomicMin((unsigned long long*)&t.lo[slot], (unsigned long long)((uint64_t)ts ^ 0x8000000000000000ULL));
+  atomicMax((unsigned long long*)&t.hi[slot], (unsigned long long)((uint64_t)(ts + c.dur[a]) ^ 0x8000000000000000ULL));
+  if (ts == 0) t.zero[slot] = 1u;
+}
+/* createUserGpuSpan: the first row of a span names it (single writer per slot) */
+__global__ void k_span_owner(const ktj_extcorr_rec* u, const ktj_generic_rec* g, uint64_t n, Columns c, uint64_t first_device,
+                             Table cpu, const uint32_t* cpu_row, SpanTables t) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint64_t a = first_device + i;
+  if (!(c.meta[a] & KTJ_M_VALID)) return;
+  uint64_t ext; uint32_t cs;
+  if (!span_of_row(u, t, cpu, c.corr[a], &ext, &cs)) return;
+  const uint32_t slot = table_find(t.hash, t.mask, span_hash(c.dev[a], c.res[a], ext));
+  if (slot == KTJ_NOSLOT || t.first[slot] != (uint32_t)i) return;
+  t.dev[slot] = (int32_t)c.dev[a]; t.res[slot] = c.res[a]; t.ext[slot] = ext;
+  const uint32_t row = cpu_row[cs]; /* the annotation is the last record with that id */
+  t.name[slot] = row ? g[row - 1u].name_id : KTJ_NONE;
+}
+__global__ void k_span_compact(SpanTables t, SpanOut* out, uint32_t* n_out) {
+  const uint64_t s = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (s > (uint64_t)t.mask + 1u || t.hash[s] == KTJ_EMPTY_KEY || t.first[s] == 0xFFFFFFFFu) return;
+  SpanOut o;
+  o.res = t.res[s]; o.ext = t.ext[s];
+  o.start = (int64_t)(t.lo[s] ^ 0x8000000000000000ULL); o.end = (int64_t)(t.hi[s] ^ 0x8000000000000000ULL);
+  o.dev = t.dev[s]; o.name = t.name[s]; o.first = t.first[s]; o.zero = t.zero[s] ? (uint32_t)s + 1u : 0u;
+  out[atomicAdd(n_out, 1u)] = o;
+}
+/* rows of the spans whose start needs the sequential rule (a row at time 0), for the host */
+__global__ void k_span_members(const ktj_extcorr_rec* u, uint64_t n, Columns c, uint64_t first_device, Table cpu,
+                               SpanTables t, SpanMember* out, uint32_t cap_out, uint32_t* n_out) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint64_t a = first_device + i;
+  if (!(c.meta[a] & KTJ_M_VALID)) return;
+  uint64_t ext; uint32_t cs;
+  if (!span_of_row(u, t, cpu, c.corr[a], &ext, &cs)) return;
+  const uint32_t slot = table_find(t.hash, t.mask, span_hash(c.dev[a], c.res[a], ext));
+  if (slot == KTJ_NOSLOT || t.zero[slot] == 0) return;
+  const uint32_t k = atomicAdd(n_out, 1u);
+  if (k < cap_out) { SpanMember m; m.slot = slot + 1u; m.row = (uint32_t)i; m.ts = c.ts[a]; out[k] = m; }
+}
+hipError_t build_usercorr(const ktj_extcorr_rec* u, uint64_t n, SpanTables t, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_build_usercorr, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, u, n, t, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t group_spans(const ktj_extcorr_rec* u, const ktj_generic_rec* g, uint64_t n_device, Columns c, uint64_t first_device,
+                       Table cpu, const uint32_t* cpu_row, SpanTables t, SpanOut* out, uint32_t* n_out, Scalars* sc,
+                       hipStream_t st) {
+  hipError_t e = fill_u32(n_out, 0, 1, st);
+  if (e != hipSuccess || n_device == 0) return e;
+  const dim3 grid(grid_for(n_device, KTJ_BLOCK)), block(KTJ_BLOCK);
+  hipLaunchKernelGGL(k_span_extend, grid, block, 0, st, u, n_device, c, first_device, cpu, t, sc);
+  hipLaunchKernelGGL(k_span_owner, grid, block, 0, st, u, g, n_device, c, first_device, cpu, cpu_row, t);
+  hipLaunchKernelGGL(k_span_compact, dim3(grid_for((uint64_t)t.mask + 2u, KTJ_BLOCK)), block, 0, st, t, out, n_out);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t span_members(const ktj_extcorr_rec* u, uint64_t n_device, Columns c, uint64_t first_device, Table cpu,
+                        SpanTables t, SpanMember* out, uint32_t cap_out, uint32_t* n_out, hipStream_t st) {
+  hipError_t e = fill_u32(n_out, 0, 1, st);
+  if (e != hipSuccess || n_device == 0) return e;
+  hipLaunchKernelGGL(k_span_members, dim3(grid_for(n_device, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, u, n_device, c, first_device,
+                     cpu, t, out, cap_out, n_out);
+  return KTJ_LAUNCH_CHECK();
+}
+
 /* ---- stream back-fill: libkineto/src/RocmStreamQueue.h:42-136 (its first pass, the stream of
  * the correlation-matched runtime row, is part of k_link_device) ---- */
 /* pass 2a: queue → stream, ambiguous when one queue shows two different streams.  Passes 2a/2b
@@ -1315,8 +1417,8 @@ hipError_t stream_sync_first(const uint32_t* perm, uint64_t n_sorted, const ktj_
   return KTJ_LAUNCH_CHECK();
 }
 
-__global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, const uint32_t* sync_first, MatRow* mat,
-                              uint32_t* len, Scalars* sc) {
+__global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, uint64_t first, EmitCtx ctx, const uint32_t* sync_first,
+                              MatRow* mat, uint32_t* len, Scalars* sc) {
   RowStats rs;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const ktj_generic_rec rec = g[i];
@@ -1324,8 +1426,8 @@ __global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx,
     if (!generic_record_prints(rec, ctx)) m.meta &= ~KTJ_M_VALID;
     attach_own_collective(m, rec, ctx);
     mark_stream_sync(m, ctx, sync_first != nullptr && sync_first[i] != 0);
-    store_row(&mat[i], m);
-    len[i] = row_length(m, ctx, sc);
+    store_row(&mat[first + i], m);
+    len[first + i] = row_length(m, ctx, sc);
     count_row_stats(m, ctx, &rs);
   }
   flush_row_stats(rs, sc);
@@ -1425,11 +1527,11 @@ __global__ void k_gather_len(const uint32_t* perm, const uint32_t* len, uint64_t
   if (i < n) len_sorted[i] = len[perm[i]] & 0x3FFFFFFFu;
 }
 
-hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, EmitCtx ctx, const uint32_t* sync_first, MatRow* mat,
-                            uint32_t* len, Scalars* sc, hipStream_t st) {
+hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, uint64_t first, EmitCtx ctx, const uint32_t* sync_first,
+                            MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_mat_generic, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, ctx, sync_first, mat,
-                     len, sc);
+  hipLaunchKernelGGL(k_mat_generic, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, first, ctx, sync_first,
+                     mat, len, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullCols fc,

@@ -59,7 +59,8 @@ class TraceEngine:
         self._chk(lib.ktj_set_clock_model(h, C.byref(s.clock)), "ktj_set_clock_model")
         self._chk(lib.ktj_set_window(h, s.window_start_ns, s.window_end_ns), "ktj_set_window")
         for cls, ptr, n in ((abi.REC_GENERIC, s.generic, s.n_generic), (abi.REC_RUNTIME, s.runtime, s.n_runtime),
-                            (abi.REC_DEVICE, s.device, s.n_device), (abi.REC_EXTCORR, s.extcorr, s.n_extcorr)):
+                            (abi.REC_DEVICE, s.device, s.n_device), (abi.REC_EXTCORR, s.extcorr, s.n_extcorr),
+                            (abi.REC_USERCORR, s.usercorr, s.n_usercorr)):
             if n:
                 self._chk(lib.ktj_submit_records(h, cls, C.cast(ptr, C.c_void_p), n), "ktj_submit_records")
         for kind, ptr, n in ((abi.INFO_DEVICE, s.device_infos, s.n_device_infos),

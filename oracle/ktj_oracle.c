@@ -33,6 +33,9 @@
  *       hand-made cases (tests/kat_cases.py: case_collective_*).  The order of the process groups
  *       is the iteration order of a std::unordered_map and is taken from the C++ library
  *       (map_order.cpp), as the logger takes it.
+ *   - GPU user-annotation spans: the expectations of test/RocmActivityProfilerTest.cpp:770-833 and
+ *       the sequential Python statement of tests/test_join_bruteforce.py; the spans' relative order
+ *       is the iteration order of the profiler's own maps, taken from the C++ library (map_order.cpp).
  *   - rocprofiler-sdk buffer records -> device rows (sdk_rows.c): PARITY UNPINNED by the reference
  *       (its buffer callback needs a live profiling session); hand-written expectations only.
  */
@@ -471,6 +474,14 @@ static uint32_t ptr_string(ktj_oracle* o, uint64_t p) { /* fmt "{}" of const voi
   return add_xstring(o, b, (size_t)n);
 }
 
+/* a GPU-side span of one user annotation on one stream (GenericActivityProfiler.h:324-347) */
+typedef struct user_span {
+  int64_t device, resource, cpu_id, start, end;
+  uint64_t cpu_row;
+} user_span;
+void ktj_oracle_span_map_order(const int64_t* device, const int64_t* resource, const int64_t* id, uint64_t n,
+                               uint64_t* order); /* map_order.cpp */
+
 static int stage_join(ktj_oracle* o) {
   const ktj_stream* s = o->s;
   const ktj_clock_model* cm = &s->clock;
@@ -523,6 +534,10 @@ static int stage_join(ktj_oracle* o) {
   }
   for (uint64_t i = 0; i < s->n_extcorr; ++i)
     *umap_slot(&cpu_corr, s->extcorr[i].correlation, NULL) = s->extcorr[i].external_id;
+  umap user_corr; umap_init(&user_corr, s->n_usercorr); /* userCorrelationMap_: RocmActivityProfiler.cpp:141-142 */
+  for (uint64_t i = 0; i < s->n_usercorr; ++i)
+    *umap_slot(&user_corr, s->usercorr[i].correlation, NULL) = s->usercorr[i].external_id;
+  user_span* spans = NULL; uint64_t n_spans = 0, cap_spans = 0;
 
   /* ---- stream back-fill: libkineto/src/RocmStreamQueue.h:42-136 ---- */
   uint64_t* dev_stream = (uint64_t*)malloc(8 * (s->n_device ? s->n_device : 1));
@@ -692,6 +707,28 @@ static int stage_join(ktj_oracle* o) {
     a->flow_type = KTJ_LINK_ASYNC_CPU_GPU;
     a->flow_start = 0;
     a->arrival = s->n_generic + s->n_runtime + i;
+    if (s->n_usercorr) { /* handleGpuActivity: GenericActivityProfiler.cpp:423-433 */
+      const uint64_t* ext = umap_find(&user_corr, d->id);
+      const uint64_t* op = ext ? umap_find(&activity_map, *ext) : NULL;
+      if (op) { /* GpuUserEventMap::insertOrExtendEvent: :292-311 */
+        const int64_t cpu_id = s->generic[*op].id;
+        user_span* sp = NULL;
+        for (uint64_t k = 0; k < n_spans && !sp; ++k)
+          if (spans[k].device == a->device && spans[k].resource == a->resource && spans[k].cpu_id == cpu_id) sp = &spans[k];
+        if (!sp) { /* createUserGpuSpan: :277-290 */
+          if (n_spans == cap_spans) {
+            cap_spans = cap_spans ? cap_spans * 2 : 64;
+            spans = (user_span*)realloc(spans, cap_spans * sizeof *spans);
+            if (!spans) abort();
+          }
+          sp = &spans[n_spans++];
+          sp->device = a->device; sp->resource = a->resource; sp->cpu_id = cpu_id; sp->cpu_row = *op;
+          sp->start = ts; sp->end = ts + dur;
+        }
+        if (ts < sp->start || sp->start == 0) sp->start = ts;
+        if (ts + dur > sp->end) sp->end = ts + dur;
+      }
+    }
     if (linked >= 0) {
       a->has_linked = 1; a->linked_corr = s->generic[linked].id; o->n_linked++;
       const ktj_generic_rec* op = &s->generic[linked]; /* the op hands its collective metadata to kernels */
@@ -760,6 +797,30 @@ static int stage_join(ktj_oracle* o) {
     }
   }
 
+  /* GpuUserEventMap::logEvents (GenericActivityProfiler.cpp:313-319, called at :726): after every
+   * GPU activity, stream by stream (std::map order) and, inside a stream, in the iteration order
+   * of a std::unordered_map keyed by the annotation's id (taken from the C++ library) */
+  if (n_spans) {
+    int64_t* kd = (int64_t*)malloc(8 * n_spans); int64_t* kr = (int64_t*)malloc(8 * n_spans);
+    int64_t* ki = (int64_t*)malloc(8 * n_spans); uint64_t* ord = (uint64_t*)malloc(8 * n_spans);
+    if (!kd || !kr || !ki || !ord) abort();
+    for (uint64_t k = 0; k < n_spans; ++k) { kd[k] = spans[k].device; kr[k] = spans[k].resource; ki[k] = spans[k].cpu_id; }
+    ktj_oracle_span_map_order(kd, kr, ki, n_spans, ord);
+    for (uint64_t k = 0; k < n_spans; ++k) {
+      const user_span* sp = &spans[ord[k]];
+      const ktj_generic_rec* op = &s->generic[sp->cpu_row];
+      ktj_mat_activity* a = new_act(o);
+      a->ts = sp->start; a->dur = sp->end - sp->start;
+      a->device = sp->device; a->resource = sp->resource;
+      a->corr = sp->cpu_id;
+      a->type = KTJ_TYPE_GPU_USER_ANNOTATION;
+      a->name_id = op->name_id == KTJ_NONE ? o->builtin0 + BS_EMPTY : op->name_id;
+      a->arrival = s->n_generic + s->n_runtime + s->n_device + k;
+    }
+    free(kd); free(kr); free(ki); free(ord);
+  }
+  free(spans);
+  umap_free(&user_corr);
   free(flow_start);
   free(dev_stream);
   free(ents);

@@ -9,6 +9,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <set>
 #include <string>
 #include <unordered_map>
@@ -217,6 +218,45 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
     uint64_t grid[3];
     if (ksrc) pack_grid(*ksrc, grid);
     mat[ng + nr + i] = mat_device(d, ts, dur, res, valid, ext_of(d.id), ksrc ? grid : nullptr, has_size, size, coll_of(d.id));
+  }
+
+  // GPU user annotations (GenericActivityProfiler.cpp:277-327, 423-433): one span per (device,
+  // resource, annotation) over the in-window device rows, appended in the profiler's log order
+  if (s->n_usercorr) {
+    std::unordered_map<uint64_t, uint64_t> user;
+    for (uint64_t i = 0; i < s->n_usercorr; ++i) user[s->usercorr[i].correlation] = s->usercorr[i].external_id;
+    struct Span { int64_t dev, res, id, start, end; uint64_t op; };
+    std::vector<Span> spans;
+    std::map<std::pair<int64_t, int64_t>, std::unordered_map<int64_t, size_t>> streams;
+    for (uint64_t i = 0; i < nd; ++i) {
+      const MatRow& m = mat[ng + nr + i];
+      if (!(m.meta & KTJ_M_VALID)) continue;
+      auto ui = user.find(s->device[i].id);
+      if (ui == user.end()) continue;
+      auto ci = cpu_ids.find(ui->second);
+      if (ci == cpu_ids.end()) continue;
+      const int64_t id = s->generic[ci->second].id;
+      auto& per_stream = streams[{m.dev, m.res}];
+      auto it = per_stream.find(id);
+      if (it == per_stream.end()) {
+        it = per_stream.insert({id, spans.size()}).first;
+        spans.push_back({m.dev, m.res, id, m.ts, m.ts + m.dur, ci->second});
+      }
+      Span& sp = spans[it->second];
+      if (m.ts < sp.start || sp.start == 0) sp.start = m.ts;
+      if (m.ts + m.dur > sp.end) sp.end = m.ts + m.dur;
+    }
+    for (const auto& stream : streams) {
+      for (const auto& entry : stream.second) {
+        const Span& sp = spans[entry.second];
+        ktj_generic_rec r;
+        memset(&r, 0, sizeof r);
+        r.start_ns = sp.start; r.end_ns = sp.end; r.resource = sp.res; r.device = (int32_t)sp.dev;
+        r.id = (int32_t)sp.id; r.name_id = s->generic[sp.op].name_id; r.schema_id = KTJ_NONE;
+        r.type = KTJ_TYPE_GPU_USER_ANNOTATION;
+        mat.push_back(mat_generic(r));
+      }
+    }
   }
 
   // canonical order over valid rows

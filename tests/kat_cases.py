@@ -322,7 +322,64 @@ def case_collective_joined():
     return b, expect
 
 
-SUBSTRING_CASES = [case_collective_reference_test, case_collective_reference_test_quoted, case_collective_joined, case_counter_events, case_instant_and_stream_sync, case_logger_events, case_trace_span, case_benchmark_cpu_op, case_typed_kernel_args,
+def case_gpu_user_annotation_reference_test():
+    """The trace of libkineto/test/RocmActivityProfilerTest.cpp:770-833: one CPU annotation, two
+    kernels correlated with it in the user domain; an extra GPU_USER_ANNOTATION activity covers
+    both kernels on their device and queue: ts = first kernel's, duration = end of the second -
+    start of the first, correlation id and name of the CPU annotation.  It is printed one ns early
+    and two ns longer (output_json.cpp:862-869) with the annotation's id as External id."""
+    b = StreamBuilder(window=(B, B + 300), end_time=B + 300)
+    L = B + 20
+    b.add_generic("annotation", CPU_OP, L, L + 10, 4000, 4001, id=1)
+    b.add_usercorr(1, 1)
+    b.add_device(1, L + 5, L + 10, domain=0, name="kernel", queue=1)
+    b.add_usercorr(1, 1)
+    b.add_device(1, L + 15, L + 25, domain=0, name="kernel", queue=1)
+    expect = [
+        # kernel 1: ts = begin + 1 = 26 ns; kernel 2 ends at 45 ns: span 26..45, printed from 25 for 21
+        '"ph": "X",\n    "cat": "gpu_user_annotation",\n    "name": "annotation",\n    "pid": 0,\n    "tid": 1,\n    "ts": 0.025,\n    "dur": 0.021\n    ,\n    "args": {\n      "External id": 1\n    }\n  },',
+        '"cat": "kernel",\n    "name": "Kernel",\n    "pid": 0,\n    "tid": 1,\n    "ts": 0.026,\n    "dur": 0.004',
+        '"cat": "kernel",\n    "name": "Kernel",\n    "pid": 0,\n    "tid": 1,\n    "ts": 0.036,\n    "dur": 0.009',
+    ]
+    return b, expect
+
+
+def case_gpu_user_annotations():
+    """GPU user annotations over several streams and annotations (GenericActivityProfiler.cpp:277-327,
+    423-433): one span per (device, stream, annotation); rows outside the window, rows whose
+    correlation has no user record and user records that name no CPU activity add nothing; the
+    last user record of a correlation id and the last CPU activity of an id are the ones used; a
+    row that starts at time 0 makes the next row's start replace the span's (start rule :304-306)."""
+    b = StreamBuilder(window=(0, B + 10**6), end_time=B + 10**6)
+    b.add_generic("step A", 1, B + 10, B + 500, 7, 8, id=50)                  # USER_ANNOTATION
+    b.add_generic("step B (shadowed)", 1, B + 20, B + 600, 7, 8, id=51)
+    b.add_generic('step B "final"', 1, B + 30, B + 700, 7, 8, id=51)          # same id: this one is looked up
+    b.add_generic("no kernels", 1, B + 40, B + 800, 7, 8, id=52)
+    b.add_generic("zero", 1, B + 50, B + 900, 7, 8, id=0)                     # id 0: no External id printed
+    for corr, ext in [(1, 50), (2, 50), (3, 51), (4, 51), (5, 99), (6, 50), (3, 52), (3, 51), (7, 0), (8, 0), (9, 0), (10, 50)]:
+        b.add_usercorr(corr, ext)
+    b.add_device(2, B + 3000, B + 3500, domain=0, name="k2", queue=1)         # A on queue 1 (later in time, first in arrival)
+    b.add_device(1, B + 1000, B + 1200, domain=0, name="k1", queue=1)         # A on queue 1: earliest
+    b.add_device(6, B + 2000, B + 9000, domain=1, op=2, queue=2)              # A on queue 2 (a copy)
+    b.add_device(3, B + 4000, B + 4100, domain=0, name="k3", queue=1)         # B on queue 1
+    b.add_device(4, B + 100, B + 200, domain=0, name="k4", queue=1, device=1) # B on another device
+    b.add_device(5, B + 5000, B + 5100, domain=0, name="k5", queue=1)         # annotation 99 does not exist
+    b.add_device(11, B + 6000, B + 6100, domain=0, name="k11", queue=1)       # no user record
+    b.add_device(10, B + 2 * 10**6, B + 2 * 10**6 + 9, domain=0, name="late", queue=3)  # outside the window
+    b.add_device(7, 40, 60, domain=2, stream=9, queue=5, nbytes=16)           # memset rows start at `begin`
+    b.add_device(8, 0, 30, domain=2, stream=9, queue=5, nbytes=16)            # starts at time 0 ...
+    b.add_device(9, 70, 90, domain=2, stream=9, queue=5, nbytes=16)           # ... so this start replaces it
+    expect = [
+        '"cat": "gpu_user_annotation",\n    "name": "step A",\n    "pid": 0,\n    "tid": 1,\n    "ts": 1.000,\n    "dur": 2.501\n    ,\n    "args": {\n      "External id": 50\n    }',
+        '"cat": "gpu_user_annotation",\n    "name": "step A",\n    "pid": 0,\n    "tid": 2,\n    "ts": 2.000,\n    "dur": 7.001\n    ,\n    "args": {\n      "External id": 50\n    }',
+        '"cat": "gpu_user_annotation",\n    "name": "step B \\"final\\"",\n    "pid": 0,\n    "tid": 1,\n    "ts": 4.000,\n    "dur": 0.101\n    ,',
+        '"cat": "gpu_user_annotation",\n    "name": "step B \\"final\\"",\n    "pid": 1,\n    "tid": 1,\n    "ts": 0.100,\n    "dur": 0.101\n    ,',
+        '"cat": "gpu_user_annotation",\n    "name": "zero",\n    "pid": 0,\n    "tid": 9,\n    "ts": 0.000,\n    "dur": 0.022\n    \n  },',
+    ]
+    return b, expect
+
+
+SUBSTRING_CASES = [case_gpu_user_annotation_reference_test, case_gpu_user_annotations, case_collective_reference_test, case_collective_reference_test_quoted, case_collective_joined, case_counter_events, case_instant_and_stream_sync, case_logger_events, case_trace_span, case_benchmark_cpu_op, case_typed_kernel_args,
                    case_typed_metadata_pins, case_names, case_resource_infos]
 
 

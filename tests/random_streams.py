@@ -134,6 +134,9 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False)
                      queue=rng.choice([0, 1, 2, 3, 2**63 + 5]), stream=rng.choice([0, 0, 0, 5, 0x7000]), nbytes=rng.choice([0, 1000, 2**40]))
     for _ in range(rng.randrange(0, 40)):
         b.add_extcorr(rng.choice(ids + [0xFFFFFFFFFFFFFFFF]), rng.choice([5, 6, 7, 8, 0, 2**31 - 1, 0xFFFFFFFF80000000, 2**40, 12345]))
+    if rng.random() < 0.5:  # user-domain correlation: GPU user-annotation spans
+        for _ in range(rng.randrange(1, 40)):
+            b.add_usercorr(rng.choice(ids + [100, 0]), rng.choice([5, 6, 7, 8, 0, 2**31 - 1, 0xFFFFFFFF80000000, 2**40, 12345]))
     if rng.random() < 0.5:
         b.add_device_info(0, 5000000, 'GPU "zero"', "GPU 0", B + 10)
         b.add_resource_info(5, 5, 0, 'stream "5"', False, B + 10)

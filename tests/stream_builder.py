@@ -27,6 +27,7 @@ class StreamBuilder:
         self.generic, self.runtime, self.device, self.extcorr = [], [], [], []
         self.device_infos, self.resource_infos, self.overhead_infos, self.spans = [], [], [], []
         self.collectives = []
+        self.usercorr = []
         self._keep = []
 
     # ---- dictionary / schemas ----
@@ -112,6 +113,9 @@ class StreamBuilder:
     def add_extcorr(self, corr, ext):
         self.extcorr.append(abi.ExtCorrRec(corr, ext))
 
+    def add_usercorr(self, corr, ext):
+        self.usercorr.append(abi.ExtCorrRec(corr & 0xFFFFFFFFFFFFFFFF, ext & 0xFFFFFFFFFFFFFFFF))
+
     def add_device_info(self, id, sort_index, name, label, t=None):
         self.device_infos.append(abi.DeviceInfo(id, sort_index, name.encode(), label.encode(), self.base if t is None else t))
 
@@ -166,6 +170,7 @@ class StreamBuilder:
         st.end_time_ns = self.end_time
         for name, ctype, items in (("generic", abi.GenericRec, self.generic), ("runtime", abi.RuntimeRec, self.runtime),
                                    ("device", abi.DeviceRec, self.device), ("extcorr", abi.ExtCorrRec, self.extcorr),
+                                   ("usercorr", abi.ExtCorrRec, self.usercorr),
                                    ("device_infos", abi.DeviceInfo, self.device_infos),
                                    ("resource_infos", abi.ResourceInfo, self.resource_infos),
                                    ("overhead_infos", abi.OverheadInfo, self.overhead_infos),

@@ -125,6 +125,21 @@ def test_random_streams_on_gpu(seed):
     _engine_vs_oracle(sp, hash_join=True, tile_emit=True)
 
 
+@pytest.mark.parametrize("cfg,n", [(3, 20000), (4, 6000), (2, 9000)])
+def test_user_annotation_spans_at_scale(cfg, n):
+    """Thousands of GPU user-annotation spans: every external-correlation record of a synthetic stream
+    is also submitted in the user domain, so each (stream, CPU op) pair with kernels gets a span."""
+    print(f"user annotation spans cfg={cfg} n={n}", flush=True)
+    sp, release = abi.synth_stream(cfg, n, host_name="box")
+    try:
+        s = sp.contents
+        s.usercorr, s.n_usercorr = s.extcorr, s.n_extcorr
+        _engine_vs_oracle(sp, check_substrings=('"cat": "gpu_user_annotation"',))
+        _engine_vs_oracle(sp, hash_join=True)
+    finally:
+        release()
+
+
 def test_join_edge_cases_on_gpu():
     import test_join_bruteforce as tj
     import inspect

@@ -4,6 +4,8 @@ reference's ROCm post-processing does row by row (dicts in arrival order):
   stream back-fill       RocmStreamQueue.h:42-136
   grid/block/bytes       RocprofActivity_inl.h:28-30, 147-180, 208-277 (thread_local maps keyed by int)
   window filter / order  GenericActivityProfiler.cpp:329-340, 363-395
+  GPU user annotations   GenericActivityProfiler.cpp:277-327, 423-433 (spans compared as a set: their
+                         relative order is the iteration order of the profiler's own maps)
 on small synthetic streams and on hand-made streams with duplicate ids, ids that collide after
 narrowing, ambiguous queues and out-of-window launch rows."""
 import ctypes as C
@@ -56,7 +58,7 @@ def brute(sp):
     for i in range(s.n_generic):
         g = s.generic[i]
         acts.append(dict(arrival=i, ts=g.start_ns, dur=g.end_ns - g.start_ns, device=g.device, resource=g.resource,
-                         type=g.type, linked=None, extra={}))
+                         type=g.type, linked=(g.linked_id if g.flags & 2 else None), extra={}))
         activity_map[g.id] = i
     cpu_corr = {}
     for i in range(s.n_extcorr):
@@ -139,6 +141,11 @@ def brute(sp):
                 m[key] = len(m) + 1
             dstream[i] = m[key]
 
+    user_corr = {}
+    for i in range(s.n_usercorr):
+        user_corr[to_i64(s.usercorr[i].correlation)] = to_i64(s.usercorr[i].external_id)
+    spans = {}  # (device, resource, annotation id) -> [start, end, generic index], insertion-ordered
+
     to_grid, to_size = {}, {}
     for i in range(s.n_runtime):
         r = s.runtime[i]
@@ -185,7 +192,19 @@ def brute(sp):
         typ = 4 if d.domain == 2 else (3 if d.domain == 1 else 5)
         acts.append(dict(arrival=s.n_generic + s.n_runtime + i, ts=ts, dur=dur, device=d.device, resource=res, type=typ,
                          linked=lk, extra=extra))
-    return acts, counters
+        ext = user_corr.get(to_i64(d.id)) if s.n_usercorr else None
+        gi = activity_map.get(ext) if ext is not None else None
+        if gi is not None:
+            key = (d.device, res, s.generic[gi].id)
+            if key not in spans:
+                spans[key] = [ts, ts + dur, gi]
+            sp = spans[key]
+            if ts < sp[0] or sp[0] == 0:
+                sp[0] = ts
+            sp[1] = max(sp[1], ts + dur)
+    span_acts = [dict(ts=v[0], dur=v[1] - v[0], device=k[0], resource=k[1], type=2, linked=None, corr=k[2],
+                      name=s.generic[v[2]].name_id) for k, v in spans.items()]
+    return acts, counters, span_acts
 
 
 def oracle_extra(o, a):
@@ -208,10 +227,21 @@ def oracle_extra(o, a):
 
 
 def compare(sp):
-    want, counters = brute(sp)
+    want, counters, want_spans = brute(sp)
     o = og.OracleRun(sp)
-    acts, n = o.activities()
-    assert n == len(want)
+    acts, n_all = o.activities()
+    n = len(want)
+    assert n_all == n + len(want_spans)
+    # the synthesised spans follow every other activity; compared as a set
+    def stream_string(sid):
+        s = sp.contents
+        return b"" if sid == abi.KTJ_NONE else C.string_at(s.str_blob + s.str_off[sid], s.str_off[sid + 1] - s.str_off[sid])
+    got_spans = sorted((acts[i].device, acts[i].resource, acts[i].corr, acts[i].ts, acts[i].dur, acts[i].type,
+                        o.string(acts[i].name_id), acts[i].has_linked) for i in range(n, n_all))
+    assert got_spans == sorted((w["device"], w["resource"], w["corr"], w["ts"], w["dur"], 2, stream_string(w["name"]), 0)
+                               for w in want_spans)
+    assert [acts[i].arrival for i in range(n, n_all)] == [sp.contents.n_generic + sp.contents.n_runtime + sp.contents.n_device + k
+                                                          for k in range(n_all - n)]
     for i in range(n):
         a, w = acts[i], want[i]
         got = dict(arrival=a.arrival, ts=a.ts, dur=a.dur, device=a.device, resource=a.resource, type=a.type,
@@ -225,7 +255,8 @@ def compare(sp):
     assert c["out_of_order"] == counters["out_of_order"]
     # canonical order: stable sort by (device, resource, ts)
     order = o.order()
-    exp = sorted(range(n), key=lambda i: (want[i]["device"], want[i]["resource"], want[i]["ts"]))
+    keys = [(w["device"], w["resource"], w["ts"]) for w in want] + [(acts[i].device, acts[i].resource, acts[i].ts) for i in range(n, n_all)]
+    exp = sorted(range(n_all), key=lambda i: keys[i])
     assert order == exp
     o.close()
 
@@ -235,6 +266,18 @@ def test_join_on_small_synthetic_streams(cfg, n):
     sp, release = abi.synth_stream(cfg, n)
     compare(sp)
     release()
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_join_on_random_streams(seed):
+    import random_streams
+    compare(random_streams.random_stream(seed, wide_ids=seed % 2 == 1).build())
+
+
+def test_user_annotation_spans():
+    import kat_cases
+    for case in (kat_cases.case_gpu_user_annotation_reference_test, kat_cases.case_gpu_user_annotations):
+        compare(case()[0].build())
 
 
 def test_join_edge_cases():
