@@ -32,9 +32,17 @@ using namespace ktj::gpu;
 
 namespace {
 
-struct DevBuf {
+struct DevBuf { /* owns one device allocation; freed with the engine (the engine's device is current then) */
   void* p = nullptr;
   size_t cap = 0;
+  DevBuf() = default;
+  DevBuf(const DevBuf&) = delete;
+  DevBuf& operator=(const DevBuf&) = delete;
+  DevBuf& operator=(DevBuf&& o) noexcept {
+    if (this != &o) { release(); p = o.p; cap = o.cap; o.p = nullptr; o.cap = 0; }
+    return *this;
+  }
+  ~DevBuf() { release(); }
   hipError_t ensure(size_t bytes) {
     if (bytes <= cap) return hipSuccess;
     if (p) { hipError_t e = hipFree(p); p = nullptr; cap = 0; if (e != hipSuccess) return e; }
@@ -62,8 +70,7 @@ struct DevVec {
       if (bytes) { e = hipMemcpyAsync(nb.p, buf.p, bytes, hipMemcpyDeviceToDevice, st); if (e != hipSuccess) return e; }
       e = hipStreamSynchronize(st);
       if (e != hipSuccess) return e;
-      buf.release();
-      buf = nb;
+      buf = std::move(nb);
     }
     hipError_t e = hipMemcpyAsync(static_cast<char*>(buf.p) + bytes, src, n, hipMemcpyHostToDevice, st);
     if (e != hipSuccess) return e;
@@ -138,7 +145,7 @@ struct ktj_engine {
   DevBuf q_keys, q_stream, q_amb, dn_hash, dn_first, dn_dev, dn_key, dn_rank;
   DevBuf s_dev_k, s_dev_r, s_res_k, s_res_r;
   DevBuf keys_a, keys_b, vals_a, vals_b, hist, scan_tmp;
-  DevBuf mat, len, len_sorted, offs, out, tile_start;
+  DevBuf mat, len, len_sorted, kind_sorted, offs, out, tile_start;
   void* pinned_small = nullptr; size_t pinned_small_cap = 0;
   char* pinned_out = nullptr; size_t pinned_out_cap = 0;
   bool host_copy_valid = false;
@@ -315,17 +322,7 @@ void ktj_destroy(ktj_engine* e) {
   if (!e) return;
   (void)hipSetDevice(e->device);
   if (e->stream) (void)hipStreamSynchronize(e->stream);
-  DevBuf* bufs[] = {&e->d_fields, &e->d_schemas, &e->d_cid_names, &e->d_flow_bits, &e->d_scalars, &e->d_name_len,
-                    &e->d_arg_len, &e->d_sflags, &e->d_name_off, &e->d_arg_off, &e->d_name_blob, &e->d_arg_blob,
-                    &e->c_ts, &e->c_dur, &e->c_corr, &e->c_dev, &e->c_res, &e->c_meta, &e->c_ext, &e->t_full,
-                    &e->t_narrow, &e->t_cpu, &e->f_first, &e->f_stream_src, &e->f_pay, &e->n_ext_src, &e->n_kern_src,
-                    &e->n_copy_src, &e->n_pay, &e->slot_ext, &e->slot_f, &e->slot_n, &e->slot_f_dev, &e->dev_link, &e->dev_brief, &e->sync_keys, &e->sync_pos, &e->sync_first, &e->q_keys, &e->q_stream, &e->q_amb, &e->dn_hash, &e->dn_first, &e->dn_dev,
-                    &e->dn_key, &e->dn_rank, &e->s_dev_k, &e->s_dev_r, &e->s_res_k, &e->s_res_r, &e->keys_a,
-                    &e->keys_b, &e->vals_a, &e->vals_b, &e->hist, &e->scan_tmp, &e->mat, &e->len, &e->len_sorted,
-                    &e->offs, &e->out, &e->tile_start};
-  for (DevBuf* b : bufs) b->release();
-  e->str_blob.release(); e->str_off.release(); e->args.release();
-  e->generic.owned.release(); e->runtime.owned.release(); e->devrows.owned.release(); e->extcorr.owned.release();
+  /* device buffers free themselves when the engine is deleted below */
   if (e->pinned_small) (void)hipHostFree(e->pinned_small);
   if (e->pinned_out) (void)hipHostFree(e->pinned_out);
   for (auto& ev : e->ev) if (ev) (void)hipEventDestroy(ev);
@@ -621,7 +618,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
     if (m3 > m) m = m3;
     HIPCHK(e->scan_tmp.ensure(m * 8));
   }
-  HIPCHK(e->mat.ensure(Na * sizeof(MatRow))); HIPCHK(e->len.ensure(Na * 4)); HIPCHK(e->len_sorted.ensure(Na * 4));
+  HIPCHK(e->mat.ensure(Na * sizeof(MatRow))); HIPCHK(e->len.ensure(Na * 4)); HIPCHK(e->len_sorted.ensure(Na * 4)); HIPCHK(e->kind_sorted.ensure(Na + 16));
   HIPCHK(e->offs.ensure((Na + 1) * 8));
 
   Scalars* sc = e->d_scalars.as<Scalars>();
@@ -785,7 +782,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(mat_generic_rows(e->synth_recs.as<ktj_generic_rec>(), e->n_spans, ng + nr + nd, ctx, nullptr, mat, e->len.as<uint32_t>(),
                           sc, st));
   HIPCHK(mat_device_rows(d_recs, nd, c, ng + nr, e->dev_link.as<DevLink>(), ctx, mat, e->len.as<uint32_t>(), sc, st));
-  HIPCHK(gather_len(e->perm, e->len.as<uint32_t>(), N, e->len_sorted.as<uint32_t>(), st));
+  HIPCHK(gather_len(e->perm, e->len.as<uint32_t>(), N, e->len_sorted.as<uint32_t>(), e->kind_sorted.as<uint8_t>(), st));
   if (n_coll) HIPCHK(collective_first(mat, e->perm, e->scalars.n_valid, n_coll, e->d_coll_first.as<uint32_t>(), st));
   HIPCHK(hipEventRecord(e->ev[EV_SIZE], st));
 
@@ -841,7 +838,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
       HIPCHK(emit(mat, e->perm, e->offs.as<uint64_t>(), N, ctx, e->out.as<char>(), e->prefix_len, act_bytes, tile,
                   e->tile_start.as<uint32_t>(), st));
     else
-      HIPCHK(emit_direct(mat, e->perm, e->offs.as<uint64_t>(), e->len.as<uint32_t>(), e->scalars.n_valid, act_bytes, ctx,
+      HIPCHK(emit_direct(mat, e->perm, e->offs.as<uint64_t>(), e->kind_sorted.as<uint8_t>(), e->scalars.n_valid, act_bytes, ctx,
                          e->out.as<char>(), e->prefix_len, st));
   }
   HIPCHK(hipEventRecord(e->ev[EV_EMIT], st));

@@ -270,7 +270,8 @@ hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uin
                             uint32_t* len, Scalars* sc, hipStream_t st);
 hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const DevLink* link,
                            EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st);
-hipError_t gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted, hipStream_t st);
+hipError_t gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted, uint8_t* kind_sorted,
+                      hipStream_t st);
 
 /* ---- stage 4b: emit ---- */
 /* tile size (bytes of output per workgroup) for a document whose activity section has act_bytes
@@ -281,9 +282,9 @@ hipError_t emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs /*
                 EmitCtx ctx, char* out, uint64_t prefix_len, uint64_t act_bytes, uint32_t tile,
                 uint32_t* tile_start /* tiles + 1 */, hipStream_t st);
 
-/* direct variant: one lane per activity, no LDS staging; len_kind is the arrival-order length
- * array whose top two bits carry the tail kind; n_rows = number of activities that are written */
-hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint32_t* len_kind,
+/* direct variant: one lane per activity, no LDS staging; kind_sorted holds the tail kind of every
+ * activity in emission order (gather_len); n_rows = number of activities that are written */
+hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint8_t* kind_sorted,
                        uint64_t n_rows, uint64_t act_bytes, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st);
 
 }  // namespace gpu

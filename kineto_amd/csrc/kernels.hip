@@ -1522,9 +1522,13 @@ hipError_t collective_first(const MatRow* mat, const uint32_t* perm, uint64_t n_
                      first);
   return KTJ_LAUNCH_CHECK();
 }
-__global__ void k_gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted) {
+/* lengths and tail kinds in emission order (the size pass leaves both in one word per arrival index) */
+__global__ void k_gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted, uint8_t* kind_sorted) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) len_sorted[i] = len[perm[i]] & 0x3FFFFFFFu;
+  if (i >= n) return;
+  const uint32_t v = len[perm[i]];
+  len_sorted[i] = v & 0x3FFFFFFFu;
+  kind_sorted[i] = (uint8_t)(v >> 30);
 }
 
 hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, uint64_t first, EmitCtx ctx, const uint32_t* sync_first,
@@ -1549,9 +1553,10 @@ hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint6
                      mat, len, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted, hipStream_t st) {
+hipError_t gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted, uint8_t* kind_sorted,
+                      hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_gather_len, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, perm, len, n, len_sorted);
+  hipLaunchKernelGGL(k_gather_len, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, perm, len, n, len_sorted, kind_sorted);
   return KTJ_LAUNCH_CHECK();
 }
 
@@ -1666,7 +1671,7 @@ k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n
  * prefix and suffix are already in place when this kernel runs; the first and the last activity
  * merge with them. */
 __global__ void __launch_bounds__(KTJ_BLOCK)
-k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint32_t* len_kind, uint64_t n_rows,
+k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint8_t* kind_sorted, uint64_t n_rows,
               EmitCtx ctx, char* out, uint64_t prefix_len) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n_rows) return;
@@ -1678,7 +1683,7 @@ k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, con
   uint64_t low = 0;
   if (fill) {
     if (i == 0) low = *reinterpret_cast<const uint64_t*>(out + (pos & ~7ULL)) & ((1ULL << (8 * fill)) - 1ULL);
-    else low = tail_bytes(len_kind[perm[i - 1]] >> 30, fill);
+    else low = tail_bytes(kind_sorted[i - 1], fill);
   }
   GlobalWriter w;
   w.begin(out, pos, low);
@@ -1689,7 +1694,7 @@ k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, con
     *last = (*last & ~mask) | (w.acc & mask);
   }
 }
-hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint32_t* len_kind,
+hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint8_t* kind_sorted,
                        uint64_t n_rows, uint64_t act_bytes, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st) {
   if (n_rows == 0) return hipSuccess;
   /* Every lane keeps one partially written 128-byte line open at a time.  At full occupancy
@@ -1701,7 +1706,7 @@ hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* 
    * (measured 13% slower at 1.4 KB per activity), so it is applied below 768 bytes per activity. */
   const size_t residency_lds = act_bytes / n_rows < 768 ? 60000 : 0;
   hipLaunchKernelGGL(k_emit_direct, dim3(grid_for(n_rows, KTJ_BLOCK)), dim3(KTJ_BLOCK), residency_lds, st, mat, perm, offs,
-                     len_kind, n_rows, ctx, out, prefix_len);
+                     kind_sorted, n_rows, ctx, out, prefix_len);
   return KTJ_LAUNCH_CHECK();
 }
 
