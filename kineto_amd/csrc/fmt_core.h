@@ -544,6 +544,158 @@ struct WordWriter {
 };
 typedef WordWriter<DirectSink> GlobalWriter;
 
+/* Pass B with 16-byte blocks.  Like WordWriter, but bytes are gathered in a 128-bit accumulator and
+ * leave as aligned 16-byte stores, and literal text is appended sixteen bytes at a time, so that
+ * all lanes of a wavefront complete a block at the same append and half as many store
+ * instructions are issued.  Every block of the document has exactly one writer who knows all of
+ * its bytes: a block that holds the end of activity A and the start of activity B is written
+ *   - by B, if fewer than eight bytes of it are A's: they are one of the fixed tails (tail_kind);
+ *   - by A otherwise: the at most eight bytes of B in it are the same for every activity
+ *     ("\n  {\n    ", the start of each event of every kind).
+ * The first activity reads what precedes it from the document, the last one merges with what
+ * follows it; both were put in place by the host before the kernel runs. */
+struct BlockWriter {
+  uint64_t* wptr;     /* the 16-byte block being gathered (as two words) */
+  uint64_t lo, hi;    /* its first `fill` bytes */
+  uint32_t fill;      /* 0..15 */
+  bool foreign;       /* the block belongs to the predecessor: gathered but not stored */
+
+  KTJ_HD KTJ_FI static uint64_t head_bytes() { constexpr auto h = pack_lit("\n  {\n   "); return h.w[0]; }
+  KTJ_HD KTJ_FI void store_block() {
+    if (!foreign) {
+#if defined(__HIP_DEVICE_COMPILE__)
+      typedef unsigned long long v2u64 __attribute__((ext_vector_type(2)));
+      v2u64 v; v.x = lo; v.y = hi;
+      *reinterpret_cast<v2u64*>(wptr) = v;
+#else
+      wptr[0] = lo; wptr[1] = hi;
+#endif
+    }
+    foreign = false;
+    wptr += 2;
+  }
+  /* pos: where the activity starts; tail_kind_before: kind of the activity before it */
+  KTJ_HD KTJ_FI void begin(char* doc, uint64_t pos, uint32_t tail_kind_before, bool first);
+  KTJ_HD KTJ_FI void end(bool last);
+  /* bytes gathered so far count from the document start */
+  KTJ_HD KTJ_FI uint64_t position(const char* doc) const { return (uint64_t)((const char*)wptr - doc) + fill; }
+
+  /* append the n (0..8) low bytes of v; bytes above n must be zero */
+  KTJ_HD KTJ_FI void append(uint64_t v, uint32_t n) {
+    const uint32_t r = (fill & 7u) * 8u;
+    const uint64_t t0 = v << r, t1 = r ? v >> (64u - r) : 0;
+    if (fill < 8) { lo |= t0; hi |= t1; }
+    else hi |= t0;
+    const uint32_t total = fill + n;
+    if (total >= 16) { /* only from the upper half: t1 starts the next block */
+      store_block();
+      lo = t1; hi = 0;
+      fill = total - 16;
+    } else fill = total;
+  }
+  /* sixteen bytes at once: completes exactly one block whatever the fill */
+  KTJ_HD KTJ_FI void append16(uint64_t a, uint64_t b) {
+    const uint32_t r = (fill & 7u) * 8u;
+    const uint64_t t0 = a << r;
+    const uint64_t t1 = r ? (b << r) | (a >> (64u - r)) : b;
+    const uint64_t t2 = r ? b >> (64u - r) : 0;
+    if (fill < 8) { lo |= t0; hi |= t1; store_block(); lo = t2; hi = 0; }
+    else { hi |= t0; store_block(); lo = t1; hi = t2; }
+  }
+  KTJ_HD KTJ_FI void ch(char c) { append((uint64_t)(unsigned char)c, 1); }
+  template <unsigned N> KTJ_HD KTJ_FI void lit(const PackedLit<N>& l) {
+    for (unsigned i = 0; i < N / 16; ++i) append16(l.w[2 * i], l.w[2 * i + 1]);
+    if ((N % 16) >= 8) append(l.w[(N / 16) * 2], 8);
+    if (N % 8) append(l.w[N / 8], N % 8);
+  }
+  KTJ_HD KTJ_FI void dec_wide(uint64_t v) {
+    const uint64_t top = v / 10000000000000000ULL;
+    const uint64_t rest = v - top * 10000000000000000ULL;
+    const uint64_t mid = rest / 100000000ULL;
+    const uint32_t low = (uint32_t)(rest - mid * 100000000ULL);
+    uint64_t a0 = 0, a1;
+    uint32_t n0 = 0, n1;
+    if (top) {
+      a0 = ascii8((uint32_t)top);
+      const uint32_t z = leading_zero_chars(a0);
+      a0 >>= 8 * z; n0 = 8 - z;
+      a1 = ascii8((uint32_t)mid); n1 = 8;
+    } else {
+      a1 = ascii8((uint32_t)mid);
+      const uint32_t z = leading_zero_chars(a1);
+      a1 >>= 8 * z; n1 = 8 - z;
+    }
+    append(a0, n0);
+    append(a1, n1);
+    append(ascii8(low), 8);
+  }
+  KTJ_HD KTJ_FI void dec(uint64_t v) {
+    if (__builtin_expect(v < 100000000ULL, 1)) {
+      const uint64_t a = ascii8((uint32_t)v);
+      const uint32_t z = leading_zero_chars(a);
+      append(a >> (8 * z), 8 - z);
+    } else dec_wide(v);
+  }
+  typedef Num Prepared;
+  KTJ_HD KTJ_FI static Prepared prepare(uint64_t v) { return make_num(v); }
+  KTJ_HD KTJ_FI void num(const Num& n) {
+    if (__builtin_expect(n.len != 0, 1)) append(n.word, n.len); else dec_wide(n.value);
+  }
+  KTJ_HD KTJ_FI void dec3(uint32_t x) { append((uint64_t)(ascii4(x) >> 8), 3); }
+  /* a dictionary string copied by this lane: aligned 8-byte loads, funnel-shifted, sixteen bytes
+   * per append while they last */
+  KTJ_HD KTJ_FI void str_own(const char* src, uint64_t len) {
+    if (len == 0) return;
+    const uintptr_t sa = (uintptr_t)src;
+    const uint32_t sh = (uint32_t)(sa & 7u) * 8u;
+    const uint64_t* sp = reinterpret_cast<const uint64_t*>(sa & ~(uintptr_t)7);
+    uint64_t cur = sp[0];
+    const uint64_t full = len >> 3;
+    uint64_t k = 0;
+    KTJ_NOUNROLL
+    for (; k + 2 <= full; k += 2) {
+      const uint64_t n1 = sp[k + 1], n2 = sp[k + 2];
+      append16(sh ? (cur >> sh) | (n1 << (64u - sh)) : cur, sh ? (n1 >> sh) | (n2 << (64u - sh)) : n1);
+      cur = n2;
+    }
+    if (k < full) {
+      const uint64_t next = sp[k + 1];
+      append(sh ? (cur >> sh) | (next << (64u - sh)) : cur, 8);
+      cur = next;
+    }
+    const uint32_t rem = (uint32_t)(len & 7u);
+    if (rem) {
+      uint64_t v = cur >> sh;
+      if (sh && rem * 8u > 64u - sh) v |= sp[full + 1] << (64u - sh);
+      append(v & ((1ULL << (8 * rem)) - 1ULL), rem);
+    }
+  }
+  KTJ_HD KTJ_FI void str(const char* src, uint64_t len) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const bool big = len >= KTJ_COOP_MIN_BYTES;
+    if (__any(big)) { /* see cooperative_word_copy */
+      const char* body = src;
+      uint64_t* dst = nullptr;
+      uint32_t n_words = 0;
+      uint64_t tail = 0;
+      if (big) {
+        const uint32_t head = (16u - fill) & 15u;   /* bytes that complete the block being gathered */
+        str_own(src, head);                          /* now fill == 0 and the accumulator is empty */
+        body = src + head;
+        n_words = (uint32_t)((len - head) >> 4) * 2u; /* whole blocks, as words */
+        tail = (len - head) & 15u;
+        dst = wptr;
+        wptr += n_words;
+      } else str_own(src, len);
+      cooperative_word_copy(body, dst, n_words);
+      if (big) str_own(body + (uint64_t)n_words * 8u, tail);
+      return;
+    }
+#endif
+    str_own(src, len);
+  }
+};
+
 /* The last seven bytes of a formatted activity, by kind (see format_activity):
  *   0: `  \n  },`   complete event without args, or a flow-start event
  *   1: ` }\n  },`   complete or instant event with args and no flow event, or a counter event
@@ -562,6 +714,35 @@ KTJ_HD KTJ_FI inline uint64_t tail_bytes(uint32_t kind, uint32_t count) { /* las
   constexpr auto t2 = pack_lit("e\"\n  },");
   const uint64_t t = kind == 0 ? t0.w[0] : (kind == 1 ? t1.w[0] : t2.w[0]);
   return t >> (8 * (7 - count));
+}
+
+KTJ_HD KTJ_FI inline void BlockWriter::begin(char* doc, uint64_t pos, uint32_t tail_kind_before, bool first) {
+  wptr = reinterpret_cast<uint64_t*>(doc + (pos & ~15ULL));
+  fill = (uint32_t)(pos & 15ULL);
+  lo = 0; hi = 0;
+  foreign = false;
+  if (fill == 0) return;
+  if (first) { /* what precedes the first activity is in the document already */
+    lo = wptr[0]; hi = wptr[1];
+    if (fill < 8) { lo &= (1ULL << (8 * fill)) - 1ULL; hi = 0; }
+    else if (fill > 8) hi &= (1ULL << (8 * (fill - 8))) - 1ULL;
+    else hi = 0;
+  } else if (fill < 8) lo = tail_bytes(tail_kind_before, fill);
+  else foreign = true; /* the predecessor wrote this block, my first bytes included */
+}
+KTJ_HD KTJ_FI inline void BlockWriter::end(bool last) {
+  if (fill == 0) return;
+  if (last) { /* merge with the bytes that follow the last activity */
+    if (fill < 8) { const uint64_t m = (1ULL << (8 * fill)) - 1ULL; lo |= wptr[0] & ~m; hi = wptr[1]; }
+    else if (fill > 8) { const uint64_t m = (1ULL << (8 * (fill - 8))) - 1ULL; hi |= wptr[1] & ~m; }
+    else hi = wptr[1];
+    store_block();
+    return;
+  }
+  if (fill >= 8) { /* my block: the successor's first bytes complete it */
+    const uint32_t n = 16u - fill;
+    append(n == 8 ? head_bytes() : head_bytes() & ((1ULL << (8 * n)) - 1ULL), n);
+  }
 }
 
 /* ---------------------------------------------------------------------------------------- */

@@ -1678,21 +1678,10 @@ k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, con
   const uint64_t o = offs[i];
   if (offs[i + 1] == o) return;
   const MatRow m = mat[perm[i]];
-  const uint64_t pos = prefix_len + o;
-  const uint32_t fill = (uint32_t)(pos & 7ULL);
-  uint64_t low = 0;
-  if (fill) {
-    if (i == 0) low = *reinterpret_cast<const uint64_t*>(out + (pos & ~7ULL)) & ((1ULL << (8 * fill)) - 1ULL);
-    else low = tail_bytes(kind_sorted[i - 1], fill);
-  }
-  GlobalWriter w;
-  w.begin(out, pos, low);
+  BlockWriter w;
+  w.begin(out, prefix_len + o, i ? kind_sorted[i - 1] : 0u, i == 0);
   format_activity(w, m, ctx);
-  if (w.fill && i + 1 == n_rows) { /* last activity: merge with the suffix bytes behind it */
-    const uint64_t mask = (1ULL << (8 * w.fill)) - 1ULL;
-    uint64_t* last = w.sink.next_word();
-    *last = (*last & ~mask) | (w.acc & mask);
-  }
+  w.end(i + 1 == n_rows);
 }
 hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint8_t* kind_sorted,
                        uint64_t n_rows, uint64_t act_bytes, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st) {

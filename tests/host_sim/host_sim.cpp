@@ -313,7 +313,7 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   // document bytes [k*T, (k+1)*T) clipped to the activity section; tile-local coordinate
   // L = absolute offset - k*T
   if (tile_bytes == 0) {
-    // direct variant: one "lane" per activity, aligned 8-byte stores; the buffer is over-allocated
+    // direct variant: one "lane" per activity, aligned 16-byte blocks; the buffer is over-allocated
     // so that aligned accesses at the end stay inside it
     std::vector<uint32_t> kinds(perm.size());
     for (size_t i = 0; i < perm.size(); ++i) {
@@ -322,22 +322,11 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
     }
     const uint64_t P = prefix.size();
     for (size_t i = 0; i < perm.size(); ++i) {
-      const uint64_t pos = P + offs[i];
-      const uint32_t fill = (uint32_t)(pos & 7);
-      uint64_t low = 0;
-      if (fill) {
-        if (i == 0) { uint64_t cur; memcpy(&cur, buf + (pos & ~7ULL), 8); low = cur & ((1ULL << (8 * fill)) - 1); }
-        else low = tail_bytes(kinds[i - 1], fill);
-      }
-      GlobalWriter w;
-      w.begin(buf, pos, low);
+      BlockWriter w;
+      w.begin(buf, P + offs[i], i ? kinds[i - 1] : 0u, i == 0);
       format_activity(w, mat[perm[i]], ctx);
-      if ((uint64_t)((char*)w.sink.next_word() - buf) + w.fill != P + offs[i + 1]) { free(buf); return -2; }
-      if (w.fill && i + 1 == perm.size()) {
-        const uint64_t mask = (1ULL << (8 * w.fill)) - 1;
-        uint64_t* last = w.sink.next_word();
-        *last = (*last & ~mask) | (w.acc & mask);
-      }
+      if (w.position(buf) != P + offs[i + 1]) { free(buf); return -2; }
+      w.end(i + 1 == perm.size());
     }
     *out = buf;
     *out_n = total;
