@@ -387,20 +387,13 @@ struct TileWriter {
   }
 };
 
-/* Pass B: one lane formats one activity straight into the document in device memory.  Bytes are
- * gathered in a 64-bit accumulator and leave as aligned 8-byte words through a sink.  An
- * activity's first word also holds the last bytes of its predecessor; those are one of three
- * fixed strings (see tail_kind), so the successor writes the whole shared word and the
- * predecessor never writes its trailing partial word.  Dictionary strings are appended inline,
- * eight bytes at a time, through a funnel shift over aligned loads (dictionary blobs are padded
- * by 16 bytes so that the last load stays inside the allocation). */
-
 /* Long dictionary strings (templated C++ kernel names run to kilobytes) are not copied by the lane
  * that owns the activity but by all lanes that are active with it: for one owner at a time,
  * neighbouring lanes move neighbouring 8-byte words, so loads and stores are whole lines.  The
- * owner has already brought its output to a word boundary; `src` is the first byte that lands on
- * that boundary (any alignment: two aligned loads are funnel-shifted), `dst` the word, `n_words`
- * the whole words (0 for lanes that only help).  Works under any set of active lanes. */
+ * owner has already brought its output to a block boundary; `src` is the first byte that lands on
+ * that boundary (any alignment: two aligned loads are funnel-shifted), `dst` the block, `n_words`
+ * the 8-byte words of the whole blocks (0 for lanes that only help).  Works under any set of
+ * active lanes. */
 #define KTJ_COOP_MIN_BYTES 256u
 #if defined(__HIP_DEVICE_COMPILE__)
 static __device__ __attribute__((noinline)) void cooperative_word_copy(const char* src, uint64_t* dst, uint32_t n_words) {
@@ -427,127 +420,12 @@ static __device__ __attribute__((noinline)) void cooperative_word_copy(const cha
 }
 #endif
 
-/* every finished word is stored at once by the lane that gathered it */
-struct DirectSink {
-  uint64_t* wptr;     /* aligned address of the word being gathered */
-  KTJ_HD KTJ_FI void open(uint64_t* first_word) { wptr = first_word; }
-  KTJ_HD KTJ_FI void put(uint64_t w) { *wptr++ = w; }
-  KTJ_HD KTJ_FI void close() {}
-  KTJ_HD KTJ_FI uint64_t* next_word() const { return wptr; }
-  /* hands out `n` whole words that somebody else fills */
-  KTJ_HD KTJ_FI uint64_t* reserve(uint32_t n) { uint64_t* p = wptr; wptr += n; return p; }
-};
-
-template <class Sink>
-struct WordWriter {
-  Sink sink;
-  uint64_t acc;
-  uint32_t fill;      /* bytes gathered in acc, 0..7 */
-
-  KTJ_HD KTJ_FI void begin(char* doc, uint64_t pos, uint64_t low_bytes) {
-    sink.open(reinterpret_cast<uint64_t*>(doc + (pos & ~7ULL)));
-    fill = (uint32_t)(pos & 7ULL);
-    acc = low_bytes; /* the `fill` bytes that precede this activity in its first word */
-  }
-  KTJ_HD KTJ_FI void append(uint64_t v, uint32_t n) {
-    acc |= v << (8 * fill);
-    const uint32_t total = fill + n;
-    if (total >= 8) {
-      sink.put(acc);
-      const uint32_t rest = total - 8;
-      acc = rest ? v >> (8 * (n - rest)) : 0;
-      fill = rest;
-    } else fill = total;
-  }
-  KTJ_HD KTJ_FI void ch(char c) { append((uint64_t)(unsigned char)c, 1); }
-  template <unsigned N> KTJ_HD KTJ_FI void lit(const PackedLit<N>& l) {
-    for (unsigned i = 0; i < N / 8; ++i) append(l.w[i], 8);
-    if (N % 8) append(l.w[N / 8], N % 8);
-  }
-  KTJ_HD KTJ_FI void dec_wide(uint64_t v) {
-    const uint64_t top = v / 10000000000000000ULL;
-    const uint64_t rest = v - top * 10000000000000000ULL;
-    const uint64_t mid = rest / 100000000ULL;
-    const uint32_t low = (uint32_t)(rest - mid * 100000000ULL);
-    uint64_t a0 = 0, a1;
-    uint32_t n0 = 0, n1;
-    if (top) {
-      a0 = ascii8((uint32_t)top);
-      const uint32_t z = leading_zero_chars(a0);
-      a0 >>= 8 * z; n0 = 8 - z;
-      a1 = ascii8((uint32_t)mid); n1 = 8;
-    } else {
-      a1 = ascii8((uint32_t)mid);
-      const uint32_t z = leading_zero_chars(a1);
-      a1 >>= 8 * z; n1 = 8 - z;
-    }
-    append(a0, n0);
-    append(a1, n1);
-    append(ascii8(low), 8);
-  }
-  KTJ_HD KTJ_FI void dec(uint64_t v) {
-    if (__builtin_expect(v < 100000000ULL, 1)) {
-      const uint64_t a = ascii8((uint32_t)v);
-      const uint32_t z = leading_zero_chars(a);
-      append(a >> (8 * z), 8 - z);
-    } else dec_wide(v);
-  }
-  typedef Num Prepared;
-  KTJ_HD KTJ_FI static Prepared prepare(uint64_t v) { return make_num(v); }
-  KTJ_HD KTJ_FI void num(const Num& n) {
-    if (__builtin_expect(n.len != 0, 1)) append(n.word, n.len); else dec_wide(n.value);
-  }
-  KTJ_HD KTJ_FI void dec3(uint32_t x) { append((uint64_t)(ascii4(x) >> 8), 3); }
-  KTJ_HD KTJ_FI void str_own(const char* src, uint64_t len) {
-    if (len == 0) return;
-    const uintptr_t sa = (uintptr_t)src;
-    const uint32_t sh = (uint32_t)(sa & 7u) * 8u;
-    const uint64_t* sp = reinterpret_cast<const uint64_t*>(sa & ~(uintptr_t)7);
-    uint64_t cur = sp[0];
-    const uint64_t full = len >> 3;
-    KTJ_NOUNROLL
-    for (uint64_t k = 0; k < full; ++k) {
-      const uint64_t next = sp[k + 1];
-      append(sh ? (cur >> sh) | (next << (64u - sh)) : cur, 8);
-      cur = next;
-    }
-    const uint32_t rem = (uint32_t)(len & 7u);
-    if (rem) {
-      uint64_t v = cur >> sh;
-      if (sh && rem * 8u > 64u - sh) v |= sp[full + 1] << (64u - sh);
-      append(v & ((1ULL << (8 * rem)) - 1ULL), rem);
-    }
-  }
-  KTJ_HD KTJ_FI void str(const char* src, uint64_t len) {
-#if defined(__HIP_DEVICE_COMPILE__)
-    const bool big = len >= KTJ_COOP_MIN_BYTES;
-    if (__any(big)) { /* see cooperative_word_copy */
-      const char* body = src;
-      uint64_t* dst = nullptr;
-      uint32_t n_words = 0;
-      uint64_t tail = 0;
-      if (big) {
-        const uint32_t head = (8u - fill) & 7u;     /* bytes that complete the word being gathered */
-        str_own(src, head);                          /* now fill == 0 and acc == 0 */
-        body = src + head;
-        n_words = (uint32_t)((len - head) >> 3);
-        tail = (len - head) & 7u;
-        dst = sink.reserve(n_words);
-      } else str_own(src, len);
-      cooperative_word_copy(body, dst, n_words);
-      if (big) str_own(body + (uint64_t)n_words * 8u, tail);
-      return;
-    }
-#endif
-    str_own(src, len);
-  }
-};
-typedef WordWriter<DirectSink> GlobalWriter;
-
-/* Pass B with 16-byte blocks.  Like WordWriter, but bytes are gathered in a 128-bit accumulator and
- * leave as aligned 16-byte stores, and literal text is appended sixteen bytes at a time, so that
- * all lanes of a wavefront complete a block at the same append and half as many store
- * instructions are issued.  Every block of the document has exactly one writer who knows all of
+/* Pass B: one lane formats one activity straight into the document in device memory.  Bytes are
+ * gathered in a 128-bit accumulator and leave as aligned 16-byte stores; literal text is appended
+ * sixteen bytes at a time, so that all lanes of a wavefront complete a block at the same append
+ * and the wave issues one full store there, whatever the lanes' phases.  Dictionary strings are
+ * appended inline through a funnel shift over aligned 8-byte loads (dictionary blobs are padded by
+ * 16 bytes so that the last load stays inside the allocation).  Every block of the document has exactly one writer who knows all of
  * its bytes: a block that holds the end of activity A and the start of activity B is written
  *   - by B, if fewer than eight bytes of it are A's: they are one of the fixed tails (tail_kind);
  *   - by A otherwise: the at most eight bytes of B in it are the same for every activity
@@ -583,7 +461,7 @@ struct BlockWriter {
   /* append the n (0..8) low bytes of v; bytes above n must be zero */
   KTJ_HD KTJ_FI void append(uint64_t v, uint32_t n) {
     const uint32_t r = (fill & 7u) * 8u;
-    const uint64_t t0 = v << r, t1 = r ? v >> (64u - r) : 0;
+    const uint64_t t0 = v << r, t1 = (v >> 1) >> (63u - r); /* v >> (64 - r), 0 for r == 0 */
     if (fill < 8) { lo |= t0; hi |= t1; }
     else hi |= t0;
     const uint32_t total = fill + n;
@@ -597,8 +475,8 @@ struct BlockWriter {
   KTJ_HD KTJ_FI void append16(uint64_t a, uint64_t b) {
     const uint32_t r = (fill & 7u) * 8u;
     const uint64_t t0 = a << r;
-    const uint64_t t1 = r ? (b << r) | (a >> (64u - r)) : b;
-    const uint64_t t2 = r ? b >> (64u - r) : 0;
+    const uint64_t t1 = (b << r) | ((a >> 1) >> (63u - r)); /* x >> (64 - r), 0 for r == 0 */
+    const uint64_t t2 = (b >> 1) >> (63u - r);
     if (fill < 8) { lo |= t0; hi |= t1; store_block(); lo = t2; hi = 0; }
     else { hi |= t0; store_block(); lo = t1; hi = t2; }
   }

@@ -1670,7 +1670,7 @@ k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n
  * activity's lane together with the (fixed) last bytes of its predecessor.  The document's
  * prefix and suffix are already in place when this kernel runs; the first and the last activity
  * merge with them. */
-__global__ void __launch_bounds__(KTJ_BLOCK)
+__global__ void __launch_bounds__(KTJ_BLOCK) __attribute__((amdgpu_waves_per_eu(3)))
 k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint8_t* kind_sorted, uint64_t n_rows,
               EmitCtx ctx, char* out, uint64_t prefix_len) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
