@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0
 # (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter reads for the 1 GiB
 # k_copy_reference launch at the end of the run (2048 and 1024 bytes per unit).  Keyed by
 # (configuration, device rows); a counter run cannot share a process with the timed run.
-MEASURED_EMIT_TRAFFIC = {(3, 10000000): 3.64e9 + 13.31e9}
+MEASURED_EMIT_TRAFFIC = {(3, 10000000): 3.64e9 + 13.32e9}
 FULL_SIZE = {1: 10000, 2: 1000000, 3: 10000000, 4: 11000000, 5: 5000000}
 WORKLOAD = {
     1: "config1: 10k CPU ops + 10k launches + 10k kernels, 4 streams",

@@ -707,12 +707,11 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   MatRow* mat = e->mat.as<MatRow>();
   HIPCHK(build_extcorr(x_recs, nx, tn, nc, e->slot_ext.as<uint32_t>(), sc, st));
   HIPCHK(build_cpu_ids(g_recs, ng, t_cpu, cpu_row, sc, st));
-  HIPCHK(build_runtime(nr, c, ng, tf, fc, tn, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), sc, st));
-  HIPCHK(insert_device_first(nd, c, ng + nr, tf, fc, e->slot_f_dev.as<uint32_t>(), sc, st));
   HIPCHK(resolve_external(x_recs, nx, nc, e->slot_ext.as<uint32_t>(), t_cpu, cpu_row, g_recs, ctx, st));
-  /* second pass over the runtime rows: publishes into the tables and writes the joined rows */
-  HIPCHK(mat_runtime_rows(r_recs, nr, c, ng, api, fc, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), ctx, mat,
-                          e->len.as<uint32_t>(), sc, st));
+  HIPCHK(join_runtime_rows(r_recs, nr, c, ng, api, tf, fc, tn, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), ctx, mat,
+                           e->len.as<uint32_t>(), sc, st));
+  HIPCHK(insert_device_first(nd, c, ng + nr, tf, fc, e->slot_f_dev.as<uint32_t>(), sc, st));
+  HIPCHK(republish_runtime_rows(r_recs, nr, c, ng, fc, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), sc, st));
   HIPCHK(link_device_rows(nd, c, ng + nr, fc, tn, nc, e->slot_f_dev.as<uint32_t>(), e->dev_link.as<DevLink>(), sc, st));
   HIPCHK(backfill_streams(e->dev_brief.as<DevBrief>(), nd, c, ng + nr, stt, sc, st));
   if (max_spans) {

@@ -118,7 +118,7 @@ struct Scalars {
   unsigned int n_dev_ranks;           /* distinct deviceId values */
   unsigned int n_res_ranks;           /* distinct resourceId values */
   unsigned int n_dense;               /* distinct (device, stream key) pairs */
-  unsigned int pad;
+  unsigned int runtime_ids_repeat;    /* two runtime rows share a slot of the full table */
   JoinPlan plan;                      /* key ranges and modes of the join tables */
 };
 #define KTJ_DEVERR_TABLE_FULL 1u
@@ -175,8 +175,6 @@ hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowC
                          hipStream_t st);
 hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, uint32_t* cpu_row, Scalars* sc, hipStream_t st);
 /* the build passes read the columns only (correlation id, kind and has-stream bits of meta) */
-hipError_t build_runtime(uint64_t n, Columns c, uint64_t first_runtime, Table tf, FullCols fc, Table tn, NarrowCols nc,
-                         uint32_t* slot_f, uint32_t* slot_n, Scalars* sc, hipStream_t st);
 hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, uint32_t* slot_f_dev,
                                Scalars* sc, hipStream_t st);
 hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
@@ -265,9 +263,15 @@ hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, uint64_t first
 /* runtime rows: also publishes what device rows take over (first timestamp, stream, grid, size)
  * into the tables, reads the "External id" and counts timestamp-order violations; runs after
  * resolve_external and before link_device_rows */
-hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullCols fc,
-                            NarrowCols nc, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
-                            uint32_t* len, Scalars* sc, hipStream_t st);
+/* the pass over the runtime rows: table updates, payload for the device rows, joined rows and lengths;
+ * resolve_external must have run */
+hipError_t join_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, Table tf, FullCols fc,
+                             Table tn, NarrowCols nc, uint32_t* slot_f, uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
+                             uint32_t* len, Scalars* sc, hipStream_t st);
+/* winners write the payload again and repeated ids are checked; returns at once where no two
+ * runtime rows share a slot */
+hipError_t republish_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, FullCols fc, NarrowCols nc,
+                                  const uint32_t* slot_f, const uint32_t* slot_n, Scalars* sc, hipStream_t st);
 hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const DevLink* link,
                            EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st);
 hipError_t gather_len(const uint32_t* perm, const uint32_t* len, uint64_t n, uint32_t* len_sorted, uint8_t* kind_sorted,

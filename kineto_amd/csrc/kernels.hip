@@ -159,7 +159,7 @@ __global__ void k_init_scalars(Scalars* s) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     s->ts_min_biased = ~0ULL; s->ts_max_biased = 0;
     s->out_of_range = 0; s->out_of_order = 0; s->n_flow = 0; s->n_linked = 0; s->n_blank_names = 0; s->n_valid = 0;
-    s->n_unresolved = 0; s->n_sync_typed = 0; s->error = 0; s->have_stream_src = 0; s->n_dev_ranks = 0; s->n_res_ranks = 0; s->n_dense = 0; s->pad = 0;
+    s->n_unresolved = 0; s->n_sync_typed = 0; s->error = 0; s->have_stream_src = 0; s->n_dev_ranks = 0; s->n_res_ranks = 0; s->n_dense = 0; s->runtime_ids_repeat = 0;
     for (int k = 0; k < 3; ++k) {
       s->plan.range[k].lo = ~0ULL; s->plan.range[k].hi = 0;
       s->plan.ctl[k].base = 0; s->plan.ctl[k].span = 0; s->plan.ctl[k].direct = 0; s->plan.ctl[k].pad = 0;
@@ -621,45 +621,6 @@ __global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu,
   if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
   if (cpu_row) atomicMax(&cpu_row[slot], (uint32_t)i + 1u);
 }
-/* full table : correlation id → stream_src = last runtime row that carries a stream
- *              (RocmStreamQueue.h:47-54), first = first arrival index seen, for checkTimestampOrder
- *              (GenericActivityProfiler.cpp:363-395)
- * narrow table: int-narrowed id → kern_src = last in-range kernel row, copy_src = last in-range
- *              copy/malloc row (thread_local correlationToGrid/Block/Size,
- *              RocprofActivity_inl.h:28-30, 221-223, 245, 267)
- * The slots are remembered per row (slot_f, slot_n) for the second pass over the runtime rows;
- * slot_n also serves the "External id" lookup, so rows that insert nothing look their key up. */
-__global__ void k_build_runtime(uint64_t n, Columns c, uint64_t first_runtime, Table tf, FullCols fc, Table tn,
-                                NarrowCols nc, uint32_t* slot_f, uint32_t* slot_n, Scalars* sc) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  /* one store per workgroup at most: every lane storing the same flag would queue up in L2 */
-  const bool carries_stream = i < n && (c.meta[first_runtime + i] & KTJ_M_HAS_STREAM);
-  if (__syncthreads_or(carries_stream ? 1 : 0) && threadIdx.x == 0) sc->have_stream_src = 1;
-  if (i >= n) return;
-  const uint64_t a = first_runtime + i;
-  const uint64_t id = c.corr[a];
-  const uint32_t meta = c.meta[a];
-  const uint32_t kind = (meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
-  const uint32_t sf = slot_insert(tf, id);
-  slot_f[i] = sf;
-  if (sf == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
-  else {
-    if (fc.first[sf] > (uint32_t)a) atomicMin(&fc.first[sf], (uint32_t)a);
-    if (meta & KTJ_M_HAS_STREAM) atomicMax(&fc.stream_src[sf], (uint32_t)i + 1u);
-  }
-  const bool publishes = (meta & KTJ_M_VALID) && kind != KTJ_RT_DEFAULT;
-  uint32_t sn;
-  if (publishes) {
-    sn = slot_insert(tn, narrow_corr_key(id));
-    if (sn == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
-    else if (kind == KTJ_RT_KERNEL) atomicMax(&nc.kern_src[sn], (uint32_t)i + 1u);
-    else atomicMax(&nc.copy_src[sn], (uint32_t)i + 1u);
-  } else {
-    /* every slot that carries an external id exists already (k_build_extcorr ran before) */
-    sn = slot_find(tn, narrow_corr_key(id));
-  }
-  slot_n[i] = sn;
-}
 /* Device rows take part in "first seen" only when they are inside the window; every device row
  * remembers its slot (rows outside the window still take a stream from it). */
 __global__ void k_insert_device_first(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc,
@@ -764,13 +725,6 @@ hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowC
 hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, uint32_t* cpu_row, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
   hipLaunchKernelGGL(k_build_cpu_ids, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, cpu, cpu_row, sc);
-  return KTJ_LAUNCH_CHECK();
-}
-hipError_t build_runtime(uint64_t n, Columns c, uint64_t first_runtime, Table tf, FullCols fc, Table tn, NarrowCols nc,
-                         uint32_t* slot_f, uint32_t* slot_n, Scalars* sc, hipStream_t st) {
-  if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_build_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_runtime, tf, fc, tn,
-                     nc, slot_f, slot_n, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, uint32_t* slot_f_dev,
@@ -1432,43 +1386,80 @@ __global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, uint64_t fir
   }
   flush_row_stats(rs, sc);
 }
-/* Second pass over the runtime rows.  The row that won a slot field publishes what device rows
- * take over (timestamp of the first row, stream, grid/block, size); every row reads its
- * "External id" from the narrow slot and is checked against the first row of its id. */
-__global__ void k_mat_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullCols fc,
-                              NarrowCols nc, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
-                              uint32_t* len, Scalars* sc) {
+/* The pass over the runtime rows.
+ * full table : correlation id → stream_src = last runtime row that carries a stream
+ *              (RocmStreamQueue.h:47-54), first = first arrival index seen, for checkTimestampOrder
+ *              (GenericActivityProfiler.cpp:363-395)
+ * narrow table: int-narrowed id → kern_src = last in-window kernel row, copy_src = last in-window
+ *              copy/malloc row (thread_local correlationToGrid/Block/Size,
+ *              RocprofActivity_inl.h:28-30, 221-223, 245, 267)
+ * Every row also writes what device rows take over from it (timestamp, stream, grid/block or
+ * size) into the payload of its slots straight away.  That is final when no two runtime rows
+ * share a slot, which the returning atomicMin on `first` tells; otherwise k_republish_runtime
+ * lets the winners write again.  The "External id" was resolved before this pass, so the joined
+ * row and its length are produced here too.  The slots are remembered per row for the republish
+ * pass. */
+__device__ __forceinline__ bool runtime_rows_share_slots(const Scalars* sc) {
+  /* ids beyond 31 bits may coincide after narrowing without sharing a slot of the full table */
+  const KeyRange r = sc->plan.range[KTJ_TBL_FULL];
+  return sc->runtime_ids_repeat != 0 || (r.lo <= r.hi && r.hi >= 0x80000000ULL);
+}
+__global__ void k_join_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, ApiTable api, Table tf,
+                               FullCols fc, Table tn, NarrowCols nc, uint32_t* slot_f, uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
+                               uint32_t* len, Scalars* sc) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   RowStats rs;
-  uint32_t n_linked = 0, n_bad = 0;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    const uint64_t a = first + i;
+  uint32_t n_linked = 0;
+  bool carries_stream = false, repeats = false;
+  if (i < n) {
+    const uint64_t a = first_runtime + i;
     const ktj_runtime_rec rec = r[i];
+    const uint64_t id = c.corr[a];
+    const uint32_t meta = c.meta[a];
     const int64_t ts = c.ts[a];
-    const bool valid = (c.meta[a] & KTJ_M_VALID) != 0;
-    const uint32_t sf = slot_f[i], sn = slot_n[i];
-    if (sf != KTJ_NOSLOT) {
-      const uint64_t f = fc.first[sf];
-      if (f == a) fc.pay[sf].first_ts = ts;
-      else if (f != 0xFFFFFFFFull) { /* an earlier runtime row has this id: checkTimestampOrder, swapped */
-        const int64_t t1 = c.ts[f];
-        if (ts != 0 && t1 > ts) ++n_bad;
+    const uint32_t kind = (meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
+    const bool valid = (meta & KTJ_M_VALID) != 0;
+    carries_stream = (meta & KTJ_M_HAS_STREAM) != 0;
+    const uint32_t sf = slot_insert(tf, id);
+    slot_f[i] = sf;
+    if (sf == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+    else {
+      repeats = atomicMin(&fc.first[sf], (uint32_t)a) != 0xFFFFFFFFu;
+      FullPay fp;
+      fp.first_ts = ts;
+      fp.stream = 0;
+      if (carries_stream) {
+        atomicMax(&fc.stream_src[sf], (uint32_t)i + 1u);
+        fp.stream = rec.kind == KTJ_RT_KERNEL ? rec.u.kernel.stream : rec.u.copy.stream;
       }
-      if (fc.stream_src[sf] == (uint32_t)i + 1u)
-        fc.pay[sf].stream = rec.kind == KTJ_RT_KERNEL ? rec.u.kernel.stream : rec.u.copy.stream;
+      fc.pay[sf] = fp;
     }
+    const bool publishes = valid && kind != KTJ_RT_DEFAULT;
+    uint32_t sn;
     int32_t ext = 0;
-    if (sn != KTJ_NOSLOT) {
-      NarrowPay* np = &nc.pay[sn];
-      ext = np->ext_val;
-      if (np->linked && valid) ++n_linked;
-      const uint32_t copy_src = nc.copy_src[sn]; /* final: the build pass has ended */
-      if (copy_src == (uint32_t)i + 1u) {
-        np->pay[0] = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
-        np->kind = KTJ_DL_HAS_SIZE;
-      } else if (copy_src == 0 && nc.kern_src[sn] == (uint32_t)i + 1u) {
-        pack_grid(rec, np->pay);
-        np->kind = KTJ_DL_HAS_GRID;
+    if (publishes) {
+      sn = slot_insert(tn, narrow_corr_key(id));
+      if (sn == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+      else {
+        NarrowPay* np = &nc.pay[sn];
+        if (kind == KTJ_RT_KERNEL) {
+          atomicMax(&nc.kern_src[sn], (uint32_t)i + 1u);
+          pack_grid(rec, np->pay);
+          np->kind = KTJ_DL_HAS_GRID;
+        } else {
+          atomicMax(&nc.copy_src[sn], (uint32_t)i + 1u);
+          np->pay[0] = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
+          np->kind = KTJ_DL_HAS_SIZE;
+        }
       }
+    } else {
+      /* every slot that carries an external id exists already (k_build_extcorr ran before) */
+      sn = slot_find(tn, narrow_corr_key(id));
+    }
+    slot_n[i] = sn;
+    if (sn != KTJ_NOSLOT) {
+      ext = nc.pay[sn].ext_val;
+      if (nc.pay[sn].linked && valid) ++n_linked;
     }
     c.ext[a] = ext;
     const bool known = rec.cid < api.n_cids;
@@ -1479,8 +1470,53 @@ __global__ void k_mat_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, u
     len[a] = row_length(m, ctx, sc);
     count_row_stats(m, ctx, &rs);
   }
+  /* one store per workgroup at most: every lane storing the same flag would queue up in L2 */
+  const int any_stream = __syncthreads_or(carries_stream ? 1 : 0);
+  const int any_repeat = __syncthreads_or(repeats ? 1 : 0);
+  if (threadIdx.x == 0) {
+    if (any_stream) sc->have_stream_src = 1;
+    if (any_repeat) sc->runtime_ids_repeat = 1;
+  }
   flush_row_stats(rs, sc);
   block_add(&sc->n_linked, n_linked);
+}
+/* Only when runtime rows share slots: the row that won a slot field writes the payload again, and
+ * every row is checked against the first row of its id (checkTimestampOrder with the roles
+ * swapped).  Where no two runtime rows share a slot each row is the first of its id and what it
+ * wrote in k_join_runtime stands. */
+__global__ void k_republish_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, FullCols fc, NarrowCols nc,
+                                    const uint32_t* slot_f, const uint32_t* slot_n, Scalars* sc) {
+  if (!runtime_rows_share_slots(sc)) return;
+  uint32_t n_bad = 0;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t a = first + i;
+    const ktj_runtime_rec rec = r[i];
+    const int64_t ts = c.ts[a];
+    const uint32_t sf = slot_f[i], sn = slot_n[i];
+    if (sf != KTJ_NOSLOT) {
+      const uint64_t f = fc.first[sf];
+      if (f == a) fc.pay[sf].first_ts = ts;
+      else if (f != 0xFFFFFFFFull) { /* an earlier runtime row has this id */
+        const int64_t t1 = c.ts[f];
+        if (ts != 0 && t1 > ts) ++n_bad;
+      }
+      const uint32_t stream_src = fc.stream_src[sf];
+      if (stream_src == (uint32_t)i + 1u)
+        fc.pay[sf].stream = rec.kind == KTJ_RT_KERNEL ? rec.u.kernel.stream : rec.u.copy.stream;
+      else if (stream_src == 0) fc.pay[sf].stream = 0; /* no row of this id carries one */
+    }
+    if (sn != KTJ_NOSLOT) {
+      NarrowPay* np = &nc.pay[sn];
+      const uint32_t copy_src = nc.copy_src[sn]; /* final: the pass above has ended */
+      if (copy_src == (uint32_t)i + 1u) {
+        np->pay[0] = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
+        np->kind = KTJ_DL_HAS_SIZE;
+      } else if (copy_src == 0 && nc.kern_src[sn] == (uint32_t)i + 1u) {
+        pack_grid(rec, np->pay);
+        np->kind = KTJ_DL_HAS_GRID;
+      }
+    }
+  }
   block_add(&sc->out_of_order, n_bad);
 }
 __global__ void k_mat_device(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const DevLink* link,
@@ -1538,12 +1574,19 @@ hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, uint64_t first
                      mat, len, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t mat_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, FullCols fc,
-                            NarrowCols nc, const uint32_t* slot_f, const uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
-                            uint32_t* len, Scalars* sc, hipStream_t st) {
+hipError_t join_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, Table tf, FullCols fc,
+                             Table tn, NarrowCols nc, uint32_t* slot_f, uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
+                             uint32_t* len, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_mat_runtime, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, fc, nc,
+  hipLaunchKernelGGL(k_join_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, tf, fc, tn, nc,
                      slot_f, slot_n, ctx, mat, len, sc);
+  return KTJ_LAUNCH_CHECK();
+}
+hipError_t republish_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, FullCols fc, NarrowCols nc,
+                                  const uint32_t* slot_f, const uint32_t* slot_n, Scalars* sc, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_republish_runtime, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, fc, nc,
+                     slot_f, slot_n, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t mat_device_rows(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const DevLink* link,

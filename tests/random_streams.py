@@ -36,7 +36,7 @@ def _f64(rng):
     return v
 
 
-def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False):
+def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False, unique_runtime_ids=False):
     rng = random.Random(seed)
     lo, hi = B + 1000, B + 10**7
     window = (lo, hi) if rng.random() < 0.7 else (B + 3 * 10**6, B + 6 * 10**6)
@@ -111,7 +111,10 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False)
                       rng.choice(pids), rng.choice(tids), id=rng.choice([0, -2, 5, 6, 7, 8, 2**31 - 1, -(2**31)] + ids[:8]),
                       schema=sid, values=values, flow_id=rng.choice([0, 0, 1, 77, 2**32 - 1, 2**40 + 3, -4]), flow_type=rng.choice([0, 1, 2, 3]),
                       flow_start=rng.random() < 0.5, linked=rng.choice([None, None, 5, -9, 2**40 + 1]))
-    for _ in range(n_runtime):
+    # with unique_runtime_ids no two runtime rows share a correlation id (the engine then keeps what
+    # each row wrote for the device rows in its single pass); device rows still repeat ids
+    unique_pool = rng.sample(range(1, max(4 * n_runtime, 64)), n_runtime) if unique_runtime_ids else None
+    for k_rt in range(n_runtime):
         kind = rng.randrange(4)
         s0 = t()
         kw = {}
@@ -124,19 +127,19 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False)
                       stream=rng.choice([0, 0x7000, 0xA000]), copy_kind=rng.choice([0, 1, 2, 3, 4, 0xFFFFFFFF]))
         elif kind == 3:
             kw = dict(ptr=rng.getrandbits(47), size=rng.choice([0, 777, 2**33]))
-        b.add_runtime(rng.choice(ids), s0, s0 + rng.choice([0, 5, 5000, -7]), rng.choice([0, 1, 2, 3, 4, 5, 6, 9, 10**6]),
+        b.add_runtime(unique_pool[k_rt] if unique_pool else rng.choice(ids), s0, s0 + rng.choice([0, 5, 5000, -7]), rng.choice([0, 1, 2, 3, 4, 5, 6, 9, 10**6]),
                       rng.choice([10, 11]), rng.choice([20, 21, 22]), kind=kind, **kw)
     for _ in range(n_device):
         dom = rng.choice([0, 0, 0, 1, 1, 2, 7])
         s0 = t()
-        b.add_device(rng.choice(ids + [100, 101, 0]), s0, s0 + rng.choice([0, 1, 2, 900, 10**5]), domain=dom,
+        b.add_device(rng.choice((unique_pool[:40] if unique_pool else []) + ids + [100, 101, 0]), s0, s0 + rng.choice([0, 1, 2, 900, 10**5]), domain=dom,
                      op=rng.choice([0, 1, 2, 3, 4, 9]), device=rng.choice([0, 0, 1, -1]), name=rng.choice(names + [None]),
                      queue=rng.choice([0, 1, 2, 3, 2**63 + 5]), stream=rng.choice([0, 0, 0, 5, 0x7000]), nbytes=rng.choice([0, 1000, 2**40]))
     for _ in range(rng.randrange(0, 40)):
-        b.add_extcorr(rng.choice(ids + [0xFFFFFFFFFFFFFFFF]), rng.choice([5, 6, 7, 8, 0, 2**31 - 1, 0xFFFFFFFF80000000, 2**40, 12345]))
+        b.add_extcorr(rng.choice((unique_pool[:30] if unique_pool else []) + ids + [0xFFFFFFFFFFFFFFFF]), rng.choice([5, 6, 7, 8, 0, 2**31 - 1, 0xFFFFFFFF80000000, 2**40, 12345]))
     if rng.random() < 0.5:  # user-domain correlation: GPU user-annotation spans
         for _ in range(rng.randrange(1, 40)):
-            b.add_usercorr(rng.choice(ids + [100, 0]), rng.choice([5, 6, 7, 8, 0, 2**31 - 1, 0xFFFFFFFF80000000, 2**40, 12345]))
+            b.add_usercorr(rng.choice((unique_pool[:20] if unique_pool else []) + ids + [100, 0]), rng.choice([5, 6, 7, 8, 0, 2**31 - 1, 0xFFFFFFFF80000000, 2**40, 12345]))
     if rng.random() < 0.5:
         b.add_device_info(0, 5000000, 'GPU "zero"', "GPU 0", B + 10)
         b.add_resource_info(5, 5, 0, 'stream "5"', False, B + 10)

@@ -120,7 +120,7 @@ def test_random_streams_on_gpu(seed):
     with direct-addressed and with hash-mode join tables and both emit kernels."""
     import random_streams
     print(f"random stream seed={seed}", flush=True)
-    sp = random_streams.random_stream(seed, wide_ids=seed % 2 == 1).build()
+    sp = random_streams.random_stream(seed, wide_ids=seed % 2 == 1, unique_runtime_ids=seed % 3 == 2).build()
     _engine_vs_oracle(sp)
     _engine_vs_oracle(sp, hash_join=True, tile_emit=True)
 

@@ -271,7 +271,7 @@ def test_join_on_small_synthetic_streams(cfg, n):
 @pytest.mark.parametrize("seed", range(16))
 def test_join_on_random_streams(seed):
     import random_streams
-    compare(random_streams.random_stream(seed, wide_ids=seed % 2 == 1).build())
+    compare(random_streams.random_stream(seed, wide_ids=seed % 2 == 1, unique_runtime_ids=seed % 3 == 2).build())
 
 
 def test_user_annotation_spans():
