@@ -1707,10 +1707,8 @@ k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n
   for (uint32_t k = pre + body * 16u + threadIdx.x; k < nbytes; k += EMIT_THREADS) g[k] = s[k];
 }
 
-/* Direct variant: one lane per activity, aligned 8-byte stores straight into the document, no
- * LDS.  Lane i owns every word that starts inside its activity, including the one it shares
- * with activity i+1's predecessor bytes... i.e. the first word of an activity is written by that
- * activity's lane together with the (fixed) last bytes of its predecessor.  The document's
+/* Direct variant: one lane per activity, aligned 16-byte stores straight into the document, no
+ * LDS (see BlockWriter for who writes the blocks that two activities share).  The document's
  * prefix and suffix are already in place when this kernel runs; the first and the last activity
  * merge with them. */
 __global__ void __launch_bounds__(KTJ_BLOCK) __attribute__((amdgpu_waves_per_eu(3)))
