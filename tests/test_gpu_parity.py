@@ -240,10 +240,11 @@ def test_device_resident_submission():
     assert got == want
 
 
-@pytest.mark.parametrize("cfg", [3])
-def test_full_size_headline_config_digest(cfg):
-    """The headline configuration at its full size: the engine's document and the CPU checker's
-    must have the same length and the same BLAKE2 digest (hashed in place, chunk by chunk)."""
+@pytest.mark.parametrize("cfg", [3, 2, 4, 5])
+def test_full_size_config_digest(cfg):
+    """Configurations 2 to 5 at their full sizes (1 is at its full size among the cases above): the
+    engine's document and the CPU checker's must have the same length and the same BLAKE2 digest
+    (hashed in place, chunk by chunk)."""
     import hashlib
     import oracle_glue as og
     from kineto_amd.engine import TraceEngine
