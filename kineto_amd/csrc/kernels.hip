@@ -1393,12 +1393,12 @@ __global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, uint64_t fir
  * narrow table: int-narrowed id → kern_src = last in-window kernel row, copy_src = last in-window
  *              copy/malloc row (thread_local correlationToGrid/Block/Size,
  *              RocprofActivity_inl.h:28-30, 221-223, 245, 267)
- * Every row also writes what device rows take over from it (timestamp, stream, grid/block or
- * size) into the payload of its slots straight away.  That is final when no two runtime rows
- * share a slot, which the returning atomicMin on `first` tells; otherwise k_republish_runtime
- * lets the winners write again.  The "External id" was resolved before this pass, so the joined
- * row and its length are produced here too.  The slots are remembered per row for the republish
- * pass. */
+ * Every row writes what device rows take over from it (timestamp, stream, grid/block or size)
+ * into the payload of its slots straight away.  That is final when no two runtime rows share a
+ * slot, which the returning atomicMin on `first` tells; only otherwise k_runtime_winners finds
+ * the winning row of each slot field and k_republish_runtime lets the winners write again.  The
+ * "External id" was resolved before this pass, so the joined row and its length are produced here
+ * too.  The slots are remembered per row for those two passes. */
 __device__ __forceinline__ bool runtime_rows_share_slots(const Scalars* sc) {
   /* ids beyond 31 bits may coincide after narrowing without sharing a slot of the full table */
   const KeyRange r = sc->plan.range[KTJ_TBL_FULL];
@@ -1428,10 +1428,7 @@ __global__ void k_join_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, 
       FullPay fp;
       fp.first_ts = ts;
       fp.stream = 0;
-      if (carries_stream) {
-        atomicMax(&fc.stream_src[sf], (uint32_t)i + 1u);
-        fp.stream = rec.kind == KTJ_RT_KERNEL ? rec.u.kernel.stream : rec.u.copy.stream;
-      }
+      if (carries_stream) fp.stream = rec.kind == KTJ_RT_KERNEL ? rec.u.kernel.stream : rec.u.copy.stream;
       fc.pay[sf] = fp;
     }
     const bool publishes = valid && kind != KTJ_RT_DEFAULT;
@@ -1443,11 +1440,9 @@ __global__ void k_join_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, 
       else {
         NarrowPay* np = &nc.pay[sn];
         if (kind == KTJ_RT_KERNEL) {
-          atomicMax(&nc.kern_src[sn], (uint32_t)i + 1u);
           pack_grid(rec, np->pay);
           np->kind = KTJ_DL_HAS_GRID;
         } else {
-          atomicMax(&nc.copy_src[sn], (uint32_t)i + 1u);
           np->pay[0] = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
           np->kind = KTJ_DL_HAS_SIZE;
         }
@@ -1479,6 +1474,21 @@ __global__ void k_join_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, 
   }
   flush_row_stats(rs, sc);
   block_add(&sc->n_linked, n_linked);
+}
+/* Only when runtime rows share slots: which row of a slot the device rows take each value from
+ * (the last row that carries a stream; the last in-window kernel launch; the last in-window copy
+ * or allocation), by atomicMax over row indices.  k_republish_runtime reads the winners. */
+__global__ void k_runtime_winners(uint64_t n, Columns c, uint64_t first, FullCols fc, NarrowCols nc, const uint32_t* slot_f,
+                                  const uint32_t* slot_n, const Scalars* sc) {
+  if (!runtime_rows_share_slots(sc)) return;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const uint32_t meta = c.meta[first + i];
+    const uint32_t kind = (meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
+    const uint32_t sf = slot_f[i], sn = slot_n[i];
+    if (sf != KTJ_NOSLOT && (meta & KTJ_M_HAS_STREAM)) atomicMax(&fc.stream_src[sf], (uint32_t)i + 1u);
+    if (sn != KTJ_NOSLOT && (meta & KTJ_M_VALID) && kind != KTJ_RT_DEFAULT)
+      atomicMax(kind == KTJ_RT_KERNEL ? &nc.kern_src[sn] : &nc.copy_src[sn], (uint32_t)i + 1u);
+  }
 }
 /* Only when runtime rows share slots: the row that won a slot field writes the payload again, and
  * every row is checked against the first row of its id (checkTimestampOrder with the roles
@@ -1585,6 +1595,8 @@ hipError_t join_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, ui
 hipError_t republish_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, FullCols fc, NarrowCols nc,
                                   const uint32_t* slot_f, const uint32_t* slot_n, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_runtime_winners, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first, fc, nc, slot_f,
+                     slot_n, (const Scalars*)sc);
   hipLaunchKernelGGL(k_republish_runtime, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, fc, nc,
                      slot_f, slot_n, sc);
   return KTJ_LAUNCH_CHECK();
