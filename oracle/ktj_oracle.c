@@ -67,6 +67,7 @@ static void sb_reserve(sbuf* b, size_t extra) {
   b->cap = nc;
 }
 static void sb_put(sbuf* b, const char* s, size_t n) {
+  if (n == 0) return;
   sb_reserve(b, n);
   memcpy(b->p + b->n, s, n);
   b->n += n;
@@ -293,9 +294,10 @@ int64_t ktj_oracle_convert_ts(const ktj_clock_model* m, uint64_t t) {
   int64_t t_approx = (int64_t)t;
   int64_t t0_approx = (int64_t)m->t0_approx;
   long double scale_factor = (long double)m->scale;
-  return t_approx > t0_approx
-      ? (int64_t)((double)(t_approx - t0_approx) * scale_factor) + m->t0
-      : 0;
+  if (!(t_approx > t0_approx)) return 0;
+  /* the sum wraps where the reference's signed addition overflows, as its machine code does */
+  const int64_t scaled = (int64_t)((double)(t_approx - t0_approx) * scale_factor);
+  return (int64_t)((uint64_t)scaled + (uint64_t)m->t0);
 }
 
 /* ------------------------------------------------------------------------------------------ */
