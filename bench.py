@@ -7,6 +7,7 @@ ops, 128 streams), with the raw records already resident in HBM and the JSON doc
 device buffer.  Prints one JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--n-device N] [--config C]
+  python bench.py --logger-benchmark small|medium|large   (the reference's logger benchmark, both loggers)
 """
 import argparse
 import ctypes as C
@@ -67,6 +68,65 @@ def cpu_baseline(config, sample_device_rows):
     }
 
 
+def logger_benchmark(scenario, iterations, threads):
+    """The reference's own logger benchmark (benchmarks/json_output_benchmark.cpp: a fixed-seed stream
+    of GenericTraceActivity objects, timed from logger construction to the end of finalizeTrace,
+    file included) run on the reference's ChromeTraceLogger and on the GpuChromeTraceLogger shim in
+    the same process.  Needs oracle/_ref/libktj_shim_test.so (built where the reference is present).
+    Prints one JSON line; the shim's file is compared byte for byte with the reference's."""
+    import statistics
+    import tempfile
+    so = os.path.join(ROOT, "oracle", "_ref", "libktj_shim_test.so")
+    if not os.path.exists(so):
+        print("bench.py: oracle/_ref/libktj_shim_test.so is not built (it needs the reference's sources)", file=sys.stderr)
+        sys.exit(1)
+    lib = C.CDLL(so)
+    lib.ktj_logger_bench_create.restype = C.c_void_p
+    lib.ktj_logger_bench_create.argtypes = [C.c_uint64, C.c_uint32]
+    lib.ktj_logger_bench_destroy.argtypes = [C.c_void_p]
+    lib.ktj_logger_bench_run.restype = C.c_double
+    lib.ktj_logger_bench_run.argtypes = [C.c_void_p, C.c_int, C.c_char_p, C.c_int, C.c_int]
+    n = {"small": 5, "medium": 6000, "large": 6000000}[scenario]
+    if iterations <= 0:
+        iterations = {"small": 100, "medium": 20, "large": 2}[scenario]
+    w = lib.ktj_logger_bench_create(n, 42)
+    legs = {"reference": 0, "reference_sorted_input": 1, "shim_per_activity": 2, "shim_bulk": 3}
+    out = {}
+    digests = {}
+    with tempfile.TemporaryDirectory() as top:
+        for name, which in legs.items():
+            d = os.path.join(top, name)
+            os.makedirs(d)
+            path = os.path.join(d, "benchmark_%s.json" % scenario)
+            times = []
+            for it in range(iterations + 1):  # the first iteration is a warm-up for every leg
+                ms = lib.ktj_logger_bench_run(w, which, path.encode(), 0, threads)
+                if ms < 0:
+                    print("bench.py: logger benchmark leg %s failed (%g)" % (name, ms), file=sys.stderr)
+                    sys.exit(1)
+                if it:
+                    times.append(ms)
+            size = os.path.getsize(path)
+            with open(path, "rb") as f:
+                data = f.read().replace(path.encode(), b"FILE")
+            import hashlib
+            digests[name] = hashlib.blake2b(data).hexdigest()
+            del data
+            os.remove(path)
+            mean = statistics.mean(times)
+            out[name] = {"mean_ms": mean, "min_ms": min(times), "stddev_ms": statistics.pstdev(times), "file_bytes": size,
+                         "activities_per_s": n / (mean / 1e3), "mib_per_s": size / 1048576.0 / (mean / 1e3)}
+    lib.ktj_logger_bench_destroy(w)
+    print(json.dumps({
+        "metric": "logger_benchmark_activities_per_s", "scenario": scenario, "activities": n, "iterations": iterations,
+        "packing_threads": threads, "legs": out,
+        "shim_identical_to_reference": digests["shim_per_activity"] == digests["reference_sorted_input"]
+        and digests["shim_bulk"] == digests["reference_sorted_input"],
+        "speedup_bulk_vs_reference": out["reference"]["mean_ms"] / out["shim_bulk"]["mean_ms"],
+        "note": "file output included in every leg; the shim writes activities in (device, resource, start) order, "
+                "so its file is compared with the reference logger fed in that order"}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -78,6 +138,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-bytes", type=int, default=1 << 30, help="size of the reference copy kernel run (0 = skip)")
     ap.add_argument("--traffic", type=str, default="", help="JSON file with measured HBM bytes per emit launch (from rocprofv3 --pmc)")
+    ap.add_argument("--logger-benchmark", choices=["small", "medium", "large"], default=None,
+                    help="run the reference's logger benchmark on both loggers instead of the hot-path bench")
+    ap.add_argument("--iterations", type=int, default=0, help="iterations of --logger-benchmark (0 = the reference's defaults)")
+    ap.add_argument("--threads", type=int, default=16, help="packing workers of the shim's bulk leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path runs on exactly one GPU (no sharding, no collectives); use --gpus 1",
@@ -88,6 +152,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+    if args.logger_benchmark:
+        logger_benchmark(args.logger_benchmark, args.iterations, args.threads)
+        return
     from kineto_amd import abi
     from kineto_amd.engine import TraceEngine
 

@@ -359,7 +359,7 @@ enum {
   KTJ_STAGE_SIZE = 5,     /* exact byte length per record                                      */
   KTJ_STAGE_SCAN = 6,     /* device-wide exclusive scan                                        */
   KTJ_STAGE_EMIT = 7,     /* JSON formatting into the output buffer                            */
-  KTJ_STAGE_D2H = 8,      /* device → pinned host copy                                         */
+  KTJ_STAGE_D2H = 8,      /* device → pinned host copy (file sink: time spent waiting for it)  */
   KTJ_STAGE_FILE = 9,     /* write + rename (host)                                             */
   KTJ_STAGE_TOTAL_GPU = 10 /* first kernel start → last kernel end                             */
 };

@@ -148,6 +148,9 @@ struct ktj_engine {
   DevBuf mat, len, len_sorted, kind_sorted, offs, out, tile_start;
   void* pinned_small = nullptr; size_t pinned_small_cap = 0;
   char* pinned_out = nullptr; size_t pinned_out_cap = 0;
+  char* file_stage[2] = {nullptr, nullptr};   /* pinned staging of the file sink, at most KTJ_FILE_STAGE_BYTES each */
+  size_t file_stage_cap[2] = {0, 0};
+  hipEvent_t ev_file_stage[2] = {};
   bool host_copy_valid = false;
 
   /* results */
@@ -325,6 +328,8 @@ void ktj_destroy(ktj_engine* e) {
   /* device buffers free themselves when the engine is deleted below */
   if (e->pinned_small) (void)hipHostFree(e->pinned_small);
   if (e->pinned_out) (void)hipHostFree(e->pinned_out);
+  for (auto& p : e->file_stage) if (p) (void)hipHostFree(p);
+  for (auto& ev : e->ev_file_stage) if (ev) (void)hipEventDestroy(ev);
   for (auto& ev : e->ev) if (ev) (void)hipEventDestroy(ev);
   for (auto& ev : e->ev_d2h) if (ev) (void)hipEventDestroy(ev);
   if (e->stream) (void)hipStreamDestroy(e->stream);
@@ -925,6 +930,56 @@ int ktj_output_host(ktj_engine* e, const char** host_ptr, uint64_t* n_bytes) {
   return KTJ_OK;
 }
 
+/* The file sink streams the document from HBM through two small pinned buffers: the copy of one
+ * chunk runs while the previous one is written.  One pinned buffer for the whole document would
+ * cost more than the copy and the write together: its pages are mapped for the CPU one fault at a
+ * time when write() first reads them (0.9 s for 1.6 GB, against 0.03 s for the copy and 0.15 s for
+ * the write into the page cache). */
+#define KTJ_FILE_STAGE_BYTES (16ull << 20)
+static int stream_document_to_file(ktj_engine* e, int fd, float* copy_wait_ms) {
+  const uint64_t n = e->total_bytes;
+  const uint64_t n_chunks = (n + KTJ_FILE_STAGE_BYTES - 1) / KTJ_FILE_STAGE_BYTES;
+  for (uint64_t k = 0; k < 2 && k < n_chunks; ++k) { /* small documents take one small buffer */
+    const size_t need = (size_t)((std::min<uint64_t>(KTJ_FILE_STAGE_BYTES, n) + 65535) & ~65535ull);
+    if (e->file_stage_cap[k] < need) {
+      if (e->file_stage[k]) HIPCHK(hipHostFree(e->file_stage[k]));
+      e->file_stage[k] = nullptr; e->file_stage_cap[k] = 0;
+      void* p = nullptr;
+      HIPCHK(hipHostMalloc(&p, need, hipHostMallocDefault));
+      e->file_stage[k] = static_cast<char*>(p);
+      e->file_stage_cap[k] = need;
+    }
+    if (!e->ev_file_stage[k]) HIPCHK(hipEventCreateWithFlags(&e->ev_file_stage[k], hipEventDisableTiming));
+  }
+  auto chunk_len = [n](uint64_t c) { return std::min<uint64_t>(KTJ_FILE_STAGE_BYTES, n - c * KTJ_FILE_STAGE_BYTES); };
+  auto start_copy = [e, &chunk_len](uint64_t c) -> hipError_t {
+    hipError_t rc = hipMemcpyAsync(e->file_stage[c & 1], static_cast<const char*>(e->out.p) + c * KTJ_FILE_STAGE_BYTES,
+                                   chunk_len(c), hipMemcpyDeviceToHost, e->stream);
+    return rc != hipSuccess ? rc : hipEventRecord(e->ev_file_stage[c & 1], e->stream);
+  };
+  double waited = 0;
+  if (n_chunks) HIPCHK(start_copy(0));
+  for (uint64_t c = 0; c < n_chunks; ++c) {
+    /* the other buffer is free: its chunk (c - 1) has been written */
+    if (c + 1 < n_chunks) HIPCHK(start_copy(c + 1));
+    struct timespec t0, t1;
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    HIPCHK(hipEventSynchronize(e->ev_file_stage[c & 1]));
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    waited += (t1.tv_sec - t0.tv_sec) * 1e3 + (t1.tv_nsec - t0.tv_nsec) * 1e-6;
+    const char* src = e->file_stage[c & 1];
+    uint64_t left = chunk_len(c);
+    while (left) {
+      const ssize_t w = write(fd, src, left);
+      if (w < 0 && errno == EINTR) continue;
+      if (w <= 0) { (void)hipStreamSynchronize(e->stream); return KTJ_ERR_IO; }
+      src += w; left -= (uint64_t)w;
+    }
+  }
+  if (copy_wait_ms) *copy_wait_ms = (float)waited;
+  return KTJ_OK;
+}
+
 int ktj_finalize(ktj_engine* e, int64_t end_time_ns, uint64_t* bytes_written) {
   if (!e) return KTJ_ERR_ARG;
   if (bytes_written) *bytes_written = 0;
@@ -938,17 +993,19 @@ int ktj_finalize(ktj_engine* e, int64_t end_time_ns, uint64_t* bytes_written) {
     if (bytes_written) *bytes_written = e->total_bytes;
     return KTJ_OK;
   }
-  const char* host = nullptr;
-  uint64_t n = 0;
-  rc = ktj_output_host(e, &host, &n);
-  if (rc != KTJ_OK) return rc;
+  HIPCHK(hipSetDevice(e->device));
+  const uint64_t n = e->total_bytes;
   struct timespec t0, t1;
   clock_gettime(CLOCK_MONOTONIC, &t0);
   if (!e->sink) return KTJ_ERR_STATE;
-  const size_t w = fwrite(host, 1, n, e->sink);
+  float copy_wait_ms = 0;
+  rc = fflush(e->sink) == 0 ? stream_document_to_file(e, fileno(e->sink), &copy_wait_ms) : KTJ_ERR_IO;
   const int crc = fclose(e->sink);
   e->sink = nullptr;
-  if (w != n || crc != 0) { e->last_error = "short write to " + e->tmp_path; return KTJ_ERR_IO; }
+  if (rc == KTJ_ERR_IO || (rc == KTJ_OK && crc != 0)) { e->last_error = "short write to " + e->tmp_path; return KTJ_ERR_IO; }
+  if (rc != KTJ_OK) return rc;
+  e->stats.stage_ms[KTJ_STAGE_D2H] = copy_wait_ms; /* time the writer waited for copies */
+  e->stats.stage_bytes[KTJ_STAGE_D2H] = n;
   remove(e->out_path.c_str()); /* output_json.cpp:1100-1107 */
   if (rename(e->tmp_path.c_str(), e->out_path.c_str()) != 0) {
     e->last_error = "Failed to rename " + e->tmp_path + " to " + e->out_path + ": " + strerror(errno);
