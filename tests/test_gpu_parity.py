@@ -189,6 +189,29 @@ def test_process_is_repeatable_and_file_output(tmp_path):
     release()
 
 
+def test_file_output_of_a_document_of_several_staging_chunks(tmp_path):
+    """The file sink streams the document through pinned staging buffers, one chunk being copied
+    while the previous one is written: a document of several chunks (and a ragged last one) must
+    reach the file byte for byte, and a second trace through the same engine settings too."""
+    import oracle_glue as og
+    from kineto_amd.engine import TraceEngine
+    for n_dev in (60000, 17000):
+        path = str(tmp_path / f"trace_{n_dev}.json")
+        sp, release = abi.synth_stream(3, n_dev, host_name="gpubox", trace_name=path)
+        ora = og.OracleRun(sp)
+        want = ora.output()
+        ora.close()
+        with TraceEngine(path, device=0, no_file=False) as eng:
+            eng.submit_stream(sp)
+            n = eng.finalize()
+        release()
+        assert n == len(want)
+        if n_dev == 60000:
+            assert n > 3 * (16 << 20)
+        with open(path, "rb") as f:
+            assert f.read() == want
+
+
 def test_unwritable_sink_is_a_silent_noop():
     """ChromeTraceLogger with a file it cannot open: every handler returns silently and only
     finalizeTrace reports (output_json.cpp:485-505, 1067-1070)."""
