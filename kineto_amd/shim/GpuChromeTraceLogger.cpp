@@ -56,7 +56,7 @@ struct GpuChromeTraceLogger::Packed {
   std::vector<std::string> names; /* activity and counter names: few distinct ones, kept once */
   std::unordered_map<std::string, uint32_t> nameIndex;
   std::string fragmentBlob;       /* metadataJson() texts: nearly all distinct (sequence numbers, */
-  std::vector<uint64_t> fragmentEnd; /* correlation ids), so they are stored as they come         */
+  std::vector<uint64_t> fragmentOff{0}; /* correlation ids), so they are stored as they come; n + 1 offsets */
   std::vector<std::string> collectives; /* the 17 values of an op, each followed by NUL */
   std::unordered_map<std::string, uint32_t> collectiveIndex;
   std::vector<std::vector<uint32_t>> counterSchemas; /* local ids of the counter names */
@@ -77,12 +77,12 @@ struct GpuChromeTraceLogger::Packed {
   }
   uint32_t fragment(const std::string& s) {
     fragmentBlob.append(s);
-    fragmentEnd.push_back(fragmentBlob.size());
-    return static_cast<uint32_t>(fragmentEnd.size() - 1);
+    fragmentOff.push_back(fragmentBlob.size());
+    return static_cast<uint32_t>(fragmentOff.size() - 2);
   }
   void slot(uint64_t v, uint8_t kind) { slots.push_back(v); slotKind.push_back(kind); }
   void clearRecords() {
-    records.clear(); origin.clear(); slots.clear(); slotKind.clear(); fragmentBlob.clear(); fragmentEnd.clear();
+    records.clear(); origin.clear(); slots.clear(); slotKind.clear(); fragmentBlob.clear(); fragmentOff.assign(1, 0);
   }
 };
 
@@ -223,14 +223,28 @@ void GpuChromeTraceLogger::translate(Packed& p) {
   }
   for (size_t i = p.nameGlobal.size(); i < p.names.size(); ++i) p.nameGlobal.push_back(intern(p.names[i]));
   /* the fragments of this batch get consecutive ids */
-  p.fragmentBase = nextStringId_;
-  if (!p.fragmentEnd.empty()) {
-    const uint64_t at = pendingBlob_.size();
-    pendingBlob_.append(p.fragmentBlob);
-    pendingOffsets_.reserve(pendingOffsets_.size() + p.fragmentEnd.size());
-    for (uint64_t end : p.fragmentEnd) pendingOffsets_.push_back(at + end);
-    nextStringId_ += static_cast<uint32_t>(p.fragmentEnd.size());
-    if (pendingBlob_.size() >= kStringBatchBytes) flushStrings();
+  const size_t nFragments = p.fragmentOff.size() - 1;
+  if (nFragments != 0 && p.fragmentBlob.size() >= kStringBatchBytes) {
+    /* a batch of its own: handed to the engine where it lies, after whatever is pending */
+    flushStrings();
+    p.fragmentBase = nextStringId_;
+    uint32_t first = 0;
+    if (ok()) {
+      note(ktj_intern_strings(engine_, p.fragmentBlob.data(), p.fragmentOff.data(), nFragments, &first), "ktj_intern_strings");
+      if (status_ == 0 && first != p.fragmentBase) note(KTJ_ERR_STATE, "string id bookkeeping");
+    }
+    nextStringId_ += static_cast<uint32_t>(nFragments);
+    pendingFirstId_ = nextStringId_;
+  } else {
+    p.fragmentBase = nextStringId_;
+    if (nFragments != 0) {
+      const uint64_t at = pendingBlob_.size();
+      pendingBlob_.append(p.fragmentBlob);
+      pendingOffsets_.reserve(pendingOffsets_.size() + nFragments);
+      for (size_t i = 1; i <= nFragments; ++i) pendingOffsets_.push_back(at + p.fragmentOff[i]);
+      nextStringId_ += static_cast<uint32_t>(nFragments);
+      if (pendingBlob_.size() >= kStringBatchBytes) flushStrings();
+    }
   }
   for (size_t i = p.collectiveGlobal.size(); i < p.collectives.size(); ++i) {
     const std::string& key = p.collectives[i];
@@ -310,13 +324,19 @@ void GpuChromeTraceLogger::flushStrings() {
 }
 
 void GpuChromeTraceLogger::flushRecords() {
-  if (records_.empty() || !ok()) return;
-  uint64_t first = 0;
-  note(ktj_submit_args(engine_, slots_.data(), slots_.size(), &first), "ktj_submit_args");
-  if (status_ == 0 && first + slots_.size() != nextSlot_) note(KTJ_ERR_STATE, "args slot bookkeeping");
-  note(ktj_submit_records(engine_, KTJ_REC_GENERIC, records_.data(), records_.size()), "ktj_submit_records");
+  submitRecords(records_.data(), records_.size());
   records_.clear();
-  slots_.clear();
+}
+
+/* the pending args slots, then the records that refer to them */
+void GpuChromeTraceLogger::submitRecords(const ktj_generic_rec* records, size_t count) {
+  if (count != 0 && ok()) {
+    uint64_t first = 0;
+    note(ktj_submit_args(engine_, slots_.data(), slots_.size(), &first), "ktj_submit_args");
+    if (status_ == 0 && first + slots_.size() != nextSlot_) note(KTJ_ERR_STATE, "args slot bookkeeping");
+    note(ktj_submit_records(engine_, KTJ_REC_GENERIC, records, count), "ktj_submit_records");
+  }
+  slots_.clear(); /* slots only ever come with records */
 }
 
 void GpuChromeTraceLogger::handleTraceStart(const std::unordered_map<std::string, std::string>& metadata,
@@ -380,38 +400,67 @@ void GpuChromeTraceLogger::handleActivities(const std::vector<const ITraceActivi
   const size_t n = activities.size();
   if (threads == 0) threads = std::max(1u, std::thread::hardware_concurrency());
   threads = static_cast<unsigned>(std::min<size_t>(threads, (n + 4095) / 4096));
-  std::vector<uint8_t> generic(n);
-  for (size_t i = 0; i < n; ++i) generic[i] = dynamic_cast<const GenericTraceActivity*>(activities[i]) != nullptr;
   std::vector<Packed> parts(threads + 1); /* parts[threads]: the calling thread's, everything that is not generic */
-  auto work = [&](unsigned w) {
-    const size_t lo = n * w / threads, hi = n * (w + 1) / threads;
-    for (size_t i = lo; i < hi; ++i)
-      if (generic[i]) pack(*activities[i], i, parts[w]);
+  auto run = [threads](auto&& job) { /* job(w) for every w < threads, w = 0 on the calling thread */
+    std::vector<std::thread> pool;
+    for (unsigned w = 1; w < threads; ++w) pool.emplace_back(job, w);
+    job(0u);
+    for (auto& t : pool) t.join();
   };
-  std::vector<std::thread> pool;
-  for (unsigned w = 1; w < threads; ++w) pool.emplace_back(work, w);
-  for (size_t i = 0; i < n; ++i)
-    if (!generic[i]) pack(*activities[i], i, parts[threads]);
-  work(0);
-  for (auto& t : pool) t.join();
+  auto is_generic = [](const ITraceActivity* a) { return dynamic_cast<const GenericTraceActivity*>(a) != nullptr; };
+  {
+    std::vector<std::thread> pool;
+    for (unsigned w = 0; w < threads; ++w)
+      pool.emplace_back([&, w] {
+        const size_t lo = n * w / threads, hi = n * (w + 1) / threads;
+        for (size_t i = lo; i < hi; ++i)
+          if (is_generic(activities[i])) pack(*activities[i], i, parts[w]);
+      });
+    for (size_t i = 0; i < n; ++i) /* meanwhile, here and in order: everything else */
+      if (!is_generic(activities[i])) pack(*activities[i], i, parts[threads]);
+    for (auto& t : pool) t.join();
+  }
 
-  /* merge: which packer holds position i, and where */
-  constexpr uint32_t kNobody = 0xFFFFFFFFu;
-  std::vector<uint32_t> owner(n, kNobody), at(n, 0);
+  /* merge.  In sequence: the local dictionaries become engine ids and every part learns where its
+   * slots go.  Then, part by part on the workers: slots and records move to their final places
+   * (a record's place is its activity's position; activities that were dropped leave holes). */
   std::vector<uint64_t> base(parts.size());
+  size_t nRecords = 0, nSlots = 0;
   for (size_t w = 0; w < parts.size(); ++w) {
     translate(parts[w]);
-    base[w] = appendSlots(parts[w]);
-    for (size_t j = 0; j < parts[w].records.size(); ++j) {
-      owner[parts[w].origin[j]] = static_cast<uint32_t>(w);
-      at[parts[w].origin[j]] = static_cast<uint32_t>(j);
-    }
+    base[w] = nextSlot_ + nSlots;
+    nSlots += parts[w].slots.size();
+    nRecords += parts[w].records.size();
   }
-  records_.reserve(n);
-  for (size_t i = 0; i < n; ++i)
-    if (owner[i] != kNobody) records_.push_back(translated(parts[owner[i]], at[i], base[owner[i]]));
+  const size_t slot0 = slots_.size();
+  slots_.resize(slot0 + nSlots);
+  std::unique_ptr<ktj_generic_rec[]> placed(new ktj_generic_rec[n]); /* not zero-filled: every kept place is written */
+  std::vector<uint8_t> present(nRecords == n ? 0 : n, 0);
+  const unsigned nParts = static_cast<unsigned>(parts.size());
+  const uint64_t firstSlot = nextSlot_;
+  run([&](unsigned w0) {
+    for (unsigned w = w0; w < nParts; w += threads) {
+      const Packed& p = parts[w];
+      uint64_t* out = slots_.data() + slot0 + (base[w] - firstSlot);
+      for (size_t i = 0; i < p.slots.size(); ++i) {
+        const uint64_t v = p.slots[i];
+        out[i] = p.slotKind[i] == kSlotFragment ? p.fragmentBase + v : p.slotKind[i] == kSlotCollective ? p.collectiveGlobal[v] : v;
+      }
+      for (size_t j = 0; j < p.records.size(); ++j) {
+        placed[p.origin[j]] = translated(p, j, base[w]);
+        if (!present.empty()) present[p.origin[j]] = 1;
+      }
+    }
+  });
+  nextSlot_ += nSlots;
+  size_t kept = n;
+  if (!present.empty()) { /* close the holes */
+    kept = 0;
+    for (size_t i = 0; i < n; ++i)
+      if (present[i]) placed[kept++] = placed[i];
+  }
   flushStrings();
-  flushRecords();
+  submitRecords(placed.get(), kept); /* records_ is empty here: mergeInOrder above flushed it */
 }
 
 void GpuChromeTraceLogger::handleGenericActivity(const GenericTraceActivity& op) {

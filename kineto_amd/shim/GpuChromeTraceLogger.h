@@ -72,6 +72,7 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
   uint64_t appendSlots(const Packed& p);
   ktj_generic_rec translated(const Packed& p, size_t i, uint64_t slotBase) const;
   void mergeInOrder(Packed& p);
+  void submitRecords(const ktj_generic_rec* records, size_t count);
   void flushStrings();
   void flushRecords();
   bool ok() const { return engine_ != nullptr && status_ == 0; }

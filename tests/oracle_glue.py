@@ -104,7 +104,7 @@ def load_shim():
         lib.ktj_shim_base_time.restype = C.c_int64
         lib.ktj_shim_render.restype = C.c_int
         lib.ktj_shim_render.argtypes = [C.POINTER(abi.Stream), C.POINTER(MatActivity), C.c_uint64,
-                                        C.c_void_p, C.c_void_p, C.c_char_p, C.c_int, C.POINTER(C.c_uint64), C.c_int]
+                                        C.c_void_p, C.c_void_p, C.c_char_p, C.c_int, C.POINTER(C.c_uint64), C.c_int, C.c_int]
         _shim = lib
     return _shim
 
@@ -164,11 +164,18 @@ class OracleRun:
             self.h = None
 
 
-def ref_render(stream_ptr, oracle_run):
+def ref_render(stream_ptr, oracle_run, skip_arrival_mod=0):
     """Renders the stream with the reference's own ChromeTraceLogger, fed with the activities the
-    oracle's join stage produced (arrival order; the driver sorts them itself)."""
+    oracle's join stage produced (arrival order; the driver sorts them itself).  skip_arrival_mod >
+    0 leaves out every activity whose arrival index is 1 modulo it."""
     ref = load_ref()
     acts, n = oracle_run.activities()
+    if skip_arrival_mod > 0:
+        keep = [i for i in range(n) if acts[i].arrival % skip_arrival_mod != 1]
+        kept = (MatActivity * max(len(keep), 1))()
+        for j, i in enumerate(keep):
+            C.memmove(C.byref(kept, j * C.sizeof(MatActivity)), C.byref(acts[i]), C.sizeof(MatActivity))
+        acts, n = kept, len(keep)
     fn = C.cast(load_oracle().ktj_oracle_string, C.c_void_p)
     with tempfile.TemporaryDirectory() as d:
         path = os.path.join(d, stream_ptr.contents.trace_name.decode())
@@ -181,10 +188,12 @@ def ref_render(stream_ptr, oracle_run):
     return data.replace(path.encode(), stream_ptr.contents.trace_name)
 
 
-def shim_render(stream_ptr, oracle_run, protocol="gpujson", directory=None, bulk_threads=0):
+def shim_render(stream_ptr, oracle_run, protocol="gpujson", directory=None, bulk_threads=0, huge_device_mod=0):
     """Renders the stream through the GpuChromeTraceLogger shim obtained from a logger factory by
     URL, fed with the same activities as ref_render, one handleActivity() call each or, with
-    bulk_threads > 0, in one handleActivities() call.  Returns (status, bytes or None, dropped)."""
+    bulk_threads > 0, in one handleActivities() call.  huge_device_mod > 0: every activity whose
+    arrival index is 1 modulo it reports a deviceId beyond 32 bits (the shim drops those).
+    Returns (status, bytes or None, dropped)."""
     shim = load_shim()
     acts, n = oracle_run.activities()
     fn = C.cast(load_oracle().ktj_oracle_string, C.c_void_p)
@@ -192,7 +201,7 @@ def shim_render(stream_ptr, oracle_run, protocol="gpujson", directory=None, bulk
     with tempfile.TemporaryDirectory() as d:
         path = os.path.join(directory or d, stream_ptr.contents.trace_name.decode())
         url = f"{protocol}://{path}"
-        rc = shim.ktj_shim_render(stream_ptr, acts, n, fn, oracle_run.h, url.encode(), 0, C.byref(dropped), bulk_threads)
+        rc = shim.ktj_shim_render(stream_ptr, acts, n, fn, oracle_run.h, url.encode(), 0, C.byref(dropped), bulk_threads, huge_device_mod)
         data = None
         if rc == 0:
             with open(path, "rb") as f:
