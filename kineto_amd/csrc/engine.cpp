@@ -141,7 +141,7 @@ struct ktj_engine {
   /* working buffers */
   DevBuf d_scalars, d_name_len, d_arg_len, d_sflags, d_name_off, d_arg_off, d_name_blob, d_arg_blob;
   DevBuf c_ts, c_dur, c_corr, c_dev, c_res, c_meta, c_ext;
-  DevBuf t_full, t_narrow, t_cpu, f_first, f_stream_src, f_pay, n_ext_src, n_kern_src, n_copy_src, n_pay, slot_ext, slot_f, slot_n, slot_f_dev, dev_link, dev_brief, sync_keys, sync_pos, sync_first;
+  DevBuf t_full, t_narrow, t_cpu, f_has_runtime, f_first, f_stream_src, f_pay, n_ext_src, n_kern_src, n_copy_src, n_pay, slot_ext, slot_f, slot_n, dev_link, dev_brief, sync_keys, sync_pos, sync_first;
   DevBuf q_keys, q_stream, q_amb, dn_hash, dn_first, dn_dev, dn_key, dn_rank;
   DevBuf s_dev_k, s_dev_r, s_res_k, s_res_r;
   DevBuf keys_a, keys_b, vals_a, vals_b, hist, scan_tmp;
@@ -601,10 +601,11 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(e->t_cpu.ensure((cap_cpu + 1ull) * 8));
   HIPCHK(e->f_first.ensure((cap_full + 1ull) * 4)); HIPCHK(e->f_stream_src.ensure((cap_full + 1ull) * 4));
   HIPCHK(e->f_pay.ensure((cap_full + 1ull) * sizeof(FullPay)));
+  HIPCHK(e->f_has_runtime.ensure((cap_full / 32 + 2ull) * 4));
   HIPCHK(e->n_ext_src.ensure((cap_narrow + 1ull) * 4)); HIPCHK(e->n_kern_src.ensure((cap_narrow + 1ull) * 4));
   HIPCHK(e->n_copy_src.ensure((cap_narrow + 1ull) * 4)); HIPCHK(e->n_pay.ensure((cap_narrow + 1ull) * sizeof(NarrowPay)));
   HIPCHK(e->slot_ext.ensure(nx * 4 + 16)); HIPCHK(e->slot_f.ensure(nr * 4 + 16)); HIPCHK(e->slot_n.ensure(nr * 4 + 16));
-  HIPCHK(e->slot_f_dev.ensure(nd * 4 + 16)); HIPCHK(e->dev_link.ensure(nd * sizeof(DevLink) + 16));
+  HIPCHK(e->dev_link.ensure(nd * sizeof(DevLink) + 16));
   HIPCHK(e->dev_brief.ensure(nd * sizeof(DevBrief) + 16));
   HIPCHK(e->q_keys.ensure((KTJ_QUEUE_CAP + 1ull) * 8)); HIPCHK(e->q_stream.ensure((KTJ_QUEUE_CAP + 1ull) * 8));
   HIPCHK(e->q_amb.ensure((KTJ_QUEUE_CAP + 1ull) * 4));
@@ -698,7 +699,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   Table tf{e->t_full.as<uint64_t>(), cap_full - 1, 0u, &sc->plan.ctl[KTJ_TBL_FULL]};
   Table tn{e->t_narrow.as<uint64_t>(), cap_narrow - 1, 0u, &sc->plan.ctl[KTJ_TBL_NARROW]};
   Table t_cpu{e->t_cpu.as<uint64_t>(), cap_cpu - 1, 1u, &sc->plan.ctl[KTJ_TBL_CPU]};
-  FullCols fc{e->f_first.as<uint32_t>(), e->f_stream_src.as<uint32_t>(), e->f_pay.as<FullPay>()};
+  FullCols fc{e->f_has_runtime.as<uint32_t>(), e->f_first.as<uint32_t>(), e->f_stream_src.as<uint32_t>(), e->f_pay.as<FullPay>()};
   NarrowCols nc{e->n_ext_src.as<uint32_t>(), e->n_kern_src.as<uint32_t>(), e->n_copy_src.as<uint32_t>(), e->n_pay.as<NarrowPay>()};
   HIPCHK(plan_tables(c, ng, nr, nd, x_recs, nx, cap_full, cap_narrow, cap_cpu, (e->flags & KTJ_CREATE_HASH_JOIN) != 0, sc, st));
   HIPCHK(clear_tables(tf, fc, tn, nc, t_cpu, st));
@@ -715,9 +716,8 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(resolve_external(x_recs, nx, nc, e->slot_ext.as<uint32_t>(), t_cpu, cpu_row, g_recs, ctx, st));
   HIPCHK(join_runtime_rows(r_recs, nr, c, ng, api, tf, fc, tn, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), ctx, mat,
                            e->len.as<uint32_t>(), sc, st));
-  HIPCHK(insert_device_first(nd, c, ng + nr, tf, fc, e->slot_f_dev.as<uint32_t>(), sc, st));
   HIPCHK(republish_runtime_rows(r_recs, nr, c, ng, fc, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), sc, st));
-  HIPCHK(link_device_rows(nd, c, ng + nr, fc, tn, nc, e->slot_f_dev.as<uint32_t>(), e->dev_link.as<DevLink>(), sc, st));
+  HIPCHK(link_device_rows(nd, c, ng + nr, tf, fc, tn, nc, e->dev_link.as<DevLink>(), sc, st));
   HIPCHK(backfill_streams(e->dev_brief.as<DevBrief>(), nd, c, ng + nr, stt, sc, st));
   if (max_spans) {
     const int rc = synthesise_user_spans(e, c, ctx, t_cpu, cpu_row, sc, N);

@@ -44,11 +44,17 @@ struct Table {
 };
 /* per slot of the table keyed by the full correlation id */
 struct FullPay {           /* published by the winning runtime row, read by device rows */
-  int64_t first_ts;        /* timestamp of row first[slot] when that is a runtime row          */
+  int64_t first_ts;        /* timestamp of the first runtime row with this id                   */
   uint64_t stream;         /* stream of row stream_src[slot]; 0 = no row carries one            */
 };                         /* 16 bytes */
 struct FullCols {
-  uint32_t* first;         /* smallest arrival index seen with this id, 0xFFFFFFFF = none (atomicMin) */
+  uint32_t* has_runtime;   /* one bit per slot: some runtime row has this id.  Runtime rows arrive
+                              before device rows, so where the bit is set the first row of the id is
+                              a runtime row and its timestamp is in the payload; the bitmap is small
+                              enough to stay in cache, unlike the array of first rows              */
+  uint32_t* first;         /* smallest arrival index seen with this id, 0xFFFFFFFF = none (atomicMin);
+                              filled for runtime rows only where they share ids, and for device rows
+                              whose id no runtime row has                                          */
   uint32_t* stream_src;    /* last runtime row (index + 1) that carries a stream (atomicMax)    */
   FullPay* pay;
 };
@@ -89,6 +95,7 @@ struct DevBrief {
 };                         /* 16 bytes */
 #define KTJ_DL_HAS_SIZE 1u
 #define KTJ_DL_HAS_GRID 2u
+#define KTJ_DL_ORPHAN 4u   /* no runtime row has the id: the order check runs in a pass of its own */
 
 /* columns in arrival order: generic rows, then runtime rows, then device rows */
 struct Columns {
@@ -113,6 +120,7 @@ struct Scalars {
   unsigned long long n_valid;
   unsigned long long n_unresolved;    /* device rows still without a stream after the correlation pass */
   unsigned long long n_sync_typed;    /* generic rows of type CUDA_SYNC */
+  unsigned long long n_device_orphans; /* in-window device rows whose id no runtime row has */
   unsigned int error;                 /* KTJ_DEVERR_* bits */
   unsigned int have_stream_src;       /* some runtime row carries a stream */
   unsigned int n_dev_ranks;           /* distinct deviceId values */
@@ -175,16 +183,14 @@ hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowC
                          hipStream_t st);
 hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, uint32_t* cpu_row, Scalars* sc, hipStream_t st);
 /* the build passes read the columns only (correlation id, kind and has-stream bits of meta) */
-hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, uint32_t* slot_f_dev,
-                               Scalars* sc, hipStream_t st);
 hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
                             const uint32_t* cpu_row, const ktj_generic_rec* g, EmitCtx ctx, hipStream_t st);
 hipError_t collective_first(const MatRow* mat, const uint32_t* perm, uint64_t n_rows, uint32_t n_coll, uint32_t* first,
                             hipStream_t st);
 /* per device row: "External id", timestamp-order check, stream of the launching row, and the
  * size / grid hand-over (into link[]) */
-hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, FullCols fc, Table tn, NarrowCols nc,
-                            const uint32_t* slot_f_dev, DevLink* link, Scalars* sc, hipStream_t st);
+hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, Table tn, NarrowCols nc,
+                            DevLink* link, Scalars* sc, hipStream_t st);
 /* stream back-fill: queue table (keys/vals/ambiguous) and dense table are caller-provided, zeroed */
 struct StreamTables {
   uint64_t* q_keys;   /* KTJ_QUEUE_CAP + 1, filled with KTJ_EMPTY_KEY */

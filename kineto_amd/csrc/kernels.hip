@@ -563,6 +563,10 @@ __global__ void k_clear_full(Table t, FullCols c) {
     const uint64_t k = i < n ? i : t.mask + 1ull; /* the last iteration clears the reserved slot */
     c.first[k] = 0xFFFFFFFFu; c.stream_src[k] = 0; c.pay[k] = z;
   }
+  /* the bitmap: whole words up to the extent, and the word of the reserved slot */
+  const uint64_t words = (n + 31) / 32;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i <= words; i += (uint64_t)gridDim.x * blockDim.x)
+    c.has_runtime[i < words ? i : (t.mask + 1ull) / 32] = 0;
 }
 __global__ void k_clear_narrow(Table t, NarrowCols c) {
   const uint64_t n = table_extent(t);
@@ -621,25 +625,6 @@ __global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu,
   if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
   if (cpu_row) atomicMax(&cpu_row[slot], (uint32_t)i + 1u);
 }
-/* Device rows take part in "first seen" only when they are inside the window; every device row
- * remembers its slot (rows outside the window still take a stream from it). */
-__global__ void k_insert_device_first(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc,
-                                      uint32_t* slot_f_dev, Scalars* sc) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const uint64_t a = first_device + i;
-  const uint64_t id = c.corr[a];
-  uint32_t slot;
-  if (c.meta[a] & KTJ_M_VALID) {
-    slot = slot_insert(tf, id);
-    if (slot == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
-    else if (fc.first[slot] > (uint32_t)a) atomicMin(&fc.first[slot], (uint32_t)a);
-  } else {
-    /* slots with a stream come from runtime rows and exist already */
-    slot = slot_find(tf, id);
-  }
-  slot_f_dev[i] = slot;
-}
 /* linkedActivity(): GenericActivityProfiler.cpp:397-408.  The record that won the slot resolves
  * its external id against the CPU-op ids once, for every row that will read the slot. */
 __global__ void k_resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
@@ -665,10 +650,15 @@ __device__ __forceinline__ bool is_async_op(uint32_t domain) { return domain != 
  *  - "External id" (output_json.cpp:871-874) from the narrow slot,
  *  - checkTimestampOrder (GenericActivityProfiler.cpp:363-395) against the first row of the id,
  *  - the stream of the correlation-matched runtime row (RocmStreamQueue.h:56-75, first pass),
- *  - the size or grid/block the launching row hands over (RocprofActivity_inl.h:161-180). */
-__global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, FullCols fc, Table tn, NarrowCols nc,
-                              const uint32_t* slot_f_dev, DevLink* link, Scalars* sc) {
-  uint32_t n_linked = 0, n_bad = 0, n_unresolved = 0;
+ *  - the size or grid/block the launching row hands over (RocprofActivity_inl.h:161-180).
+ * The first row of an id is its first runtime row wherever one exists (runtime rows arrive before
+ * device rows), which a bitmap tells, and the slot's payload holds that row's timestamp, so the
+ * array of first rows is only touched for ids that no runtime row has: in-window device rows take part in "first seen" there and are
+ * checked afterwards by k_device_orphans.  Rows outside the window still take a stream from the
+ * slot (slots with a stream come from runtime rows and exist already). */
+__global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, Table tn, NarrowCols nc,
+                              DevLink* link, Scalars* sc) {
+  uint32_t n_linked = 0, n_bad = 0, n_unresolved = 0, n_orphans = 0;
   const bool have_stream_src = sc->have_stream_src != 0;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t a = first_device + i;
@@ -691,29 +681,52 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Full
       l.coll = np.coll;
     }
     c.ext[a] = ext;
-    link[i] = l;
     int64_t res = c.res[a];
-    const uint32_t sf = slot_f_dev[i];
+    uint32_t sf;
+    if (valid) {
+      sf = slot_insert(tf, id);
+      if (sf == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+    } else sf = slot_find(tf, id);
     if (sf != KTJ_NOSLOT) {
       const FullPay fp = fc.pay[sf];
       if (valid) {
-        const uint64_t f = fc.first[sf];
-        if (f != a && f != 0xFFFFFFFFull) {
-          /* act1 = this row, act2 = first row; swapped when the first one is a runtime row */
-          const bool first_is_runtime = f < first_device;
-          const int64_t tf_ts = first_is_runtime ? fp.first_ts : c.ts[f];
-          const int64_t t1 = first_is_runtime ? tf_ts : c.ts[a];
-          const int64_t t2 = first_is_runtime ? c.ts[a] : tf_ts;
+        if ((fc.has_runtime[sf >> 5] >> (sf & 31u)) & 1u) { /* act1 = the first runtime row, act2 = this row */
+          const int64_t t1 = fp.first_ts, t2 = c.ts[a];
           if (t2 != 0 && t1 > t2) ++n_bad;
+        } else {
+          if (fc.first[sf] > (uint32_t)a) atomicMin(&fc.first[sf], (uint32_t)a);
+          l.flags |= KTJ_DL_ORPHAN;
+          ++n_orphans;
         }
       }
       if (have_stream_src && is_async_op(domain) && res == 0 && fp.stream != 0) { res = (int64_t)fp.stream; c.res[a] = res; }
     }
+    link[i] = l;
     if (is_async_op(domain) && res == 0) ++n_unresolved;
   }
   block_add(&sc->n_linked, n_linked);
   block_add(&sc->out_of_order, n_bad);
   block_add(&sc->n_unresolved, n_unresolved);
+  block_add(&sc->n_device_orphans, n_orphans);
+}
+/* Only when some in-window device row has an id that no runtime row has: such a row is checked
+ * against the first device row of its id (act1 = this row, act2 = the first one). */
+__global__ void k_device_orphans(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, const DevLink* link,
+                                 Scalars* sc) {
+  if (sc->n_device_orphans == 0) return;
+  uint32_t n_bad = 0;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    if (!(link[i].flags & KTJ_DL_ORPHAN)) continue;
+    const uint64_t a = first_device + i;
+    const uint32_t sf = slot_find(tf, c.corr[a]);
+    if (sf == KTJ_NOSLOT) continue;
+    const uint64_t f = fc.first[sf];
+    if (f != a && f != 0xFFFFFFFFull) {
+      const int64_t t1 = c.ts[a], t2 = c.ts[f];
+      if (t2 != 0 && t1 > t2) ++n_bad;
+    }
+  }
+  block_add(&sc->out_of_order, n_bad);
 }
 
 hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, uint32_t* slot_ext, Scalars* sc,
@@ -727,13 +740,6 @@ hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, uint32
   hipLaunchKernelGGL(k_build_cpu_ids, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, cpu, cpu_row, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t insert_device_first(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, uint32_t* slot_f_dev,
-                               Scalars* sc, hipStream_t st) {
-  if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_insert_device_first, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_device, tf, fc,
-                     slot_f_dev, sc);
-  return KTJ_LAUNCH_CHECK();
-}
 hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
                             const uint32_t* cpu_row, const ktj_generic_rec* g, EmitCtx ctx, hipStream_t st) {
   if (n == 0) return hipSuccess;
@@ -741,11 +747,13 @@ hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc,
                      g, ctx);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, FullCols fc, Table tn, NarrowCols nc,
-                            const uint32_t* slot_f_dev, DevLink* link, Scalars* sc, hipStream_t st) {
+hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, Table tn, NarrowCols nc,
+                            DevLink* link, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_link_device, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_device, fc, tn,
-                     nc, slot_f_dev, link, sc);
+  hipLaunchKernelGGL(k_link_device, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_device, tf, fc, tn,
+                     nc, link, sc);
+  hipLaunchKernelGGL(k_device_orphans, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, n, c, first_device, tf, fc,
+                     (const DevLink*)link, sc);
   return KTJ_LAUNCH_CHECK();
 }
 
@@ -1404,13 +1412,58 @@ __device__ __forceinline__ bool runtime_rows_share_slots(const Scalars* sc) {
   const KeyRange r = sc->plan.range[KTJ_TBL_FULL];
   return sc->runtime_ids_repeat != 0 || (r.lo <= r.hi && r.hi >= 0x80000000ULL);
 }
+/* Sets the slot's bit in a bitmap and tells whether it was set before.  All lanes of the wavefront
+ * call it (active = the lane has a slot).  Rows that arrive in id order put up to 32 neighbouring
+ * lanes on one word: where the wave's slots fall into at most two words, one lane per word sets
+ * all their bits at once; otherwise every lane sets its own.  Two lanes of the wave with the same
+ * slot are reported as "set before" for every lane of their word (callers only ask whether any
+ * slot is shared). */
+__device__ __forceinline__ uint32_t wave_or_u32(uint32_t v) {
+  for (int o = 32; o > 0; o >>= 1) v |= (uint32_t)__shfl_xor((int)v, o);
+  return v;
+}
+__device__ __forceinline__ bool bitmap_test_and_set(uint32_t* bitmap, uint32_t slot, bool active) {
+  const uint32_t word = slot >> 5, bit = active ? 1u << (slot & 31u) : 0u;
+  const uint64_t todo = __ballot(active);
+  if (!todo) return false;
+  const int l1 = __ffsll((unsigned long long)todo) - 1;
+  const uint32_t w1 = (uint32_t)__shfl((int)word, l1);
+  const bool in1 = active && word == w1;
+  const uint64_t m1 = __ballot(in1);
+  const uint64_t rest = todo & ~m1;
+  int l2 = 0;
+  uint32_t w2 = 0;
+  uint64_t m2 = 0;
+  if (rest) {
+    l2 = __ffsll((unsigned long long)rest) - 1;
+    w2 = (uint32_t)__shfl((int)word, l2);
+    m2 = __ballot(active && word == w2);
+  }
+  if ((m1 | m2) != todo) return active ? (atomicOr(&bitmap[word], bit) & bit) != 0 : false;
+  const bool in2 = active && !in1;
+  const uint32_t b1 = wave_or_u32(in1 ? bit : 0u), b2 = wave_or_u32(in2 ? bit : 0u);
+  uint32_t old1 = 0, old2 = 0;
+  if ((int)lane_id() == l1) old1 = atomicOr(&bitmap[w1], b1);
+  old1 = (uint32_t)__shfl((int)old1, l1);
+  if (m2) {
+    if ((int)lane_id() == l2) old2 = atomicOr(&bitmap[w2], b2);
+    old2 = (uint32_t)__shfl((int)old2, l2);
+  }
+  const bool twice1 = (uint32_t)__popc(b1) != (uint32_t)__popcll(m1), twice2 = (uint32_t)__popc(b2) != (uint32_t)__popcll(m2);
+  if (in1) return twice1 || (old1 & bit) != 0;
+  if (in2) return twice2 || (old2 & bit) != 0;
+  return false;
+}
 __global__ void k_join_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, ApiTable api, Table tf,
                                FullCols fc, Table tn, NarrowCols nc, uint32_t* slot_f, uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
                                uint32_t* len, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   RowStats rs;
   uint32_t n_linked = 0;
-  bool carries_stream = false, repeats = false;
+  bool carries_stream = false;
+  uint32_t sf = KTJ_NOSLOT;
+  if (i < n) sf = slot_insert(tf, c.corr[first_runtime + i]);
+  const bool repeats = bitmap_test_and_set(fc.has_runtime, sf, sf != KTJ_NOSLOT);
   if (i < n) {
     const uint64_t a = first_runtime + i;
     const ktj_runtime_rec rec = r[i];
@@ -1420,11 +1473,9 @@ __global__ void k_join_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, 
     const uint32_t kind = (meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
     const bool valid = (meta & KTJ_M_VALID) != 0;
     carries_stream = (meta & KTJ_M_HAS_STREAM) != 0;
-    const uint32_t sf = slot_insert(tf, id);
     slot_f[i] = sf;
     if (sf == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
     else {
-      repeats = atomicMin(&fc.first[sf], (uint32_t)a) != 0xFFFFFFFFu;
       FullPay fp;
       fp.first_ts = ts;
       fp.stream = 0;
@@ -1485,7 +1536,10 @@ __global__ void k_runtime_winners(uint64_t n, Columns c, uint64_t first, FullCol
     const uint32_t meta = c.meta[first + i];
     const uint32_t kind = (meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
     const uint32_t sf = slot_f[i], sn = slot_n[i];
-    if (sf != KTJ_NOSLOT && (meta & KTJ_M_HAS_STREAM)) atomicMax(&fc.stream_src[sf], (uint32_t)i + 1u);
+    if (sf != KTJ_NOSLOT) {
+      atomicMin(&fc.first[sf], (uint32_t)(first + i));
+      if (meta & KTJ_M_HAS_STREAM) atomicMax(&fc.stream_src[sf], (uint32_t)i + 1u);
+    }
     if (sn != KTJ_NOSLOT && (meta & KTJ_M_VALID) && kind != KTJ_RT_DEFAULT)
       atomicMax(kind == KTJ_RT_KERNEL ? &nc.kern_src[sn] : &nc.copy_src[sn], (uint32_t)i + 1u);
   }
