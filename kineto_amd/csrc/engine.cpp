@@ -389,7 +389,7 @@ int ktj_register_schema(ktj_engine* e, const ktj_field* f, size_t n_fields, uint
 
 int ktj_add_collective(ktj_engine* e, const ktj_collective_meta* meta, uint32_t* index) {
   if (!e || !meta) return KTJ_ERR_ARG;
-  if (e->collectives.size() >= 0x7FFFFFFEull) return KTJ_ERR_LIMIT;
+  if (e->collectives.size() >= KTJ_MAX_COLLECTIVES) return KTJ_ERR_LIMIT; /* the join tables keep 1 + index in 29 bits */
   if (index) *index = (uint32_t)e->collectives.size();
   e->collectives.push_back(make_collective(*meta));
   e->coll_dirty = true;

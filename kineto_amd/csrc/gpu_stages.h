@@ -60,14 +60,18 @@ struct FullCols {
 };
 /* per slot of the table keyed by the int-narrowed correlation id (and by the external-correlation
  * records' full id) */
-struct NarrowPay {         /* two writers, each with whole 8-byte words of its own */
+struct NarrowPay {         /* two writers (external-correlation records, runtime rows), in different passes */
   int32_t ext_val;         /* external id if a CPU op with that id exists, else 0               */
-  uint32_t linked;         /* 1 when ext_val names an existing CPU op                           */
-  uint32_t kind;           /* KTJ_DL_*: what pay[] holds                                        */
-  uint32_t coll;           /* 1 + index of the collective metadata of the linked CPU op, 0 = none */
+  uint32_t info;           /* bits 0-1: KTJ_DL_HAS_SIZE / KTJ_DL_HAS_GRID, what pay[] holds;
+                              bit 2: ext_val names an existing CPU op; bits 3-31: 1 + index of the
+                              collective metadata of the linked CPU op, 0 = none                  */
   uint64_t pay[3];         /* bytes of the winning copy / malloc row in pay[0], or packed grid /
                               workgroup of the winning kernel-launch row (see pack_grid)        */
-};                         /* 40 bytes */
+};                         /* 32 bytes: a slot never straddles a line */
+#define KTJ_NP_KIND_MASK 3u
+#define KTJ_NP_LINKED 4u
+#define KTJ_NP_COLL_SHIFT 3
+#define KTJ_MAX_COLLECTIVES ((1u << 29) - 2u)
 struct NarrowCols {
   uint32_t* ext_src;       /* last external-correlation record (index + 1), 0 = none            */
   uint32_t* kern_src;      /* last in-window kernel-launch row (index + 1)                     */

@@ -570,7 +570,7 @@ __global__ void k_clear_full(Table t, FullCols c) {
 }
 __global__ void k_clear_narrow(Table t, NarrowCols c) {
   const uint64_t n = table_extent(t);
-  NarrowPay z; z.ext_val = 0; z.linked = 0; z.kind = 0; z.coll = 0; z.pay[0] = z.pay[1] = z.pay[2] = 0;
+  NarrowPay z; z.ext_val = 0; z.info = 0; z.pay[0] = z.pay[1] = z.pay[2] = 0;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i <= n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t k = i < n ? i : t.mask + 1ull;
     c.ext_src[k] = 0; c.kern_src[k] = 0; c.copy_src[k] = 0; c.pay[k] = z;
@@ -637,11 +637,12 @@ __global__ void k_resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowC
   const uint32_t cs = slot_find(cpu, ext_id);
   if (cs != KTJ_NOSLOT) {
     nc.pay[slot].ext_val = (int32_t)(int64_t)ext_id;
-    nc.pay[slot].linked = 1u;
+    uint32_t info = KTJ_NP_LINKED;
     if (cpu_row) { /* the linked op is the last record with that id (activityMap_, GenericActivityProfiler.cpp:262) */
       const uint32_t row = cpu_row[cs];
-      if (row) nc.pay[slot].coll = collective_for_linked(g[row - 1], ctx);
+      if (row) info |= collective_for_linked(g[row - 1], ctx) << KTJ_NP_COLL_SHIFT;
     }
+    nc.pay[slot].info = info; /* the table was cleared, and the runtime rows come later */
   }
 }
 __device__ __forceinline__ bool is_async_op(uint32_t domain) { return domain != KTJ_DOM_MEMSET; }
@@ -673,12 +674,12 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Tabl
     if (sn != KTJ_NOSLOT) {
       const NarrowPay np = nc.pay[sn];
       ext = np.ext_val;
-      if (np.linked && valid) ++n_linked;
-      if (domain != KTJ_DOM_MEMSET && np.kind != 0) {
-        l.flags = np.kind;
+      if ((np.info & KTJ_NP_LINKED) && valid) ++n_linked;
+      if (domain != KTJ_DOM_MEMSET && (np.info & KTJ_NP_KIND_MASK) != 0) {
+        l.flags = np.info & KTJ_NP_KIND_MASK;
         l.p[0] = np.pay[0]; l.p[1] = np.pay[1]; l.p[2] = np.pay[2];
       }
-      l.coll = np.coll;
+      l.coll = np.info >> KTJ_NP_COLL_SHIFT;
     }
     c.ext[a] = ext;
     int64_t res = c.res[a];
@@ -1492,10 +1493,10 @@ __global__ void k_join_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, 
         NarrowPay* np = &nc.pay[sn];
         if (kind == KTJ_RT_KERNEL) {
           pack_grid(rec, np->pay);
-          np->kind = KTJ_DL_HAS_GRID;
+          np->info = (np->info & ~KTJ_NP_KIND_MASK) | KTJ_DL_HAS_GRID;
         } else {
           np->pay[0] = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
-          np->kind = KTJ_DL_HAS_SIZE;
+          np->info = (np->info & ~KTJ_NP_KIND_MASK) | KTJ_DL_HAS_SIZE;
         }
       }
     } else {
@@ -1505,7 +1506,7 @@ __global__ void k_join_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, 
     slot_n[i] = sn;
     if (sn != KTJ_NOSLOT) {
       ext = nc.pay[sn].ext_val;
-      if (nc.pay[sn].linked && valid) ++n_linked;
+      if ((nc.pay[sn].info & KTJ_NP_LINKED) && valid) ++n_linked;
     }
     c.ext[a] = ext;
     const bool known = rec.cid < api.n_cids;
@@ -1574,10 +1575,10 @@ __global__ void k_republish_runtime(const ktj_runtime_rec* r, uint64_t n, Column
       const uint32_t copy_src = nc.copy_src[sn]; /* final: the pass above has ended */
       if (copy_src == (uint32_t)i + 1u) {
         np->pay[0] = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
-        np->kind = KTJ_DL_HAS_SIZE;
+        np->info = (np->info & ~KTJ_NP_KIND_MASK) | KTJ_DL_HAS_SIZE;
       } else if (copy_src == 0 && nc.kern_src[sn] == (uint32_t)i + 1u) {
         pack_grid(rec, np->pay);
-        np->kind = KTJ_DL_HAS_GRID;
+        np->info = (np->info & ~KTJ_NP_KIND_MASK) | KTJ_DL_HAS_GRID;
       }
     }
   }
