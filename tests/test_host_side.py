@@ -155,3 +155,17 @@ def test_golden_digests():
         release()
         assert len(out) == g["output_bytes"], key
         assert hashlib.sha256(out).hexdigest() == g["output_sha256"], key
+
+
+def test_bench_refuses_more_than_one_gpu_and_fails_without_one():
+    """bench.py measures one GPU: --gpus above 1 exits with a message that says so; where no GPU is
+    visible it fails instead of measuring anything else."""
+    import subprocess
+    import sys
+    import torch
+    bench = os.path.join(ROOT, "bench.py")
+    r = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
+    if not torch.cuda.is_available():
+        r = subprocess.run([sys.executable, bench, "--steps", "1", "--warmup", "0"], capture_output=True, text=True, timeout=300)
+        assert r.returncode != 0 and "no GPU" in r.stderr and r.stdout.strip() == ""
