@@ -169,3 +169,18 @@ def test_bench_refuses_more_than_one_gpu_and_fails_without_one():
     if not torch.cuda.is_available():
         r = subprocess.run([sys.executable, bench, "--steps", "1", "--warmup", "0"], capture_output=True, text=True, timeout=300)
         assert r.returncode != 0 and "no GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_product_fails_loudly_without_its_library_or_a_gpu(tmp_path, monkeypatch):
+    """There is no CPU fallback: without the built HIP library the loader raises, and where the
+    library is there but no GPU is visible the engine cannot be created."""
+    import torch
+    from kineto_amd import engine
+    monkeypatch.setattr(abi, "_engine", None)
+    monkeypatch.setattr(abi, "LIB_DIR", str(tmp_path))
+    with pytest.raises(RuntimeError, match="not built"):
+        abi.load_engine()
+    monkeypatch.undo()
+    if not torch.cuda.is_available():
+        with pytest.raises(engine.EngineError):
+            engine.TraceEngine("t.json", device=0)
