@@ -159,7 +159,7 @@ __global__ void k_init_scalars(Scalars* s) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     s->ts_min_biased = ~0ULL; s->ts_max_biased = 0;
     s->out_of_range = 0; s->out_of_order = 0; s->n_flow = 0; s->n_linked = 0; s->n_blank_names = 0; s->n_valid = 0;
-    s->n_unresolved = 0; s->n_sync_typed = 0; s->error = 0; s->have_stream_src = 0; s->n_dev_ranks = 0; s->n_res_ranks = 0; s->n_dense = 0; s->runtime_ids_repeat = 0;
+    s->n_unresolved = 0; s->n_sync_typed = 0; s->n_device_orphans = 0; s->error = 0; s->have_stream_src = 0; s->n_dev_ranks = 0; s->n_res_ranks = 0; s->n_dense = 0; s->runtime_ids_repeat = 0;
     for (int k = 0; k < 3; ++k) {
       s->plan.range[k].lo = ~0ULL; s->plan.range[k].hi = 0;
       s->plan.ctl[k].base = 0; s->plan.ctl[k].span = 0; s->plan.ctl[k].direct = 0; s->plan.ctl[k].pad = 0;

@@ -1,0 +1,163 @@
+/*
+ * sdk_ref_driver.cpp — TEST INFRASTRUCTURE ONLY.
+ *
+ * Runs the reference's own RocprofLogger callbacks (libkineto/src/RocprofLogger.cpp:561-679
+ * api_callback, :681-749 buffer_callback) on records built in memory, without a profiling
+ * session, and prints the rocprof*Row objects they produce.  The reference translation unit is
+ * compiled where it lies (this file includes it, so that the file-local global context and the
+ * private callbacks are reachable; built with -fno-access-control) and linked against the
+ * rocprofiler-sdk of this image; nothing of either is copied.
+ *
+ * A separate executable, never loaded into a test process: the translation unit defines
+ * rocprofiler_configure, which a process that initialises HIP would hand to the SDK.
+ *
+ * stdin (binary, little endian):
+ *   u32 mode                       1 = buffer records, 2 = HIP runtime API records
+ * mode 1:
+ *   u64 n_rows, ktj_device_rec rows[n_rows], u64 agent_base, u64 kernel_base, u32 unknown_name_id,
+ *   u32 noise, u64 n_agents, {u64 handle, i64 device}[n_agents], u64 n_kernels,
+ *   {u64 kernel_id, u64 name_id}[n_kernels]
+ *   The SDK records are built by tests/host_sim/sdk_records.cpp from the rows, as in the tests.
+ * mode 2:
+ *   u64 n_records, {u32 operation, u32 pad, u64 correlation_id, u8 args[sizeof(rocprofiler_hip_api_args_t)]}[n]
+ * stdout: one text line per row the logger holds afterwards.
+ */
+#include "RocprofLogger.cpp"  // NOLINT: the reference's translation unit, found through -I$(REF)/libkineto/src
+
+#include <cinttypes>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include <rocprofiler-sdk/hip/api_args.h>
+
+#include "../../include/ktj.h"
+
+extern "C" {
+void* ktjsim_sdk_buffer_create(const ktj_device_rec* rows, uint64_t n, uint64_t agent_base, uint64_t kernel_base,
+                               uint32_t unknown_name_id, int noise);
+void* const* ktjsim_sdk_buffer_headers(void* buf);
+uint64_t ktjsim_sdk_buffer_count(void* buf);
+}
+
+namespace {
+
+template <typename T> T rd() {
+  T v;
+  if (fread(&v, sizeof v, 1, stdin) != 1) { fprintf(stderr, "sdk_ref_driver: short input\n"); exit(2); }
+  return v;
+}
+
+void print_rows() {
+  for (const rocprofBase* b : RocprofLogger::singleton().rows_) {
+    switch (b->type) {
+      case ROCTRACER_ACTIVITY_ASYNC: {
+        const auto* r = static_cast<const rocprofAsyncRow*>(b);
+        printf("async id=%" PRIu64 " begin=%" PRIu64 " end=%" PRIu64 " domain=%u kind=%u op=%u device=%d queue=%" PRIu64
+               " stream=%" PRIu64 " name=%s\n",
+               r->id, r->begin, r->end, r->domain, r->kind, r->op, r->device, r->queue, r->stream, r->kernelName.c_str());
+        break;
+      }
+      case ROCTRACER_ACTIVITY_KERNEL: {
+        const auto* r = static_cast<const rocprofKernelRow*>(b);
+        printf("kernel id=%" PRIu64 " domain=%u cid=%u grid=%u,%u,%u workgroup=%u,%u,%u gss=%zu stream=%" PRIu64
+               " faddr=%" PRIu64 " function=%" PRIu64 "\n",
+               r->id, r->domain, r->cid, r->gridX, r->gridY, r->gridZ, r->workgroupX, r->workgroupY, r->workgroupZ,
+               r->groupSegmentSize, (uint64_t)(uintptr_t)r->stream, (uint64_t)(uintptr_t)r->functionAddr,
+               (uint64_t)(uintptr_t)r->function);
+        break;
+      }
+      case ROCTRACER_ACTIVITY_COPY: {
+        const auto* r = static_cast<const rocprofCopyRow*>(b);
+        /* src and dst hold the SDK's rendering of the argument (a C string), see RocprofLogger.cpp:611-624 */
+        printf("copy id=%" PRIu64 " domain=%u cid=%u src=%s dst=%s size=%zu kind=%d stream=%" PRIu64 "\n", r->id, r->domain,
+               r->cid, static_cast<const char*>(r->src), static_cast<const char*>(r->dst), r->size, (int)r->kind,
+               (uint64_t)(uintptr_t)r->stream);
+        break;
+      }
+      case ROCTRACER_ACTIVITY_MALLOC: {
+        const auto* r = static_cast<const rocprofMallocRow*>(b);
+        printf("malloc id=%" PRIu64 " domain=%u cid=%u ptr=%s size=%zu\n", r->id, r->domain, r->cid,
+               static_cast<const char*>(r->ptr), r->size);
+        break;
+      }
+      case ROCTRACER_ACTIVITY_DEFAULT: {
+        const auto* r = static_cast<const rocprofRow*>(b);
+        printf("default id=%" PRIu64 " domain=%u cid=%u\n", r->id, r->domain, r->cid);
+        break;
+      }
+      default: printf("other type=%d\n", (int)b->type); break;
+    }
+  }
+}
+
+int run_buffer_records() {
+  const uint64_t n = rd<uint64_t>();
+  std::vector<ktj_device_rec> rows(n);
+  if (n && fread(rows.data(), sizeof(ktj_device_rec), n, stdin) != n) return 2;
+  const uint64_t agent_base = rd<uint64_t>(), kernel_base = rd<uint64_t>();
+  const uint32_t unknown = rd<uint32_t>(), noise = rd<uint32_t>();
+  auto& g = getGlobalContext();
+  const uint64_t n_agents = rd<uint64_t>();
+  for (uint64_t i = 0; i < n_agents; ++i) {
+    const uint64_t handle = rd<uint64_t>();
+    const int64_t device = rd<int64_t>();
+    rocprofiler_agent_v0_t a;
+    std::memset(&a, 0, sizeof a);
+    a.id.handle = handle;
+    a.logical_node_type_id = (int32_t)device;
+    g.agents[handle] = a;
+  }
+  const uint64_t n_kernels = rd<uint64_t>();
+  for (uint64_t i = 0; i < n_kernels; ++i) {
+    const uint64_t id = rd<uint64_t>(), name_id = rd<uint64_t>();
+    g.kernel_names[id] = "name#" + std::to_string(name_id);
+  }
+  /* the SDK's numbers for the two record kinds, so that the reader need not know them */
+  printf("kinds dispatch=%d copy=%d\n", (int)ROCPROFILER_BUFFER_TRACING_KERNEL_DISPATCH, (int)ROCPROFILER_BUFFER_TRACING_MEMORY_COPY);
+  void* buf = ktjsim_sdk_buffer_create(rows.data(), n, agent_base, kernel_base, unknown, (int)noise);
+  auto** headers = reinterpret_cast<rocprofiler_record_header_t**>(const_cast<void**>(ktjsim_sdk_buffer_headers(buf)));
+  RocprofLogger::buffer_callback(rocprofiler_context_id_t{0}, rocprofiler_buffer_id_t{0}, headers, ktjsim_sdk_buffer_count(buf),
+                                 nullptr, 0);
+  print_rows();
+  return 0;
+}
+
+int run_api_records() {
+  const uint64_t n = rd<uint64_t>();
+  for (uint64_t i = 0; i < n; ++i) {
+    const uint32_t op = rd<uint32_t>();
+    (void)rd<uint32_t>();
+    const uint64_t corr = rd<uint64_t>();
+    rocprofiler_callback_tracing_hip_api_data_t data;
+    std::memset(&data, 0, sizeof data);
+    data.size = sizeof data;
+    if (fread(&data.args, sizeof data.args, 1, stdin) != 1) return 2;
+    rocprofiler_callback_tracing_record_t rec;
+    std::memset(&rec, 0, sizeof rec);
+    rec.correlation_id.internal = corr;
+    rec.kind = ROCPROFILER_CALLBACK_TRACING_HIP_RUNTIME_API;
+    rec.operation = (rocprofiler_tracing_operation_t)op;
+    rec.payload = &data;
+    rec.phase = ROCPROFILER_CALLBACK_PHASE_ENTER;
+    RocprofLogger::api_callback(rec, nullptr, nullptr);
+    rec.phase = ROCPROFILER_CALLBACK_PHASE_EXIT;
+    RocprofLogger::api_callback(rec, nullptr, nullptr);
+    /* the rows of copies and allocations point at strings the SDK renders per call: print now */
+    print_rows();
+    RocprofLogger::singleton().rows_.clear();
+  }
+  return 0;
+}
+
+}  // namespace
+
+int main() {
+  const uint32_t mode = rd<uint32_t>();
+  int rc = 2;
+  if (mode == 1) rc = run_buffer_records();
+  else if (mode == 2) rc = run_api_records();
+  fflush(stdout);
+  _exit(rc); /* no destructors: the logger's would stop a tracing context that was never created */
+}

@@ -5,9 +5,11 @@
  * rocprofiler-sdk buffer records become rocprofAsyncRow objects (src/RocLogger.h:216-240) and
  * with which fields.  The rows come out as ktj_device_rec, the packed form of rocprofAsyncRow.
  *
- * Parity unpinned by the reference: the function itself needs a live rocprofiler-sdk context
- * (agent query, code-object callbacks) and is not part of oracle/_ref; the reference's tests do
- * not cover it.  The tests pin this restatement with hand-written records and expected rows.
+ * Pinned against the reference's own function: oracle/_ref/sdk_ref_driver compiles
+ * RocprofLogger.cpp where it lies, fills the logger's agent and kernel-name tables and calls
+ * buffer_callback on the same SDK records; tests/test_sdk_ingest.py compares the rows field by
+ * field (hand-written records and the device rows of four synthetic configurations, with and
+ * without records of other kinds mixed in).
  */
 #include <rocprofiler-sdk/buffer_tracing.h>
 #include <stdint.h>

@@ -280,7 +280,8 @@ def test_user_annotation_spans():
         compare(case()[0].build())
 
 
-def test_join_edge_cases():
+def join_edge_case_builder():
+    """The hand-made stream of join edge cases (shared with the GPU parity suite)."""
     b = StreamBuilder(window=(B + 100, B + 10**9))
     b.api(["hipLaunchKernel", "hipMemcpyAsync", "hipMalloc", "hipGraphLaunch"], flow_start=[0, 1, 2, 3], malloc_cid=2)
     pid, tid = 10, 11
@@ -310,7 +311,11 @@ def test_join_edge_cases():
     b.add_device(80, B + 1090, B + 1100, domain=2, queue=1, stream=5, nbytes=1000)    # memset
     b.add_device(0xFFFFFFFFFFFFFFFF, B + 1110, B + 1120, domain=0, name="k", queue=4, device=1)
     b.add_device(81, 0, B + 1130, domain=0, name="k", queue=4, device=1)              # begin 0
-    compare(b.build())
+    return b
+
+
+def test_join_edge_cases():
+    compare(join_edge_case_builder().build())
 
 
 def test_join_without_any_runtime_stream():

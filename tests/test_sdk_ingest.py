@@ -1,12 +1,14 @@
 """rocprofiler-sdk buffer records as device rows (include/ktj_rocprofiler.h).
 
 The record structs come from the SDK's own header (tests/host_sim/sdk_records.cpp builds them).
-CPU: the checker's restatement of RocprofLogger::buffer_callback (oracle/sdk_rows.c) against
-hand-written expectations.  GPU: ktj_submit_sdk_buffer against the checker, end to end.  The
-reference's buffer_callback needs a live profiling session and is not built, so these
-expectations are this repository's reading of libkineto/src/RocprofLogger.cpp:681-749."""
+CPU: the checker's restatement of RocprofLogger::buffer_callback (oracle/sdk_rows.c) against the
+reference's own function (libkineto/src/RocprofLogger.cpp:681-749, compiled where it lies into
+oracle/_ref/sdk_ref_driver and run on the same records) and against hand-written expectations.
+GPU: ktj_submit_sdk_buffer against the checker, end to end."""
 import ctypes as C
 import os
+import struct
+import subprocess
 
 import pytest
 
@@ -81,6 +83,76 @@ def test_checker_restatement_on_hand_written_records():
         ((1 << 40) + 3, 5000, 5001, 0, 1, -1, unknown, (1 << 63) + 2, 0, 0),  # unknown agent and kernel
         (14, 0, 0, 1, 4, -1, abi.KTJ_NONE, 0, 0, 0),
     ]
+
+
+SDK_REF_DRIVER = os.path.join(ROOT, "oracle", "_ref", "sdk_ref_driver")
+
+
+def _reference_rows(rows, agents, kernels, unknown, noise):
+    """The rocprofAsyncRow objects the reference's buffer_callback makes of the SDK records that
+    tests/host_sim/sdk_records.cpp builds from `rows`, as DeviceRec-shaped tuples."""
+    req = struct.pack("<IQ", 1, len(rows)) + b"".join(bytes(r) for r in rows)
+    req += struct.pack("<QQIIQ", AGENT_BASE, KERNEL_BASE, unknown, noise, len(agents))
+    req += b"".join(struct.pack("<Qq", a, d) for a, d in agents)
+    req += struct.pack("<Q", len(kernels)) + b"".join(struct.pack("<QQ", k, v) for k, v in kernels)
+    out = subprocess.run([SDK_REF_DRIVER], input=req, stdout=subprocess.PIPE, check=True, timeout=120).stdout.decode("latin1")
+    lines = out.split("\n")
+    kinds = dict(kv.split("=") for kv in lines[0].split()[1:])
+    domain_of = {int(kinds["dispatch"]): 0, int(kinds["copy"]): 1}
+    got = []
+    for line in lines[1:]:
+        if not line:
+            continue
+        head, name = line.split(" name=", 1)
+        kind, *kv = head.split()
+        assert kind == "async", line
+        f = dict(x.split("=") for x in kv)
+        if name == "":
+            name_id = abi.KTJ_NONE
+        elif name == "<unknown kernel>":
+            name_id = unknown
+        else:
+            assert name.startswith("name#"), line
+            name_id = int(name[5:])
+        assert f["kind"] == f["op"]     # "shared op" placeholder, RocprofLogger.cpp:716-720
+        got.append((int(f["id"]), int(f["begin"]), int(f["end"]), domain_of[int(f["domain"])], int(f["op"]), int(f["device"]),
+                    name_id, int(f["queue"]), int(f["stream"])))
+    return got
+
+
+@pytest.mark.skipif(not os.path.exists(SDK_REF_DRIVER), reason="oracle/_ref/sdk_ref_driver is not built (needs the reference's sources)")
+@pytest.mark.parametrize("case", ["hand", 1, 2, 3, 4])
+def test_checker_restatement_matches_the_reference_buffer_callback(case):
+    """Pins ktj_oracle_sdk_rows: same SDK records through the reference's RocprofLogger::buffer_callback
+    and through the checker's restatement give the same rows, field by field, in the same order;
+    records of other kinds and categories are skipped by both."""
+    sim = _sim()
+    if case == "hand":
+        unknown = 900
+        rows = [_row(id=11, begin=1000, end=2000, domain=0, op=1, device=0, name_id=5, queue=77),
+                _row(id=12, begin=3000, end=3500, domain=1, op=2, device=1, name_id=123, queue=99, stream=7, bytes=4096),
+                _row(id=(1 << 40) + 3, begin=5000, end=5001, domain=0, op=1, device=-1, name_id=unknown, queue=(1 << 63) + 2),
+                _row(id=(1 << 64) - 1, begin=(1 << 64) - 1, end=0, domain=0, op=0xFFFFFFFF, device=7, name_id=0, queue=(1 << 64) - 1),
+                _row(id=14, begin=0, end=0, domain=1, op=4, device=-1),
+                _row(id=0, begin=9, end=8, domain=1, op=0, device=3)]
+        release = None
+    else:
+        sp, release, rows, unknown = _sdk_case(case, 4000)
+    try:
+        arr = (abi.DeviceRec * max(len(rows), 1))(*rows)
+        agents, kernels = _tables(rows, unknown)
+        for noise in (0, 1):
+            want = _reference_rows(rows, agents, kernels, unknown, noise)
+            buf = sim.ktjsim_sdk_buffer_create(arr, len(rows), AGENT_BASE, KERNEL_BASE, unknown, noise)
+            n_headers = sim.ktjsim_sdk_buffer_count(buf)
+            out, n = _oracle_rows(sim.ktjsim_sdk_buffer_headers(buf), n_headers, agents, kernels, unknown)
+            got = [(r.id, r.begin, r.end, r.domain, r.op, r.device, r.name_id, r.queue, r.stream) for r in out[:n]]
+            sim.ktjsim_sdk_buffer_free(buf)
+            assert n == len(rows) == len(want)
+            assert got == want
+    finally:
+        if release:
+            release()
 
 
 def _sdk_case(cfg, n):
