@@ -445,6 +445,26 @@ int ktj_submit_info(ktj_engine* e, int info_kind, const void* info);
  * be called again after more ktj_submit_* calls (everything is re-processed). */
 int ktj_process(ktj_engine* e, int64_t end_time_ns);
 
+/* ktj_process for callers that cannot allocate device memory while they run: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same pass and same document as ktj_process, but
+ *   - every working buffer is a piece of a static array in device memory that the library holds
+ *     once per GPU (KTJ_NOALLOC_SCRATCH_BYTES, until the process ends) instead of an allocation;
+ *   - the document is written to out_device, a buffer of out_capacity bytes in device memory of the
+ *     engine's GPU, 16-byte aligned, which must hold the document plus 64 bytes;
+ *   - the call makes no hipMalloc, hipFree, hipHostMalloc or other allocating HIP call.
+ * Records, strings, schemas and infos are submitted before, as for ktj_process (those calls may
+ * allocate; ktj_submit_records_device does not).  *n_bytes receives the document's length.
+ * KTJ_ERR_LIMIT: the trace needs more working memory than the scratch array holds (roughly
+ * 100 000 records; ktj_last_error says how much was asked for), or the output buffer is too small
+ * (*n_bytes then holds the document's length), or the trace has user-domain correlation records
+ * (KTJ_REC_USERCORR), which this entry point does not take.  All engines on one GPU share that
+ * GPU's array and it keeps the last call's contents (the pass clears what it needs cleared):
+ * calls that overlap in time on one GPU race and must be serialised by the caller. */
+#define KTJ_NOALLOC_SCRATCH_BYTES (64u << 20)
+int ktj_process_noalloc(ktj_engine* e, int64_t end_time_ns, void* out_device, uint64_t out_capacity,
+                        uint64_t* n_bytes);
+
 /* Device / host views of the finished document (valid until the next ktj_process/destroy). */
 int ktj_output_device(ktj_engine* e, const void** device_ptr, uint64_t* n_bytes);
 int ktj_output_host(ktj_engine* e, const char** host_ptr, uint64_t* n_bytes); /* pinned; D2H on first call */

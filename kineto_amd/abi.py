@@ -182,7 +182,7 @@ ENGINE_SYMBOLS = [
     "ktj_create", "ktj_destroy", "ktj_last_error", "ktj_trace_start", "ktj_intern_strings",
     "ktj_register_schema", "ktj_add_collective", "ktj_submit_args", "ktj_set_api_table", "ktj_set_clock_model",
     "ktj_set_window", "ktj_submit_records", "ktj_submit_records_device", "ktj_submit_info",
-    "ktj_process", "ktj_output_device", "ktj_output_host", "ktj_finalize", "ktj_get_stats",
+    "ktj_process", "ktj_process_noalloc", "ktj_output_device", "ktj_output_host", "ktj_finalize", "ktj_get_stats",
     "ktj_version",
     # include/ktj_rocprofiler.h
     "ktj_set_sdk_agents", "ktj_set_sdk_kernel_names", "ktj_submit_sdk_buffer",
@@ -236,6 +236,8 @@ def load_engine():
         lib.ktj_submit_sdk_buffer.argtypes = [vp, C.POINTER(C.c_void_p), C.c_size_t, C.POINTER(C.c_uint64)]
         lib.ktj_process.restype = C.c_int
         lib.ktj_process.argtypes = [vp, C.c_int64]
+        lib.ktj_process_noalloc.restype = C.c_int
+        lib.ktj_process_noalloc.argtypes = [vp, C.c_int64, C.c_void_p, C.c_uint64, C.POINTER(C.c_uint64)]
         lib.ktj_output_device.restype = C.c_int
         lib.ktj_output_device.argtypes = [vp, C.POINTER(C.c_void_p), C.POINTER(C.c_uint64)]
         lib.ktj_output_host.restype = C.c_int

@@ -32,27 +32,36 @@ using namespace ktj::gpu;
 
 namespace {
 
-struct DevBuf { /* owns one device allocation; freed with the engine (the engine's device is current then) */
+/* One working buffer in device memory.  `p` is what the kernels use: either the buffer's own
+ * allocation (freed with the engine; the engine's device is current then) or, for the entry point
+ * that allocates nothing, a borrowed range that somebody else owns (a piece of the library's static
+ * scratch array, or the caller's output buffer).  The own allocation survives a borrow. */
+struct DevBuf {
   void* p = nullptr;
   size_t cap = 0;
+  void* own = nullptr;
+  size_t own_cap = 0;
   DevBuf() = default;
   DevBuf(const DevBuf&) = delete;
   DevBuf& operator=(const DevBuf&) = delete;
   DevBuf& operator=(DevBuf&& o) noexcept {
-    if (this != &o) { release(); p = o.p; cap = o.cap; o.p = nullptr; o.cap = 0; }
+    if (this != &o) { release(); p = o.p; cap = o.cap; own = o.own; own_cap = o.own_cap; o.p = o.own = nullptr; o.cap = o.own_cap = 0; }
     return *this;
   }
   ~DevBuf() { release(); }
   hipError_t ensure(size_t bytes) {
+    if (p != own) { p = own; cap = own_cap; } /* back from a borrowed range */
     if (bytes <= cap) return hipSuccess;
-    if (p) { hipError_t e = hipFree(p); p = nullptr; cap = 0; if (e != hipSuccess) return e; }
+    if (own) { hipError_t e = hipFree(own); p = own = nullptr; cap = own_cap = 0; if (e != hipSuccess) return e; }
     size_t want = bytes + bytes / 8 + 256;
-    hipError_t e = hipMalloc(&p, want);
-    if (e != hipSuccess) { p = nullptr; return e; }
-    cap = want;
+    hipError_t e = hipMalloc(&own, want);
+    if (e != hipSuccess) { p = own = nullptr; return e; }
+    p = own;
+    cap = own_cap = want;
     return hipSuccess;
   }
-  void release() { if (p) (void)hipFree(p); p = nullptr; cap = 0; }
+  void borrow(void* ptr, size_t bytes) { p = ptr; cap = bytes; }
+  void release() { if (own) (void)hipFree(own); p = own = nullptr; cap = own_cap = 0; }
   template <typename T> T* as() const { return reinterpret_cast<T*>(p); }
 };
 
@@ -88,6 +97,15 @@ struct RecordSet {
   uint64_t n = 0;
   const void* ptr() const { return external ? external : owned.buf.p; }
 };
+
+/* read-backs of one pass land in pinned host memory (no staging inside the runtime) */
+struct HostCtl {
+  Scalars scalars;
+  uint64_t act_bytes;
+  uint32_t n_out;
+  uint32_t pad;
+};
+#define KTJ_PINNED_SMALL_BYTES (256u << 10) /* header/footer text and small tables of a pass that may not allocate */
 
 enum { EV_START = 0, EV_DICT, EV_DECODE, EV_CONVERT, EV_JOIN, EV_SORT_A, EV_SORT_B, EV_SORT, EV_SIZE, EV_SCAN,
        EV_EMIT_START, EV_EMIT, EV_COUNT };
@@ -147,6 +165,10 @@ struct ktj_engine {
   DevBuf keys_a, keys_b, vals_a, vals_b, hist, scan_tmp;
   DevBuf mat, len, len_sorted, kind_sorted, offs, out, tile_start;
   void* pinned_small = nullptr; size_t pinned_small_cap = 0;
+  HostCtl* h_ctl = nullptr;                  /* pinned: what the device hands back during a pass */
+  /* ktj_process_noalloc: working buffers are carved out of the library's static scratch array */
+  bool noalloc = false;
+  char* arena = nullptr; size_t arena_cap = 0, arena_used = 0;
   char* pinned_out = nullptr; size_t pinned_out_cap = 0;
   char* file_stage[2] = {nullptr, nullptr};   /* pinned staging of the file sink, at most KTJ_FILE_STAGE_BYTES each */
   size_t file_stage_cap[2] = {0, 0};
@@ -182,8 +204,39 @@ std::string default_file_name() { /* output_json.cpp:65-70, 481-483 */
   return "/tmp/libkineto_activities_" + std::to_string((long)getpid()) + ".json";
 }
 
+/* Room for `bytes` in a working buffer.  Normally the buffer grows by allocation; in a pass that
+ * may not allocate it becomes the next piece of the scratch array (256-byte aligned), or the pass
+ * fails with KTJ_ERR_LIMIT. */
+int need(ktj_engine* e, DevBuf& b, size_t bytes) {
+  if (!e->noalloc) { HIPCHK(b.ensure(bytes)); return KTJ_OK; }
+  const size_t off = (e->arena_used + 255) & ~(size_t)255;
+  if (off > e->arena_cap || bytes > e->arena_cap - off) {
+    e->last_error = "ktj_process_noalloc: the trace needs more than the " + std::to_string(e->arena_cap) +
+                    " bytes of the static scratch array (asked for " + std::to_string(bytes) + " more at " + std::to_string(off) + ")";
+    return KTJ_ERR_LIMIT;
+  }
+  b.borrow(e->arena + off, bytes);
+  e->arena_used = off + bytes;
+  return KTJ_OK;
+}
+#define NEED(buf, bytes)                                  \
+  do {                                                    \
+    const int _rc = need(e, buf, bytes);                  \
+    if (_rc != KTJ_OK) return _rc;                        \
+  } while (0)
+
+/* A small host table to the device.  A pass that may not allocate stages it through the pinned
+ * buffer of the engine (allocated with the engine) instead of the runtime's own staging. */
 int upload_small(ktj_engine* e, DevBuf& dst, const void* src, size_t bytes) {
-  HIPCHK(dst.ensure(bytes ? bytes : 16));
+  NEED(dst, bytes ? bytes : 16);
+  if (bytes && e->noalloc) {
+    if (bytes > e->pinned_small_cap) {
+      e->last_error = "ktj_process_noalloc: a table of " + std::to_string(bytes) + " bytes exceeds the pinned staging buffer";
+      return KTJ_ERR_LIMIT;
+    }
+    memcpy(e->pinned_small, src, bytes);
+    src = e->pinned_small;
+  }
   if (bytes) HIPCHK(hipMemcpyAsync(dst.p, src, bytes, hipMemcpyHostToDevice, e->stream));
   HIPCHK(hipStreamSynchronize(e->stream));
   return KTJ_OK;
@@ -208,13 +261,13 @@ int synthesise_user_spans(ktj_engine* e, Columns c, const EmitCtx& ctx, Table t_
   const ktj_generic_rec* g_recs = static_cast<const ktj_generic_rec*>(e->generic.ptr());
   const ktj_extcorr_rec* u_recs = static_cast<const ktj_extcorr_rec*>(e->usercorr.ptr());
   const uint32_t cap_user = pow2_at_least(2 * nu), cap_span = pow2_at_least(2 * nd);
-  HIPCHK(e->u_keys.ensure((cap_user + 1ull) * 8)); HIPCHK(e->u_src.ensure((cap_user + 1ull) * 4));
-  HIPCHK(e->sp_hash.ensure((cap_span + 1ull) * 8)); HIPCHK(e->sp_first.ensure((cap_span + 1ull) * 4));
-  HIPCHK(e->sp_lo.ensure((cap_span + 1ull) * 8)); HIPCHK(e->sp_hi.ensure((cap_span + 1ull) * 8));
-  HIPCHK(e->sp_zero.ensure((cap_span + 1ull) * 4)); HIPCHK(e->sp_dev.ensure((cap_span + 1ull) * 4));
-  HIPCHK(e->sp_res.ensure((cap_span + 1ull) * 8)); HIPCHK(e->sp_ext.ensure((cap_span + 1ull) * 8));
-  HIPCHK(e->sp_name.ensure((cap_span + 1ull) * 4)); HIPCHK(e->sp_out.ensure((nd + 1ull) * sizeof(SpanOut)));
-  HIPCHK(e->sp_count.ensure(16));
+  NEED(e->u_keys, (cap_user + 1ull) * 8); NEED(e->u_src, (cap_user + 1ull) * 4);
+  NEED(e->sp_hash, (cap_span + 1ull) * 8); NEED(e->sp_first, (cap_span + 1ull) * 4);
+  NEED(e->sp_lo, (cap_span + 1ull) * 8); NEED(e->sp_hi, (cap_span + 1ull) * 8);
+  NEED(e->sp_zero, (cap_span + 1ull) * 4); NEED(e->sp_dev, (cap_span + 1ull) * 4);
+  NEED(e->sp_res, (cap_span + 1ull) * 8); NEED(e->sp_ext, (cap_span + 1ull) * 8);
+  NEED(e->sp_name, (cap_span + 1ull) * 4); NEED(e->sp_out, (nd + 1ull) * sizeof(SpanOut));
+  NEED(e->sp_count, 16);
   SpanTables t{e->u_keys.as<uint64_t>(), e->u_src.as<uint32_t>(), cap_user - 1,
                e->sp_hash.as<uint64_t>(), e->sp_first.as<uint32_t>(), e->sp_lo.as<uint64_t>(), e->sp_hi.as<uint64_t>(),
                e->sp_zero.as<uint32_t>(), cap_span - 1,
@@ -225,9 +278,9 @@ int synthesise_user_spans(ktj_engine* e, Columns c, const EmitCtx& ctx, Table t_
   HIPCHK(fill_u32(t.zero, 0, cap_span + 1ull, st));
   HIPCHK(build_usercorr(u_recs, nu, t, sc, st));
   HIPCHK(group_spans(u_recs, g_recs, nd, c, ng + nr, t_cpu, cpu_row, t, e->sp_out.as<SpanOut>(), e->sp_count.as<uint32_t>(), sc, st));
-  uint32_t n_out = 0;
-  HIPCHK(hipMemcpyAsync(&n_out, e->sp_count.p, 4, hipMemcpyDeviceToHost, st));
+  HIPCHK(hipMemcpyAsync(&e->h_ctl->n_out, e->sp_count.p, 4, hipMemcpyDeviceToHost, st));
   HIPCHK(hipStreamSynchronize(st));
+  const uint32_t n_out = e->h_ctl->n_out;
   if (n_out == 0) return KTJ_OK;
   std::vector<SpanOut> spans(n_out);
   HIPCHK(hipMemcpyAsync(spans.data(), e->sp_out.p, n_out * sizeof(SpanOut), hipMemcpyDeviceToHost, st));
@@ -240,11 +293,11 @@ int synthesise_user_spans(ktj_engine* e, Columns c, const EmitCtx& ctx, Table t_
   bool any_zero = false;
   for (const SpanOut& sp : spans) any_zero = any_zero || sp.zero != 0;
   if (any_zero) {
-    HIPCHK(e->sp_members.ensure((nd + 1ull) * sizeof(SpanMember)));
+    NEED(e->sp_members, (nd + 1ull) * sizeof(SpanMember));
     HIPCHK(span_members(u_recs, nd, c, ng + nr, t_cpu, t, e->sp_members.as<SpanMember>(), (uint32_t)nd, e->sp_count.as<uint32_t>(), st));
-    uint32_t n_members = 0;
-    HIPCHK(hipMemcpyAsync(&n_members, e->sp_count.p, 4, hipMemcpyDeviceToHost, st));
+    HIPCHK(hipMemcpyAsync(&e->h_ctl->n_out, e->sp_count.p, 4, hipMemcpyDeviceToHost, st));
     HIPCHK(hipStreamSynchronize(st));
+    const uint32_t n_members = e->h_ctl->n_out;
     std::vector<SpanMember> members(n_members);
     if (n_members) HIPCHK(hipMemcpyAsync(members.data(), e->sp_members.p, n_members * sizeof(SpanMember), hipMemcpyDeviceToHost, st));
     HIPCHK(hipStreamSynchronize(st));
@@ -283,7 +336,7 @@ int synthesise_user_spans(ktj_engine* e, Columns c, const EmitCtx& ctx, Table t_
       recs.push_back(r);
     }
   }
-  HIPCHK(e->synth_recs.ensure(recs.size() * sizeof(ktj_generic_rec) + 16));
+  NEED(e->synth_recs, recs.size() * sizeof(ktj_generic_rec) + 16);
   HIPCHK(hipMemcpyAsync(e->synth_recs.p, recs.data(), recs.size() * sizeof(ktj_generic_rec), hipMemcpyHostToDevice, st));
   HIPCHK(hipStreamSynchronize(st));
   HIPCHK(decode_generic(e->synth_recs.as<ktj_generic_rec>(), recs.size(), c, first_row, sc, ctx, st));
@@ -318,6 +371,21 @@ int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int
   for (auto& ev : e->ev) HIPCHK(hipEventCreate(&ev));
   for (auto& ev : e->ev_d2h) HIPCHK(hipEventCreate(&ev));
   HIPCHK(e->d_scalars.ensure(sizeof(Scalars)));
+  HIPCHK(hipHostMalloc(&e->pinned_small, KTJ_PINNED_SMALL_BYTES, hipHostMallocDefault));
+  e->pinned_small_cap = KTJ_PINNED_SMALL_BYTES;
+  {
+    void* p = nullptr;
+    HIPCHK(hipHostMalloc(&p, sizeof(HostCtl), hipHostMallocDefault));
+    e->h_ctl = static_cast<HostCtl*>(p);
+    memset(e->h_ctl, 0, sizeof(HostCtl));
+  }
+  { /* this device's copy of the static scratch array (ktj_process_noalloc) */
+    void* p = nullptr;
+    size_t bytes = 0;
+    HIPCHK(scratch_address(hip_device, &p, &bytes));
+    e->arena = static_cast<char*>(p);
+    e->arena_cap = bytes;
+  }
   return KTJ_OK;
 }
 
@@ -327,6 +395,7 @@ void ktj_destroy(ktj_engine* e) {
   if (e->stream) (void)hipStreamSynchronize(e->stream);
   /* device buffers free themselves when the engine is deleted below */
   if (e->pinned_small) (void)hipHostFree(e->pinned_small);
+  if (e->h_ctl) (void)hipHostFree(e->h_ctl);
   if (e->pinned_out) (void)hipHostFree(e->pinned_out);
   for (auto& p : e->file_stage) if (p) (void)hipHostFree(p);
   for (auto& ev : e->ev_file_stage) if (ev) (void)hipEventDestroy(ev);
@@ -553,11 +622,17 @@ int ktj_submit_info(ktj_engine* e, int info_kind, const void* info) {
   return KTJ_OK;
 }
 
-int ktj_process(ktj_engine* e, int64_t end_time_ns) {
-  if (!e) return KTJ_ERR_ARG;
-  if (e->bad_sink) return KTJ_OK;
+/* One pass of the whole path.  out_device == nullptr: the document goes into the engine's own
+ * buffer and working memory is allocated as needed (ktj_process).  Otherwise (ktj_process_noalloc,
+ * e->noalloc set by the caller): the document goes into the caller's buffer of out_cap bytes and
+ * every working buffer is a piece of the scratch array. */
+static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, uint64_t out_cap) {
   HIPCHK(hipSetDevice(e->device));
   hipStream_t st = e->stream;
+  e->arena_used = 0;
+  e->processed = false;
+  e->total_bytes = 0;
+  if (e->noalloc) e->schemas_dirty = e->api_dirty = e->coll_dirty = true; /* small tables live in the scratch array too */
   const uint64_t ng = e->generic.n, nr = e->runtime.n, nd = e->devrows.n, nx = e->extcorr.n, nu = e->usercorr.n;
   uint64_t N = ng + nr + nd; /* grows by the synthesised GPU user-annotation spans, at most one per device row */
   const uint64_t max_spans = nu ? nd : 0;
@@ -586,46 +661,46 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
 
   /* working memory */
   const uint32_t ns = (uint32_t)e->n_strings;
-  HIPCHK(e->d_name_len.ensure((ns + 1) * 4ull)); HIPCHK(e->d_arg_len.ensure((ns + 1) * 4ull));
-  HIPCHK(e->d_sflags.ensure((ns + 1) * 4ull));
-  HIPCHK(e->d_name_off.ensure((ns + 2) * 8ull)); HIPCHK(e->d_arg_off.ensure((ns + 2) * 8ull));
-  HIPCHK(e->d_name_blob.ensure(e->blob_bytes * 2 + 8ull * ns + 16)); HIPCHK(e->d_arg_blob.ensure(e->blob_bytes + 16));
-  HIPCHK(e->c_ts.ensure(Na * 8)); HIPCHK(e->c_dur.ensure(Na * 8)); HIPCHK(e->c_corr.ensure(Na * 8));
-  HIPCHK(e->c_dev.ensure(Na * 8)); HIPCHK(e->c_res.ensure(Na * 8)); HIPCHK(e->c_meta.ensure(Na * 4));
-  HIPCHK(e->c_ext.ensure(Na * 4));
+  NEED(e->d_name_len, (ns + 1) * 4ull); NEED(e->d_arg_len, (ns + 1) * 4ull);
+  NEED(e->d_sflags, (ns + 1) * 4ull);
+  NEED(e->d_name_off, (ns + 2) * 8ull); NEED(e->d_arg_off, (ns + 2) * 8ull);
+  NEED(e->d_name_blob, e->blob_bytes * 2 + 8ull * ns + 16); NEED(e->d_arg_blob, e->blob_bytes + 16);
+  NEED(e->c_ts, Na * 8); NEED(e->c_dur, Na * 8); NEED(e->c_corr, Na * 8);
+  NEED(e->c_dev, Na * 8); NEED(e->c_res, Na * 8); NEED(e->c_meta, Na * 4);
+  NEED(e->c_ext, Na * 4);
   if (nx >= 0x7FFFFFFFull || nr >= 0x7FFFFFFFull) { e->last_error = "more than 2^31 - 2 records of one class"; return KTJ_ERR_LIMIT; }
   /* capacities for the hash mode (load <= 2/3); the direct mode uses a prefix of the same buffers */
   const uint32_t cap_full = pow2_at_least((nr + nd) + (nr + nd) / 2);
   const uint32_t cap_narrow = pow2_at_least((nx + nr) + (nx + nr) / 2), cap_cpu = pow2_at_least(2 * ng);
-  HIPCHK(e->t_full.ensure((cap_full + 1ull) * 8)); HIPCHK(e->t_narrow.ensure((cap_narrow + 1ull) * 8));
-  HIPCHK(e->t_cpu.ensure((cap_cpu + 1ull) * 8));
-  HIPCHK(e->f_first.ensure((cap_full + 1ull) * 4)); HIPCHK(e->f_stream_src.ensure((cap_full + 1ull) * 4));
-  HIPCHK(e->f_pay.ensure((cap_full + 1ull) * sizeof(FullPay)));
-  HIPCHK(e->f_has_runtime.ensure((cap_full / 32 + 2ull) * 4));
-  HIPCHK(e->n_ext_src.ensure((cap_narrow + 1ull) * 4)); HIPCHK(e->n_kern_src.ensure((cap_narrow + 1ull) * 4));
-  HIPCHK(e->n_copy_src.ensure((cap_narrow + 1ull) * 4)); HIPCHK(e->n_pay.ensure((cap_narrow + 1ull) * sizeof(NarrowPay)));
-  HIPCHK(e->slot_ext.ensure(nx * 4 + 16)); HIPCHK(e->slot_f.ensure(nr * 4 + 16)); HIPCHK(e->slot_n.ensure(nr * 4 + 16));
-  HIPCHK(e->dev_link.ensure(nd * sizeof(DevLink) + 16));
-  HIPCHK(e->dev_brief.ensure(nd * sizeof(DevBrief) + 16));
-  HIPCHK(e->q_keys.ensure((KTJ_QUEUE_CAP + 1ull) * 8)); HIPCHK(e->q_stream.ensure((KTJ_QUEUE_CAP + 1ull) * 8));
-  HIPCHK(e->q_amb.ensure((KTJ_QUEUE_CAP + 1ull) * 4));
-  HIPCHK(e->dn_hash.ensure((KTJ_DENSE_CAP + 1ull) * 8)); HIPCHK(e->dn_first.ensure((KTJ_DENSE_CAP + 1ull) * 4));
-  HIPCHK(e->dn_dev.ensure((KTJ_DENSE_CAP + 1ull) * 4)); HIPCHK(e->dn_key.ensure((KTJ_DENSE_CAP + 1ull) * 8));
-  HIPCHK(e->dn_rank.ensure((KTJ_DENSE_CAP + 1ull) * 4));
-  HIPCHK(e->s_dev_k.ensure((KTJ_SET_CAP + 1ull) * 8)); HIPCHK(e->s_dev_r.ensure((KTJ_SET_CAP + 1ull) * 4));
-  HIPCHK(e->s_res_k.ensure((KTJ_SET_CAP + 1ull) * 8)); HIPCHK(e->s_res_r.ensure((KTJ_SET_CAP + 1ull) * 4));
-  HIPCHK(e->keys_a.ensure(Na * 8)); HIPCHK(e->keys_b.ensure(Na * 8));
-  HIPCHK(e->vals_a.ensure(Na * 4)); HIPCHK(e->vals_b.ensure(Na * 4));
-  HIPCHK(e->hist.ensure(radix_tmp_elems(Na) * 4));
+  NEED(e->t_full, (cap_full + 1ull) * 8); NEED(e->t_narrow, (cap_narrow + 1ull) * 8);
+  NEED(e->t_cpu, (cap_cpu + 1ull) * 8);
+  NEED(e->f_first, (cap_full + 1ull) * 4); NEED(e->f_stream_src, (cap_full + 1ull) * 4);
+  NEED(e->f_pay, (cap_full + 1ull) * sizeof(FullPay));
+  NEED(e->f_has_runtime, (cap_full / 32 + 2ull) * 4);
+  NEED(e->n_ext_src, (cap_narrow + 1ull) * 4); NEED(e->n_kern_src, (cap_narrow + 1ull) * 4);
+  NEED(e->n_copy_src, (cap_narrow + 1ull) * 4); NEED(e->n_pay, (cap_narrow + 1ull) * sizeof(NarrowPay));
+  NEED(e->slot_ext, nx * 4 + 16); NEED(e->slot_f, nr * 4 + 16); NEED(e->slot_n, nr * 4 + 16);
+  NEED(e->dev_link, nd * sizeof(DevLink) + 16);
+  NEED(e->dev_brief, nd * sizeof(DevBrief) + 16);
+  NEED(e->q_keys, (KTJ_QUEUE_CAP + 1ull) * 8); NEED(e->q_stream, (KTJ_QUEUE_CAP + 1ull) * 8);
+  NEED(e->q_amb, (KTJ_QUEUE_CAP + 1ull) * 4);
+  NEED(e->dn_hash, (KTJ_DENSE_CAP + 1ull) * 8); NEED(e->dn_first, (KTJ_DENSE_CAP + 1ull) * 4);
+  NEED(e->dn_dev, (KTJ_DENSE_CAP + 1ull) * 4); NEED(e->dn_key, (KTJ_DENSE_CAP + 1ull) * 8);
+  NEED(e->dn_rank, (KTJ_DENSE_CAP + 1ull) * 4);
+  NEED(e->s_dev_k, (KTJ_SET_CAP + 1ull) * 8); NEED(e->s_dev_r, (KTJ_SET_CAP + 1ull) * 4);
+  NEED(e->s_res_k, (KTJ_SET_CAP + 1ull) * 8); NEED(e->s_res_r, (KTJ_SET_CAP + 1ull) * 4);
+  NEED(e->keys_a, Na * 8); NEED(e->keys_b, Na * 8);
+  NEED(e->vals_a, Na * 4); NEED(e->vals_b, Na * 4);
+  NEED(e->hist, radix_tmp_elems(Na) * 4);
   {
     uint64_t m = scan_tmp_elems(radix_tmp_elems(Na));
     const uint64_t m2 = scan_tmp_elems(Na), m3 = scan_tmp_elems(ns + 1ull);
     if (m2 > m) m = m2;
     if (m3 > m) m = m3;
-    HIPCHK(e->scan_tmp.ensure(m * 8));
+    NEED(e->scan_tmp, m * 8);
   }
-  HIPCHK(e->mat.ensure(Na * sizeof(MatRow))); HIPCHK(e->len.ensure(Na * 4)); HIPCHK(e->len_sorted.ensure(Na * 4)); HIPCHK(e->kind_sorted.ensure(Na + 16));
-  HIPCHK(e->offs.ensure((Na + 1) * 8));
+  NEED(e->mat, Na * sizeof(MatRow)); NEED(e->len, Na * 4); NEED(e->len_sorted, Na * 4); NEED(e->kind_sorted, Na + 16);
+  NEED(e->offs, (Na + 1) * 8);
 
   Scalars* sc = e->d_scalars.as<Scalars>();
   Columns c;
@@ -665,11 +740,11 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   ctx.coll_blob = e->d_coll_blob.as<char>(); ctx.coll_off = e->d_coll_off.as<uint64_t>(); ctx.n_coll = n_coll;
   uint32_t* cpu_row = nullptr; /* last CPU op per id: only where something is read from that op */
   if (n_coll || max_spans) {
-    HIPCHK(e->cpu_row.ensure((cap_cpu + 1ull) * 4));
+    NEED(e->cpu_row, (cap_cpu + 1ull) * 4);
     cpu_row = e->cpu_row.as<uint32_t>();
     HIPCHK(fill_u32(cpu_row, 0, cap_cpu + 1ull, st));
   }
-  if (n_coll) HIPCHK(e->d_coll_first.ensure(2ull * n_coll * 4));
+  if (n_coll) NEED(e->d_coll_first, 2ull * n_coll * 4);
   if (ns) {
     HIPCHK(dict_measure(e->str_blob.buf.as<char>(), e->str_off.buf.as<uint64_t>(), ns, e->d_name_len.as<uint32_t>(),
                         e->d_arg_len.as<uint32_t>(), e->d_sflags.as<uint32_t>(), st));
@@ -734,8 +809,9 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(collect_distinct(c, N, sets, sc, st));
   HIPCHK(rank_distinct(sets, sc, st));
   HIPCHK(hipEventRecord(e->ev[EV_SORT_A], st));
-  HIPCHK(hipMemcpyAsync(&e->scalars, sc, sizeof(Scalars), hipMemcpyDeviceToHost, st));
+  HIPCHK(hipMemcpyAsync(&e->h_ctl->scalars, sc, sizeof(Scalars), hipMemcpyDeviceToHost, st));
   HIPCHK(hipStreamSynchronize(st));
+  e->scalars = e->h_ctl->scalars;
   if (e->scalars.error) {
     e->last_error = "device-side limit hit before sort, error bits " + std::to_string(e->scalars.error);
     return KTJ_ERR_LIMIT;
@@ -776,8 +852,8 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   /* ---- stage 4a: joined rows + lengths ---- */
   const uint32_t* sync_first = nullptr;
   if (e->scalars.n_sync_typed != 0) { /* known since the read-back before the sort */
-    HIPCHK(e->sync_keys.ensure((KTJ_SYNC_CAP + 1ull) * 8)); HIPCHK(e->sync_pos.ensure((KTJ_SYNC_CAP + 1ull) * 4));
-    HIPCHK(e->sync_first.ensure(ng * 4 + 16));
+    NEED(e->sync_keys, (KTJ_SYNC_CAP + 1ull) * 8); NEED(e->sync_pos, (KTJ_SYNC_CAP + 1ull) * 4);
+    NEED(e->sync_first, ng * 4 + 16);
     HIPCHK(stream_sync_first(e->perm, e->scalars.n_valid, g_recs, ng, ctx.dict, e->sync_keys.as<uint64_t>(),
                              e->sync_pos.as<uint32_t>(), e->sync_first.as<uint32_t>(), sc, st));
     sync_first = e->sync_first.as<uint32_t>();
@@ -794,11 +870,20 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(scan_u32_to_u64(e->len_sorted.as<uint32_t>(), e->offs.as<uint64_t>(), N, e->scan_tmp.as<uint64_t>(), st));
   HIPCHK(hipEventRecord(e->ev[EV_SCAN], st));
   uint64_t act_bytes = 0;
-  HIPCHK(hipMemcpyAsync(&act_bytes, e->offs.as<uint64_t>() + N, 8, hipMemcpyDeviceToHost, st));
-  HIPCHK(hipMemcpyAsync(&e->scalars, sc, sizeof(Scalars), hipMemcpyDeviceToHost, st));
+  HIPCHK(hipMemcpyAsync(&e->h_ctl->act_bytes, e->offs.as<uint64_t>() + N, 8, hipMemcpyDeviceToHost, st));
+  HIPCHK(hipMemcpyAsync(&e->h_ctl->scalars, sc, sizeof(Scalars), hipMemcpyDeviceToHost, st));
   e->coll_first.assign(2ull * n_coll, 0xFFFFFFFFu);
-  if (n_coll) HIPCHK(hipMemcpyAsync(e->coll_first.data(), e->d_coll_first.p, 2ull * n_coll * 4, hipMemcpyDeviceToHost, st));
+  if (n_coll && e->noalloc) { /* through the engine's pinned buffer */
+    if (2ull * n_coll * 4 > e->pinned_small_cap) {
+      e->last_error = "ktj_process_noalloc: too many collective entries for the pinned staging buffer";
+      return KTJ_ERR_LIMIT;
+    }
+    HIPCHK(hipMemcpyAsync(e->pinned_small, e->d_coll_first.p, 2ull * n_coll * 4, hipMemcpyDeviceToHost, st));
+  } else if (n_coll) HIPCHK(hipMemcpyAsync(e->coll_first.data(), e->d_coll_first.p, 2ull * n_coll * 4, hipMemcpyDeviceToHost, st));
   HIPCHK(hipStreamSynchronize(st));
+  if (n_coll && e->noalloc) memcpy(e->coll_first.data(), e->pinned_small, 2ull * n_coll * 4);
+  act_bytes = e->h_ctl->act_bytes;
+  e->scalars = e->h_ctl->scalars;
   if (e->scalars.error) {
     e->last_error = "device-side limit hit, error bits " + std::to_string(e->scalars.error);
     return KTJ_ERR_LIMIT;
@@ -821,8 +906,19 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   e->prefix_len = prefix.size();
   e->act_bytes = act_bytes;
   e->total_bytes = prefix.size() + act_bytes + suffix.size();
-  HIPCHK(e->out.ensure(e->total_bytes + 64));
+  if (out_device) { /* the caller's buffer: whole 16-byte blocks are stored, so a little room past the end is needed */
+    if (e->total_bytes + 64 > out_cap) {
+      e->last_error = "ktj_process_noalloc: the document has " + std::to_string(e->total_bytes) + " bytes and needs an output buffer of " +
+                      std::to_string(e->total_bytes + 64);
+      return KTJ_ERR_LIMIT;
+    }
+    e->out.borrow(out_device, out_cap);
+  } else NEED(e->out, e->total_bytes + 64);
   const size_t small = prefix.size() + suffix.size();
+  if (small > e->pinned_small_cap && e->noalloc) {
+    e->last_error = "ktj_process_noalloc: header and footer text of " + std::to_string(small) + " bytes exceeds the pinned staging buffer";
+    return KTJ_ERR_LIMIT;
+  }
   if (small > e->pinned_small_cap) {
     if (e->pinned_small) HIPCHK(hipHostFree(e->pinned_small));
     e->pinned_small = nullptr;
@@ -835,7 +931,7 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   HIPCHK(hipMemcpyAsync(e->out.as<char>() + prefix.size() + act_bytes, static_cast<char*>(e->pinned_small) + prefix.size(),
                         suffix.size(), hipMemcpyHostToDevice, st));
   const uint32_t tile = emit_tile_bytes(act_bytes, e->scalars.n_valid);
-  HIPCHK(e->tile_start.ensure((emit_tile_count(e->prefix_len, act_bytes, tile) + 2) * 4));
+  NEED(e->tile_start, (emit_tile_count(e->prefix_len, act_bytes, tile) + 2) * 4);
   HIPCHK(hipEventRecord(e->ev[EV_EMIT_START], st));
   {
     if (e->flags & KTJ_CREATE_TILE_EMIT)
@@ -892,6 +988,32 @@ int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   s.stage_bytes[KTJ_STAGE_EMIT] = e->scalars.n_valid * (sizeof(MatRow) + 12) + act_bytes;
   e->processed = true;
   return KTJ_OK;
+}
+
+int ktj_process(ktj_engine* e, int64_t end_time_ns) {
+  if (!e) return KTJ_ERR_ARG;
+  if (e->bad_sink) return KTJ_OK;
+  e->noalloc = false;
+  return process_pass(e, end_time_ns, nullptr, 0);
+}
+
+/* The pass with no allocation in it: working memory is this GPU's copy of the static scratch
+ * array, the document goes to the caller's buffer, small tables and read-backs go through the
+ * pinned buffers that ktj_create allocated. */
+int ktj_process_noalloc(ktj_engine* e, int64_t end_time_ns, void* out_device, uint64_t out_capacity, uint64_t* n_bytes) {
+  if (n_bytes) *n_bytes = 0;
+  if (!e || !out_device || ((uintptr_t)out_device & 15u) != 0) return KTJ_ERR_ARG;
+  if (e->bad_sink) return KTJ_OK;
+  if (!e->arena) { e->last_error = "ktj_process_noalloc: no scratch array on this device"; return KTJ_ERR_STATE; }
+  if (e->usercorr.n != 0) {
+    e->last_error = "ktj_process_noalloc: user-domain correlation records (GPU user annotations) are not supported here";
+    return KTJ_ERR_LIMIT;
+  }
+  e->noalloc = true;
+  const int rc = process_pass(e, end_time_ns, out_device, out_capacity);
+  e->noalloc = false;
+  if (n_bytes) *n_bytes = e->total_bytes; /* on KTJ_ERR_LIMIT for a short output buffer: the size that is needed */
+  return rc;
 }
 
 int ktj_output_device(ktj_engine* e, const void** device_ptr, uint64_t* n_bytes) {

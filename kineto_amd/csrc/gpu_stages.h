@@ -156,6 +156,11 @@ hipError_t fill_u32(uint32_t* p, uint32_t v, uint64_t n, hipStream_t st);
 hipError_t init_scalars(Scalars* s, hipStream_t st);
 hipError_t copy_reference(const void* src, void* dst, uint64_t bytes, hipStream_t st);
 
+/* Working memory for callers that cannot allocate: a static array in device memory, one copy per
+ * GPU, KTJ_NOALLOC_SCRATCH_BYTES long.  Returns the address of the copy on `device` (which must be
+ * the current device); the address is looked up once per device and kept. */
+hipError_t scratch_address(int device, void** ptr, size_t* bytes);
+
 /* exclusive scans; tmp must hold scan_tmp_elems(n) uint64 values */
 uint64_t scan_tmp_elems(uint64_t n);
 hipError_t scan_u32_to_u64(const uint32_t* in, uint64_t* out /* n+1 */, uint64_t n, uint64_t* tmp, hipStream_t st);

@@ -16,6 +16,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
+#include <mutex>
 
 #include "gpu_stages.h"
 
@@ -187,6 +188,32 @@ hipError_t fill_u32(uint32_t* p, uint32_t v, uint64_t n, hipStream_t st) {
 hipError_t init_scalars(Scalars* s, hipStream_t st) {
   hipLaunchKernelGGL(k_init_scalars, dim3(1), dim3(64), 0, st, s);
   return KTJ_LAUNCH_CHECK();
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* static scratch array: the working memory of ktj_process_noalloc.  Every GPU the library runs  */
+/* on holds its own copy, at its own address, until the process ends.  In host code the array's  */
+/* name is only a handle for hipGetSymbolAddress; everything else uses the looked-up address.    */
+/* ------------------------------------------------------------------------------------------ */
+static __device__ __align__(256) unsigned char scratch[KTJ_NOALLOC_SCRATCH_BYTES];
+#define KTJ_MAX_DEVICES 64
+static void* g_scratch_ptr[KTJ_MAX_DEVICES];
+static std::mutex g_scratch_lock;
+
+hipError_t scratch_address(int device, void** ptr, size_t* bytes) {
+  *ptr = nullptr;
+  *bytes = 0;
+  if (device < 0 || device >= KTJ_MAX_DEVICES) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    const hipError_t rc = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (rc != hipSuccess) return rc;
+    g_scratch_ptr[device] = p;
+  }
+  *ptr = g_scratch_ptr[device];
+  *bytes = KTJ_NOALLOC_SCRATCH_BYTES;
+  return hipSuccess;
 }
 
 /* ------------------------------------------------------------------------------------------ */
