@@ -228,14 +228,31 @@ enum {
   KTJ_F_STR = 4,   /* slot = string id, emitted in double quotes          (1 slot)            */
   KTJ_F_RAW = 5,   /* slot = string id, emitted verbatim (RawJson)        (1 slot)            */
   KTJ_F_I64_ARRAY = 6, /* [a, b, c] with `count` int64 elements           (count slots)       */
-  KTJ_F_COLLECTIVE = 7 /* slot = index from ktj_add_collective; keyless, recognised only as the
+  KTJ_F_COLLECTIVE = 7, /* slot = index from ktj_add_collective; keyless, recognised only as the
                           first field of a schema; prints nothing in the fragment (1 slot)    */
+  KTJ_F_STR_ARRAY = 8, /* ["a", "b"] with `count` quoted strings, slots = string ids
+                          (std::vector<std::string>, TypedMetadataJson.h:52-64) (count slots) */
+  KTJ_F_DICT_BEGIN = 9, /* "key": { — the fields up to the matching KTJ_F_DICT_END are the dict's
+                          children (beginDict, TypedMetadataJson.h:128-132); dicts nest (0 slots) */
+  KTJ_F_DICT_END = 10, /* } (endDict, TypedMetadataJson.h:134-137); keyless             (0 slots) */
+  KTJ_F_SHAPES = 11,   /* InputShapes ("Input Dims": [[2, 2], [[4, 1], [4, 1]]], TypedMetadata.h:
+                          39-47): the slot holds the index of the first slot of the value's
+                          encoding elsewhere in the args blob, see below              (1 slot) */
+  KTJ_F_UNSUPPORTED = 12 /* "key": "<unsupported metadata type>" (visitUnsupported,
+                          TypedMetadataJson.h:122-126)                                (0 slots) */
 };
+/* Encoding of a KTJ_F_SHAPES value in 8-byte slots: [n] then n entries; an entry is either
+ * [KTJ_SHAPE_TENSOR | rank][rank dims] (one tensor's shape, printed [d0, d1]) or
+ * [KTJ_SHAPE_LIST | m] followed by m times [rank][rank dims] (a TensorList argument, printed
+ * [[..], [..]]).  Dims are int64. */
+#define KTJ_SHAPE_TENSOR 0ull
+#define KTJ_SHAPE_LIST (1ull << 32)
 
 typedef struct ktj_field {
   uint32_t key_id; /* string id of the key; KTJ_NONE = the slot's string is a whole fragment   */
   uint16_t type;   /* KTJ_F_*                                                                 */
-  uint16_t count;  /* slots consumed (1 except for arrays)                                    */
+  uint16_t count;  /* slots consumed: 1, the element count of an array, 0 for dict brackets and
+                      KTJ_F_UNSUPPORTED                                                        */
 } ktj_field;
 
 #define KTJ_MAX_SCHEMA_FIELDS 1024
@@ -437,8 +454,20 @@ int ktj_submit_records_device(ktj_engine* e, int rec_class, const void* device_p
                               size_t n_records);
 
 /* handleDeviceInfo / handleResourceInfo / handleOverheadInfo / handleTraceSpan
- * (output_json.cpp:507-658).  Strings are copied. */
+ * (output_json.cpp:507-658).  Strings are copied.  ChromeTraceLogger writes each of these events
+ * where the call arrives, and libkineto calls arrive in two orders: the buffering logger's replay
+ * issues device and resource infos before the activities and spans after them
+ * (src/output_membuf.h:91-107), the profiler itself issues resource infos, device infos, GPU spans
+ * and overhead infos after the activities (src/GenericActivityProfiler.cpp:178-224, 655-740).  The
+ * engine keeps the activities in one sorted section and the other events on either side of it, in
+ * call order: what is submitted before the first activity goes in front of the section, what is
+ * submitted after it goes behind. */
 int ktj_submit_info(ktj_engine* e, int info_kind, const void* info);
+
+/* Tells the engine that the first activity has arrived (see ktj_submit_info).  Every record
+ * submission of an activity class does so by itself; a caller that batches its records and
+ * submits them later (like the ActivityLogger shim) calls this when it receives the first one. */
+int ktj_begin_activities(ktj_engine* e);
 
 /* Runs decode → convert → join → sort → size → scan → emit on the GPU and leaves the finished
  * document in a device buffer.  end_time_ns is finalizeTrace's endTime.  Idempotent inputs: may

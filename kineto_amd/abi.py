@@ -16,7 +16,8 @@ KTJ_CREATE_HASH_JOIN = 0x4
 
 REC_GENERIC, REC_RUNTIME, REC_DEVICE, REC_EXTCORR, REC_USERCORR = 0, 1, 2, 3, 4
 INFO_DEVICE, INFO_RESOURCE, INFO_OVERHEAD, INFO_SPAN = 0, 1, 2, 3
-F_I64, F_U64, F_F64, F_BOOL, F_STR, F_RAW, F_I64_ARRAY, F_COLLECTIVE = range(8)
+F_I64, F_U64, F_F64, F_BOOL, F_STR, F_RAW, F_I64_ARRAY, F_COLLECTIVE, F_STR_ARRAY, F_DICT_BEGIN, F_DICT_END, F_SHAPES, F_UNSUPPORTED = range(13)
+SHAPE_LIST = 1 << 32
 N_STAGES = 12
 STAGE_NAMES = ["dict", "decode", "convert", "join", "sort", "size", "scan", "emit", "d2h", "file",
                "total_gpu", "reserved"]
@@ -181,7 +182,7 @@ def load_synth():
 ENGINE_SYMBOLS = [
     "ktj_create", "ktj_destroy", "ktj_last_error", "ktj_trace_start", "ktj_intern_strings",
     "ktj_register_schema", "ktj_add_collective", "ktj_submit_args", "ktj_set_api_table", "ktj_set_clock_model",
-    "ktj_set_window", "ktj_submit_records", "ktj_submit_records_device", "ktj_submit_info",
+    "ktj_set_window", "ktj_submit_records", "ktj_submit_records_device", "ktj_submit_info", "ktj_begin_activities",
     "ktj_process", "ktj_process_noalloc", "ktj_output_device", "ktj_output_host", "ktj_finalize", "ktj_get_stats",
     "ktj_version",
     # include/ktj_rocprofiler.h
@@ -226,6 +227,8 @@ def load_engine():
         lib.ktj_submit_records.argtypes = [vp, C.c_int, C.c_void_p, C.c_size_t]
         lib.ktj_submit_records_device.restype = C.c_int
         lib.ktj_submit_records_device.argtypes = [vp, C.c_int, C.c_void_p, C.c_size_t]
+        lib.ktj_begin_activities.restype = C.c_int
+        lib.ktj_begin_activities.argtypes = [vp]
         lib.ktj_submit_info.restype = C.c_int
         lib.ktj_submit_info.argtypes = [vp, C.c_int, C.c_void_p]
         lib.ktj_set_sdk_agents.restype = C.c_int

@@ -126,7 +126,8 @@ struct ktj_engine {
   hipEvent_t ev_d2h[2] = {};
 
   /* inputs */
-  std::string txt_header, txt_dev, txt_res, txt_ovh, txt_span;
+  std::string txt_header, txt_before, txt_after; /* events in front of and behind the activity section, call order */
+  bool activities_begun = false;
   DevVec str_blob, str_off; /* str_off holds n_strings + 1 absolute offsets */
   uint64_t n_strings = 0, blob_bytes = 0;
   std::vector<ktj_field> fields;
@@ -442,8 +443,18 @@ int ktj_intern_strings(ktj_engine* e, const char* blob, const uint64_t* offsets,
 int ktj_register_schema(ktj_engine* e, const ktj_field* f, size_t n_fields, uint32_t* schema_id) {
   if (!e || (n_fields && !f)) return KTJ_ERR_ARG;
   if (n_fields > KTJ_MAX_SCHEMA_FIELDS) return KTJ_ERR_LIMIT;
-  for (size_t i = 0; i < n_fields; ++i)
-    if (f[i].type > KTJ_F_COLLECTIVE || f[i].count == 0 || (f[i].type != KTJ_F_I64_ARRAY && f[i].count != 1)) return KTJ_ERR_ARG;
+  int depth = 0;
+  for (size_t i = 0; i < n_fields; ++i) {
+    const uint16_t t = f[i].type;
+    if (t > KTJ_F_UNSUPPORTED) return KTJ_ERR_ARG;
+    const bool no_slots = t == KTJ_F_DICT_BEGIN || t == KTJ_F_DICT_END || t == KTJ_F_UNSUPPORTED;
+    const bool array = t == KTJ_F_I64_ARRAY || t == KTJ_F_STR_ARRAY;
+    if (no_slots ? f[i].count != 0 : array ? false : f[i].count != 1) return KTJ_ERR_ARG; /* arrays may be empty */
+    if ((t == KTJ_F_DICT_BEGIN || t == KTJ_F_UNSUPPORTED) && f[i].key_id == KTJ_NONE) return KTJ_ERR_ARG;
+    if (t == KTJ_F_DICT_BEGIN) ++depth;
+    if (t == KTJ_F_DICT_END && --depth < 0) return KTJ_ERR_ARG;
+  }
+  if (depth != 0) return KTJ_ERR_ARG; /* every dict is closed */
   if (n_fields && f[0].type == KTJ_F_COLLECTIVE) e->coll_schemas = true;
   ktj_schema_desc d;
   d.first_field = (uint32_t)e->fields.size();
@@ -527,6 +538,7 @@ int ktj_submit_records(ktj_engine* e, int rec_class, const void* packed, size_t 
   HIPCHK(hipSetDevice(e->device));
   HIPCHK(set->owned.append(packed, n_records * rs, e->stream));
   set->n += n_records;
+  if (rec_class == KTJ_REC_GENERIC || rec_class == KTJ_REC_RUNTIME || rec_class == KTJ_REC_DEVICE) e->activities_begun = true;
   e->processed = false;
   return KTJ_OK;
 }
@@ -541,6 +553,7 @@ int ktj_submit_records_device(ktj_engine* e, int rec_class, const void* device_p
   if (set->owned.bytes != 0) return KTJ_ERR_STATE;
   set->external = n_records ? device_ptr : nullptr;
   set->n = n_records;
+  if (n_records && (rec_class == KTJ_REC_GENERIC || rec_class == KTJ_REC_RUNTIME || rec_class == KTJ_REC_DEVICE)) e->activities_begun = true;
   e->processed = false;
   return KTJ_OK;
 }
@@ -608,14 +621,21 @@ int ktj_submit_sdk_buffer(ktj_engine* e, void* const* headers, size_t num_header
   return ktj_submit_records(e, KTJ_REC_DEVICE, rows.data(), rows.size());
 }
 
+int ktj_begin_activities(ktj_engine* e) {
+  if (!e) return KTJ_ERR_ARG;
+  e->activities_begun = true;
+  return KTJ_OK;
+}
+
 int ktj_submit_info(ktj_engine* e, int info_kind, const void* info) {
   if (!e || !info) return KTJ_ERR_ARG;
   if (e->bad_sink) return KTJ_OK;
+  std::string& txt = e->activities_begun ? e->txt_after : e->txt_before;
   switch (info_kind) {
-    case KTJ_INFO_DEVICE: append_device_info(e->txt_dev, *static_cast<const ktj_device_info*>(info), e->base_time_ns); break;
-    case KTJ_INFO_RESOURCE: append_resource_info(e->txt_res, *static_cast<const ktj_resource_info*>(info), e->base_time_ns); break;
-    case KTJ_INFO_OVERHEAD: append_overhead_info(e->txt_ovh, *static_cast<const ktj_overhead_info*>(info), e->base_time_ns); break;
-    case KTJ_INFO_SPAN: append_trace_span(e->txt_span, *static_cast<const ktj_trace_span*>(info), e->base_time_ns); break;
+    case KTJ_INFO_DEVICE: append_device_info(txt, *static_cast<const ktj_device_info*>(info), e->base_time_ns); break;
+    case KTJ_INFO_RESOURCE: append_resource_info(txt, *static_cast<const ktj_resource_info*>(info), e->base_time_ns); break;
+    case KTJ_INFO_OVERHEAD: append_overhead_info(txt, *static_cast<const ktj_overhead_info*>(info), e->base_time_ns); break;
+    case KTJ_INFO_SPAN: append_trace_span(txt, *static_cast<const ktj_trace_span*>(info), e->base_time_ns); break;
     default: return KTJ_ERR_ARG;
   }
   e->processed = false;
@@ -900,8 +920,8 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   }
 
   /* ---- emit ---- */
-  std::string prefix = e->txt_header + e->txt_dev + e->txt_res + e->txt_ovh;
-  std::string suffix = e->txt_span;
+  std::string prefix = e->txt_header + e->txt_before;
+  std::string suffix = e->txt_after;
   append_trace_end(suffix, end_time_ns, e->base_time_ns, e->out_path, distributed_info);
   e->prefix_len = prefix.size();
   e->act_bytes = act_bytes;

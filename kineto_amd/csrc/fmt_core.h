@@ -420,6 +420,15 @@ static __device__ __attribute__((noinline)) void cooperative_word_copy(const cha
 }
 #endif
 
+#if defined(__HIPCC__)
+/* blocks per lane in the stage; odd, so that neither the lanes' writes (same block index, lane
+ * stride 16 * KTJ_STAGE_BLOCKS bytes) nor the quads' reads collide on LDS banks */
+#define KTJ_STAGE_BLOCKS 11u
+#define KTJ_FLUSH_LANES 4u
+#define KTJ_FLUSH_ROUNDS ((KTJ_STAGE_BLOCKS + 2u * KTJ_FLUSH_LANES - 2u) / KTJ_FLUSH_LANES) /* blocks plus up to LANES - 1 of misalignment */
+extern __shared__ __attribute__((aligned(16))) char ktj_stage_lds[];
+#endif
+
 /* Pass B: one lane formats one activity straight into the document in device memory.  Bytes are
  * gathered in a 128-bit accumulator and leave as aligned 16-byte stores; literal text is appended
  * sixteen bytes at a time, so that all lanes of a wavefront complete a block at the same append
@@ -437,6 +446,17 @@ struct BlockWriter {
   uint64_t lo, hi;    /* its first `fill` bytes */
   uint32_t fill;      /* 0..15 */
   bool foreign;       /* the block belongs to the predecessor: gathered but not stored */
+#if defined(__HIPCC__)
+  /* Device: finished blocks do not go to the document one by one (64 lanes, 64 different lines per
+   * store instruction) but wait in LDS, up to KTJ_STAGE_BLOCKS consecutive blocks per lane, until
+   * the wavefront reaches flush(): there the four lanes of a quad write each other's blocks, four
+   * consecutive blocks of one activity per store instruction (64 contiguous bytes).  Blocks
+   * beyond the stage's capacity, and blocks after a jump of wptr, are stored directly. */
+  uint32_t stage_lds;   /* byte offset of this lane's stage in the workgroup's dynamic LDS */
+  uint32_t n_staged;    /* blocks waiting; staged block j belongs at stage_base + 2 j */
+  uint32_t stage_cap;   /* KTJ_STAGE_BLOCKS, or n_staged once the stage is closed until the next flush */
+  uint64_t* stage_base;
+#endif
 
   KTJ_HD KTJ_FI static uint64_t head_bytes() { constexpr auto h = pack_lit("\n  {\n   "); return h.w[0]; }
   KTJ_HD KTJ_FI void store_block() {
@@ -444,7 +464,11 @@ struct BlockWriter {
 #if defined(__HIP_DEVICE_COMPILE__)
       typedef unsigned long long v2u64 __attribute__((ext_vector_type(2)));
       v2u64 v; v.x = lo; v.y = hi;
-      *reinterpret_cast<v2u64*>(wptr) = v;
+      if (n_staged < stage_cap) {
+        if (n_staged == 0) stage_base = wptr;
+        *reinterpret_cast<v2u64*>(ktj_stage_lds + stage_lds + n_staged * 16u) = v;
+        ++n_staged;
+      } else *reinterpret_cast<v2u64*>(wptr) = v;
 #else
       wptr[0] = lo; wptr[1] = hi;
 #endif
@@ -452,6 +476,55 @@ struct BlockWriter {
     foreign = false;
     wptr += 2;
   }
+#if defined(__HIPCC__)
+  __device__ KTJ_FI void stage_init(uint32_t lds_offset) {
+    stage_lds = lds_offset; n_staged = 0; stage_cap = KTJ_STAGE_BLOCKS; stage_base = nullptr;
+    wptr = nullptr; lo = hi = 0; fill = 0; foreign = false;
+  }
+  /* wptr is about to move by more than one block: what is staged stays, nothing more is staged */
+  __device__ KTJ_FI void stage_close() { stage_cap = n_staged; }
+  /* Every lane of the wavefront must call this together (lanes without an activity included). */
+  __device__ KTJ_FI void flush() {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef unsigned long long v2u64 __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(1))) v2u64* gptr; /* the document is global memory: no flat stores */
+    const uint32_t k = (uint32_t)threadIdx.x & 3u;
+    const uint32_t base_lo = (uint32_t)(uintptr_t)stage_base, base_hi = (uint32_t)((uintptr_t)stage_base >> 32);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#define KTJ_QUAD_BCAST(v, t) ((uint32_t)__builtin_amdgcn_mov_dpp((int)(v), (t) * 0x55, 0xF, 0xF, true))
+#define KTJ_FLUSH_FROM(t)                                                                       \
+    {                                                                                           \
+      const uint32_t n_s = KTJ_QUAD_BCAST(n_staged, t);                                         \
+      const uint32_t lds_s = KTJ_QUAD_BCAST(stage_lds, t);                                      \
+      const uint32_t lo_s = KTJ_QUAD_BCAST(base_lo, t);                                         \
+      gptr d = reinterpret_cast<gptr>(((uintptr_t)KTJ_QUAD_BCAST(base_hi, t) << 32) | (uintptr_t)lo_s); \
+      /* lane k takes the blocks whose index in the document is k mod 4: a store instruction     \
+       * then covers one aligned 64-byte piece of the activity */                                \
+      const int32_t j0 = (int32_t)k - (int32_t)((lo_s >> 4) & 3u);                              \
+      v2u64 x[KTJ_FLUSH_ROUNDS];                                                                \
+      _Pragma("unroll")                                                                         \
+      for (uint32_t m = 0; m < KTJ_FLUSH_ROUNDS; ++m) { /* all reads first: one wait for them */ \
+        const int32_t j = j0 + (int32_t)(KTJ_FLUSH_LANES * m);                                  \
+        x[m] = *reinterpret_cast<const v2u64*>(ktj_stage_lds + lds_s + ((uint32_t)j < KTJ_STAGE_BLOCKS ? (uint32_t)j : 0u) * 16u); \
+      }                                                                                         \
+      _Pragma("unroll")                                                                         \
+      for (uint32_t m = 0; m < KTJ_FLUSH_ROUNDS; ++m) {                                         \
+        const int32_t j = j0 + (int32_t)(KTJ_FLUSH_LANES * m);                                  \
+        if ((uint32_t)j < n_s) d[j] = x[m];                                                     \
+      }                                                                                         \
+    }
+    KTJ_FLUSH_FROM(0) KTJ_FLUSH_FROM(1) KTJ_FLUSH_FROM(2) KTJ_FLUSH_FROM(3)
+#undef KTJ_FLUSH_FROM
+#undef KTJ_QUAD_BCAST
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    n_staged = 0;
+    stage_cap = KTJ_STAGE_BLOCKS;
+#endif
+  }
+#endif
   /* pos: where the activity starts; tail_kind_before: kind of the activity before it */
   KTJ_HD KTJ_FI void begin(char* doc, uint64_t pos, uint32_t tail_kind_before, bool first);
   KTJ_HD KTJ_FI void end(bool last);
@@ -563,6 +636,7 @@ struct BlockWriter {
         n_words = (uint32_t)((len - head) >> 4) * 2u; /* whole blocks, as words */
         tail = (len - head) & 15u;
         dst = wptr;
+        stage_close();
         wptr += n_words;
       } else str_own(src, len);
       cooperative_word_copy(body, dst, n_words);
@@ -860,6 +934,42 @@ KTJ_HD KTJ_FI inline uint32_t collective_for_linked(const ktj_generic_rec& g, co
   return k < c.n_coll ? (uint32_t)k + 1u : 0u;
 }
 
+/* one shape of `rank` dims at slot p: [d0, d1] */
+template <class W> KTJ_HD KTJ_FI inline uint64_t put_shape(W& w, const EmitCtx& c, uint64_t p, uint64_t rank) {
+  w.ch('[');
+  KTJ_NOUNROLL
+  for (uint64_t k = 0; k < rank; ++k) {
+    if (k) KTJ_PUT(w, ", ");
+    put_i64(w, (int64_t)(p + k < c.n_args ? c.args[p + k] : 0));
+  }
+  w.ch(']');
+  return p + rank;
+}
+/* InputShapes through appendArray (TypedMetadataJson.h:52-64, 186-201); the encoding is described
+ * at KTJ_F_SHAPES.  Counts are clipped to the blob, so a damaged encoding cannot run away. */
+template <class W> KTJ_HD KTJ_FI inline void put_shapes(W& w, const EmitCtx& c, uint64_t p) {
+  const uint64_t n = p < c.n_args ? c.args[p] : 0;
+  ++p;
+  w.ch('[');
+  KTJ_NOUNROLL
+  for (uint64_t e = 0; e < n && p < c.n_args; ++e) {
+    if (e) KTJ_PUT(w, ", ");
+    const uint64_t head = c.args[p++];
+    const uint64_t m = head & 0xFFFFFFFFull;
+    if (head & KTJ_SHAPE_LIST) {
+      w.ch('[');
+      KTJ_NOUNROLL
+      for (uint64_t t = 0; t < m && p < c.n_args; ++t) {
+        if (t) KTJ_PUT(w, ", ");
+        const uint64_t rank = c.args[p++] & 0xFFFFFFFFull;
+        p = put_shape(w, c, p, rank);
+      }
+      w.ch(']');
+    } else p = put_shape(w, c, p, m);
+  }
+  w.ch(']');
+}
+
 /* the metadataJson() fragment, after sanitizeStrForJSON (raw: as metadataJson() returned it) */
 template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r, const EmitCtx& c, bool raw = false) {
   const uint32_t cls = (r.meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT;
@@ -871,13 +981,25 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
     for (uint32_t f = 0; f < sd.n_fields; ++f) {
       const ktj_field fd = c.fields[sd.first_field + f];
       if (fd.type == KTJ_F_COLLECTIVE) { slot += fd.count; continue; }
-      if (fd.key_id != KTJ_NONE) {
+      if (fd.key_id != KTJ_NONE) { /* appendKey, TypedMetadataJson.h:145-152 */
         if (!first) KTJ_PUT(w, ", ");
         first = false;
         w.ch('"'); put_arg_string(w, c.dict, fd.key_id, raw); KTJ_PUT(w, "\": ");
       }
       const uint64_t v = slot < c.n_args ? c.args[slot] : 0;
       switch (fd.type) {
+        case KTJ_F_DICT_BEGIN: w.ch('{'); first = true; break;   /* beginDict :128-132 */
+        case KTJ_F_DICT_END: w.ch('}'); first = false; break;    /* endDict :134-137 */
+        case KTJ_F_UNSUPPORTED: KTJ_PUT(w, "\"<unsupported metadata type>\""); break;
+        case KTJ_F_STR_ARRAY:
+          w.ch('[');
+          for (uint32_t k = 0; k < fd.count; ++k) {
+            if (k) KTJ_PUT(w, ", ");
+            w.ch('"'); put_arg_string(w, c.dict, (uint32_t)(slot + k < c.n_args ? c.args[slot + k] : KTJ_NONE), raw); w.ch('"');
+          }
+          w.ch(']');
+          break;
+        case KTJ_F_SHAPES: put_shapes(w, c, v); break;
         case KTJ_F_I64: put_i64(w, (int64_t)v); break;
         case KTJ_F_U64: w.dec(v); break;
         case KTJ_F_F64: put_f64(w, v); break;
@@ -1077,13 +1199,26 @@ template <class W> KTJ_HD KTJ_FI inline void format_counter(W& w, const MatRow& 
   if (!hw) KTJ_PUT(w, "\n    }\n  },");
 }
 
-/* One activity: the complete event and, if it takes part in a flow, the flow event after it. */
-template <class W> KTJ_HD KTJ_FI inline void format_activity(W& w, const MatRow& r, const EmitCtx& c) {
+/* One activity: the complete event and, if it takes part in a flow, the flow event after it.
+ * Formatting comes in three parts that run one after the other — head (everything up to "dur", or
+ * the whole event for instant and counter events), args, flow event — so that the emit kernel can
+ * let the wavefront hand over finished blocks between them (BlockWriter::flush). */
+template <class W> struct ActivityParts {
+  typename W::Prepared pid, tidn;  /* printed by the complete event and again by the flow event */
+  bool pid_neg;
+  bool complete;                   /* a complete event: args and flow parts follow the head */
+};
+template <class W> KTJ_HD KTJ_FI inline void format_head(W& w, const MatRow& r, const EmitCtx& c, ActivityParts<W>& st) {
   const uint32_t type = r.meta & KTJ_M_TYPE_MASK;
+  st.complete = false;
+  st.pid_neg = false;
+  st.pid = W::prepare(0);
+  st.tidn = st.pid;
   if (((r.meta & KTJ_M_CLASS_MASK) >> KTJ_M_CLASS_SHIFT) == KTJ_CLASS_GENERIC) {
     if (type == KTJ_TYPE_CPU_INSTANT_EVENT) { format_instant(w, r, c); return; }
     if (is_counter_type(type)) { format_counter(w, r, c); return; }
   }
+  st.complete = true;
   int64_t ts = r.ts;
   int64_t dur = r.dur < 0 ? 0 : r.dur;                       /* output_json.cpp:860 */
   if (type == KTJ_TYPE_GPU_USER_ANNOTATION) { ts -= 1; dur += 2; } /* :862-869 */
@@ -1091,11 +1226,9 @@ template <class W> KTJ_HD KTJ_FI inline void format_activity(W& w, const MatRow&
   if (rel < 0) rel = 0;
   /* Stream Sync activities sit on a row of their own (output_json.cpp:913-943, 1008-1013) */
   const int64_t tid = sanitize_tid((r.meta & KTJ_M_SYNC) ? sync_row_tid(r.res) : r.res);
-  const bool flow = (r.meta & KTJ_M_FLOW) != 0;
-  /* pid and tid are printed again by the flow event */
-  const bool pid_neg = r.dev < 0;
-  const typename W::Prepared pid = W::prepare(pid_neg ? 0ULL - (uint64_t)r.dev : (uint64_t)r.dev);
-  const typename W::Prepared tidn = W::prepare((uint64_t)tid);
+  st.pid_neg = r.dev < 0;
+  st.pid = W::prepare(st.pid_neg ? 0ULL - (uint64_t)r.dev : (uint64_t)r.dev);
+  st.tidn = W::prepare((uint64_t)tid);
   if (r.meta & KTJ_M_SYNC_FIRST) { /* the row is announced once, before its first activity */
     KTJ_PUT(w, "\n  {\n    \"name\": \"thread_name\", \"ph\": \"M\", \"ts\": "); put_ts(w, rel);
     KTJ_PUT(w, ", \"pid\": "); put_i64(w, r.dev); KTJ_PUT(w, ", \"tid\": "); put_i64(w, sync_row_tid(r.res));
@@ -1108,10 +1241,13 @@ template <class W> KTJ_HD KTJ_FI inline void format_activity(W& w, const MatRow&
   put_category(w, type);
   KTJ_PUT(w, "\",\n    \"name\": \"");
   put_name(w, r, c);
-  KTJ_PUT(w, "\",\n    \"pid\": "); if (pid_neg) w.ch('-'); w.num(pid);
-  KTJ_PUT(w, ",\n    \"tid\": "); w.num(tidn);
+  KTJ_PUT(w, "\",\n    \"pid\": "); if (st.pid_neg) w.ch('-'); w.num(st.pid);
+  KTJ_PUT(w, ",\n    \"tid\": "); w.num(st.tidn);
   KTJ_PUT(w, ",\n    \"ts\": "); put_ts(w, rel);
   KTJ_PUT(w, ",\n    \"dur\": "); put_ts(w, dur);
+}
+template <class W> KTJ_HD KTJ_FI inline void format_args(W& w, const MatRow& r, const EmitCtx& c, const ActivityParts<W>& st) {
+  if (!st.complete) return;
   const bool frag = has_fragment(r, c);
   const bool coll = has_collective_args(r, c);
   if (r.ext != 0 || frag || coll) {                          /* ArgsBuilder :157-212 */
@@ -1125,19 +1261,26 @@ template <class W> KTJ_HD KTJ_FI inline void format_activity(W& w, const MatRow&
     }
     KTJ_PUT(w, "\n    }\n  },");
   } else KTJ_PUT(w, "\n    \n  },");
-  if (flow) {                                                /* :960-1021, writeFlowEvent :318-345 */
-    int64_t frel = r.ts - c.base_time_ns;
-    if (frel < 0) frel = 0;
-    if (r.meta & KTJ_M_FLOW_START) KTJ_PUT(w, "\n  {\n    \"ph\": \"s\",\n    \"id\": ");
-    else KTJ_PUT(w, "\n  {\n    \"ph\": \"f\",\n    \"id\": ");
-    put_i64(w, r.flow_id);
-    KTJ_PUT(w, ",\n    \"pid\": "); if (pid_neg) w.ch('-'); w.num(pid);
-    KTJ_PUT(w, ",\n    \"tid\": "); w.num(tidn);
-    KTJ_PUT(w, ",\n    \"ts\": "); put_ts(w, frel);
-    if (r.meta & KTJ_M_FLOW_FWDBWD) KTJ_PUT(w, ",\n    \"cat\": \"fwdbwd\",\n    \"name\": \"fwdbwd\"\n    ");
-    else KTJ_PUT(w, ",\n    \"cat\": \"ac2g\",\n    \"name\": \"ac2g\"\n    ");
-    if (r.meta & KTJ_M_FLOW_START) KTJ_PUT(w, "\n  },"); else KTJ_PUT(w, ", \"bp\": \"e\"\n  },");
-  }
+}
+template <class W> KTJ_HD KTJ_FI inline void format_flow(W& w, const MatRow& r, const EmitCtx& c, const ActivityParts<W>& st) {
+  if (!st.complete || !(r.meta & KTJ_M_FLOW)) return;       /* :960-1021, writeFlowEvent :318-345 */
+  int64_t frel = r.ts - c.base_time_ns;
+  if (frel < 0) frel = 0;
+  if (r.meta & KTJ_M_FLOW_START) KTJ_PUT(w, "\n  {\n    \"ph\": \"s\",\n    \"id\": ");
+  else KTJ_PUT(w, "\n  {\n    \"ph\": \"f\",\n    \"id\": ");
+  put_i64(w, r.flow_id);
+  KTJ_PUT(w, ",\n    \"pid\": "); if (st.pid_neg) w.ch('-'); w.num(st.pid);
+  KTJ_PUT(w, ",\n    \"tid\": "); w.num(st.tidn);
+  KTJ_PUT(w, ",\n    \"ts\": "); put_ts(w, frel);
+  if (r.meta & KTJ_M_FLOW_FWDBWD) KTJ_PUT(w, ",\n    \"cat\": \"fwdbwd\",\n    \"name\": \"fwdbwd\"\n    ");
+  else KTJ_PUT(w, ",\n    \"cat\": \"ac2g\",\n    \"name\": \"ac2g\"\n    ");
+  if (r.meta & KTJ_M_FLOW_START) KTJ_PUT(w, "\n  },"); else KTJ_PUT(w, ", \"bp\": \"e\"\n  },");
+}
+template <class W> KTJ_HD KTJ_FI inline void format_activity(W& w, const MatRow& r, const EmitCtx& c) {
+  ActivityParts<W> st;
+  format_head(w, r, c, st);
+  format_args(w, r, c, st);
+  format_flow(w, r, c, st);
 }
 
 }  // namespace ktj

@@ -1801,35 +1801,44 @@ k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n
   for (uint32_t k = pre + body * 16u + threadIdx.x; k < nbytes; k += EMIT_THREADS) g[k] = s[k];
 }
 
-/* Direct variant: one lane per activity, aligned 16-byte stores straight into the document, no
- * LDS (see BlockWriter for who writes the blocks that two activities share).  The document's
- * prefix and suffix are already in place when this kernel runs; the first and the last activity
- * merge with them. */
+/* Direct variant: one lane per activity; blocks of 16 bytes, aligned in the document (see
+ * BlockWriter for who writes the blocks that two activities share).  Finished blocks wait in LDS
+ * and leave at the three points where the whole wavefront meets: after the head of the event,
+ * after its args and after the flow event; there four neighbouring lanes store four consecutive
+ * blocks of one activity at a time.  Lanes without an activity stay until the end for that.  The
+ * document's prefix and suffix are already in place when this kernel runs; the first and the last
+ * activity merge with them. */
 __global__ void __launch_bounds__(KTJ_BLOCK) __attribute__((amdgpu_waves_per_eu(3)))
 k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint8_t* kind_sorted, uint64_t n_rows,
               EmitCtx ctx, char* out, uint64_t prefix_len) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n_rows) return;
-  const uint64_t o = offs[i];
-  if (offs[i + 1] == o) return;
-  const MatRow m = mat[perm[i]];
+  uint64_t o = 0;
+  bool active = i < n_rows;
+  if (active) { o = offs[i]; active = offs[i + 1] != o; }
+  MatRow m;
   BlockWriter w;
-  w.begin(out, prefix_len + o, i ? kind_sorted[i - 1] : 0u, i == 0);
-  format_activity(w, m, ctx);
-  w.end(i + 1 == n_rows);
+  w.stage_init((uint32_t)threadIdx.x * (KTJ_STAGE_BLOCKS * 16u));
+  ActivityParts<BlockWriter> parts;
+  if (active) {
+    m = mat[perm[i]];
+    w.begin(out, prefix_len + o, i ? kind_sorted[i - 1] : 0u, i == 0);
+    format_head(w, m, ctx, parts);
+  }
+  w.flush();
+  if (active) format_args(w, m, ctx, parts);
+  w.flush();
+  if (active) {
+    format_flow(w, m, ctx, parts);
+    w.end(i + 1 == n_rows);
+  }
+  w.flush();
 }
 hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint8_t* kind_sorted,
                        uint64_t n_rows, uint64_t act_bytes, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st) {
   if (n_rows == 0) return hipSuccess;
-  /* Every lane keeps one partially written 128-byte line open at a time.  At full occupancy
-   * (2048 lanes per CU, 256 CUs) those lines exceed the L2 capacity and are evicted half-filled,
-   * which doubles the HBM writes.  Unused dynamic LDS caps residency at two workgroups per CU
-   * (8 waves), so the open lines stay in L2 until complete; measured 15-20% faster than
-   * unrestricted residency where activities are short.  Where most bytes are long dictionary
-   * strings, which the lanes copy together as whole lines, the cap only costs parallelism
-   * (measured 13% slower at 1.4 KB per activity), so it is applied below 768 bytes per activity. */
-  const size_t residency_lds = act_bytes / n_rows < 768 ? 60000 : 0;
-  hipLaunchKernelGGL(k_emit_direct, dim3(grid_for(n_rows, KTJ_BLOCK)), dim3(KTJ_BLOCK), residency_lds, st, mat, perm, offs,
+  (void)act_bytes;
+  const size_t stage_lds = (size_t)KTJ_BLOCK * KTJ_STAGE_BLOCKS * 16u;
+  hipLaunchKernelGGL(k_emit_direct, dim3(grid_for(n_rows, KTJ_BLOCK)), dim3(KTJ_BLOCK), stage_lds, st, mat, perm, offs,
                      kind_sorted, n_rows, ctx, out, prefix_len);
   return KTJ_LAUNCH_CHECK();
 }

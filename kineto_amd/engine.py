@@ -58,17 +58,21 @@ class TraceEngine:
                   "ktj_set_api_table")
         self._chk(lib.ktj_set_clock_model(h, C.byref(s.clock)), "ktj_set_clock_model")
         self._chk(lib.ktj_set_window(h, s.window_start_ns, s.window_end_ns), "ktj_set_window")
+        # call order of the buffering logger's replay (libkineto/src/output_membuf.h:91-107): device
+        # and resource infos, the activities, then the spans
+        for kind, ptr, n in ((abi.INFO_DEVICE, s.device_infos, s.n_device_infos),
+                             (abi.INFO_RESOURCE, s.resource_infos, s.n_resource_infos),
+                             (abi.INFO_OVERHEAD, s.overhead_infos, s.n_overhead_infos)):
+            for i in range(n):
+                self._chk(lib.ktj_submit_info(h, kind, C.byref(ptr[i])), "ktj_submit_info")
+        self._chk(lib.ktj_begin_activities(h), "ktj_begin_activities")
         for cls, ptr, n in ((abi.REC_GENERIC, s.generic, s.n_generic), (abi.REC_RUNTIME, s.runtime, s.n_runtime),
                             (abi.REC_DEVICE, s.device, s.n_device), (abi.REC_EXTCORR, s.extcorr, s.n_extcorr),
                             (abi.REC_USERCORR, s.usercorr, s.n_usercorr)):
             if n:
                 self._chk(lib.ktj_submit_records(h, cls, C.cast(ptr, C.c_void_p), n), "ktj_submit_records")
-        for kind, ptr, n in ((abi.INFO_DEVICE, s.device_infos, s.n_device_infos),
-                             (abi.INFO_RESOURCE, s.resource_infos, s.n_resource_infos),
-                             (abi.INFO_OVERHEAD, s.overhead_infos, s.n_overhead_infos),
-                             (abi.INFO_SPAN, s.spans, s.n_spans)):
-            for i in range(n):
-                self._chk(lib.ktj_submit_info(h, kind, C.byref(ptr[i])), "ktj_submit_info")
+        for i in range(s.n_spans):
+            self._chk(lib.ktj_submit_info(h, abi.INFO_SPAN, C.byref(s.spans[i])), "ktj_submit_info")
         self.end_time_ns = s.end_time_ns
 
     def process(self, end_time_ns=None):

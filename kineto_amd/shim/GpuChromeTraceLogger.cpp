@@ -381,8 +381,18 @@ void GpuChromeTraceLogger::handleTraceSpan(const TraceSpan& span) {
   note(ktj_submit_info(engine_, KTJ_INFO_SPAN, &s), "ktj_submit_info(span)");
 }
 
+/* The records are batched and reach the engine later; the engine is told now that the activities
+ * have begun, so that infos and spans that follow go behind the activity section, as they do in
+ * the reference logger's file when it is driven by GenericActivityProfiler::processTraceInternal. */
+void GpuChromeTraceLogger::noteFirstActivity() {
+  if (activitiesBegun_) return;
+  activitiesBegun_ = true;
+  note(ktj_begin_activities(engine_), "ktj_begin_activities");
+}
+
 void GpuChromeTraceLogger::handleActivity(const ITraceActivity& op) {
   if (!ok()) return;
+  noteFirstActivity();
   pack(op, 0, *staging_);
   if (staging_->records.size() >= kRecordBatch) mergeInOrder(*staging_);
 }
@@ -396,6 +406,7 @@ void GpuChromeTraceLogger::handleActivity(const ITraceActivity& op) {
  * one thread and in sequence.  The records reach the engine in the order of `activities`. */
 void GpuChromeTraceLogger::handleActivities(const std::vector<const ITraceActivity*>& activities, unsigned threads) {
   if (!ok() || activities.empty()) return;
+  noteFirstActivity();
   mergeInOrder(*staging_); /* what single calls left behind comes first */
   const size_t n = activities.size();
   if (threads == 0) threads = std::max(1u, std::thread::hardware_concurrency());

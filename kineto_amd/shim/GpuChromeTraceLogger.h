@@ -77,10 +77,12 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
   void flushRecords();
   bool ok() const { return engine_ != nullptr && status_ == 0; }
   void note(int rc, const char* what);
+  void noteFirstActivity();
 
   ktj_engine* engine_ = nullptr;
   std::string fileName_;
   int status_ = 0;
+  bool activitiesBegun_ = false;
   uint64_t unsupported_ = 0;
   uint32_t fragmentSchema_ = KTJ_NONE;
   uint32_t collectiveSchema_ = KTJ_NONE;         /* collective metadata only        */

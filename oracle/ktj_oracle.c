@@ -409,6 +409,20 @@ static void visit(ktj_oracle* o, ktj_mat_activity* a, uint32_t key_id, uint16_t 
   o->n_spool += count;
   a->n_fields++;
 }
+/* slots of one KTJ_F_SHAPES value that starts at args[at] (see include/ktj.h), clipped to the blob
+ * and to what a field's 16-bit count can say */
+static uint64_t shapes_encoded_slots(const uint64_t* args, uint64_t n_args, uint64_t at) {
+  if (at >= n_args) return 0;
+  uint64_t p = at + 1;
+  for (uint64_t e = 0; e < args[at] && p < n_args; ++e) {
+    const uint64_t head = args[p++], m = head & 0xFFFFFFFFull;
+    if (head & KTJ_SHAPE_LIST) {
+      for (uint64_t t = 0; t < m && p < n_args; ++t) p += 1 + (args[p] & 0xFFFFFFFFull);
+    } else p += m;
+  }
+  if (p > n_args) p = n_args;
+  return p - at > 65535 ? 65535 : p - at;
+}
 static void visit1(ktj_oracle* o, ktj_mat_activity* a, int builtin_key, uint16_t type, uint64_t v) {
   visit(o, a, o->builtin0 + (uint32_t)builtin_key, type, 1, &v);
 }
@@ -525,7 +539,11 @@ static int stage_join(ktj_oracle* o) {
       uint64_t slot = r->args_off;
       for (uint32_t f = 0; f < d->n_fields; ++f) {
         const ktj_field* fd = &s->fields[d->first_field + f];
-        if (fd->type != KTJ_F_COLLECTIVE) visit(o, a, fd->key_id, fd->type, fd->count, s->args + slot);
+        if (fd->type == KTJ_F_SHAPES) { /* the value's encoding lives elsewhere in the blob: materialised inline */
+          const uint64_t at = slot < s->n_args ? s->args[slot] : s->n_args;
+          const uint64_t len = shapes_encoded_slots(s->args, s->n_args, at);
+          visit(o, a, fd->key_id, fd->type, (uint16_t)len, len ? s->args + at : NULL);
+        } else if (fd->type != KTJ_F_COLLECTIVE) visit(o, a, fd->key_id, fd->type, fd->count, s->args + slot);
         slot += fd->count;
       }
     }
@@ -1100,6 +1118,43 @@ static void render_metadata(const ktj_oracle* o, const ktj_mat_activity* a, sbuf
         }
         sb_putc(json, ']');
         break;
+      case KTJ_F_STR_ARRAY: /* appendArray over appendQuoted: TypedMetadataJson.h:52-64, 184-186 */
+        sb_putc(json, '[');
+        for (uint32_t k = 0; k < fd->count; ++k) {
+          if (k) sb_puts(json, ", ");
+          ktj_oracle_string(o, (uint32_t)slot[k], &p, &len);
+          sb_putc(json, '"'); sb_put(json, p, len); sb_putc(json, '"');
+        }
+        sb_putc(json, ']');
+        break;
+      case KTJ_F_DICT_BEGIN: sb_putc(json, '{'); first = 1; break;  /* beginDict: TypedMetadataJson.h:128-132 */
+      case KTJ_F_DICT_END: sb_putc(json, '}'); first = 0; break;    /* endDict: :134-137 */
+      case KTJ_F_UNSUPPORTED: sb_puts(json, "\"<unsupported metadata type>\""); break; /* :122-126 */
+      case KTJ_F_SHAPES: { /* appendArray over the nested shapes: TypedMetadataJson.h:186-201; inline encoding */
+        const uint64_t* q = slot; const uint64_t* end = slot + fd->count;
+        const uint64_t entries = q < end ? *q++ : 0;
+        sb_putc(json, '[');
+        for (uint64_t e = 0; e < entries && q < end; ++e) {
+          if (e) sb_puts(json, ", ");
+          const uint64_t head = *q++, m = head & 0xFFFFFFFFull;
+          const uint64_t tensors = (head & KTJ_SHAPE_LIST) ? m : 1;
+          if (head & KTJ_SHAPE_LIST) sb_putc(json, '[');
+          for (uint64_t t = 0; t < tensors && ((head & KTJ_SHAPE_LIST) == 0 || q < end); ++t) {
+            if (t) sb_puts(json, ", ");
+            const uint64_t rank = (head & KTJ_SHAPE_LIST) ? (*q++ & 0xFFFFFFFFull) : m;
+            sb_putc(json, '[');
+            for (uint64_t k = 0; k < rank; ++k) {
+              if (k) sb_puts(json, ", ");
+              sb_put(json, n, fmt_i64(q < end ? (int64_t)*q : 0, n));
+              if (q < end) ++q;
+            }
+            sb_putc(json, ']');
+          }
+          if (head & KTJ_SHAPE_LIST) sb_putc(json, ']');
+        }
+        sb_putc(json, ']');
+        break;
+      }
       default: break;
     }
     slot += fd->count;

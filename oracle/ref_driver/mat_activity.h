@@ -81,45 +81,87 @@ struct MatActivity : public ITraceActivity {
   void log(ActivityLogger& logger) const override { logger.handleActivity(*this); }
 
   void visitTypedMetadata(ITypedMetadataVisitor& visitor) const override {
-    const uint64_t* slot = a->slots;
     std::vector<std::string> keep;  // MetadataField holds a string_view
     keep.reserve(a->n_fields);
-    for (uint32_t f = 0; f < a->n_fields; ++f) {
-      const ktj_field& fd = a->fields[f];
+    uint32_t f = 0;
+    const uint64_t* slot = a->slots;
+    visitFields(visitor, f, slot, keep);
+  }
+  // Visits fields from index f on; returns after the KTJ_F_DICT_END that closes the dict this
+  // call was made for (or at the end of the fields).
+  void visitFields(ITypedMetadataVisitor& visitor, uint32_t& f, const uint64_t*& slot, std::vector<std::string>& keep) const {
+    while (f < a->n_fields) {
+      const ktj_field& fd = a->fields[f++];
       keep.push_back(fd.key_id == KTJ_NONE ? std::string() : st->get(fd.key_id));
       const std::string& key = keep.back();
+      const uint64_t* v = slot;
+      slot += fd.count;
       switch (fd.type) {
         case KTJ_F_I64:
-          visitor.visit(MetadataField<int64_t>{key}, static_cast<int64_t>(slot[0]));
+          visitor.visit(MetadataField<int64_t>{key}, static_cast<int64_t>(v[0]));
           break;
         case KTJ_F_U64:
-          visitor.visit(MetadataField<uint64_t>{key}, static_cast<uint64_t>(slot[0]));
+          visitor.visit(MetadataField<uint64_t>{key}, static_cast<uint64_t>(v[0]));
           break;
         case KTJ_F_F64: {
           double d;
-          std::memcpy(&d, &slot[0], 8);
+          std::memcpy(&d, &v[0], 8);
           visitor.visit(MetadataField<double>{key}, d);
           break;
         }
         case KTJ_F_BOOL:
-          visitor.visit(MetadataField<bool>{key}, slot[0] != 0);
+          visitor.visit(MetadataField<bool>{key}, v[0] != 0);
           break;
         case KTJ_F_STR:
-          visitor.visit(MetadataField<std::string>{key}, st->get(static_cast<uint32_t>(slot[0])));
+          visitor.visit(MetadataField<std::string>{key}, st->get(static_cast<uint32_t>(v[0])));
           break;
         case KTJ_F_RAW:
-          visitor.visit(MetadataField<RawJson>{key}, RawJson{st->get(static_cast<uint32_t>(slot[0]))});
+          visitor.visit(MetadataField<RawJson>{key}, RawJson{st->get(static_cast<uint32_t>(v[0]))});
           break;
         case KTJ_F_I64_ARRAY: {
-          std::vector<int64_t> v(fd.count);
-          for (uint32_t k = 0; k < fd.count; ++k) v[k] = static_cast<int64_t>(slot[k]);
-          visitor.visit(MetadataField<std::vector<int64_t>>{key}, v);
+          std::vector<int64_t> arr(fd.count);
+          for (uint32_t k = 0; k < fd.count; ++k) arr[k] = static_cast<int64_t>(v[k]);
+          visitor.visit(MetadataField<std::vector<int64_t>>{key}, arr);
+          break;
+        }
+        case KTJ_F_STR_ARRAY: {
+          std::vector<std::string> arr;
+          for (uint32_t k = 0; k < fd.count; ++k) arr.push_back(st->get(static_cast<uint32_t>(v[k])));
+          visitor.visit(MetadataField<std::vector<std::string>>{key}, arr);
+          break;
+        }
+        case KTJ_F_DICT_BEGIN:
+          visitor.visit(MetadataDict{key}, [&](ITypedMetadataVisitor& d) { visitFields(d, f, slot, keep); });
+          break;
+        case KTJ_F_DICT_END:
+          return;
+        case KTJ_F_UNSUPPORTED:  // a field type the visitor has no overload for
+          visitor.visit(MetadataField<std::pair<int64_t, int64_t>>{key}, std::pair<int64_t, int64_t>{1, 2});
+          break;
+        case KTJ_F_SHAPES: {  // the checker hands the encoding over inline (see include/ktj.h)
+          InputShapes shapes;
+          const uint64_t* q = v;
+          const uint64_t* end = v + fd.count;
+          const uint64_t entries = q < end ? *q++ : 0;
+          auto shape = [&](uint64_t rank) {
+            std::vector<int64_t> dims;
+            for (uint64_t k = 0; k < rank; ++k) { dims.push_back(q < end ? static_cast<int64_t>(*q) : 0); if (q < end) ++q; }
+            return dims;
+          };
+          for (uint64_t e = 0; e < entries && q < end; ++e) {
+            const uint64_t head = *q++, m = head & 0xFFFFFFFFull;
+            if (head & KTJ_SHAPE_LIST) {
+              TensorListShapes list;
+              for (uint64_t t = 0; t < m && q < end; ++t) { const uint64_t rank = *q++ & 0xFFFFFFFFull; list.push_back(shape(rank)); }
+              shapes.emplace_back(std::move(list));
+            } else shapes.emplace_back(shape(m));
+          }
+          visitor.visit(MetadataField<InputShapes>{key}, shapes);
           break;
         }
         default:
           break;
       }
-      slot += fd.count;
     }
   }
   // The keyed double fields are the activity's counter values (read for counter kinds only).
@@ -177,54 +219,101 @@ struct GenericMatActivity : public GenericTraceActivity {
 // Replays one stream into a logger in the order of the reference's buffering logger
 // (src/output_membuf.h:91-107): trace start, device / resource / overhead infos, the activities
 // stable-sorted by (deviceId, resourceId, timestamp), spans, finalizeTrace(endTime).  L must
-// expose finalizeTrace(int64_t).  `log_all` hands the sorted activities to the logger; the default
+// expose finalizeTrace(int64_t).  `log_all` hands a list of activities to the logger; the default
 // is the replay loop of src/output_membuf.h:101-103, one log() call each.
+//
+// call_order 0: the order of the buffering logger's replay (src/output_membuf.h:91-107): trace
+//   start, device infos, resource infos, (overhead infos,) the activities stable-sorted by
+//   (deviceId, resourceId, timestamp), the spans, finalizeTrace.
+// call_order 1: the order in which GenericActivityProfiler drives a logger directly
+//   (src/GenericActivityProfiler.cpp:178-224 processTraceInternal, :655-740 finalizeTrace): trace
+//   start, the activities, the CPU buffer's span, resource infos, device infos, the GPU spans,
+//   overhead infos, finalizeTrace — with the activity segment sorted as above, so that it is what
+//   a logger that keeps its activities in one sorted section must write.
+// call_order 2: the same calls as 1 but with the activities where the profiler issues them and in
+//   arrival order: CPU-side activities, the CPU buffer's span, then the GPU-side activities and the
+//   rest.  Only a logger that sorts by itself writes the file of call_order 1 from it.
 template <class L, class LogAll>
 void replay_stream(L& logger, const ktj_stream* s, const ktj_mat_activity* acts, uint64_t n_acts, string_fn fn,
-                   const void* ctx, LogAll log_all) {
+                   const void* ctx, LogAll log_all, int call_order = 0) {
   StringTable st{fn, ctx};
   std::vector<MatActivity> wrapped;
   wrapped.reserve(n_acts);
   for (uint64_t i = 0; i < n_acts; ++i) wrapped.emplace_back(&acts[i], &st, s->collectives);
   std::vector<const MatActivity*> order(n_acts);
   for (uint64_t i = 0; i < n_acts; ++i) order[i] = &wrapped[i];
-  std::stable_sort(order.begin(), order.end(), [](const MatActivity* x, const MatActivity* y) {
-    return std::make_tuple(x->deviceId(), x->resourceId(), x->timestamp()) <
-        std::make_tuple(y->deviceId(), y->resourceId(), y->timestamp());
-  });
+  if (call_order != 2)
+    std::stable_sort(order.begin(), order.end(), [](const MatActivity* x, const MatActivity* y) {
+      return std::make_tuple(x->deviceId(), x->resourceId(), x->timestamp()) <
+          std::make_tuple(y->deviceId(), y->resourceId(), y->timestamp());
+    });
+  auto device_infos = [&] {
+    for (uint64_t i = 0; i < s->n_device_infos; ++i) {
+      const ktj_device_info& d = s->device_infos[i];
+      logger.handleDeviceInfo({d.id, d.sort_index, d.name, d.label}, d.time_ns);
+    }
+  };
+  auto resource_infos = [&] {
+    for (uint64_t i = 0; i < s->n_resource_infos; ++i) {
+      const ktj_resource_info& r = s->resource_infos[i];
+      logger.handleResourceInfo(
+          {r.id, r.sort_index, r.device_id, r.name, r.host_thread ? ResourceType::HOST_THREAD : ResourceType::UNKNOWN},
+          r.time_ns);
+    }
+  };
+  auto overhead_infos = [&] {
+    for (uint64_t i = 0; i < s->n_overhead_infos; ++i)
+      logger.handleOverheadInfo(ActivityLogger::OverheadInfo(s->overhead_infos[i].name), s->overhead_infos[i].time_ns);
+  };
+  auto spans = [&](uint64_t from, uint64_t to) {
+    for (uint64_t i = from; i < to && i < s->n_spans; ++i) {
+      const ktj_trace_span& sp = s->spans[i];
+      TraceSpan span(sp.op_count, sp.iteration, sp.name, sp.prefix);
+      span.startTime = sp.start_ns;
+      span.endTime = sp.end_ns;
+      logger.handleTraceSpan(span);
+    }
+  };
 
   std::unordered_map<std::string, std::string> metadata;  // env metadata (host_name) is added by the logger
   logger.handleTraceStart(metadata, s->device_properties ? s->device_properties : "");
-  for (uint64_t i = 0; i < s->n_device_infos; ++i) {
-    const ktj_device_info& d = s->device_infos[i];
-    logger.handleDeviceInfo({d.id, d.sort_index, d.name, d.label}, d.time_ns);
-  }
-  for (uint64_t i = 0; i < s->n_resource_infos; ++i) {
-    const ktj_resource_info& r = s->resource_infos[i];
-    logger.handleResourceInfo(
-        {r.id, r.sort_index, r.device_id, r.name, r.host_thread ? ResourceType::HOST_THREAD : ResourceType::UNKNOWN},
-        r.time_ns);
-  }
-  for (uint64_t i = 0; i < s->n_overhead_infos; ++i) {
-    logger.handleOverheadInfo(ActivityLogger::OverheadInfo(s->overhead_infos[i].name), s->overhead_infos[i].time_ns);
-  }
-  log_all(logger, order);
-  for (uint64_t i = 0; i < s->n_spans; ++i) {
-    const ktj_trace_span& sp = s->spans[i];
-    TraceSpan span(sp.op_count, sp.iteration, sp.name, sp.prefix);
-    span.startTime = sp.start_ns;
-    span.endTime = sp.end_ns;
-    logger.handleTraceSpan(span);
+  if (call_order == 0) {
+    device_infos();
+    resource_infos();
+    overhead_infos();
+    log_all(logger, order);
+    spans(0, s->n_spans);
+  } else {
+    if (call_order == 1) {
+      log_all(logger, order);
+      spans(0, 1);
+    } else { /* CPU-side activities (processCpuTrace), their span, then everything else (processGpuActivities) */
+      std::vector<const MatActivity*> cpu_side, gpu_side;
+      for (const MatActivity* a : order) {
+        const ActivityType t = a->type();
+        (t == ActivityType::CPU_OP || t == ActivityType::USER_ANNOTATION || t == ActivityType::CPU_INSTANT_EVENT ||
+                 t == ActivityType::PYTHON_FUNCTION
+             ? cpu_side : gpu_side).push_back(a);
+      }
+      if (cpu_side.empty() && !gpu_side.empty()) { cpu_side.push_back(gpu_side.front()); gpu_side.erase(gpu_side.begin()); }
+      log_all(logger, cpu_side);
+      spans(0, 1);
+      log_all(logger, gpu_side);
+    }
+    resource_infos();
+    device_infos();
+    spans(1, s->n_spans);
+    overhead_infos();
   }
   logger.finalizeTrace(s->end_time_ns);
 }
 
 template <class L>
 void replay_stream(L& logger, const ktj_stream* s, const ktj_mat_activity* acts, uint64_t n_acts, string_fn fn,
-                   const void* ctx) {
+                   const void* ctx, int call_order = 0) {
   replay_stream(logger, s, acts, n_acts, fn, ctx, [](L& l, const std::vector<const MatActivity*>& order) {
     for (const MatActivity* a : order) a->log(l);
-  });
+  }, call_order);
 }
 
 }  // namespace ktj_ref_driver

@@ -40,9 +40,11 @@ int64_t ktj_shim_base_time(void) { return ChromeTraceBaseTime::singleton().get()
 // workers, as GenericTraceActivity objects (so that the workers pack them).
 // huge_device_mod > 0: every activity whose arrival index is 1 modulo it reports a deviceId
 // beyond 32 bits, which the shim drops (and counts in *unsupported).
+// call_order: see replay_stream (0: the buffering logger's replay; 2: the calls as
+// GenericActivityProfiler issues them, activities unsorted and split around the CPU span).
 int ktj_shim_render(const ktj_stream* s, const ktj_mat_activity* acts, uint64_t n_acts, string_fn fn,
                     const void* ctx, const char* url, int hip_device, uint64_t* unsupported, int bulk_threads,
-                    int huge_device_mod) {
+                    int huge_device_mod, int call_order) {
   SET_LOG_SEVERITY_LEVEL(3);
   if (s->base_time_ns != ChromeTraceBaseTime::singleton().get()) return -2;
   ActivityLoggerFactory factory;
@@ -78,16 +80,16 @@ int ktj_shim_render(const ktj_stream* s, const ktj_mat_activity* acts, uint64_t 
         else { generic.emplace_back(order[i]); all.push_back(&generic.back()); }
       }
       l.handleActivities(all, static_cast<unsigned>(bulk_threads));
-    });
+    }, call_order);
   } else if (huge_device_mod > 0) {
     replay_stream(*shim, s, acts, n_acts, fn, ctx, [&](ShimLogger& l, const std::vector<const MatActivity*>& order) {
       for (const MatActivity* a : order) {
         if (huge(a)) { const HugeDevice h(a); l.handleActivity(h); }
         else a->log(l);
       }
-    });
+    }, call_order);
   } else {
-    replay_stream(*shim, s, acts, n_acts, fn, ctx);
+    replay_stream(*shim, s, acts, n_acts, fn, ctx, call_order);
   }
   if (unsupported) *unsupported = shim->unsupportedActivities();
   return shim->engineStatus();

@@ -89,6 +89,66 @@ def case_typed_metadata_pins():
     return b, expect
 
 
+def case_typed_metadata_collections():
+    """libkineto/test/TypedMetadataTest.cpp:145-178 (string array, nested dict with a field after
+    it), :186-200 (a dict inside a dict with siblings on both sides), :209 (a type the visitor does
+    not know), :229-244 (uint64 and InputShapes)."""
+    b = StreamBuilder()
+    D, E = (abi.F_DICT_BEGIN, 0), (abi.F_DICT_END, 0)
+    one = b.schema([("count", abi.F_I64, 1), ("ids", abi.F_I64_ARRAY, 2), ("label", abi.F_STR, 1), ("ratio", abi.F_F64, 1),
+                    ("enabled", abi.F_BOOL, 1), ("names", abi.F_STR_ARRAY, 2), ("special", abi.F_STR, 1),
+                    ("nested",) + D, ("nested_count", abi.F_I64, 1), ("nested_other", abi.F_I64, 1), (None,) + E,
+                    ("after_nested", abi.F_I64, 1)])
+    b.add_generic("op1", CPU_OP, B + 1, B + 2, 1, 2, id=0, schema=one,
+                  values=[5, 1, 2, b.s("label"), 1.5, 1, b.s("a"), b.s("b"), b.s('quote " slash \\ newline\n'), 7, 8, 9])
+    two = b.schema([("outer",) + D, ("count", abi.F_I64, 1), ("inner",) + D, ("enabled", abi.F_BOOL, 1), (None,) + E,
+                    ("ratio", abi.F_F64, 1), (None,) + E, ("after_nested", abi.F_I64, 1)])
+    b.add_generic("op2", CPU_OP, B + 3, B + 4, 1, 2, id=0, schema=two, values=[1, 1, 2.5, 9])
+    three = b.schema([("count", abi.F_I64, 1), ("pair", abi.F_UNSUPPORTED, 0), ("address", abi.F_U64, 1),
+                      ("input_dims", abi.F_SHAPES, 1), ("empty", abi.F_STR_ARRAY, 0), ("first",) + D, (None,) + E,
+                      ("strides", abi.F_SHAPES, 1)])
+    dims = b.shapes([[2, 2], [[4, 1], [4, 1]]])
+    strides = b.shapes([[], [[]], [[7], [], [-1, 0, 9223372036854775807]], [1]])
+    b.add_generic("op3", CPU_OP, B + 5, B + 6, 1, 2, id=0, schema=three, values=[5, 0xFFFFFFFFFFFFFFFF, dims, strides])
+    # a dict as the first and only field, and a schema of brackets alone
+    four = b.schema([("occupancy",) + D, ("active_blocks_per_multiprocessor", abi.F_I64, 1), ("limiting_factors", abi.F_STR, 1), (None,) + E])
+    b.add_generic("op4", CPU_OP, B + 7, B + 8, 1, 2, id=0, schema=four, values=[4, b.s("warps, registers")])
+    expect = ['"count": 5, "ids": [1, 2], "label": "label", "ratio": 1.5, "enabled": true, "names": ["a", "b"], '
+              '"special": "quote " slash / newline", "nested": {"nested_count": 7, "nested_other": 8}, "after_nested": 9',
+              '"outer": {"count": 1, "inner": {"enabled": true}, "ratio": 2.5}, "after_nested": 9',
+              '"count": 5, "pair": "<unsupported metadata type>", "address": 18446744073709551615, '
+              '"input_dims": [[2, 2], [[4, 1], [4, 1]]], "empty": [], "first": {}, '
+              '"strides": [[], [[]], [[7], [], [-1, 0, 9223372036854775807]], [1]]',
+              '"occupancy": {"active_blocks_per_multiprocessor": 4, "limiting_factors": "warps, registers"}']
+    return b, expect
+
+
+def case_cuda_shaped_kernel_args():
+    """The typed metadata of a CUDA kernel activity (libkineto/src/CuptiActivity.h:499-576): fifteen
+    fields, the last a dict of nine, as a schema of a generic kernel record."""
+    b = StreamBuilder()
+    D, E = (abi.F_DICT_BEGIN, 0), (abi.F_DICT_END, 0)
+    sch = b.schema([("queued", abi.F_U64, 1), ("device", abi.F_I64, 1), ("context", abi.F_U64, 1), ("stream", abi.F_I64, 1),
+                    ("correlation", abi.F_U64, 1), ("registers per thread", abi.F_U64, 1), ("shared memory", abi.F_I64, 1),
+                    ("blocks per SM", abi.F_F64, 1), ("warps per SM", abi.F_F64, 1), ("grid", abi.F_I64_ARRAY, 3),
+                    ("block", abi.F_I64_ARRAY, 3), ("est. achieved occupancy %", abi.F_I64, 1),
+                    ("occupancy",) + D, ("active_blocks_per_multiprocessor", abi.F_I64, 1), ("limiting_factors", abi.F_STR, 1),
+                    ("block_limit_regs", abi.F_I64, 1), ("block_limit_shared_mem", abi.F_I64, 1), ("block_limit_warps", abi.F_I64, 1),
+                    ("block_limit_blocks", abi.F_I64, 1), ("block_limit_barriers", abi.F_I64, 1),
+                    ("allocated_registers_per_block", abi.F_I64, 1), ("allocated_shared_mem_per_block", abi.F_U64, 1), (None,) + E])
+    for k in range(3):
+        b.add_generic("void gemm<float>(int)", KERNEL, B + 100 * k, B + 100 * k + 40, 0, 7, id=50 + k, schema=sch,
+                      values=[0, 0, 1, 7, 50 + k, 64 + k, 49152, 0.5945945945945946, 4.756756756756757, 88, 1, 1, 256, 1, 1, 38,
+                              3, b.s("registers"), 3, 4, 8, 32, 16, 16384 + k, 49152], flow_id=50 + k, flow_type=2)
+    expect = ['"queued": 0, "device": 0, "context": 1, "stream": 7, "correlation": 50, "registers per thread": 64, '
+              '"shared memory": 49152, "blocks per SM": 0.5945945945945946, "warps per SM": 4.756756756756757, '
+              '"grid": [88, 1, 1], "block": [256, 1, 1], "est. achieved occupancy %": 38, '
+              '"occupancy": {"active_blocks_per_multiprocessor": 3, "limiting_factors": "registers", "block_limit_regs": 3, '
+              '"block_limit_shared_mem": 4, "block_limit_warps": 8, "block_limit_blocks": 32, "block_limit_barriers": 16, '
+              '"allocated_registers_per_block": 16384, "allocated_shared_mem_per_block": 49152}']
+    return b, expect
+
+
 def case_names():
     """Observed from the real logger: UTF-8, TAB and DEL make the whole name 'unknown'; printable
     punctuation is untouched; newlines vanish; quotes are escaped after backslashes became slashes."""
@@ -380,7 +440,7 @@ def case_gpu_user_annotations():
 
 
 SUBSTRING_CASES = [case_gpu_user_annotation_reference_test, case_gpu_user_annotations, case_collective_reference_test, case_collective_reference_test_quoted, case_collective_joined, case_counter_events, case_instant_and_stream_sync, case_logger_events, case_trace_span, case_benchmark_cpu_op, case_typed_kernel_args,
-                   case_typed_metadata_pins, case_names, case_resource_infos]
+                   case_typed_metadata_pins, case_typed_metadata_collections, case_cuda_shaped_kernel_args, case_names, case_resource_infos]
 
 
 def build_for_real_logger(case, ref_args):

@@ -52,12 +52,30 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False,
         return rng.choice([rng.randrange(lo - 500, hi + 500), rng.randrange(lo, hi), 0, lo, hi])
 
     # schemas
+    def random_fields(n_max):
+        """Fields of every kind; now and then a run of them sits inside a dict, and all of them in another."""
+        fields = []
+        for _k in range(rng.randrange(0, n_max)):
+            typ = rng.choice([0, 1, 2, 3, 4, 5, 6, abi.F_STR_ARRAY, abi.F_SHAPES, abi.F_UNSUPPORTED])
+            cnt = rng.randrange(1, 5) if typ == abi.F_I64_ARRAY else rng.randrange(0, 4) if typ == abi.F_STR_ARRAY else 0 if typ == abi.F_UNSUPPORTED else 1
+            fields.append((_name(rng)[:12] or "k", typ, cnt))
+        if rng.random() < 0.5:
+            i = rng.randrange(0, len(fields) + 1)
+            j = rng.randrange(i, len(fields) + 1)
+            fields[j:j] = [(None, abi.F_DICT_END, 0)]
+            fields[i:i] = [(_name(rng)[:8] or "d", abi.F_DICT_BEGIN, 0)]
+        if rng.random() < 0.3:
+            fields = [("all", abi.F_DICT_BEGIN, 0)] + fields + [(None, abi.F_DICT_END, 0)]
+        return fields
+
+    def random_shapes():
+        def shape():
+            return [_i64(rng) for _ in range(rng.randrange(0, 4))]
+        return [([shape() for _ in range(rng.randrange(1, 4))] if rng.random() < 0.3 else shape()) for _ in range(rng.randrange(0, 4))]
+
     schemas = [None, b.schema([(None, abi.F_RAW, 1)])]
     for _ in range(4):
-        fields = []
-        for _k in range(rng.randrange(0, 6)):
-            typ = rng.randrange(7)
-            fields.append((_name(rng)[:12] or "k", typ, rng.randrange(1, 5) if typ == abi.F_I64_ARRAY else 1))
+        fields = random_fields(6)
         schemas.append((b.schema(fields), fields))
     # collective metadata: entries with random subsets of the keys, schemas that start with a reference to one
     n_coll = rng.choice([0, 0, 1, 5])
@@ -74,10 +92,7 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False,
         b.add_collective(**vals)
     if n_coll:
         for _ in range(3):
-            fields = [(None, abi.F_COLLECTIVE, 1)]
-            for _k in range(rng.randrange(0, 3)):
-                typ = rng.randrange(7)
-                fields.append((_name(rng)[:12] or "k", typ, rng.randrange(1, 5) if typ == abi.F_I64_ARRAY else 1))
+            fields = [(None, abi.F_COLLECTIVE, 1)] + random_fields(3)
             schemas.append((b.schema(fields), fields))
         schemas.append((b.schema([(None, abi.F_COLLECTIVE, 1), (None, abi.F_RAW, 1)]), [(None, abi.F_COLLECTIVE, 1), (None, abi.F_RAW, 1)]))
     pids, tids = [0, 1, 7, -3, 4242], [0, 5, -5, 4243, I64_MIN, I64_MAX, 10**12]
@@ -100,6 +115,12 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False,
                     values.append(_f64(rng))
                 elif typ in (abi.F_STR, abi.F_RAW):
                     values.append(b.s(_name(rng)))
+                elif typ == abi.F_STR_ARRAY:
+                    values += [b.s(_name(rng)) for _ in range(cnt)]
+                elif typ == abi.F_SHAPES:
+                    values.append(rng.choice([b.shapes(random_shapes()), 2**50]))   # now and then a slot that points nowhere
+                elif typ in (abi.F_DICT_BEGIN, abi.F_DICT_END, abi.F_UNSUPPORTED):
+                    pass
                 elif typ == abi.F_BOOL:
                     values.append(rng.randrange(3))
                 elif typ == abi.F_I64_ARRAY:

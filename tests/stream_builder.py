@@ -62,6 +62,20 @@ class StreamBuilder:
             self.args.append(v & 0xFFFFFFFFFFFFFFFF)
         return off
 
+    def shapes(self, value):
+        """Encodes an InputShapes value (a list whose entries are a shape, e.g. [2, 2], or a list of
+        shapes, e.g. [[4, 1], [4, 1]]; an empty entry is an empty shape) in the args blob and returns
+        the slot index for a F_SHAPES field (include/ktj.h: KTJ_F_SHAPES)."""
+        enc = [len(value)]
+        for entry in value:
+            if entry and isinstance(entry[0], (list, tuple)):
+                enc.append(abi.SHAPE_LIST | len(entry))
+                for shape in entry:
+                    enc += [len(shape)] + list(shape)
+            else:
+                enc += [len(entry)] + list(entry)
+        return self.arg_slots(enc)
+
     def api(self, names, flow_start=(), malloc_cid=abi.KTJ_NONE):
         self.cid_names = [abi.KTJ_NONE if n is None else self.s(n) for n in names]
         self.flow_start = list(flow_start)

@@ -69,6 +69,39 @@ def test_shim_random_streams(seed):
     _compare(sp)
 
 
+@pytest.mark.parametrize("case", [(1, 3000), (2, 6000), (3, 20000), (4, 9000), (5, 800), "random3", "random8", "kat"])
+def test_shim_in_the_profilers_call_order(case):
+    """GenericActivityProfiler drives a logger in another order than the buffering logger's replay
+    (src/GenericActivityProfiler.cpp:178-224, 655-740): CPU-side activities, the CPU buffer's span,
+    GPU-side activities, then resource infos, device infos, GPU spans and overhead infos.  The
+    reference logger writes every event where its call arrives; fed those calls, the shim must write
+    the reference's file for the same calls with the activity segment sorted."""
+    import random_streams
+    if case == "kat":
+        sp, release = kat_cases.build_for_real_logger(kat_cases.case_rocm_sync_trace, og.ref_stream_args()), None
+    elif isinstance(case, str):
+        seed = int(case[6:])
+        sp, release = kat_cases.build_for_real_logger(lambda: (random_streams.random_stream(seed), None), og.ref_stream_args()), None
+    else:
+        sp, release = abi.synth_stream(case[0], case[1], **og.ref_stream_args())
+    o = og.OracleRun(sp)
+    try:
+        theirs = og.ref_render(sp, o, call_order=1)
+        if sp.contents.n_device_infos or sp.contents.n_resource_infos:
+            assert theirs != og.ref_render(sp, o)          # the two orders give different files
+        for threads in (0, 4):
+            rc, mine, dropped = og.shim_render(sp, o, bulk_threads=threads, call_order=2)
+            assert rc == 0 and dropped == 0
+            if mine != theirs:
+                i = _first_diff(mine, theirs)
+                raise AssertionError(f"threads={threads}: byte {i} of {len(theirs)}: shim {mine[max(0, i - 80):i + 80]!r} "
+                                     f"reference {theirs[max(0, i - 80):i + 80]!r}")
+    finally:
+        o.close()
+        if release:
+            release()
+
+
 def test_shim_bulk_packing_is_independent_of_the_worker_count():
     """handleActivities() with 1, 2, 5 and 16 workers writes the same file as the reference."""
     sp, release = abi.synth_stream(3, 40000, **og.ref_stream_args())
