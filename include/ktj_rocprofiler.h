@@ -1,5 +1,7 @@
 /*
- * ktj_rocprofiler.h — rocprofiler-sdk buffer records straight into the engine.
+ * ktj_rocprofiler.h — rocprofiler-sdk records straight into the engine: the buffer records of
+ * kernel dispatches and memory copies (device rows) and the callback records of HIP runtime API
+ * calls (runtime rows).
  *
  * Replaces the body of RocprofLogger::buffer_callback (libkineto/src/RocprofLogger.cpp:681-749),
  * which turns every kernel-dispatch and memory-copy record of an SDK buffer into a heap-allocated
@@ -37,6 +39,23 @@ int ktj_set_sdk_kernel_names(ktj_engine* e, const uint64_t* kernel_ids, const ui
  * skipped, as the reference skips it.  *n_rows receives the number of rows taken.  The SDK's
  * buffer may be released when the call returns. */
 int ktj_submit_sdk_buffer(ktj_engine* e, void* const* headers, size_t num_headers, uint64_t* n_rows);
+
+/* One HIP runtime API call, at ROCPROFILER_CALLBACK_PHASE_EXIT of the SDK's callback tracing
+ * service: replaces the row construction of RocprofLogger::api_callback
+ * (libkineto/src/RocprofLogger.cpp:561-679).  `record` is the SDK's
+ * `const rocprofiler_callback_tracing_record_t*` (kind ROCPROFILER_CALLBACK_TRACING_HIP_RUNTIME_API,
+ * anything else is ignored as the reference ignores it; its payload is the SDK's
+ * rocprofiler_callback_tracing_hip_api_data_t).  begin / end are the caller's timestamps of the
+ * enter and exit phases (the reference takes getApproximateTime() in both, :569-574), pid / tid the
+ * calling process and thread.  The call becomes one runtime row (ktj_runtime_rec: kernel launch,
+ * copy, malloc/free or plain, by operation) after the rows submitted so far; its arguments are read
+ * from the SDK's argument union by the names the reference looks for.  external_id /
+ * user_external_id: the innermost id of the caller's external-correlation stack of domain 0 / 1, or
+ * NULL where that stack is empty (:661-672): each gives one KTJ_REC_EXTCORR / KTJ_REC_USERCORR pair
+ * for the call's correlation id.  Rows are buffered on the host and reach the device in batches and
+ * with the next ktj_process / ktj_finalize. */
+int ktj_submit_sdk_api_record(ktj_engine* e, const void* record, uint64_t begin, uint64_t end, uint32_t pid,
+                              uint32_t tid, const uint64_t* external_id, const uint64_t* user_external_id);
 
 #ifdef __cplusplus
 }

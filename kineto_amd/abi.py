@@ -186,7 +186,7 @@ ENGINE_SYMBOLS = [
     "ktj_process", "ktj_process_noalloc", "ktj_output_device", "ktj_output_host", "ktj_finalize", "ktj_get_stats",
     "ktj_version",
     # include/ktj_rocprofiler.h
-    "ktj_set_sdk_agents", "ktj_set_sdk_kernel_names", "ktj_submit_sdk_buffer",
+    "ktj_set_sdk_agents", "ktj_set_sdk_kernel_names", "ktj_submit_sdk_buffer", "ktj_submit_sdk_api_record",
 ]
 
 
@@ -237,6 +237,9 @@ def load_engine():
         lib.ktj_set_sdk_kernel_names.argtypes = [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), C.c_size_t, C.c_uint32]
         lib.ktj_submit_sdk_buffer.restype = C.c_int
         lib.ktj_submit_sdk_buffer.argtypes = [vp, C.POINTER(C.c_void_p), C.c_size_t, C.POINTER(C.c_uint64)]
+        lib.ktj_submit_sdk_api_record.restype = C.c_int
+        lib.ktj_submit_sdk_api_record.argtypes = [vp, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint32, C.c_uint32,
+                                                  C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
         lib.ktj_process.restype = C.c_int
         lib.ktj_process.argtypes = [vp, C.c_int64]
         lib.ktj_process_noalloc.restype = C.c_int

@@ -26,6 +26,7 @@
 #include "../../include/ktj_rocprofiler.h"
 #include "gpu_stages.h"
 #include "host_events.h"
+#include "sdk_api_rows.h"
 
 using namespace ktj;
 using namespace ktj::gpu;
@@ -149,6 +150,8 @@ struct ktj_engine {
   std::unordered_map<uint64_t, uint32_t> sdk_kernel_names; /* kernel id -> string id of its name */
   uint32_t sdk_unknown_name = KTJ_NONE;
   std::vector<ktj_device_rec> sdk_rows;                    /* conversion buffer, reused */
+  std::vector<ktj_runtime_rec> sdk_api_rows;               /* runtime rows of ktj_submit_sdk_api_record, not yet on the device */
+  std::vector<ktj_extcorr_rec> sdk_api_ext, sdk_api_user;  /* their external-correlation pairs */
   std::vector<uint32_t> cid_names, flow_bits;
   uint32_t malloc_cid = KTJ_NONE;
   DevBuf d_cid_names, d_flow_bits;
@@ -621,6 +624,34 @@ int ktj_submit_sdk_buffer(ktj_engine* e, void* const* headers, size_t num_header
   return ktj_submit_records(e, KTJ_REC_DEVICE, rows.data(), rows.size());
 }
 
+/* runtime rows and correlation pairs that ktj_submit_sdk_api_record collected go to the device */
+static int flush_sdk_api_rows(ktj_engine* e) {
+  int rc = KTJ_OK;
+  if (!e->sdk_api_rows.empty()) rc = ktj_submit_records(e, KTJ_REC_RUNTIME, e->sdk_api_rows.data(), e->sdk_api_rows.size());
+  if (rc == KTJ_OK && !e->sdk_api_ext.empty()) rc = ktj_submit_records(e, KTJ_REC_EXTCORR, e->sdk_api_ext.data(), e->sdk_api_ext.size());
+  if (rc == KTJ_OK && !e->sdk_api_user.empty()) rc = ktj_submit_records(e, KTJ_REC_USERCORR, e->sdk_api_user.data(), e->sdk_api_user.size());
+  if (rc == KTJ_OK) { e->sdk_api_rows.clear(); e->sdk_api_ext.clear(); e->sdk_api_user.clear(); }
+  return rc;
+}
+
+#define KTJ_SDK_API_BATCH 65536u
+int ktj_submit_sdk_api_record(ktj_engine* e, const void* record, uint64_t begin, uint64_t end, uint32_t pid, uint32_t tid,
+                              const uint64_t* external_id, const uint64_t* user_external_id) {
+  if (!e || !record) return KTJ_ERR_ARG;
+  if (e->bad_sink) return KTJ_OK;
+  const auto& rec = *static_cast<const rocprofiler_callback_tracing_record_t*>(record);
+  if (rec.kind != ROCPROFILER_CALLBACK_TRACING_HIP_RUNTIME_API || !rec.payload) return KTJ_OK; /* RocprofLogger.cpp:567 */
+  const auto& data = *static_cast<const rocprofiler_callback_tracing_hip_api_data_t*>(rec.payload);
+  ktj_runtime_rec row;
+  sdk_api::runtime_row(static_cast<uint32_t>(rec.operation), rec.correlation_id.internal, data.args, begin, end, pid, tid, &row);
+  e->sdk_api_rows.push_back(row);
+  if (external_id) e->sdk_api_ext.push_back(ktj_extcorr_rec{rec.correlation_id.internal, *external_id});
+  if (user_external_id) e->sdk_api_user.push_back(ktj_extcorr_rec{rec.correlation_id.internal, *user_external_id});
+  e->activities_begun = true;
+  e->processed = false;
+  return e->sdk_api_rows.size() >= KTJ_SDK_API_BATCH ? flush_sdk_api_rows(e) : KTJ_OK;
+}
+
 int ktj_begin_activities(ktj_engine* e) {
   if (!e) return KTJ_ERR_ARG;
   e->activities_begun = true;
@@ -1013,6 +1044,8 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
 int ktj_process(ktj_engine* e, int64_t end_time_ns) {
   if (!e) return KTJ_ERR_ARG;
   if (e->bad_sink) return KTJ_OK;
+  const int flushed = flush_sdk_api_rows(e);
+  if (flushed != KTJ_OK) return flushed;
   e->noalloc = false;
   return process_pass(e, end_time_ns, nullptr, 0);
 }
@@ -1025,6 +1058,10 @@ int ktj_process_noalloc(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   if (!e || !out_device || ((uintptr_t)out_device & 15u) != 0) return KTJ_ERR_ARG;
   if (e->bad_sink) return KTJ_OK;
   if (!e->arena) { e->last_error = "ktj_process_noalloc: no scratch array on this device"; return KTJ_ERR_STATE; }
+  if (!e->sdk_api_rows.empty() || !e->sdk_api_ext.empty() || !e->sdk_api_user.empty()) {
+    e->last_error = "ktj_process_noalloc: rows of ktj_submit_sdk_api_record are still buffered on the host (ktj_process takes them over)";
+    return KTJ_ERR_STATE;
+  }
   if (e->usercorr.n != 0) {
     e->last_error = "ktj_process_noalloc: user-domain correlation records (GPU user annotations) are not supported here";
     return KTJ_ERR_LIMIT;

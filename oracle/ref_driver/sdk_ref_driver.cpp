@@ -20,9 +20,16 @@
  *   The SDK records are built by tests/host_sim/sdk_records.cpp from the rows, as in the tests.
  * mode 2:
  *   u64 n_records, {u32 operation, u32 pad, u64 correlation_id, u8 args[sizeof(rocprofiler_hip_api_args_t)]}[n]
- * stdout: one text line per row the logger holds afterwards.
+ *   Each record goes through api_callback twice (enter, exit).  Pointer-typed arguments should point
+ *   into [KTJ_ARG_ARENA, KTJ_ARG_ARENA + 16 MiB): the driver maps zero pages there, because the SDK's
+ *   argument iterator follows pointers when it renders them.
+ * stdout: one text line per row the logger holds afterwards; in mode 2 the row's line is followed by
+ * an "args" line with the SDK's own rendering of every argument (name=text), which is what the
+ * reference keeps of dst, src and ptr.
  */
 #include "RocprofLogger.cpp"  // NOLINT: the reference's translation unit, found through -I$(REF)/libkineto/src
+
+#include <sys/mman.h>
 
 #include <cinttypes>
 #include <cstdio>
@@ -70,16 +77,15 @@ void print_rows() {
       }
       case ROCTRACER_ACTIVITY_COPY: {
         const auto* r = static_cast<const rocprofCopyRow*>(b);
-        /* src and dst hold the SDK's rendering of the argument (a C string), see RocprofLogger.cpp:611-624 */
-        printf("copy id=%" PRIu64 " domain=%u cid=%u src=%s dst=%s size=%zu kind=%d stream=%" PRIu64 "\n", r->id, r->domain,
-               r->cid, static_cast<const char*>(r->src), static_cast<const char*>(r->dst), r->size, (int)r->kind,
-               (uint64_t)(uintptr_t)r->stream);
+        /* src and dst hold the address of the SDK's rendering of the argument (RocprofLogger.cpp:52-58,
+         * 611-624), which is gone by now: not followed */
+        printf("copy id=%" PRIu64 " domain=%u cid=%u size=%zu kind=%d stream=%" PRIu64 "\n", r->id, r->domain, r->cid, r->size,
+               (int)r->kind, (uint64_t)(uintptr_t)r->stream);
         break;
       }
       case ROCTRACER_ACTIVITY_MALLOC: {
         const auto* r = static_cast<const rocprofMallocRow*>(b);
-        printf("malloc id=%" PRIu64 " domain=%u cid=%u ptr=%s size=%zu\n", r->id, r->domain, r->cid,
-               static_cast<const char*>(r->ptr), r->size);
+        printf("malloc id=%" PRIu64 " domain=%u cid=%u size=%zu\n", r->id, r->domain, r->cid, r->size);
         break;
       }
       case ROCTRACER_ACTIVITY_DEFAULT: {
@@ -124,7 +130,20 @@ int run_buffer_records() {
   return 0;
 }
 
+#define KTJ_ARG_ARENA 0x700000000000ull
+int print_arg(rocprofiler_callback_tracing_kind_t, rocprofiler_tracing_operation_t, uint32_t, const void* const, int32_t,
+              const char*, const char* arg_name, const char* arg_value_str, int32_t, void*) {
+  printf(" %s=%s;", arg_name, arg_value_str);
+  return 0;
+}
+
 int run_api_records() {
+  if (mmap(reinterpret_cast<void*>(KTJ_ARG_ARENA), 16u << 20, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_FIXED,
+           -1, 0) == MAP_FAILED) {
+    fprintf(stderr, "sdk_ref_driver: cannot map the argument arena\n");
+    return 2;
+  }
+  printf("kind hip_runtime_api=%d\n", (int)ROCPROFILER_CALLBACK_TRACING_HIP_RUNTIME_API);
   const uint64_t n = rd<uint64_t>();
   for (uint64_t i = 0; i < n; ++i) {
     const uint32_t op = rd<uint32_t>();
@@ -144,9 +163,11 @@ int run_api_records() {
     RocprofLogger::api_callback(rec, nullptr, nullptr);
     rec.phase = ROCPROFILER_CALLBACK_PHASE_EXIT;
     RocprofLogger::api_callback(rec, nullptr, nullptr);
-    /* the rows of copies and allocations point at strings the SDK renders per call: print now */
     print_rows();
     RocprofLogger::singleton().rows_.clear();
+    printf("args");
+    rocprofiler_iterate_callback_tracing_kind_operation_args(rec, print_arg, 1, nullptr);
+    printf("\n");
   }
   return 0;
 }

@@ -15,6 +15,7 @@
 #include <vector>
 
 #include "../../include/ktj.h"
+#include "../../kineto_amd/csrc/sdk_api_rows.h"
 
 namespace {
 struct SdkBuffer {
@@ -90,5 +91,35 @@ void* ktjsim_sdk_buffer_create(const ktj_device_rec* rows, uint64_t n, uint64_t 
 void* const* ktjsim_sdk_buffer_headers(void* buf) { return static_cast<SdkBuffer*>(buf)->header_ptrs.data(); }
 uint64_t ktjsim_sdk_buffer_count(void* buf) { return static_cast<SdkBuffer*>(buf)->header_ptrs.size(); }
 void ktjsim_sdk_buffer_free(void* buf) { delete static_cast<SdkBuffer*>(buf); }
+
+/* ---- HIP runtime API callback records (ktj_submit_sdk_api_record) ---- */
+uint64_t ktjsim_sdk_api_args_size(void) { return sizeof(rocprofiler_hip_api_args_t); }
+uint32_t ktjsim_sdk_api_last_op(void) { return ROCPROFILER_HIP_RUNTIME_API_ID_LAST; }
+/* the engine's conversion (kineto_amd/csrc/sdk_api_rows.h) of one call whose argument union holds
+ * the given bytes */
+uint32_t ktjsim_sdk_api_row(uint32_t operation, uint64_t correlation_id, const void* args_bytes, uint64_t begin, uint64_t end,
+                            uint32_t pid, uint32_t tid, ktj_runtime_rec* out) {
+  rocprofiler_hip_api_args_t args;
+  std::memcpy(&args, args_bytes, sizeof args);
+  return ktj::sdk_api::runtime_row(operation, correlation_id, args, begin, end, pid, tid, out);
+}
+/* a callback record as the SDK hands it over, around the same bytes (for ktj_submit_sdk_api_record);
+ * freed with ktjsim_sdk_api_record_free */
+struct ApiRecordHolder { rocprofiler_callback_tracing_record_t rec; rocprofiler_callback_tracing_hip_api_data_t data; };
+void* ktjsim_sdk_api_record_create(uint32_t kind, uint32_t operation, uint64_t correlation_id, const void* args_bytes) {
+  typedef ApiRecordHolder Holder;
+  Holder* h = new Holder;
+  std::memset(h, 0, sizeof *h);
+  h->data.size = sizeof h->data;
+  std::memcpy(&h->data.args, args_bytes, sizeof h->data.args);
+  h->rec.kind = static_cast<rocprofiler_callback_tracing_kind_t>(kind);
+  h->rec.operation = static_cast<rocprofiler_tracing_operation_t>(operation);
+  h->rec.correlation_id.internal = correlation_id;
+  h->rec.phase = ROCPROFILER_CALLBACK_PHASE_EXIT;
+  h->rec.payload = &h->data;
+  return h;
+}
+void ktjsim_sdk_api_record_free(void* p) { delete static_cast<ApiRecordHolder*>(p); }
+uint32_t ktjsim_sdk_api_kind_hip_runtime(void) { return ROCPROFILER_CALLBACK_TRACING_HIP_RUNTIME_API; }
 
 }  // extern "C"

@@ -155,6 +155,56 @@ def test_checker_restatement_matches_the_reference_buffer_callback(case):
             release()
 
 
+def _golden_api_rows():
+    """tests/golden/sdk_api_rows.txt (written by tests/golden/make_sdk_api_golden.py from the
+    reference's api_callback): per operation id the row line and, for rows that read arguments, the
+    SDK's rendering of the call's arguments."""
+    lines = open(os.path.join(ROOT, "tests", "golden", "sdk_api_rows.txt")).read().split("\n")
+    domain = int(lines[0].split("=")[1])
+    rows, k = [], 1
+    while k < len(lines) and lines[k]:
+        args = None
+        if k + 1 < len(lines) and lines[k + 1].startswith("args"):
+            args = dict(kv.strip().split("=", 1) for kv in lines[k + 1][4:].split(";") if "=" in kv and "{" not in kv)
+            rows.append((lines[k], args))
+            k += 2
+        else:
+            rows.append((lines[k], None))
+            k += 1
+    return domain, rows
+
+
+def test_api_callback_rows_match_the_reference_for_every_hip_operation():
+    """ktj_submit_sdk_api_record's conversion (kineto_amd/csrc/sdk_api_rows.h) against the rows the
+    reference's RocprofLogger::api_callback makes of the same calls: one call of every HIP runtime
+    API operation of this SDK, arguments filled with a fixed pattern.  Row class, operation,
+    correlation id and every argument the reference keeps must agree; dst, src and ptr, of which the
+    reference only keeps a text, must read as that text."""
+    import sdk_api_pattern as pat
+    domain, golden = _golden_api_rows()
+    assert len(golden) == pat.n_ops() > 400
+    kinds = {"kernel": 0, "copy": 0, "malloc": 0, "default": 0}
+    for op, (want, args) in enumerate(golden):
+        got, r = pat.engine_line(op, domain)
+        assert got == want, op
+        kinds[want.split()[0]] += 1
+        if want.startswith("copy"):
+            assert ("dst" in args) == (r.u.copy.dst != 0) and ("src" in args) == (r.u.copy.src != 0), op
+            for name, value in (("dst", r.u.copy.dst), ("src", r.u.copy.src)):
+                if name in args:
+                    assert args[name] == hex(value), (op, name)
+        if want.startswith("malloc") and "ptr" in args:
+            assert args["ptr"] == hex(r.u.malloc_.ptr), op
+    assert kinds["kernel"] == 12 and kinds["copy"] == 29 and kinds["malloc"] == 2   # RocprofLogger.cpp:165-245
+
+
+@pytest.mark.skipif(not os.path.exists(SDK_REF_DRIVER), reason="oracle/_ref/sdk_ref_driver is not built (needs the reference's sources)")
+def test_api_callback_golden_file_is_what_the_reference_produces():
+    import sdk_api_pattern as pat
+    want = open(os.path.join(ROOT, "tests", "golden", "sdk_api_rows.txt")).read().split("\n")
+    assert pat.reference_lines() == [line for line in want if line]
+
+
 def _sdk_case(cfg, n):
     """A synthetic stream whose kernel and copy rows went through SDK records: returns the stream
     with its device rows replaced by the checker's reading of those records, and what the engine
@@ -229,3 +279,60 @@ def test_sdk_buffer_ingestion_matches_checker(cfg, n):
         assert b"<unknown kernel>" in want and b'"pid": -1,' in want
     finally:
         release()
+
+
+@pytest.mark.gpu
+def test_sdk_api_records_end_to_end():
+    """HIP runtime API callback records through ktj_submit_sdk_api_record give the document of the
+    same calls submitted as packed runtime rows and external-correlation pairs (and the checker's)."""
+    import sdk_api_pattern as pat
+    from kineto_amd.engine import TraceEngine
+    sim = pat.sim()
+    golden_domain, golden = _golden_api_rows()
+    by_class = {}
+    for op, (line, _) in enumerate(golden):
+        by_class.setdefault(line.split()[0], []).append(op)
+    ops = by_class["kernel"] + by_class["copy"][:8] + by_class["malloc"] + by_class["default"][:5]
+    calls = [(ops[k % len(ops)], 1000 + k, B + 1000 * k, B + 1000 * k + 300 + k, 77, 100 + k % 3) for k in range(5 * len(ops))]
+
+    def base_stream():
+        b = StreamBuilder()
+        b.api(["op%d" % c for c in range(pat.n_ops())], flow_start=by_class["kernel"][:3] + by_class["copy"][:2], malloc_cid=by_class["malloc"][0])
+        for k in range(4):
+            b.add_generic("cpu_op", 0, B + 10 * k, B + 10 * k + 5, 77, 100, id=500 + k)
+        return b
+
+    # the calls as packed rows
+    b = base_stream()
+    for op, corr, t0, t1, pid, tid in calls:
+        r = abi.RuntimeRec()
+        sim.ktjsim_sdk_api_row(op, corr, pat.args_bytes(op), t0, t1, pid, tid, C.byref(r))
+        r.id = corr
+        b.runtime.append(r)
+        if corr % 2 == 0:
+            b.add_extcorr(corr, 500 + corr % 4)
+    sp = b.build()
+    ora = og.OracleRun(sp)
+    want = ora.output()
+    ora.close()
+    with TraceEngine(sp.contents.trace_name.decode(), device=0) as eng:
+        eng.submit_stream(sp)
+        eng.process()
+        rows_doc = eng.output()
+    assert rows_doc == want
+    # the same calls as SDK callback records
+    sp2 = base_stream().build()
+    with TraceEngine(sp2.contents.trace_name.decode(), device=0) as eng:
+        eng.submit_stream(sp2)
+        other = sim.ktjsim_sdk_api_record_create(sim.ktjsim_sdk_api_kind_hip_runtime() + 1, 5, 1, pat.args_bytes(5))
+        assert eng.lib.ktj_submit_sdk_api_record(eng.h, other, 1, 2, 3, 4, None, None) == 0   # not a HIP runtime API record: ignored
+        sim.ktjsim_sdk_api_record_free(other)
+        for op, corr, t0, t1, pid, tid in calls:
+            rec = sim.ktjsim_sdk_api_record_create(sim.ktjsim_sdk_api_kind_hip_runtime(), op, corr, pat.args_bytes(op))
+            ext = C.c_uint64(500 + corr % 4)
+            assert eng.lib.ktj_submit_sdk_api_record(eng.h, rec, t0, t1, pid, tid, C.byref(ext) if corr % 2 == 0 else None, None) == 0
+            sim.ktjsim_sdk_api_record_free(rec)
+        eng.process()
+        got = eng.output()
+    assert got == want
+    assert got.count(b'"cat": "cuda_runtime"') == len(calls)
