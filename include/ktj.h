@@ -31,6 +31,23 @@ extern "C" {
 #define KTJ_ERR_NOMEM (-5)    /* host or device allocation failed                               */
 #define KTJ_ERR_LIMIT (-6)    /* input exceeds a documented limit                               */
 
+/* ------------------------------------------------------------------------------------------
+ * Limits of one trace.  A trace beyond one of them is refused by ktj_process with KTJ_ERR_LIMIT
+ * and a ktj_last_error() text that names the limit; nothing is written.  The reference keeps
+ * these in node-based maps and has no such limits.
+ *   - (device, stream) pairs among the device records (the pairs that RocprofActivity's dense
+ *     stream index numbers, libkineto/src/RocprofActivity_inl.h:118-146);
+ *   - distinct hardware queue ids among the device records (used where a device record's stream
+ *     has to be found through its queue);
+ *   - (deviceId, resourceId) pairs of "Stream Sync" CUDA_SYNC activities (output_json.cpp:913-943).
+ * The number of distinct deviceId and resourceId values is not limited; above 4096 of either the
+ * sort works on the raw 64-bit values instead of ranks, which is several times slower.
+ * Record counts are limited by device memory and by 32-bit row indices (fewer than 2^32 - 16 rows).
+ * ---------------------------------------------------------------------------------------- */
+#define KTJ_MAX_STREAM_PAIRS 4096u
+#define KTJ_MAX_QUEUES 32768u
+#define KTJ_MAX_SYNC_ROWS 32768u
+
 #define KTJ_NONE 0xFFFFFFFFu  /* "no string" / "no schema" sentinel for 32-bit ids              */
 
 /* ------------------------------------------------------------------------------------------
@@ -396,10 +413,13 @@ typedef struct ktj_engine ktj_engine;
  * the same bytes.
  * KTJ_CREATE_HASH_JOIN keeps the join tables in hash mode even when the correlation ids are dense
  * enough for direct addressing (the engine chooses per table otherwise); same results, slower.
+ * KTJ_CREATE_PAIR_SORT sorts (key, arrival index) pairs also where key and index fit one 64-bit
+ * word (the engine sorts single words then otherwise); same results, slower.
  * ---------------------------------------------------------------------------------------- */
 #define KTJ_CREATE_NO_FILE 0x1u
 #define KTJ_CREATE_TILE_EMIT 0x2u
 #define KTJ_CREATE_HASH_JOIN 0x4u
+#define KTJ_CREATE_PAIR_SORT 0x8u
 int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int hip_device,
                uint32_t flags);
 void ktj_destroy(ktj_engine* e);

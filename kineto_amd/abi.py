@@ -13,6 +13,7 @@ KTJ_OK, KTJ_ERR_ARG, KTJ_ERR_STATE, KTJ_ERR_HIP, KTJ_ERR_IO, KTJ_ERR_NOMEM, KTJ_
 KTJ_CREATE_NO_FILE = 0x1
 KTJ_CREATE_TILE_EMIT = 0x2
 KTJ_CREATE_HASH_JOIN = 0x4
+KTJ_CREATE_PAIR_SORT = 0x8
 
 REC_GENERIC, REC_RUNTIME, REC_DEVICE, REC_EXTCORR, REC_USERCORR = 0, 1, 2, 3, 4
 INFO_DEVICE, INFO_RESOURCE, INFO_OVERHEAD, INFO_SPAN = 0, 1, 2, 3

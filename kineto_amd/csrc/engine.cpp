@@ -164,7 +164,7 @@ struct ktj_engine {
   DevBuf d_scalars, d_name_len, d_arg_len, d_sflags, d_name_off, d_arg_off, d_name_blob, d_arg_blob;
   DevBuf c_ts, c_dur, c_corr, c_dev, c_res, c_meta, c_ext;
   DevBuf t_full, t_narrow, t_cpu, f_has_runtime, f_first, f_stream_src, f_pay, n_ext_src, n_kern_src, n_copy_src, n_pay, slot_ext, slot_f, slot_n, dev_link, dev_brief, sync_keys, sync_pos, sync_first;
-  DevBuf q_keys, q_stream, q_amb, dn_hash, dn_first, dn_dev, dn_key, dn_rank;
+  DevBuf q_keys, q_stream, q_amb, dn_hash, dn_first, dn_dev, dn_key, dn_rank, range_parts;
   DevBuf s_dev_k, s_dev_r, s_res_k, s_res_r;
   DevBuf keys_a, keys_b, vals_a, vals_b, hist, scan_tmp;
   DevBuf mat, len, len_sorted, kind_sorted, offs, out, tile_start;
@@ -182,6 +182,7 @@ struct ktj_engine {
   /* results */
   uint64_t N = 0, prefix_len = 0, act_bytes = 0, total_bytes = 0;
   uint32_t* perm = nullptr; uint64_t* sorted_keys = nullptr;
+  int sort_mode = 0; /* 0: key and index in one word; 1: (key, index) pairs */
   Scalars scalars{};
   ktj_stats stats{};
 };
@@ -197,6 +198,23 @@ int fail_hip(ktj_engine* e, hipError_t err, const char* what) {
     hipError_t _e = (call);                                     \
     if (_e != hipSuccess) return fail_hip(e, _e, #call);        \
   } while (0)
+
+/* the ktj_last_error() text for the KTJ_DEVERR_* bits that end a pass */
+std::string limit_text(unsigned bits) {
+  std::string t;
+  auto add = [&](const std::string& x) { t += (t.empty() ? "" : "; ") + x; };
+  if (bits & KTJ_DEVERR_STREAMS)
+    add("more than KTJ_MAX_STREAM_PAIRS (" + std::to_string(KTJ_MAX_STREAM_PAIRS) + ") distinct (device, stream) pairs among the device records");
+  if (bits & KTJ_DEVERR_QUEUES)
+    add("more than KTJ_MAX_QUEUES (" + std::to_string(KTJ_MAX_QUEUES) + ") distinct hardware queues among the device records");
+  if (bits & KTJ_DEVERR_SYNC_ROWS)
+    add("more than KTJ_MAX_SYNC_ROWS (" + std::to_string(KTJ_MAX_SYNC_ROWS) + ") distinct (device, row) pairs of Stream Sync activities");
+  if (bits & KTJ_DEVERR_RECORD_TOO_LONG) add("an activity's JSON text is 1 GiB or longer");
+  if (bits & KTJ_DEVERR_HASH_COLLISION) add("two (device, stream) pairs share a 64-bit hash");
+  if (bits & KTJ_DEVERR_TABLE_FULL) add("a join table sized from the record counts is full (internal error)");
+  if (bits & (KTJ_DEVERR_DISTINCT_DEVICES | KTJ_DEVERR_DISTINCT_RESOURCES)) add("distinct-value set overflow after the sort (internal error)");
+  return "limit exceeded: " + t + " [bits " + std::to_string(bits) + "]";
+}
 
 uint32_t pow2_at_least(uint64_t v) {
   uint64_t c = 1024;
@@ -343,7 +361,7 @@ int synthesise_user_spans(ktj_engine* e, Columns c, const EmitCtx& ctx, Table t_
   NEED(e->synth_recs, recs.size() * sizeof(ktj_generic_rec) + 16);
   HIPCHK(hipMemcpyAsync(e->synth_recs.p, recs.data(), recs.size() * sizeof(ktj_generic_rec), hipMemcpyHostToDevice, st));
   HIPCHK(hipStreamSynchronize(st));
-  HIPCHK(decode_generic(e->synth_recs.as<ktj_generic_rec>(), recs.size(), c, first_row, sc, ctx, st));
+  HIPCHK(decode_generic(e->synth_recs.as<ktj_generic_rec>(), recs.size(), c, first_row, sc, ctx, nullptr, st));
   e->n_spans = recs.size();
   return KTJ_OK;
 }
@@ -364,6 +382,7 @@ int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int
   e->base_time_ns = base_time_ns;
   e->device = hip_device;
   e->flags = flags;
+  e->sort_mode = (flags & KTJ_CREATE_PAIR_SORT) ? 1 : 0;
   e->clock.scale = 1.0;
   *out = e; /* from here on errors are reported through the handle */
   if (!(flags & KTJ_CREATE_NO_FILE)) { /* openTraceFile, output_json.cpp:485-493 */
@@ -742,6 +761,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   NEED(e->s_res_k, (KTJ_SET_CAP + 1ull) * 8); NEED(e->s_res_r, (KTJ_SET_CAP + 1ull) * 4);
   NEED(e->keys_a, Na * 8); NEED(e->keys_b, Na * 8);
   NEED(e->vals_a, Na * 4); NEED(e->vals_b, Na * 4);
+  NEED(e->range_parts, (decode_blocks(ng) + 2 * decode_blocks(nr) + decode_blocks(nd) + 1) * sizeof(KeyRange));
   NEED(e->hist, radix_tmp_elems(Na) * 4);
   {
     uint64_t m = scan_tmp_elems(radix_tmp_elems(Na));
@@ -808,9 +828,10 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   HIPCHK(hipEventRecord(e->ev[EV_DICT], st));
 
   /* ---- stage 1: decode ---- */
-  HIPCHK(decode_generic(g_recs, ng, c, 0, sc, ctx, st));
-  HIPCHK(decode_runtime(r_recs, nr, c, ng, st));
-  HIPCHK(decode_device(d_recs, nd, c, ng + nr, e->dev_brief.as<DevBrief>(), st));
+  KeyRange* parts = e->range_parts.as<KeyRange>(); /* [generic | runtime | runtime narrowed | device] */
+  HIPCHK(decode_generic(g_recs, ng, c, 0, sc, ctx, parts, st));
+  HIPCHK(decode_runtime(r_recs, nr, c, ng, parts + decode_blocks(ng), parts + decode_blocks(ng) + decode_blocks(nr), st));
+  HIPCHK(decode_device(d_recs, nd, c, ng + nr, e->dev_brief.as<DevBrief>(), parts + decode_blocks(ng) + 2 * decode_blocks(nr), st));
   HIPCHK(hipEventRecord(e->ev[EV_DECODE], st));
 
   /* ---- stage 2a: clock + window ---- */
@@ -827,7 +848,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   Table t_cpu{e->t_cpu.as<uint64_t>(), cap_cpu - 1, 1u, &sc->plan.ctl[KTJ_TBL_CPU]};
   FullCols fc{e->f_has_runtime.as<uint32_t>(), e->f_first.as<uint32_t>(), e->f_stream_src.as<uint32_t>(), e->f_pay.as<FullPay>()};
   NarrowCols nc{e->n_ext_src.as<uint32_t>(), e->n_kern_src.as<uint32_t>(), e->n_copy_src.as<uint32_t>(), e->n_pay.as<NarrowPay>()};
-  HIPCHK(plan_tables(c, ng, nr, nd, x_recs, nx, cap_full, cap_narrow, cap_cpu, (e->flags & KTJ_CREATE_HASH_JOIN) != 0, sc, st));
+  HIPCHK(plan_tables(parts, ng, nr, nd, x_recs, nx, cap_full, cap_narrow, cap_cpu, (e->flags & KTJ_CREATE_HASH_JOIN) != 0, sc, st));
   HIPCHK(clear_tables(tf, fc, tn, nc, t_cpu, st));
   StreamTables stt{e->q_keys.as<uint64_t>(), e->q_stream.as<uint64_t>(), e->q_amb.as<uint32_t>(), e->dn_hash.as<uint64_t>(),
                    e->dn_first.as<uint32_t>(), e->dn_dev.as<int32_t>(), e->dn_key.as<uint64_t>(), e->dn_rank.as<uint32_t>()};
@@ -863,8 +884,9 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   HIPCHK(hipMemcpyAsync(&e->h_ctl->scalars, sc, sizeof(Scalars), hipMemcpyDeviceToHost, st));
   HIPCHK(hipStreamSynchronize(st));
   e->scalars = e->h_ctl->scalars;
-  if (e->scalars.error) {
-    e->last_error = "device-side limit hit before sort, error bits " + std::to_string(e->scalars.error);
+  const unsigned distinct_overflow = e->scalars.error & (KTJ_DEVERR_DISTINCT_DEVICES | KTJ_DEVERR_DISTINCT_RESOURCES);
+  if (e->scalars.error & ~distinct_overflow) {
+    e->last_error = limit_text(e->scalars.error);
     return KTJ_ERR_LIMIT;
   }
   uint32_t ts_bits = 0, res_bits = 0, key_bits = 0, rank_bits = 0;
@@ -876,26 +898,43 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
     rank_bits = res_bits + dev_bits;
   }
   HIPCHK(hipEventRecord(e->ev[EV_SORT_B], st));
-  if (key_bits <= 62) {
-    HIPCHK(make_keys(c, N, sets, sc, ts_bits, res_bits, key_bits, e->keys_a.as<uint64_t>(), e->vals_a.as<uint32_t>(), st));
-    HIPCHK(radix_sort(e->keys_a.as<uint64_t>(), e->vals_a.as<uint32_t>(), e->keys_b.as<uint64_t>(), e->vals_b.as<uint32_t>(),
-                      N, key_bits + 1, e->hist.as<uint32_t>(), e->scan_tmp.as<uint64_t>(), &e->sorted_keys, &e->perm, st));
-  } else {
-    /* timestamp span too wide for one composite key: stable sort by timestamp, then by ranks */
-    if (rank_bits > 62) {
-      e->last_error = "sort key needs " + std::to_string(rank_bits) + " bits for device and resource ranks";
-      return KTJ_ERR_LIMIT;
-    }
+  {
     uint64_t* ka = e->keys_a.as<uint64_t>(); uint32_t* va = e->vals_a.as<uint32_t>();
     uint64_t* kb = e->keys_b.as<uint64_t>(); uint32_t* vb = e->vals_b.as<uint32_t>();
-    HIPCHK(make_ts_keys(c, N, sc, ka, va, st));
-    HIPCHK(radix_sort(ka, va, kb, vb, N, ts_bits, e->hist.as<uint32_t>(), e->scan_tmp.as<uint64_t>(), &e->sorted_keys, &e->perm, st));
-    if (e->perm == va) { /* result in the first pair: rank keys go into the second */
-      HIPCHK(make_rank_keys(c, va, N, sets, res_bits, rank_bits, kb, vb, st));
-      HIPCHK(radix_sort(kb, vb, ka, va, N, rank_bits + 1, e->hist.as<uint32_t>(), e->scan_tmp.as<uint64_t>(), &e->sorted_keys, &e->perm, st));
+    uint32_t* hist = e->hist.as<uint32_t>(); uint64_t* scan_tmp = e->scan_tmp.as<uint64_t>();
+    /* one more stable sort on top of the order so far: keys made from the rows in that order,
+     * into the pair of buffers that does not hold it */
+    auto sort_again = [&](auto make, uint32_t bits) -> int {
+      const uint32_t* order = e->perm;
+      if (order == va) { HIPCHK(make(order, kb, vb)); HIPCHK(radix_sort(kb, vb, ka, va, N, bits, hist, scan_tmp, &e->sorted_keys, &e->perm, st)); }
+      else { HIPCHK(make(order, ka, va)); HIPCHK(radix_sort(ka, va, kb, vb, N, bits, hist, scan_tmp, &e->sorted_keys, &e->perm, st)); }
+      return KTJ_OK;
+    };
+    if (distinct_overflow) {
+      /* too many distinct deviceId or resourceId values for ranks: timestamp, then resourceId, then
+       * deviceId, each on the raw values, then dropped rows to the back */
+      HIPCHK(clear_error_bits(sc, distinct_overflow, st));
+      HIPCHK(make_ts_keys(c, N, sc, ka, va, st));
+      HIPCHK(radix_sort(ka, va, kb, vb, N, ts_bits, hist, scan_tmp, &e->sorted_keys, &e->perm, st));
+      int rc = sort_again([&](const uint32_t* o, uint64_t* k, uint32_t* v) { return make_column_keys(c.res, c.meta, o, N, 0, k, v, st); }, 64);
+      if (rc == KTJ_OK) rc = sort_again([&](const uint32_t* o, uint64_t* k, uint32_t* v) { return make_column_keys(c.dev, c.meta, o, N, 0, k, v, st); }, 64);
+      if (rc == KTJ_OK) rc = sort_again([&](const uint32_t* o, uint64_t* k, uint32_t* v) { return make_column_keys(c.dev, c.meta, o, N, 1, k, v, st); }, 1);
+      if (rc != KTJ_OK) return rc;
+    } else if (key_bits <= 62 && e->sort_mode != 1 && sort_packed_fits(N, key_bits)) {
+      HIPCHK(sort_packed(c, N, sets, sc, ts_bits, res_bits, key_bits, ka, kb, va, hist, scan_tmp, st));
+      e->perm = va;
+      e->sorted_keys = nullptr;
+    } else if (key_bits <= 62) {
+      HIPCHK(make_keys(c, N, sets, sc, ts_bits, res_bits, key_bits, ka, va, st));
+      HIPCHK(radix_sort(ka, va, kb, vb, N, key_bits + 1, hist, scan_tmp, &e->sorted_keys, &e->perm, st));
     } else {
-      HIPCHK(make_rank_keys(c, vb, N, sets, res_bits, rank_bits, ka, va, st));
-      HIPCHK(radix_sort(ka, va, kb, vb, N, rank_bits + 1, e->hist.as<uint32_t>(), e->scan_tmp.as<uint64_t>(), &e->sorted_keys, &e->perm, st));
+      /* timestamp span too wide for one composite key: stable sort by timestamp, then by ranks
+       * (at most 2 x 12 bits) */
+      HIPCHK(make_ts_keys(c, N, sc, ka, va, st));
+      HIPCHK(radix_sort(ka, va, kb, vb, N, ts_bits, hist, scan_tmp, &e->sorted_keys, &e->perm, st));
+      const int rc = sort_again([&](const uint32_t* o, uint64_t* k, uint32_t* v) { return make_rank_keys(c, o, N, sets, res_bits, rank_bits, k, v, st); },
+                                rank_bits + 1);
+      if (rc != KTJ_OK) return rc;
     }
   }
   HIPCHK(hipEventRecord(e->ev[EV_SORT], st));
@@ -936,7 +975,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   act_bytes = e->h_ctl->act_bytes;
   e->scalars = e->h_ctl->scalars;
   if (e->scalars.error) {
-    e->last_error = "device-side limit hit, error bits " + std::to_string(e->scalars.error);
+    e->last_error = limit_text(e->scalars.error);
     return KTJ_ERR_LIMIT;
   }
   std::string distributed_info;

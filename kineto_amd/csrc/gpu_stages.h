@@ -133,15 +133,22 @@ struct Scalars {
   unsigned int runtime_ids_repeat;    /* two runtime rows share a slot of the full table */
   JoinPlan plan;                      /* key ranges and modes of the join tables */
 };
-#define KTJ_DEVERR_TABLE_FULL 1u
-#define KTJ_DEVERR_TOO_MANY_DISTINCT 2u
+#define KTJ_DEVERR_TABLE_FULL 1u         /* a join table sized from the record counts filled up (a defect) */
+#define KTJ_DEVERR_DISTINCT_DEVICES 2u   /* more distinct deviceId values than the rank set holds: the sort
+                                            takes its slower path without ranks, no error reaches the caller */
 #define KTJ_DEVERR_HASH_COLLISION 4u
 #define KTJ_DEVERR_RECORD_TOO_LONG 8u
+#define KTJ_DEVERR_DISTINCT_RESOURCES 16u /* as DISTINCT_DEVICES, for resourceId values */
+#define KTJ_DEVERR_STREAMS 32u            /* more than KTJ_MAX_STREAM_PAIRS (device, stream) pairs */
+#define KTJ_DEVERR_QUEUES 64u             /* more than KTJ_MAX_QUEUES hardware queues */
+#define KTJ_DEVERR_SYNC_ROWS 128u         /* more than KTJ_MAX_SYNC_ROWS (device, row) pairs of Stream Sync events */
 
-#define KTJ_SET_CAP 16384u     /* slots of the distinct-value sets (at most half may be used) */
-#define KTJ_DENSE_CAP 8192u    /* slots of the (device, stream) table */
-#define KTJ_QUEUE_CAP 65536u   /* slots of the queue -> stream table */
-#define KTJ_SYNC_CAP 65536u    /* slots of the Stream Sync (device, row) table */
+#define KTJ_SET_CAP 16384u     /* slots of the distinct-value sets; KTJ_SET_MAX values get a rank */
+#define KTJ_SET_MAX 4096u
+#define KTJ_DENSE_CAP (2u * KTJ_MAX_STREAM_PAIRS) /* slots of the (device, stream) table */
+#define KTJ_QUEUE_CAP (2u * KTJ_MAX_QUEUES)       /* slots of the queue -> stream table */
+#define KTJ_SYNC_CAP (2u * KTJ_MAX_SYNC_ROWS)     /* slots of the Stream Sync (device, row) table */
+#define KTJ_TABLE_PROBES 256u  /* linear probing of these small tables gives up after this many slots */
 
 struct ApiTable {
   const uint32_t* cid_name_ids;
@@ -173,20 +180,27 @@ hipError_t dict_write(const char* blob, const uint64_t* off, uint32_t n, const u
                       const uint64_t* arg_off, const uint32_t* flags, char* name_blob, char* arg_blob, hipStream_t st);
 
 /* ---- stage 1: decode ---- */
+/* id_range / narrow_range: one KeyRange per workgroup (decode_blocks(n) entries), smallest and
+ * largest id of the workgroup's records; id_range of decode_generic may be null */
+uint64_t decode_blocks(uint64_t n);
 hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, Scalars* sc, EmitCtx ctx,
-                          hipStream_t st);
-hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st);
-hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, DevBrief* brief, hipStream_t st);
+                          KeyRange* id_range, hipStream_t st);
+hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, KeyRange* id_range,
+                          KeyRange* narrow_range, hipStream_t st);
+hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, DevBrief* brief, KeyRange* id_range,
+                         hipStream_t st);
 
 /* ---- stage 2a: clock conversion + window filter (runtime and device rows) ---- */
 hipError_t convert_rows(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, ClockDev clk,
                         int64_t win_start, int64_t win_end, Scalars* sc, hipStream_t st);
 
 /* ---- stage 2b: joins ---- */
-/* key ranges of the three tables, then their modes (direct unless force_hash or the span is too wide) */
-hipError_t plan_tables(Columns c, uint64_t n_generic, uint64_t n_runtime, uint64_t n_device, const ktj_extcorr_rec* e,
-                       uint64_t n_ext, uint32_t cap_full, uint32_t cap_narrow, uint32_t cap_cpu, bool force_hash,
-                       Scalars* sc, hipStream_t st);
+/* key ranges of the three tables, then their modes (direct unless force_hash or the span is too wide).
+ * parts: the decode kernels' per-workgroup ranges, laid out as [generic ids | runtime ids | runtime ids
+ * narrowed | device ids] with decode_blocks() entries each */
+hipError_t plan_tables(const KeyRange* parts, uint64_t n_generic, uint64_t n_runtime, uint64_t n_device,
+                       const ktj_extcorr_rec* e, uint64_t n_ext, uint32_t cap_full, uint32_t cap_narrow, uint32_t cap_cpu,
+                       bool force_hash, Scalars* sc, hipStream_t st);
 hipError_t clear_tables(Table tf, FullCols fc, Table tn, NarrowCols nc, Table cpu, hipStream_t st);
 hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, uint32_t* slot_ext, Scalars* sc,
                          hipStream_t st);
@@ -257,6 +271,16 @@ hipError_t make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint3
  * index, then keys = composite rank of row order[p] with vals = order[p] (dropped rows get
  * 1 << rank_bits) */
 hipError_t make_ts_keys(Columns c, uint64_t n, const Scalars* sc, uint64_t* keys, uint32_t* vals, hipStream_t st);
+/* keys[p] = sign-biased column value of row order[p] (validity != 0: 0 for kept rows, 1 for dropped ones) */
+hipError_t make_column_keys(const int64_t* column, const uint32_t* meta, const uint32_t* order, uint64_t n, int validity,
+                            uint64_t* keys, uint32_t* vals, hipStream_t st);
+hipError_t clear_error_bits(Scalars* sc, unsigned int bits, hipStream_t st);
+/* The composite-key sort on single 64-bit words (key above the arrival index); perm receives the
+ * arrival index per sorted position.  Usable when sort_packed_fits(n, key_bits). */
+bool sort_packed_fits(uint64_t n, uint32_t key_bits);
+hipError_t sort_packed(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits,
+                       uint32_t key_bits, uint64_t* buf_a, uint64_t* buf_b, uint32_t* perm, uint32_t* hist, uint64_t* scan_tmp,
+                       hipStream_t st);
 hipError_t make_rank_keys(Columns c, const uint32_t* order, uint64_t n, SortSets s, uint32_t res_bits, uint32_t rank_bits,
                           uint64_t* keys, uint32_t* vals, hipStream_t st);
 /* stable LSD radix sort of (key, val) pairs on the low `bits` bits; result ends in keys_out/vals_out

@@ -36,12 +36,14 @@ __device__ __forceinline__ uint64_t hash64(uint64_t x) {
 __device__ __forceinline__ uint32_t lane_id() { return threadIdx.x & 63u; }
 __device__ __forceinline__ uint64_t lanemask_lt() { return (1ULL << lane_id()) - 1ULL; }
 
-/* Returns the slot holding `key`, inserting it if absent; KTJ_NOSLOT when the table is full.
- * The probe sequence is bounded by the table size, so every lane leaves the loop. */
+/* Returns the slot holding `key`, inserting it if absent; KTJ_NOSLOT when no free slot lies within
+ * KTJ_TABLE_PROBES slots of the key's home slot (a table that is at most half full never gets
+ * there; one that is close to full does at once, so that an input with far too many distinct keys
+ * costs a bounded number of probes per row and is reported instead of crawling). */
 __device__ uint32_t table_insert(uint64_t* keys, uint32_t mask, uint64_t key) {
   if (key == KTJ_EMPTY_KEY) { keys[mask + 1u] = 0; return mask + 1u; }
   uint32_t slot = (uint32_t)hash64(key) & mask;
-  for (uint32_t probe = 0; probe <= mask; ++probe) {
+  for (uint32_t probe = 0; probe <= mask && probe < KTJ_TABLE_PROBES; ++probe) {
     uint64_t cur = keys[slot];
     if (cur == key) return slot;
     if (cur == KTJ_EMPTY_KEY) {
@@ -56,7 +58,7 @@ __device__ uint32_t table_insert(uint64_t* keys, uint32_t mask, uint64_t key) {
 __device__ uint32_t table_find(const uint64_t* keys, uint32_t mask, uint64_t key) {
   if (key == KTJ_EMPTY_KEY) return keys[mask + 1u] == 0 ? mask + 1u : KTJ_NOSLOT;
   uint32_t slot = (uint32_t)hash64(key) & mask;
-  for (uint32_t probe = 0; probe <= mask; ++probe) {
+  for (uint32_t probe = 0; probe <= mask && probe < KTJ_TABLE_PROBES; ++probe) {
     uint64_t cur = keys[slot];
     if (cur == key) return slot;
     if (cur == KTJ_EMPTY_KEY) return KTJ_NOSLOT;
@@ -146,7 +148,8 @@ __device__ __forceinline__ void block_add(unsigned long long* counter, uint32_t 
     if (t) atomicAdd(counter, (unsigned long long)t);
   }
 }
-#define KTJ_MAX_GRID 4096u /* grid-stride kernels: enough workgroups to fill 256 CUs several times over */
+/* grid-stride kernels: enough workgroups to fill 256 CUs several times over */
+#define KTJ_MAX_GRID 4096u
 
 __global__ void k_fill_u64(uint64_t* p, uint64_t v, uint64_t n) {
   uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -419,14 +422,36 @@ __device__ __forceinline__ const Rec* stage_records(const Rec* recs, uint64_t n,
   return reinterpret_cast<const Rec*>(stage);
 }
 
+/* Smallest and largest key of the workgroup's rows into part[blockIdx.x] (empty: lo > hi).  The
+ * join tables are planned from these ranges; collecting them here saves a pass over the ids.
+ * Must be reached by every thread of the workgroup. */
+__device__ __forceinline__ void block_key_range(bool has, uint64_t key, KeyRange* part) {
+  __shared__ unsigned long long s_lo[KTJ_BLOCK >> 6], s_hi[KTJ_BLOCK >> 6];
+  unsigned long long lo = has ? key : ~0ULL, hi = has ? key : 0ULL;
+  for (int o = 32; o > 0; o >>= 1) {
+    const unsigned long long l2 = __shfl_xor(lo, o), h2 = __shfl_xor(hi, o);
+    lo = l2 < lo ? l2 : lo;
+    hi = h2 > hi ? h2 : hi;
+  }
+  __syncthreads();
+  if (lane_id() == 0) { s_lo[threadIdx.x >> 6] = lo; s_hi[threadIdx.x >> 6] = hi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (uint32_t k = 1; k < (blockDim.x >> 6); ++k) { lo = s_lo[k] < lo ? s_lo[k] : lo; hi = s_hi[k] > hi ? s_hi[k] : hi; }
+    KeyRange r;
+    r.lo = lo; r.hi = hi;
+    part[blockIdx.x] = r;
+  }
+}
 __global__ void k_decode_generic(const ktj_generic_rec* recs, uint64_t n, Columns c, uint64_t first, Scalars* sc,
-                                 EmitCtx ctx) {
+                                 EmitCtx ctx, KeyRange* id_range) {
   __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_generic_rec) / 16];
   uint32_t cnt;
   const ktj_generic_rec* l = stage_records(recs, n, stage, &cnt);
   /* rows that may need a Stream Sync row of their own are rare: the extra passes run only if any */
   const bool sync_typed = threadIdx.x < cnt && l[threadIdx.x].type == KTJ_TYPE_CUDA_SYNC;
   if (__syncthreads_or(sync_typed ? 1 : 0)) block_add(&sc->n_sync_typed, sync_typed ? 1u : 0u);
+  if (id_range) block_key_range(threadIdx.x < cnt, threadIdx.x < cnt ? (uint64_t)(int64_t)l[threadIdx.x].id : 0, id_range);
   if (threadIdx.x >= cnt) return;
   const ktj_generic_rec g = l[threadIdx.x];
   const uint64_t a = first + (uint64_t)blockIdx.x * KTJ_BLOCK + threadIdx.x;
@@ -438,10 +463,17 @@ __global__ void k_decode_generic(const ktj_generic_rec* recs, uint64_t n, Column
   c.meta[a] = (generic_record_prints(g, ctx) ? KTJ_M_VALID : 0u) | (KTJ_CLASS_GENERIC << KTJ_M_CLASS_SHIFT);
   c.ext[a] = 0;
 }
-__global__ void k_decode_runtime(const ktj_runtime_rec* recs, uint64_t n, Columns c, uint64_t first) {
+__global__ void k_decode_runtime(const ktj_runtime_rec* recs, uint64_t n, Columns c, uint64_t first, KeyRange* id_range,
+                                 KeyRange* narrow_range) {
   __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_runtime_rec) / 16];
   uint32_t cnt;
   const ktj_runtime_rec* l = stage_records(recs, n, stage, &cnt);
+  {
+    const bool has = threadIdx.x < cnt;
+    const uint64_t id = has ? l[threadIdx.x].id : 0;
+    block_key_range(has, id, id_range);
+    block_key_range(has, narrow_corr_key(id), narrow_range);
+  }
   if (threadIdx.x >= cnt) return;
   const ktj_runtime_rec* r = &l[threadIdx.x];
   const uint64_t a = first + (uint64_t)blockIdx.x * KTJ_BLOCK + threadIdx.x;
@@ -455,10 +487,12 @@ __global__ void k_decode_runtime(const ktj_runtime_rec* recs, uint64_t n, Column
   c.meta[a] = (KTJ_CLASS_RUNTIME << KTJ_M_CLASS_SHIFT) | (kind << KTJ_M_KIND_SHIFT) | (stream != 0 ? KTJ_M_HAS_STREAM : 0u);
   c.ext[a] = 0;
 }
-__global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns c, uint64_t first, DevBrief* brief) {
+__global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns c, uint64_t first, DevBrief* brief,
+                                KeyRange* id_range) {
   __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_device_rec) / 16];
   uint32_t cnt;
   const ktj_device_rec* l = stage_records(recs, n, stage, &cnt);
+  block_key_range(threadIdx.x < cnt, threadIdx.x < cnt ? l[threadIdx.x].id : 0, id_range);
   if (threadIdx.x >= cnt) return;
   const ktj_device_rec* d = &l[threadIdx.x];
   const uint64_t a = first + (uint64_t)blockIdx.x * KTJ_BLOCK + threadIdx.x;
@@ -475,20 +509,24 @@ __global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns 
   brief[a - first] = b;
 }
 
+uint64_t decode_blocks(uint64_t n) { return grid_for(n, KTJ_BLOCK); }
 hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, Scalars* sc, EmitCtx ctx,
-                          hipStream_t st) {
+                          KeyRange* id_range, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_decode_generic, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, sc, ctx);
+  hipLaunchKernelGGL(k_decode_generic, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, sc, ctx, id_range);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, hipStream_t st) {
+hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, KeyRange* id_range,
+                          KeyRange* narrow_range, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_decode_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first);
+  hipLaunchKernelGGL(k_decode_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, id_range,
+                     narrow_range);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, DevBrief* brief, hipStream_t st) {
+hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, DevBrief* brief, KeyRange* id_range,
+                         hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_decode_device, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, brief);
+  hipLaunchKernelGGL(k_decode_device, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, brief, id_range);
   return KTJ_LAUNCH_CHECK();
 }
 
@@ -543,11 +581,17 @@ __device__ __forceinline__ void flag_error(Scalars* sc, unsigned bit) { atomicOr
 __global__ void k_key_range(const uint64_t* p, uint32_t stride, uint64_t n, int narrow, KeyRange* out) {
   __shared__ unsigned long long s_lo[KTJ_BLOCK >> 6], s_hi[KTJ_BLOCK >> 6];
   unsigned long long lo = ~0ULL, hi = 0;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    uint64_t k = p[i * stride];
-    if (narrow) k = narrow_corr_key(k);
-    lo = k < lo ? k : lo;
-    hi = k > hi ? k : hi;
+  const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i0 = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i0 < n; i0 += 4 * step) {
+    uint64_t k[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) { const uint64_t i = i0 + u * step; k[u] = i < n ? p[i * stride] : p[i0 * stride]; }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint64_t v = narrow ? narrow_corr_key(k[u]) : k[u];
+      lo = v < lo ? v : lo;
+      hi = v > hi ? v : hi;
+    }
   }
   for (int o = 32; o > 0; o >>= 1) {
     const unsigned long long l2 = __shfl_xor(lo, o), h2 = __shfl_xor(hi, o);
@@ -558,6 +602,34 @@ __global__ void k_key_range(const uint64_t* p, uint32_t stride, uint64_t n, int 
   __syncthreads();
   if (threadIdx.x == 0) {
     for (uint32_t k = 1; k < (blockDim.x >> 6); ++k) { lo = s_lo[k] < lo ? s_lo[k] : lo; hi = s_hi[k] > hi ? s_hi[k] : hi; }
+    if (lo <= hi) { atomicMin(&out->lo, lo); atomicMax(&out->hi, hi); }
+  }
+}
+/* the per-workgroup ranges of the decode kernels into the plan's ranges: one workgroup per job */
+struct RangeJobs {
+  const KeyRange* src[4];
+  uint64_t n[4];
+  uint32_t dst[4]; /* KTJ_TBL_* */
+};
+__global__ void k_merge_ranges(RangeJobs jobs, Scalars* sc) {
+  __shared__ unsigned long long s_lo[1024 >> 6], s_hi[1024 >> 6];
+  const KeyRange* src = jobs.src[blockIdx.x];
+  const uint64_t n = jobs.n[blockIdx.x];
+  unsigned long long lo = ~0ULL, hi = 0;
+  for (uint64_t i = threadIdx.x; i < n; i += blockDim.x) {
+    const KeyRange r = src[i];
+    if (r.lo <= r.hi) { lo = r.lo < lo ? r.lo : lo; hi = r.hi > hi ? r.hi : hi; }
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    const unsigned long long l2 = __shfl_xor(lo, o), h2 = __shfl_xor(hi, o);
+    lo = l2 < lo ? l2 : lo;
+    hi = h2 > hi ? h2 : hi;
+  }
+  if (lane_id() == 0) { s_lo[threadIdx.x >> 6] = lo; s_hi[threadIdx.x >> 6] = hi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (uint32_t k = 1; k < (blockDim.x >> 6); ++k) { lo = s_lo[k] < lo ? s_lo[k] : lo; hi = s_hi[k] > hi ? s_hi[k] : hi; }
+    KeyRange* out = &sc->plan.range[jobs.dst[blockIdx.x]];
     if (lo <= hi) { atomicMin(&out->lo, lo); atomicMax(&out->hi, hi); }
   }
 }
@@ -604,22 +676,24 @@ __global__ void k_clear_narrow(Table t, NarrowCols c) {
   }
 }
 
-hipError_t plan_tables(Columns c, uint64_t n_generic, uint64_t n_runtime, uint64_t n_device, const ktj_extcorr_rec* e,
-                       uint64_t n_ext, uint32_t cap_full, uint32_t cap_narrow, uint32_t cap_cpu, bool force_hash,
-                       Scalars* sc, hipStream_t st) {
+hipError_t plan_tables(const KeyRange* parts, uint64_t n_generic, uint64_t n_runtime, uint64_t n_device,
+                       const ktj_extcorr_rec* e, uint64_t n_ext, uint32_t cap_full, uint32_t cap_narrow, uint32_t cap_cpu,
+                       bool force_hash, Scalars* sc, hipStream_t st) {
   const dim3 b(KTJ_BLOCK);
-  auto grid = [](uint64_t n) { const uint64_t g = (n + KTJ_BLOCK * 8 - 1) / (KTJ_BLOCK * 8); return dim3((unsigned)(g < 1024 ? (g ? g : 1) : 1024)); };
-  if (n_runtime + n_device)
-    hipLaunchKernelGGL(k_key_range, grid(n_runtime + n_device), b, 0, st, c.corr + n_generic, 1u, n_runtime + n_device, 0,
-                       &sc->plan.range[KTJ_TBL_FULL]);
-  if (n_runtime)
-    hipLaunchKernelGGL(k_key_range, grid(n_runtime), b, 0, st, c.corr + n_generic, 1u, n_runtime, 1,
-                       &sc->plan.range[KTJ_TBL_NARROW]);
+  /* parts: [generic ids | runtime ids | runtime ids narrowed | device ids], decode_blocks() entries each */
+  const uint64_t bg = decode_blocks(n_generic), br = decode_blocks(n_runtime), bd = decode_blocks(n_device);
+  RangeJobs jobs;
+  uint32_t n_jobs = 0;
+  auto job = [&](const KeyRange* src, uint64_t n, uint32_t dst) { if (n) { jobs.src[n_jobs] = src; jobs.n[n_jobs] = n; jobs.dst[n_jobs] = dst; ++n_jobs; } };
+  job(parts, bg, KTJ_TBL_CPU);
+  job(parts + bg, br, KTJ_TBL_FULL);
+  job(parts + bg + br, br, KTJ_TBL_NARROW);
+  job(parts + bg + 2 * br, bd, KTJ_TBL_FULL);
+  for (uint32_t k = n_jobs; k < 4; ++k) { jobs.src[k] = nullptr; jobs.n[k] = 0; jobs.dst[k] = 0; }
+  if (n_jobs) hipLaunchKernelGGL(k_merge_ranges, dim3(n_jobs), dim3(1024), 0, st, jobs, sc);
   if (n_ext)
-    hipLaunchKernelGGL(k_key_range, grid(n_ext), b, 0, st, reinterpret_cast<const uint64_t*>(e), 2u, n_ext, 0,
-                       &sc->plan.range[KTJ_TBL_NARROW]);
-  if (n_generic)
-    hipLaunchKernelGGL(k_key_range, grid(n_generic), b, 0, st, c.corr, 1u, n_generic, 0, &sc->plan.range[KTJ_TBL_CPU]);
+    hipLaunchKernelGGL(k_key_range, dim3(n_ext < 512ull * KTJ_BLOCK * 4 ? grid_for(n_ext, KTJ_BLOCK * 4) : 512u), b, 0, st, reinterpret_cast<const uint64_t*>(e), 2u,
+                       n_ext, 0, &sc->plan.range[KTJ_TBL_NARROW]);
   hipLaunchKernelGGL(k_plan_tables, dim3(1), dim3(64), 0, st, sc, cap_full, cap_narrow, cap_cpu, force_hash ? 1 : 0);
   return KTJ_LAUNCH_CHECK();
 }
@@ -690,17 +764,26 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Tabl
   const bool have_stream_src = sc->have_stream_src != 0;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t a = first_device + i;
+    /* all reads first (the row's columns, then one slot of each table), all writes after them:
+     * the round trips overlap instead of queueing behind each other */
     const uint64_t id = c.corr[a];
     const uint32_t meta = c.meta[a];
+    int64_t res = c.res[a];
+    const int64_t t2 = c.ts[a];
     const uint32_t domain = (meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
     const bool valid = (meta & KTJ_M_VALID) != 0;
+    const uint32_t sn = slot_find(tn, narrow_corr_key(id));
+    const uint32_t sf = valid ? slot_insert(tf, id) : slot_find(tf, id);
+    NarrowPay np;
+    np.ext_val = 0; np.info = 0; np.pay[0] = np.pay[1] = np.pay[2] = 0;
+    FullPay fp;
+    fp.first_ts = 0; fp.stream = 0;
+    uint32_t runtime_bits = 0;
+    if (sn != KTJ_NOSLOT) np = nc.pay[sn];
+    if (sf != KTJ_NOSLOT) { fp = fc.pay[sf]; runtime_bits = fc.has_runtime[sf >> 5]; }
     DevLink l;
     l.p[0] = l.p[1] = l.p[2] = 0; l.flags = 0; l.coll = 0;
-    int32_t ext = 0;
-    const uint32_t sn = slot_find(tn, narrow_corr_key(id));
     if (sn != KTJ_NOSLOT) {
-      const NarrowPay np = nc.pay[sn];
-      ext = np.ext_val;
       if ((np.info & KTJ_NP_LINKED) && valid) ++n_linked;
       if (domain != KTJ_DOM_MEMSET && (np.info & KTJ_NP_KIND_MASK) != 0) {
         l.flags = np.info & KTJ_NP_KIND_MASK;
@@ -708,18 +791,12 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Tabl
       }
       l.coll = np.info >> KTJ_NP_COLL_SHIFT;
     }
-    c.ext[a] = ext;
-    int64_t res = c.res[a];
-    uint32_t sf;
-    if (valid) {
-      sf = slot_insert(tf, id);
-      if (sf == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
-    } else sf = slot_find(tf, id);
+    c.ext[a] = np.ext_val;
+    if (valid && sf == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
     if (sf != KTJ_NOSLOT) {
-      const FullPay fp = fc.pay[sf];
       if (valid) {
-        if ((fc.has_runtime[sf >> 5] >> (sf & 31u)) & 1u) { /* act1 = the first runtime row, act2 = this row */
-          const int64_t t1 = fp.first_ts, t2 = c.ts[a];
+        if ((runtime_bits >> (sf & 31u)) & 1u) { /* act1 = the first runtime row, act2 = this row */
+          const int64_t t1 = fp.first_ts;
           if (t2 != 0 && t1 > t2) ++n_bad;
         } else {
           if (fc.first[sf] > (uint32_t)a) atomicMin(&fc.first[sf], (uint32_t)a);
@@ -901,7 +978,7 @@ __global__ void k_queue_build(const DevBrief* d, uint64_t n, Columns c, uint64_t
   const uint64_t queue = d[i].queue;
   if (!is_async_op(d[i].domain) || stream == 0 || queue == 0) return;
   const uint32_t slot = table_insert(t.q_keys, KTJ_QUEUE_CAP - 1u, queue);
-  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
+  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_QUEUES); return; }
   unsigned long long cur = t.q_stream[slot];
   if (cur == 0) cur = atomicCAS((unsigned long long*)&t.q_stream[slot], 0ULL, (unsigned long long)stream);
   if (cur != 0 && cur != stream) t.q_amb[slot] = 1u;
@@ -954,7 +1031,7 @@ __global__ void k_dense_first(const DevBrief* d, uint64_t n, Columns c, uint64_t
     }
     if (!placed) { /* local table crowded: straight to the global one */
       const uint32_t g = table_insert(t.d_hash, KTJ_DENSE_CAP - 1u, h);
-      if (g == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT);
+      if (g == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_STREAMS);
       else if (t.d_first[g] > (uint32_t)i) atomicMin(&t.d_first[g], (uint32_t)i);
     }
   }
@@ -963,7 +1040,7 @@ __global__ void k_dense_first(const DevBrief* d, uint64_t n, Columns c, uint64_t
     const unsigned long long h = l_key[k];
     if (h == KTJ_EMPTY_KEY) continue;
     const uint32_t g = table_insert(t.d_hash, KTJ_DENSE_CAP - 1u, h);
-    if (g == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT); continue; }
+    if (g == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_STREAMS); continue; }
     if (t.d_first[g] > l_min[k]) atomicMin(&t.d_first[g], l_min[k]);
   }
 }
@@ -980,7 +1057,7 @@ __global__ void k_dense_owner(const DevBrief* d, uint64_t n, Columns c, uint64_t
   if (t.d_first[slot] == (uint32_t)i) { t.d_dev[slot] = d[i].device; t.d_key[slot] = key; }
 }
 /* pass 3c (one workgroup): index = 1 + number of pairs of the same device seen earlier */
-#define KTJ_DENSE_MAX 4096
+#define KTJ_DENSE_MAX KTJ_MAX_STREAM_PAIRS
 __global__ void k_dense_rank(StreamTables t, Scalars* sc) {
   __shared__ uint32_t slots[KTJ_DENSE_MAX];
   __shared__ uint32_t count;
@@ -995,7 +1072,7 @@ __global__ void k_dense_rank(StreamTables t, Scalars* sc) {
   }
   __syncthreads();
   const uint32_t m = count;
-  if (m > KTJ_DENSE_MAX) { if (threadIdx.x == 0) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT); return; }
+  if (m > KTJ_DENSE_MAX) { if (threadIdx.x == 0) flag_error(sc, KTJ_DEVERR_STREAMS); return; }
   if (threadIdx.x == 0) sc->n_dense = m;
   for (uint32_t k = threadIdx.x; k < m; k += blockDim.x) {
     const uint32_t s = slots[k];
@@ -1046,7 +1123,6 @@ hipError_t backfill_streams(const DevBrief* d, uint64_t n, Columns c, uint64_t f
 /* ------------------------------------------------------------------------------------------ */
 /* stage 3: canonical order = stable sort by (deviceId, resourceId, timestamp), signed            */
 /* ------------------------------------------------------------------------------------------ */
-#define KTJ_SET_MAX 4096
 /* Workgroup-local set in LDS in front of the global set: a value reaches the global table once
  * per workgroup instead of once per row.  (All rows share a handful of device/resource ids, and
  * millions of probes of the same few global slots serialise in L2.)  Returns true when the
@@ -1067,6 +1143,15 @@ __device__ __forceinline__ bool local_set_first(unsigned long long* lds, uint64_
   }
   return true;
 }
+/* a wavefront's rows mostly share one value: only one lane of those that hold the value of the
+ * first active lane goes on to probe, and lanes with another value probe for themselves */
+__device__ __forceinline__ bool wave_representative(uint64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  const uint64_t first = ((uint64_t)hi << 32) | lo;
+  const uint64_t same = __ballot(v == first); /* never empty: the first active lane is in it */
+  return v != first || (uint32_t)__builtin_ctzll(same) == lane_id();
+}
+#define COLLECT_ROWS 4
 __global__ void k_collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* sc) {
   __shared__ uint64_t red_min[KTJ_BLOCK >> 6], red_max[KTJ_BLOCK >> 6];
   __shared__ unsigned long long seen_dev[LOCAL_SET_SLOTS], seen_res[LOCAL_SET_SLOTS];
@@ -1074,19 +1159,33 @@ __global__ void k_collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* s
   __syncthreads();
   uint64_t mn = ~0ULL, mx = 0ULL;
   uint32_t n_valid = 0;
-  for (uint64_t a = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; a < n; a += (uint64_t)gridDim.x * blockDim.x) {
-    if (!(c.meta[a] & KTJ_M_VALID)) continue;
-    const uint64_t dev = (uint64_t)c.dev[a], res = (uint64_t)c.res[a];
-    if (dev == KTJ_EMPTY_KEY || local_set_first(seen_dev, dev)) {
-      if (table_insert(s.dev_keys, KTJ_SET_CAP - 1u, dev) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT);
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t a0 = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; a0 < n; a0 += stride * COLLECT_ROWS) {
+    uint32_t meta[COLLECT_ROWS];
+    uint64_t dev[COLLECT_ROWS], res[COLLECT_ROWS], ts[COLLECT_ROWS];
+#pragma unroll
+    for (int r = 0; r < COLLECT_ROWS; ++r) { /* all loads of the group in flight together */
+      const uint64_t a = a0 + (uint64_t)r * stride;
+      const bool in = a < n;
+      meta[r] = in ? c.meta[a] : 0u;
+      dev[r] = in ? (uint64_t)c.dev[a] : 0;
+      res[r] = in ? (uint64_t)c.res[a] : 0;
+      ts[r] = in ? (uint64_t)c.ts[a] : 0;
     }
-    if (res == KTJ_EMPTY_KEY || local_set_first(seen_res, res)) {
-      if (table_insert(s.res_keys, KTJ_SET_CAP - 1u, res) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT);
+#pragma unroll
+    for (int r = 0; r < COLLECT_ROWS; ++r) {
+      if (!(meta[r] & KTJ_M_VALID)) continue;
+      if (wave_representative(dev[r]) && (dev[r] == KTJ_EMPTY_KEY || local_set_first(seen_dev, dev[r]))) {
+        if (table_insert(s.dev_keys, KTJ_SET_CAP - 1u, dev[r]) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_DISTINCT_DEVICES);
+      }
+      if (wave_representative(res[r]) && (res[r] == KTJ_EMPTY_KEY || local_set_first(seen_res, res[r]))) {
+        if (table_insert(s.res_keys, KTJ_SET_CAP - 1u, res[r]) == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_DISTINCT_RESOURCES);
+      }
+      const uint64_t tb = ts[r] ^ 0x8000000000000000ULL;
+      mn = tb < mn ? tb : mn;
+      mx = tb > mx ? tb : mx;
+      ++n_valid;
     }
-    const uint64_t tb = (uint64_t)c.ts[a] ^ 0x8000000000000000ULL;
-    mn = tb < mn ? tb : mn;
-    mx = tb > mx ? tb : mx;
-    ++n_valid;
   }
   for (int o = 32; o > 0; o >>= 1) {
     const uint64_t on = __shfl_xor((unsigned long long)mn, o), ox = __shfl_xor((unsigned long long)mx, o);
@@ -1100,9 +1199,9 @@ __global__ void k_collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* s
       mn = red_min[k] < mn ? red_min[k] : mn;
       mx = red_max[k] > mx ? red_max[k] : mx;
     }
-    if (mn <= mx) {
-      atomicMin(&sc->ts_min_biased, (unsigned long long)mn);
-      atomicMax(&sc->ts_max_biased, (unsigned long long)mx);
+    if (mn <= mx) { /* the atomics only where the workgroup widens the range (rare after the first few) */
+      if (mn < sc->ts_min_biased) atomicMin(&sc->ts_min_biased, (unsigned long long)mn);
+      if (mx > sc->ts_max_biased) atomicMax(&sc->ts_max_biased, (unsigned long long)mx);
     }
   }
   block_add(&sc->n_valid, n_valid);
@@ -1125,7 +1224,10 @@ __global__ void k_rank_distinct(SortSets s, Scalars* sc) {
   }
   __syncthreads();
   const uint32_t m = count;
-  if (m > KTJ_SET_MAX) { if (threadIdx.x == 0) flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT); return; }
+  if (m > KTJ_SET_MAX) {
+    if (threadIdx.x == 0) flag_error(sc, blockIdx.x == 0 ? KTJ_DEVERR_DISTINCT_DEVICES : KTJ_DEVERR_DISTINCT_RESOURCES);
+    return;
+  }
   if (threadIdx.x == 0) { if (blockIdx.x == 0) sc->n_dev_ranks = m; else sc->n_res_ranks = m; }
   for (uint32_t k = threadIdx.x; k < m; k += blockDim.x) {
     const int64_t v = vals[k];
@@ -1134,16 +1236,27 @@ __global__ void k_rank_distinct(SortSets s, Scalars* sc) {
     rank[slots[k]] = r;
   }
 }
+/* Rank of a value through its set.  The rows of a wavefront mostly share one value: then a single
+ * lookup with a wavefront-uniform key (which the compiler can keep on the scalar unit) serves all
+ * lanes. */
+__device__ __forceinline__ uint64_t set_rank(const uint64_t* keys, const uint32_t* rank, uint64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  const uint64_t first = ((uint64_t)hi << 32) | lo;
+  if (__ballot(v != first) == 0) {
+    const uint32_t slot = table_find(keys, KTJ_SET_CAP - 1u, first);
+    return slot != KTJ_NOSLOT ? rank[slot] : 0;
+  }
+  const uint32_t slot = table_find(keys, KTJ_SET_CAP - 1u, v);
+  return slot != KTJ_NOSLOT ? rank[slot] : 0;
+}
 __global__ void k_make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits,
                             uint32_t key_bits, uint64_t* keys, uint32_t* vals) {
   const uint64_t a = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (a >= n) return;
   uint64_t key = key_bits >= 64 ? ~0ULL : (1ULL << key_bits); /* dropped rows sort behind everything */
   if (c.meta[a] & KTJ_M_VALID) {
-    const uint32_t sd = table_find(s.dev_keys, KTJ_SET_CAP - 1u, (uint64_t)c.dev[a]);
-    const uint32_t sr = table_find(s.res_keys, KTJ_SET_CAP - 1u, (uint64_t)c.res[a]);
-    const uint64_t rd = sd != KTJ_NOSLOT ? s.dev_rank[sd] : 0;
-    const uint64_t rr = sr != KTJ_NOSLOT ? s.res_rank[sr] : 0;
+    const uint64_t rd = set_rank(s.dev_keys, s.dev_rank, (uint64_t)c.dev[a]);
+    const uint64_t rr = set_rank(s.res_keys, s.res_rank, (uint64_t)c.res[a]);
     const uint64_t rel = ((uint64_t)c.ts[a] ^ 0x8000000000000000ULL) - sc->ts_min_biased;
     uint64_t hi = (rd << res_bits) | rr;
     key = ts_bits >= 64 ? rel : ((hi << ts_bits) | rel);
@@ -1168,14 +1281,36 @@ __global__ void k_make_rank_keys(Columns c, const uint32_t* order, uint64_t n, S
   const uint32_t a = order[p];
   uint64_t key = 1ULL << rank_bits; /* dropped rows sort behind everything */
   if (c.meta[a] & KTJ_M_VALID) {
-    const uint32_t sd = table_find(s.dev_keys, KTJ_SET_CAP - 1u, (uint64_t)c.dev[a]);
-    const uint32_t sr = table_find(s.res_keys, KTJ_SET_CAP - 1u, (uint64_t)c.res[a]);
-    const uint64_t rd = sd != KTJ_NOSLOT ? s.dev_rank[sd] : 0;
-    const uint64_t rr = sr != KTJ_NOSLOT ? s.res_rank[sr] : 0;
+    const uint64_t rd = set_rank(s.dev_keys, s.dev_rank, (uint64_t)c.dev[a]);
+    const uint64_t rr = set_rank(s.res_keys, s.res_rank, (uint64_t)c.res[a]);
     key = (rd << res_bits) | rr;
   }
   keys[p] = key;
   vals[p] = a;
+}
+/* Traces with more distinct deviceId or resourceId values than the rank sets hold are ordered by
+ * the raw values: one more stable sort per column (sign-biased 64-bit keys), and a last one that
+ * moves the dropped rows behind the kept ones. */
+__global__ void k_make_column_keys(const int64_t* column, const uint32_t* meta, const uint32_t* order, uint64_t n, int validity,
+                                   uint64_t* keys, uint32_t* vals) {
+  const uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n) return;
+  const uint32_t a = order[p];
+  const bool valid = (meta[a] & KTJ_M_VALID) != 0;
+  keys[p] = validity ? (valid ? 0ull : 1ull) : (valid ? ((uint64_t)column[a] ^ 0x8000000000000000ULL) : 0ull);
+  vals[p] = a;
+}
+hipError_t make_column_keys(const int64_t* column, const uint32_t* meta, const uint32_t* order, uint64_t n, int validity,
+                            uint64_t* keys, uint32_t* vals, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_make_column_keys, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, column, meta, order, n, validity,
+                     keys, vals);
+  return KTJ_LAUNCH_CHECK();
+}
+__global__ void k_clear_error_bits(Scalars* sc, unsigned int bits) { sc->error &= ~bits; }
+hipError_t clear_error_bits(Scalars* sc, unsigned int bits, hipStream_t st) {
+  hipLaunchKernelGGL(k_clear_error_bits, dim3(1), dim3(1), 0, st, sc, bits);
+  return KTJ_LAUNCH_CHECK();
 }
 hipError_t make_ts_keys(Columns c, uint64_t n, const Scalars* sc, uint64_t* keys, uint32_t* vals, hipStream_t st) {
   if (n == 0) return hipSuccess;
@@ -1332,6 +1467,236 @@ hipError_t radix_sort(uint64_t* keys_a, uint32_t* vals_a, uint64_t* keys_b, uint
   return KTJ_LAUNCH_CHECK();
 }
 
+/* ---- the same sort on single 64-bit words ----
+ * When the composite key and the arrival index fit one word, the sort moves 8 bytes per row and
+ * pass instead of 12 and needs no separate index array.  The first pass reads the full keys
+ * (arrival index = position) and consumes their lowest digit, so the words it writes hold only
+ * the remaining key bits above the index: word = (key >> BITS) << idx_bits | index.  Later passes
+ * take their digit from the word; the last one writes the bare indices.  The per-tile digit
+ * counts of the first pass come from the kernel that builds the keys. */
+enum { SORTP_KEYS_TO_WORDS = 0, SORTP_WORDS_TO_WORDS = 1, SORTP_WORDS_TO_PERM = 2, SORTP_KEYS_TO_PERM = 3 };
+template <int BITS, int THREADS> struct SortP {
+  static constexpr int NB = 1 << BITS;
+  static constexpr int WAVES = THREADS / 64;
+  static constexpr int ITEMS = 16;
+  static constexpr int TILE = THREADS * ITEMS;
+  static constexpr int WAVE_KEYS = 64 * ITEMS;
+  static_assert(NB % THREADS == 0 || THREADS % NB == 0, "digits and threads must divide");
+};
+
+template <int BITS, int THREADS>
+__global__ void __launch_bounds__(THREADS)
+k_sortp_make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits, uint32_t key_bits,
+                  uint64_t* keys, uint32_t* hist, uint32_t n_blocks) {
+  using P = SortP<BITS, THREADS>;
+  __shared__ uint32_t h[P::NB];
+  for (int d = threadIdx.x; d < P::NB; d += THREADS) h[d] = 0;
+  __syncthreads();
+  const uint64_t base = (uint64_t)blockIdx.x * P::TILE;
+  const uint64_t ts_min = sc->ts_min_biased;
+  constexpr int G = 4; /* rows per thread whose loads are in flight together */
+  for (int r0 = 0; r0 < P::ITEMS; r0 += G) {
+    uint32_t meta[G];
+    uint64_t dev[G], res[G], ts[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const uint64_t a = base + (uint64_t)(r0 + g) * THREADS + threadIdx.x;
+      const bool in = a < n;
+      meta[g] = in ? c.meta[a] : 0u;
+      dev[g] = in ? (uint64_t)c.dev[a] : 0;
+      res[g] = in ? (uint64_t)c.res[a] : 0;
+      ts[g] = in ? (uint64_t)c.ts[a] : 0;
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const uint64_t a = base + (uint64_t)(r0 + g) * THREADS + threadIdx.x;
+      if (a >= n) continue;
+      uint64_t key = 1ULL << key_bits; /* dropped rows sort behind everything */
+      if (meta[g] & KTJ_M_VALID) {
+        const uint64_t rd = set_rank(s.dev_keys, s.dev_rank, dev[g]);
+        const uint64_t rr = set_rank(s.res_keys, s.res_rank, res[g]);
+        const uint64_t rel = (ts[g] ^ 0x8000000000000000ULL) - ts_min;
+        key = ((((rd << res_bits) | rr)) << ts_bits) | rel;
+      }
+      keys[a] = key;
+      atomicAdd(&h[(uint32_t)key & (P::NB - 1u)], 1u);
+    }
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < P::NB; d += THREADS) hist[(uint64_t)d * n_blocks + blockIdx.x] = h[d]; /* digit-major */
+}
+template <int BITS, int THREADS>
+__global__ void __launch_bounds__(THREADS)
+k_sortp_hist(const uint64_t* words, uint64_t n, uint32_t shift, uint32_t* hist, uint32_t n_blocks) {
+  using P = SortP<BITS, THREADS>;
+  __shared__ uint32_t h[P::NB];
+  for (int d = threadIdx.x; d < P::NB; d += THREADS) h[d] = 0;
+  __syncthreads();
+  const uint64_t base = (uint64_t)blockIdx.x * P::TILE;
+#pragma unroll
+  for (int r = 0; r < P::ITEMS; ++r) {
+    const uint64_t i = base + (uint64_t)r * THREADS + threadIdx.x;
+    if (i < n) atomicAdd(&h[(uint32_t)(words[i] >> shift) & (P::NB - 1u)], 1u);
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < P::NB; d += THREADS) hist[(uint64_t)d * n_blocks + blockIdx.x] = h[d];
+}
+template <int BITS, int THREADS, int MODE>
+__global__ void __launch_bounds__(THREADS)
+k_sortp_scatter(const uint64_t* in, uint64_t* words_out, uint32_t* perm_out, uint64_t n, uint32_t shift, uint32_t idx_bits,
+                const uint32_t* hist_scanned, uint32_t n_blocks) {
+  using P = SortP<BITS, THREADS>;
+  constexpr bool FROM_KEYS = MODE == SORTP_KEYS_TO_WORDS || MODE == SORTP_KEYS_TO_PERM;
+  constexpr bool TO_PERM = MODE == SORTP_WORDS_TO_PERM || MODE == SORTP_KEYS_TO_PERM;
+  __shared__ uint64_t s_word[P::TILE];
+  __shared__ uint16_t s_digit[FROM_KEYS ? P::TILE : 1]; /* the first pass's digit is no longer part of the word */
+  __shared__ uint32_t wave_run[P::WAVES][P::NB]; /* count per (wavefront, digit), then its start inside the digit's run */
+  __shared__ uint32_t digit_start[P::NB];        /* start of the digit's run inside the tile     */
+  __shared__ uint32_t base_of[P::NB];            /* global offset of this tile's run per digit   */
+  __shared__ uint32_t wave_tot[P::WAVES];
+  for (int d = threadIdx.x; d < P::NB; d += THREADS) {
+    base_of[d] = hist_scanned[(uint64_t)d * n_blocks + blockIdx.x];
+    for (int k = 0; k < P::WAVES; ++k) wave_run[k][d] = 0;
+  }
+  __syncthreads();
+  const uint32_t w = threadIdx.x >> 6, lane = lane_id();
+  const uint64_t lt = lanemask_lt();
+  const uint64_t tile_base = (uint64_t)blockIdx.x * P::TILE;
+  const uint64_t chunk = tile_base + (uint64_t)w * P::WAVE_KEYS;
+  volatile uint32_t* my_run = wave_run[w];
+  uint64_t word[P::ITEMS];
+  uint32_t rank[P::ITEMS];
+  uint16_t dig[P::ITEMS];
+#pragma unroll
+  for (int r = 0; r < P::ITEMS; ++r) {
+    const uint64_t i = chunk + (uint64_t)r * 64u + lane;
+    word[r] = i < n ? in[i] : ~0ULL;
+  }
+#pragma unroll
+  for (int r = 0; r < P::ITEMS; ++r) {
+    const uint64_t i = chunk + (uint64_t)r * 64u + lane;
+    const bool valid = i < n;
+    uint32_t digit;
+    if (FROM_KEYS) {
+      digit = (uint32_t)word[r] & (P::NB - 1u);
+      word[r] = (MODE == SORTP_KEYS_TO_PERM) ? i : ((((word[r] >> BITS)) << idx_bits) | i);
+    } else {
+      digit = (uint32_t)(word[r] >> shift) & (P::NB - 1u);
+    }
+    dig[r] = (uint16_t)digit;
+    /* lanes of this wavefront holding the same digit */
+    uint64_t peers = __ballot(valid ? 1 : 0);
+#pragma unroll
+    for (int b = 0; b < BITS; ++b) {
+      const uint64_t bal = __ballot((digit >> b) & 1u);
+      peers &= ((digit >> b) & 1u) ? bal : ~bal;
+    }
+    const uint32_t rank_in_wave = (uint32_t)__popcll(peers & lt);
+    const uint32_t before = my_run[digit];   /* same digit in earlier rounds of this wavefront */
+    rank[r] = before + rank_in_wave;
+    if (valid && rank_in_wave == 0) my_run[digit] = before + (uint32_t)__popcll(peers);
+  }
+  __syncthreads();
+  {
+    /* per digit: wavefront counts -> starts inside the digit's run; digit totals -> exclusive scan.
+     * A thread owns K consecutive digits (or none, where there are more threads than digits). */
+    constexpr int K = P::NB >= THREADS ? P::NB / THREADS : 1;
+    const bool owner = (int)threadIdx.x * K < P::NB;
+    uint32_t tot[K], sum = 0;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      uint32_t t = 0;
+      if (owner) {
+        const int d = (int)threadIdx.x * K + j;
+        for (int k = 0; k < P::WAVES; ++k) { const uint32_t cnt = wave_run[k][d]; wave_run[k][d] = t; t += cnt; }
+      }
+      tot[j] = t;
+      sum += t;
+    }
+    uint32_t inc = sum;
+    for (int o = 1; o < 64; o <<= 1) { const uint32_t t = __shfl_up(inc, o); if (lane >= (uint32_t)o) inc += t; }
+    if (lane == 63) wave_tot[w] = inc;
+    __syncthreads();
+    uint32_t start = inc - sum;
+    for (uint32_t k = 0; k < w; ++k) start += wave_tot[k];
+    if (owner) {
+#pragma unroll
+      for (int j = 0; j < K; ++j) { digit_start[(int)threadIdx.x * K + j] = start; start += tot[j]; }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < P::ITEMS; ++r) {
+    if (chunk + (uint64_t)r * 64u + lane < n) {
+      const uint32_t digit = dig[r];
+      const uint32_t p = digit_start[digit] + wave_run[w][digit] + rank[r];
+      s_word[p] = word[r];
+      if (FROM_KEYS) s_digit[p] = dig[r];
+    }
+  }
+  __syncthreads();
+  const uint32_t cnt = (uint32_t)(n - tile_base < (uint64_t)P::TILE ? n - tile_base : (uint64_t)P::TILE);
+  const uint64_t idx_mask = idx_bits >= 64 ? ~0ULL : ((1ULL << idx_bits) - 1ULL);
+  for (uint32_t p = threadIdx.x; p < cnt; p += THREADS) {
+    const uint64_t v = s_word[p];
+    const uint32_t digit = FROM_KEYS ? (uint32_t)s_digit[p] : ((uint32_t)(v >> shift) & (P::NB - 1u));
+    const uint64_t dst = (uint64_t)base_of[digit] + (p - digit_start[digit]);
+    if (TO_PERM) perm_out[dst] = (uint32_t)(v & idx_mask);
+    else words_out[dst] = v;
+  }
+}
+
+template <int BITS, int THREADS>
+static hipError_t sort_packed_t(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits,
+                                uint32_t key_bits, uint32_t idx_bits, uint64_t* buf_a, uint64_t* buf_b, uint32_t* perm,
+                                uint32_t* hist, uint64_t* scan_tmp, hipStream_t st) {
+  using P = SortP<BITS, THREADS>;
+  const uint32_t n_blocks = (uint32_t)((n + P::TILE - 1) / P::TILE);
+  const uint32_t total_bits = key_bits + 1u;
+  const uint32_t passes = (total_bits + BITS - 1) / BITS;
+  const dim3 g(n_blocks), b(THREADS);
+  hipLaunchKernelGGL((k_sortp_make_keys<BITS, THREADS>), g, b, 0, st, c, n, s, sc, ts_bits, res_bits, key_bits, buf_a, hist, n_blocks);
+  hipError_t e = scan_u32_inplace(hist, (uint64_t)P::NB * n_blocks, scan_tmp, st);
+  if (e != hipSuccess) return e;
+  if (passes == 1) {
+    hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_KEYS_TO_PERM>), g, b, 0, st, (const uint64_t*)buf_a, buf_b, perm, n,
+                       0u, idx_bits, (const uint32_t*)hist, n_blocks);
+    return KTJ_LAUNCH_CHECK();
+  }
+  hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_KEYS_TO_WORDS>), g, b, 0, st, (const uint64_t*)buf_a, buf_b, perm, n,
+                     0u, idx_bits, (const uint32_t*)hist, n_blocks);
+  uint64_t* in = buf_b; uint64_t* out = buf_a;
+  for (uint32_t p = 1; p < passes; ++p) {
+    const uint32_t shift = idx_bits + (p - 1u) * BITS;
+    hipLaunchKernelGGL((k_sortp_hist<BITS, THREADS>), g, b, 0, st, (const uint64_t*)in, n, shift, hist, n_blocks);
+    e = scan_u32_inplace(hist, (uint64_t)P::NB * n_blocks, scan_tmp, st);
+    if (e != hipSuccess) return e;
+    if (p + 1 == passes)
+      hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_WORDS_TO_PERM>), g, b, 0, st, (const uint64_t*)in, out, perm, n,
+                         shift, idx_bits, (const uint32_t*)hist, n_blocks);
+    else
+      hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_WORDS_TO_WORDS>), g, b, 0, st, (const uint64_t*)in, out, perm, n,
+                         shift, idx_bits, (const uint32_t*)hist, n_blocks);
+    uint64_t* t = in; in = out; out = t;
+  }
+  return KTJ_LAUNCH_CHECK();
+}
+#define SORTP_BITS 8
+#define SORTP_THREADS 256
+bool sort_packed_fits(uint64_t n, uint32_t key_bits) {
+  const uint32_t total_bits = key_bits + 1u;
+  const uint32_t idx_bits = (uint32_t)(64 - __builtin_clzll(n > 1 ? n - 1 : 1));
+  return (total_bits > SORTP_BITS ? total_bits - SORTP_BITS : 0u) + idx_bits <= 64u;
+}
+hipError_t sort_packed(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits,
+                       uint32_t key_bits, uint64_t* buf_a, uint64_t* buf_b, uint32_t* perm, uint32_t* hist, uint64_t* scan_tmp,
+                       hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  const uint32_t idx_bits = (uint32_t)(64 - __builtin_clzll(n > 1 ? n - 1 : 1));
+  return sort_packed_t<SORTP_BITS, SORTP_THREADS>(c, n, s, sc, ts_bits, res_bits, key_bits, idx_bits, buf_a, buf_b, perm, hist,
+                                                  scan_tmp, st);
+}
+
 /* ------------------------------------------------------------------------------------------ */
 /* stage 4a: joined rows and exact byte lengths, arrival order                                  */
 /* ------------------------------------------------------------------------------------------ */
@@ -1339,6 +1704,35 @@ __device__ __forceinline__ void store_row(MatRow* dst, const MatRow& m) {
   const uint4* s = reinterpret_cast<const uint4*>(&m);
   uint4* d = reinterpret_cast<uint4*>(dst);
   for (int k = 0; k < (int)(sizeof(MatRow) / 16); ++k) d[k] = s[k];
+}
+/* Packed rows between global memory and LDS: a lane that loads or stores its own 64- or 96-byte
+ * row touches a cache line (or two) of its own with every 16-byte access, 64 lines per
+ * instruction; moved by the workgroup with lane-consecutive 16-byte accesses the same bytes are
+ * whole lines.  `rows` is the workgroup's first row, `cnt` its number of rows; the callers put
+ * the barriers. */
+template <typename T>
+__device__ __forceinline__ void rows_global_to_lds(const T* rows, uint32_t cnt, uint4* lds) {
+  const uint4* g = reinterpret_cast<const uint4*>(rows);
+  for (uint32_t k = threadIdx.x; k < cnt * (uint32_t)(sizeof(T) / 16); k += blockDim.x) lds[k] = g[k];
+}
+template <typename T>
+__device__ __forceinline__ void rows_lds_to_global(T* rows, uint32_t cnt, const uint4* lds) {
+  uint4* g = reinterpret_cast<uint4*>(rows);
+  for (uint32_t k = threadIdx.x; k < cnt * (uint32_t)(sizeof(T) / 16); k += blockDim.x) g[k] = lds[k];
+}
+template <typename T>
+__device__ __forceinline__ T row_from_lds(const uint4* lds) {
+  T r;
+  uint4* d = reinterpret_cast<uint4*>(&r);
+#pragma unroll
+  for (int k = 0; k < (int)(sizeof(T) / 16); ++k) d[k] = lds[threadIdx.x * (sizeof(T) / 16) + k];
+  return r;
+}
+template <typename T>
+__device__ __forceinline__ void row_to_lds(const T& r, uint4* lds) {
+  const uint4* s = reinterpret_cast<const uint4*>(&r);
+#pragma unroll
+  for (int k = 0; k < (int)(sizeof(T) / 16); ++k) lds[threadIdx.x * (sizeof(T) / 16) + k] = s[k];
 }
 /* exact byte length in the low 30 bits, tail kind (see tail_kind) in the top two */
 __device__ __forceinline__ uint32_t row_length(const MatRow& m, const EmitCtx& ctx, Scalars* sc) {
@@ -1374,7 +1768,7 @@ __global__ void k_sync_first_a(const uint32_t* perm, uint64_t n_sorted, const kt
   const uint64_t a = perm[p];
   if (a >= n_generic || !is_stream_sync(g[a], d)) return;
   const uint32_t slot = table_insert(keys, KTJ_SYNC_CAP - 1u, stream_sync_key(g[a].device, g[a].resource));
-  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TOO_MANY_DISTINCT); return; }
+  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_SYNC_ROWS); return; }
   atomicMin(&first_pos[slot], (uint32_t)p);
 }
 __global__ void k_sync_first_b(const uint32_t* perm, uint64_t n_sorted, const ktj_generic_rec* g, uint64_t n_generic,
@@ -1442,111 +1836,131 @@ __device__ __forceinline__ bool runtime_rows_share_slots(const Scalars* sc) {
 }
 /* Sets the slot's bit in a bitmap and tells whether it was set before.  All lanes of the wavefront
  * call it (active = the lane has a slot).  Rows that arrive in id order put up to 32 neighbouring
- * lanes on one word: where the wave's slots fall into at most two words, one lane per word sets
- * all their bits at once; otherwise every lane sets its own.  Two lanes of the wave with the same
- * slot are reported as "set before" for every lane of their word (callers only ask whether any
- * slot is shared). */
+ * lanes on one word, so the lanes are grouped by word (up to BITMAP_GROUPS groups, found with
+ * ballots; 64 consecutive slots lie in two or three words) and the lowest lane of each group sets
+ * all of its group's bits in one atomic; the groups' atomics leave in a single instruction.  Lanes
+ * beyond the last group set their own bit.  Two lanes of the wavefront with the same slot are
+ * reported as "set before" for every lane of their group (callers only ask whether any slot is
+ * shared). */
+#define BITMAP_GROUPS 4
 __device__ __forceinline__ uint32_t wave_or_u32(uint32_t v) {
   for (int o = 32; o > 0; o >>= 1) v |= (uint32_t)__shfl_xor((int)v, o);
   return v;
 }
 __device__ __forceinline__ bool bitmap_test_and_set(uint32_t* bitmap, uint32_t slot, bool active) {
   const uint32_t word = slot >> 5, bit = active ? 1u << (slot & 31u) : 0u;
-  const uint64_t todo = __ballot(active);
+  uint64_t todo = __ballot(active);
   if (!todo) return false;
-  const int l1 = __ffsll((unsigned long long)todo) - 1;
-  const uint32_t w1 = (uint32_t)__shfl((int)word, l1);
-  const bool in1 = active && word == w1;
-  const uint64_t m1 = __ballot(in1);
-  const uint64_t rest = todo & ~m1;
-  int l2 = 0;
-  uint32_t w2 = 0;
-  uint64_t m2 = 0;
-  if (rest) {
-    l2 = __ffsll((unsigned long long)rest) - 1;
-    w2 = (uint32_t)__shfl((int)word, l2);
-    m2 = __ballot(active && word == w2);
+  int leader = (int)lane_id();   /* lanes outside every group lead themselves */
+  uint32_t bits = bit;
+  bool twice = false;
+  for (int g = 0; g < BITMAP_GROUPS && todo; ++g) {
+    const int l = __ffsll((unsigned long long)todo) - 1;
+    const uint32_t w = (uint32_t)__shfl((int)word, l);
+    const bool in = ((todo >> lane_id()) & 1ull) != 0 && word == w;
+    const uint64_t m = __ballot(in);
+    const uint32_t all = wave_or_u32(in ? bit : 0u);
+    if (in) { leader = l; bits = all; twice = (uint32_t)__popc(all) != (uint32_t)__popcll(m); }
+    todo &= ~m;
   }
-  if ((m1 | m2) != todo) return active ? (atomicOr(&bitmap[word], bit) & bit) != 0 : false;
-  const bool in2 = active && !in1;
-  const uint32_t b1 = wave_or_u32(in1 ? bit : 0u), b2 = wave_or_u32(in2 ? bit : 0u);
-  uint32_t old1 = 0, old2 = 0;
-  if ((int)lane_id() == l1) old1 = atomicOr(&bitmap[w1], b1);
-  old1 = (uint32_t)__shfl((int)old1, l1);
-  if (m2) {
-    if ((int)lane_id() == l2) old2 = atomicOr(&bitmap[w2], b2);
-    old2 = (uint32_t)__shfl((int)old2, l2);
-  }
-  const bool twice1 = (uint32_t)__popc(b1) != (uint32_t)__popcll(m1), twice2 = (uint32_t)__popc(b2) != (uint32_t)__popcll(m2);
-  if (in1) return twice1 || (old1 & bit) != 0;
-  if (in2) return twice2 || (old2 & bit) != 0;
-  return false;
+  uint32_t old = 0;
+  if (active && leader == (int)lane_id()) old = atomicOr(&bitmap[word], bits);
+  old = (uint32_t)__shfl((int)old, leader);
+  return active && (twice || (old & bit) != 0);
 }
-__global__ void k_join_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, ApiTable api, Table tf,
+#define JOIN_ROWS 4
+#ifndef KX_JOIN_ATTR
+#define KX_JOIN_ATTR
+#endif
+__global__ void KX_JOIN_ATTR k_join_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, ApiTable api, Table tf,
                                FullCols fc, Table tn, NarrowCols nc, uint32_t* slot_f, uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
                                uint32_t* len, Scalars* sc) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   RowStats rs;
   uint32_t n_linked = 0;
-  bool carries_stream = false;
-  uint32_t sf = KTJ_NOSLOT;
-  if (i < n) sf = slot_insert(tf, c.corr[first_runtime + i]);
-  const bool repeats = bitmap_test_and_set(fc.has_runtime, sf, sf != KTJ_NOSLOT);
-  if (i < n) {
-    const uint64_t a = first_runtime + i;
-    const ktj_runtime_rec rec = r[i];
-    const uint64_t id = c.corr[a];
-    const uint32_t meta = c.meta[a];
-    const int64_t ts = c.ts[a];
+  bool any_carries_stream = false, any_repeats = false;
+  /* a workgroup takes JOIN_ROWS consecutive groups of blockDim.x rows: the per-workgroup counters
+   * at the end (one atomic each on a hot address) are paid once for all of them */
+  static_assert(sizeof(MatRow) == sizeof(ktj_runtime_rec), "the staging area holds the records, then the joined rows");
+  __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_runtime_rec) / 16];
+  for (int round = 0; round < JOIN_ROWS; ++round) {
+    const uint64_t base = ((uint64_t)blockIdx.x * JOIN_ROWS + round) * blockDim.x;
+    if (base >= n) break;
+    const uint32_t cnt = (uint32_t)(n - base < blockDim.x ? n - base : blockDim.x);
+    __syncthreads(); /* the previous round's rows have left the staging area */
+    rows_global_to_lds(r + base, cnt, stage);
+    __syncthreads();
+    const uint64_t i = base + threadIdx.x;
+    bool carries_stream = false;
+    uint32_t sf = KTJ_NOSLOT;
+    /* everything the row reads from its own record and columns is requested up front, so that the
+     * table accesses below (each a round trip of its own) overlap with it */
+    const uint64_t a = first_runtime + (i < n ? i : 0);
+    /* the lane's record stays in LDS and is read field by field; the joined row takes its place */
+    uint4* my_slot = &stage[threadIdx.x * (sizeof(ktj_runtime_rec) / 16)];
+    const ktj_runtime_rec& rec = *reinterpret_cast<const ktj_runtime_rec*>(my_slot);
+    uint64_t id = 0;
+    uint32_t meta = 0;
+    int64_t ts = 0, dur = 0;
+    if (i < n) {
+      id = c.corr[a];
+      meta = c.meta[a];
+      ts = c.ts[a];
+      dur = c.dur[a];
+      sf = slot_insert(tf, id);
+    }
     const uint32_t kind = (meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT;
     const bool valid = (meta & KTJ_M_VALID) != 0;
-    carries_stream = (meta & KTJ_M_HAS_STREAM) != 0;
-    slot_f[i] = sf;
-    if (sf == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
-    else {
-      FullPay fp;
-      fp.first_ts = ts;
-      fp.stream = 0;
-      if (carries_stream) fp.stream = rec.kind == KTJ_RT_KERNEL ? rec.u.kernel.stream : rec.u.copy.stream;
-      fc.pay[sf] = fp;
-    }
     const bool publishes = valid && kind != KTJ_RT_DEFAULT;
-    uint32_t sn;
+    /* every slot that carries an external id exists already (k_build_extcorr ran before) */
+    uint32_t sn = KTJ_NOSLOT;
+    if (i < n) sn = publishes ? slot_insert(tn, narrow_corr_key(id)) : slot_find(tn, narrow_corr_key(id));
     int32_t ext = 0;
-    if (publishes) {
-      sn = slot_insert(tn, narrow_corr_key(id));
-      if (sn == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+    uint32_t np_info = 0;
+    if (sn != KTJ_NOSLOT) { ext = nc.pay[sn].ext_val; np_info = nc.pay[sn].info; }
+    const bool repeats = bitmap_test_and_set(fc.has_runtime, sf, sf != KTJ_NOSLOT);
+    if (i < n) {
+      carries_stream = (meta & KTJ_M_HAS_STREAM) != 0;
+      slot_f[i] = sf;
+      if (sf == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
       else {
-        NarrowPay* np = &nc.pay[sn];
-        if (kind == KTJ_RT_KERNEL) {
-          pack_grid(rec, np->pay);
-          np->info = (np->info & ~KTJ_NP_KIND_MASK) | KTJ_DL_HAS_GRID;
-        } else {
-          np->pay[0] = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
-          np->info = (np->info & ~KTJ_NP_KIND_MASK) | KTJ_DL_HAS_SIZE;
+        FullPay fp;
+        fp.first_ts = ts;
+        fp.stream = 0;
+        if (carries_stream) fp.stream = rec.kind == KTJ_RT_KERNEL ? rec.u.kernel.stream : rec.u.copy.stream;
+        fc.pay[sf] = fp;
+      }
+      if (publishes) {
+        if (sn == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+        else {
+          NarrowPay* np = &nc.pay[sn];
+          if (kind == KTJ_RT_KERNEL) {
+            pack_grid(rec, np->pay);
+            np->info = (np_info & ~KTJ_NP_KIND_MASK) | KTJ_DL_HAS_GRID;
+          } else {
+            np->pay[0] = rec.kind == KTJ_RT_COPY ? rec.u.copy.size : rec.u.malloc_.size;
+            np->info = (np_info & ~KTJ_NP_KIND_MASK) | KTJ_DL_HAS_SIZE;
+          }
         }
       }
-    } else {
-      /* every slot that carries an external id exists already (k_build_extcorr ran before) */
-      sn = slot_find(tn, narrow_corr_key(id));
+      slot_n[i] = sn;
+      if ((np_info & KTJ_NP_LINKED) && valid) ++n_linked;
+      c.ext[a] = ext;
+      const bool known = rec.cid < api.n_cids;
+      const uint32_t name = known ? api.cid_name_ids[rec.cid] : KTJ_NONE;
+      const bool fstart = known && ((api.flow_start_bits[rec.cid >> 5] >> (rec.cid & 31u)) & 1u);
+      MatRow* m = reinterpret_cast<MatRow*>(my_slot);
+      *m = mat_runtime(rec, ts, dur, valid, ext, name, fstart, rec.cid == api.malloc_cid);
+      len[a] = row_length(*m, ctx, sc);
+      count_row_stats(*m, ctx, &rs);
     }
-    slot_n[i] = sn;
-    if (sn != KTJ_NOSLOT) {
-      ext = nc.pay[sn].ext_val;
-      if ((nc.pay[sn].info & KTJ_NP_LINKED) && valid) ++n_linked;
-    }
-    c.ext[a] = ext;
-    const bool known = rec.cid < api.n_cids;
-    const uint32_t name = known ? api.cid_name_ids[rec.cid] : KTJ_NONE;
-    const bool fstart = known && ((api.flow_start_bits[rec.cid >> 5] >> (rec.cid & 31u)) & 1u);
-    const MatRow m = mat_runtime(rec, ts, c.dur[a], valid, ext, name, fstart, rec.cid == api.malloc_cid);
-    store_row(&mat[a], m);
-    len[a] = row_length(m, ctx, sc);
-    count_row_stats(m, ctx, &rs);
+    __syncthreads(); /* the joined rows go out the way the records came in */
+    rows_lds_to_global(mat + first_runtime + base, cnt, stage);
+    any_carries_stream |= carries_stream;
+    any_repeats |= repeats;
   }
   /* one store per workgroup at most: every lane storing the same flag would queue up in L2 */
-  const int any_stream = __syncthreads_or(carries_stream ? 1 : 0);
-  const int any_repeat = __syncthreads_or(repeats ? 1 : 0);
+  const int any_stream = __syncthreads_or(any_carries_stream ? 1 : 0);
+  const int any_repeat = __syncthreads_or(any_repeats ? 1 : 0);
   if (threadIdx.x == 0) {
     if (any_stream) sc->have_stream_src = 1;
     if (any_repeat) sc->runtime_ids_repeat = 1;
@@ -1613,16 +2027,28 @@ __global__ void k_republish_runtime(const ktj_runtime_rec* r, uint64_t n, Column
 }
 __global__ void k_mat_device(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const DevLink* link,
                              EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc) {
+  __shared__ uint4 stage[KTJ_BLOCK * sizeof(MatRow) / 16]; /* the records, then the joined rows */
   RowStats rs;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    const uint64_t a = first + i;
-    const ktj_device_rec rec = d[i];
-    const DevLink l = link[i];
-    const MatRow m = mat_device(rec, c.ts[a], c.dur[a], c.res[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a],
-                                (l.flags & KTJ_DL_HAS_GRID) ? l.p : nullptr, (l.flags & KTJ_DL_HAS_SIZE) != 0, l.p[0], l.coll);
-    store_row(&mat[a], m);
-    len[a] = row_length(m, ctx, sc);
-    count_row_stats(m, ctx, &rs);
+  for (uint64_t base = (uint64_t)blockIdx.x * blockDim.x; base < n; base += (uint64_t)gridDim.x * blockDim.x) {
+    const uint32_t cnt = (uint32_t)(n - base < blockDim.x ? n - base : blockDim.x);
+    __syncthreads(); /* the previous round's rows have left the staging area */
+    rows_global_to_lds(d + base, cnt, stage);
+    __syncthreads();
+    const uint64_t i = base + threadIdx.x, a = first + i;
+    const bool active = threadIdx.x < cnt;
+    MatRow m;
+    if (active) {
+      const ktj_device_rec rec = row_from_lds<ktj_device_rec>(stage);
+      const DevLink l = link[i];
+      m = mat_device_v(rec, c.ts[a], c.dur[a], c.res[a], (c.meta[a] & KTJ_M_VALID) != 0, c.ext[a],
+                       (l.flags & KTJ_DL_HAS_GRID) != 0, l.p[0], l.p[1], l.p[2], (l.flags & KTJ_DL_HAS_SIZE) != 0, l.p[0], l.coll);
+      len[a] = row_length(m, ctx, sc);
+      count_row_stats(m, ctx, &rs);
+    }
+    __syncthreads(); /* every lane has taken its record */
+    if (active) row_to_lds(m, stage);
+    __syncthreads();
+    rows_lds_to_global(mat + first + base, cnt, stage);
   }
   flush_row_stats(rs, sc);
 }
@@ -1670,7 +2096,7 @@ hipError_t join_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, ui
                              Table tn, NarrowCols nc, uint32_t* slot_f, uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
                              uint32_t* len, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_join_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, tf, fc, tn, nc,
+  hipLaunchKernelGGL(k_join_runtime, dim3(grid_for(n, KTJ_BLOCK * JOIN_ROWS)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, tf, fc, tn, nc,
                      slot_f, slot_n, ctx, mat, len, sc);
   return KTJ_LAUNCH_CHECK();
 }

@@ -132,8 +132,9 @@ KTJ_HD inline MatRow mat_runtime(const ktj_runtime_rec& r, int64_t ts, int64_t d
 /* res: resourceId() after stream back-fill.  grid: packed grid and block of the launching kernel
  * row that the reference hands over (null = none); size: bytes handed over by a copy/malloc row. */
 /* coll: 1 + index of the collective metadata of the linked CPU op, 0 = none (kernels only) */
-KTJ_HD inline MatRow mat_device(const ktj_device_rec& d, int64_t ts, int64_t dur, int64_t res, bool valid,
-                                int32_t ext, const uint64_t* grid, bool has_size, uint64_t size, uint32_t coll = 0) {
+KTJ_HD inline MatRow mat_device_v(const ktj_device_rec& d, int64_t ts, int64_t dur, int64_t res, bool valid, int32_t ext,
+                                  bool has_grid, uint64_t g0, uint64_t g1, uint64_t g2, bool has_size, uint64_t size,
+                                  uint32_t coll) {
   MatRow m;
   m.ts = ts; m.dur = dur; m.dev = (int64_t)d.device; m.res = res;
   m.flow_id = (int64_t)d.id;
@@ -157,14 +158,19 @@ KTJ_HD inline MatRow mat_device(const ktj_device_rec& d, int64_t ts, int64_t dur
     } else if (d.name_id == KTJ_NONE) { meta |= KTJ_M_NAME_BUILTIN; m.name_id = KTJ_NAME_UNKNOWN_OP; }
     else m.name_id = d.name_id;
     if (has_size) { meta |= KTJ_M_HAS_SIZE; m.p[0] = size; }
-    else if (grid) {
+    else if (has_grid) {
       meta |= KTJ_M_HAS_GRID;
-      m.p[0] = grid[0]; m.p[1] = grid[1]; m.p[2] = grid[2];
+      m.p[0] = g0; m.p[1] = g1; m.p[2] = g2;
     }
     if (dom == KTJ_DOM_KERNEL_DISPATCH) m.p[4] = coll;
   }
   m.meta = meta;
   return m;
+}
+KTJ_HD inline MatRow mat_device(const ktj_device_rec& d, int64_t ts, int64_t dur, int64_t res, bool valid,
+                                int32_t ext, const uint64_t* grid, bool has_size, uint64_t size, uint32_t coll = 0) {
+  return mat_device_v(d, ts, dur, res, valid, ext, grid != nullptr, grid ? grid[0] : 0, grid ? grid[1] : 0, grid ? grid[2] : 0,
+                      has_size, size, coll);
 }
 
 }  // namespace ktj

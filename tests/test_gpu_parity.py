@@ -55,11 +55,13 @@ def run_case(cfg, n, check_stages=True):
             assert st.n_linked == cnt["n_linked"]
         got = eng.output()
     # the output-partitioned emit kernel and hash-mode join tables must produce the same document
-    with TraceEngine(sp.contents.trace_name.decode(), device=0, tile_emit=True, hash_join=True) as eng:
+    with TraceEngine(sp.contents.trace_name.decode(), device=0, tile_emit=True, hash_join=True, pair_sort=True) as eng:
         eng.submit_stream(sp)
         eng.process()
         st_hash = eng.stats()
         got_tile = eng.output()
+        if check_stages:
+            assert np.array_equal(eng.debug("perm")[:n_acts].astype(np.int64), perm), "pair sort and word sort disagree"
     if check_stages:  # hash-mode join tables: same counters as the direct-addressed ones
         assert st_hash.gpu_and_cpu_op_out_of_order == st.gpu_and_cpu_op_out_of_order and st_hash.n_linked == st.n_linked
     ora.close()
@@ -122,7 +124,7 @@ def test_random_streams_on_gpu(seed):
     print(f"random stream seed={seed}", flush=True)
     sp = random_streams.random_stream(seed, wide_ids=seed % 2 == 1, unique_runtime_ids=seed % 3 == 2).build()
     _engine_vs_oracle(sp)
-    _engine_vs_oracle(sp, hash_join=True, tile_emit=True)
+    _engine_vs_oracle(sp, hash_join=True, tile_emit=True, pair_sort=True)
 
 
 @pytest.mark.parametrize("cfg,n", [(3, 20000), (4, 6000), (2, 9000)])
@@ -146,6 +148,56 @@ def test_join_edge_cases_on_gpu():
     assert got.count(b'"ph": "X"') == 20   # every in-window row of the hand-made stream printed
 
 
+KTJ_MAX_STREAM_PAIRS = 4096   # include/ktj.h
+
+
+def _many_ids_builder(n_resources, n_devices, n_streams=0, n_queues=0, n_sync_rows=0):
+    """CPU ops on n_resources distinct threads of n_devices distinct processes (ids spread over the
+    whole signed 64-bit / 32-bit range, arrival order scrambled), plus optional device rows on
+    n_streams distinct streams or n_queues distinct queues, plus n_sync_rows Stream Sync events on
+    distinct rows."""
+    from stream_builder import StreamBuilder, B
+    b = StreamBuilder(host_name="many")
+    b.api(["hipLaunchKernel"], flow_start=[0])
+    n = max(n_resources, n_devices)
+    for i in range(n):
+        j = (i * 7919) % n
+        res = ((j % n_resources) * 0x9E3779B97F4A7C15 + 12345) % (1 << 64) - (1 << 63)
+        dev = (((j % n_devices) * 0x45D9F3B + 77) % (1 << 32)) - (1 << 31)
+        b.add_generic("op%d" % (i % 5), 0, B + 1000 + 13 * ((i * 31) % n), B + 1500 + 13 * ((i * 31) % n), dev, res, id=i + 1)
+    for i in range(max(n_streams, n_queues)):
+        b.add_runtime(10**6 + i, B + 5000 + i, B + 5400 + i, 0, 1, 1, kind=1, stream=(0x7000 + 8 * i) if n_streams else 0)
+        b.add_device(10**6 + i, B + 6000 + i, B + 6300 + i, domain=0,
+                     device=i % 3, name="k%d" % (i % 4), queue=0x100 + i)
+    for i in range(n_sync_rows):
+        b.add_generic("Stream Sync", 15, B + 9000 + i, B + 9100 + i, 0, 1000 + i, id=2 * 10**6 + i)
+    return b
+
+
+def test_more_distinct_ids_than_the_rank_sets_hold():
+    """Above 4096 distinct resourceId or deviceId values the sort works on the raw values: same bytes
+    as the checker, no error."""
+    for n_res, n_dev in ((5000, 3), (300, 4200), (20000, 4500)):
+        print(f"distinct ids: {n_res} resources, {n_dev} devices", flush=True)
+        _engine_vs_oracle(_many_ids_builder(n_res, n_dev).build())
+
+
+def test_limits_end_in_a_named_error():
+    """A trace beyond one of the engine's documented limits is refused with KTJ_ERR_LIMIT and a text
+    that names the limit (include/ktj.h: KTJ_MAX_*)."""
+    from kineto_amd.engine import TraceEngine, EngineError
+    for kw, name in ((dict(n_streams=KTJ_MAX_STREAM_PAIRS + 200), "KTJ_MAX_STREAM_PAIRS"),):
+        print("limit", name, flush=True)
+        sp = _many_ids_builder(10, 1, **kw).build()
+        with TraceEngine("t.json", device=0) as eng:
+            eng.submit_stream(sp)
+            with pytest.raises(EngineError) as ei:
+                eng.process()
+            assert "rc=%d" % abi.KTJ_ERR_LIMIT in str(ei.value) and name in str(ei.value)
+    # just inside the limit: accepted and identical to the checker
+    _engine_vs_oracle(_many_ids_builder(10, 1, n_streams=KTJ_MAX_STREAM_PAIRS - 96).build())
+
+
 def test_golden_digests_on_gpu():
     """The engine's document against the committed digests (tests/golden/digests.json, written where
     the checker's output had just been compared byte for byte with the reference logger's): no
@@ -161,7 +213,7 @@ def test_golden_digests_on_gpu():
         cfg, n = (int(x) for x in key.split(":"))
         print("golden", key, flush=True)
         sp, release = abi.synth_stream(cfg, n, host_name="golden", trace_name="golden.json")
-        for opts in ({}, {"tile_emit": True, "hash_join": True}):
+        for opts in ({}, {"tile_emit": True, "hash_join": True, "pair_sort": True}):
             with TraceEngine(sp.contents.trace_name.decode(), device=0, **opts) as eng:
                 eng.submit_stream(sp)
                 eng.process()
