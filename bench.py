@@ -8,6 +8,9 @@ device buffer.  Prints one JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--n-device N] [--config C]
   python bench.py --logger-benchmark small|medium|large   (the reference's logger benchmark, both loggers)
+  python bench.py --summarize-kernel-trace STATS.csv      (table of a `rocprofv3 --kernel-trace --stats` run)
+  python bench.py --summarize-hbm FETCH_DIR WRITE_DIR STATS.csv --config C
+                                                          (table of two `rocprofv3 --pmc` runs, see profiles/)
 """
 import argparse
 import ctypes as C
@@ -21,11 +24,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per k_emit_direct launch, from two separate `rocprofv3 --pmc` runs of this script
-# (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter reads for the 1 GiB
-# k_copy_reference launch at the end of the run (2048 and 1024 bytes per unit).  Keyed by
-# (configuration, device rows); a counter run cannot share a process with the timed run.
-MEASURED_EMIT_TRAFFIC = {(3, 10000000): 3.64e9 + 13.32e9}
+DOMINANT_KERNEL = "k_emit_direct"
 FULL_SIZE = {1: 10000, 2: 1000000, 3: 10000000, 4: 11000000, 5: 5000000}
 WORKLOAD = {
     1: "config1: 10k CPU ops + 10k launches + 10k kernels, 4 streams",
@@ -34,6 +33,140 @@ WORKLOAD = {
     4: "config4: graph launches with 100-1000 kernel fan-out (~11M kernels), 5% orphans each way",
     5: "config5: 5M string-heavy generic kernel records with typed args",
 }
+
+
+def short_kernel_name(name):
+    """ktj::gpu::k_x<...>(args) -> k_x<...>"""
+    name = name.strip().strip('"')
+    if name.startswith("void "):
+        name = name[5:]
+    depth = 0
+    for i, ch in enumerate(name):
+        if ch == "<":
+            depth += 1
+        elif ch == ">":
+            depth -= 1
+        elif ch == "(" and depth == 0:
+            name = name[:i]
+            break
+    return name.replace("ktj::gpu::", "")
+
+
+def read_kernel_stats(path):
+    import csv
+    rows = []
+    for r in csv.DictReader(open(path)):
+        rows.append((short_kernel_name(r["Name"]), int(r["Calls"]), float(r["AverageNs"]) / 1e3, float(r["MinNs"]) / 1e3,
+                     float(r["MaxNs"]) / 1e3, float(r["Percentage"])))
+    return rows
+
+
+def summarize_kernel_trace(stats_csv):
+    """Prints the per-kernel table of a `rocprofv3 --kernel-trace --stats --output-format csv` run."""
+    print("%-44s %6s %10s %10s %10s %6s" % ("kernel", "calls", "avg_us", "min_us", "max_us", "pct"))
+    for name, calls, avg, mn, mx, pct in read_kernel_stats(stats_csv):
+        print("%-44s %6d %10.1f %10.1f %10.1f %6.2f" % (name[:44], calls, avg, mn, mx, pct))
+
+
+def read_counter(directory, counter):
+    """Sum and launch count per kernel of one counter in a `rocprofv3 --pmc` output directory."""
+    import collections
+    import csv
+    import glob
+    files = glob.glob(os.path.join(directory, "**", "*counter_collection.csv"), recursive=True)
+    if not files:
+        raise SystemExit("bench.py: no *counter_collection.csv under " + directory)
+    total = collections.defaultdict(float)
+    launches = collections.defaultdict(set)
+    for r in csv.DictReader(open(files[0])):
+        if r["Counter_Name"] != counter:
+            continue
+        k = short_kernel_name(r["Kernel_Name"])
+        total[k] += float(r["Counter_Value"])
+        launches[k].add(r["Dispatch_Id"])
+    return {k: (total[k], len(launches[k])) for k in total}
+
+
+def summarize_hbm(fetch_dir, write_dir, stats_csv, config, copy_bytes=1 << 30):
+    """Prints HBM bytes per launch and kernel from a FETCH_SIZE run and a WRITE_SIZE run of this script
+    (one pass each, both ending with the k_copy_reference launch of copy_bytes that scales the
+    counters), with the kernels' average durations from a separate kernel-trace run."""
+    fetch, write = read_counter(fetch_dir, "FETCH_SIZE"), read_counter(write_dir, "WRITE_SIZE")
+    ref = "k_copy_reference"
+    if ref not in fetch or ref not in write:
+        raise SystemExit("bench.py: the counter runs hold no k_copy_reference launch to scale by")
+    f_unit = copy_bytes / (fetch[ref][0] / fetch[ref][1])
+    w_unit = copy_bytes / (write[ref][0] / write[ref][1])
+    avg = {name: a for name, _, a, _, _, _ in read_kernel_stats(stats_csv)}
+    print("scale: k_copy_reference copies %d bytes per launch: FETCH_SIZE %.1f bytes per unit, WRITE_SIZE %.1f bytes per unit"
+          % (copy_bytes, f_unit, w_unit))
+    print("%-36s %8s %10s %10s %9s %7s %7s" % ("kernel", "launches", "fetch_MB", "write_MB", "avg_us", "GB/s", "of_peak"))
+    rows = []
+    for k in set(fetch) | set(write):
+        n = max(fetch.get(k, (0, 0))[1], write.get(k, (0, 0))[1]) or 1
+        fb = fetch.get(k, (0, 0))[0] * f_unit / n
+        wb = write.get(k, (0, 0))[0] * w_unit / n
+        rows.append((k, n, fb, wb, avg.get(k)))
+    rows.sort(key=lambda r: -(r[2] + r[3]) * r[1])
+    for k, n, fb, wb, a in rows:
+        gbs = (fb + wb) / (a * 1e-6) / 1e9 if a else 0.0
+        print("%-36s %8d %10.1f %10.1f %9s %7.0f %7.3f" % (k[:36], n, fb / 1e6, wb / 1e6, "%.1f" % a if a else "-", gbs,
+                                                          gbs / HBM_PEAK_GBS))
+    for k, n, fb, wb, a in rows:
+        if k == DOMINANT_KERNEL:
+            print("traffic_json: " + json.dumps({"kernel": k, "config": config, "fetch_bytes_per_launch": round(fb),
+                                                 "write_bytes_per_launch": round(wb), "hbm_bytes_per_launch": round(fb + wb)}))
+
+
+def measured_traffic(config, device_rows):
+    """HBM bytes per launch of the dominant kernel, from the committed summary of the counter runs
+    (profiles/hbm_counters_config<C>_full.txt, written by --summarize-hbm); None when there is none
+    for this workload."""
+    if device_rows != FULL_SIZE[config]:
+        return None
+    path = os.path.join(ROOT, "profiles", "hbm_counters_config%d_full.txt" % config)
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("traffic_json:"):
+            t = json.loads(line[len("traffic_json:"):])
+            if t.get("kernel") == DOMINANT_KERNEL and t.get("config") == config:
+                return t["hbm_bytes_per_launch"]
+    return None
+
+
+def host_cpu():
+    model = None
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count()
+    return {"model": model, "logical_cpus": os.cpu_count(), "usable_cpus": usable}
+
+
+def reference_logger_leg(sp, ora, engine_bytes):
+    """The reference's own ChromeTraceLogger (oracle/_ref/libktj_ref.so, built from the reference's
+    sources) fed the sample's joined activities, timed from logger construction to the end of
+    finalizeTrace, file included; None where that library is not built."""
+    import oracle_glue as og
+    if not og.have_ref():
+        return None
+    t0 = time.perf_counter()
+    data = og.ref_render(sp, ora, call_order=0)
+    dt = time.perf_counter() - t0
+    _, n_acts = ora.activities()
+    return {"value": n_acts / dt, "unit": "activities/s", "cores": 1, "kind": "reference",
+            "seconds": dt, "activities": int(n_acts), "output_bytes": len(data),
+            "note": "logger only: the reference's join stages need a profiling session and are not part of this leg; "
+                    "includes building the activity objects and writing the file to a temporary directory",
+            "identical_to_engine_output_on_sample": bool(data == engine_bytes)}
 
 
 def cpu_baseline(config, sample_device_rows):
@@ -55,11 +188,14 @@ def cpu_baseline(config, sample_device_rows):
         eng.process()
         got = eng.output_view()
         same = got.shape == want.shape and bool(np.array_equal(got, want))
+        engine_bytes = bytes(got) if same else eng.output()
     stages = ora.timings()
+    ref_leg = reference_logger_leg(sp, ora, engine_bytes)
+    del engine_bytes
     ora.close()
     release()
-    return {
-        "value": n_records / dt, "unit": "records/s", "cores": 1, "kind": "port",
+    return ref_leg, {
+        "value": n_records / dt, "unit": "records/s", "cores": 1, "kind": "port", "host_cpu": host_cpu(),
         "sample": f"same workload scaled to {sample_device_rows} device rows ({n_records} records, "
                   f"{len(want)} output bytes) in {dt:.2f} s on one host core "
                   f"(join {stages[0]:.2f} s, sort {stages[1]:.2f} s, emit {stages[2]:.2f} s)",
@@ -137,7 +273,8 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=0, help="device rows of the CPU-baseline sample (0 = auto)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-bytes", type=int, default=1 << 30, help="size of the reference copy kernel run (0 = skip)")
-    ap.add_argument("--traffic", type=str, default="", help="JSON file with measured HBM bytes per emit launch (from rocprofv3 --pmc)")
+    ap.add_argument("--summarize-kernel-trace", metavar="STATS_CSV", default=None)
+    ap.add_argument("--summarize-hbm", nargs=3, metavar=("FETCH_DIR", "WRITE_DIR", "STATS_CSV"), default=None)
     ap.add_argument("--logger-benchmark", choices=["small", "medium", "large"], default=None,
                     help="run the reference's logger benchmark on both loggers instead of the hot-path bench")
     ap.add_argument("--iterations", type=int, default=0, help="iterations of --logger-benchmark (0 = the reference's defaults)")
@@ -148,6 +285,12 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    if args.summarize_kernel_trace:
+        summarize_kernel_trace(args.summarize_kernel_trace)
+        return
+    if args.summarize_hbm:
+        summarize_hbm(*args.summarize_hbm, config=args.config, copy_bytes=args.copy_bytes)
+        return
     import torch
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -175,8 +318,13 @@ def main():
     h2d_s = time.perf_counter() - t0
     release()
 
-    for _ in range(args.warmup):
-        eng.process()
+    cold_first_step_ms = None
+    for w in range(args.warmup):
+        t0 = time.perf_counter()
+        eng.process()              # the first pass allocates every working buffer and the document
+        if w == 0:
+            torch.cuda.synchronize()
+            cold_first_step_ms = (time.perf_counter() - t0) * 1e3
     torch.cuda.synchronize()
     stage_sum = [0.0] * abi.N_STAGES
     t0 = time.perf_counter()
@@ -223,6 +371,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "cold_first_step_ms": cold_first_step_ms,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -235,7 +384,7 @@ def main():
         "output_frac_of_hbm_peak": out_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "stage_ms": stage_ms,
         "stage_algorithmic_gb_per_s": stage_gbs,
-        "roofline": {"bound": "hbm", "kernel": "k_emit_direct", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "roofline": {"bound": "hbm", "kernel": DOMINANT_KERNEL, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": emit_alg, "avg_launch_ms": emit_ms},
         "pcie": {"h2d_submit_s": h2d_s, "d2h_document_ms": d2h_ms, "d2h_wall_s": d2h_s,
@@ -245,12 +394,12 @@ def main():
     }
     if copy_gbs:
         result["roofline"]["frac_of_copy_kernel"] = achieved / copy_gbs
-    result["roofline"]["traffic"] = MEASURED_EMIT_TRAFFIC.get((cfg, n_dev))
-    if args.traffic and os.path.exists(args.traffic):
-        result["roofline"]["traffic"] = json.load(open(args.traffic)).get("emit_hbm_bytes_per_launch")
+    result["roofline"]["traffic"] = measured_traffic(cfg, n_dev)
     if not args.no_cpu_baseline:
         sample = args.cpu_sample or max(1000, min(n_dev, {1: 10000, 2: 1000000, 3: 2500000, 4: 4000000, 5: 1000000}[cfg]))
-        result["cpu_baseline"] = cpu_baseline(cfg, sample)
+        ref_leg, result["cpu_baseline"] = cpu_baseline(cfg, sample)
+        if ref_leg:
+            result["reference_logger"] = ref_leg
     print(json.dumps(result))
 
 

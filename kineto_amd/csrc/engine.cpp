@@ -852,10 +852,17 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   HIPCHK(clear_tables(tf, fc, tn, nc, t_cpu, st));
   StreamTables stt{e->q_keys.as<uint64_t>(), e->q_stream.as<uint64_t>(), e->q_amb.as<uint32_t>(), e->dn_hash.as<uint64_t>(),
                    e->dn_first.as<uint32_t>(), e->dn_dev.as<int32_t>(), e->dn_key.as<uint64_t>(), e->dn_rank.as<uint32_t>()};
-  HIPCHK(fill_u64(stt.q_keys, KTJ_EMPTY_KEY, KTJ_QUEUE_CAP + 1ull, st)); HIPCHK(fill_u64(stt.q_stream, 0, KTJ_QUEUE_CAP + 1ull, st));
-  HIPCHK(fill_u32(stt.q_amb, 0, KTJ_QUEUE_CAP + 1ull, st));
-  HIPCHK(fill_u64(stt.d_hash, KTJ_EMPTY_KEY, KTJ_DENSE_CAP + 1ull, st)); HIPCHK(fill_u32(stt.d_first, 0xFFFFFFFFu, KTJ_DENSE_CAP + 1ull, st));
-  HIPCHK(fill_u32(stt.d_rank, 0, KTJ_DENSE_CAP + 1ull, st));
+  SortSets sets{e->s_dev_k.as<uint64_t>(), e->s_dev_r.as<uint32_t>(), e->s_res_k.as<uint64_t>(), e->s_res_r.as<uint32_t>()};
+  {
+    FillJobs f;
+    f.count = 0;
+    f.add(stt.q_keys, KTJ_EMPTY_KEY, KTJ_QUEUE_CAP + 1ull, 8); f.add(stt.q_stream, 0, KTJ_QUEUE_CAP + 1ull, 8);
+    f.add(stt.q_amb, 0, KTJ_QUEUE_CAP + 1ull, 4);
+    f.add(stt.d_hash, KTJ_EMPTY_KEY, KTJ_DENSE_CAP + 1ull, 8); f.add(stt.d_first, 0xFFFFFFFFu, KTJ_DENSE_CAP + 1ull, 4);
+    f.add(stt.d_rank, 0, KTJ_DENSE_CAP + 1ull, 4);
+    f.add(sets.dev_keys, KTJ_EMPTY_KEY, KTJ_SET_CAP + 1ull, 8); f.add(sets.res_keys, KTJ_EMPTY_KEY, KTJ_SET_CAP + 1ull, 8);
+    HIPCHK(fill_many(f, st));
+  }
   ApiTable api{e->d_cid_names.as<uint32_t>(), (uint32_t)e->cid_names.size(), e->d_flow_bits.as<uint32_t>(), e->malloc_cid};
   MatRow* mat = e->mat.as<MatRow>();
   HIPCHK(build_extcorr(x_recs, nx, tn, nc, e->slot_ext.as<uint32_t>(), sc, st));
@@ -875,9 +882,6 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   HIPCHK(hipEventRecord(e->ev[EV_JOIN], st));
 
   /* ---- stage 3: canonical order ---- */
-  SortSets sets{e->s_dev_k.as<uint64_t>(), e->s_dev_r.as<uint32_t>(), e->s_res_k.as<uint64_t>(), e->s_res_r.as<uint32_t>()};
-  HIPCHK(fill_u64(sets.dev_keys, KTJ_EMPTY_KEY, KTJ_SET_CAP + 1ull, st));
-  HIPCHK(fill_u64(sets.res_keys, KTJ_EMPTY_KEY, KTJ_SET_CAP + 1ull, st));
   HIPCHK(collect_distinct(c, N, sets, sc, st));
   HIPCHK(rank_distinct(sets, sc, st));
   HIPCHK(hipEventRecord(e->ev[EV_SORT_A], st));

@@ -160,6 +160,15 @@ struct ApiTable {
 /* ---- utilities ---- */
 hipError_t fill_u64(uint64_t* p, uint64_t v, uint64_t n, hipStream_t st);
 hipError_t fill_u32(uint32_t* p, uint32_t v, uint64_t n, hipStream_t st);
+struct FillJobs {          /* up to 12 fills in one launch */
+  void* p[12];
+  uint64_t value[12];
+  uint64_t n[12];
+  uint32_t bytes_each[12]; /* 4 or 8 */
+  uint32_t count;
+  void add(void* ptr, uint64_t v, uint64_t elems, uint32_t width) { p[count] = ptr; value[count] = v; n[count] = elems; bytes_each[count] = width; ++count; }
+};
+hipError_t fill_many(const FillJobs& jobs, hipStream_t st);
 hipError_t init_scalars(Scalars* s, hipStream_t st);
 hipError_t copy_reference(const void* src, void* dst, uint64_t bytes, hipStream_t st);
 

@@ -188,6 +188,25 @@ hipError_t fill_u32(uint32_t* p, uint32_t v, uint64_t n, hipStream_t st) {
   hipLaunchKernelGGL(k_fill_u32, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, p, v, n);
   return KTJ_LAUNCH_CHECK();
 }
+/* several fills in one launch (blockIdx.y picks the job): a small trace pays per launch, not per byte */
+__global__ void k_fill_many(FillJobs jobs) {
+  const uint32_t j = blockIdx.y;
+  const uint64_t n = jobs.n[j], v = jobs.value[j];
+  if (jobs.bytes_each[j] == 8) {
+    uint64_t* p = static_cast<uint64_t*>(jobs.p[j]);
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) p[i] = v;
+  } else {
+    uint32_t* p = static_cast<uint32_t*>(jobs.p[j]);
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) p[i] = (uint32_t)v;
+  }
+}
+hipError_t fill_many(const FillJobs& jobs, hipStream_t st) {
+  if (jobs.count == 0) return hipSuccess;
+  uint64_t most = 1;
+  for (uint32_t j = 0; j < jobs.count; ++j) most = jobs.n[j] > most ? jobs.n[j] : most;
+  hipLaunchKernelGGL(k_fill_many, dim3(grid_stride_for(most, KTJ_BLOCK * 4), jobs.count), dim3(KTJ_BLOCK), 0, st, jobs);
+  return KTJ_LAUNCH_CHECK();
+}
 hipError_t init_scalars(Scalars* s, hipStream_t st) {
   hipLaunchKernelGGL(k_init_scalars, dim3(1), dim3(64), 0, st, s);
   return KTJ_LAUNCH_CHECK();
@@ -286,10 +305,36 @@ __global__ void k_scan_final(const uint32_t* in, uint64_t n, const uint64_t* sum
   if (write_total && blockIdx.x == 0 && threadIdx.x == 0) out[n] = (OutT)sums[m];
 }
 
+/* small inputs: the whole scan in one workgroup, tile after tile with a running carry */
+#define SCAN_SMALL_TILES 16u
+template <typename OutT>
+__global__ void k_scan_small(const uint32_t* in, uint64_t n, OutT* out, bool write_total) {
+  __shared__ uint64_t lds_wave[KTJ_BLOCK >> 6];
+  uint64_t carry = 0;
+  for (uint64_t tile = 0; tile < n; tile += SCAN_TILE) {
+    const uint64_t base = tile + (uint64_t)threadIdx.x * SCAN_ITEMS;
+    uint32_t v[SCAN_ITEMS];
+    uint64_t s = 0;
+    for (int k = 0; k < SCAN_ITEMS; ++k) { v[k] = base + k < n ? in[base + k] : 0u; s += v[k]; }
+    uint64_t tot;
+    uint64_t ex = block_exclusive_scan_u64(s, lds_wave, &tot) + carry;
+    for (int k = 0; k < SCAN_ITEMS; ++k) { /* a lane reads its items before it writes them: in place is fine */
+      if (base + k < n) out[base + k] = (OutT)ex;
+      ex += v[k];
+    }
+    carry += tot;
+  }
+  if (write_total && threadIdx.x == 0) out[n] = (OutT)carry;
+}
+
 uint64_t scan_tmp_elems(uint64_t n) { return (n + SCAN_TILE - 1) / SCAN_TILE + 2; }
 
 hipError_t scan_u32_to_u64(const uint32_t* in, uint64_t* out, uint64_t n, uint64_t* tmp, hipStream_t st) {
   const uint64_t m = (n + SCAN_TILE - 1) / SCAN_TILE;
+  if (m <= SCAN_SMALL_TILES) {
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(k_scan_small<uint64_t>), dim3(1), dim3(KTJ_BLOCK), 0, st, in, n, out, true);
+    return KTJ_LAUNCH_CHECK();
+  }
   if (m > 0) hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st, in, n, tmp);
   hipLaunchKernelGGL(k_scan_of_sums, dim3(1), dim3(KTJ_BLOCK), 0, st, tmp, m);
   if (m > 0)
@@ -302,6 +347,10 @@ hipError_t scan_u32_to_u64(const uint32_t* in, uint64_t* out, uint64_t n, uint64
 hipError_t scan_u32_inplace(uint32_t* data, uint64_t n, uint64_t* tmp, hipStream_t st) {
   const uint64_t m = (n + SCAN_TILE - 1) / SCAN_TILE;
   if (m == 0) return hipSuccess;
+  if (m <= SCAN_SMALL_TILES) {
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(k_scan_small<uint32_t>), dim3(1), dim3(KTJ_BLOCK), 0, st, (const uint32_t*)data, n, data, false);
+    return KTJ_LAUNCH_CHECK();
+  }
   hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st, (const uint32_t*)data, n, tmp);
   hipLaunchKernelGGL(k_scan_of_sums, dim3(1), dim3(KTJ_BLOCK), 0, st, tmp, m);
   /* every block reads its tile completely before writing it, and tiles do not overlap */
@@ -605,7 +654,8 @@ __global__ void k_key_range(const uint64_t* p, uint32_t stride, uint64_t n, int 
     if (lo <= hi) { atomicMin(&out->lo, lo); atomicMax(&out->hi, hi); }
   }
 }
-/* the per-workgroup ranges of the decode kernels into the plan's ranges: one workgroup per job */
+/* the per-workgroup ranges of the decode kernels into the plan's ranges: MERGE_SPLIT workgroups per job */
+#define MERGE_SPLIT 16u
 struct RangeJobs {
   const KeyRange* src[4];
   uint64_t n[4];
@@ -613,10 +663,11 @@ struct RangeJobs {
 };
 __global__ void k_merge_ranges(RangeJobs jobs, Scalars* sc) {
   __shared__ unsigned long long s_lo[1024 >> 6], s_hi[1024 >> 6];
-  const KeyRange* src = jobs.src[blockIdx.x];
-  const uint64_t n = jobs.n[blockIdx.x];
+  const uint32_t job = blockIdx.x / MERGE_SPLIT, part = blockIdx.x % MERGE_SPLIT;
+  const KeyRange* src = jobs.src[job];
+  const uint64_t n = jobs.n[job];
   unsigned long long lo = ~0ULL, hi = 0;
-  for (uint64_t i = threadIdx.x; i < n; i += blockDim.x) {
+  for (uint64_t i = (uint64_t)part * blockDim.x + threadIdx.x; i < n; i += (uint64_t)MERGE_SPLIT * blockDim.x) {
     const KeyRange r = src[i];
     if (r.lo <= r.hi) { lo = r.lo < lo ? r.lo : lo; hi = r.hi > hi ? r.hi : hi; }
   }
@@ -629,7 +680,7 @@ __global__ void k_merge_ranges(RangeJobs jobs, Scalars* sc) {
   __syncthreads();
   if (threadIdx.x == 0) {
     for (uint32_t k = 1; k < (blockDim.x >> 6); ++k) { lo = s_lo[k] < lo ? s_lo[k] : lo; hi = s_hi[k] > hi ? s_hi[k] : hi; }
-    KeyRange* out = &sc->plan.range[jobs.dst[blockIdx.x]];
+    KeyRange* out = &sc->plan.range[jobs.dst[job]];
     if (lo <= hi) { atomicMin(&out->lo, lo); atomicMax(&out->hi, hi); }
   }
 }
@@ -649,13 +700,13 @@ __global__ void k_plan_tables(Scalars* sc, uint32_t cap_full, uint32_t cap_narro
 __device__ __forceinline__ uint64_t table_extent(const Table& t) {
   return t.ctl->direct ? t.ctl->span + 1ull : (uint64_t)t.mask + 1ull;
 }
-__global__ void k_clear_keys(Table t) {
+__device__ __forceinline__ void clear_keys(const Table& t) {
   if (t.ctl->direct && !t.keyed_direct) return; /* keys are not used at all */
   const uint64_t n = table_extent(t);
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) t.keys[i] = KTJ_EMPTY_KEY;
   if (blockIdx.x == 0 && threadIdx.x == 0) t.keys[t.mask + 1ull] = KTJ_EMPTY_KEY;
 }
-__global__ void k_clear_full(Table t, FullCols c) {
+__device__ __forceinline__ void clear_full(const Table& t, const FullCols& c) {
   const uint64_t n = table_extent(t);
   FullPay z; z.first_ts = 0; z.stream = 0;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i <= n; i += (uint64_t)gridDim.x * blockDim.x) {
@@ -667,12 +718,23 @@ __global__ void k_clear_full(Table t, FullCols c) {
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i <= words; i += (uint64_t)gridDim.x * blockDim.x)
     c.has_runtime[i < words ? i : (t.mask + 1ull) / 32] = 0;
 }
-__global__ void k_clear_narrow(Table t, NarrowCols c) {
+__device__ __forceinline__ void clear_narrow(const Table& t, const NarrowCols& c) {
   const uint64_t n = table_extent(t);
   NarrowPay z; z.ext_val = 0; z.info = 0; z.pay[0] = z.pay[1] = z.pay[2] = 0;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i <= n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t k = i < n ? i : t.mask + 1ull;
     c.ext_src[k] = 0; c.kern_src[k] = 0; c.copy_src[k] = 0; c.pay[k] = z;
+  }
+}
+
+/* all five in one launch: blockIdx.y picks the part */
+__global__ void k_clear_tables(Table tf, FullCols fc, Table tn, NarrowCols nc, Table cpu) {
+  switch (blockIdx.y) {
+    case 0: clear_keys(tf); break;
+    case 1: clear_keys(tn); break;
+    case 2: clear_keys(cpu); break;
+    case 3: clear_full(tf, fc); break;
+    default: clear_narrow(tn, nc); break;
   }
 }
 
@@ -690,7 +752,7 @@ hipError_t plan_tables(const KeyRange* parts, uint64_t n_generic, uint64_t n_run
   job(parts + bg + br, br, KTJ_TBL_NARROW);
   job(parts + bg + 2 * br, bd, KTJ_TBL_FULL);
   for (uint32_t k = n_jobs; k < 4; ++k) { jobs.src[k] = nullptr; jobs.n[k] = 0; jobs.dst[k] = 0; }
-  if (n_jobs) hipLaunchKernelGGL(k_merge_ranges, dim3(n_jobs), dim3(1024), 0, st, jobs, sc);
+  if (n_jobs) hipLaunchKernelGGL(k_merge_ranges, dim3(n_jobs * MERGE_SPLIT), dim3(256), 0, st, jobs, sc);
   if (n_ext)
     hipLaunchKernelGGL(k_key_range, dim3(n_ext < 512ull * KTJ_BLOCK * 4 ? grid_for(n_ext, KTJ_BLOCK * 4) : 512u), b, 0, st, reinterpret_cast<const uint64_t*>(e), 2u,
                        n_ext, 0, &sc->plan.range[KTJ_TBL_NARROW]);
@@ -698,12 +760,10 @@ hipError_t plan_tables(const KeyRange* parts, uint64_t n_generic, uint64_t n_run
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t clear_tables(Table tf, FullCols fc, Table tn, NarrowCols nc, Table cpu, hipStream_t st) {
-  const dim3 b(KTJ_BLOCK);
-  hipLaunchKernelGGL(k_clear_keys, dim3(grid_stride_for((uint64_t)tf.mask + 1, KTJ_BLOCK * 4)), b, 0, st, tf);
-  hipLaunchKernelGGL(k_clear_keys, dim3(grid_stride_for((uint64_t)tn.mask + 1, KTJ_BLOCK * 4)), b, 0, st, tn);
-  hipLaunchKernelGGL(k_clear_keys, dim3(grid_stride_for((uint64_t)cpu.mask + 1, KTJ_BLOCK * 4)), b, 0, st, cpu);
-  hipLaunchKernelGGL(k_clear_full, dim3(grid_stride_for((uint64_t)tf.mask + 1, KTJ_BLOCK * 4)), b, 0, st, tf, fc);
-  hipLaunchKernelGGL(k_clear_narrow, dim3(grid_stride_for((uint64_t)tn.mask + 1, KTJ_BLOCK * 4)), b, 0, st, tn, nc);
+  uint64_t most = (uint64_t)tf.mask + 1;
+  if ((uint64_t)tn.mask + 1 > most) most = (uint64_t)tn.mask + 1;
+  if ((uint64_t)cpu.mask + 1 > most) most = (uint64_t)cpu.mask + 1;
+  hipLaunchKernelGGL(k_clear_tables, dim3(grid_stride_for(most, KTJ_BLOCK * 4), 5), dim3(KTJ_BLOCK), 0, st, tf, fc, tn, nc, cpu);
   return KTJ_LAUNCH_CHECK();
 }
 
