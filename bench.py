@@ -175,7 +175,10 @@ def cpu_baseline(config, sample_device_rows):
     from kineto_amd import abi
     from kineto_amd.engine import TraceEngine
     import oracle_glue as og
-    sp, release = abi.synth_stream(config, sample_device_rows, host_name="bench")
+    # with the reference logger at hand the sample takes its base time and host name, so that the
+    # three documents (engine, port, reference logger) can be compared byte for byte
+    stream_args = og.ref_stream_args() if og.have_ref() else dict(host_name="bench")
+    sp, release = abi.synth_stream(config, sample_device_rows, **stream_args)
     s = sp.contents
     n_records = s.n_generic + s.n_runtime + s.n_device
     t0 = time.perf_counter()
@@ -183,7 +186,7 @@ def cpu_baseline(config, sample_device_rows):
     dt = time.perf_counter() - t0
     import numpy as np
     want = ora.output_view()
-    with TraceEngine(s.trace_name.decode(), device=0) as eng:
+    with TraceEngine(s.trace_name.decode(), base_time_ns=s.base_time_ns, device=0) as eng:
         eng.submit_stream(sp)
         eng.process()
         got = eng.output_view()

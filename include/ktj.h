@@ -413,6 +413,8 @@ typedef struct ktj_engine ktj_engine;
  * the same bytes.
  * KTJ_CREATE_HASH_JOIN keeps the join tables in hash mode even when the correlation ids are dense
  * enough for direct addressing (the engine chooses per table otherwise); same results, slower.
+ * KTJ_CREATE_DISPLAY_NS writes "displayTimeUnit": "ns" instead of "ms" in the header, as a reference
+ * built with DISPLAY_TRACE_IN_NS does (output_json.cpp:451-454); nothing else changes.
  * KTJ_CREATE_PAIR_SORT sorts (key, arrival index) pairs also where key and index fit one 64-bit
  * word (the engine sorts single words then otherwise); same results, slower.
  * ---------------------------------------------------------------------------------------- */
@@ -420,6 +422,7 @@ typedef struct ktj_engine ktj_engine;
 #define KTJ_CREATE_TILE_EMIT 0x2u
 #define KTJ_CREATE_HASH_JOIN 0x4u
 #define KTJ_CREATE_PAIR_SORT 0x8u
+#define KTJ_CREATE_DISPLAY_NS 0x10u
 int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int hip_device,
                uint32_t flags);
 void ktj_destroy(ktj_engine* e);

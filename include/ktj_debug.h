@@ -22,7 +22,8 @@ enum {
   KTJ_DBG_LEN = 7,        /* uint32[N] byte length per sorted position          */
   KTJ_DBG_OFFS = 8,       /* uint64[N+1] exclusive scan of the lengths          */
   KTJ_DBG_MAT = 9,        /* 96-byte joined rows per arrival index              */
-  KTJ_DBG_SORT_KEYS = 10, /* uint64[N] sorted composite keys                    */
+  KTJ_DBG_SORT_KEYS = 10, /* uint64[N] sorted composite keys (engines created with
+                             KTJ_CREATE_PAIR_SORT only: KTJ_ERR_STATE otherwise)  */
   KTJ_DBG_NAME_VIEW = 11, /* bytes: all names after the name pipeline           */
   KTJ_DBG_NAME_OFF = 12,  /* uint64[n_strings+1]                                */
   KTJ_DBG_ARG_VIEW = 13,

@@ -435,7 +435,7 @@ int ktj_trace_start(ktj_engine* e, const char* const* meta_kv, size_t n_kv, cons
   if (!e || (n_kv && !meta_kv)) return KTJ_ERR_ARG;
   if (e->bad_sink) return KTJ_OK;
   e->txt_header.clear();
-  append_trace_start(e->txt_header, meta_kv, n_kv, device_properties, e->base_time_ns);
+  append_trace_start(e->txt_header, meta_kv, n_kv, device_properties, e->base_time_ns, (e->flags & KTJ_CREATE_DISPLAY_NS) != 0);
   e->started = true;
   e->processed = false;
   return KTJ_OK;
@@ -1281,7 +1281,9 @@ int ktj_debug_fetch(ktj_engine* e, int what, void* dst, uint64_t cap, uint64_t* 
     case KTJ_DBG_LEN: src = e->len_sorted.p; n = N * 4; break;
     case KTJ_DBG_OFFS: src = e->offs.p; n = (N + 1) * 8; break;
     case KTJ_DBG_MAT: src = e->mat.p; n = N * sizeof(MatRow); break;
-    case KTJ_DBG_SORT_KEYS: src = e->sorted_keys; n = N * 8; break;
+    case KTJ_DBG_SORT_KEYS:
+      if (!e->sorted_keys) { e->last_error = "the sorted keys exist only in an engine created with KTJ_CREATE_PAIR_SORT"; return KTJ_ERR_STATE; }
+      src = e->sorted_keys; n = N * 8; break;
     case KTJ_DBG_NAME_VIEW: src = e->d_name_blob.p; n = e->blob_bytes * 2 + 8ull * e->n_strings; break;
     case KTJ_DBG_NAME_OFF: src = e->d_name_off.p; n = (e->n_strings + 1) * 8; break;
     case KTJ_DBG_ARG_VIEW: src = e->d_arg_blob.p; n = e->blob_bytes; break;

@@ -75,7 +75,7 @@ void metadata_event(std::string& out, const char* name, int64_t ts, const std::s
 }  // namespace
 
 void append_trace_start(std::string& out, const char* const* meta_kv, size_t n_kv,
-                        const char* device_properties, int64_t base_time_ns) {
+                        const char* device_properties, int64_t base_time_ns, bool display_ns) {
   out += " {\n    \"schemaVersion\": 1,\n    \"deviceProperties\": [";
   out += device_properties ? device_properties : "";
   out += "],\n    ";
@@ -86,7 +86,8 @@ void append_trace_start(std::string& out, const char* const* meta_kv, size_t n_k
     out += sanitize_only(meta_kv[2 * i + 1]);
     out += ',';
   }
-  out += "\n    \"displayTimeUnit\": \"ms\",\n    \"baseTimeNanoseconds\": ";
+  out += display_ns ? "\n    \"displayTimeUnit\": \"ns\",\n    \"baseTimeNanoseconds\": "   /* DISPLAY_TRACE_IN_NS, output_json.cpp:451-454 */
+                    : "\n    \"displayTimeUnit\": \"ms\",\n    \"baseTimeNanoseconds\": ";
   out += std::to_string(base_time_ns);
   out += ",\n    \"traceEvents\": [\n    ";
 }

@@ -15,7 +15,7 @@ namespace ktj {
 
 /* ChromeTraceLogger::handleTraceStart + metadataToJSON (libkineto/src/output_json.cpp:414-479) */
 void append_trace_start(std::string& out, const char* const* meta_kv, size_t n_kv,
-                        const char* device_properties, int64_t base_time_ns);
+                        const char* device_properties, int64_t base_time_ns, bool display_ns = false);
 /* handleDeviceInfo (output_json.cpp:507-542) */
 void append_device_info(std::string& out, const ktj_device_info& info, int64_t base_time_ns);
 /* handleResourceInfo (output_json.cpp:544-577) */

@@ -89,7 +89,11 @@ struct GpuChromeTraceLogger::Packed {
 GpuChromeTraceLogger::GpuChromeTraceLogger(const std::string& traceFileName, int hipDevice)
     : fileName_(traceFileName), staging_(new Packed) {
   /* the engine applies the default-file-name rule (output_json.cpp:481-483) for an empty name */
-  const int rc = ktj_create(&engine_, traceFileName.c_str(), ChromeTraceBaseTime::singleton().get(), hipDevice, 0);
+  uint32_t flags = 0;
+#ifdef DISPLAY_TRACE_IN_NS /* the reference's compile-time switch (output_json.cpp:451-454) */
+  flags |= KTJ_CREATE_DISPLAY_NS;
+#endif
+  const int rc = ktj_create(&engine_, traceFileName.c_str(), ChromeTraceBaseTime::singleton().get(), hipDevice, flags);
   if (rc != KTJ_OK) {
     LOG(ERROR) << "GPU trace engine unavailable (ktj_create rc=" << rc << "): "
                << (engine_ ? ktj_last_error(engine_) : "no engine");

@@ -10,7 +10,8 @@ from kineto_amd import abi
 
 pytestmark = pytest.mark.gpu
 
-CASES = [(1, 10000), (2, 20000), (3, 30000), (4, 30000), (5, 5000), (1, 1), (3, 4097), (5, 3)]
+# (1, 10922) and (1, 10923): 32766 and 32769 rows, either side of the single-workgroup scan's limit
+CASES = [(1, 10000), (2, 20000), (3, 30000), (4, 30000), (5, 5000), (1, 1), (3, 4097), (5, 3), (1, 10922), (1, 10923)]
 
 
 def _first_diff(a, b):
@@ -221,6 +222,24 @@ def test_golden_digests_on_gpu():
             assert len(got) == g["output_bytes"], key
             assert hashlib.sha256(got).hexdigest() == g["output_sha256"], key
         release()
+
+
+def test_display_unit_switch():
+    """KTJ_CREATE_DISPLAY_NS is the reference's DISPLAY_TRACE_IN_NS build switch (output_json.cpp:451-454):
+    one word of the header changes."""
+    import oracle_glue as og
+    from kineto_amd.engine import TraceEngine
+    sp, release = abi.synth_stream(1, 300, host_name="unit")
+    ora = og.OracleRun(sp)
+    want = ora.output()
+    ora.close()
+    with TraceEngine(sp.contents.trace_name.decode(), device=0, display_ns=True) as eng:
+        eng.submit_stream(sp)
+        eng.process()
+        got = eng.output()
+    release()
+    assert want.count(b'"displayTimeUnit": "ms"') == 1
+    assert got == want.replace(b'"displayTimeUnit": "ms"', b'"displayTimeUnit": "ns"')
 
 
 def test_empty_and_tiny_streams_on_gpu():
