@@ -387,7 +387,7 @@ typedef struct ktj_stats {
 enum {
   KTJ_STAGE_DICT = 0,     /* name / string dictionary sanitising                               */
   KTJ_STAGE_DECODE = 1,   /* raw records → columns                                             */
-  KTJ_STAGE_CONVERT = 2,  /* clock conversion + window filter                                  */
+  KTJ_STAGE_CONVERT = 2,  /* clock conversion + window filter: done inside decode, reads 0            */
   KTJ_STAGE_JOIN = 3,     /* hash build + probe (ext-corr, runtime↔device, streams)            */
   KTJ_STAGE_SORT = 4,     /* key build + stable radix sort                                     */
   KTJ_STAGE_SIZE = 5,     /* exact byte length per record                                      */

@@ -829,17 +829,17 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
 
   /* ---- stage 1: decode ---- */
   KeyRange* parts = e->range_parts.as<KeyRange>(); /* [generic | runtime | runtime narrowed | device] */
-  HIPCHK(decode_generic(g_recs, ng, c, 0, sc, ctx, parts, st));
-  HIPCHK(decode_runtime(r_recs, nr, c, ng, parts + decode_blocks(ng), parts + decode_blocks(ng) + decode_blocks(nr), st));
-  HIPCHK(decode_device(d_recs, nd, c, ng + nr, e->dev_brief.as<DevBrief>(), parts + decode_blocks(ng) + 2 * decode_blocks(nr), st));
-  HIPCHK(hipEventRecord(e->ev[EV_DECODE], st));
-
-  /* ---- stage 2a: clock + window ---- */
+  /* stage 2a, clock conversion and window filter, happens inside the runtime and device decode */
   ClockDev clk;
   clk.t0_approx = e->clock.t0_approx; clk.t0 = e->clock.t0;
   memcpy(&clk.scale_bits, &e->clock.scale, 8);
   clk.async_offset = e->clock.async_offset; clk.runtime_mode = e->clock.runtime_mode; clk.device_mode = e->clock.device_mode;
-  HIPCHK(convert_rows(c, ng, nr, nd, clk, e->win_start, e->win_end, sc, st));
+  HIPCHK(decode_generic(g_recs, ng, c, 0, sc, ctx, parts, st));
+  HIPCHK(decode_runtime(r_recs, nr, c, ng, parts + decode_blocks(ng), parts + decode_blocks(ng) + decode_blocks(nr), clk,
+                        e->win_start, e->win_end, sc, st));
+  HIPCHK(decode_device(d_recs, nd, c, ng + nr, e->dev_brief.as<DevBrief>(), parts + decode_blocks(ng) + 2 * decode_blocks(nr), clk,
+                       e->win_start, e->win_end, sc, st));
+  HIPCHK(hipEventRecord(e->ev[EV_DECODE], st));
   HIPCHK(hipEventRecord(e->ev[EV_CONVERT], st));
 
   /* ---- stage 2b: joins ---- */

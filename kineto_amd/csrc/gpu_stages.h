@@ -194,14 +194,11 @@ hipError_t dict_write(const char* blob, const uint64_t* off, uint32_t n, const u
 uint64_t decode_blocks(uint64_t n);
 hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint64_t first, Scalars* sc, EmitCtx ctx,
                           KeyRange* id_range, hipStream_t st);
+/* the runtime and device kernels also convert the clock and apply the capture window */
 hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, KeyRange* id_range,
-                          KeyRange* narrow_range, hipStream_t st);
+                          KeyRange* narrow_range, ClockDev clk, int64_t win_start, int64_t win_end, Scalars* sc, hipStream_t st);
 hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, DevBrief* brief, KeyRange* id_range,
-                         hipStream_t st);
-
-/* ---- stage 2a: clock conversion + window filter (runtime and device rows) ---- */
-hipError_t convert_rows(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, ClockDev clk,
-                        int64_t win_start, int64_t win_end, Scalars* sc, hipStream_t st);
+                         ClockDev clk, int64_t win_start, int64_t win_end, Scalars* sc, hipStream_t st);
 
 /* ---- stage 2b: joins ---- */
 /* key ranges of the three tables, then their modes (direct unless force_hash or the span is too wide).

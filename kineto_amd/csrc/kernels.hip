@@ -512,8 +512,11 @@ __global__ void k_decode_generic(const ktj_generic_rec* recs, uint64_t n, Column
   c.meta[a] = (generic_record_prints(g, ctx) ? KTJ_M_VALID : 0u) | (KTJ_CLASS_GENERIC << KTJ_M_CLASS_SHIFT);
   c.ext[a] = 0;
 }
+/* The runtime and device kernels also convert the clock and apply the capture window (stage 2a:
+ * RocprofActivityApi.cpp:166-175, ApproximateClock.cpp:83-90, RocprofActivity.h:42-47 and 122-127,
+ * GenericActivityProfiler.cpp:329-340), so that timestamp and duration are written once. */
 __global__ void k_decode_runtime(const ktj_runtime_rec* recs, uint64_t n, Columns c, uint64_t first, KeyRange* id_range,
-                                 KeyRange* narrow_range) {
+                                 KeyRange* narrow_range, ClockDev clk, int64_t win_start, int64_t win_end, Scalars* sc) {
   __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_runtime_rec) / 16];
   uint32_t cnt;
   const ktj_runtime_rec* l = stage_records(recs, n, stage, &cnt);
@@ -523,39 +526,55 @@ __global__ void k_decode_runtime(const ktj_runtime_rec* recs, uint64_t n, Column
     block_key_range(has, id, id_range);
     block_key_range(has, narrow_corr_key(id), narrow_range);
   }
-  if (threadIdx.x >= cnt) return;
+  uint32_t oor = 0;
+  if (threadIdx.x < cnt) {
   const ktj_runtime_rec* r = &l[threadIdx.x];
   const uint64_t a = first + (uint64_t)blockIdx.x * KTJ_BLOCK + threadIdx.x;
-  c.ts[a] = (int64_t)r->begin;
-  c.dur[a] = (int64_t)r->end;
+  uint64_t b = r->begin, e = r->end;
+  convert_range(clk, clk.runtime_mode, &b, &e);
+  const int64_t ts = (int64_t)b, dur = (int64_t)(e - b);   /* RocprofActivity.h:42-47 */
+  oor = out_of_range(ts, dur, win_start, win_end) ? 1u : 0u;
+  c.ts[a] = ts;
+  c.dur[a] = dur;
   c.corr[a] = r->id;
   c.dev[a] = (int64_t)r->pid;
   c.res[a] = (int64_t)r->tid;
   const uint32_t kind = r->kind <= KTJ_RT_MALLOC ? r->kind : KTJ_RT_DEFAULT;
   const uint64_t stream = kind == KTJ_RT_KERNEL ? r->u.kernel.stream : (kind == KTJ_RT_COPY ? r->u.copy.stream : 0);
-  c.meta[a] = (KTJ_CLASS_RUNTIME << KTJ_M_CLASS_SHIFT) | (kind << KTJ_M_KIND_SHIFT) | (stream != 0 ? KTJ_M_HAS_STREAM : 0u);
+  c.meta[a] = (KTJ_CLASS_RUNTIME << KTJ_M_CLASS_SHIFT) | (kind << KTJ_M_KIND_SHIFT) | (stream != 0 ? KTJ_M_HAS_STREAM : 0u) |
+              (oor ? 0u : KTJ_M_VALID);
   c.ext[a] = 0;
+  }
+  block_add(&sc->out_of_range, oor);
 }
 __global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns c, uint64_t first, DevBrief* brief,
-                                KeyRange* id_range) {
+                                KeyRange* id_range, ClockDev clk, int64_t win_start, int64_t win_end, Scalars* sc) {
   __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_device_rec) / 16];
   uint32_t cnt;
   const ktj_device_rec* l = stage_records(recs, n, stage, &cnt);
   block_key_range(threadIdx.x < cnt, threadIdx.x < cnt ? l[threadIdx.x].id : 0, id_range);
-  if (threadIdx.x >= cnt) return;
+  uint32_t oor = 0;
+  if (threadIdx.x < cnt) {
   const ktj_device_rec* d = &l[threadIdx.x];
   const uint64_t a = first + (uint64_t)blockIdx.x * KTJ_BLOCK + threadIdx.x;
   const uint32_t dom = d->domain <= KTJ_DOM_MEMSET ? d->domain : KTJ_DOM_KERNEL_DISPATCH;
-  c.ts[a] = (int64_t)d->begin;
-  c.dur[a] = (int64_t)d->end;
+  uint64_t b = d->begin, e = d->end;
+  convert_range(clk, clk.device_mode, &b, &e);
+  int64_t ts, dur;
+  device_times(dom, b, e, &ts, &dur);
+  oor = out_of_range(ts, dur, win_start, win_end) ? 1u : 0u;
+  c.ts[a] = ts;
+  c.dur[a] = dur;
   c.corr[a] = d->id;
   c.dev[a] = (int64_t)d->device;
   c.res[a] = (int64_t)d->stream;
-  c.meta[a] = (KTJ_CLASS_DEVICE << KTJ_M_CLASS_SHIFT) | (dom << KTJ_M_KIND_SHIFT);
+  c.meta[a] = (KTJ_CLASS_DEVICE << KTJ_M_CLASS_SHIFT) | (dom << KTJ_M_KIND_SHIFT) | (oor ? 0u : KTJ_M_VALID);
   c.ext[a] = 0;
-  DevBrief b;
-  b.queue = d->queue; b.device = d->device; b.domain = d->domain;
-  brief[a - first] = b;
+  DevBrief br;
+  br.queue = d->queue; br.device = d->device; br.domain = d->domain;
+  brief[a - first] = br;
+  }
+  block_add(&sc->out_of_range, oor);
 }
 
 uint64_t decode_blocks(uint64_t n) { return grid_for(n, KTJ_BLOCK); }
@@ -566,55 +585,17 @@ hipError_t decode_generic(const ktj_generic_rec* r, uint64_t n, Columns c, uint6
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t decode_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, KeyRange* id_range,
-                          KeyRange* narrow_range, hipStream_t st) {
+                          KeyRange* narrow_range, ClockDev clk, int64_t win_start, int64_t win_end, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
   hipLaunchKernelGGL(k_decode_runtime, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, id_range,
-                     narrow_range);
+                     narrow_range, clk, win_start, win_end, sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t decode_device(const ktj_device_rec* r, uint64_t n, Columns c, uint64_t first, DevBrief* brief, KeyRange* id_range,
-                         hipStream_t st) {
+                         ClockDev clk, int64_t win_start, int64_t win_end, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_decode_device, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, brief, id_range);
-  return KTJ_LAUNCH_CHECK();
-}
-
-/* ------------------------------------------------------------------------------------------ */
-/* stage 2a: clock conversion and window filter                                                 */
-/*   RocprofActivityApi.cpp:166-175, ApproximateClock.cpp:83-90, RocprofActivity.h:122-127,      */
-/*   GenericActivityProfiler.cpp:329-340                                                        */
-/* ------------------------------------------------------------------------------------------ */
-__global__ void k_convert(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, ClockDev clk,
-                          int64_t win_start, int64_t win_end, Scalars* sc) {
-  uint32_t n_oor = 0;
-  const uint64_t n = n_runtime + n_device;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    const uint64_t a = first_runtime + i;
-    uint64_t b = (uint64_t)c.ts[a], e = (uint64_t)c.dur[a];
-    uint32_t meta = c.meta[a];
-    int64_t ts, dur;
-    if (i < n_runtime) {
-      convert_range(clk, clk.runtime_mode, &b, &e);
-      ts = (int64_t)b;                 /* RocprofActivity.h:42-47 */
-      dur = (int64_t)(e - b);
-    } else {
-      convert_range(clk, clk.device_mode, &b, &e);
-      device_times((meta & KTJ_M_KIND_MASK) >> KTJ_M_KIND_SHIFT, b, e, &ts, &dur);
-    }
-    if (out_of_range(ts, dur, win_start, win_end)) ++n_oor;
-    else meta |= KTJ_M_VALID;
-    c.ts[a] = ts;
-    c.dur[a] = dur;
-    c.meta[a] = meta;
-  }
-  block_add(&sc->out_of_range, n_oor);
-}
-hipError_t convert_rows(Columns c, uint64_t first_runtime, uint64_t n_runtime, uint64_t n_device, ClockDev clk,
-                        int64_t win_start, int64_t win_end, Scalars* sc, hipStream_t st) {
-  const uint64_t n = n_runtime + n_device;
-  if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_convert, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, c, first_runtime, n_runtime,
-                     n_device, clk, win_start, win_end, sc);
+  hipLaunchKernelGGL(k_decode_device, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, brief, id_range,
+                     clk, win_start, win_end, sc);
   return KTJ_LAUNCH_CHECK();
 }
 
