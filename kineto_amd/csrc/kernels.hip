@@ -1054,26 +1054,37 @@ __device__ __forceinline__ uint64_t dense_hash(int32_t device, uint64_t key) {
 __global__ void k_dense_first(const DevBrief* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
                               Scalars* sc) {
   __shared__ unsigned long long l_key[DENSE_LOCAL_SLOTS];
+  __shared__ unsigned long long l_pair_key[DENSE_LOCAL_SLOTS];
+  __shared__ int32_t l_pair_dev[DENSE_LOCAL_SLOTS];
   __shared__ uint32_t l_min[DENSE_LOCAL_SLOTS];
   if (sc->have_stream_src == 0) return;
   for (uint32_t k = threadIdx.x; k < DENSE_LOCAL_SLOTS; k += blockDim.x) { l_key[k] = KTJ_EMPTY_KEY; l_min[k] = 0xFFFFFFFFu; }
   __syncthreads();
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     uint64_t key;
-    if (!dense_key(d[i], (uint64_t)c.res[first_device + i], &key)) continue;
-    const uint64_t h = dense_hash(d[i].device, key);
+    const DevBrief b = d[i];
+    if (!dense_key(b, (uint64_t)c.res[first_device + i], &key)) continue;
+    const uint64_t h = dense_hash(b.device, key);
     uint32_t slot = (uint32_t)(h >> 20) & (DENSE_LOCAL_SLOTS - 1u);
     bool placed = false;
     for (uint32_t probe = 0; probe < 16 && !placed; ++probe) {
       unsigned long long cur = l_key[slot];
-      if (cur == KTJ_EMPTY_KEY) cur = atomicCAS(&l_key[slot], (unsigned long long)KTJ_EMPTY_KEY, (unsigned long long)h);
+      if (cur == KTJ_EMPTY_KEY) {
+        cur = atomicCAS(&l_key[slot], (unsigned long long)KTJ_EMPTY_KEY, (unsigned long long)h);
+        /* the pair itself, for the table entry: every row of the pair would write the same two values
+         * (two pairs with one hash are told apart when the rows read the table back) */
+        if (cur == KTJ_EMPTY_KEY) { l_pair_dev[slot] = b.device; l_pair_key[slot] = key; }
+      }
       if (cur == KTJ_EMPTY_KEY || cur == h) { atomicMin(&l_min[slot], (uint32_t)i); placed = true; }
       else slot = (slot + 1u) & (DENSE_LOCAL_SLOTS - 1u);
     }
     if (!placed) { /* local table crowded: straight to the global one */
       const uint32_t g = table_insert(t.d_hash, KTJ_DENSE_CAP - 1u, h);
       if (g == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_STREAMS);
-      else if (t.d_first[g] > (uint32_t)i) atomicMin(&t.d_first[g], (uint32_t)i);
+      else {
+        if (t.d_first[g] > (uint32_t)i) atomicMin(&t.d_first[g], (uint32_t)i);
+        t.d_dev[g] = b.device; t.d_key[g] = key;
+      }
     }
   }
   __syncthreads();
@@ -1083,21 +1094,10 @@ __global__ void k_dense_first(const DevBrief* d, uint64_t n, Columns c, uint64_t
     const uint32_t g = table_insert(t.d_hash, KTJ_DENSE_CAP - 1u, h);
     if (g == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_STREAMS); continue; }
     if (t.d_first[g] > l_min[k]) atomicMin(&t.d_first[g], l_min[k]);
+    t.d_dev[g] = l_pair_dev[k]; t.d_key[g] = l_pair_key[k];
   }
 }
-/* pass 3b: the first row of each pair records the pair itself (single writer per slot) */
-__global__ void k_dense_owner(const DevBrief* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
-                              const Scalars* sc) {
-  if (sc->have_stream_src == 0) return;
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  uint64_t key;
-  if (!dense_key(d[i], (uint64_t)c.res[first_device + i], &key)) return;
-  const uint32_t slot = table_find(t.d_hash, KTJ_DENSE_CAP - 1u, dense_hash(d[i].device, key));
-  if (slot == KTJ_NOSLOT) return;
-  if (t.d_first[slot] == (uint32_t)i) { t.d_dev[slot] = d[i].device; t.d_key[slot] = key; }
-}
-/* pass 3c (one workgroup): index = 1 + number of pairs of the same device seen earlier */
+/* pass 3b (one workgroup): index = 1 + number of pairs of the same device seen earlier */
 #define KTJ_DENSE_MAX KTJ_MAX_STREAM_PAIRS
 __global__ void k_dense_rank(StreamTables t, Scalars* sc) {
   __shared__ uint32_t slots[KTJ_DENSE_MAX];
@@ -1127,7 +1127,7 @@ __global__ void k_dense_rank(StreamTables t, Scalars* sc) {
     t.d_rank[s] = rank;
   }
 }
-/* pass 3d: resourceId() = stream != 0 ? stream : queue (RocprofActivity.h:100-102) */
+/* pass 3c: resourceId() = stream != 0 ? stream : queue (RocprofActivity.h:100-102) */
 __global__ void k_dense_assign(const DevBrief* d, uint64_t n, Columns c, uint64_t first_device, StreamTables t,
                                Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1155,7 +1155,6 @@ hipError_t backfill_streams(const DevBrief* d, uint64_t n, Columns c, uint64_t f
   hipLaunchKernelGGL(k_queue_build, g, b, 0, st, d, n, c, first_device, t, sc);
   hipLaunchKernelGGL(k_queue_fill, g, b, 0, st, d, n, c, first_device, t, (const Scalars*)sc);
   hipLaunchKernelGGL(k_dense_first, dim3(grid_stride_for(n, KTJ_BLOCK * 8)), b, 0, st, d, n, c, first_device, t, sc);
-  hipLaunchKernelGGL(k_dense_owner, g, b, 0, st, d, n, c, first_device, t, (const Scalars*)sc);
   hipLaunchKernelGGL(k_dense_rank, dim3(1), dim3(1024), 0, st, t, sc);
   hipLaunchKernelGGL(k_dense_assign, g, b, 0, st, d, n, c, first_device, t, sc);
   return KTJ_LAUNCH_CHECK();
