@@ -131,7 +131,8 @@ struct Scalars {
   unsigned int n_res_ranks;           /* distinct resourceId values */
   unsigned int n_dense;               /* distinct (device, stream key) pairs */
   unsigned int runtime_ids_repeat;    /* two runtime rows share a slot of the full table */
-  JoinPlan plan;                      /* key ranges and modes of the join tables */
+  alignas(256) JoinPlan plan;         /* key ranges and modes of the join tables: read by every row of the join
+                                         kernels, so kept off the cache lines that take the counters' atomics */
 };
 #define KTJ_DEVERR_TABLE_FULL 1u         /* a join table sized from the record counts filled up (a defect) */
 #define KTJ_DEVERR_DISTINCT_DEVICES 2u   /* more distinct deviceId values than the rank set holds: the sort

@@ -1239,9 +1239,9 @@ __global__ void k_collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* s
       mn = red_min[k] < mn ? red_min[k] : mn;
       mx = red_max[k] > mx ? red_max[k] : mx;
     }
-    if (mn <= mx) { /* the atomics only where the workgroup widens the range (rare after the first few) */
-      if (mn < sc->ts_min_biased) atomicMin(&sc->ts_min_biased, (unsigned long long)mn);
-      if (mx > sc->ts_max_biased) atomicMax(&sc->ts_max_biased, (unsigned long long)mx);
+    if (mn <= mx) { /* (reading the current range first, to skip the atomics, costs more than they do) */
+      atomicMin(&sc->ts_min_biased, (unsigned long long)mn);
+      atomicMax(&sc->ts_max_biased, (unsigned long long)mx);
     }
   }
   block_add(&sc->n_valid, n_valid);
