@@ -389,7 +389,7 @@ struct TileWriter {
 
 /* Long dictionary strings (templated C++ kernel names run to kilobytes) are not copied by the lane
  * that owns the activity but by all lanes that are active with it: for one owner at a time,
- * neighbouring lanes move neighbouring 8-byte words, so loads and stores are whole lines.  The
+ * neighbouring lanes move neighbouring 16-byte blocks, so loads and stores are whole lines.  The
  * owner has already brought its output to a block boundary; `src` is the first byte that lands on
  * that boundary (any alignment: two aligned loads are funnel-shifted), `dst` the block, `n_words`
  * the 8-byte words of the whole blocks (0 for lanes that only help).  Works under any set of
@@ -397,6 +397,9 @@ struct TileWriter {
 #define KTJ_COOP_MIN_BYTES 256u
 #if defined(__HIP_DEVICE_COMPILE__)
 static __device__ __attribute__((noinline)) void cooperative_word_copy(const char* src, uint64_t* dst, uint32_t n_words) {
+  typedef unsigned long long v2u64 __attribute__((ext_vector_type(2)));
+  typedef __attribute__((address_space(1))) v2u64* gblocks;            /* document and dictionary are */
+  typedef const __attribute__((address_space(1))) uint64_t* gwords;    /* global memory: no flat accesses */
   const uint64_t active = __ballot(1);
   const uint32_t lane = (uint32_t)(threadIdx.x & 63u);
   const uint32_t n_active = (uint32_t)__popcll(active);
@@ -405,15 +408,21 @@ static __device__ __attribute__((noinline)) void cooperative_word_copy(const cha
   while (todo) {
     const int owner = __ffsll((unsigned long long)todo) - 1;
     todo &= todo - 1;
-    const uint32_t n = (uint32_t)__shfl((int)n_words, owner);
+    const uint32_t n = (uint32_t)__shfl((int)n_words, owner) >> 1; /* whole blocks: a lane moves sixteen bytes at a time */
     const uintptr_t sa = (uintptr_t)__shfl((unsigned long long)(uintptr_t)src, owner);
-    uint64_t* d = reinterpret_cast<uint64_t*>((uintptr_t)__shfl((unsigned long long)(uintptr_t)dst, owner));
+    gblocks d = reinterpret_cast<gblocks>((uintptr_t)__shfl((unsigned long long)(uintptr_t)dst, owner));
     const uint32_t sh = (uint32_t)(sa & 7u) * 8u;
-    const uint64_t* sp = reinterpret_cast<const uint64_t*>(sa & ~(uintptr_t)7);
+    gwords sp = reinterpret_cast<gwords>(sa & ~(uintptr_t)7);
     KTJ_NOUNROLL
     for (uint32_t k = rank; k < n; k += n_active) {
-      uint64_t v = sp[k];
-      if (sh) v = (v >> sh) | (sp[k + 1] << (64u - sh));
+      const uint64_t w0 = sp[2u * k], w1 = sp[2u * k + 1u];
+      v2u64 v;
+      v.x = w0; v.y = w1;
+      if (sh) {
+        const uint64_t w2 = sp[2u * k + 2u];
+        v.x = (w0 >> sh) | (w1 << (64u - sh));
+        v.y = (w1 >> sh) | (w2 << (64u - sh));
+      }
       d[k] = v;
     }
   }
