@@ -608,7 +608,13 @@ struct BlockWriter {
     if (len == 0) return;
     const uintptr_t sa = (uintptr_t)src;
     const uint32_t sh = (uint32_t)(sa & 7u) * 8u;
-    const uint64_t* sp = reinterpret_cast<const uint64_t*>(sa & ~(uintptr_t)7);
+#if defined(__HIP_DEVICE_COMPILE__)
+    /* every string lives in a dictionary blob in device memory: global loads, not flat ones */
+    typedef const __attribute__((address_space(1))) uint64_t* words;
+#else
+    typedef const uint64_t* words;
+#endif
+    words sp = reinterpret_cast<words>(sa & ~(uintptr_t)7);
     uint64_t cur = sp[0];
     const uint64_t full = len >> 3;
     uint64_t k = 0;

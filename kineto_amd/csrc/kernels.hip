@@ -1423,7 +1423,10 @@ k_radix_scatter(const uint64_t* keys_in, const uint32_t* vals_in, uint64_t* keys
   const uint64_t lt = lanemask_lt();
   const uint64_t tile_base = (uint64_t)blockIdx.x * RADIX_TILE;
   const uint64_t chunk = tile_base + (uint64_t)w * RADIX_WAVE_KEYS;
-  volatile uint32_t* my_run = wave_run[w];
+  /* my_run: this wavefront's running counts; accessed as LDS (a plain pointer to the row would
+   * turn into flat accesses), re-read every round because other lanes of the wavefront update it */
+  typedef volatile __attribute__((address_space(3))) uint32_t* lds_counts;
+  lds_counts my_run = (lds_counts)&wave_run[w][0];
   uint64_t key[RADIX_ITEMS];
   uint32_t val[RADIX_ITEMS], rank[RADIX_ITEMS];
 #pragma unroll
@@ -1603,7 +1606,10 @@ k_sortp_scatter(const uint64_t* in, uint64_t* words_out, uint32_t* perm_out, uin
   const uint64_t lt = lanemask_lt();
   const uint64_t tile_base = (uint64_t)blockIdx.x * P::TILE;
   const uint64_t chunk = tile_base + (uint64_t)w * P::WAVE_KEYS;
-  volatile uint32_t* my_run = wave_run[w];
+  /* my_run: this wavefront's running counts; accessed as LDS (a plain pointer to the row would
+   * turn into flat accesses), re-read every round because other lanes of the wavefront update it */
+  typedef volatile __attribute__((address_space(3))) uint32_t* lds_counts;
+  lds_counts my_run = (lds_counts)&wave_run[w][0];
   uint64_t word[P::ITEMS];
   uint32_t rank[P::ITEMS];
   uint16_t dig[P::ITEMS];
