@@ -113,6 +113,23 @@ template <class T> inline void malloc_args(const T& a, ktj_runtime_rec* r) {
   X(hipMemcpyPeerAsync) X(hipMemcpyToArray) X(hipMemcpyToSymbol) X(hipMemcpyToSymbolAsync)         \
   X(hipMemcpyWithStream)
 #define KTJ_SDK_MALLOC_APIS(X) X(hipMalloc) X(hipFree)
+/* RuntimeActivity<T>::flowStart (libkineto/src/RocprofActivity_inl.h:185-200) */
+#define KTJ_SDK_FLOW_START_APIS(X)                                                                 \
+  X(hipLaunchKernel) X(hipExtLaunchKernel) X(hipLaunchCooperativeKernel) X(hipHccModuleLaunchKernel) \
+  X(hipModuleLaunchKernel) X(hipExtModuleLaunchKernel) X(hipMalloc) X(hipFree) X(hipMemcpy)        \
+  X(hipMemcpyAsync) X(hipMemcpyWithStream) X(hipGraphLaunch)
+
+/* whether a runtime row of this operation starts a flow to its device rows: what a caller puts into
+ * ktj_set_api_table's flow_start_cids for a trace of rocprofiler-sdk HIP runtime API records */
+inline bool is_flow_start(uint32_t operation) {
+  switch (operation) {
+#define X(op) case ROCPROFILER_HIP_RUNTIME_API_ID_##op:
+    KTJ_SDK_FLOW_START_APIS(X)
+#undef X
+      return true;
+    default: return false;
+  }
+}
 
 /* Fills *out (zeroed first) from one HIP runtime API call: operation id, the SDK's internal
  * correlation id, the call's arguments, its begin/end on the caller's clock and the calling

@@ -36,8 +36,16 @@
  *   - GPU user-annotation spans: the expectations of test/RocmActivityProfilerTest.cpp:770-833 and
  *       the sequential Python statement of tests/test_join_bruteforce.py; the spans' relative order
  *       is the iteration order of the profiler's own maps, taken from the C++ library (map_order.cpp).
- *   - rocprofiler-sdk buffer records -> device rows (sdk_rows.c): PARITY UNPINNED by the reference
- *       (its buffer callback needs a live profiling session); hand-written expectations only.
+ *   - rocprofiler-sdk buffer records -> device rows (sdk_rows.c): against the reference's own
+ *       RocprofLogger::buffer_callback, run by oracle/_ref/sdk_ref_driver on records built in
+ *       memory (tests/test_sdk_ingest.py).
+ *   - the ROCm wrapper layer (what runtime and device rows report as activities: names, the args'
+ *       keys, order and values, the hand-over of grid, block and size from runtime rows to device
+ *       rows, device timestamps, flow starts): against the reference's own RuntimeActivity<T> and
+ *       GpuActivity classes, run by the same driver on packed rows (tests/test_rocm_wrappers.py).
+ *       Memset rows are CUDA-shaped (CuptiActivity.h:682-713); those wrappers need CUPTI's headers
+ *       and cannot be built here: PARITY UNPINNED for the args order of that one row kind, which
+ *       is read from the source.
  */
 #define _GNU_SOURCE
 #include "ktj_oracle.h"

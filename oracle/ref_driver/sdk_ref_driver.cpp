@@ -12,7 +12,7 @@
  * rocprofiler_configure, which a process that initialises HIP would hand to the SDK.
  *
  * stdin (binary, little endian):
- *   u32 mode                       1 = buffer records, 2 = HIP runtime API records
+ *   u32 mode                       1 = buffer records, 2 = HIP runtime API records, 3 = activity wrappers
  * mode 1:
  *   u64 n_rows, ktj_device_rec rows[n_rows], u64 agent_base, u64 kernel_base, u32 unknown_name_id,
  *   u32 noise, u64 n_agents, {u64 handle, i64 device}[n_agents], u64 n_kernels,
@@ -23,11 +23,20 @@
  *   Each record goes through api_callback twice (enter, exit).  Pointer-typed arguments should point
  *   into [KTJ_ARG_ARENA, KTJ_ARG_ARENA + 16 MiB): the driver maps zero pages there, because the SDK's
  *   argument iterator follows pointers when it renders them.
+ * mode 3:
+ *   u64 n_runtime, ktj_runtime_rec rows[n_runtime], u64 n_device, ktj_device_rec rows[n_device],
+ *   u64 n_names, {u32 length, bytes}[n_names]      (the device rows' name_id indexes these)
+ *   The rows become rocprofRow / rocprofKernelRow / rocprofCopyRow / rocprofMallocRow and rocprofAsyncRow
+ *   objects and are wrapped in the reference's RuntimeActivity<T> and GpuActivity
+ *   (libkineto/src/RocprofActivity.h:37-162, RocprofActivity_inl.h), runtime rows first, in the order
+ *   given: what each wrapper reports through ITraceActivity (and the args text of metadataJson(),
+ *   which also passes grid, block and size from a runtime row to the device rows of its id) is printed.
  * stdout: one text line per row the logger holds afterwards; in mode 2 the row's line is followed by
  * an "args" line with the SDK's own rendering of every argument (name=text), which is what the
  * reference keeps of dst, src and ptr.
  */
 #include "RocprofLogger.cpp"  // NOLINT: the reference's translation unit, found through -I$(REF)/libkineto/src
+#include "RocprofActivity.h"  // NOLINT: the reference's activity wrappers (header-only)
 
 #include <sys/mman.h>
 
@@ -172,6 +181,72 @@ int run_api_records() {
   return 0;
 }
 
+template <class A> void print_wrapper(const char* what, uint64_t index, const A& a) {
+  printf("%s idx=%" PRIu64 " corr=%" PRId64 " type=%d dev=%" PRId64 " res=%" PRId64 " ts=%" PRId64 " dur=%" PRId64
+         " flowstart=%d flowid=%" PRId64 " flowtype=%d name=%s json=%s\n",
+         what, index, a.correlationId(), (int)a.type(), a.deviceId(), a.resourceId(), a.timestamp(), a.duration(),
+         a.flowStart() ? 1 : 0, a.flowId(), a.flowType(), a.name().c_str(), a.metadataJson().c_str());
+}
+
+int run_wrappers() {
+  const uint64_t nr = rd<uint64_t>();
+  std::vector<ktj_runtime_rec> rt(nr);
+  if (nr && fread(rt.data(), sizeof(ktj_runtime_rec), nr, stdin) != nr) return 2;
+  const uint64_t nd = rd<uint64_t>();
+  std::vector<ktj_device_rec> dev(nd);
+  if (nd && fread(dev.data(), sizeof(ktj_device_rec), nd, stdin) != nd) return 2;
+  const uint64_t nn = rd<uint64_t>();
+  std::vector<std::string> names(nn);
+  for (auto& n : names) {
+    n.resize(rd<uint32_t>());
+    if (!n.empty() && fread(&n[0], 1, n.size(), stdin) != n.size()) return 2;
+  }
+  /* the operation names, as the reference's tool initialisation takes them from the SDK (RocprofLogger.cpp:346-347) */
+  getGlobalContext().name_info = rocprofiler::sdk::get_callback_tracing_names();
+  getGlobalContext().buff_name_info = rocprofiler::sdk::get_buffer_tracing_names();
+  const uint32_t dom = ROCPROFILER_CALLBACK_TRACING_HIP_RUNTIME_API;
+  for (uint64_t i = 0; i < nr; ++i) {
+    const ktj_runtime_rec& r = rt[i];
+    switch (r.kind) {
+      case KTJ_RT_KERNEL: {
+        rocprofKernelRow row(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end, nullptr, nullptr, r.u.kernel.grid[0], r.u.kernel.grid[1],
+                             r.u.kernel.grid[2], r.u.kernel.workgroup[0], r.u.kernel.workgroup[1], r.u.kernel.workgroup[2],
+                             r.u.kernel.group_segment_size, reinterpret_cast<hipStream_t>(r.u.kernel.stream));
+        print_wrapper("runtime", i, RuntimeActivity<rocprofKernelRow>(&row, nullptr));
+        break;
+      }
+      case KTJ_RT_COPY: {
+        rocprofCopyRow row(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end, reinterpret_cast<const void*>(r.u.copy.src),
+                           reinterpret_cast<const void*>(r.u.copy.dst), r.u.copy.size, static_cast<hipMemcpyKind>(r.u.copy.copy_kind),
+                           reinterpret_cast<hipStream_t>(r.u.copy.stream));
+        print_wrapper("runtime", i, RuntimeActivity<rocprofCopyRow>(&row, nullptr));
+        break;
+      }
+      case KTJ_RT_MALLOC: {
+        rocprofMallocRow row(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end, reinterpret_cast<const void*>(r.u.malloc_.ptr),
+                             r.u.malloc_.size);
+        print_wrapper("runtime", i, RuntimeActivity<rocprofMallocRow>(&row, nullptr));
+        break;
+      }
+      default: {
+        rocprofRow row(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end);
+        print_wrapper("runtime", i, RuntimeActivity<rocprofRow>(&row, nullptr));
+        break;
+      }
+    }
+  }
+  for (uint64_t i = 0; i < nd; ++i) {
+    const ktj_device_rec& d = dev[i];
+    const uint32_t kind = d.domain == KTJ_DOM_MEMORY_COPY ? (uint32_t)ROCPROFILER_BUFFER_TRACING_MEMORY_COPY
+                                                          : (uint32_t)ROCPROFILER_BUFFER_TRACING_KERNEL_DISPATCH;
+    rocprofAsyncRow row(d.id, kind, kind, d.op, d.device, d.queue, d.begin, d.end,
+                        d.name_id < names.size() ? names[d.name_id] : std::string());
+    row.stream = d.stream;
+    print_wrapper("device", i, GpuActivity(&row, nullptr));
+  }
+  return 0;
+}
+
 }  // namespace
 
 int main() {
@@ -179,6 +254,7 @@ int main() {
   int rc = 2;
   if (mode == 1) rc = run_buffer_records();
   else if (mode == 2) rc = run_api_records();
+  else if (mode == 3) rc = run_wrappers();
   fflush(stdout);
   _exit(rc); /* no destructors: the logger's would stop a tracing context that was never created */
 }

@@ -121,5 +121,13 @@ void* ktjsim_sdk_api_record_create(uint32_t kind, uint32_t operation, uint64_t c
 }
 void ktjsim_sdk_api_record_free(void* p) { delete static_cast<ApiRecordHolder*>(p); }
 uint32_t ktjsim_sdk_api_kind_hip_runtime(void) { return ROCPROFILER_CALLBACK_TRACING_HIP_RUNTIME_API; }
+int ktjsim_sdk_api_is_flow_start(uint32_t operation) { return ktj::sdk_api::is_flow_start(operation) ? 1 : 0; }
+/* the SDK's number of a few operations the tests name */
+int64_t ktjsim_sdk_api_op_id(const char* name) {
+#define X(op) if (std::strcmp(name, #op) == 0) return ROCPROFILER_HIP_RUNTIME_API_ID_##op;
+  KTJ_SDK_FLOW_START_APIS(X) X(hipMemcpyDtoD) X(hipDeviceSynchronize) X(hipGetDevice)
+#undef X
+  return -1;
+}
 
 }  // extern "C"

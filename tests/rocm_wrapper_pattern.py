@@ -1,0 +1,148 @@
+"""Test-only: a fixed set of ROCm runtime and device rows, what the reference's own activity wrappers
+(RuntimeActivity<T>, GpuActivity; libkineto/src/RocprofActivity.h, RocprofActivity_inl.h) report for
+them through oracle/_ref/sdk_ref_driver, and the same rows as a stream for the checker and the
+engine."""
+import os
+import re
+import struct
+import subprocess
+
+from kineto_amd import abi
+import sdk_api_pattern as sp
+from stream_builder import B, StreamBuilder
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "rocm_wrapper_rows.txt")
+WIDE = 1 << 32   # two ids this far apart are one key of the reference's int-keyed hand-over maps
+
+
+def op(name):
+    lib = sp.sim()
+    lib.ktjsim_sdk_api_op_id.restype = abi.C.c_int64
+    lib.ktjsim_sdk_api_op_id.argtypes = [abi.C.c_char_p]
+    v = lib.ktjsim_sdk_api_op_id(name.encode())
+    assert v >= 0, name
+    return v
+
+
+def rows():
+    """(runtime rows, device rows, device names): every row kind, every copy direction, ids shared by
+    several runtime rows (the last one hands over), a copy and a launch with one id (size wins over
+    grid), ids that coincide after narrowing to int, device rows without a stream or without a
+    runtime row, zero-length copies (no bandwidth).  No runtime row carries a stream: the stream
+    back-fill (RocmStreamQueue.h), which precedes the wrappers in the profiler and renumbers the
+    streams of the device rows, then leaves the device rows' streams as they are."""
+    launch, memcpy_async, malloc, free = op("hipLaunchKernel"), op("hipMemcpyAsync"), op("hipMalloc"), op("hipFree")
+    sync, graph = op("hipDeviceSynchronize"), op("hipGraphLaunch")
+    t = B + 1000
+    rt = [
+        # (id, begin, end, cid, pid, tid, kind, fields)
+        (101, t + 10, t + 20, launch, 4242, 77, 1, dict(grid=(7, 2, 1), workgroup=(256, 1, 1), lds=4096, stream=0)),
+        (102, t + 30, t + 45, memcpy_async, 4242, 77, 2, dict(src=0x7000a000, dst=0x7000b000, size=65536, copy_kind=1, stream=0)),
+        (103, t + 50, t + 55, malloc, 4242, 78, 3, dict(ptr=0x7000c000, size=1 << 20)),
+        (104, t + 60, t + 61, free, 4242, 78, 3, dict(ptr=0x7000c000, size=0)),
+        (105, t + 70, t + 90, sync, 4242, 77, 0, {}),
+        (106, t + 100, t + 110, launch, 4242, 77, 1, dict(grid=(1, 1, 1), workgroup=(64, 1, 1), lds=0, stream=0)),
+        (106, t + 111, t + 120, launch, 4242, 79, 1, dict(grid=(9, 9, 9), workgroup=(32, 2, 2), lds=128, stream=0)),
+        (107, t + 130, t + 140, launch, 4242, 77, 1, dict(grid=(3, 1, 1), workgroup=(128, 1, 1), lds=0, stream=0)),
+        (107, t + 141, t + 150, memcpy_async, 4242, 77, 2, dict(src=0x10, dst=0x20, size=4096, copy_kind=3, stream=0)),
+        (108 + WIDE, t + 160, t + 170, launch, 4242, 77, 1, dict(grid=(5, 5, 1), workgroup=(16, 16, 1), lds=0, stream=0)),
+        (109, t + 180, t + 190, graph, 4242, 77, 0, {}),
+        (110, t + 200, t + 210, memcpy_async, 4242, 80, 2, dict(src=0, dst=0xffffffffffff, size=0, copy_kind=4, stream=0)),
+    ]
+    names = ["void gemm<float>(float*, int)", "vector_add", ""]
+    dv = [
+        # (id, begin, end, domain, op, device, name_id, queue, stream)
+        (101, t + 500, t + 700, 0, 0, 0, 0, 11, 3),          # kernel with its launch: grid and block
+        (102, t + 710, t + 910, 1, 2, 1, 2, 12, 3),          # HtoD with its copy: bytes and bandwidth
+        (106, t + 920, t + 930, 0, 0, 0, 1, 11, 0),          # two launches share the id; stream 0: the queue is the row
+        (107, t + 940, t + 960, 1, 4, 0, 2, 12, 5),          # a launch and a copy share the id: bytes, no grid
+        (108, t + 970, t + 980, 0, 0, 2, 1, 13, 7),          # the launch's id differs by 2^32: same int key
+        (555, t + 990, t + 995, 0, 0, 0, 0, 11, 3),          # no runtime row
+        (110, t + 1000, t + 1000, 1, 3, 0, 2, 12, 3),        # begin == end: no bandwidth
+        (103, t + 1010, t + 1020, 1, 1, 0, 2, 12, 3),        # HtoH after a malloc of the same id: bytes handed over
+        (556, t + 1030, t + 1040, 1, 9, 0, 2, 12, 3),        # unknown copy direction
+    ]
+    return rt, dv, names
+
+
+def _runtime_rec(r):
+    rid, begin, end, cid, pid, tid, kind, f = r
+    x = abi.RuntimeRec()
+    x.id, x.begin, x.end, x.cid, x.pid, x.tid, x.kind = rid, begin, end, cid, pid, tid, kind
+    if kind == 1:
+        for i in range(3):
+            x.u.kernel.grid[i] = f["grid"][i]
+            x.u.kernel.workgroup[i] = f["workgroup"][i]
+        x.u.kernel.group_segment_size, x.u.kernel.stream, x.u.kernel.kernel_name_id = f["lds"], f["stream"], abi.KTJ_NONE
+    elif kind == 2:
+        x.u.copy.src, x.u.copy.dst, x.u.copy.size = f["src"], f["dst"], f["size"]
+        x.u.copy.copy_kind, x.u.copy.stream = f["copy_kind"], f["stream"]
+    elif kind == 3:
+        x.u.malloc_.ptr, x.u.malloc_.size = f["ptr"], f["size"]
+    return x
+
+
+def _device_rec(d):
+    rid, begin, end, domain, opn, device, name_id, queue, stream = d
+    x = abi.DeviceRec()
+    x.id, x.begin, x.end, x.domain, x.op, x.device, x.name_id, x.queue, x.stream = rid, begin, end, domain, opn, device, name_id, queue, stream
+    return x
+
+
+def driver_lines():
+    rt, dv, names = rows()
+    req = struct.pack("<IQ", 3, len(rt)) + b"".join(bytes(_runtime_rec(r)) for r in rt)
+    req += struct.pack("<Q", len(dv)) + b"".join(bytes(_device_rec(d)) for d in dv)
+    req += struct.pack("<Q", len(names)) + b"".join(struct.pack("<I", len(n)) + n.encode() for n in names)
+    out = subprocess.run([sp.SDK_REF_DRIVER], input=req, stdout=subprocess.PIPE, check=True, timeout=120).stdout.decode("latin1")
+    return [line for line in out.split("\n") if line]
+
+
+def reference_lines():
+    if os.path.exists(sp.SDK_REF_DRIVER):
+        return driver_lines()
+    return [line for line in open(GOLDEN).read().split("\n") if line]
+
+
+_LINE = re.compile(r"^(runtime|device) idx=(\d+) corr=(-?\d+) type=(\d+) dev=(-?\d+) res=(-?\d+) ts=(-?\d+) dur=(-?\d+) "
+                   r"flowstart=(\d) flowid=(-?\d+) flowtype=(\d+) name=(.*?) json=(.*)$")
+
+
+def parse(line):
+    m = _LINE.match(line)
+    assert m, line
+    what, idx, corr, typ, dev, res, ts, dur, fs, fid, ft, name, js = m.groups()
+    return dict(what=what, idx=int(idx), corr=int(corr), type=int(typ), dev=int(dev), res=int(res), ts=int(ts), dur=int(dur),
+                flowstart=int(fs), flowid=int(fid), flowtype=int(ft), name=name, json=js)
+
+
+def stream(ref):
+    """The same rows as a ktj_stream (no clock conversion, wide window).  The API names and the
+    flow-start set are what a caller of the engine provides: the names come from the reference's
+    lines, the flow-start operations from kineto_amd/csrc/sdk_api_rows.h."""
+    rt, dv, names = rows()
+    b = StreamBuilder(host_name="wrap")
+    n_cids = max(r[3] for r in rt) + 1
+    api_names = [None] * n_cids
+    for r, line in zip(rt, ref):
+        api_names[r[3]] = parse(line)["name"]
+    flow = [c for c in range(n_cids) if sp.sim().ktjsim_sdk_api_is_flow_start(c)]
+    b.api(api_names, flow_start=flow, malloc_cid=op("hipMalloc"))
+    for rid, begin, end, cid, pid, tid, kind, f in rt:
+        kw = dict(f)
+        if kind == 1:
+            kw["kernel_name"] = None
+        b.add_runtime(rid, begin, end, cid, pid, tid, kind=kind, **kw)
+    for rid, begin, end, domain, opn, device, name_id, queue, stream_ in dv:
+        b.add_device(rid, begin, end, domain=domain, op=opn, device=device, name=names[name_id] if names[name_id] else None,
+                     queue=queue, stream=stream_)
+    return b
+
+
+_EVENT = re.compile(r'"ph": "X",\n    "cat": "([^"]*)",\n    "name": "(.*)",\n    "pid": (-?\d+),\n    "tid": (-?\d+),\n'
+                    r'    "ts": ([0-9.]+),\n    "dur": ([0-9.]+)\n    (?:,\n    "args": \{\n      (.*)\n    \}\n  \},|\n  \},)')
+
+
+def events(document):
+    """(cat, name, pid, tid, ts, dur, args text or None) of every complete event, in document order."""
+    return [m.groups() for m in _EVENT.finditer(document.decode("latin1"))]

@@ -1,0 +1,83 @@
+"""The ROCm wrapper layer (RuntimeActivity<T>, GpuActivity: libkineto/src/RocprofActivity.h:37-162,
+RocprofActivity_inl.h:98-299) pinned against the reference's own wrapper code: what those classes
+report for a fixed set of rows (oracle/_ref/sdk_ref_driver, mode 3; kept in
+tests/golden/rocm_wrapper_rows.txt for machines without the reference) against the checker's
+activities and document, and, on the GPU, the engine's document."""
+import os
+
+import pytest
+
+import oracle_glue as og
+import rocm_wrapper_pattern as rw
+import sdk_api_pattern as sp
+
+HAVE_DRIVER = os.path.exists(sp.SDK_REF_DRIVER)
+
+
+def _flow_start_ops(lines):
+    last = [line for line in lines if line.startswith("flowstart_ops=")]
+    assert len(last) == 1
+    return [int(x) for x in last[0].split("=", 1)[1].split()]
+
+
+def _all_lines():
+    if HAVE_DRIVER:
+        import golden.make_rocm_wrapper_golden as mk
+        return mk.lines()
+    return [line for line in open(rw.GOLDEN).read().split("\n") if line]
+
+
+def test_checker_matches_the_reference_wrappers():
+    lines = _all_lines()
+    ref = [rw.parse(line) for line in lines if not line.startswith("flowstart_ops=")]
+    rt, dv, names = rw.rows()
+    assert len(ref) == len(rt) + len(dv)
+    sp_ = rw.stream([line for line in lines if not line.startswith("flowstart_ops=")]).build()
+    ora = og.OracleRun(sp_)
+    acts, n = ora.activities()
+    order = ora.order()
+    doc = ora.output()
+    assert n == len(ref), "every row is inside the window"
+    by_arrival = {int(acts[i].arrival): i for i in range(n)}
+    ev = rw.events(doc)
+    assert len(ev) == n
+    for k, r in enumerate(ref):
+        a = acts[by_arrival[k]]
+        what = f"{r['what']} row {r['idx']}"
+        assert (a.ts, a.dur, a.device, a.resource) == (r["ts"], r["dur"], r["dev"], r["res"]), what
+        assert a.type == r["type"] and a.flow_id == r["flowid"] and a.flow_type == r["flowtype"], what
+        assert bool(a.flow_start) == bool(r["flowstart"]), what
+    # the document: events come in canonical order; position p holds activity order[p]
+    for p, e in enumerate(ev):
+        a = acts[order[p]]
+        r = ref[int(a.arrival)]
+        cat, name, pid, tid, ts, dur, args = e
+        what = f"{r['what']} row {r['idx']}"
+        assert name == r["name"], what
+        assert args == r["json"], what
+        assert int(pid) == r["dev"] and int(tid) == r["res"], what
+    ora.close()
+
+
+def test_flow_start_operations_are_the_references():
+    """kineto_amd/csrc/sdk_api_rows.h:is_flow_start against RuntimeActivity<T>::flowStart for every HIP
+    runtime operation of the SDK."""
+    want = _flow_start_ops(_all_lines())
+    got = [op for op in range(sp.n_ops()) if sp.sim().ktjsim_sdk_api_is_flow_start(op)]
+    assert got == want and len(got) == 12
+
+
+@pytest.mark.skipif(not HAVE_DRIVER, reason="oracle/_ref/sdk_ref_driver is built only where the reference's sources are")
+def test_wrapper_golden_file_is_what_the_reference_produces():
+    import golden.make_rocm_wrapper_golden as mk
+    assert mk.lines() == [line for line in open(rw.GOLDEN).read().split("\n") if line]
+
+
+@pytest.mark.gpu
+def test_engine_matches_the_reference_wrappers():
+    import test_gpu_parity as tp
+    lines = [line for line in _all_lines() if not line.startswith("flowstart_ops=")]
+    got = tp._engine_vs_oracle(rw.stream(lines).build())
+    ev = rw.events(got)
+    ref = [rw.parse(line) for line in lines]
+    assert sorted(e[6] or "" for e in ev) == sorted(r["json"] for r in ref)
