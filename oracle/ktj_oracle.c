@@ -42,7 +42,9 @@
  *   - the ROCm wrapper layer (what runtime and device rows report as activities: names, the args'
  *       keys, order and values, the hand-over of grid, block and size from runtime rows to device
  *       rows, device timestamps, flow starts): against the reference's own RuntimeActivity<T> and
- *       GpuActivity classes, run by the same driver on packed rows (tests/test_rocm_wrappers.py).
+ *       GpuActivity classes, run by the same driver on packed rows (tests/test_rocm_wrappers.py);
+ *       the stream back-fill against the reference's own detail::backfillAsyncStreams
+ *       (RocmStreamQueue.h:42-136) on seeded rows, same driver, same test file.
  *       Memset rows are CUDA-shaped (CuptiActivity.h:682-713); those wrappers need CUPTI's headers
  *       and cannot be built here: PARITY UNPINNED for the args order of that one row kind, which
  *       is read from the source.

@@ -12,7 +12,8 @@
  * rocprofiler_configure, which a process that initialises HIP would hand to the SDK.
  *
  * stdin (binary, little endian):
- *   u32 mode                       1 = buffer records, 2 = HIP runtime API records, 3 = activity wrappers
+ *   u32 mode                       1 = buffer records, 2 = HIP runtime API records, 3 = activity wrappers,
+ *                                  4 = stream back-fill, then activity wrappers
  * mode 1:
  *   u64 n_rows, ktj_device_rec rows[n_rows], u64 agent_base, u64 kernel_base, u32 unknown_name_id,
  *   u32 noise, u64 n_agents, {u64 handle, i64 device}[n_agents], u64 n_kernels,
@@ -31,12 +32,15 @@
  *   (libkineto/src/RocprofActivity.h:37-162, RocprofActivity_inl.h), runtime rows first, in the order
  *   given: what each wrapper reports through ITraceActivity (and the args text of metadataJson(),
  *   which also passes grid, block and size from a runtime row to the device rows of its id) is printed.
+ *   Mode 4 first runs the reference's detail::backfillAsyncStreams (RocmStreamQueue.h:42-136) over the
+ *   rows, as RocprofActivityApi::processActivities does (RocprofActivityApi.cpp:134-142).
  * stdout: one text line per row the logger holds afterwards; in mode 2 the row's line is followed by
  * an "args" line with the SDK's own rendering of every argument (name=text), which is what the
  * reference keeps of dst, src and ptr.
  */
 #include "RocprofLogger.cpp"  // NOLINT: the reference's translation unit, found through -I$(REF)/libkineto/src
 #include "RocprofActivity.h"  // NOLINT: the reference's activity wrappers (header-only)
+#include "RocmStreamQueue.h"  // NOLINT: the reference's stream back-fill (header-only)
 
 #include <sys/mman.h>
 
@@ -188,7 +192,7 @@ template <class A> void print_wrapper(const char* what, uint64_t index, const A&
          a.flowStart() ? 1 : 0, a.flowId(), a.flowType(), a.name().c_str(), a.metadataJson().c_str());
 }
 
-int run_wrappers() {
+int run_wrappers(bool backfill) {
   const uint64_t nr = rd<uint64_t>();
   std::vector<ktj_runtime_rec> rt(nr);
   if (nr && fread(rt.data(), sizeof(ktj_runtime_rec), nr, stdin) != nr) return 2;
@@ -205,44 +209,50 @@ int run_wrappers() {
   getGlobalContext().name_info = rocprofiler::sdk::get_callback_tracing_names();
   getGlobalContext().buff_name_info = rocprofiler::sdk::get_buffer_tracing_names();
   const uint32_t dom = ROCPROFILER_CALLBACK_TRACING_HIP_RUNTIME_API;
+  std::vector<rocprofBase*> rows; /* as RocprofLogger holds them: runtime rows, then device rows */
   for (uint64_t i = 0; i < nr; ++i) {
     const ktj_runtime_rec& r = rt[i];
     switch (r.kind) {
-      case KTJ_RT_KERNEL: {
-        rocprofKernelRow row(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end, nullptr, nullptr, r.u.kernel.grid[0], r.u.kernel.grid[1],
-                             r.u.kernel.grid[2], r.u.kernel.workgroup[0], r.u.kernel.workgroup[1], r.u.kernel.workgroup[2],
-                             r.u.kernel.group_segment_size, reinterpret_cast<hipStream_t>(r.u.kernel.stream));
-        print_wrapper("runtime", i, RuntimeActivity<rocprofKernelRow>(&row, nullptr));
+      case KTJ_RT_KERNEL:
+        rows.push_back(new rocprofKernelRow(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end, nullptr, nullptr, r.u.kernel.grid[0],
+                                            r.u.kernel.grid[1], r.u.kernel.grid[2], r.u.kernel.workgroup[0], r.u.kernel.workgroup[1],
+                                            r.u.kernel.workgroup[2], r.u.kernel.group_segment_size,
+                                            reinterpret_cast<hipStream_t>(r.u.kernel.stream)));
         break;
-      }
-      case KTJ_RT_COPY: {
-        rocprofCopyRow row(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end, reinterpret_cast<const void*>(r.u.copy.src),
-                           reinterpret_cast<const void*>(r.u.copy.dst), r.u.copy.size, static_cast<hipMemcpyKind>(r.u.copy.copy_kind),
-                           reinterpret_cast<hipStream_t>(r.u.copy.stream));
-        print_wrapper("runtime", i, RuntimeActivity<rocprofCopyRow>(&row, nullptr));
+      case KTJ_RT_COPY:
+        rows.push_back(new rocprofCopyRow(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end, reinterpret_cast<const void*>(r.u.copy.src),
+                                          reinterpret_cast<const void*>(r.u.copy.dst), r.u.copy.size,
+                                          static_cast<hipMemcpyKind>(r.u.copy.copy_kind), reinterpret_cast<hipStream_t>(r.u.copy.stream)));
         break;
-      }
-      case KTJ_RT_MALLOC: {
-        rocprofMallocRow row(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end, reinterpret_cast<const void*>(r.u.malloc_.ptr),
-                             r.u.malloc_.size);
-        print_wrapper("runtime", i, RuntimeActivity<rocprofMallocRow>(&row, nullptr));
+      case KTJ_RT_MALLOC:
+        rows.push_back(new rocprofMallocRow(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end,
+                                            reinterpret_cast<const void*>(r.u.malloc_.ptr), r.u.malloc_.size));
         break;
-      }
-      default: {
-        rocprofRow row(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end);
-        print_wrapper("runtime", i, RuntimeActivity<rocprofRow>(&row, nullptr));
-        break;
-      }
+      default: rows.push_back(new rocprofRow(r.id, dom, r.cid, r.pid, r.tid, r.begin, r.end)); break;
     }
   }
   for (uint64_t i = 0; i < nd; ++i) {
     const ktj_device_rec& d = dev[i];
     const uint32_t kind = d.domain == KTJ_DOM_MEMORY_COPY ? (uint32_t)ROCPROFILER_BUFFER_TRACING_MEMORY_COPY
                                                           : (uint32_t)ROCPROFILER_BUFFER_TRACING_KERNEL_DISPATCH;
-    rocprofAsyncRow row(d.id, kind, kind, d.op, d.device, d.queue, d.begin, d.end,
-                        d.name_id < names.size() ? names[d.name_id] : std::string());
-    row.stream = d.stream;
-    print_wrapper("device", i, GpuActivity(&row, nullptr));
+    auto* row = new rocprofAsyncRow(d.id, kind, kind, d.op, d.device, d.queue, d.begin, d.end,
+                                    d.name_id < names.size() ? names[d.name_id] : std::string());
+    row->stream = d.stream;
+    rows.push_back(row);
+  }
+  if (backfill) /* RocprofActivityApi.cpp:134-142 with copies and kernels both logged */
+    KINETO_NAMESPACE::detail::backfillAsyncStreams(rows, [](const rocprofAsyncRow& a) {
+      return a.domain == ROCPROFILER_BUFFER_TRACING_MEMORY_COPY || a.domain == ROCPROFILER_BUFFER_TRACING_KERNEL_DISPATCH;
+    });
+  for (uint64_t i = 0; i < rows.size(); ++i) {
+    const rocprofBase* b = rows[i];
+    switch (b->type) {
+      case ROCTRACER_ACTIVITY_KERNEL: print_wrapper("runtime", i, RuntimeActivity<rocprofKernelRow>(static_cast<const rocprofKernelRow*>(b), nullptr)); break;
+      case ROCTRACER_ACTIVITY_COPY: print_wrapper("runtime", i, RuntimeActivity<rocprofCopyRow>(static_cast<const rocprofCopyRow*>(b), nullptr)); break;
+      case ROCTRACER_ACTIVITY_MALLOC: print_wrapper("runtime", i, RuntimeActivity<rocprofMallocRow>(static_cast<const rocprofMallocRow*>(b), nullptr)); break;
+      case ROCTRACER_ACTIVITY_ASYNC: print_wrapper("device", i - nr, GpuActivity(static_cast<const rocprofAsyncRow*>(b), nullptr)); break;
+      default: print_wrapper("runtime", i, RuntimeActivity<rocprofRow>(static_cast<const rocprofRow*>(b), nullptr)); break;
+    }
   }
   return 0;
 }
@@ -254,7 +264,7 @@ int main() {
   int rc = 2;
   if (mode == 1) rc = run_buffer_records();
   else if (mode == 2) rc = run_api_records();
-  else if (mode == 3) rc = run_wrappers();
+  else if (mode == 3 || mode == 4) rc = run_wrappers(mode == 4);
   fflush(stdout);
   _exit(rc); /* no destructors: the logger's would stop a tracing context that was never created */
 }

@@ -89,9 +89,44 @@ def _device_rec(d):
     return x
 
 
-def driver_lines():
-    rt, dv, names = rows()
-    req = struct.pack("<IQ", 3, len(rt)) + b"".join(bytes(_runtime_rec(r)) for r in rt)
+def random_rows(seed):
+    """Seeded rows for the stream back-fill (RocmStreamQueue.h:42-136): runtime rows with and without
+    a stream, ids shared between them, device rows with and without a stream on several devices and
+    queues (one queue used by two streams: ambiguous), device rows with neither stream nor queue."""
+    import random
+    rng = random.Random(seed)
+    launch, memcpy_async, malloc, sync = op("hipLaunchKernel"), op("hipMemcpyAsync"), op("hipMalloc"), op("hipDeviceSynchronize")
+    streams = [0, 0, 0x7f10, 0x7f20, 0x7f30, 0x7f40]
+    t = B + 5000
+    rt, dv = [], []
+    for i in range(80):
+        rid = rng.randrange(1, 60)
+        kind = rng.choice([0, 1, 1, 1, 2, 2, 3])
+        begin = t + 10 * i
+        if kind == 1:
+            f = dict(grid=(rng.randrange(1, 9), 1, 1), workgroup=(64, 1, 1), lds=0, stream=rng.choice(streams))
+            cid = launch
+        elif kind == 2:
+            f = dict(src=0x1000, dst=0x2000, size=rng.randrange(0, 1 << 20), copy_kind=rng.randrange(0, 5), stream=rng.choice(streams))
+            cid = memcpy_async
+        elif kind == 3:
+            f = dict(ptr=0x3000, size=rng.randrange(0, 1 << 16))
+            cid = malloc
+        else:
+            f, cid = {}, sync
+        rt.append((rid, begin, begin + rng.randrange(1, 9), cid, 4242, 70 + rng.randrange(3), kind, f))
+    for i in range(160):
+        rid = rng.randrange(1, 75)   # some ids have no runtime row
+        domain = rng.choice([0, 0, 1])
+        begin = t + 2000 + 10 * i
+        dv.append((rid, begin, begin + rng.randrange(0, 9), domain, rng.randrange(1, 5) if domain else 0, rng.randrange(3),
+                   rng.randrange(2), rng.choice([0, 11, 12, 13, 14, 15]), rng.choice([0, 0, 0, 0x7f10, 0x7f50])))
+    return rt, dv, ["kernel_a", "kernel_b"]
+
+
+def driver_lines(all_rows=None, mode=3):
+    rt, dv, names = all_rows or rows()
+    req = struct.pack("<IQ", mode, len(rt)) + b"".join(bytes(_runtime_rec(r)) for r in rt)
     req += struct.pack("<Q", len(dv)) + b"".join(bytes(_device_rec(d)) for d in dv)
     req += struct.pack("<Q", len(names)) + b"".join(struct.pack("<I", len(n)) + n.encode() for n in names)
     out = subprocess.run([sp.SDK_REF_DRIVER], input=req, stdout=subprocess.PIPE, check=True, timeout=120).stdout.decode("latin1")
@@ -116,11 +151,11 @@ def parse(line):
                 flowstart=int(fs), flowid=int(fid), flowtype=int(ft), name=name, json=js)
 
 
-def stream(ref):
+def stream(ref, all_rows=None):
     """The same rows as a ktj_stream (no clock conversion, wide window).  The API names and the
     flow-start set are what a caller of the engine provides: the names come from the reference's
     lines, the flow-start operations from kineto_amd/csrc/sdk_api_rows.h."""
-    rt, dv, names = rows()
+    rt, dv, names = all_rows or rows()
     b = StreamBuilder(host_name="wrap")
     n_cids = max(r[3] for r in rt) + 1
     api_names = [None] * n_cids

@@ -27,12 +27,11 @@ def _all_lines():
     return [line for line in open(rw.GOLDEN).read().split("\n") if line]
 
 
-def test_checker_matches_the_reference_wrappers():
-    lines = _all_lines()
-    ref = [rw.parse(line) for line in lines if not line.startswith("flowstart_ops=")]
-    rt, dv, names = rw.rows()
+def _compare_checker_with_reference(lines, all_rows):
+    ref = [rw.parse(line) for line in lines]
+    rt, dv, names = all_rows
     assert len(ref) == len(rt) + len(dv)
-    sp_ = rw.stream([line for line in lines if not line.startswith("flowstart_ops=")]).build()
+    sp_ = rw.stream(lines, all_rows).build()
     ora = og.OracleRun(sp_)
     acts, n = ora.activities()
     order = ora.order()
@@ -57,6 +56,20 @@ def test_checker_matches_the_reference_wrappers():
         assert args == r["json"], what
         assert int(pid) == r["dev"] and int(tid) == r["res"], what
     ora.close()
+
+
+def test_checker_matches_the_reference_wrappers():
+    lines = [line for line in _all_lines() if not line.startswith("flowstart_ops=")]
+    _compare_checker_with_reference(lines, rw.rows())
+
+
+@pytest.mark.skipif(not HAVE_DRIVER, reason="oracle/_ref/sdk_ref_driver is built only where the reference's sources are")
+@pytest.mark.parametrize("seed", range(12))
+def test_stream_backfill_matches_the_reference(seed):
+    """The reference's own detail::backfillAsyncStreams (RocmStreamQueue.h:42-136) over seeded rows,
+    then its wrappers: the device rows' resourceId and "stream" against the checker's."""
+    all_rows = rw.random_rows(seed)
+    _compare_checker_with_reference(rw.driver_lines(all_rows, mode=4), all_rows)
 
 
 def test_flow_start_operations_are_the_references():
