@@ -19,10 +19,12 @@
  *   - clock conversion: x86 `long double` arithmetic, the very expression of
  *       ApproximateClock.cpp:83-90; checked against exact rational arithmetic in the tests.
  *   - join (external correlation, stream back-fill, grid/block/bytes hand-over, window filter,
- *       timestamp-order counter): brute-force nested-loop re-implementation in the tests on small
- *       streams, and the expectations of test/RocmActivityProfilerTest.cpp:370-397, 486-503, 552-554.
- *       The reference's own join code (RocmActivityProfiler / RocprofActivityApi) needs a live
- *       rocprofiler-sdk context and is not part of oracle/_ref.
+ *       timestamp-order counter, GPU user-annotation spans): the reference's own
+ *       GenericActivityProfiler::processTraceInternal with the ROCm handlers and the real logger,
+ *       run by oracle/_ref/profiler_ref_driver on rows placed in memory; every event it writes and
+ *       its counters are compared on seeded cases (tests/test_rocm_wrappers.py).  Also a
+ *       brute-force nested-loop re-implementation in the tests on small streams, and the
+ *       expectations of test/RocmActivityProfilerTest.cpp:370-397, 486-503, 552-554.
  *   - canonical order: stable merge sort here; std::stable_sort on tuples inside oracle/_ref.
  *   - instant events and the Stream Sync row remap: byte-compared with the real logger on a
  *       hand-made case (tests/kat_cases.py: case_instant_and_stream_sync).

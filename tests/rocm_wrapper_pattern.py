@@ -181,3 +181,139 @@ _EVENT = re.compile(r'"ph": "X",\n    "cat": "([^"]*)",\n    "name": "(.*)",\n  
 def events(document):
     """(cat, name, pid, tid, ts, dur, args text or None) of every complete event, in document order."""
     return [m.groups() for m in _EVENT.finditer(document.decode("latin1"))]
+
+
+# ---- the reference's whole post-processing loop (oracle/_ref/profiler_ref_driver) ----
+PROFILER_REF_DRIVER = os.path.join(sp.ROOT, "oracle", "_ref", "profiler_ref_driver")
+
+
+MARKER_ID = 99999   # the first device row: inside the window, its id used by no other row
+
+
+def profiler_case(seed):
+    """CPU ops, external-correlation pairs of both domains, runtime rows and device rows for the
+    reference's processTraceInternal: ids linked to existing and to missing CPU ops, rows before,
+    across and after the capture window, device rows that start before their launch, ids shared by
+    several rows, ids beyond 32 bits.  Times are milliseconds apart and rows keep 5 ms from the
+    window's edges (or lie 5 ms and more outside): the reference shifts device rows by a clock
+    offset it samples while it runs, known only to within a millisecond beforehand."""
+    import random
+    rng = random.Random(1000 + seed)
+    ms = 1_000_000
+    t0 = B + 100 * ms
+    window = (t0, t0 + 1000 * ms)
+    launch, memcpy_async, malloc, sync = op("hipLaunchKernel"), op("hipMemcpyAsync"), op("hipMalloc"), op("hipDeviceSynchronize")
+    names = ["aten::mm", "aten::add", "annotation_a", "gemm_kernel", "copy_kernel", ""]
+
+    def when():   # a start time: mostly inside the window, sometimes well before or after it
+        r = rng.random()
+        if r < 0.08:
+            return t0 - rng.randrange(5 * ms, 50 * ms)
+        if r < 0.16:
+            return t0 + 1000 * ms + rng.randrange(5 * ms, 50 * ms)
+        return t0 + rng.randrange(5 * ms, 900 * ms)
+
+    def length(start):   # rows that start inside end inside, or stick out by 5 ms and more
+        if rng.random() < 0.06:
+            return (t0 + 1000 * ms - start) + rng.randrange(5 * ms, 20 * ms) if start < t0 + 1000 * ms else 3 * ms
+        return rng.randrange(0, 40 * ms)
+
+    cpu_ops, ext, user, rt, dv = [], [], [], [], []
+    for i in range(12):
+        start = t0 + 6 * ms + 70 * ms * i
+        cpu_ops.append(dict(name_id=rng.randrange(2), start=start, end=start + rng.randrange(1 * ms, 60 * ms), id=10 + i, device=4242,
+                            resource=77 + (i % 2), type=0))
+    for i in range(3):
+        start = t0 + 8 * ms + 300 * ms * i
+        cpu_ops.append(dict(name_id=2, start=start, end=start + 250 * ms, id=40 + i, device=4242, resource=77, type=1))  # user annotations
+    for i in range(70):
+        rid = rng.choice([rng.randrange(100, 140), rng.randrange(100, 140) + WIDE * rng.randrange(2)])
+        begin = when()
+        kind = rng.choice([0, 1, 1, 1, 2, 2, 3])
+        if kind == 1:
+            f, cid = dict(grid=(rng.randrange(1, 9), 1, 1), workgroup=(64, 1, 1), lds=0, stream=rng.choice([0, 0x7f10, 0x7f20])), launch
+        elif kind == 2:
+            f, cid = dict(src=0x1000, dst=0x2000, size=rng.randrange(0, 1 << 20), copy_kind=rng.randrange(0, 5), stream=rng.choice([0, 0x7f10])), memcpy_async
+        elif kind == 3:
+            f, cid = dict(ptr=0x3000, size=rng.randrange(0, 1 << 16)), malloc
+        else:
+            f, cid = {}, sync
+        end = min(begin + length(begin), begin + 30 * ms) if begin >= t0 and begin + 30 * ms < t0 + 995 * ms else begin + length(begin)
+        rt.append((rid, begin, end, cid, 4242, 77 + rng.randrange(2), kind, f))
+        if rng.random() < 0.7:
+            ext.append((rid, rng.choice([10 + rng.randrange(12), 10 + rng.randrange(12), 500 + rng.randrange(5)])))
+        if rng.random() < 0.4:
+            user.append((rid, 40 + rng.randrange(4)))
+    dv.append((MARKER_ID, t0 + 500 * ms, t0 + 501 * ms, 0, 0, 0, 3, 11, 0x7f10))
+    for i in range(110):
+        rid = rng.randrange(100, 150)
+        domain = rng.choice([0, 0, 1])
+        begin = when()
+        dv.append((rid, begin, begin + length(begin), domain, rng.randrange(1, 5) if domain else 0, rng.randrange(2),
+                   3 + rng.randrange(2), rng.choice([0, 11, 12, 13]), rng.choice([0, 0, 0x7f10, 0x7f50])))
+    return dict(window=window, cpu_ops=cpu_ops, ext=ext, user=user, rows=(rt, dv, names))
+
+
+def _generic_rec(o):
+    g = abi.GenericRec()
+    g.start_ns, g.end_ns, g.resource, g.id, g.device = o["start"], o["end"], o["resource"], o["id"], o["device"]
+    g.name_id, g.type, g.schema_id = o["name_id"], o["type"], abi.KTJ_NONE
+    return g
+
+
+def run_reference_profiler(case, path):
+    """Runs oracle/_ref/profiler_ref_driver on the case; returns (info dict, trace bytes)."""
+    rt, dv, names = case["rows"]
+    req = struct.pack("<qq", *case["window"])
+    req += struct.pack("<Q", len(case["cpu_ops"])) + b"".join(bytes(_generic_rec(o)) for o in case["cpu_ops"])
+    for pairs in (case["ext"], case["user"]):
+        req += struct.pack("<Q", len(pairs)) + b"".join(struct.pack("<QQ", c, e) for c, e in pairs)
+    req += struct.pack("<Q", len(rt)) + b"".join(bytes(_runtime_rec(r)) for r in rt)
+    req += struct.pack("<Q", len(dv)) + b"".join(bytes(_device_rec(d)) for d in dv)
+    req += struct.pack("<Q", len(names)) + b"".join(struct.pack("<I", len(n)) + n.encode() for n in names)
+    out = subprocess.run([PROFILER_REF_DRIVER, path], input=req, stdout=subprocess.PIPE, stderr=subprocess.PIPE, check=True, timeout=120)
+    info = dict(line.split("=", 1) for line in out.stdout.decode().split("\n") if "=" in line)
+    return {k: int(v) for k, v in info.items()}, open(path, "rb").read()
+
+
+_FLOW = re.compile(r'"ph": "([sf])",\n    "id": (-?\d+),\n    "pid": (-?\d+),\n    "tid": (-?\d+),\n    "ts": ([0-9.]+),\n'
+                   r'    "cat": "([^"]*)",\n    "name": "([^"]*)"\n    (\n  \},|, "bp": "e"\n  \},)')
+
+
+def flow_events(document):
+    return [m.groups() for m in _FLOW.finditer(document.decode("latin1"))]
+
+
+def profiler_stream(case, base_time, device_offset, reference_events):
+    """The case as a ktj_stream for the checker and the engine: the reference's base time, device
+    rows shifted by device_offset (what the reference's clock sampling left over), API names as
+    the reference printed them."""
+    rt, dv, names = case["rows"]
+    b = StreamBuilder(base=base_time, host_name="prof", window=case["window"], end_time=case["window"][1])
+    n_cids = max(r[3] for r in rt) + 1
+    api_names = [None] * n_cids
+    for cat, name, pid, tid, ts, dur, args in reference_events:
+        m = re.match(r'"cid": (\d+),', args or "") or re.search(r', "cid": (\d+),', args or "")
+        if cat == "cuda_runtime" and m:
+            api_names[int(m.group(1))] = name
+    for r in rt:   # operations whose rows were all outside the window are not in the trace: any name will do
+        if api_names[r[3]] is None:
+            api_names[r[3]] = "op%d" % r[3]
+    flow = [c for c in range(n_cids) if sp.sim().ktjsim_sdk_api_is_flow_start(c)]
+    b.api(api_names, flow_start=flow, malloc_cid=op("hipMalloc"))
+    b.clock = abi.ClockModel(0, 0, 1.0, device_offset, 0, 2)   # runtime rows as they are, device rows + offset
+    for o in case["cpu_ops"]:
+        b.add_generic(names[o["name_id"]], o["type"], o["start"], o["end"], o["device"], o["resource"], id=o["id"])
+    for c, e in case["ext"]:
+        b.add_extcorr(c, e)
+    for c, e in case["user"]:
+        b.add_usercorr(c, e)
+    for rid, begin, end, cid, pid, tid, kind, f in rt:
+        kw = dict(f)
+        if kind == 1:
+            kw["kernel_name"] = None
+        b.add_runtime(rid, begin, end, cid, pid, tid, kind=kind, **kw)
+    for rid, begin, end, domain, opn, device, name_id, queue, stream_ in dv:
+        b.add_device(rid, begin, end, domain=domain, op=opn, device=device, name=names[name_id] if names[name_id] else None,
+                     queue=queue, stream=stream_)
+    return b

@@ -94,3 +94,81 @@ def test_engine_matches_the_reference_wrappers():
     ev = rw.events(got)
     ref = [rw.parse(line) for line in lines]
     assert sorted(e[6] or "" for e in ev) == sorted(r["json"] for r in ref)
+
+
+HAVE_PROFILER_DRIVER = os.path.exists(rw.PROFILER_REF_DRIVER)
+
+
+def _reference_profiler_run(seed, tmp_path):
+    """Runs the reference's processTraceInternal on the seeded case; returns the case, the reference's
+    complete and flow events, its counters, and the stream that gives the checker the same input."""
+    case = rw.profiler_case(seed)
+    info, doc = rw.run_reference_profiler(case, str(tmp_path / "ref_trace.json"))
+    ev, fl = rw.events(doc), rw.flow_events(doc)
+    marker = [e for e in ev if e[6] and '"correlation": %d,' % rw.MARKER_ID in e[6]]
+    assert len(marker) == 1
+    marker_begin = case["rows"][1][0][1]
+    whole, frac = marker[0][4].split(".")
+    shown_ns = int(whole) * 1000 + int(frac)                       # "ts" is microseconds with three decimals
+    offset = info["base_time"] + shown_ns - (marker_begin + 1)     # device rows start one nanosecond late
+    assert abs(offset) < 4_000_000, "the rows keep 5 ms from the window's edges"
+    return case, ev, fl, info, rw.profiler_stream(case, info["base_time"], offset, ev)
+
+
+@pytest.mark.skipif(not HAVE_PROFILER_DRIVER, reason="oracle/_ref/profiler_ref_driver is built only where the reference's sources are")
+@pytest.mark.parametrize("seed", range(8))
+def test_checker_matches_the_reference_profiler_loop(seed, tmp_path):
+    """The reference's own GenericActivityProfiler::processTraceInternal (with RocmActivityProfiler's
+    handlers, RocprofActivityApi::processActivities and the real ChromeTraceLogger) on seeded CPU
+    ops, external-correlation pairs, runtime rows and device rows: every complete event and flow
+    event it writes, as text, and its two counters against the checker's.  The reference writes in
+    call order, the checker in canonical order: the events are compared as sorted lists."""
+    case, ev, fl, info, b = _reference_profiler_run(seed, tmp_path)
+    ora = og.OracleRun(b.build())
+    doc = ora.output()
+    cnt = ora.counters()
+    ora.close()
+    mine_ev, mine_fl = rw.events(doc), rw.flow_events(doc)
+    assert sorted(mine_ev) == sorted(ev)
+    assert sorted(mine_fl) == sorted(fl)
+    assert len(ev) > 150 and len(fl) > 100
+    assert cnt["out_of_range"] == info["out_of_range"]
+    assert cnt["out_of_order"] == info["out_of_order"]
+
+
+@pytest.mark.parametrize("seed", (0, 1))
+def test_checker_matches_the_committed_profiler_loop_output(seed):
+    """The same comparison against tests/golden/profiler_loop_seed<k>.json (written by
+    tests/golden/make_profiler_loop_golden.py where the reference is present), for machines without it."""
+    import json
+    import golden.make_profiler_loop_golden as mk
+    g = json.load(open(mk.golden_path(seed)))
+    ev, fl = [tuple(e) for e in g["events"]], [tuple(f) for f in g["flows"]]
+    b = rw.profiler_stream(rw.profiler_case(seed), g["base_time"], g["device_offset"], ev)
+    ora = og.OracleRun(b.build())
+    doc = ora.output()
+    cnt = ora.counters()
+    ora.close()
+    assert sorted(rw.events(doc)) == sorted(ev) and sorted(rw.flow_events(doc)) == sorted(fl)
+    assert (cnt["out_of_range"], cnt["out_of_order"]) == (g["out_of_range"], g["out_of_order"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", (0, 1))
+def test_engine_matches_the_reference_profiler_loop(seed):
+    """The engine's document on the seeded cases: the same events as the reference's own profiler loop
+    wrote (committed fixture), the reference's counters, and the checker's bytes."""
+    import json
+    import golden.make_profiler_loop_golden as mk
+    import test_gpu_parity as tp
+    from kineto_amd.engine import TraceEngine
+    g = json.load(open(mk.golden_path(seed)))
+    ev, fl = [tuple(e) for e in g["events"]], [tuple(f) for f in g["flows"]]
+    sp_ = rw.profiler_stream(rw.profiler_case(seed), g["base_time"], g["device_offset"], ev).build()
+    got = tp._engine_vs_oracle(sp_, base_time_ns=g["base_time"])
+    assert sorted(rw.events(got)) == sorted(ev) and sorted(rw.flow_events(got)) == sorted(fl)
+    with TraceEngine("t.json", base_time_ns=g["base_time"], device=0) as eng:
+        eng.submit_stream(sp_)
+        eng.process()
+        st = eng.stats()
+    assert (st.out_of_range_events, st.gpu_and_cpu_op_out_of_order) == (g["out_of_range"], g["out_of_order"])
