@@ -127,7 +127,8 @@ typedef struct ktj_generic_rec {
   uint64_t args_off;     /* first 8-byte slot of this record's values in the args blob         */
   int32_t id;            /* correlationId() as the logger reads it: `int external_id`
                             (output_json.cpp:871-893); GenericTraceActivity::id is int32       */
-  int32_t device;        /* deviceId() — process id for CPU ops                                */
+  int32_t device;        /* deviceId() — process id for CPU ops.  A deviceId that does not fit 32
+                            bits goes into the args slot before args_off, with KTJ_GF_WIDE_DEVICE */
   uint32_t name_id;      /* string id of name()                                                */
   int32_t linked_id;     /* linkedActivity()->correlationId(), int-truncated like the logger's
                             `int external_id`; read only if KTJ_GF_LINKED                      */
@@ -140,6 +141,7 @@ typedef struct ktj_generic_rec {
 
 #define KTJ_GF_FLOW_START 0x01u /* flow.start                                                  */
 #define KTJ_GF_LINKED 0x02u     /* linkedActivity() != nullptr                                 */
+#define KTJ_GF_WIDE_DEVICE 0x04u /* deviceId() is args[args_off - 1] (an int64), `device` is unused */
 
 /* Kinds of runtime rows: libkineto/src/RocLogger.h:74-81 (rocprof_activity_types). */
 enum {

@@ -948,7 +948,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   if (e->scalars.n_sync_typed != 0) { /* known since the read-back before the sort */
     NEED(e->sync_keys, (KTJ_SYNC_CAP + 1ull) * 8); NEED(e->sync_pos, (KTJ_SYNC_CAP + 1ull) * 4);
     NEED(e->sync_first, ng * 4 + 16);
-    HIPCHK(stream_sync_first(e->perm, e->scalars.n_valid, g_recs, ng, ctx.dict, e->sync_keys.as<uint64_t>(),
+    HIPCHK(stream_sync_first(e->perm, e->scalars.n_valid, g_recs, ng, c.dev, ctx.dict, e->sync_keys.as<uint64_t>(),
                              e->sync_pos.as<uint32_t>(), e->sync_first.as<uint32_t>(), sc, st));
     sync_first = e->sync_first.as<uint32_t>();
   }

@@ -298,9 +298,10 @@ hipError_t radix_sort(uint64_t* keys_a, uint32_t* vals_a, uint64_t* keys_b, uint
                       uint64_t** res_keys, uint32_t** res_vals, hipStream_t st);
 
 /* ---- stage 4a: joined rows + exact byte length (arrival order) ---- */
-/* keys: KTJ_SYNC_CAP + 1, first_pos: KTJ_SYNC_CAP + 1, is_first: n_generic (all caller-provided) */
+/* keys: KTJ_SYNC_CAP + 1, first_pos: KTJ_SYNC_CAP + 1, is_first: n_generic (all caller-provided);
+ * dev: the deviceId column */
 hipError_t stream_sync_first(const uint32_t* perm, uint64_t n_sorted, const ktj_generic_rec* g, uint64_t n_generic,
-                             DictViews d, uint64_t* keys, uint32_t* first_pos, uint32_t* is_first, Scalars* sc,
+                             const int64_t* dev, DictViews d, uint64_t* keys, uint32_t* first_pos, uint32_t* is_first, Scalars* sc,
                              hipStream_t st);
 /* sync_first: per generic row, from stream_sync_first, or null when there are no such rows */
 /* generic records whose rows start at arrival index `first` */

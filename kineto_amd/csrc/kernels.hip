@@ -507,7 +507,7 @@ __global__ void k_decode_generic(const ktj_generic_rec* recs, uint64_t n, Column
   c.ts[a] = g.start_ns;
   c.dur[a] = g.end_ns - g.start_ns;               /* GenericTraceActivity.h:65-67 */
   c.corr[a] = (uint64_t)(int64_t)g.id;
-  c.dev[a] = g.device;
+  c.dev[a] = generic_device(g, ctx.args, ctx.n_args);
   c.res[a] = g.resource;
   c.meta[a] = (generic_record_prints(g, ctx) ? KTJ_M_VALID : 0u) | (KTJ_CLASS_GENERIC << KTJ_M_CLASS_SHIFT);
   c.ext[a] = 0;
@@ -1808,30 +1808,30 @@ __device__ __forceinline__ bool is_stream_sync(const ktj_generic_rec& g, const D
   return g.type == KTJ_TYPE_CUDA_SYNC && g.name_id < d.n && (d.flags[g.name_id] & KTJ_SF_STREAM_SYNC);
 }
 __global__ void k_sync_first_a(const uint32_t* perm, uint64_t n_sorted, const ktj_generic_rec* g, uint64_t n_generic,
-                               DictViews d, uint64_t* keys, uint32_t* first_pos, Scalars* sc) {
+                               const int64_t* dev, DictViews d, uint64_t* keys, uint32_t* first_pos, Scalars* sc) {
   const uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= n_sorted) return;
   const uint64_t a = perm[p];
   if (a >= n_generic || !is_stream_sync(g[a], d)) return;
-  const uint32_t slot = table_insert(keys, KTJ_SYNC_CAP - 1u, stream_sync_key(g[a].device, g[a].resource));
+  const uint32_t slot = table_insert(keys, KTJ_SYNC_CAP - 1u, stream_sync_key(dev[a], g[a].resource));
   if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_SYNC_ROWS); return; }
   atomicMin(&first_pos[slot], (uint32_t)p);
 }
 __global__ void k_sync_first_b(const uint32_t* perm, uint64_t n_sorted, const ktj_generic_rec* g, uint64_t n_generic,
-                               DictViews d, const uint64_t* keys, const uint32_t* first_pos, uint32_t* is_first) {
+                               const int64_t* dev, DictViews d, const uint64_t* keys, const uint32_t* first_pos, uint32_t* is_first) {
   const uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= n_sorted) return;
   const uint64_t a = perm[p];
   if (a >= n_generic) return;
   uint32_t first = 0;
   if (is_stream_sync(g[a], d)) {
-    const uint32_t slot = table_find(keys, KTJ_SYNC_CAP - 1u, stream_sync_key(g[a].device, g[a].resource));
+    const uint32_t slot = table_find(keys, KTJ_SYNC_CAP - 1u, stream_sync_key(dev[a], g[a].resource));
     first = slot != KTJ_NOSLOT && first_pos[slot] == (uint32_t)p;
   }
   is_first[a] = first;
 }
 hipError_t stream_sync_first(const uint32_t* perm, uint64_t n_sorted, const ktj_generic_rec* g, uint64_t n_generic,
-                             DictViews d, uint64_t* keys, uint32_t* first_pos, uint32_t* is_first, Scalars* sc,
+                             const int64_t* dev, DictViews d, uint64_t* keys, uint32_t* first_pos, uint32_t* is_first, Scalars* sc,
                              hipStream_t st) {
   if (n_sorted == 0 || n_generic == 0) return hipSuccess;
   hipError_t e = fill_u64(keys, KTJ_EMPTY_KEY, KTJ_SYNC_CAP + 1ull, st);
@@ -1841,8 +1841,8 @@ hipError_t stream_sync_first(const uint32_t* perm, uint64_t n_sorted, const ktj_
   e = fill_u32(is_first, 0u, n_generic, st);
   if (e != hipSuccess) return e;
   const dim3 grid(grid_for(n_sorted, KTJ_BLOCK)), b(KTJ_BLOCK);
-  hipLaunchKernelGGL(k_sync_first_a, grid, b, 0, st, perm, n_sorted, g, n_generic, d, keys, first_pos, sc);
-  hipLaunchKernelGGL(k_sync_first_b, grid, b, 0, st, perm, n_sorted, g, n_generic, d, (const uint64_t*)keys,
+  hipLaunchKernelGGL(k_sync_first_a, grid, b, 0, st, perm, n_sorted, g, n_generic, dev, d, keys, first_pos, sc);
+  hipLaunchKernelGGL(k_sync_first_b, grid, b, 0, st, perm, n_sorted, g, n_generic, dev, d, (const uint64_t*)keys,
                      (const uint32_t*)first_pos, is_first);
   return KTJ_LAUNCH_CHECK();
 }
@@ -1852,7 +1852,7 @@ __global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, uint64_t fir
   RowStats rs;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const ktj_generic_rec rec = g[i];
-    MatRow m = mat_generic(rec);
+    MatRow m = mat_generic(rec, generic_device(rec, ctx.args, ctx.n_args));
     if (!generic_record_prints(rec, ctx)) m.meta &= ~KTJ_M_VALID;
     attach_own_collective(m, rec, ctx);
     mark_stream_sync(m, ctx, sync_first != nullptr && sync_first[i] != 0);

@@ -64,11 +64,17 @@ KTJ_HD inline bool type_hides_own_external_id(uint32_t type) { /* output_json.cp
   }
 }
 
-KTJ_HD inline MatRow mat_generic(const ktj_generic_rec& g) {
+/* deviceId() of a generic record: the 32-bit field, or the args slot before the record's values */
+KTJ_HD inline int64_t generic_device(const ktj_generic_rec& g, const uint64_t* args, uint64_t n_args) {
+  if ((g.flags & KTJ_GF_WIDE_DEVICE) && g.args_off >= 1 && g.args_off - 1 < n_args) return (int64_t)args[g.args_off - 1];
+  return g.device;
+}
+
+KTJ_HD inline MatRow mat_generic(const ktj_generic_rec& g, int64_t device) {
   MatRow m;
   m.ts = g.start_ns;
   m.dur = g.end_ns - g.start_ns;
-  m.dev = g.device;
+  m.dev = device;
   m.res = g.resource;
   m.flow_id = g.flow_id;
   uint32_t meta = (g.type & KTJ_M_TYPE_MASK) | (KTJ_CLASS_GENERIC << KTJ_M_CLASS_SHIFT) | KTJ_M_VALID;

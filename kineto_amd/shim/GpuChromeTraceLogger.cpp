@@ -61,8 +61,6 @@ struct GpuChromeTraceLogger::Packed {
   std::unordered_map<std::string, uint32_t> collectiveIndex;
   std::vector<std::vector<uint32_t>> counterSchemas; /* local ids of the counter names */
   std::unordered_map<std::string, uint32_t> counterIndex;
-  uint64_t unsupported = 0;
-  std::string firstUnsupported;
   /* engine ids of the local entries translated so far (merge) */
   std::vector<uint32_t> nameGlobal, collectiveGlobal, counterGlobal;
   uint32_t fragmentBase = 0; /* engine id of local fragment 0 */
@@ -135,15 +133,12 @@ void GpuChromeTraceLogger::pack(const ITraceActivity& op, uint64_t origin, Packe
   const bool collective = !counter && linked != nullptr &&
       (type == ActivityType::CONCURRENT_KERNEL || (type == ActivityType::MTIA_CCP_EVENTS && name.rfind("hccl::", 0) == 0)) &&
       linked->name() == kParamCommsName;
-  if (device < std::numeric_limits<int32_t>::min() || device > std::numeric_limits<int32_t>::max()) {
-    if (out.unsupported++ == 0) out.firstUnsupported = name;
-    return;
-  }
+  const bool wideDevice = device < std::numeric_limits<int32_t>::min() || device > std::numeric_limits<int32_t>::max();
   ktj_generic_rec r{};
   r.start_ns = op.timestamp();
   r.end_ns = r.start_ns + op.duration();
   r.resource = op.resourceId();
-  r.device = static_cast<int32_t>(device);
+  r.device = wideDevice ? 0 : static_cast<int32_t>(device);
   r.id = static_cast<int32_t>(op.correlationId()); /* `int external_id = op.correlationId()`, :893 */
   r.type = static_cast<uint8_t>(type);
   r.name_id = out.name(name);
@@ -156,6 +151,10 @@ void GpuChromeTraceLogger::pack(const ITraceActivity& op, uint64_t origin, Packe
     r.linked_id = static_cast<int32_t>(linked->correlationId()); /* `int external_id = …`, :873 */
   }
   r.schema_id = KTJ_NONE;
+  if (wideDevice) { /* the record's device field is 32 bits: the value goes into the slot before the record's values */
+    r.flags |= KTJ_GF_WIDE_DEVICE;
+    out.slot(static_cast<uint64_t>(device), kSlotPlain);
+  }
   r.args_off = out.slots.size();
   if (counter) { /* handleCounterEvent (:679-716) prints counterValues() and nothing else */
     const auto& values = op.counterValues();
@@ -217,14 +216,6 @@ uint32_t GpuChromeTraceLogger::intern(const std::string& s) {
 /* Brings the packer's dictionaries up to date with the engine's: every local string, collective
  * entry and counter schema that has no engine id yet gets one. */
 void GpuChromeTraceLogger::translate(Packed& p) {
-  if (p.unsupported != 0) {
-    if (unsupported_ == 0) {
-      LOG(WARNING) << "GpuChromeTraceLogger: activity '" << p.firstUnsupported
-                   << "' has a deviceId outside 32 bits; such activities are dropped";
-    }
-    unsupported_ += p.unsupported;
-    p.unsupported = 0;
-  }
   for (size_t i = p.nameGlobal.size(); i < p.names.size(); ++i) p.nameGlobal.push_back(intern(p.names[i]));
   /* the fragments of this batch get consecutive ids */
   const size_t nFragments = p.fragmentOff.size() - 1;
@@ -438,7 +429,7 @@ void GpuChromeTraceLogger::handleActivities(const std::vector<const ITraceActivi
 
   /* merge.  In sequence: the local dictionaries become engine ids and every part learns where its
    * slots go.  Then, part by part on the workers: slots and records move to their final places
-   * (a record's place is its activity's position; activities that were dropped leave holes). */
+   * (a record's place is its activity's position). */
   std::vector<uint64_t> base(parts.size());
   size_t nRecords = 0, nSlots = 0;
   for (size_t w = 0; w < parts.size(); ++w) {
@@ -447,10 +438,10 @@ void GpuChromeTraceLogger::handleActivities(const std::vector<const ITraceActivi
     nSlots += parts[w].slots.size();
     nRecords += parts[w].records.size();
   }
+  if (nRecords != n) { note(KTJ_ERR_STATE, "record bookkeeping"); return; } /* every activity packs into one record */
   const size_t slot0 = slots_.size();
   slots_.resize(slot0 + nSlots);
-  std::unique_ptr<ktj_generic_rec[]> placed(new ktj_generic_rec[n]); /* not zero-filled: every kept place is written */
-  std::vector<uint8_t> present(nRecords == n ? 0 : n, 0);
+  std::unique_ptr<ktj_generic_rec[]> placed(new ktj_generic_rec[n]); /* not zero-filled: every place is written */
   const unsigned nParts = static_cast<unsigned>(parts.size());
   const uint64_t firstSlot = nextSlot_;
   run([&](unsigned w0) {
@@ -461,21 +452,12 @@ void GpuChromeTraceLogger::handleActivities(const std::vector<const ITraceActivi
         const uint64_t v = p.slots[i];
         out[i] = p.slotKind[i] == kSlotFragment ? p.fragmentBase + v : p.slotKind[i] == kSlotCollective ? p.collectiveGlobal[v] : v;
       }
-      for (size_t j = 0; j < p.records.size(); ++j) {
-        placed[p.origin[j]] = translated(p, j, base[w]);
-        if (!present.empty()) present[p.origin[j]] = 1;
-      }
+      for (size_t j = 0; j < p.records.size(); ++j) placed[p.origin[j]] = translated(p, j, base[w]);
     }
   });
   nextSlot_ += nSlots;
-  size_t kept = n;
-  if (!present.empty()) { /* close the holes */
-    kept = 0;
-    for (size_t i = 0; i < n; ++i)
-      if (present[i]) placed[kept++] = placed[i];
-  }
   flushStrings();
-  submitRecords(placed.get(), kept); /* records_ is empty here: mergeInOrder above flushed it */
+  submitRecords(placed.get(), n); /* records_ is empty here: mergeInOrder above flushed it */
 }
 
 void GpuChromeTraceLogger::handleGenericActivity(const GenericTraceActivity& op) {

@@ -56,7 +56,7 @@ class GpuChromeTraceLogger : public libkineto::ActivityLogger {
                      int64_t endTime) override;
 
   std::string traceFileName() const { return fileName_; }
-  /* activities the engine cannot take (a deviceId outside 32 bits): dropped and counted here */
+  /* activities the engine could not take; every kind is taken at present, so this reads 0 */
   uint64_t unsupportedActivities() const { return unsupported_; }
   /* ktj status of the first failed engine call, 0 if none */
   int engineStatus() const { return status_; }

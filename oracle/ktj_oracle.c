@@ -535,7 +535,9 @@ static int stage_join(ktj_oracle* o) {
     ktj_mat_activity* a = new_act(o);
     a->ts = r->start_ns;
     a->dur = r->end_ns - r->start_ns;
-    a->device = r->device;
+    /* a deviceId beyond 32 bits travels in the args slot before the record's values (include/ktj.h) */
+    a->device = ((r->flags & KTJ_GF_WIDE_DEVICE) && r->args_off >= 1 && r->args_off - 1 < s->n_args)
+                    ? (int64_t)s->args[r->args_off - 1] : r->device;
     a->resource = r->resource;
     a->corr = r->id;
     a->flow_id = r->flow_id;

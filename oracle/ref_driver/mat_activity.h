@@ -44,6 +44,7 @@ struct MatActivity : public ITraceActivity {
   const StringTable* st;
   mutable GenericTraceActivity linkedStub;  // only correlationId()/name() are read from it
   bool hasLinked;
+  bool wideDevice = false;  // reports a deviceId beyond 32 bits (set by replay_stream)
 
   // collectives: ktj_stream::collectives; an activity whose linked op carries collective metadata
   // gets a record_param_comms op with those values as its linked activity
@@ -65,7 +66,8 @@ struct MatActivity : public ITraceActivity {
         if (e.second != nullptr && e.second[0] != 0) linkedStub.addMetadata(std::string(e.first), std::string(e.second));
     }
   }
-  int64_t deviceId() const override { return a->device; }
+  int64_t deviceId() const override { return wideDevice ? kWideDeviceId : a->device; }
+  static constexpr int64_t kWideDeviceId = int64_t{1} << 40;
   int64_t resourceId() const override { return a->resource; }
   int32_t getThreadId() const override { return 0; }
   int64_t timestamp() const override { return a->ts; }
@@ -235,11 +237,14 @@ struct GenericMatActivity : public GenericTraceActivity {
 //   rest.  Only a logger that sorts by itself writes the file of call_order 1 from it.
 template <class L, class LogAll>
 void replay_stream(L& logger, const ktj_stream* s, const ktj_mat_activity* acts, uint64_t n_acts, string_fn fn,
-                   const void* ctx, LogAll log_all, int call_order = 0) {
+                   const void* ctx, LogAll log_all, int call_order = 0, int wide_device_mod = 0) {
   StringTable st{fn, ctx};
   std::vector<MatActivity> wrapped;
   wrapped.reserve(n_acts);
-  for (uint64_t i = 0; i < n_acts; ++i) wrapped.emplace_back(&acts[i], &st, s->collectives);
+  for (uint64_t i = 0; i < n_acts; ++i) {
+    wrapped.emplace_back(&acts[i], &st, s->collectives);
+    wrapped.back().wideDevice = wide_device_mod > 0 && acts[i].arrival % static_cast<uint64_t>(wide_device_mod) == 1;
+  }
   std::vector<const MatActivity*> order(n_acts);
   for (uint64_t i = 0; i < n_acts; ++i) order[i] = &wrapped[i];
   if (call_order != 2)
@@ -310,10 +315,10 @@ void replay_stream(L& logger, const ktj_stream* s, const ktj_mat_activity* acts,
 
 template <class L>
 void replay_stream(L& logger, const ktj_stream* s, const ktj_mat_activity* acts, uint64_t n_acts, string_fn fn,
-                   const void* ctx, int call_order = 0) {
+                   const void* ctx, int call_order = 0, int wide_device_mod = 0) {
   replay_stream(logger, s, acts, n_acts, fn, ctx, [](L& l, const std::vector<const MatActivity*>& order) {
     for (const MatActivity* a : order) a->log(l);
-  }, call_order);
+  }, call_order, wide_device_mod);
 }
 
 }  // namespace ktj_ref_driver

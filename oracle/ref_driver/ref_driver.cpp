@@ -48,13 +48,14 @@ int64_t ktj_ref_base_time(void) { return ChromeTraceBaseTime::singleton().get();
 
 // Renders the stream's header/infos/spans and the given activities with the real logger into
 // out_path, with the activities stable-sorted by (deviceId, resourceId, timestamp); call_order as
-// described at replay_stream (0: the buffering logger's replay, 1: the profiler's own order).
+// described at replay_stream (0: the buffering logger's replay, 1: the profiler's own order), and
+// so is wide_device_mod (activities that report a deviceId beyond 32 bits).
 int ktj_ref_render(const ktj_stream* s, const ktj_mat_activity* acts, uint64_t n_acts, string_fn fn,
-                   const void* ctx, const char* out_path, int call_order) {
+                   const void* ctx, const char* out_path, int call_order, int wide_device_mod) {
   SET_LOG_SEVERITY_LEVEL(3);  // ERROR: silence per-name WARNING lines
   if (s->base_time_ns != ChromeTraceBaseTime::singleton().get()) return -2;
   RefLogger logger{std::string(out_path)};
-  replay_stream(logger, s, acts, n_acts, fn, ctx, call_order);
+  replay_stream(logger, s, acts, n_acts, fn, ctx, call_order, wide_device_mod);
   return 0;
 }
 

@@ -39,7 +39,7 @@ int64_t ktj_shim_base_time(void) { return ChromeTraceBaseTime::singleton().get()
 // bulk_threads > 0: the activities are handed over in one handleActivities() call with that many
 // workers, as GenericTraceActivity objects (so that the workers pack them).
 // huge_device_mod > 0: every activity whose arrival index is 1 modulo it reports a deviceId
-// beyond 32 bits, which the shim drops (and counts in *unsupported).
+// beyond 32 bits (replay_stream's wide_device_mod); *unsupported stays 0 for them.
 // call_order: see replay_stream (0: the buffering logger's replay; 2: the calls as
 // GenericActivityProfiler issues them, activities unsorted and split around the CPU span).
 int ktj_shim_render(const ktj_stream* s, const ktj_mat_activity* acts, uint64_t n_acts, string_fn fn,
@@ -59,35 +59,25 @@ int ktj_shim_render(const ktj_stream* s, const ktj_mat_activity* acts, uint64_t 
   }
   auto* shim = dynamic_cast<ShimLogger*>(logger.get());
   if (shim == nullptr) return -3;
-  struct HugeDevice : public GenericMatActivity {
-    using GenericMatActivity::GenericMatActivity;
-    int64_t deviceId() const override { return int64_t{1} << 40; }
-  };
-  auto huge = [huge_device_mod](const MatActivity* a) {
-    return huge_device_mod > 0 && a->a->arrival % static_cast<uint64_t>(huge_device_mod) == 1;
-  };
   if (bulk_threads > 0) {
     replay_stream(*shim, s, acts, n_acts, fn, ctx, [&](ShimLogger& l, const std::vector<const MatActivity*>& order) {
       std::vector<GenericMatActivity> generic;
-      std::vector<HugeDevice> dropped;
       generic.reserve(order.size());
-      dropped.reserve(order.size());
       std::vector<const ITraceActivity*> all;
       all.reserve(order.size());
       for (size_t i = 0; i < order.size(); ++i) {
-        if (huge(order[i])) { dropped.emplace_back(order[i]); all.push_back(&dropped.back()); }
-        else if (i % 7 == 3) all.push_back(order[i]); /* some stay plain ITraceActivity: packed by the calling thread */
+        if (i % 7 == 3) all.push_back(order[i]); /* some stay plain ITraceActivity: packed by the calling thread */
         else { generic.emplace_back(order[i]); all.push_back(&generic.back()); }
       }
       l.handleActivities(all, static_cast<unsigned>(bulk_threads));
-    }, call_order);
+    }, call_order, huge_device_mod);
   } else if (huge_device_mod > 0) {
     replay_stream(*shim, s, acts, n_acts, fn, ctx, [&](ShimLogger& l, const std::vector<const MatActivity*>& order) {
       for (const MatActivity* a : order) {
-        if (huge(a)) { const HugeDevice h(a); l.handleActivity(h); }
+        if (a->wideDevice) { const GenericMatActivity g(a); l.handleActivity(g); }
         else a->log(l);
       }
-    }, call_order);
+    }, call_order, huge_device_mod);
   } else {
     replay_stream(*shim, s, acts, n_acts, fn, ctx, call_order);
   }

@@ -116,7 +116,7 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   for (uint64_t i = 0; i < s->n_flow_start; ++i) if (s->flow_start_cids[i] < s->n_cids) flow_start[s->flow_start_cids[i]] = 1;
 
   for (uint64_t i = 0; i < ng; ++i) {
-    mat[i] = mat_generic(s->generic[i]);
+    mat[i] = mat_generic(s->generic[i], generic_device(s->generic[i], s->args, s->n_args));
     if (!generic_record_prints(s->generic[i], ctx)) mat[i].meta &= ~KTJ_M_VALID;
     attach_own_collective(mat[i], s->generic[i], ctx);
   }
@@ -254,7 +254,7 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
         r.start_ns = sp.start; r.end_ns = sp.end; r.resource = sp.res; r.device = (int32_t)sp.dev;
         r.id = (int32_t)sp.id; r.name_id = s->generic[sp.op].name_id; r.schema_id = KTJ_NONE;
         r.type = KTJ_TYPE_GPU_USER_ANNOTATION;
-        mat.push_back(mat_generic(r));
+        mat.push_back(mat_generic(r, sp.dev));
       }
     }
   }

@@ -77,7 +77,7 @@ def load_ref():
         lib.ktj_ref_base_time.restype = C.c_int64
         lib.ktj_ref_render.restype = C.c_int
         lib.ktj_ref_render.argtypes = [C.POINTER(abi.Stream), C.POINTER(MatActivity), C.c_uint64,
-                                       C.c_void_p, C.c_void_p, C.c_char_p, C.c_int]
+                                       C.c_void_p, C.c_void_p, C.c_char_p, C.c_int, C.c_int]
         lib.ktj_ref_fmt_double.restype = C.c_size_t
         lib.ktj_ref_fmt_double.argtypes = [C.c_double, C.c_char_p]
         lib.ktj_ref_metadata_order.restype = C.c_size_t
@@ -164,12 +164,13 @@ class OracleRun:
             self.h = None
 
 
-def ref_render(stream_ptr, oracle_run, skip_arrival_mod=0, call_order=0):
+def ref_render(stream_ptr, oracle_run, skip_arrival_mod=0, call_order=0, wide_device_mod=0):
     """Renders the stream with the reference's own ChromeTraceLogger, fed with the activities the
     oracle's join stage produced (arrival order; the driver sorts them itself).  skip_arrival_mod >
     0 leaves out every activity whose arrival index is 1 modulo it.  call_order 1: infos and spans
     arrive after the activities, as GenericActivityProfiler issues them (see replay_stream in
-    oracle/ref_driver/mat_activity.h)."""
+    oracle/ref_driver/mat_activity.h).  wide_device_mod > 0: every activity whose arrival index is
+    1 modulo it reports a deviceId of 2^40."""
     ref = load_ref()
     acts, n = oracle_run.activities()
     if skip_arrival_mod > 0:
@@ -181,7 +182,7 @@ def ref_render(stream_ptr, oracle_run, skip_arrival_mod=0, call_order=0):
     fn = C.cast(load_oracle().ktj_oracle_string, C.c_void_p)
     with tempfile.TemporaryDirectory() as d:
         path = os.path.join(d, stream_ptr.contents.trace_name.decode())
-        rc = ref.ktj_ref_render(stream_ptr, acts, n, fn, oracle_run.h, path.encode(), call_order)
+        rc = ref.ktj_ref_render(stream_ptr, acts, n, fn, oracle_run.h, path.encode(), call_order, wide_device_mod)
         if rc != 0:
             raise RuntimeError(f"ktj_ref_render rc={rc}")
         with open(path, "rb") as f:
@@ -194,7 +195,7 @@ def shim_render(stream_ptr, oracle_run, protocol="gpujson", directory=None, bulk
     """Renders the stream through the GpuChromeTraceLogger shim obtained from a logger factory by
     URL, fed with the same activities as ref_render, one handleActivity() call each or, with
     bulk_threads > 0, in one handleActivities() call.  huge_device_mod > 0: every activity whose
-    arrival index is 1 modulo it reports a deviceId beyond 32 bits (the shim drops those).
+    arrival index is 1 modulo it reports a deviceId of 2^40.
     Returns (status, bytes or None, dropped)."""
     shim = load_shim()
     acts, n = oracle_run.activities()

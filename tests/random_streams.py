@@ -96,6 +96,8 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False,
             schemas.append((b.schema(fields), fields))
         schemas.append((b.schema([(None, abi.F_COLLECTIVE, 1), (None, abi.F_RAW, 1)]), [(None, abi.F_COLLECTIVE, 1), (None, abi.F_RAW, 1)]))
     pids, tids = [0, 1, 7, -3, 4242], [0, 5, -5, 4243, I64_MIN, I64_MAX, 10**12]
+    if wide_ids:  # deviceId values that do not fit the record's 32-bit field
+        pids += [2**40, -(2**33) - 5]
     ids = list(range(1, 30))
     if wide_ids:
         ids += [(1 << 32) + 3, (1 << 31) + 1, 0xFFFFFFFFFFFFFFFF, 0xFFFFFFFF00000001, 1 << 40]

@@ -86,14 +86,17 @@ class StreamBuilder:
                     flow_type=0, flow_start=False, linked=None):
         r = abi.GenericRec()
         r.start_ns, r.end_ns, r.resource = start, end, resource
-        r.id, r.device = id, device
+        wide = not -(1 << 31) <= device < (1 << 31)  # travels in the slot before the record's values
+        r.id, r.device = id, 0 if wide else device
         r.name_id = abi.KTJ_NONE if name is None else self.s(name)
         r.type = typ
         r.flow_id, r.flow_type = flow_id, flow_type
-        r.flags = (1 if flow_start else 0) | (2 if linked is not None else 0)
+        r.flags = (1 if flow_start else 0) | (2 if linked is not None else 0) | (abi.KTJ_GF_WIDE_DEVICE if wide else 0)
         r.linked_id = 0 if linked is None else C.c_int32(linked & 0xFFFFFFFF).value
         r.schema_id = abi.KTJ_NONE if schema is None else schema
-        r.args_off = self.arg_slots(values) if schema is not None else 0
+        if wide:
+            self.arg_slots([device])
+        r.args_off = self.arg_slots(values) if schema is not None else (len(self.args) if wide else 0)
         self.generic.append(r)
         return r
 

@@ -57,7 +57,10 @@ def brute(sp):
     activity_map = {}  # int64(int32 id) -> generic index
     for i in range(s.n_generic):
         g = s.generic[i]
-        acts.append(dict(arrival=i, ts=g.start_ns, dur=g.end_ns - g.start_ns, device=g.device, resource=g.resource,
+        device = g.device
+        if g.flags & abi.KTJ_GF_WIDE_DEVICE:  # the slot before the record's values, read as a signed 64-bit value
+            device = C.c_int64(s.args[g.args_off - 1]).value
+        acts.append(dict(arrival=i, ts=g.start_ns, dur=g.end_ns - g.start_ns, device=device, resource=g.resource,
                          type=g.type, linked=(g.linked_id if g.flags & 2 else None), extra={}))
         activity_map[g.id] = i
     cpu_corr = {}
