@@ -432,7 +432,7 @@ static __device__ __attribute__((noinline)) void cooperative_word_copy(const cha
 #if defined(__HIPCC__)
 /* blocks per lane in the stage; odd, so that neither the lanes' writes (same block index, lane
  * stride 16 * KTJ_STAGE_BLOCKS bytes) nor the quads' reads collide on LDS banks */
-#define KTJ_STAGE_BLOCKS 11u
+#define KTJ_STAGE_BLOCKS 13u
 #define KTJ_FLUSH_LANES 4u
 #define KTJ_FLUSH_ROUNDS ((KTJ_STAGE_BLOCKS + 2u * KTJ_FLUSH_LANES - 2u) / KTJ_FLUSH_LANES) /* blocks plus up to LANES - 1 of misalignment */
 extern __shared__ __attribute__((aligned(16))) char ktj_stage_lds[];
@@ -492,20 +492,30 @@ struct BlockWriter {
   }
   /* wptr is about to move by more than one block: what is staged stays, nothing more is staged */
   __device__ KTJ_FI void stage_close() { stage_cap = n_staged; }
-  /* Every lane of the wavefront must call this together (lanes without an activity included). */
-  __device__ KTJ_FI void flush() {
+  /* Every lane of the wavefront must call this together (lanes without an activity included).
+   * Unless `last`, a lane whose stage is still open (every block since the stage's first one is in
+   * it) lets only whole 128-byte lines of the document go and keeps the blocks of the line it has
+   * not finished: they move to the front of the stage and leave with the rest of their line at the
+   * next flush, so that the line reaches memory in one piece. */
+  __device__ KTJ_FI void flush(bool last) {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef unsigned long long v2u64 __attribute__((ext_vector_type(2)));
     typedef __attribute__((address_space(1))) v2u64* gptr; /* the document is global memory: no flat stores */
     const uint32_t k = (uint32_t)threadIdx.x & 3u;
     const uint32_t base_lo = (uint32_t)(uintptr_t)stage_base, base_hi = (uint32_t)((uintptr_t)stage_base >> 32);
+    uint32_t n_out = n_staged;
+    if (!last && n_staged < stage_cap) {
+      const uint32_t end_lo = base_lo + 16u * n_staged;         /* the low address bits decide */
+      const uint32_t whole = (end_lo & ~127u) - base_lo;        /* bytes up to the last line boundary, if any */
+      n_out = (int32_t)whole > 0 ? whole >> 4 : 0u;
+    }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #define KTJ_QUAD_BCAST(v, t) ((uint32_t)__builtin_amdgcn_mov_dpp((int)(v), (t) * 0x55, 0xF, 0xF, true))
 #define KTJ_FLUSH_FROM(t)                                                                       \
     {                                                                                           \
-      const uint32_t n_s = KTJ_QUAD_BCAST(n_staged, t);                                         \
+      const uint32_t n_s = KTJ_QUAD_BCAST(n_out, t);                                            \
       const uint32_t lds_s = KTJ_QUAD_BCAST(stage_lds, t);                                      \
       const uint32_t lo_s = KTJ_QUAD_BCAST(base_lo, t);                                         \
       gptr d = reinterpret_cast<gptr>(((uintptr_t)KTJ_QUAD_BCAST(base_hi, t) << 32) | (uintptr_t)lo_s); \
@@ -527,9 +537,22 @@ struct BlockWriter {
     KTJ_FLUSH_FROM(0) KTJ_FLUSH_FROM(1) KTJ_FLUSH_FROM(2) KTJ_FLUSH_FROM(3)
 #undef KTJ_FLUSH_FROM
 #undef KTJ_QUAD_BCAST
+    /* the blocks that stay move to the front (at most seven: less than a line); the wavefront's LDS
+     * accesses keep their order, so the quads have read them by now */
+    const uint32_t keep = n_staged - n_out;
+    if (keep != 0 && n_out != 0) {
+      v2u64 t[7];
+      _Pragma("unroll")
+      for (uint32_t m = 0; m < 7; ++m)
+        t[m] = *reinterpret_cast<const v2u64*>(ktj_stage_lds + stage_lds + (m < keep ? n_out + m : 0u) * 16u);
+      _Pragma("unroll")
+      for (uint32_t m = 0; m < 7; ++m)
+        if (m < keep) *reinterpret_cast<v2u64*>(ktj_stage_lds + stage_lds + m * 16u) = t[m];
+    }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    n_staged = 0;
+    stage_base += 2u * n_out;
+    n_staged = keep;
     stage_cap = KTJ_STAGE_BLOCKS;
 #endif
   }

@@ -2277,7 +2277,9 @@ k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n
  * BlockWriter for who writes the blocks that two activities share).  Finished blocks wait in LDS
  * and leave at the three points where the whole wavefront meets: after the head of the event,
  * after its args and after the flow event; there four neighbouring lanes store four consecutive
- * blocks of one activity at a time.  Lanes without an activity stay until the end for that.  The
+ * blocks of one activity at a time, whole 128-byte lines only until the last of the three (a line
+ * written in two pieces some microseconds apart leaves the L2 cache twice).  Lanes without an
+ * activity stay until the end for that.  The
  * document's prefix and suffix are already in place when this kernel runs; the first and the last
  * activity merge with them. */
 __global__ void __launch_bounds__(KTJ_BLOCK) __attribute__((amdgpu_waves_per_eu(3)))
@@ -2285,25 +2287,26 @@ k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, con
               EmitCtx ctx, char* out, uint64_t prefix_len) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   uint64_t o = 0;
+  uint32_t row = 0;
   bool active = i < n_rows;
-  if (active) { o = offs[i]; active = offs[i + 1] != o; }
+  if (active) { row = perm[i]; o = offs[i]; active = offs[i + 1] != o; } /* one wait for both */
   MatRow m;
   BlockWriter w;
   w.stage_init((uint32_t)threadIdx.x * (KTJ_STAGE_BLOCKS * 16u));
   ActivityParts<BlockWriter> parts;
   if (active) {
-    m = mat[perm[i]];
+    m = mat[row];
     w.begin(out, prefix_len + o, i ? kind_sorted[i - 1] : 0u, i == 0);
     format_head(w, m, ctx, parts);
   }
-  w.flush();
+  w.flush(false);
   if (active) format_args(w, m, ctx, parts);
-  w.flush();
+  w.flush(false);
   if (active) {
     format_flow(w, m, ctx, parts);
     w.end(i + 1 == n_rows);
   }
-  w.flush();
+  w.flush(true);
 }
 hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint8_t* kind_sorted,
                        uint64_t n_rows, uint64_t act_bytes, EmitCtx ctx, char* out, uint64_t prefix_len, hipStream_t st) {
