@@ -170,6 +170,8 @@ struct ktj_engine {
   DevBuf mat, len, len_sorted, kind_sorted, offs, out, tile_start;
   void* pinned_small = nullptr; size_t pinned_small_cap = 0;
   HostCtl* h_ctl = nullptr;                  /* pinned: what the device hands back during a pass */
+  HostCtl* h_ctl_dev = nullptr;              /* the same memory as the kernels address it */
+  char* pinned_small_dev = nullptr;
   /* ktj_process_noalloc: working buffers are carved out of the library's static scratch array */
   bool noalloc = false;
   char* arena = nullptr; size_t arena_cap = 0, arena_used = 0;
@@ -401,6 +403,11 @@ int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int
     HIPCHK(hipHostMalloc(&p, sizeof(HostCtl), hipHostMallocDefault));
     e->h_ctl = static_cast<HostCtl*>(p);
     memset(e->h_ctl, 0, sizeof(HostCtl));
+    void* d = nullptr;
+    HIPCHK(hipHostGetDevicePointer(&d, e->h_ctl, 0));
+    e->h_ctl_dev = static_cast<HostCtl*>(d);
+    HIPCHK(hipHostGetDevicePointer(&d, e->pinned_small, 0));
+    e->pinned_small_dev = static_cast<char*>(d);
   }
   { /* this device's copy of the static scratch array (ktj_process_noalloc) */
     void* p = nullptr;
@@ -885,7 +892,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   HIPCHK(collect_distinct(c, N, sets, sc, st));
   HIPCHK(rank_distinct(sets, sc, st));
   HIPCHK(hipEventRecord(e->ev[EV_SORT_A], st));
-  HIPCHK(hipMemcpyAsync(&e->h_ctl->scalars, sc, sizeof(Scalars), hipMemcpyDeviceToHost, st));
+  HIPCHK(publish(sc, nullptr, nullptr, 0, &e->h_ctl_dev->scalars, nullptr, nullptr, st));
   HIPCHK(hipStreamSynchronize(st));
   e->scalars = e->h_ctl->scalars;
   const unsigned distinct_overflow = e->scalars.error & (KTJ_DEVERR_DISTINCT_DEVICES | KTJ_DEVERR_DISTINCT_RESOURCES);
@@ -964,18 +971,17 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   HIPCHK(scan_u32_to_u64(e->len_sorted.as<uint32_t>(), e->offs.as<uint64_t>(), N, e->scan_tmp.as<uint64_t>(), st));
   HIPCHK(hipEventRecord(e->ev[EV_SCAN], st));
   uint64_t act_bytes = 0;
-  HIPCHK(hipMemcpyAsync(&e->h_ctl->act_bytes, e->offs.as<uint64_t>() + N, 8, hipMemcpyDeviceToHost, st));
-  HIPCHK(hipMemcpyAsync(&e->h_ctl->scalars, sc, sizeof(Scalars), hipMemcpyDeviceToHost, st));
   e->coll_first.assign(2ull * n_coll, 0xFFFFFFFFu);
-  if (n_coll && e->noalloc) { /* through the engine's pinned buffer */
-    if (2ull * n_coll * 4 > e->pinned_small_cap) {
-      e->last_error = "ktj_process_noalloc: too many collective entries for the pinned staging buffer";
-      return KTJ_ERR_LIMIT;
-    }
-    HIPCHK(hipMemcpyAsync(e->pinned_small, e->d_coll_first.p, 2ull * n_coll * 4, hipMemcpyDeviceToHost, st));
-  } else if (n_coll) HIPCHK(hipMemcpyAsync(e->coll_first.data(), e->d_coll_first.p, 2ull * n_coll * 4, hipMemcpyDeviceToHost, st));
+  const bool list_fits = 2ull * n_coll * 4 <= e->pinned_small_cap; /* through the engine's pinned buffer when it fits */
+  if (n_coll && !list_fits && e->noalloc) {
+    e->last_error = "ktj_process_noalloc: too many collective entries for the pinned staging buffer";
+    return KTJ_ERR_LIMIT;
+  }
+  HIPCHK(publish(sc, e->offs.as<uint64_t>() + N, e->d_coll_first.as<uint32_t>(), list_fits ? 2u * n_coll : 0u, &e->h_ctl_dev->scalars,
+                 &e->h_ctl_dev->act_bytes, reinterpret_cast<uint32_t*>(e->pinned_small_dev), st));
+  if (n_coll && !list_fits) HIPCHK(hipMemcpyAsync(e->coll_first.data(), e->d_coll_first.p, 2ull * n_coll * 4, hipMemcpyDeviceToHost, st));
   HIPCHK(hipStreamSynchronize(st));
-  if (n_coll && e->noalloc) memcpy(e->coll_first.data(), e->pinned_small, 2ull * n_coll * 4);
+  if (n_coll && list_fits) memcpy(e->coll_first.data(), e->pinned_small, 2ull * n_coll * 4);
   act_bytes = e->h_ctl->act_bytes;
   e->scalars = e->h_ctl->scalars;
   if (e->scalars.error) {
@@ -1008,7 +1014,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
     }
     e->out.borrow(out_device, out_cap);
   } else NEED(e->out, e->total_bytes + 64);
-  const size_t small = prefix.size() + suffix.size();
+  const size_t small = prefix.size() + suffix.size() + 64; /* each piece starts where its place in the document does, modulo 16 */
   if (small > e->pinned_small_cap && e->noalloc) {
     e->last_error = "ktj_process_noalloc: header and footer text of " + std::to_string(small) + " bytes exceeds the pinned staging buffer";
     return KTJ_ERR_LIMIT;
@@ -1016,14 +1022,23 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   if (small > e->pinned_small_cap) {
     if (e->pinned_small) HIPCHK(hipHostFree(e->pinned_small));
     e->pinned_small = nullptr;
+    e->pinned_small_cap = 0;
     HIPCHK(hipHostMalloc(&e->pinned_small, small * 2 + 4096, hipHostMallocDefault));
     e->pinned_small_cap = small * 2 + 4096;
+    void* d = nullptr;
+    HIPCHK(hipHostGetDevicePointer(&d, e->pinned_small, 0));
+    e->pinned_small_dev = static_cast<char*>(d);
   }
-  memcpy(e->pinned_small, prefix.data(), prefix.size());
-  memcpy(static_cast<char*>(e->pinned_small) + prefix.size(), suffix.data(), suffix.size());
-  HIPCHK(hipMemcpyAsync(e->out.p, e->pinned_small, prefix.size(), hipMemcpyHostToDevice, st));
-  HIPCHK(hipMemcpyAsync(e->out.as<char>() + prefix.size() + act_bytes, static_cast<char*>(e->pinned_small) + prefix.size(),
-                        suffix.size(), hipMemcpyHostToDevice, st));
+  {
+    char* dst_a = e->out.as<char>();
+    char* dst_b = dst_a + prefix.size() + act_bytes;
+    const size_t at_a = (size_t)(((uintptr_t)dst_a - (uintptr_t)e->pinned_small_dev) & 15u);
+    const size_t after_a = (at_a + prefix.size() + 15u) & ~(size_t)15u;
+    const size_t at_b = after_a + (size_t)(((uintptr_t)dst_b - (uintptr_t)(e->pinned_small_dev + after_a)) & 15u);
+    memcpy(static_cast<char*>(e->pinned_small) + at_a, prefix.data(), prefix.size());
+    memcpy(static_cast<char*>(e->pinned_small) + at_b, suffix.data(), suffix.size());
+    HIPCHK(put_text(e->pinned_small_dev + at_a, dst_a, prefix.size(), e->pinned_small_dev + at_b, dst_b, suffix.size(), st));
+  }
   const uint32_t tile = emit_tile_bytes(act_bytes, e->scalars.n_valid);
   NEED(e->tile_start, (emit_tile_count(e->prefix_len, act_bytes, tile) + 2) * 4);
   HIPCHK(hipEventRecord(e->ev[EV_EMIT_START], st));

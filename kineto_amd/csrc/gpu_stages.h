@@ -158,6 +158,12 @@ struct ApiTable {
   uint32_t malloc_cid;
 };
 
+/* read-backs and text of a pass without the copy engine: sc, *total (may be null) and list[0..n_list)
+ * into pinned host memory (device-visible addresses); two pieces of host text to their places in the
+ * document (source and destination of a piece must agree modulo 16) */
+hipError_t publish(const Scalars* sc, const uint64_t* total, const uint32_t* list, uint32_t n_list, Scalars* h_sc,
+                   uint64_t* h_total, uint32_t* h_list, hipStream_t st);
+hipError_t put_text(const char* src_a, char* dst_a, uint64_t n_a, const char* src_b, char* dst_b, uint64_t n_b, hipStream_t st);
 /* ---- utilities ---- */
 hipError_t fill_u64(uint64_t* p, uint64_t v, uint64_t n, hipStream_t st);
 hipError_t fill_u32(uint32_t* p, uint32_t v, uint64_t n, hipStream_t st);

@@ -305,34 +305,47 @@ __global__ void k_scan_final(const uint32_t* in, uint64_t n, const uint64_t* sum
   if (write_total && blockIdx.x == 0 && threadIdx.x == 0) out[n] = (OutT)sums[m];
 }
 
-/* small inputs: the whole scan in one workgroup, tile after tile with a running carry */
-#define SCAN_SMALL_TILES 16u
+/* small inputs (one tile of SCAN_SMALL_THREADS lanes): the whole scan in one workgroup and one pass.
+ * More tiles in one workgroup measured slower than the three launches over many workgroups. */
+#define SCAN_SMALL_THREADS 1024u
+#define SCAN_SMALL_MAX (SCAN_SMALL_THREADS * SCAN_ITEMS)
 template <typename OutT>
-__global__ void k_scan_small(const uint32_t* in, uint64_t n, OutT* out, bool write_total) {
-  __shared__ uint64_t lds_wave[KTJ_BLOCK >> 6];
-  uint64_t carry = 0;
-  for (uint64_t tile = 0; tile < n; tile += SCAN_TILE) {
-    const uint64_t base = tile + (uint64_t)threadIdx.x * SCAN_ITEMS;
-    uint32_t v[SCAN_ITEMS];
-    uint64_t s = 0;
-    for (int k = 0; k < SCAN_ITEMS; ++k) { v[k] = base + k < n ? in[base + k] : 0u; s += v[k]; }
-    uint64_t tot;
-    uint64_t ex = block_exclusive_scan_u64(s, lds_wave, &tot) + carry;
-    for (int k = 0; k < SCAN_ITEMS; ++k) { /* a lane reads its items before it writes them: in place is fine */
-      if (base + k < n) out[base + k] = (OutT)ex;
-      ex += v[k];
-    }
-    carry += tot;
+__global__ void __launch_bounds__(SCAN_SMALL_THREADS) k_scan_small(const uint32_t* in, uint64_t n, OutT* out, bool write_total) {
+  __shared__ uint64_t wave_sum[SCAN_SMALL_THREADS >> 6];
+  const uint64_t base = (uint64_t)threadIdx.x * SCAN_ITEMS;
+  uint32_t v[SCAN_ITEMS];
+  uint64_t s = 0;
+#pragma unroll
+  for (int k = 0; k < SCAN_ITEMS; ++k) { v[k] = base + k < n ? in[base + k] : 0u; s += v[k]; }
+  unsigned long long x = s; /* inclusive scan inside the wavefront, then over the wavefronts' sums */
+  for (int o = 1; o < 64; o <<= 1) {
+    const unsigned long long y = __shfl_up(x, (unsigned)o);
+    if ((int)lane_id() >= o) x += y;
   }
-  if (write_total && threadIdx.x == 0) out[n] = (OutT)carry;
+  const uint32_t w = threadIdx.x >> 6;
+  if (lane_id() == 63) wave_sum[w] = x;
+  __syncthreads();
+  uint64_t before = 0, tot = 0;
+  for (uint32_t k = 0; k < (SCAN_SMALL_THREADS >> 6); ++k) {
+    const uint64_t t = wave_sum[k];
+    if (k < w) before += t;
+    tot += t;
+  }
+  uint64_t ex = before + x - s;
+#pragma unroll
+  for (int k = 0; k < SCAN_ITEMS; ++k) { /* a lane reads and writes its own items only: in place is fine */
+    if (base + k < n) out[base + k] = (OutT)ex;
+    ex += v[k];
+  }
+  if (write_total && threadIdx.x == 0) out[n] = (OutT)tot;
 }
 
 uint64_t scan_tmp_elems(uint64_t n) { return (n + SCAN_TILE - 1) / SCAN_TILE + 2; }
 
 hipError_t scan_u32_to_u64(const uint32_t* in, uint64_t* out, uint64_t n, uint64_t* tmp, hipStream_t st) {
   const uint64_t m = (n + SCAN_TILE - 1) / SCAN_TILE;
-  if (m <= SCAN_SMALL_TILES) {
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(k_scan_small<uint64_t>), dim3(1), dim3(KTJ_BLOCK), 0, st, in, n, out, true);
+  if (n <= SCAN_SMALL_MAX) {
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(k_scan_small<uint64_t>), dim3(1), dim3(SCAN_SMALL_THREADS), 0, st, in, n, out, true);
     return KTJ_LAUNCH_CHECK();
   }
   if (m > 0) hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st, in, n, tmp);
@@ -347,8 +360,8 @@ hipError_t scan_u32_to_u64(const uint32_t* in, uint64_t* out, uint64_t n, uint64
 hipError_t scan_u32_inplace(uint32_t* data, uint64_t n, uint64_t* tmp, hipStream_t st) {
   const uint64_t m = (n + SCAN_TILE - 1) / SCAN_TILE;
   if (m == 0) return hipSuccess;
-  if (m <= SCAN_SMALL_TILES) {
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(k_scan_small<uint32_t>), dim3(1), dim3(KTJ_BLOCK), 0, st, (const uint32_t*)data, n, data, false);
+  if (n <= SCAN_SMALL_MAX) {
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(k_scan_small<uint32_t>), dim3(1), dim3(SCAN_SMALL_THREADS), 0, st, (const uint32_t*)data, n, data, false);
     return KTJ_LAUNCH_CHECK();
   }
   hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st, (const uint32_t*)data, n, tmp);
@@ -1367,8 +1380,8 @@ hipError_t make_rank_keys(Columns c, const uint32_t* order, uint64_t n, SortSets
 
 hipError_t collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  /* few, fat workgroups: each one pays for its own local set once */
-  const unsigned g = grid_stride_for(n, KTJ_BLOCK * 16);
+  /* few, fat workgroups: each one pays for its own local set once (few rows: one group each) */
+  const unsigned g = grid_stride_for(n, n < (1u << 20) ? KTJ_BLOCK * COLLECT_ROWS : KTJ_BLOCK * 16);
   hipLaunchKernelGGL(k_collect_distinct, dim3(g), dim3(KTJ_BLOCK), 0, st, c, n, s, sc);
   return KTJ_LAUNCH_CHECK();
 }
@@ -1915,21 +1928,22 @@ __device__ __forceinline__ bool bitmap_test_and_set(uint32_t* bitmap, uint32_t s
   return active && (twice || (old & bit) != 0);
 }
 #define JOIN_ROWS 4
+#define JOIN_SMALL_ROWS (1u << 18)
 #ifndef KX_JOIN_ATTR
 #define KX_JOIN_ATTR
 #endif
 __global__ void KX_JOIN_ATTR k_join_runtime(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first_runtime, ApiTable api, Table tf,
                                FullCols fc, Table tn, NarrowCols nc, uint32_t* slot_f, uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
-                               uint32_t* len, Scalars* sc) {
+                               uint32_t* len, Scalars* sc, int rounds) {
   RowStats rs;
   uint32_t n_linked = 0;
   bool any_carries_stream = false, any_repeats = false;
-  /* a workgroup takes JOIN_ROWS consecutive groups of blockDim.x rows: the per-workgroup counters
+  /* a workgroup takes `rounds` consecutive groups of blockDim.x rows: the per-workgroup counters
    * at the end (one atomic each on a hot address) are paid once for all of them */
   static_assert(sizeof(MatRow) == sizeof(ktj_runtime_rec), "the staging area holds the records, then the joined rows");
   __shared__ uint4 stage[KTJ_BLOCK * sizeof(ktj_runtime_rec) / 16];
-  for (int round = 0; round < JOIN_ROWS; ++round) {
-    const uint64_t base = ((uint64_t)blockIdx.x * JOIN_ROWS + round) * blockDim.x;
+  for (int round = 0; round < rounds; ++round) {
+    const uint64_t base = ((uint64_t)blockIdx.x * rounds + round) * blockDim.x;
     if (base >= n) break;
     const uint32_t cnt = (uint32_t)(n - base < blockDim.x ? n - base : blockDim.x);
     __syncthreads(); /* the previous round's rows have left the staging area */
@@ -2142,8 +2156,10 @@ hipError_t join_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, ui
                              Table tn, NarrowCols nc, uint32_t* slot_f, uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
                              uint32_t* len, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_join_runtime, dim3(grid_for(n, KTJ_BLOCK * JOIN_ROWS)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, tf, fc, tn, nc,
-                     slot_f, slot_n, ctx, mat, len, sc);
+  /* few rows: one group per workgroup, so that the launch is as wide and as short as it can be */
+  const int rounds = n < JOIN_SMALL_ROWS ? 1 : JOIN_ROWS;
+  hipLaunchKernelGGL(k_join_runtime, dim3(grid_for(n, KTJ_BLOCK * rounds)), dim3(KTJ_BLOCK), 0, st, r, n, c, first, api, tf, fc, tn, nc,
+                     slot_f, slot_n, ctx, mat, len, sc, rounds);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t republish_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, FullCols fc, NarrowCols nc,
@@ -2315,6 +2331,49 @@ hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* 
   const size_t stage_lds = (size_t)KTJ_BLOCK * KTJ_STAGE_BLOCKS * 16u;
   hipLaunchKernelGGL(k_emit_direct, dim3(grid_for(n_rows, KTJ_BLOCK)), dim3(KTJ_BLOCK), stage_lds, st, mat, perm, offs,
                      kind_sorted, n_rows, ctx, out, prefix_len);
+  return KTJ_LAUNCH_CHECK();
+}
+
+/* What the host needs during a pass goes straight into its pinned memory, and the text it made
+ * (header, infos, footer) comes straight out of it: one small kernel each instead of one copy
+ * engine transfer per value. */
+__global__ void k_publish(const Scalars* sc, const uint64_t* total, const uint32_t* list, uint32_t n_list, Scalars* h_sc,
+                          uint64_t* h_total, uint32_t* h_list) {
+  const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x, stride = gridDim.x * blockDim.x;
+  static_assert(sizeof(Scalars) % 4 == 0, "copied as 32-bit words");
+  const uint32_t* src = reinterpret_cast<const uint32_t*>(sc);
+  uint32_t* dst = reinterpret_cast<uint32_t*>(h_sc);
+  for (uint32_t k = t; k < sizeof(Scalars) / 4; k += stride) dst[k] = src[k];
+  for (uint32_t k = t; k < n_list; k += stride) h_list[k] = list[k];
+  if (t == 0 && total != nullptr) *h_total = *total;
+  __threadfence_system();
+}
+hipError_t publish(const Scalars* sc, const uint64_t* total, const uint32_t* list, uint32_t n_list, Scalars* h_sc,
+                   uint64_t* h_total, uint32_t* h_list, hipStream_t st) {
+  hipLaunchKernelGGL(k_publish, dim3(n_list > 4096 ? 16 : 1), dim3(KTJ_BLOCK), 0, st, sc, total, list, n_list, h_sc, h_total, h_list);
+  return KTJ_LAUNCH_CHECK();
+}
+/* two pieces of text, each to its place; source and destination of a piece agree modulo 16 */
+__global__ void k_put_text(const char* src_a, char* dst_a, uint64_t n_a, const char* src_b, char* dst_b, uint64_t n_b) {
+  const char* src = blockIdx.y ? src_b : src_a;
+  char* dst = blockIdx.y ? dst_b : dst_a;
+  const uint64_t n = blockIdx.y ? n_b : n_a;
+  uint64_t head = (16u - (uint32_t)((uintptr_t)dst & 15u)) & 15u;
+  if (head > n) head = n;
+  const uint64_t body = (n - head) >> 4, tail = (n - head) & 15u;
+  const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  if (t < head) dst[t] = src[t];
+  const uint4* sv = reinterpret_cast<const uint4*>(src + head);
+  uint4* dv = reinterpret_cast<uint4*>(dst + head);
+  for (uint64_t k = t; k < body; k += stride) dv[k] = sv[k];
+  if (t < tail) dst[head + body * 16u + t] = src[head + body * 16u + t];
+}
+hipError_t put_text(const char* src_a, char* dst_a, uint64_t n_a, const char* src_b, char* dst_b, uint64_t n_b, hipStream_t st) {
+  if ((((uintptr_t)src_a ^ (uintptr_t)dst_a) & 15u) || (((uintptr_t)src_b ^ (uintptr_t)dst_b) & 15u)) return hipErrorInvalidValue;
+  const uint64_t most = n_a > n_b ? n_a : n_b;
+  if (most == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_put_text, dim3(grid_stride_for((most >> 4) + 1, KTJ_BLOCK), 2), dim3(KTJ_BLOCK), 0, st, src_a, dst_a, n_a, src_b,
+                     dst_b, n_b);
   return KTJ_LAUNCH_CHECK();
 }
 
