@@ -199,6 +199,23 @@ def test_limits_end_in_a_named_error():
     _engine_vs_oracle(_many_ids_builder(10, 1, n_streams=KTJ_MAX_STREAM_PAIRS - 96).build())
 
 
+def test_header_text_beyond_the_pinned_staging_buffer():
+    """Thousands of resource infos make the text around the activities larger than the engine's
+    256 KiB pinned staging buffer: the buffer grows and the text still lands byte for byte
+    (both pieces, whatever the alignment of the place after the activities)."""
+    from stream_builder import StreamBuilder, B
+    for extra in (0, 1, 7, 9):  # shifts the suffix to different positions modulo 16
+        print(f"large header, name length +{extra}", flush=True)
+        b = StreamBuilder(host_name="big" + "x" * extra)
+        b.api(["hipLaunchKernel"], flow_start=[0])
+        for k in range(4000):
+            b.add_resource_info(100 + k, 100 + k, 7, "worker thread %d" % k, host_thread=(k % 2 == 0))
+        for k in range(50):
+            b.add_generic("op%d" % (k % 3), 0, B + 1000 + 10 * k, B + 1005 + 10 * k, 7, 100 + k, id=k + 1)
+        b.add_span(B, B + 10**6, 50, 0, "PyTorch Profiler")
+        _engine_vs_oracle(b.build())
+
+
 def test_golden_digests_on_gpu():
     """The engine's document against the committed digests (tests/golden/digests.json, written where
     the checker's output had just been compared byte for byte with the reference logger's): no
