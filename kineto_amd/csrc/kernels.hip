@@ -244,7 +244,19 @@ hipError_t scratch_address(int device, void** ptr, size_t* bytes) {
 #define SCAN_ITEMS 8
 #define SCAN_TILE (KTJ_BLOCK * SCAN_ITEMS)
 
-__device__ __forceinline__ uint64_t block_exclusive_scan_u64(uint64_t v, uint64_t* lds_wave /* 4 */, uint64_t* total) {
+#define SCAN_MAX_WAVES 16 /* workgroups of up to 1024 lanes */
+/* a lane's SCAN_ITEMS consecutive values: two 16-byte loads where the whole run is inside the input
+ * (the inputs are 16-byte aligned device buffers), single values at the end */
+__device__ __forceinline__ void scan_load_items(const uint32_t* in, uint64_t n, uint64_t base, uint32_t (&v)[SCAN_ITEMS]) {
+  static_assert(SCAN_ITEMS == 8, "two uint4 per lane");
+  if (base + SCAN_ITEMS <= n) {
+    const uint4 a = *reinterpret_cast<const uint4*>(in + base), b = *reinterpret_cast<const uint4*>(in + base + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  } else {
+    for (int k = 0; k < SCAN_ITEMS; ++k) v[k] = base + k < n ? in[base + k] : 0u;
+  }
+}
+__device__ __forceinline__ uint64_t block_exclusive_scan_u64(uint64_t v, uint64_t* lds_wave /* SCAN_MAX_WAVES */, uint64_t* total) {
   /* inclusive scan inside the wave */
   unsigned long long x = v;
   for (int o = 1; o < 64; o <<= 1) {
@@ -255,7 +267,7 @@ __device__ __forceinline__ uint64_t block_exclusive_scan_u64(uint64_t v, uint64_
   if (lane_id() == 63) lds_wave[w] = x;
   __syncthreads();
   uint64_t base = 0, tot = 0;
-  for (uint32_t k = 0; k < (KTJ_BLOCK >> 6); ++k) {
+  for (uint32_t k = 0; k < (blockDim.x >> 6); ++k) {
     const uint64_t s = lds_wave[k];
     if (k < w) base += s;
     tot += s;
@@ -266,19 +278,21 @@ __device__ __forceinline__ uint64_t block_exclusive_scan_u64(uint64_t v, uint64_
 }
 
 __global__ void k_scan_sums(const uint32_t* in, uint64_t n, uint64_t* sums) {
-  __shared__ uint64_t lds_wave[KTJ_BLOCK >> 6];
+  __shared__ uint64_t lds_wave[SCAN_MAX_WAVES];
   const uint64_t base = (uint64_t)blockIdx.x * SCAN_TILE + (uint64_t)threadIdx.x * SCAN_ITEMS;
+  uint32_t v[SCAN_ITEMS];
+  scan_load_items(in, n, base, v);
   uint64_t s = 0;
-  for (int k = 0; k < SCAN_ITEMS; ++k) if (base + k < n) s += in[base + k];
+  for (int k = 0; k < SCAN_ITEMS; ++k) s += v[k];
   uint64_t tot;
   block_exclusive_scan_u64(s, lds_wave, &tot);
   if (threadIdx.x == 0) sums[blockIdx.x] = tot;
 }
 /* one block: sums[0..m) → exclusive prefix in place, grand total → sums[m] */
 __global__ void k_scan_of_sums(uint64_t* sums, uint64_t m) {
-  __shared__ uint64_t lds_wave[KTJ_BLOCK >> 6];
+  __shared__ uint64_t lds_wave[SCAN_MAX_WAVES];
   uint64_t carry = 0;
-  for (uint64_t base = 0; base < m; base += KTJ_BLOCK) {
+  for (uint64_t base = 0; base < m; base += blockDim.x) {
     const uint64_t i = base + threadIdx.x;
     const uint64_t v = i < m ? sums[i] : 0;
     uint64_t tot;
@@ -291,16 +305,30 @@ __global__ void k_scan_of_sums(uint64_t* sums, uint64_t m) {
 template <typename OutT>
 __global__ void k_scan_final(const uint32_t* in, uint64_t n, const uint64_t* sums, uint64_t m, OutT* out,
                              bool write_total) {
-  __shared__ uint64_t lds_wave[KTJ_BLOCK >> 6];
+  __shared__ uint64_t lds_wave[SCAN_MAX_WAVES];
   const uint64_t base = (uint64_t)blockIdx.x * SCAN_TILE + (uint64_t)threadIdx.x * SCAN_ITEMS;
   uint32_t v[SCAN_ITEMS];
+  scan_load_items(in, n, base, v);
   uint64_t s = 0;
-  for (int k = 0; k < SCAN_ITEMS; ++k) { v[k] = base + k < n ? in[base + k] : 0u; s += v[k]; }
+  for (int k = 0; k < SCAN_ITEMS; ++k) s += v[k];
   uint64_t tot;
   uint64_t ex = block_exclusive_scan_u64(s, lds_wave, &tot) + sums[blockIdx.x];
-  for (int k = 0; k < SCAN_ITEMS; ++k) {
-    if (base + k < n) out[base + k] = (OutT)ex;
-    ex += v[k];
+  if (base + SCAN_ITEMS <= n) { /* the lane's run as 16-byte stores (the outputs are 16-byte aligned device buffers) */
+    OutT r[SCAN_ITEMS];
+    for (int k = 0; k < SCAN_ITEMS; ++k) { r[k] = (OutT)ex; ex += v[k]; }
+    constexpr int PER = 16 / sizeof(OutT);
+    typedef OutT vec __attribute__((ext_vector_type(PER)));
+    vec* dst = reinterpret_cast<vec*>(out + base);
+    for (int q = 0; q < SCAN_ITEMS / PER; ++q) {
+      vec x;
+      for (int j = 0; j < PER; ++j) x[j] = r[q * PER + j];
+      dst[q] = x;
+    }
+  } else {
+    for (int k = 0; k < SCAN_ITEMS; ++k) {
+      if (base + k < n) out[base + k] = (OutT)ex;
+      ex += v[k];
+    }
   }
   if (write_total && blockIdx.x == 0 && threadIdx.x == 0) out[n] = (OutT)sums[m];
 }
@@ -349,7 +377,7 @@ hipError_t scan_u32_to_u64(const uint32_t* in, uint64_t* out, uint64_t n, uint64
     return KTJ_LAUNCH_CHECK();
   }
   if (m > 0) hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st, in, n, tmp);
-  hipLaunchKernelGGL(k_scan_of_sums, dim3(1), dim3(KTJ_BLOCK), 0, st, tmp, m);
+  hipLaunchKernelGGL(k_scan_of_sums, dim3(1), dim3(m > KTJ_BLOCK ? 1024 : KTJ_BLOCK), 0, st, tmp, m);
   if (m > 0)
     hipLaunchKernelGGL(HIP_KERNEL_NAME(k_scan_final<uint64_t>), dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st, in, n,
                        (const uint64_t*)tmp, m, out, true);
@@ -365,7 +393,7 @@ hipError_t scan_u32_inplace(uint32_t* data, uint64_t n, uint64_t* tmp, hipStream
     return KTJ_LAUNCH_CHECK();
   }
   hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st, (const uint32_t*)data, n, tmp);
-  hipLaunchKernelGGL(k_scan_of_sums, dim3(1), dim3(KTJ_BLOCK), 0, st, tmp, m);
+  hipLaunchKernelGGL(k_scan_of_sums, dim3(1), dim3(m > KTJ_BLOCK ? 1024 : KTJ_BLOCK), 0, st, tmp, m);
   /* every block reads its tile completely before writing it, and tiles do not overlap */
   hipLaunchKernelGGL(HIP_KERNEL_NAME(k_scan_final<uint32_t>), dim3((unsigned)m), dim3(KTJ_BLOCK), 0, st,
                      (const uint32_t*)data, n, (const uint64_t*)tmp, m, data, false);
