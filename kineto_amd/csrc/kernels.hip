@@ -1890,16 +1890,30 @@ hipError_t stream_sync_first(const uint32_t* perm, uint64_t n_sorted, const ktj_
 
 __global__ void k_mat_generic(const ktj_generic_rec* g, uint64_t n, uint64_t first, EmitCtx ctx, const uint32_t* sync_first,
                               MatRow* mat, uint32_t* len, Scalars* sc) {
+  static_assert(sizeof(MatRow) >= sizeof(ktj_generic_rec), "the staging area holds the records, then the joined rows");
+  __shared__ uint4 stage[KTJ_BLOCK * sizeof(MatRow) / 16];
   RowStats rs;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    const ktj_generic_rec rec = g[i];
-    MatRow m = mat_generic(rec, generic_device(rec, ctx.args, ctx.n_args));
-    if (!generic_record_prints(rec, ctx)) m.meta &= ~KTJ_M_VALID;
-    attach_own_collective(m, rec, ctx);
-    mark_stream_sync(m, ctx, sync_first != nullptr && sync_first[i] != 0);
-    store_row(&mat[first + i], m);
-    len[first + i] = row_length(m, ctx, sc);
-    count_row_stats(m, ctx, &rs);
+  for (uint64_t base = (uint64_t)blockIdx.x * blockDim.x; base < n; base += (uint64_t)gridDim.x * blockDim.x) {
+    const uint32_t cnt = (uint32_t)(n - base < blockDim.x ? n - base : blockDim.x);
+    __syncthreads(); /* the previous round's rows have left the staging area */
+    rows_global_to_lds(g + base, cnt, stage);
+    __syncthreads();
+    const uint64_t i = base + threadIdx.x;
+    const bool active = threadIdx.x < cnt;
+    MatRow m;
+    if (active) {
+      const ktj_generic_rec rec = row_from_lds<ktj_generic_rec>(stage);
+      m = mat_generic(rec, generic_device(rec, ctx.args, ctx.n_args));
+      if (!generic_record_prints(rec, ctx)) m.meta &= ~KTJ_M_VALID;
+      attach_own_collective(m, rec, ctx);
+      mark_stream_sync(m, ctx, sync_first != nullptr && sync_first[i] != 0);
+      len[first + i] = row_length(m, ctx, sc);
+      count_row_stats(m, ctx, &rs);
+    }
+    __syncthreads(); /* every lane has taken its record */
+    if (active) row_to_lds(m, stage);
+    __syncthreads();
+    rows_lds_to_global(mat + first + base, cnt, stage);
   }
   flush_row_stats(rs, sc);
 }
