@@ -1607,7 +1607,8 @@ k_sortp_make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t
     }
   }
   __syncthreads();
-  for (int d = threadIdx.x; d < P::NB; d += THREADS) hist[(uint64_t)d * n_blocks + blockIdx.x] = h[d]; /* digit-major */
+  if (hist != nullptr)
+    for (int d = threadIdx.x; d < P::NB; d += THREADS) hist[(uint64_t)d * n_blocks + blockIdx.x] = h[d]; /* digit-major */
 }
 template <int BITS, int THREADS>
 __global__ void __launch_bounds__(THREADS)
@@ -1639,7 +1640,7 @@ k_sortp_scatter(const uint64_t* in, uint64_t* words_out, uint32_t* perm_out, uin
   __shared__ uint32_t base_of[P::NB];            /* global offset of this tile's run per digit   */
   __shared__ uint32_t wave_tot[P::WAVES];
   for (int d = threadIdx.x; d < P::NB; d += THREADS) {
-    base_of[d] = hist_scanned[(uint64_t)d * n_blocks + blockIdx.x];
+    base_of[d] = hist_scanned != nullptr ? hist_scanned[(uint64_t)d * n_blocks + blockIdx.x] : 0u;
     for (int k = 0; k < P::WAVES; ++k) wave_run[k][d] = 0;
   }
   __syncthreads();
@@ -1727,7 +1728,8 @@ k_sortp_scatter(const uint64_t* in, uint64_t* words_out, uint32_t* perm_out, uin
   for (uint32_t p = threadIdx.x; p < cnt; p += THREADS) {
     const uint64_t v = s_word[p];
     const uint32_t digit = FROM_KEYS ? (uint32_t)s_digit[p] : ((uint32_t)(v >> shift) & (P::NB - 1u));
-    const uint64_t dst = (uint64_t)base_of[digit] + (p - digit_start[digit]);
+    /* a single tile (no counts given): the tile's order is the output's */
+    const uint64_t dst = hist_scanned != nullptr ? (uint64_t)base_of[digit] + (p - digit_start[digit]) : (uint64_t)p;
     if (TO_PERM) perm_out[dst] = (uint32_t)(v & idx_mask);
     else words_out[dst] = v;
   }
@@ -1742,28 +1744,33 @@ static hipError_t sort_packed_t(Columns c, uint64_t n, SortSets s, const Scalars
   const uint32_t total_bits = key_bits + 1u;
   const uint32_t passes = (total_bits + BITS - 1) / BITS;
   const dim3 g(n_blocks), b(THREADS);
-  hipLaunchKernelGGL((k_sortp_make_keys<BITS, THREADS>), g, b, 0, st, c, n, s, sc, ts_bits, res_bits, key_bits, buf_a, hist, n_blocks);
-  hipError_t e = scan_u32_inplace(hist, (uint64_t)P::NB * n_blocks, scan_tmp, st);
+  /* one tile: a pass needs no counts from other tiles, so no count and scan launches */
+  const bool single = n_blocks == 1;
+  uint32_t* counts = single ? nullptr : hist;
+  hipLaunchKernelGGL((k_sortp_make_keys<BITS, THREADS>), g, b, 0, st, c, n, s, sc, ts_bits, res_bits, key_bits, buf_a, counts, n_blocks);
+  hipError_t e = single ? hipSuccess : scan_u32_inplace(hist, (uint64_t)P::NB * n_blocks, scan_tmp, st);
   if (e != hipSuccess) return e;
   if (passes == 1) {
     hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_KEYS_TO_PERM>), g, b, 0, st, (const uint64_t*)buf_a, buf_b, perm, n,
-                       0u, idx_bits, (const uint32_t*)hist, n_blocks);
+                       0u, idx_bits, (const uint32_t*)counts, n_blocks);
     return KTJ_LAUNCH_CHECK();
   }
   hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_KEYS_TO_WORDS>), g, b, 0, st, (const uint64_t*)buf_a, buf_b, perm, n,
-                     0u, idx_bits, (const uint32_t*)hist, n_blocks);
+                     0u, idx_bits, (const uint32_t*)counts, n_blocks);
   uint64_t* in = buf_b; uint64_t* out = buf_a;
   for (uint32_t p = 1; p < passes; ++p) {
     const uint32_t shift = idx_bits + (p - 1u) * BITS;
-    hipLaunchKernelGGL((k_sortp_hist<BITS, THREADS>), g, b, 0, st, (const uint64_t*)in, n, shift, hist, n_blocks);
-    e = scan_u32_inplace(hist, (uint64_t)P::NB * n_blocks, scan_tmp, st);
-    if (e != hipSuccess) return e;
+    if (!single) {
+      hipLaunchKernelGGL((k_sortp_hist<BITS, THREADS>), g, b, 0, st, (const uint64_t*)in, n, shift, hist, n_blocks);
+      e = scan_u32_inplace(hist, (uint64_t)P::NB * n_blocks, scan_tmp, st);
+      if (e != hipSuccess) return e;
+    }
     if (p + 1 == passes)
       hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_WORDS_TO_PERM>), g, b, 0, st, (const uint64_t*)in, out, perm, n,
-                         shift, idx_bits, (const uint32_t*)hist, n_blocks);
+                         shift, idx_bits, (const uint32_t*)counts, n_blocks);
     else
       hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_WORDS_TO_WORDS>), g, b, 0, st, (const uint64_t*)in, out, perm, n,
-                         shift, idx_bits, (const uint32_t*)hist, n_blocks);
+                         shift, idx_bits, (const uint32_t*)counts, n_blocks);
     uint64_t* t = in; in = out; out = t;
   }
   return KTJ_LAUNCH_CHECK();
