@@ -803,6 +803,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   ctx.n_schemas = (uint32_t)e->schemas.size();
   ctx.args = e->args.buf.as<uint64_t>(); ctx.n_args = e->n_args;
   ctx.base_time_ns = e->base_time_ns;
+  ctx.create_flags = e->flags;
   /* collective metadata is looked at only if both entries and a schema that refers to them exist */
   const uint32_t n_coll = e->coll_schemas ? (uint32_t)e->collectives.size() : 0u;
   if (n_coll && e->coll_dirty) {
@@ -1127,6 +1128,9 @@ int ktj_process_noalloc(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   e->noalloc = true;
   const int rc = process_pass(e, end_time_ns, out_device, out_capacity);
   e->noalloc = false;
+  /* The small tables of this pass sit in the scratch array, which every engine on this GPU shares:
+   * whatever the pass returned, the next allocating pass must upload them into its own buffers again. */
+  e->schemas_dirty = e->api_dirty = e->coll_dirty = true;
   if (n_bytes) *n_bytes = e->total_bytes; /* on KTJ_ERR_LIMIT for a short output buffer: the size that is needed */
   return rc;
 }

@@ -20,7 +20,10 @@ def test_noalloc_matches_process_on_two_calls_in_a_row():
     import torch
     import oracle_glue as og
     from kineto_amd.engine import TraceEngine
-    cases = [(3, 20000), (4, 3000)]            # the second input is smaller and of another shape
+    # The second input is smaller and of another shape; its args schema, API-name table and strings
+    # differ from the first one's, so an engine that went on using the small tables a later call of
+    # the other engine left in the shared scratch array would format a different document.
+    cases = [(3, 20000), (5, 1500)]
     streams, engines, wants = [], [], []
     for cfg, n in cases:
         sp, release = abi.synth_stream(cfg, n, host_name="gpubox")
@@ -54,7 +57,9 @@ def test_noalloc_matches_process_on_two_calls_in_a_row():
         assert got[k] == len(want)
         doc = bytes(out[:got[k]].cpu().numpy())
         assert bytes(out[got[k] + 64:].cpu().numpy()) == b"\xEE" * (out.numel() - got[k] - 64), "wrote beyond the document + 64 bytes"
-        eng.process()                          # the existing entry point, same engine, same records
+        # the existing entry point, same engine, same records; the last call on this GPU's scratch
+        # array was the other engine's, so this pass must bring its own small tables
+        eng.process()
         ref = eng.output()
         assert doc == ref, f"call {k}: ktj_process_noalloc differs from ktj_process"
         assert doc == want, f"call {k}: differs from the CPU checker"
