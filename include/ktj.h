@@ -208,14 +208,14 @@ enum {
 
 /*
  * Device (asynchronous) row: rocprofAsyncRow (libkineto/src/RocLogger.h:216-240).  The kernel
- * name std::string becomes a string id.  For KTJ_DOM_MEMSET rows `queue` carries the context id
- * and `stream` must be set by the producer (no back-fill).
+ * name std::string becomes a string id.  A KTJ_DOM_MEMSET row is read through ktj_memset_rec below.
  */
 typedef struct ktj_device_rec {
   uint64_t id;       /* correlation id                                                        */
   uint64_t begin;    /* device clock                                                          */
   uint64_t end;
-  uint32_t domain;   /* KTJ_DOM_*                                                             */
+  uint32_t domain;   /* KTJ_DOM_* in the low 16 bits (KTJ_ROW_DOMAIN); the upper 16 bits are read
+                        on memset rows only                                                   */
   uint32_t op;       /* KTJ_COPY_* for copies                                                 */
   int32_t device;
   uint32_t name_id;  /* kernel name, KTJ_NONE = empty                                         */
@@ -223,6 +223,52 @@ typedef struct ktj_device_rec {
   uint64_t stream;   /* 0 = unknown: back-filled from the correlated runtime row              */
   uint64_t bytes;    /* KTJ_DOM_MEMSET only                                                   */
 } ktj_device_rec;    /* 64 bytes */
+#define KTJ_ROW_DOMAIN(raw) ((uint32_t)(raw) & 0xFFFFu)
+
+/*
+ * The KTJ_DOM_MEMSET view of a device row: the fields of CUpti_ActivityMemset4 that
+ * GpuActivity<CUpti_ActivityMemsetType> reads (libkineto/src/CuptiActivity.h:682-719, with
+ * :424-458 for the graph and channel keys).  Same 64 bytes as ktj_device_rec, member by member:
+ * `domain` splits into domain / channel_type / memory_kind, `op` and `name_id` hold the two halves
+ * of the graph node id, `queue` holds context and channel id, `stream` holds stream and graph id.
+ * No ROCm producer makes such a row (the reference's ROCm GpuActivity never takes the GPU_MEMSET
+ * type, libkineto/src/RocprofActivity.h:84-98); it exists for CUDA-shaped record streams.
+ * The name is "Memset (<memory kind>)" (cupti_strings.cpp:42-66); timestamp() = begin and
+ * duration() = end - begin; the stream is not back-filled.  The args are
+ *   "device", "context", "stream", "correlation", "bytes"[, "memory bandwidth (GB/s)" unless the
+ *   duration is 0] — what a reference built against CUDA < 12 prints — and, in an engine created
+ *   with KTJ_CREATE_CUDA12_ARGS, also "graph id", "graph node id", "channel", "channel_type", as a
+ *   reference built against CUDA >= 12 prints them.
+ */
+typedef struct ktj_memset_rec {
+  uint64_t id;            /* correlationId (32 bits in CUPTI; all 64 are joined and printed)    */
+  uint64_t begin;         /* start                                                              */
+  uint64_t end;
+  uint16_t domain;        /* KTJ_DOM_MEMSET                                                     */
+  uint8_t channel_type;   /* CUpti_ChannelType                                                  */
+  uint8_t memory_kind;    /* CUpti_ActivityMemoryKind: KTJ_MEMKIND_*                            */
+  uint32_t graph_node_lo; /* graphNodeId, low half                                              */
+  int32_t device;         /* deviceId                                                           */
+  uint32_t graph_node_hi; /* graphNodeId, high half                                             */
+  uint32_t context;       /* contextId                                                          */
+  uint32_t channel_id;    /* channelID                                                          */
+  uint32_t stream;        /* streamId                                                           */
+  uint32_t graph_id;      /* graphId                                                            */
+  uint64_t bytes;
+} ktj_memset_rec;         /* 64 bytes */
+
+/* CUpti_ActivityMemoryKind as memoryKindString names it (libkineto/src/cupti_strings.cpp:42-66);
+ * any other value prints "Unrecognized". */
+enum {
+  KTJ_MEMKIND_UNKNOWN = 0,        /* "Unknown"        */
+  KTJ_MEMKIND_PAGEABLE = 1,       /* "Pageable"       */
+  KTJ_MEMKIND_PINNED = 2,         /* "Pinned"         */
+  KTJ_MEMKIND_DEVICE = 3,         /* "Device"         */
+  KTJ_MEMKIND_ARRAY = 4,          /* "Array"          */
+  KTJ_MEMKIND_MANAGED = 5,        /* "Managed"        */
+  KTJ_MEMKIND_DEVICE_STATIC = 6,  /* "Device Static"  */
+  KTJ_MEMKIND_MANAGED_STATIC = 7  /* "Managed Static" */
+};
 
 /* External-correlation pair (libkineto/src/RocmActivityProfiler.cpp:135-148).  Domain 0
  * (KTJ_REC_EXTCORR, cpuCorrelationMap_): correlation id -> CPU-op id, the "External id" link.
@@ -419,12 +465,16 @@ typedef struct ktj_engine ktj_engine;
  * built with DISPLAY_TRACE_IN_NS does (output_json.cpp:451-454); nothing else changes.
  * KTJ_CREATE_PAIR_SORT sorts (key, arrival index) pairs also where key and index fit one 64-bit
  * word (the engine sorts single words then otherwise); same results, slower.
+ * KTJ_CREATE_CUDA12_ARGS prints the "graph id", "graph node id", "channel" and "channel_type" keys
+ * of memset rows (ktj_memset_rec), which the reference compiles in for CUDA >= 12 only
+ * (CuptiActivity.h:424-458).
  * ---------------------------------------------------------------------------------------- */
 #define KTJ_CREATE_NO_FILE 0x1u
 #define KTJ_CREATE_TILE_EMIT 0x2u
 #define KTJ_CREATE_HASH_JOIN 0x4u
 #define KTJ_CREATE_PAIR_SORT 0x8u
 #define KTJ_CREATE_DISPLAY_NS 0x10u
+#define KTJ_CREATE_CUDA12_ARGS 0x20u
 int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int hip_device,
                uint32_t flags);
 void ktj_destroy(ktj_engine* e);

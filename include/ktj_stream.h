@@ -44,7 +44,8 @@ typedef struct ktj_stream {
   const uint32_t* flow_start_cids;
   uint64_t n_flow_start;
   uint32_t malloc_cid;            /* the cid of hipMalloc (its rows carry a "bytes" arg)         */
-  uint32_t pad0;
+  uint32_t create_flags;          /* the ktj_create flags that change the document
+                                     (KTJ_CREATE_CUDA12_ARGS); the engine takes them at ktj_create */
 
   /* clock + window */
   ktj_clock_model clock;

@@ -15,6 +15,7 @@ KTJ_CREATE_TILE_EMIT = 0x2
 KTJ_CREATE_HASH_JOIN = 0x4
 KTJ_CREATE_PAIR_SORT = 0x8
 KTJ_CREATE_DISPLAY_NS = 0x10
+KTJ_CREATE_CUDA12_ARGS = 0x20
 KTJ_GF_WIDE_DEVICE = 0x04
 
 REC_GENERIC, REC_RUNTIME, REC_DEVICE, REC_EXTCORR, REC_USERCORR = 0, 1, 2, 3, 4
@@ -65,6 +66,19 @@ class DeviceRec(C.Structure):
                 ("domain", C.c_uint32), ("op", C.c_uint32), ("device", C.c_int32),
                 ("name_id", C.c_uint32), ("queue", C.c_uint64), ("stream", C.c_uint64),
                 ("bytes", C.c_uint64)]
+
+
+class MemsetRec(C.Structure):
+    """ktj_memset_rec: the KTJ_DOM_MEMSET view of a device row."""
+    _fields_ = [("id", C.c_uint64), ("begin", C.c_uint64), ("end", C.c_uint64),
+                ("domain", C.c_uint16), ("channel_type", C.c_uint8), ("memory_kind", C.c_uint8),
+                ("graph_node_lo", C.c_uint32), ("device", C.c_int32), ("graph_node_hi", C.c_uint32),
+                ("context", C.c_uint32), ("channel_id", C.c_uint32), ("stream", C.c_uint32),
+                ("graph_id", C.c_uint32), ("bytes", C.c_uint64)]
+
+
+KTJ_DOM_MEMSET = 2
+KTJ_MEMKIND_DEVICE = 3
 
 
 class ExtCorrRec(C.Structure):
@@ -134,7 +148,7 @@ class Stream(C.Structure):
                 ("args", C.POINTER(C.c_uint64)), ("n_args", C.c_uint64),
                 ("cid_name_ids", C.POINTER(C.c_uint32)), ("n_cids", C.c_uint64),
                 ("flow_start_cids", C.POINTER(C.c_uint32)), ("n_flow_start", C.c_uint64),
-                ("malloc_cid", C.c_uint32), ("pad0", C.c_uint32),
+                ("malloc_cid", C.c_uint32), ("create_flags", C.c_uint32),
                 ("clock", ClockModel), ("window_start_ns", C.c_int64), ("window_end_ns", C.c_int64),
                 ("end_time_ns", C.c_int64),
                 ("generic", C.POINTER(GenericRec)), ("n_generic", C.c_uint64),

@@ -1092,7 +1092,7 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
     return;
   }
   /* device rows */
-  if (kind == KTJ_DOM_MEMSET) { /* CuptiActivity.h:682-713, 460-470 */
+  if (kind == KTJ_DOM_MEMSET) { /* CuptiActivity.h:682-719, 460-470 */
     KTJ_PUT(w, "\"device\": "); put_i64(w, r.dev);
     KTJ_PUT(w, ", \"context\": "); w.dec(r.p[3]);
     KTJ_PUT(w, ", \"stream\": "); put_i64(w, r.res);
@@ -1102,6 +1102,12 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
       const double bw = (double)r.p[0] / (double)r.dur;
       uint64_t bits; __builtin_memcpy(&bits, &bw, 8);
       KTJ_PUT(w, ", \"memory bandwidth (GB/s)\": "); put_f64(w, bits);
+    }
+    if (c.create_flags & KTJ_CREATE_CUDA12_ARGS) { /* CUDA_VERSION >= 12000: CuptiActivity.h:424-458 */
+      KTJ_PUT(w, ", \"graph id\": "); w.dec(r.p[2] & 0xFFFFFFFFu);
+      KTJ_PUT(w, ", \"graph node id\": "); w.dec(r.p[1]);
+      KTJ_PUT(w, ", \"channel\": "); w.dec(r.p[2] >> 32);
+      KTJ_PUT(w, ", \"channel_type\": "); w.dec(r.aux & 0xFFu);
     }
     return;
   }
@@ -1130,7 +1136,20 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
 template <class W> KTJ_HD KTJ_FI inline void put_name(W& w, const MatRow& r, const EmitCtx& c) {
   if (r.meta & KTJ_M_NAME_BUILTIN) {
     if (r.name_id <= 4) put_memcpy_name(w, r.name_id);
-    else if (r.name_id == KTJ_NAME_MEMSET) KTJ_PUT(w, "Memset (Device)");
+    else if (r.name_id == KTJ_NAME_MEMSET) { /* "Memset ({})" of memoryKindString, cupti_strings.cpp:42-66 */
+      KTJ_PUT(w, "Memset (");
+      switch ((r.aux >> 8) & 0xFFu) {
+        case KTJ_MEMKIND_UNKNOWN: KTJ_PUT(w, "Unknown)"); break;
+        case KTJ_MEMKIND_PAGEABLE: KTJ_PUT(w, "Pageable)"); break;
+        case KTJ_MEMKIND_PINNED: KTJ_PUT(w, "Pinned)"); break;
+        case KTJ_MEMKIND_DEVICE: KTJ_PUT(w, "Device)"); break;
+        case KTJ_MEMKIND_ARRAY: KTJ_PUT(w, "Array)"); break;
+        case KTJ_MEMKIND_MANAGED: KTJ_PUT(w, "Managed)"); break;
+        case KTJ_MEMKIND_DEVICE_STATIC: KTJ_PUT(w, "Device Static)"); break;
+        case KTJ_MEMKIND_MANAGED_STATIC: KTJ_PUT(w, "Managed Static)"); break;
+        default: KTJ_PUT(w, "Unrecognized)"); break;
+      }
+    }
     else if (r.name_id == KTJ_NAME_UNKNOWN_OP) { KTJ_PUT(w, "<unknown operation:"); w.dec(r.aux); w.ch('>'); }
     return;
   }

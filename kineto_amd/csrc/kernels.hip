@@ -598,7 +598,7 @@ __global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns 
   if (threadIdx.x < cnt) {
   const ktj_device_rec* d = &l[threadIdx.x];
   const uint64_t a = first + (uint64_t)blockIdx.x * KTJ_BLOCK + threadIdx.x;
-  const uint32_t dom = d->domain <= KTJ_DOM_MEMSET ? d->domain : KTJ_DOM_KERNEL_DISPATCH;
+  const uint32_t dom = device_row_domain(d->domain);
   uint64_t b = d->begin, e = d->end;
   convert_range(clk, clk.device_mode, &b, &e);
   int64_t ts, dur;
@@ -608,11 +608,11 @@ __global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns 
   c.dur[a] = dur;
   c.corr[a] = d->id;
   c.dev[a] = (int64_t)d->device;
-  c.res[a] = (int64_t)d->stream;
+  c.res[a] = device_row_stream(dom, d->stream);
   c.meta[a] = (KTJ_CLASS_DEVICE << KTJ_M_CLASS_SHIFT) | (dom << KTJ_M_KIND_SHIFT) | (oor ? 0u : KTJ_M_VALID);
   c.ext[a] = 0;
   DevBrief br;
-  br.queue = d->queue; br.device = d->device; br.domain = d->domain;
+  br.queue = d->queue; br.device = d->device; br.domain = dom;
   brief[a - first] = br;
   }
   block_add(&sc->out_of_range, oor);

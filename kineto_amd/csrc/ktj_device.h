@@ -37,7 +37,8 @@ struct MatRow {
  *   device kernel    p0..p2 = grid/block of the launching row (if KTJ_M_HAS_GRID), p3 = queue,
  *                    p4 = 1 + index of the collective metadata of the linked CPU op (0 = none)
  *   device copy      p0 = bytes of the launching row (if KTJ_M_HAS_SIZE), p3 = queue
- *   device memset    p0 = bytes, p3 = context id
+ *   device memset    p0 = bytes, p1 = graph node id, p2 = graph id | channel id<<32, p3 = context id;
+ *                    aux = channel type | memory kind<<8
  */
 
 #define KTJ_M_TYPE_MASK 0x1Fu
@@ -97,6 +98,7 @@ struct EmitCtx {
   const char* coll_blob;            /* collective arguments of each ktj_add_collective entry   */
   const uint64_t* coll_off;         /* n_coll + 1                                              */
   uint32_t n_coll;
+  uint32_t create_flags;            /* ktj_create flags that change the text (KTJ_CREATE_CUDA12_ARGS) */
 };
 
 #endif

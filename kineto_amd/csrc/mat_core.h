@@ -34,6 +34,17 @@ KTJ_HD inline void convert_range(const ClockDev& c, uint32_t mode, uint64_t* beg
   }
 }
 
+/* The kind of a device row: the low 16 bits of `domain`; kinds this engine does not know are
+ * kernel dispatches, as in GpuActivity's constructor (RocprofActivity.h:88-97). */
+KTJ_HD inline uint32_t device_row_domain(uint32_t raw) {
+  const uint32_t d = KTJ_ROW_DOMAIN(raw);
+  return d <= KTJ_DOM_MEMSET ? d : KTJ_DOM_KERNEL_DISPATCH;
+}
+/* resourceId() of a device row as submitted: a memset row's stream id is 32 bits wide (ktj_memset_rec) */
+KTJ_HD inline int64_t device_row_stream(uint32_t dom, uint64_t stream) {
+  return dom == KTJ_DOM_MEMSET ? (int64_t)(stream & 0xFFFFFFFFull) : (int64_t)stream;
+}
+
 /* timestamp()/duration() of a device row after clock conversion */
 KTJ_HD inline void device_times(uint32_t domain, uint64_t begin, uint64_t end, int64_t* ts, int64_t* dur) {
   if (domain == KTJ_DOM_MEMSET) {
@@ -144,7 +155,7 @@ KTJ_HD inline MatRow mat_device_v(const ktj_device_rec& d, int64_t ts, int64_t d
   MatRow m;
   m.ts = ts; m.dur = dur; m.dev = (int64_t)d.device; m.res = res;
   m.flow_id = (int64_t)d.id;
-  const uint32_t dom = d.domain <= KTJ_DOM_MEMSET ? d.domain : KTJ_DOM_KERNEL_DISPATCH;
+  const uint32_t dom = device_row_domain(d.domain);
   const uint32_t type = dom == KTJ_DOM_MEMSET ? KTJ_TYPE_GPU_MEMSET
                       : dom == KTJ_DOM_MEMORY_COPY ? KTJ_TYPE_GPU_MEMCPY : KTJ_TYPE_CONCURRENT_KERNEL;
   uint32_t meta = type | (KTJ_CLASS_DEVICE << KTJ_M_CLASS_SHIFT) | (dom << KTJ_M_KIND_SHIFT);
@@ -154,9 +165,13 @@ KTJ_HD inline MatRow mat_device_v(const ktj_device_rec& d, int64_t ts, int64_t d
   m.aux = d.op;
   m.p[0] = m.p[1] = m.p[2] = m.p[4] = 0;
   m.p[3] = d.queue;
-  if (dom == KTJ_DOM_MEMSET) {
+  if (dom == KTJ_DOM_MEMSET) { /* the row's ktj_memset_rec view */
     meta |= KTJ_M_NAME_BUILTIN; m.name_id = KTJ_NAME_MEMSET;
+    m.aux = (d.domain >> 16) & 0xFFFFu;              /* channel type | memory kind << 8 */
     m.p[0] = d.bytes;
+    m.p[1] = (uint64_t)d.op | ((uint64_t)d.name_id << 32); /* graph node id */
+    m.p[2] = (d.stream >> 32) | (d.queue & 0xFFFFFFFF00000000ull); /* graph id | channel id << 32 */
+    m.p[3] = d.queue & 0xFFFFFFFFull;                 /* context id */
   } else {
     if (dom == KTJ_DOM_MEMORY_COPY) {
       meta |= KTJ_M_NAME_BUILTIN;

@@ -576,11 +576,13 @@ static int gen_launch_chain(gen_t* g, uint32_t config, uint64_t N) {
       memset(r, 0, sizeof *r);
       r->id = corr; r->begin = rb; r->end = re; r->cid = CID_MEMSET_ASYNC; r->pid = PID; r->tid = tid;
       r->kind = KTJ_RT_DEFAULT;
-      ktj_device_rec* d = &dv[i];
-      memset(d, 0, sizeof *d);
-      d->id = corr; d->begin = db; d->end = de; d->domain = KTJ_DOM_MEMSET; d->op = 0; d->device = 0;
-      d->name_id = KTJ_NONE; d->queue = 1 /* context */; d->stream = 1 + sk;
-      d->bytes = lognormal(g->seed, 13, i, 65536, 65536);
+      ktj_memset_rec m; /* the memset view of a device row */
+      memset(&m, 0, sizeof m);
+      m.id = corr; m.begin = db; m.end = de; m.domain = KTJ_DOM_MEMSET; m.device = 0;
+      m.memory_kind = KTJ_MEMKIND_DEVICE; m.channel_type = 1; m.channel_id = 4 + (uint32_t)(sk % 4);
+      m.context = 1; m.stream = 1 + (uint32_t)sk;
+      m.bytes = lognormal(g->seed, 13, i, 65536, 65536);
+      memcpy(&dv[i], &m, sizeof m);
     }
     ec[i].correlation = corr;
     ec[i].external_id = j + 1;

@@ -47,9 +47,11 @@
  *       GpuActivity classes, run by the same driver on packed rows (tests/test_rocm_wrappers.py);
  *       the stream back-fill against the reference's own detail::backfillAsyncStreams
  *       (RocmStreamQueue.h:42-136) on seeded rows, same driver, same test file.
- *       Memset rows are CUDA-shaped (CuptiActivity.h:682-713); those wrappers need CUPTI's headers
- *       and cannot be built here: PARITY UNPINNED for the args order of that one row kind, which
- *       is read from the source.
+ *   - memset rows, which are CUDA-shaped (CuptiActivity.h:682-719): against the reference's own
+ *       GpuActivity<CUpti_ActivityMemsetType>, run by oracle/_ref/cupti_ref_driver on records built
+ *       in memory, compiled against the CUDA 12 and CUPTI headers of this image
+ *       (tests/test_cuda_memset_rows.py): name, type, times, ids and every args key and value, with
+ *       the four keys that the reference prints for CUDA >= 12 (KTJ_CREATE_CUDA12_ARGS) and without.
  */
 #define _GNU_SOURCE
 #include "ktj_oracle.h"
@@ -319,13 +321,18 @@ enum { /* built-in strings appended to the stream's dictionary */
   BS_DEVICE, BS_STREAM, BS_HSA_QUEUE, BS_CORRELATION, BS_KIND, BS_BYTES, BS_BANDWIDTH, BS_GRID,
   BS_BLOCK, BS_CID, BS_SHARED_MEMORY, BS_SRC, BS_DST, BS_PTR, BS_KERNEL, BS_CONTEXT,
   BS_DISPATCH_KERNEL, BS_HTOH, BS_HTOD, BS_DTOH, BS_DTOD, BS_UNKNOWN_KIND,
-  BS_MEMSET_NAME, BS_EMPTY, BS_COUNT
+  BS_MEMSET_UNKNOWN, BS_MEMSET_PAGEABLE, BS_MEMSET_PINNED, BS_MEMSET_DEVICE, BS_MEMSET_ARRAY, BS_MEMSET_MANAGED,
+  BS_MEMSET_DEVICE_STATIC, BS_MEMSET_MANAGED_STATIC, BS_MEMSET_UNRECOGNIZED,
+  BS_GRAPH_ID, BS_GRAPH_NODE_ID, BS_CHANNEL, BS_CHANNEL_TYPE, BS_EMPTY, BS_COUNT
 };
 static const char* const kBuiltin[BS_COUNT] = {
     "device", "stream", "hsa_queue", "correlation", "kind", "bytes", "memory bandwidth (GB/s)", "grid",
     "block", "cid", "shared memory", "src", "dst", "ptr", "kernel", "context",
     "Dispatch Kernel", "HtoH", "HtoD", "DtoH", "DtoD", "<unknown>",
-    "Memset (Device)", ""};
+    /* "Memset ({})" of memoryKindString, cupti_strings.cpp:42-66 */
+    "Memset (Unknown)", "Memset (Pageable)", "Memset (Pinned)", "Memset (Device)", "Memset (Array)", "Memset (Managed)",
+    "Memset (Device Static)", "Memset (Managed Static)", "Memset (Unrecognized)",
+    "graph id", "graph node id", "channel", "channel_type", ""};
 
 struct ktj_oracle {
   const ktj_stream* s;
@@ -588,7 +595,7 @@ static int stage_join(ktj_oracle* o) {
     if (by_corr.n != 0) {
       for (uint64_t i = 0; i < s->n_device; ++i) {
         const ktj_device_rec* d = &s->device[i];
-        if (d->domain == KTJ_DOM_MEMSET || dev_stream[i] != 0) continue;
+        if (KTJ_ROW_DOMAIN(d->domain) == KTJ_DOM_MEMSET || dev_stream[i] != 0) continue;
         const uint64_t* f = umap_find(&by_corr, d->id);
         if (f) dev_stream[i] = *f;
       }
@@ -597,7 +604,7 @@ static int stage_join(ktj_oracle* o) {
       umap by_queue; umap_init(&by_queue, 1024);
       for (uint64_t i = 0; i < s->n_device; ++i) {
         const ktj_device_rec* d = &s->device[i];
-        if (d->domain == KTJ_DOM_MEMSET || dev_stream[i] == 0 || d->queue == 0) continue;
+        if (KTJ_ROW_DOMAIN(d->domain) == KTJ_DOM_MEMSET || dev_stream[i] == 0 || d->queue == 0) continue;
         int inserted;
         uint64_t* v = umap_slot(&by_queue, d->queue, &inserted);
         if (inserted) *v = dev_stream[i];
@@ -605,7 +612,7 @@ static int stage_join(ktj_oracle* o) {
       }
       for (uint64_t i = 0; i < s->n_device; ++i) {
         const ktj_device_rec* d = &s->device[i];
-        if (d->domain == KTJ_DOM_MEMSET || dev_stream[i] != 0) continue;
+        if (KTJ_ROW_DOMAIN(d->domain) == KTJ_DOM_MEMSET || dev_stream[i] != 0) continue;
         const uint64_t* f = umap_find(&by_queue, d->queue);
         if (f && *f != AMBIG) dev_stream[i] = *f;
       }
@@ -615,7 +622,7 @@ static int stage_join(ktj_oracle* o) {
       dense_map dense; dense_init(&dense);
       for (uint64_t i = 0; i < s->n_device; ++i) {
         const ktj_device_rec* d = &s->device[i];
-        if (d->domain == KTJ_DOM_MEMSET) continue;
+        if (KTJ_ROW_DOMAIN(d->domain) == KTJ_DOM_MEMSET) continue;
         uint64_t key;
         if (dev_stream[i] != 0) key = dev_stream[i];
         else if (d->queue != 0) key = d->queue | (1ULL << 63);
@@ -719,11 +726,11 @@ static int stage_join(ktj_oracle* o) {
       end += (uint64_t)cm->async_offset;
     }
     int64_t ts, dur, resource;
-    if (d->domain == KTJ_DOM_MEMSET) {
+    if (KTJ_ROW_DOMAIN(d->domain) == KTJ_DOM_MEMSET) {
       /* CuptiActivity.h GpuActivity<T>::timestamp/duration via CuptiTimestamp.h:29-51 */
       ts = (int64_t)begin;
       dur = (int64_t)end - (int64_t)begin;
-      resource = (int64_t)d->stream;
+      resource = (int64_t)(uint32_t)d->stream; /* streamId is 32 bits wide: ktj_memset_rec */
     } else {
       /* RocprofActivity.h:122-127 */
       ts = (int64_t)(begin + 1);
@@ -766,25 +773,33 @@ static int stage_join(ktj_oracle* o) {
     if (linked >= 0) {
       a->has_linked = 1; a->linked_corr = s->generic[linked].id; o->n_linked++;
       const ktj_generic_rec* op = &s->generic[linked]; /* the op hands its collective metadata to kernels */
-      if (d->domain != KTJ_DOM_MEMSET && d->domain != KTJ_DOM_MEMORY_COPY && op->type != KTJ_TYPE_CONCURRENT_KERNEL &&
+      if (KTJ_ROW_DOMAIN(d->domain) != KTJ_DOM_MEMSET && KTJ_ROW_DOMAIN(d->domain) != KTJ_DOM_MEMORY_COPY && op->type != KTJ_TYPE_CONCURRENT_KERNEL &&
           op->type != KTJ_TYPE_MTIA_CCP_EVENTS)
         a->collective = collective_index(s, op);
     }
     int key = (int)(uint32_t)d->id;
-    if (d->domain == KTJ_DOM_MEMSET) { /* CuptiActivity.h:682-713 */
+    if (KTJ_ROW_DOMAIN(d->domain) == KTJ_DOM_MEMSET) { /* CuptiActivity.h:682-719 */
+      ktj_memset_rec m;
+      memcpy(&m, d, sizeof m);
       a->type = KTJ_TYPE_GPU_MEMSET;
-      a->name_id = o->builtin0 + BS_MEMSET_NAME;
-      visit1(o, a, BS_DEVICE, KTJ_F_I64, (uint64_t)(int64_t)d->device);
-      visit1(o, a, BS_CONTEXT, KTJ_F_U64, d->queue);
-      visit1(o, a, BS_STREAM, KTJ_F_I64, d->stream);
-      visit1(o, a, BS_CORRELATION, KTJ_F_U64, d->id);
-      visit1(o, a, BS_BYTES, KTJ_F_U64, d->bytes);
-      if (dur != 0) /* CuptiActivity.h:460-470 */
-        visit1(o, a, BS_BANDWIDTH, KTJ_F_F64, dbits((double)d->bytes / (double)dur));
+      a->name_id = o->builtin0 + (m.memory_kind <= KTJ_MEMKIND_MANAGED_STATIC ? BS_MEMSET_UNKNOWN + m.memory_kind : BS_MEMSET_UNRECOGNIZED);
+      visit1(o, a, BS_DEVICE, KTJ_F_I64, (uint64_t)(int64_t)m.device);
+      visit1(o, a, BS_CONTEXT, KTJ_F_U64, m.context);
+      visit1(o, a, BS_STREAM, KTJ_F_I64, m.stream);
+      visit1(o, a, BS_CORRELATION, KTJ_F_U64, m.id);
+      visit1(o, a, BS_BYTES, KTJ_F_U64, m.bytes);
+      if (dur != 0) /* addBandwidthTypedMetadata, CuptiActivity.h:460-470 */
+        visit1(o, a, BS_BANDWIDTH, KTJ_F_F64, dbits((double)m.bytes / (double)dur));
+      if (s->create_flags & KTJ_CREATE_CUDA12_ARGS) { /* CUDA_VERSION >= 12000: CuptiActivity.h:424-458 */
+        visit1(o, a, BS_GRAPH_ID, KTJ_F_U64, m.graph_id);
+        visit1(o, a, BS_GRAPH_NODE_ID, KTJ_F_U64, (uint64_t)m.graph_node_lo | ((uint64_t)m.graph_node_hi << 32));
+        visit1(o, a, BS_CHANNEL, KTJ_F_U64, m.channel_id);
+        visit1(o, a, BS_CHANNEL_TYPE, KTJ_F_I64, m.channel_type);
+      }
       continue;
     }
     int kind_str;
-    if (d->domain == KTJ_DOM_MEMORY_COPY) { /* RocprofActivity_inl.h:50-94, 98-127 */
+    if (KTJ_ROW_DOMAIN(d->domain) == KTJ_DOM_MEMORY_COPY) { /* RocprofActivity_inl.h:50-94, 98-127 */
       a->type = KTJ_TYPE_GPU_MEMCPY;
       const char *ks, *src, *dst;
       switch (d->op) {

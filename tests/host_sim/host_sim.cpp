@@ -76,6 +76,7 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   ctx.dict.flags = v.flags.data(); ctx.dict.n = (uint32_t)s->n_strings;
   ctx.fields = s->fields; ctx.schemas = s->schemas; ctx.n_schemas = (uint32_t)s->n_schemas;
   ctx.args = s->args; ctx.n_args = s->n_args; ctx.base_time_ns = s->base_time_ns;
+  ctx.create_flags = s->create_flags;
   // collective metadata: the arguments of every entry in one blob
   std::vector<ktj::CollectiveInfo> collectives;
   std::string coll_blob;
@@ -145,7 +146,7 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
   if (!stream_src.empty()) {
     for (uint64_t i = 0; i < nd; ++i) {
       const ktj_device_rec& d = s->device[i];
-      if (d.domain == KTJ_DOM_MEMSET || dstream[i]) continue;
+      if (device_row_domain(d.domain) == KTJ_DOM_MEMSET || dstream[i]) continue;
       auto it = stream_src.find(d.id);
       if (it != stream_src.end()) {
         const ktj_runtime_rec& r = s->runtime[it->second];
@@ -156,14 +157,14 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
     std::unordered_set<uint64_t> ambiguous;
     for (uint64_t i = 0; i < nd; ++i) {
       const ktj_device_rec& d = s->device[i];
-      if (d.domain == KTJ_DOM_MEMSET || !dstream[i] || !d.queue) continue;
+      if (device_row_domain(d.domain) == KTJ_DOM_MEMSET || !dstream[i] || !d.queue) continue;
       auto it = by_queue.find(d.queue);
       if (it == by_queue.end()) by_queue[d.queue] = dstream[i];
       else if (it->second != dstream[i]) ambiguous.insert(d.queue);
     }
     for (uint64_t i = 0; i < nd; ++i) {
       const ktj_device_rec& d = s->device[i];
-      if (d.domain == KTJ_DOM_MEMSET || dstream[i]) continue;
+      if (device_row_domain(d.domain) == KTJ_DOM_MEMSET || dstream[i]) continue;
       auto it = by_queue.find(d.queue);
       if (it != by_queue.end() && !ambiguous.count(d.queue)) dstream[i] = it->second;
     }
@@ -172,7 +173,7 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
     std::vector<Ent> ents;
     auto key_of = [&](uint64_t i, uint64_t* key) {
       const ktj_device_rec& d = s->device[i];
-      if (d.domain == KTJ_DOM_MEMSET) return false;
+      if (device_row_domain(d.domain) == KTJ_DOM_MEMSET) return false;
       if (dstream[i]) *key = dstream[i]; else if (d.queue) *key = d.queue | (1ULL << 63); else return false;
       return true;
     };
@@ -197,14 +198,14 @@ int ktjsim_render(const ktj_stream* s, uint32_t tile_bytes, char** out, uint64_t
     uint64_t b = d.begin, e = d.end;
     convert_range(clk, clk.device_mode, &b, &e);
     int64_t ts, dur;
-    device_times(d.domain, b, e, &ts, &dur);
+    device_times(device_row_domain(d.domain), b, e, &ts, &dur);
     const bool valid = !out_of_range(ts, dur, s->window_start_ns, s->window_end_ns);
-    const int64_t res = d.domain == KTJ_DOM_MEMSET ? (int64_t)d.stream : (int64_t)(dstream[i] ? dstream[i] : d.queue);
+    const int64_t res = device_row_domain(d.domain) == KTJ_DOM_MEMSET ? device_row_stream(KTJ_DOM_MEMSET, d.stream) : (int64_t)(dstream[i] ? dstream[i] : d.queue);
     const uint64_t key = narrow_corr_key(d.id);
     const ktj_runtime_rec* ksrc = nullptr;
     bool has_size = false;
     uint64_t size = 0;
-    if (d.domain != KTJ_DOM_MEMSET) {
+    if (device_row_domain(d.domain) != KTJ_DOM_MEMSET) {
       auto si = size_src.find(key);
       if (si != size_src.end()) {
         const ktj_runtime_rec& r = s->runtime[si->second];

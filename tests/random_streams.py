@@ -41,6 +41,8 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False,
     lo, hi = B + 1000, B + 10**7
     window = (lo, hi) if rng.random() < 0.7 else (B + 3 * 10**6, B + 6 * 10**6)
     b = StreamBuilder(window=window, host_name="rnd", end_time=hi + 5)
+    rng_memset = random.Random(seed * 7919 + 13)   # memset rows: the view's extra fields, and the CUDA >= 12 key set or not
+    b.create_flags = abi.KTJ_CREATE_CUDA12_ARGS if rng_memset.random() < 0.5 else 0
     if rng.random() < 0.5:
         b.clock = abi.ClockModel(rng.randrange(0, 1000), rng.randrange(-500, 500), rng.choice([1.0, 1.000001, 0.999]), rng.randrange(-50, 50),
                                  rng.choice([0, 1]), rng.choice([0, 1, 2]))
@@ -157,7 +159,8 @@ def random_stream(seed, n_generic=40, n_runtime=40, n_device=60, wide_ids=False,
         s0 = t()
         b.add_device(rng.choice((unique_pool[:40] if unique_pool else []) + ids + [100, 101, 0]), s0, s0 + rng.choice([0, 1, 2, 900, 10**5]), domain=dom,
                      op=rng.choice([0, 1, 2, 3, 4, 9]), device=rng.choice([0, 0, 1, -1]), name=rng.choice(names + [None]),
-                     queue=rng.choice([0, 1, 2, 3, 2**63 + 5]), stream=rng.choice([0, 0, 0, 5, 0x7000]), nbytes=rng.choice([0, 1000, 2**40]))
+                     queue=rng.choice([0, 1, 2, 3, 2**63 + 5]), stream=rng.choice([0, 0, 0, 5, 0x7000]), nbytes=rng.choice([0, 1000, 2**40]),
+                     memory_kind=rng_memset.randrange(0, 10), channel_type=rng_memset.randrange(0, 4))
     for _ in range(rng.randrange(0, 40)):
         b.add_extcorr(rng.choice((unique_pool[:30] if unique_pool else []) + ids + [0xFFFFFFFFFFFFFFFF]), rng.choice([5, 6, 7, 8, 0, 2**31 - 1, 0xFFFFFFFF80000000, 2**40, 12345]))
     if rng.random() < 0.5:  # user-domain correlation: GPU user-annotation spans

@@ -28,6 +28,7 @@ class StreamBuilder:
         self.device_infos, self.resource_infos, self.overhead_infos, self.spans = [], [], [], []
         self.collectives = []
         self.usercorr = []
+        self.create_flags = 0   # the ktj_create flags that change the document (KTJ_CREATE_CUDA12_ARGS)
         self._keep = []
 
     # ---- dictionary / schemas ----
@@ -119,11 +120,28 @@ class StreamBuilder:
         self.runtime.append(r)
         return r
 
-    def add_device(self, id, begin, end, domain=0, op=0, device=0, name=None, queue=0, stream=0, nbytes=0):
+    def add_device(self, id, begin, end, domain=0, op=0, device=0, name=None, queue=0, stream=0, nbytes=0,
+                   memory_kind=abi.KTJ_MEMKIND_DEVICE, channel_type=0):
+        """A device row.  For a memset row (domain 2) the fields are read through the ktj_memset_rec
+        view: queue = context | channel id << 32, stream = stream | graph id << 32, op and the name's
+        string id are the two halves of the graph node id (add_memset spells that out)."""
         d = abi.DeviceRec()
         d.id, d.begin, d.end, d.domain, d.op, d.device = id, begin, end, domain, op, device
+        if domain == abi.KTJ_DOM_MEMSET:
+            d.domain = domain | (channel_type & 0xFF) << 16 | (memory_kind & 0xFF) << 24
         d.name_id = abi.KTJ_NONE if name is None else self.s(name)
         d.queue, d.stream, d.bytes = queue, stream, nbytes
+        self.device.append(d)
+        return d
+
+    def add_memset(self, id, begin, end, device=0, context=0, stream=0, nbytes=0, memory_kind=abi.KTJ_MEMKIND_DEVICE,
+                   graph_id=0, graph_node_id=0, channel_id=0, channel_type=0):
+        m = abi.MemsetRec()
+        m.id, m.begin, m.end, m.domain, m.device = id, begin, end, abi.KTJ_DOM_MEMSET, device
+        m.channel_type, m.memory_kind = channel_type, memory_kind
+        m.graph_node_lo, m.graph_node_hi = graph_node_id & 0xFFFFFFFF, graph_node_id >> 32
+        m.context, m.channel_id, m.stream, m.graph_id, m.bytes = context, channel_id, stream, graph_id, nbytes
+        d = abi.DeviceRec.from_buffer_copy(bytes(m))
         self.device.append(d)
         return d
 
@@ -182,6 +200,7 @@ class StreamBuilder:
         st.flow_start_cids = self._arr(C.c_uint32, self.flow_start)
         st.n_flow_start = len(self.flow_start)
         st.malloc_cid = self.malloc_cid
+        st.create_flags = self.create_flags
         st.clock = self.clock
         st.window_start_ns, st.window_end_ns = self.window
         st.end_time_ns = self.end_time

@@ -88,6 +88,8 @@ def _engine_vs_oracle(sp, check_substrings=(), **engine_options):
     from kineto_amd.engine import TraceEngine
     ora = og.OracleRun(sp)
     want = ora.output()
+    # the create flags that change the document travel with the stream (the checker reads them there)
+    engine_options.setdefault("cuda12_args", bool(sp.contents.create_flags & abi.KTJ_CREATE_CUDA12_ARGS))
     with TraceEngine(sp.contents.trace_name.decode(), device=0, **engine_options) as eng:
         eng.submit_stream(sp)
         eng.process()

@@ -109,7 +109,7 @@ def brute(sp):
         if sid:
             stream_by_corr[r.id] = sid
     dstream = [s.device[i].stream for i in range(s.n_device)]
-    is_async = [s.device[i].domain != 2 for i in range(s.n_device)]
+    is_async = [(s.device[i].domain & 0xFFFF) != 2 for i in range(s.n_device)]
     if stream_by_corr:
         for i in range(s.n_device):
             if is_async[i] and dstream[i] == 0 and s.device[i].id in stream_by_corr:
@@ -170,8 +170,9 @@ def brute(sp):
     for i in range(s.n_device):
         d = s.device[i]
         b, e = conv(clk.device_mode, d.begin, d.end)
-        if d.domain == 2:
-            ts, dur, res = to_i64(b), to_i64(e) - to_i64(b), to_i64(d.stream)
+        dom = d.domain & 0xFFFF                       # the kind of the row; a memset row keeps more in the upper half
+        if dom == 2:
+            ts, dur, res = to_i64(b), to_i64(e) - to_i64(b), d.stream & 0xFFFFFFFF
         else:
             ts, dur = to_i64(b + 1), to_i64(e - (b + 1))
             res = to_i64(dstream[i] if dstream[i] else d.queue)
@@ -181,7 +182,7 @@ def brute(sp):
         check_order(to_i64(d.id), False, ts)
         extra = {}
         key = to_i32(d.id)
-        if d.domain != 2:
+        if dom != 2:
             if key in to_size:
                 extra["bytes"] = to_size[key]
                 if (e - b) & 0xFFFFFFFFFFFFFFFF:
@@ -192,7 +193,7 @@ def brute(sp):
             extra["bytes"] = d.bytes
             if dur != 0:
                 extra["bw"] = d.bytes / float(dur)
-        typ = 4 if d.domain == 2 else (3 if d.domain == 1 else 5)
+        typ = 4 if dom == 2 else (3 if dom == 1 else 5)
         acts.append(dict(arrival=s.n_generic + s.n_runtime + i, ts=ts, dur=dur, device=d.device, resource=res, type=typ,
                          linked=lk, extra=extra))
         ext = user_corr.get(to_i64(d.id)) if s.n_usercorr else None
