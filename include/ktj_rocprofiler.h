@@ -52,10 +52,18 @@ int ktj_submit_sdk_buffer(ktj_engine* e, void* const* headers, size_t num_header
  * from the SDK's argument union by the names the reference looks for.  external_id /
  * user_external_id: the innermost id of the caller's external-correlation stack of domain 0 / 1, or
  * NULL where that stack is empty (:661-672): each gives one KTJ_REC_EXTCORR / KTJ_REC_USERCORR pair
- * for the call's correlation id.  Rows are buffered on the host and reach the device in batches and
- * with the next ktj_process / ktj_finalize. */
+ * for the call's correlation id.  Rows are buffered on the host and reach the device in batches:
+ * when 65536 have gathered, before a ktj_submit_records / ktj_submit_records_device call of the
+ * KTJ_REC_RUNTIME, KTJ_REC_EXTCORR or KTJ_REC_USERCORR class appends (so arrival order is call
+ * order), with ktj_flush, and with the next ktj_process / ktj_finalize.  ktj_process_noalloc does
+ * not take them (growing the device arrays allocates): call ktj_flush before it. */
 int ktj_submit_sdk_api_record(ktj_engine* e, const void* record, uint64_t begin, uint64_t end, uint32_t pid,
                               uint32_t tid, const uint64_t* external_id, const uint64_t* user_external_id);
+
+/* Sends the rows that ktj_submit_sdk_api_record has buffered on the host to the device, without
+ * processing anything.  No counterpart in the reference (its rows stay in host vectors,
+ * RocprofLogger.h:84). */
+int ktj_flush(ktj_engine* e);
 
 #ifdef __cplusplus
 }

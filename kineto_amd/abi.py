@@ -17,6 +17,7 @@ KTJ_CREATE_PAIR_SORT = 0x8
 KTJ_CREATE_DISPLAY_NS = 0x10
 KTJ_CREATE_CUDA12_ARGS = 0x20
 KTJ_GF_WIDE_DEVICE = 0x04
+KTJ_REC_GENERIC, KTJ_REC_RUNTIME, KTJ_REC_DEVICE, KTJ_REC_EXTCORR, KTJ_REC_USERCORR = 0, 1, 2, 3, 4
 
 REC_GENERIC, REC_RUNTIME, REC_DEVICE, REC_EXTCORR, REC_USERCORR = 0, 1, 2, 3, 4
 INFO_DEVICE, INFO_RESOURCE, INFO_OVERHEAD, INFO_SPAN = 0, 1, 2, 3
@@ -203,7 +204,7 @@ ENGINE_SYMBOLS = [
     "ktj_process", "ktj_process_noalloc", "ktj_output_device", "ktj_output_host", "ktj_finalize", "ktj_get_stats",
     "ktj_version",
     # include/ktj_rocprofiler.h
-    "ktj_set_sdk_agents", "ktj_set_sdk_kernel_names", "ktj_submit_sdk_buffer", "ktj_submit_sdk_api_record",
+    "ktj_set_sdk_agents", "ktj_set_sdk_kernel_names", "ktj_submit_sdk_buffer", "ktj_submit_sdk_api_record", "ktj_flush",
 ]
 
 
@@ -254,6 +255,8 @@ def load_engine():
         lib.ktj_set_sdk_kernel_names.argtypes = [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), C.c_size_t, C.c_uint32]
         lib.ktj_submit_sdk_buffer.restype = C.c_int
         lib.ktj_submit_sdk_buffer.argtypes = [vp, C.POINTER(C.c_void_p), C.c_size_t, C.POINTER(C.c_uint64)]
+        lib.ktj_flush.restype = C.c_int
+        lib.ktj_flush.argtypes = [vp]
         lib.ktj_submit_sdk_api_record.restype = C.c_int
         lib.ktj_submit_sdk_api_record.argtypes = [vp, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint32, C.c_uint32,
                                                   C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]

@@ -557,12 +557,22 @@ static RecordSet* record_set(ktj_engine* e, int rec_class, size_t* rec_size) {
   }
 }
 
+static int flush_sdk_api_rows(ktj_engine* e);
+/* rows of ktj_submit_sdk_api_record that wait on the host arrived before anything submitted now */
+static bool class_has_buffered_sdk_rows(int rec_class) {
+  return rec_class == KTJ_REC_RUNTIME || rec_class == KTJ_REC_EXTCORR || rec_class == KTJ_REC_USERCORR;
+}
+
 int ktj_submit_records(ktj_engine* e, int rec_class, const void* packed, size_t n_records) {
   if (!e || (n_records && !packed)) return KTJ_ERR_ARG;
   size_t rs = 0;
   RecordSet* set = record_set(e, rec_class, &rs);
   if (!set) return KTJ_ERR_ARG;
   if (e->bad_sink || n_records == 0) return KTJ_OK;
+  if (class_has_buffered_sdk_rows(rec_class)) {
+    const int flushed = flush_sdk_api_rows(e);
+    if (flushed != KTJ_OK) return flushed;
+  }
   if (set->external) return KTJ_ERR_STATE;
   HIPCHK(hipSetDevice(e->device));
   HIPCHK(set->owned.append(packed, n_records * rs, e->stream));
@@ -579,6 +589,10 @@ int ktj_submit_records_device(ktj_engine* e, int rec_class, const void* device_p
   if (!set) return KTJ_ERR_ARG;
   if (((uintptr_t)device_ptr & 15u) != 0) return KTJ_ERR_ARG; /* kernels read 16-byte lanes */
   if (e->bad_sink) return KTJ_OK;
+  if (class_has_buffered_sdk_rows(rec_class)) {
+    const int flushed = flush_sdk_api_rows(e);
+    if (flushed != KTJ_OK) return flushed;
+  }
   if (set->owned.bytes != 0) return KTJ_ERR_STATE;
   set->external = n_records ? device_ptr : nullptr;
   set->n = n_records;
@@ -650,14 +664,28 @@ int ktj_submit_sdk_buffer(ktj_engine* e, void* const* headers, size_t num_header
   return ktj_submit_records(e, KTJ_REC_DEVICE, rows.data(), rows.size());
 }
 
-/* runtime rows and correlation pairs that ktj_submit_sdk_api_record collected go to the device */
+/* Runtime rows and correlation pairs that ktj_submit_sdk_api_record collected go to the device.  The
+ * vectors are taken out first: the submit calls below flush whatever is buffered before they append. */
 static int flush_sdk_api_rows(ktj_engine* e) {
+  if (e->sdk_api_rows.empty() && e->sdk_api_ext.empty() && e->sdk_api_user.empty()) return KTJ_OK;
+  std::vector<ktj_runtime_rec> rows; rows.swap(e->sdk_api_rows);
+  std::vector<ktj_extcorr_rec> ext, user; ext.swap(e->sdk_api_ext); user.swap(e->sdk_api_user);
   int rc = KTJ_OK;
-  if (!e->sdk_api_rows.empty()) rc = ktj_submit_records(e, KTJ_REC_RUNTIME, e->sdk_api_rows.data(), e->sdk_api_rows.size());
-  if (rc == KTJ_OK && !e->sdk_api_ext.empty()) rc = ktj_submit_records(e, KTJ_REC_EXTCORR, e->sdk_api_ext.data(), e->sdk_api_ext.size());
-  if (rc == KTJ_OK && !e->sdk_api_user.empty()) rc = ktj_submit_records(e, KTJ_REC_USERCORR, e->sdk_api_user.data(), e->sdk_api_user.size());
-  if (rc == KTJ_OK) { e->sdk_api_rows.clear(); e->sdk_api_ext.clear(); e->sdk_api_user.clear(); }
+  if (!rows.empty()) rc = ktj_submit_records(e, KTJ_REC_RUNTIME, rows.data(), rows.size());
+  if (rc == KTJ_OK && !ext.empty()) rc = ktj_submit_records(e, KTJ_REC_EXTCORR, ext.data(), ext.size());
+  if (rc == KTJ_OK && !user.empty()) rc = ktj_submit_records(e, KTJ_REC_USERCORR, user.data(), user.size());
+  if (rc != KTJ_OK) { /* nothing is lost: what a later flush finds is what this one could not place */
+    e->sdk_api_rows.swap(rows); e->sdk_api_ext.swap(ext); e->sdk_api_user.swap(user);
+  } else { /* keep the capacity for the next batch */
+    rows.clear(); e->sdk_api_rows.swap(rows);
+  }
   return rc;
+}
+
+int ktj_flush(ktj_engine* e) {
+  if (!e) return KTJ_ERR_ARG;
+  if (e->bad_sink) return KTJ_OK;
+  return flush_sdk_api_rows(e);
 }
 
 #define KTJ_SDK_API_BATCH 65536u
@@ -1118,7 +1146,7 @@ int ktj_process_noalloc(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   if (e->bad_sink) return KTJ_OK;
   if (!e->arena) { e->last_error = "ktj_process_noalloc: no scratch array on this device"; return KTJ_ERR_STATE; }
   if (!e->sdk_api_rows.empty() || !e->sdk_api_ext.empty() || !e->sdk_api_user.empty()) {
-    e->last_error = "ktj_process_noalloc: rows of ktj_submit_sdk_api_record are still buffered on the host (ktj_process takes them over)";
+    e->last_error = "ktj_process_noalloc: rows of ktj_submit_sdk_api_record are still buffered on the host (call ktj_flush first: it may allocate)";
     return KTJ_ERR_STATE;
   }
   if (e->usercorr.n != 0) {

@@ -131,6 +131,8 @@ struct Scalars {
   unsigned int n_res_ranks;           /* distinct resourceId values */
   unsigned int n_dense;               /* distinct (device, stream key) pairs */
   unsigned int runtime_ids_repeat;    /* two runtime rows share a slot of the full table */
+  unsigned int n_queues;              /* distinct hardware queues entered into the queue -> stream table */
+  unsigned int n_sync_rows;           /* distinct (device, row) pairs of Stream Sync activities */
   alignas(256) JoinPlan plan;         /* key ranges and modes of the join tables: read by every row of the join
                                          kernels, so kept off the cache lines that take the counters' atomics */
 };
@@ -149,7 +151,8 @@ struct Scalars {
 #define KTJ_DENSE_CAP (2u * KTJ_MAX_STREAM_PAIRS) /* slots of the (device, stream) table */
 #define KTJ_QUEUE_CAP (2u * KTJ_MAX_QUEUES)       /* slots of the queue -> stream table */
 #define KTJ_SYNC_CAP (2u * KTJ_MAX_SYNC_ROWS)     /* slots of the Stream Sync (device, row) table */
-#define KTJ_TABLE_PROBES 256u  /* linear probing of these small tables gives up after this many slots */
+#define KTJ_TABLE_PROBES 256u  /* linear probing of these small tables gives up after this many slots: a backstop,
+                                  the documented limits are enforced by counting the distinct keys */
 
 struct ApiTable {
   const uint32_t* cid_name_ids;

@@ -55,6 +55,29 @@ __device__ uint32_t table_insert(uint64_t* keys, uint32_t mask, uint64_t key) {
   }
   return KTJ_NOSLOT;
 }
+/* table_insert for a table with a documented limit on its distinct keys: the key that would be
+ * number `limit` + 1 is refused (KTJ_NOSLOT), whatever room the table still has, so that a trace is
+ * accepted or refused by the count the limit names and not by how its keys happen to hash. */
+__device__ uint32_t table_insert_counted(uint64_t* keys, uint32_t mask, uint64_t key, unsigned int* count, uint32_t limit) {
+  if (key == KTJ_EMPTY_KEY) {
+    if (atomicExch((unsigned long long*)&keys[mask + 1u], 0ULL) != 0ULL && atomicAdd(count, 1u) >= limit) return KTJ_NOSLOT;
+    return mask + 1u;
+  }
+  uint32_t slot = (uint32_t)hash64(key) & mask;
+  for (uint32_t probe = 0; probe <= mask && probe < KTJ_TABLE_PROBES; ++probe) {
+    uint64_t cur = keys[slot];
+    if (cur == key) return slot;
+    if (cur == KTJ_EMPTY_KEY) {
+      if (*(volatile unsigned int*)count >= limit) return KTJ_NOSLOT; /* full by count: take no further slot */
+      unsigned long long prev = atomicCAS((unsigned long long*)&keys[slot], (unsigned long long)KTJ_EMPTY_KEY,
+                                          (unsigned long long)key);
+      if (prev == KTJ_EMPTY_KEY) return atomicAdd(count, 1u) >= limit ? KTJ_NOSLOT : slot;
+      if (prev == key) return slot;
+    }
+    slot = (slot + 1u) & mask;
+  }
+  return KTJ_NOSLOT;
+}
 __device__ uint32_t table_find(const uint64_t* keys, uint32_t mask, uint64_t key) {
   if (key == KTJ_EMPTY_KEY) return keys[mask + 1u] == 0 ? mask + 1u : KTJ_NOSLOT;
   uint32_t slot = (uint32_t)hash64(key) & mask;
@@ -164,6 +187,7 @@ __global__ void k_init_scalars(Scalars* s) {
     s->ts_min_biased = ~0ULL; s->ts_max_biased = 0;
     s->out_of_range = 0; s->out_of_order = 0; s->n_flow = 0; s->n_linked = 0; s->n_blank_names = 0; s->n_valid = 0;
     s->n_unresolved = 0; s->n_sync_typed = 0; s->n_device_orphans = 0; s->error = 0; s->have_stream_src = 0; s->n_dev_ranks = 0; s->n_res_ranks = 0; s->n_dense = 0; s->runtime_ids_repeat = 0;
+    s->n_queues = 0; s->n_sync_rows = 0;
     for (int k = 0; k < 3; ++k) {
       s->plan.range[k].lo = ~0ULL; s->plan.range[k].hi = 0;
       s->plan.ctl[k].base = 0; s->plan.ctl[k].span = 0; s->plan.ctl[k].direct = 0; s->plan.ctl[k].pad = 0;
@@ -1059,7 +1083,7 @@ __global__ void k_queue_build(const DevBrief* d, uint64_t n, Columns c, uint64_t
   const uint64_t stream = (uint64_t)c.res[first_device + i];
   const uint64_t queue = d[i].queue;
   if (!is_async_op(d[i].domain) || stream == 0 || queue == 0) return;
-  const uint32_t slot = table_insert(t.q_keys, KTJ_QUEUE_CAP - 1u, queue);
+  const uint32_t slot = table_insert_counted(t.q_keys, KTJ_QUEUE_CAP - 1u, queue, &sc->n_queues, KTJ_MAX_QUEUES);
   if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_QUEUES); return; }
   unsigned long long cur = t.q_stream[slot];
   if (cur == 0) cur = atomicCAS((unsigned long long*)&t.q_stream[slot], 0ULL, (unsigned long long)stream);
@@ -1861,7 +1885,8 @@ __global__ void k_sync_first_a(const uint32_t* perm, uint64_t n_sorted, const kt
   if (p >= n_sorted) return;
   const uint64_t a = perm[p];
   if (a >= n_generic || !is_stream_sync(g[a], d)) return;
-  const uint32_t slot = table_insert(keys, KTJ_SYNC_CAP - 1u, stream_sync_key(dev[a], g[a].resource));
+  const uint32_t slot = table_insert_counted(keys, KTJ_SYNC_CAP - 1u, stream_sync_key(dev[a], g[a].resource), &sc->n_sync_rows,
+                                             KTJ_MAX_SYNC_ROWS);
   if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_SYNC_ROWS); return; }
   atomicMin(&first_pos[slot], (uint32_t)p);
 }

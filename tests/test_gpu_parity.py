@@ -151,7 +151,7 @@ def test_join_edge_cases_on_gpu():
     assert got.count(b'"ph": "X"') == 20   # every in-window row of the hand-made stream printed
 
 
-KTJ_MAX_STREAM_PAIRS = 4096   # include/ktj.h
+KTJ_MAX_STREAM_PAIRS, KTJ_MAX_QUEUES, KTJ_MAX_SYNC_ROWS = 4096, 32768, 32768   # include/ktj.h
 
 
 def _many_ids_builder(n_resources, n_devices, n_streams=0, n_queues=0, n_sync_rows=0):
@@ -177,6 +177,21 @@ def _many_ids_builder(n_resources, n_devices, n_streams=0, n_queues=0, n_sync_ro
     return b
 
 
+def _queue_limit_builder(n_queues):
+    """Device rows on n_queues distinct hardware queues in a trace where the queue -> stream table is
+    used: one runtime row carries a stream, one device row has neither a stream nor a runtime row."""
+    from stream_builder import StreamBuilder, B
+    b = StreamBuilder(host_name="queues")
+    b.api(["hipLaunchKernel"], flow_start=[0])
+    b.add_runtime(1, B + 5000, B + 5400, 0, 1, 1, kind=1, stream=0x7000)
+    b.add_device(1, B + 6000, B + 6300, domain=0, device=0, name="k", queue=0x100)
+    b.add_device(5, B + 6400, B + 6500, domain=0, device=0, name="k", queue=0x100)      # takes its queue's stream
+    for i in range(1, n_queues):
+        b.add_device(10**6 + i, B + 7000 + i, B + 7300 + i, domain=i % 2, op=2 * (i % 2), device=0, name="k%d" % (i % 4),
+                     queue=0x100 + i, stream=0x7000 + 8 * (i % 5))
+    return b
+
+
 def test_more_distinct_ids_than_the_rank_sets_hold():
     """Above 4096 distinct resourceId or deviceId values the sort works on the raw values: same bytes
     as the checker, no error."""
@@ -189,16 +204,22 @@ def test_limits_end_in_a_named_error():
     """A trace beyond one of the engine's documented limits is refused with KTJ_ERR_LIMIT and a text
     that names the limit (include/ktj.h: KTJ_MAX_*)."""
     from kineto_amd.engine import TraceEngine, EngineError
-    for kw, name in ((dict(n_streams=KTJ_MAX_STREAM_PAIRS + 200), "KTJ_MAX_STREAM_PAIRS"),):
-        print("limit", name, flush=True)
-        sp = _many_ids_builder(10, 1, **kw).build()
-        with TraceEngine("t.json", device=0) as eng:
-            eng.submit_stream(sp)
-            with pytest.raises(EngineError) as ei:
-                eng.process()
-            assert "rc=%d" % abi.KTJ_ERR_LIMIT in str(ei.value) and name in str(ei.value)
-    # just inside the limit: accepted and identical to the checker
-    _engine_vs_oracle(_many_ids_builder(10, 1, n_streams=KTJ_MAX_STREAM_PAIRS - 96).build())
+    for make, limit, name in ((lambda n: _many_ids_builder(10, 1, n_streams=n), KTJ_MAX_STREAM_PAIRS, "KTJ_MAX_STREAM_PAIRS"),
+                              (_queue_limit_builder, KTJ_MAX_QUEUES, "KTJ_MAX_QUEUES"),
+                              (lambda n: _many_ids_builder(10, 1, n_sync_rows=n), KTJ_MAX_SYNC_ROWS, "KTJ_MAX_SYNC_ROWS")):
+        # the limits are counts of distinct keys: one key more is refused, however the keys hash
+        for n in (limit + 1, limit + 200):
+            print("limit", name, n, flush=True)
+            sp = make(n).build()
+            with TraceEngine("t.json", device=0) as eng:
+                eng.submit_stream(sp)
+                with pytest.raises(EngineError) as ei:
+                    eng.process()
+                assert "rc=%d" % abi.KTJ_ERR_LIMIT in str(ei.value) and name in str(ei.value)
+                assert eng.lib.ktj_process(eng.h, eng.end_time_ns) == abi.KTJ_ERR_LIMIT   # and again: every kernel ended normally
+        # exactly at the limit: accepted and identical to the checker
+        print("at the limit", name, flush=True)
+        _engine_vs_oracle(make(limit).build())
 
 
 def test_header_text_beyond_the_pinned_staging_buffer():

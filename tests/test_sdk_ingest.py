@@ -336,3 +336,44 @@ def test_sdk_api_records_end_to_end():
         got = eng.output()
     assert got == want
     assert got.count(b'"cat": "cuda_runtime"') == len(calls)
+    # The first half as SDK callback records, the second half as packed rows: the buffered rows reach
+    # the device before the packed ones are appended, so arrival order is call order.  The last few
+    # calls come as SDK records again and stay buffered: ktj_flush sends them without processing,
+    # after which the pass that allocates nothing takes the trace too.
+    import torch
+    half, tail = len(calls) // 2, len(calls) - 7
+    sp3 = base_stream().build()
+    with TraceEngine(sp3.contents.trace_name.decode(), device=0) as eng:
+        eng.submit_stream(sp3)
+
+        def as_sdk_record(call):
+            op, corr, t0, t1, pid, tid = call
+            rec = sim.ktjsim_sdk_api_record_create(sim.ktjsim_sdk_api_kind_hip_runtime(), op, corr, pat.args_bytes(op))
+            ext = C.c_uint64(500 + corr % 4)
+            assert eng.lib.ktj_submit_sdk_api_record(eng.h, rec, t0, t1, pid, tid, C.byref(ext) if corr % 2 == 0 else None, None) == 0
+            sim.ktjsim_sdk_api_record_free(rec)
+
+        for call in calls[:half]:
+            as_sdk_record(call)
+        rows = (abi.RuntimeRec * (tail - half))()
+        pairs = []
+        for k, (op, corr, t0, t1, pid, tid) in enumerate(calls[half:tail]):
+            sim.ktjsim_sdk_api_row(op, corr, pat.args_bytes(op), t0, t1, pid, tid, C.byref(rows[k]))
+            rows[k].id = corr
+            if corr % 2 == 0:
+                pairs.append(abi.ExtCorrRec(corr, 500 + corr % 4))
+        assert eng.lib.ktj_submit_records(eng.h, abi.KTJ_REC_RUNTIME, rows, len(rows)) == 0
+        ext_arr = (abi.ExtCorrRec * len(pairs))(*pairs)
+        assert eng.lib.ktj_submit_records(eng.h, abi.KTJ_REC_EXTCORR, ext_arr, len(pairs)) == 0
+        for call in calls[tail:]:
+            as_sdk_record(call)
+        out = torch.zeros(len(want) + 4096, dtype=torch.uint8, device="cuda:0")
+        n = C.c_uint64()
+        KTJ_ERR_STATE = -2
+        assert eng.lib.ktj_process_noalloc(eng.h, eng.end_time_ns, out.data_ptr(), out.numel(), C.byref(n)) == KTJ_ERR_STATE
+        assert b"ktj_flush" in eng.lib.ktj_last_error(eng.h)
+        assert eng.lib.ktj_flush(eng.h) == 0
+        assert eng.lib.ktj_process_noalloc(eng.h, eng.end_time_ns, out.data_ptr(), out.numel(), C.byref(n)) == 0, eng.lib.ktj_last_error(eng.h)
+        assert bytes(out[:n.value].cpu().numpy()) == want
+        eng.process()
+        assert eng.output() == want
