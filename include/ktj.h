@@ -435,7 +435,7 @@ typedef struct ktj_stats {
 enum {
   KTJ_STAGE_DICT = 0,     /* name / string dictionary sanitising                               */
   KTJ_STAGE_DECODE = 1,   /* raw records → columns                                             */
-  KTJ_STAGE_CONVERT = 2,  /* clock conversion + window filter: done inside decode, reads 0            */
+  KTJ_STAGE_CONVERT = 2,  /* clock conversion + window filter: part of KTJ_STAGE_DECODE, always 0     */
   KTJ_STAGE_JOIN = 3,     /* hash build + probe (ext-corr, runtime↔device, streams)            */
   KTJ_STAGE_SORT = 4,     /* key build + stable radix sort                                     */
   KTJ_STAGE_SIZE = 5,     /* exact byte length per record                                      */
@@ -522,6 +522,15 @@ int ktj_set_window(ktj_engine* e, int64_t start_ns, int64_t end_ns);
  * call returns.  Arrival order is: all generic records, then all runtime rows, then all device
  * rows, each in submission order. */
 int ktj_submit_records(ktj_engine* e, int rec_class, const void* packed, size_t n_records);
+
+/* Page-locked host memory for record arrays (no counterpart in the reference, whose rows are heap
+ * objects: libkineto/src/RocprofLogger.h:84).  A producer that fills such a buffer and passes it to
+ * ktj_submit_records has its records copied to the GPU by DMA straight from the buffer; from ordinary
+ * memory the HIP runtime copies through a staging buffer of its own, at about half the rate.  The
+ * buffer belongs to the caller until ktj_host_free; it may be reused as soon as ktj_submit_records
+ * has returned. */
+int ktj_host_alloc(ktj_engine* e, size_t n_bytes, void** host_ptr);
+int ktj_host_free(ktj_engine* e, void* host_ptr);
 
 /* Same, for records that already live in device memory of the engine's GPU (zero copy; the
  * buffer must stay valid until ktj_finalize / ktj_process returns). */

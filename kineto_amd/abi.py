@@ -17,7 +17,6 @@ KTJ_CREATE_PAIR_SORT = 0x8
 KTJ_CREATE_DISPLAY_NS = 0x10
 KTJ_CREATE_CUDA12_ARGS = 0x20
 KTJ_GF_WIDE_DEVICE = 0x04
-KTJ_REC_GENERIC, KTJ_REC_RUNTIME, KTJ_REC_DEVICE, KTJ_REC_EXTCORR, KTJ_REC_USERCORR = 0, 1, 2, 3, 4
 
 REC_GENERIC, REC_RUNTIME, REC_DEVICE, REC_EXTCORR, REC_USERCORR = 0, 1, 2, 3, 4
 INFO_DEVICE, INFO_RESOURCE, INFO_OVERHEAD, INFO_SPAN = 0, 1, 2, 3
@@ -200,7 +199,7 @@ def load_synth():
 ENGINE_SYMBOLS = [
     "ktj_create", "ktj_destroy", "ktj_last_error", "ktj_trace_start", "ktj_intern_strings",
     "ktj_register_schema", "ktj_add_collective", "ktj_submit_args", "ktj_set_api_table", "ktj_set_clock_model",
-    "ktj_set_window", "ktj_submit_records", "ktj_submit_records_device", "ktj_submit_info", "ktj_begin_activities",
+    "ktj_set_window", "ktj_submit_records", "ktj_submit_records_device", "ktj_host_alloc", "ktj_host_free", "ktj_submit_info", "ktj_begin_activities",
     "ktj_process", "ktj_process_noalloc", "ktj_output_device", "ktj_output_host", "ktj_finalize", "ktj_get_stats",
     "ktj_version",
     # include/ktj_rocprofiler.h
@@ -255,6 +254,10 @@ def load_engine():
         lib.ktj_set_sdk_kernel_names.argtypes = [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), C.c_size_t, C.c_uint32]
         lib.ktj_submit_sdk_buffer.restype = C.c_int
         lib.ktj_submit_sdk_buffer.argtypes = [vp, C.POINTER(C.c_void_p), C.c_size_t, C.POINTER(C.c_uint64)]
+        lib.ktj_host_alloc.restype = C.c_int
+        lib.ktj_host_alloc.argtypes = [vp, C.c_size_t, C.POINTER(C.c_void_p)]
+        lib.ktj_host_free.restype = C.c_int
+        lib.ktj_host_free.argtypes = [vp, C.c_void_p]
         lib.ktj_flush.restype = C.c_int
         lib.ktj_flush.argtypes = [vp]
         lib.ktj_submit_sdk_api_record.restype = C.c_int

@@ -582,6 +582,25 @@ int ktj_submit_records(ktj_engine* e, int rec_class, const void* packed, size_t 
   return KTJ_OK;
 }
 
+int ktj_host_alloc(ktj_engine* e, size_t n_bytes, void** host_ptr) {
+  if (!e || !host_ptr) return KTJ_ERR_ARG;
+  *host_ptr = nullptr;
+  HIPCHK(hipSetDevice(e->device));
+  void* p = nullptr;
+  const hipError_t rc = hipHostMalloc(&p, n_bytes ? n_bytes : 16, hipHostMallocDefault);
+  if (rc != hipSuccess) { e->last_error = std::string("hipHostMalloc: ") + hipGetErrorString(rc); return KTJ_ERR_NOMEM; }
+  *host_ptr = p;
+  return KTJ_OK;
+}
+
+int ktj_host_free(ktj_engine* e, void* host_ptr) {
+  if (!e) return KTJ_ERR_ARG;
+  if (!host_ptr) return KTJ_OK;
+  HIPCHK(hipSetDevice(e->device));
+  HIPCHK(hipHostFree(host_ptr));
+  return KTJ_OK;
+}
+
 int ktj_submit_records_device(ktj_engine* e, int rec_class, const void* device_ptr, size_t n_records) {
   if (!e || (n_records && !device_ptr)) return KTJ_ERR_ARG;
   size_t rs = 0;
@@ -1099,7 +1118,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
    * part of KTJ_STAGE_TOTAL_GPU */
   struct { int stage, from, to; } spans[] = {
       {KTJ_STAGE_DICT, EV_START, EV_DICT},       {KTJ_STAGE_DECODE, EV_DICT, EV_DECODE},
-      {KTJ_STAGE_CONVERT, EV_DECODE, EV_CONVERT}, {KTJ_STAGE_JOIN, EV_CONVERT, EV_JOIN},
+      {KTJ_STAGE_DECODE, EV_DECODE, EV_CONVERT}, {KTJ_STAGE_JOIN, EV_CONVERT, EV_JOIN},
       {KTJ_STAGE_SORT, EV_JOIN, EV_SORT_A},      {KTJ_STAGE_SORT, EV_SORT_B, EV_SORT},
       {KTJ_STAGE_SIZE, EV_SORT, EV_SIZE},        {KTJ_STAGE_SCAN, EV_SIZE, EV_SCAN},
       {KTJ_STAGE_EMIT, EV_EMIT_START, EV_EMIT}};
@@ -1115,8 +1134,10 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   }
   const uint64_t raw_in = ng * sizeof(ktj_generic_rec) + nr * sizeof(ktj_runtime_rec) + nd * sizeof(ktj_device_rec);
   s.stage_bytes[KTJ_STAGE_DICT] = e->blob_bytes * 3;
+  /* clock conversion and window filter run inside the decode kernels on values that are in registers
+   * there: their bytes (two timestamps in, two out) are bytes of the decode stage already */
   s.stage_bytes[KTJ_STAGE_DECODE] = raw_in + N * 48;
-  s.stage_bytes[KTJ_STAGE_CONVERT] = (nr + nd) * 32;
+  s.stage_bytes[KTJ_STAGE_CONVERT] = 0;
   s.stage_bytes[KTJ_STAGE_JOIN] = nx * 12 + ng * 12 + nr * 12 + (nr + nd) * 12 * 2 +
                                    nr * (sizeof(ktj_runtime_rec) + 48 + sizeof(MatRow) + 4); /* incl. the runtime rows' joined rows */
   s.stage_bytes[KTJ_STAGE_SORT] = N * 56;

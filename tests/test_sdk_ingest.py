@@ -362,9 +362,9 @@ def test_sdk_api_records_end_to_end():
             rows[k].id = corr
             if corr % 2 == 0:
                 pairs.append(abi.ExtCorrRec(corr, 500 + corr % 4))
-        assert eng.lib.ktj_submit_records(eng.h, abi.KTJ_REC_RUNTIME, rows, len(rows)) == 0
+        assert eng.lib.ktj_submit_records(eng.h, abi.REC_RUNTIME, rows, len(rows)) == 0
         ext_arr = (abi.ExtCorrRec * len(pairs))(*pairs)
-        assert eng.lib.ktj_submit_records(eng.h, abi.KTJ_REC_EXTCORR, ext_arr, len(pairs)) == 0
+        assert eng.lib.ktj_submit_records(eng.h, abi.REC_EXTCORR, ext_arr, len(pairs)) == 0
         for call in calls[tail:]:
             as_sdk_record(call)
         out = torch.zeros(len(want) + 4096, dtype=torch.uint8, device="cuda:0")
