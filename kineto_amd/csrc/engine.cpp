@@ -163,7 +163,7 @@ struct ktj_engine {
   /* working buffers */
   DevBuf d_scalars, d_name_len, d_arg_len, d_sflags, d_name_off, d_arg_off, d_name_blob, d_arg_blob;
   DevBuf c_ts, c_dur, c_corr, c_dev, c_res, c_meta, c_ext;
-  DevBuf t_full, t_narrow, t_cpu, f_has_runtime, f_first, f_stream_src, f_pay, n_ext_src, n_kern_src, n_copy_src, n_pay, slot_ext, slot_f, slot_n, dev_link, dev_brief, sync_keys, sync_pos, sync_first;
+  DevBuf t_full, t_narrow, t_cpu, f_has_runtime, f_first, f_stream_src, f_pay, n_ext_src, n_kern_src, n_copy_src, n_pay, slot_f, slot_n, dev_link, dev_brief, sync_keys, sync_pos, sync_first;
   DevBuf q_keys, q_stream, q_amb, dn_hash, dn_first, dn_dev, dn_key, dn_rank, range_parts;
   DevBuf s_dev_k, s_dev_r, s_res_k, s_res_r;
   DevBuf keys_a, keys_b, vals_a, vals_b, hist, scan_tmp;
@@ -803,7 +803,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   NEED(e->f_has_runtime, (cap_full / 32 + 2ull) * 4);
   NEED(e->n_ext_src, (cap_narrow + 1ull) * 4); NEED(e->n_kern_src, (cap_narrow + 1ull) * 4);
   NEED(e->n_copy_src, (cap_narrow + 1ull) * 4); NEED(e->n_pay, (cap_narrow + 1ull) * sizeof(NarrowPay));
-  NEED(e->slot_ext, nx * 4 + 16); NEED(e->slot_f, nr * 4 + 16); NEED(e->slot_n, nr * 4 + 16);
+  NEED(e->slot_f, nr * 4 + 16); NEED(e->slot_n, nr * 4 + 16);
   NEED(e->dev_link, nd * sizeof(DevLink) + 16);
   NEED(e->dev_brief, nd * sizeof(DevBrief) + 16);
   NEED(e->q_keys, (KTJ_QUEUE_CAP + 1ull) * 8); NEED(e->q_stream, (KTJ_QUEUE_CAP + 1ull) * 8);
@@ -920,9 +920,8 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   }
   ApiTable api{e->d_cid_names.as<uint32_t>(), (uint32_t)e->cid_names.size(), e->d_flow_bits.as<uint32_t>(), e->malloc_cid};
   MatRow* mat = e->mat.as<MatRow>();
-  HIPCHK(build_extcorr(x_recs, nx, tn, nc, e->slot_ext.as<uint32_t>(), sc, st));
   HIPCHK(build_cpu_ids(g_recs, ng, t_cpu, cpu_row, sc, st));
-  HIPCHK(resolve_external(x_recs, nx, nc, e->slot_ext.as<uint32_t>(), t_cpu, cpu_row, g_recs, ctx, st));
+  HIPCHK(build_extcorr(x_recs, nx, tn, nc, t_cpu, cpu_row, g_recs, ctx, sc, st));
   HIPCHK(join_runtime_rows(r_recs, nr, c, ng, api, tf, fc, tn, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), ctx, mat,
                            e->len.as<uint32_t>(), sc, st));
   HIPCHK(republish_runtime_rows(r_recs, nr, c, ng, fc, nc, e->slot_f.as<uint32_t>(), e->slot_n.as<uint32_t>(), sc, st));

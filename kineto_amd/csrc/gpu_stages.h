@@ -133,6 +133,7 @@ struct Scalars {
   unsigned int runtime_ids_repeat;    /* two runtime rows share a slot of the full table */
   unsigned int n_queues;              /* distinct hardware queues entered into the queue -> stream table */
   unsigned int n_sync_rows;           /* distinct (device, row) pairs of Stream Sync activities */
+  unsigned int ext_ids_repeat;        /* two external-correlation records share a correlation id */
   alignas(256) JoinPlan plan;         /* key ranges and modes of the join tables: read by every row of the join
                                          kernels, so kept off the cache lines that take the counters' atomics */
 };
@@ -218,12 +219,10 @@ hipError_t plan_tables(const KeyRange* parts, uint64_t n_generic, uint64_t n_run
                        const ktj_extcorr_rec* e, uint64_t n_ext, uint32_t cap_full, uint32_t cap_narrow, uint32_t cap_cpu,
                        bool force_hash, Scalars* sc, hipStream_t st);
 hipError_t clear_tables(Table tf, FullCols fc, Table tn, NarrowCols nc, Table cpu, hipStream_t st);
-hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, uint32_t* slot_ext, Scalars* sc,
-                         hipStream_t st);
 hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, uint32_t* cpu_row, Scalars* sc, hipStream_t st);
-/* the build passes read the columns only (correlation id, kind and has-stream bits of meta) */
-hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
-                            const uint32_t* cpu_row, const ktj_generic_rec* g, EmitCtx ctx, hipStream_t st);
+/* after build_cpu_ids: enters the external-correlation records and resolves their external ids */
+hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, Table cpu, const uint32_t* cpu_row,
+                         const ktj_generic_rec* g, EmitCtx ctx, Scalars* sc, hipStream_t st);
 hipError_t collective_first(const MatRow* mat, const uint32_t* perm, uint64_t n_rows, uint32_t n_coll, uint32_t* first,
                             hipStream_t st);
 /* per device row: "External id", timestamp-order check, stream of the launching row, and the

@@ -187,7 +187,7 @@ __global__ void k_init_scalars(Scalars* s) {
     s->ts_min_biased = ~0ULL; s->ts_max_biased = 0;
     s->out_of_range = 0; s->out_of_order = 0; s->n_flow = 0; s->n_linked = 0; s->n_blank_names = 0; s->n_valid = 0;
     s->n_unresolved = 0; s->n_sync_typed = 0; s->n_device_orphans = 0; s->error = 0; s->have_stream_src = 0; s->n_dev_ranks = 0; s->n_res_ranks = 0; s->n_dense = 0; s->runtime_ids_repeat = 0;
-    s->n_queues = 0; s->n_sync_rows = 0;
+    s->n_queues = 0; s->n_sync_rows = 0; s->ext_ids_repeat = 0;
     for (int k = 0; k < 3; ++k) {
       s->plan.range[k].lo = ~0ULL; s->plan.range[k].hi = 0;
       s->plan.ctl[k].base = 0; s->plan.ctl[k].span = 0; s->plan.ctl[k].direct = 0; s->plan.ctl[k].pad = 0;
@@ -754,10 +754,11 @@ __device__ __forceinline__ void clear_keys(const Table& t) {
 }
 __device__ __forceinline__ void clear_full(const Table& t, const FullCols& c) {
   const uint64_t n = table_extent(t);
-  FullPay z; z.first_ts = 0; z.stream = 0;
+  /* the payload is not cleared: every runtime row writes all of its slot's payload, and a slot
+   * without a runtime row (its bit in has_runtime is clear) is never read */
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i <= n; i += (uint64_t)gridDim.x * blockDim.x) {
     const uint64_t k = i < n ? i : t.mask + 1ull; /* the last iteration clears the reserved slot */
-    c.first[k] = 0xFFFFFFFFu; c.stream_src[k] = 0; c.pay[k] = z;
+    c.first[k] = 0xFFFFFFFFu; c.stream_src[k] = 0;
   }
   /* the bitmap: whole words up to the extent, and the word of the reserved slot */
   const uint64_t words = (n + 31) / 32;
@@ -813,14 +814,45 @@ hipError_t clear_tables(Table tf, FullCols fc, Table tn, NarrowCols nc, Table cp
   return KTJ_LAUNCH_CHECK();
 }
 
-/* cpuCorrelationMap_[correlation] = externalId: RocmActivityProfiler.cpp:135-148 */
-__global__ void k_build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, uint32_t* slot_ext, Scalars* sc) {
+/* What linkedActivity() (GenericActivityProfiler.cpp:397-408) finds for an external id: the slot's
+ * "External id" value and link flags, or zeros when no CPU op has the id. */
+__device__ __forceinline__ void resolved_external(uint64_t ext_id, const Table& cpu, const uint32_t* cpu_row, const ktj_generic_rec* g,
+                                                  const EmitCtx& ctx, int32_t* ext_val, uint32_t* info) {
+  *ext_val = 0;
+  *info = 0;
+  const uint32_t cs = slot_find(cpu, ext_id);
+  if (cs == KTJ_NOSLOT) return;
+  *ext_val = (int32_t)(int64_t)ext_id;
+  *info = KTJ_NP_LINKED;
+  if (cpu_row) { /* the linked op is the last record with that id (activityMap_, GenericActivityProfiler.cpp:262) */
+    const uint32_t row = cpu_row[cs];
+    if (row) *info |= collective_for_linked(g[row - 1], ctx) << KTJ_NP_COLL_SHIFT;
+  }
+}
+/* cpuCorrelationMap_[correlation] = externalId: RocmActivityProfiler.cpp:135-148.  The last record of
+ * a correlation id stays (atomicMax over the record index).  Every record resolves its external id
+ * against the CPU-op ids at once and writes the result into the slot: that is final when no two
+ * records share a correlation id, which the returning atomicMax tells; only otherwise
+ * k_resolve_external lets the winners write again.  The CPU-op ids are in their table already, the
+ * table was cleared, and the runtime rows come later. */
+__global__ void k_build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, Table cpu, const uint32_t* cpu_row,
+                                const ktj_generic_rec* g, EmitCtx ctx, Scalars* sc) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const uint32_t slot = slot_insert(tn, e[i].correlation);
-  slot_ext[i] = slot;
-  if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
-  atomicMax(&nc.ext_src[slot], (uint32_t)i + 1u);
+  bool repeats = false;
+  if (i < n) {
+    const ktj_extcorr_rec rec = e[i];
+    const uint32_t slot = slot_insert(tn, rec.correlation);
+    if (slot == KTJ_NOSLOT) flag_error(sc, KTJ_DEVERR_TABLE_FULL);
+    else {
+      repeats = atomicMax(&nc.ext_src[slot], (uint32_t)i + 1u) != 0u;
+      int32_t ext_val;
+      uint32_t info;
+      resolved_external(rec.external_id, cpu, cpu_row, g, ctx, &ext_val, &info);
+      if (info != 0) { nc.pay[slot].ext_val = ext_val; nc.pay[slot].info = info; }
+    }
+  }
+  /* one store per workgroup at most: every lane storing the same flag would queue up in L2 */
+  if (__syncthreads_or(repeats ? 1 : 0) && threadIdx.x == 0) sc->ext_ids_repeat = 1;
 }
 /* activityMap_[act->correlationId()] = act: GenericActivityProfiler.cpp:262 */
 /* cpu_row (optional): per slot, 1 + index of the last record with that id, for the traces whose
@@ -832,24 +864,20 @@ __global__ void k_build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu,
   if (slot == KTJ_NOSLOT) { flag_error(sc, KTJ_DEVERR_TABLE_FULL); return; }
   if (cpu_row) atomicMax(&cpu_row[slot], (uint32_t)i + 1u);
 }
-/* linkedActivity(): GenericActivityProfiler.cpp:397-408.  The record that won the slot resolves
- * its external id against the CPU-op ids once, for every row that will read the slot. */
-__global__ void k_resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
-                                   const uint32_t* cpu_row, const ktj_generic_rec* g, EmitCtx ctx) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const uint32_t slot = slot_ext[i];
-  if (slot == KTJ_NOSLOT || nc.ext_src[slot] != (uint32_t)i + 1u) return;
-  const uint64_t ext_id = e[i].external_id;
-  const uint32_t cs = slot_find(cpu, ext_id);
-  if (cs != KTJ_NOSLOT) {
-    nc.pay[slot].ext_val = (int32_t)(int64_t)ext_id;
-    uint32_t info = KTJ_NP_LINKED;
-    if (cpu_row) { /* the linked op is the last record with that id (activityMap_, GenericActivityProfiler.cpp:262) */
-      const uint32_t row = cpu_row[cs];
-      if (row) info |= collective_for_linked(g[row - 1], ctx) << KTJ_NP_COLL_SHIFT;
-    }
-    nc.pay[slot].info = info; /* the table was cleared, and the runtime rows come later */
+/* Only when external-correlation records share a correlation id: the record that won the slot
+ * writes what it resolved again, zeros included, over whatever the other records of the id left. */
+__global__ void k_resolve_external(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, Table cpu,
+                                   const uint32_t* cpu_row, const ktj_generic_rec* g, EmitCtx ctx, const Scalars* sc) {
+  if (sc->ext_ids_repeat == 0) return;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const ktj_extcorr_rec rec = e[i];
+    const uint32_t slot = slot_find(tn, rec.correlation);
+    if (slot == KTJ_NOSLOT || nc.ext_src[slot] != (uint32_t)i + 1u) continue;
+    int32_t ext_val;
+    uint32_t info;
+    resolved_external(rec.external_id, cpu, cpu_row, g, ctx, &ext_val, &info);
+    nc.pay[slot].ext_val = ext_val;
+    nc.pay[slot].info = info;
   }
 }
 __device__ __forceinline__ bool is_async_op(uint32_t domain) { return domain != KTJ_DOM_MEMSET; }
@@ -886,7 +914,11 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Tabl
     fp.first_ts = 0; fp.stream = 0;
     uint32_t runtime_bits = 0;
     if (sn != KTJ_NOSLOT) np = nc.pay[sn];
-    if (sf != KTJ_NOSLOT) { fp = fc.pay[sf]; runtime_bits = fc.has_runtime[sf >> 5]; }
+    if (sf != KTJ_NOSLOT) {
+      fp = fc.pay[sf];
+      runtime_bits = fc.has_runtime[sf >> 5];
+      if (!((runtime_bits >> (sf & 31u)) & 1u)) { fp.first_ts = 0; fp.stream = 0; } /* no runtime row wrote this slot in this pass */
+    }
     DevLink l;
     l.p[0] = l.p[1] = l.p[2] = 0; l.flags = 0; l.coll = 0;
     if (sn != KTJ_NOSLOT) {
@@ -940,22 +972,18 @@ __global__ void k_device_orphans(uint64_t n, Columns c, uint64_t first_device, T
   block_add(&sc->out_of_order, n_bad);
 }
 
-hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, uint32_t* slot_ext, Scalars* sc,
-                         hipStream_t st) {
-  if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_build_extcorr, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, tn, nc, slot_ext, sc);
-  return KTJ_LAUNCH_CHECK();
-}
 hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, uint32_t* cpu_row, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
   hipLaunchKernelGGL(k_build_cpu_ids, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, g, n, cpu, cpu_row, sc);
   return KTJ_LAUNCH_CHECK();
 }
-hipError_t resolve_external(const ktj_extcorr_rec* e, uint64_t n, NarrowCols nc, const uint32_t* slot_ext, Table cpu,
-                            const uint32_t* cpu_row, const ktj_generic_rec* g, EmitCtx ctx, hipStream_t st) {
+/* after build_cpu_ids: the external ids are resolved against that table as the records pass */
+hipError_t build_extcorr(const ktj_extcorr_rec* e, uint64_t n, Table tn, NarrowCols nc, Table cpu, const uint32_t* cpu_row,
+                         const ktj_generic_rec* g, EmitCtx ctx, Scalars* sc, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_resolve_external, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, nc, slot_ext, cpu, cpu_row,
-                     g, ctx);
+  hipLaunchKernelGGL(k_build_extcorr, dim3(grid_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, tn, nc, cpu, cpu_row, g, ctx, sc);
+  hipLaunchKernelGGL(k_resolve_external, dim3(grid_stride_for(n, KTJ_BLOCK)), dim3(KTJ_BLOCK), 0, st, e, n, tn, nc, cpu, cpu_row, g,
+                     ctx, (const Scalars*)sc);
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t link_device_rows(uint64_t n, Columns c, uint64_t first_device, Table tf, FullCols fc, Table tn, NarrowCols nc,
