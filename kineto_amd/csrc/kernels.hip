@@ -1678,10 +1678,36 @@ k_sortp_hist(const uint64_t* words, uint64_t n, uint32_t shift, uint32_t* hist, 
   __syncthreads();
   for (int d = threadIdx.x; d < P::NB; d += THREADS) hist[(uint64_t)d * n_blocks + blockIdx.x] = h[d];
 }
+/* The per-tile digit counts (digit-major: hist[d * n_blocks + tile]) become, for every digit, the
+ * running count over the tiles before each tile, and the digit's total goes to totals[d]: workgroup
+ * d scans row d, every thread a contiguous piece of it.  One launch; the digits' own offsets (a scan
+ * over 256 totals) are left to every scatter workgroup. */
+template <int THREADS>
+__global__ void __launch_bounds__(THREADS)
+k_sortp_scan_digits(uint32_t* hist, uint32_t n_blocks, uint32_t* totals) {
+  __shared__ uint32_t wave_tot[THREADS / 64];
+  uint32_t* row = hist + (uint64_t)blockIdx.x * n_blocks;
+  const uint32_t per = (n_blocks + THREADS - 1) / THREADS;
+  const uint32_t lo = threadIdx.x * per < n_blocks ? threadIdx.x * per : n_blocks;
+  const uint32_t hi = lo + per < n_blocks ? lo + per : n_blocks;
+  uint32_t sum = 0;
+  for (uint32_t t = lo; t < hi; ++t) sum += row[t];
+  uint32_t inc = sum;
+  const uint32_t lane = lane_id(), w = threadIdx.x >> 6;
+  for (int o = 1; o < 64; o <<= 1) { const uint32_t v = __shfl_up(inc, o); if (lane >= (uint32_t)o) inc += v; }
+  if (lane == 63) wave_tot[w] = inc;
+  __syncthreads();
+  uint32_t run = inc - sum;
+  uint32_t all = 0;
+  for (uint32_t k = 0; k < THREADS / 64; ++k) { if (k < w) run += wave_tot[k]; all += wave_tot[k]; }
+  for (uint32_t t = lo; t < hi; ++t) { const uint32_t c = row[t]; row[t] = run; run += c; }
+  if (threadIdx.x == 0) totals[blockIdx.x] = all;
+}
+
 template <int BITS, int THREADS, int MODE>
 __global__ void __launch_bounds__(THREADS)
 k_sortp_scatter(const uint64_t* in, uint64_t* words_out, uint32_t* perm_out, uint64_t n, uint32_t shift, uint32_t idx_bits,
-                const uint32_t* hist_scanned, uint32_t n_blocks) {
+                const uint32_t* hist_scanned, const uint32_t* totals, uint32_t n_blocks) {
   using P = SortP<BITS, THREADS>;
   constexpr bool FROM_KEYS = MODE == SORTP_KEYS_TO_WORDS || MODE == SORTP_KEYS_TO_PERM;
   constexpr bool TO_PERM = MODE == SORTP_WORDS_TO_PERM || MODE == SORTP_KEYS_TO_PERM;
@@ -1691,12 +1717,26 @@ k_sortp_scatter(const uint64_t* in, uint64_t* words_out, uint32_t* perm_out, uin
   __shared__ uint32_t digit_start[P::NB];        /* start of the digit's run inside the tile     */
   __shared__ uint32_t base_of[P::NB];            /* global offset of this tile's run per digit   */
   __shared__ uint32_t wave_tot[P::WAVES];
-  for (int d = threadIdx.x; d < P::NB; d += THREADS) {
-    base_of[d] = hist_scanned != nullptr ? hist_scanned[(uint64_t)d * n_blocks + blockIdx.x] : 0u;
-    for (int k = 0; k < P::WAVES; ++k) wave_run[k][d] = 0;
+  const uint32_t w = threadIdx.x >> 6, lane = lane_id();
+  {
+    /* where a digit's run begins in the output: the totals of the digits before it, scanned here by
+     * every workgroup (256 values), plus the count of that digit in the tiles before this one */
+    static_assert(P::NB <= THREADS, "a thread scans one digit's total");
+    uint32_t tot = 0;
+    if (hist_scanned != nullptr && (int)threadIdx.x < P::NB) tot = totals[threadIdx.x];
+    uint32_t inc = tot;
+    for (int o = 1; o < 64; o <<= 1) { const uint32_t v = __shfl_up(inc, o); if (lane >= (uint32_t)o) inc += v; }
+    if (lane == 63) wave_tot[w] = inc;
+    __syncthreads();
+    uint32_t digit_base = inc - tot;
+    for (uint32_t k = 0; k < w; ++k) digit_base += wave_tot[k];
+    if ((int)threadIdx.x < P::NB) {
+      const int d = (int)threadIdx.x;
+      base_of[d] = hist_scanned != nullptr ? digit_base + hist_scanned[(uint64_t)d * n_blocks + blockIdx.x] : 0u;
+      for (int k = 0; k < P::WAVES; ++k) wave_run[k][d] = 0;
+    }
   }
   __syncthreads();
-  const uint32_t w = threadIdx.x >> 6, lane = lane_id();
   const uint64_t lt = lanemask_lt();
   const uint64_t tile_base = (uint64_t)blockIdx.x * P::TILE;
   const uint64_t chunk = tile_base + (uint64_t)w * P::WAVE_KEYS;
@@ -1799,30 +1839,32 @@ static hipError_t sort_packed_t(Columns c, uint64_t n, SortSets s, const Scalars
   /* one tile: a pass needs no counts from other tiles, so no count and scan launches */
   const bool single = n_blocks == 1;
   uint32_t* counts = single ? nullptr : hist;
+  /* the digits' totals live behind the counts (radix_tmp_elems leaves 256 spare entries) */
+  uint32_t* totals = hist + (uint64_t)P::NB * n_blocks;
+  static_assert(P::NB <= 256, "room for the totals behind the counts");
+  (void)scan_tmp;
   hipLaunchKernelGGL((k_sortp_make_keys<BITS, THREADS>), g, b, 0, st, c, n, s, sc, ts_bits, res_bits, key_bits, buf_a, counts, n_blocks);
-  hipError_t e = single ? hipSuccess : scan_u32_inplace(hist, (uint64_t)P::NB * n_blocks, scan_tmp, st);
-  if (e != hipSuccess) return e;
+  if (!single) hipLaunchKernelGGL((k_sortp_scan_digits<THREADS>), dim3(P::NB), b, 0, st, hist, n_blocks, totals);
   if (passes == 1) {
     hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_KEYS_TO_PERM>), g, b, 0, st, (const uint64_t*)buf_a, buf_b, perm, n,
-                       0u, idx_bits, (const uint32_t*)counts, n_blocks);
+                       0u, idx_bits, (const uint32_t*)counts, (const uint32_t*)totals, n_blocks);
     return KTJ_LAUNCH_CHECK();
   }
   hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_KEYS_TO_WORDS>), g, b, 0, st, (const uint64_t*)buf_a, buf_b, perm, n,
-                     0u, idx_bits, (const uint32_t*)counts, n_blocks);
+                     0u, idx_bits, (const uint32_t*)counts, (const uint32_t*)totals, n_blocks);
   uint64_t* in = buf_b; uint64_t* out = buf_a;
   for (uint32_t p = 1; p < passes; ++p) {
     const uint32_t shift = idx_bits + (p - 1u) * BITS;
     if (!single) {
       hipLaunchKernelGGL((k_sortp_hist<BITS, THREADS>), g, b, 0, st, (const uint64_t*)in, n, shift, hist, n_blocks);
-      e = scan_u32_inplace(hist, (uint64_t)P::NB * n_blocks, scan_tmp, st);
-      if (e != hipSuccess) return e;
+      hipLaunchKernelGGL((k_sortp_scan_digits<THREADS>), dim3(P::NB), b, 0, st, hist, n_blocks, totals);
     }
     if (p + 1 == passes)
       hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_WORDS_TO_PERM>), g, b, 0, st, (const uint64_t*)in, out, perm, n,
-                         shift, idx_bits, (const uint32_t*)counts, n_blocks);
+                         shift, idx_bits, (const uint32_t*)counts, (const uint32_t*)totals, n_blocks);
     else
       hipLaunchKernelGGL((k_sortp_scatter<BITS, THREADS, SORTP_WORDS_TO_WORDS>), g, b, 0, st, (const uint64_t*)in, out, perm, n,
-                         shift, idx_bits, (const uint32_t*)counts, n_blocks);
+                         shift, idx_bits, (const uint32_t*)counts, (const uint32_t*)totals, n_blocks);
     uint64_t* t = in; in = out; out = t;
   }
   return KTJ_LAUNCH_CHECK();
