@@ -94,3 +94,31 @@ def test_engine_on_seeded_memset_rows():
         sp = cm.stream(cm.random_rows(seed, n=3000), cuda12=seed != 1).build()
         tp._engine_vs_oracle(sp)
         tp._engine_vs_oracle(sp, hash_join=True, tile_emit=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not HAVE_DRIVER, reason="oracle/_ref/cupti_ref_driver is built only where the reference's sources are")
+@pytest.mark.parametrize("seed", range(4))
+def test_real_cuda_wrappers_through_the_shim(seed, tmp_path):
+    """The reference's own CUDA activity wrappers (runtime and driver API calls, overhead,
+    synchronization, CUDA events, memcpy, peer-to-peer memcpy, memset; libkineto/src/CuptiActivity.h),
+    some linked to CPU ops, logged through the reference's ChromeTraceLogger and through the
+    GpuChromeTraceLogger shim by oracle/_ref/cupti_ref_driver: the two files must be identical.
+    (Kernel wrappers are left out: their metadata asks the CUDA runtime for device properties.)"""
+    import subprocess
+    ref, shim = tmp_path / "ref.json", tmp_path / "shim.json"
+    print(f"cuda wrappers through the shim, seed={seed}", flush=True)
+    out = subprocess.run([cm.CUPTI_REF_DRIVER, "log", str(seed), str(ref), str(shim)], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                         timeout=120)
+    assert out.returncode == 0, out.stderr.decode("latin1")[-2000:]
+    assert out.stdout.decode().startswith("activities 166")
+    a = ref.read_bytes().replace(str(ref).encode(), b"FILE")
+    b = shim.read_bytes().replace(str(shim).encode(), b"FILE")
+    assert a.count(b'"ph": "X"') == 166
+    for cat in (b'"cuda_runtime"', b'"cuda_driver"', b'"overhead"', b'"cuda_sync"', b'"cuda_event"', b'"gpu_memcpy"', b'"gpu_memset"', b'"cpu_op"'):
+        assert cat in a, cat
+    assert b'"graph node id"' in a and b'"External id"' in a
+    if a != b:
+        import test_gpu_parity as tp
+        i = tp._first_diff(a, b)
+        raise AssertionError(f"files differ at byte {i}:\nREF : {a[max(0, i - 300):i + 200]!r}\nSHIM: {b[max(0, i - 300):i + 200]!r}")
