@@ -315,11 +315,9 @@ hipError_t stream_sync_first(const uint32_t* perm, uint64_t n_sorted, const ktj_
 /* generic records whose rows start at arrival index `first` */
 hipError_t mat_generic_rows(const ktj_generic_rec* g, uint64_t n, uint64_t first, EmitCtx ctx, const uint32_t* sync_first,
                             MatRow* mat, uint32_t* len, Scalars* sc, hipStream_t st);
-/* runtime rows: also publishes what device rows take over (first timestamp, stream, grid, size)
- * into the tables, reads the "External id" and counts timestamp-order violations; runs after
- * resolve_external and before link_device_rows */
-/* the pass over the runtime rows: table updates, payload for the device rows, joined rows and lengths;
- * resolve_external must have run */
+/* the pass over the runtime rows: publishes what device rows take over (first timestamp, stream, grid,
+ * size) into the tables, reads the "External id", makes the joined rows and their lengths; runs
+ * after build_extcorr and before link_device_rows */
 hipError_t join_runtime_rows(const ktj_runtime_rec* r, uint64_t n, Columns c, uint64_t first, ApiTable api, Table tf, FullCols fc,
                              Table tn, NarrowCols nc, uint32_t* slot_f, uint32_t* slot_n, EmitCtx ctx, MatRow* mat,
                              uint32_t* len, Scalars* sc, hipStream_t st);
