@@ -175,6 +175,10 @@ struct ktj_engine {
   /* ktj_process_noalloc: working buffers are carved out of the library's static scratch array */
   bool noalloc = false;
   char* arena = nullptr; size_t arena_cap = 0, arena_used = 0;
+  /* ktj_process: one allocation that the working buffers of a pass are carved out of */
+  DevBuf pool;
+  size_t pool_used = 0, pool_need = 0;
+  bool measuring = false;
   char* pinned_out = nullptr; size_t pinned_out_cap = 0;
   char* file_stage[2] = {nullptr, nullptr};   /* pinned staging of the file sink, at most KTJ_FILE_STAGE_BYTES each */
   size_t file_stage_cap[2] = {0, 0};
@@ -232,7 +236,21 @@ std::string default_file_name() { /* output_json.cpp:65-70, 481-483 */
  * may not allocate it becomes the next piece of the scratch array (256-byte aligned), or the pass
  * fails with KTJ_ERR_LIMIT. */
 int need(ktj_engine* e, DevBuf& b, size_t bytes) {
-  if (!e->noalloc) { HIPCHK(b.ensure(bytes)); return KTJ_OK; }
+  if (!e->noalloc) {
+    /* The working buffers of a pass share one allocation, the pool: a first pass then makes a handful
+     * of allocations instead of sixty.  The pass first asks for everything with `measuring` set, which
+     * only adds the sizes up, sizes the pool, and asks again.  What does not fit (buffers whose size a
+     * pass learns late) is allocated on its own as before. */
+    if (e->measuring) { e->pool_need += (bytes + 255) & ~(size_t)255; return KTJ_OK; }
+    const size_t off = (e->pool_used + 255) & ~(size_t)255;
+    if (e->pool.p && off <= e->pool.cap && bytes <= e->pool.cap - off) {
+      b.borrow(static_cast<char*>(e->pool.p) + off, bytes);
+      e->pool_used = off + bytes;
+      return KTJ_OK;
+    }
+    HIPCHK(b.ensure(bytes));
+    return KTJ_OK;
+  }
   const size_t off = (e->arena_used + 255) & ~(size_t)255;
   if (off > e->arena_cap || bytes > e->arena_cap - off) {
     e->last_error = "ktj_process_noalloc: the trace needs more than the " + std::to_string(e->arena_cap) +
@@ -252,7 +270,10 @@ int need(ktj_engine* e, DevBuf& b, size_t bytes) {
 /* A small host table to the device.  A pass that may not allocate stages it through the pinned
  * buffer of the engine (allocated with the engine) instead of the runtime's own staging. */
 int upload_small(ktj_engine* e, DevBuf& dst, const void* src, size_t bytes) {
-  NEED(dst, bytes ? bytes : 16);
+  /* these tables outlive the pass (they are uploaded only when they change), so outside a pass that
+   * may not allocate they keep allocations of their own rather than a piece of the pass's pool */
+  if (e->noalloc) NEED(dst, bytes ? bytes : 16);
+  else HIPCHK(dst.ensure(bytes ? bytes : 16));
   if (bytes && e->noalloc) {
     if (bytes > e->pinned_small_cap) {
       e->last_error = "ktj_process_noalloc: a table of " + std::to_string(bytes) + " bytes exceeds the pinned staging buffer";
@@ -785,6 +806,14 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
 
   /* working memory */
   const uint32_t ns = (uint32_t)e->n_strings;
+  if (nx >= 0x7FFFFFFFull || nr >= 0x7FFFFFFFull) { e->last_error = "more than 2^31 - 2 records of one class"; return KTJ_ERR_LIMIT; }
+  /* capacities for the hash mode (load <= 2/3); the direct mode uses a prefix of the same buffers */
+  const uint32_t cap_full = pow2_at_least((nr + nd) + (nr + nd) / 2);
+  const uint32_t cap_narrow = pow2_at_least((nx + nr) + (nx + nr) / 2), cap_cpu = pow2_at_least(2 * ng);
+  e->pool_used = 0;
+  for (int phase = e->noalloc ? 1 : 0; phase < 2; ++phase) { /* 0: add the sizes up and size the pool; 1: hand the buffers out */
+  e->measuring = phase == 0;
+  e->pool_need = 0;
   NEED(e->d_name_len, (ns + 1) * 4ull); NEED(e->d_arg_len, (ns + 1) * 4ull);
   NEED(e->d_sflags, (ns + 1) * 4ull);
   NEED(e->d_name_off, (ns + 2) * 8ull); NEED(e->d_arg_off, (ns + 2) * 8ull);
@@ -792,10 +821,6 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   NEED(e->c_ts, Na * 8); NEED(e->c_dur, Na * 8); NEED(e->c_corr, Na * 8);
   NEED(e->c_dev, Na * 8); NEED(e->c_res, Na * 8); NEED(e->c_meta, Na * 4);
   NEED(e->c_ext, Na * 4);
-  if (nx >= 0x7FFFFFFFull || nr >= 0x7FFFFFFFull) { e->last_error = "more than 2^31 - 2 records of one class"; return KTJ_ERR_LIMIT; }
-  /* capacities for the hash mode (load <= 2/3); the direct mode uses a prefix of the same buffers */
-  const uint32_t cap_full = pow2_at_least((nr + nd) + (nr + nd) / 2);
-  const uint32_t cap_narrow = pow2_at_least((nx + nr) + (nx + nr) / 2), cap_cpu = pow2_at_least(2 * ng);
   NEED(e->t_full, (cap_full + 1ull) * 8); NEED(e->t_narrow, (cap_narrow + 1ull) * 8);
   NEED(e->t_cpu, (cap_cpu + 1ull) * 8);
   NEED(e->f_first, (cap_full + 1ull) * 4); NEED(e->f_stream_src, (cap_full + 1ull) * 4);
@@ -826,6 +851,11 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   }
   NEED(e->mat, Na * sizeof(MatRow)); NEED(e->len, Na * 4); NEED(e->len_sorted, Na * 4); NEED(e->kind_sorted, Na + 16);
   NEED(e->offs, (Na + 1) * 8);
+  if (e->measuring) {
+    e->measuring = false;
+    if (e->pool.cap < e->pool_need + 4096) HIPCHK(e->pool.ensure(e->pool_need + 4096));
+  }
+  }
 
   Scalars* sc = e->d_scalars.as<Scalars>();
   Columns c;
