@@ -247,6 +247,7 @@ struct CountWriter {
   typedef uint32_t Prepared;
   KTJ_HD KTJ_FI static Prepared prepare(uint64_t v) { return (uint32_t)ndigits_u64(v); }
   KTJ_HD KTJ_FI void num(Prepared len) { n += len; }
+  KTJ_HD KTJ_FI void relief() {}
 };
 
 /* A decimal number rendered once and appended several times (pid, tid and ts appear in the
@@ -320,6 +321,7 @@ struct TileWriter {
     } else fill = total;
   }
   KTJ_HD KTJ_FI void ch(char c) { append((uint64_t)(unsigned char)c, 1); }
+  KTJ_HD KTJ_FI void relief() {}
   template <unsigned N> KTJ_HD KTJ_FI void lit(const PackedLit<N>& l) {
     for (unsigned i = 0; i < N / 8; ++i) append(l.w[i], 8);
     if (N % 8) append(l.w[N / 8], N % 8);
@@ -430,11 +432,14 @@ static __device__ __attribute__((noinline)) void cooperative_word_copy(const cha
 #endif
 
 #if defined(__HIPCC__)
-/* blocks per lane in the stage; odd, so that neither the lanes' writes (same block index, lane
- * stride 16 * KTJ_STAGE_BLOCKS bytes) nor the quads' reads collide on LDS banks */
+/* blocks per lane in the stage: one 128-byte line of the document and the first five blocks of the
+ * next one; odd, so that the lanes' accesses to the same slot (lane stride 16 * KTJ_STAGE_BLOCKS
+ * bytes) do not collide on LDS banks */
 #define KTJ_STAGE_BLOCKS 13u
-#define KTJ_FLUSH_LANES 4u
-#define KTJ_FLUSH_ROUNDS ((KTJ_STAGE_BLOCKS + 2u * KTJ_FLUSH_LANES - 2u) / KTJ_FLUSH_LANES) /* blocks plus up to LANES - 1 of misalignment */
+#define KTJ_LINE_BLOCKS 8u
+/* a lane with this many slots used asks for a relief() at the next opportunity (11 and 13 measured
+ * slower: more reliefs than needed, or too late for the blocks that follow) */
+#define KTJ_RELIEF_AT 12u
 extern __shared__ __attribute__((aligned(16))) char ktj_stage_lds[];
 #endif
 
@@ -457,14 +462,18 @@ struct BlockWriter {
   bool foreign;       /* the block belongs to the predecessor: gathered but not stored */
 #if defined(__HIPCC__)
   /* Device: finished blocks do not go to the document one by one (64 lanes, 64 different lines per
-   * store instruction) but wait in LDS, up to KTJ_STAGE_BLOCKS consecutive blocks per lane, until
-   * the wavefront reaches flush(): there the four lanes of a quad write each other's blocks, four
-   * consecutive blocks of one activity per store instruction (64 contiguous bytes).  Blocks
-   * beyond the stage's capacity, and blocks after a jump of wptr, are stored directly. */
+   * store instruction, every line written sixteen bytes at a time over some microseconds) but wait
+   * in LDS.  A lane's stage mirrors the document: slot q holds the block at line_base + 16 q, so
+   * slots 0..7 are one 128-byte line and slots 8..12 the beginning of the next.  flush() and
+   * relief() write the line out once it is complete, all of it at one moment (a line written in
+   * pieces some microseconds apart leaves the L2 cache once per piece), and move the next line's
+   * blocks down.  When the stage is full, and after a jump of wptr, blocks are stored directly
+   * until the next flush(). */
   uint32_t stage_lds;   /* byte offset of this lane's stage in the workgroup's dynamic LDS */
-  uint32_t n_staged;    /* blocks waiting; staged block j belongs at stage_base + 2 j */
-  uint32_t stage_cap;   /* KTJ_STAGE_BLOCKS, or n_staged once the stage is closed until the next flush */
-  uint64_t* stage_base;
+  uint32_t q_first;     /* slot of the first waiting block (not 0 only in an activity's first line) */
+  uint32_t q_end;       /* slot behind the last waiting block; nothing waits when q_end == q_first */
+  uint32_t stage_cap;   /* KTJ_STAGE_BLOCKS, or 0 while the stage is closed */
+  uintptr_t line_base;  /* 128-byte aligned address of the line in slots 0..7 */
 #endif
 
   KTJ_HD KTJ_FI static uint64_t head_bytes() { constexpr auto h = pack_lit("\n  {\n   "); return h.w[0]; }
@@ -473,11 +482,10 @@ struct BlockWriter {
 #if defined(__HIP_DEVICE_COMPILE__)
       typedef unsigned long long v2u64 __attribute__((ext_vector_type(2)));
       v2u64 v; v.x = lo; v.y = hi;
-      if (n_staged < stage_cap) {
-        if (n_staged == 0) stage_base = wptr;
-        *reinterpret_cast<v2u64*>(ktj_stage_lds + stage_lds + n_staged * 16u) = v;
-        ++n_staged;
-      } else *reinterpret_cast<v2u64*>(wptr) = v;
+      if (q_end < stage_cap) { /* an open stage's slot q_end is the block at wptr */
+        *reinterpret_cast<v2u64*>(ktj_stage_lds + stage_lds + q_end * 16u) = v;
+        ++q_end;
+      } else { stage_cap = 0; *reinterpret_cast<v2u64*>(wptr) = v; }
 #else
       wptr[0] = lo; wptr[1] = hi;
 #endif
@@ -487,75 +495,140 @@ struct BlockWriter {
   }
 #if defined(__HIPCC__)
   __device__ KTJ_FI void stage_init(uint32_t lds_offset) {
-    stage_lds = lds_offset; n_staged = 0; stage_cap = KTJ_STAGE_BLOCKS; stage_base = nullptr;
+    stage_lds = lds_offset; q_first = q_end = 0; stage_cap = KTJ_STAGE_BLOCKS; line_base = 0;
     wptr = nullptr; lo = hi = 0; fill = 0; foreign = false;
   }
-  /* wptr is about to move by more than one block: what is staged stays, nothing more is staged */
-  __device__ KTJ_FI void stage_close() { stage_cap = n_staged; }
-  /* Every lane of the wavefront must call this together (lanes without an activity included).
-   * Unless `last`, a lane whose stage is still open (every block since the stage's first one is in
-   * it) lets only whole 128-byte lines of the document go and keeps the blocks of the line it has
-   * not finished: they move to the front of the stage and leave with the rest of their line at the
-   * next flush, so that the line reaches memory in one piece. */
-  __device__ KTJ_FI void flush(bool last) {
+  /* wptr is about to move by more than one block: what waits stays, nothing more is staged */
+  __device__ KTJ_FI void stage_close() { stage_cap = 0; }
+  /* an empty stage takes its place in the document from wptr: after begin(), and when a closed
+   * stage opens again (a block that the predecessor writes is passed over) */
+  __device__ KTJ_FI void stage_follow() {
+    const uintptr_t a = (uintptr_t)(wptr + (foreign ? 2 : 0));
+    line_base = a & ~(uintptr_t)127;
+    q_first = q_end = (uint32_t)(a >> 4) & (KTJ_LINE_BLOCKS - 1u);
+  }
+  /* Blocks leave the stage.  Slots are read and written with constant offsets, and a lane touches
+   * only its own stage: any set of lanes may come here.  stage_line: the line in slots 0..7 leaves
+   * if it is complete, and what waits of the next line moves down. */
+  __device__ KTJ_FI void stage_line() {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef unsigned long long v2u64 __attribute__((ext_vector_type(2)));
     typedef __attribute__((address_space(1))) v2u64* gptr; /* the document is global memory: no flat stores */
-    const uint32_t k = (uint32_t)threadIdx.x & 3u;
-    const uint32_t base_lo = (uint32_t)(uintptr_t)stage_base, base_hi = (uint32_t)((uintptr_t)stage_base >> 32);
-    uint32_t n_out = n_staged;
-    if (!last && n_staged < stage_cap) {
-      const uint32_t end_lo = base_lo + 16u * n_staged;         /* the low address bits decide */
-      const uint32_t whole = (end_lo & ~127u) - base_lo;        /* bytes up to the last line boundary, if any */
-      n_out = (int32_t)whole > 0 ? whole >> 4 : 0u;
+    if (q_end < KTJ_LINE_BLOCKS) return;
+    char* s = ktj_stage_lds + stage_lds;
+    v2u64 x[KTJ_STAGE_BLOCKS];
+    _Pragma("unroll")
+    for (uint32_t p = 0; p < KTJ_STAGE_BLOCKS; ++p) x[p] = *reinterpret_cast<const v2u64*>(s + p * 16u); /* all reads first: one wait */
+    gptr d = reinterpret_cast<gptr>(line_base);
+    if (q_first == 0) { /* every line but an activity's first */
+      _Pragma("unroll")
+      for (uint32_t p = 0; p < KTJ_LINE_BLOCKS; ++p) d[p] = x[p];
+    } else {
+      _Pragma("unroll")
+      for (uint32_t p = 1; p < KTJ_LINE_BLOCKS; ++p)
+        if (p >= q_first) d[p] = x[p];
     }
+    _Pragma("unroll")
+    for (uint32_t p = KTJ_LINE_BLOCKS; p < KTJ_STAGE_BLOCKS; ++p)
+      if (p < q_end) *reinterpret_cast<v2u64*>(s + (p - KTJ_LINE_BLOCKS) * 16u) = x[p];
+    line_base += 128u;
+    q_first = 0;
+    q_end -= KTJ_LINE_BLOCKS;
+#endif
+  }
+  /* every waiting block leaves (the lane's last flush, or a closed stage: the blocks behind them are
+   * in the document already) */
+  __device__ KTJ_FI void stage_all() {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef unsigned long long v2u64 __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(1))) v2u64* gptr;
+    char* s = ktj_stage_lds + stage_lds;
+    v2u64 x[KTJ_STAGE_BLOCKS];
+    _Pragma("unroll")
+    for (uint32_t p = 0; p < KTJ_STAGE_BLOCKS; ++p) x[p] = *reinterpret_cast<const v2u64*>(s + p * 16u);
+    gptr d = reinterpret_cast<gptr>(line_base);
+    _Pragma("unroll")
+    for (uint32_t p = 0; p < KTJ_STAGE_BLOCKS; ++p)
+      if (p >= q_first && p < q_end) d[p] = x[p];
+#endif
+  }
+  /* The same for the stages of whole quads: the four lanes of a quad write each other's blocks, lane
+   * k the slots k, k + 4, ... of every stage of its quad, so that a store instruction covers 64
+   * contiguous bytes per quad.  All four lanes of a quad must be here together.  CAN_ALL: stages
+   * that are closed, and every stage when `last`, are emptied (stage_all) instead. */
+  template <bool CAN_ALL> __device__ KTJ_FI void quad_write(bool last) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef unsigned long long v2u64 __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(1))) v2u64* gptr;
+    const uint32_t k = (uint32_t)threadIdx.x & 3u;
+    const bool all = CAN_ALL && (last || stage_cap == 0);
+    const bool line = q_end >= KTJ_LINE_BLOCKS;
+    const uint32_t lim = all ? q_end : (line ? KTJ_LINE_BLOCKS : 0u); /* slots [q_first, lim) leave */
+    const uint32_t lb_lo = (uint32_t)line_base, lb_hi = (uint32_t)(line_base >> 32);
+    const uint32_t quad_lds = stage_lds - k * (KTJ_STAGE_BLOCKS * 16u);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #define KTJ_QUAD_BCAST(v, t) ((uint32_t)__builtin_amdgcn_mov_dpp((int)(v), (t) * 0x55, 0xF, 0xF, true))
-#define KTJ_FLUSH_FROM(t)                                                                       \
-    {                                                                                           \
-      const uint32_t n_s = KTJ_QUAD_BCAST(n_out, t);                                            \
-      const uint32_t lds_s = KTJ_QUAD_BCAST(stage_lds, t);                                      \
-      const uint32_t lo_s = KTJ_QUAD_BCAST(base_lo, t);                                         \
-      gptr d = reinterpret_cast<gptr>(((uintptr_t)KTJ_QUAD_BCAST(base_hi, t) << 32) | (uintptr_t)lo_s); \
-      /* lane k takes the blocks whose index in the document is k mod 4: a store instruction     \
-       * then covers one aligned 64-byte piece of the activity */                                \
-      const int32_t j0 = (int32_t)k - (int32_t)((lo_s >> 4) & 3u);                              \
-      v2u64 x[KTJ_FLUSH_ROUNDS];                                                                \
-      _Pragma("unroll")                                                                         \
-      for (uint32_t m = 0; m < KTJ_FLUSH_ROUNDS; ++m) { /* all reads first: one wait for them */ \
-        const int32_t j = j0 + (int32_t)(KTJ_FLUSH_LANES * m);                                  \
-        x[m] = *reinterpret_cast<const v2u64*>(ktj_stage_lds + lds_s + ((uint32_t)j < KTJ_STAGE_BLOCKS ? (uint32_t)j : 0u) * 16u); \
-      }                                                                                         \
-      _Pragma("unroll")                                                                         \
-      for (uint32_t m = 0; m < KTJ_FLUSH_ROUNDS; ++m) {                                         \
-        const int32_t j = j0 + (int32_t)(KTJ_FLUSH_LANES * m);                                  \
-        if ((uint32_t)j < n_s) d[j] = x[m];                                                     \
-      }                                                                                         \
+    constexpr uint32_t ROUNDS = CAN_ALL ? (KTJ_STAGE_BLOCKS + 3u) / 4u : KTJ_LINE_BLOCKS / 4u;
+#define KTJ_FLUSH_FROM(t)                                                                                   \
+    {                                                                                                       \
+      const uint32_t first_t = KTJ_QUAD_BCAST(q_first, t), lim_t = KTJ_QUAD_BCAST(lim, t);                  \
+      gptr d = reinterpret_cast<gptr>(((uintptr_t)KTJ_QUAD_BCAST(lb_hi, t) << 32) | (uintptr_t)KTJ_QUAD_BCAST(lb_lo, t)); \
+      const char* s = ktj_stage_lds + quad_lds + (t) * (KTJ_STAGE_BLOCKS * 16u);                            \
+      v2u64 x[ROUNDS];                                                                                      \
+      _Pragma("unroll")                                                                                     \
+      for (uint32_t m = 0; m < ROUNDS; ++m) {                                                               \
+        const uint32_t p = k + 4u * m;                                                                      \
+        x[m] = *reinterpret_cast<const v2u64*>(s + (p < KTJ_STAGE_BLOCKS ? p : 0u) * 16u);                  \
+      }                                                                                                     \
+      _Pragma("unroll")                                                                                     \
+      for (uint32_t m = 0; m < ROUNDS; ++m) {                                                               \
+        const uint32_t p = k + 4u * m;                                                                      \
+        if (p >= first_t && p < lim_t) d[p] = x[m];                                                         \
+      }                                                                                                     \
     }
     KTJ_FLUSH_FROM(0) KTJ_FLUSH_FROM(1) KTJ_FLUSH_FROM(2) KTJ_FLUSH_FROM(3)
 #undef KTJ_FLUSH_FROM
 #undef KTJ_QUAD_BCAST
-    /* the blocks that stay move to the front (at most seven: less than a line); the wavefront's LDS
-     * accesses keep their order, so the quads have read them by now */
-    const uint32_t keep = n_staged - n_out;
-    if (keep != 0 && n_out != 0) {
-      v2u64 t[7];
+    if (all) stage_follow();
+    else if (line) { /* the next line's blocks move down; the wavefront's LDS accesses keep their order */
+      char* s = ktj_stage_lds + stage_lds;
+      v2u64 y[KTJ_STAGE_BLOCKS - KTJ_LINE_BLOCKS];
       _Pragma("unroll")
-      for (uint32_t m = 0; m < 7; ++m)
-        t[m] = *reinterpret_cast<const v2u64*>(ktj_stage_lds + stage_lds + (m < keep ? n_out + m : 0u) * 16u);
+      for (uint32_t p = KTJ_LINE_BLOCKS; p < KTJ_STAGE_BLOCKS; ++p) y[p - KTJ_LINE_BLOCKS] = *reinterpret_cast<const v2u64*>(s + p * 16u);
       _Pragma("unroll")
-      for (uint32_t m = 0; m < 7; ++m)
-        if (m < keep) *reinterpret_cast<v2u64*>(ktj_stage_lds + stage_lds + m * 16u) = t[m];
+      for (uint32_t p = KTJ_LINE_BLOCKS; p < KTJ_STAGE_BLOCKS; ++p)
+        if (p < q_end) *reinterpret_cast<v2u64*>(s + (p - KTJ_LINE_BLOCKS) * 16u) = y[p - KTJ_LINE_BLOCKS];
+      line_base += 128u;
+      q_first = 0;
+      q_end -= KTJ_LINE_BLOCKS;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    stage_base += 2u * n_out;
-    n_staged = keep;
+#endif
+  }
+  /* The three points of an activity where the whole wavefront meets (lanes without an activity
+   * included): complete lines leave, closed stages are emptied and opened again; last: everything
+   * leaves. */
+  __device__ KTJ_FI void flush(bool last) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    if (last || __any(stage_cap == 0)) quad_write<true>(last);
+    else quad_write<false>(false);
     stage_cap = KTJ_STAGE_BLOCKS;
 #endif
   }
+  /* Between flushes, wherever the formatter calls it: when a lane's stage is nearly full, every lane
+   * that is here with a complete line writes it out (whole quads together, other lanes each on its
+   * own).  Without this a full stage sends the blocks that follow straight to the document one at a
+   * time, and the lines around such a run reach memory in pieces. */
+  __device__ KTJ_FI void relief() {
+#if defined(__HIP_DEVICE_COMPILE__)
+    if (__any(stage_cap != 0 && q_end >= KTJ_RELIEF_AT)) stage_line();
+#endif
+  }
+#else
+  KTJ_HD KTJ_FI void relief() {}
 #endif
   /* pos: where the activity starts; tail_kind_before: kind of the activity before it */
   KTJ_HD KTJ_FI void begin(char* doc, uint64_t pos, uint32_t tail_kind_before, bool first);
@@ -1055,6 +1128,7 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
         default: break;
       }
       slot += fd.count;
+      w.relief();
     }
     return;
   }
@@ -1066,6 +1140,7 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
         }
         KTJ_PUT(w, "\"cid\": "); w.dec(r.aux);
         KTJ_PUT(w, ", \"correlation\": "); w.dec((uint64_t)r.flow_id);
+        w.relief();
         KTJ_PUT(w, ", \"grid\": "); put_array3(w, r.p[0] & 0xFFFFFFFFu, r.p[0] >> 32, r.p[1] & 0xFFFFFFFFu);
         KTJ_PUT(w, ", \"block\": "); put_array3(w, r.p[1] >> 32, r.p[2] & 0xFFFFFFFFu, r.p[2] >> 32);
         KTJ_PUT(w, ", \"shared memory\": "); w.dec(r.p[3]);
@@ -1075,6 +1150,7 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
         KTJ_PUT(w, ", \"correlation\": "); w.dec((uint64_t)r.flow_id);
         KTJ_PUT(w, ", \"src\": \"0x"); put_hex(w, r.p[0]);
         KTJ_PUT(w, "\", \"dst\": \"0x"); put_hex(w, r.p[1]);
+        w.relief();
         KTJ_PUT(w, "\", \"bytes\": "); w.dec(r.p[2]);
         KTJ_PUT(w, ", \"kind\": \""); put_i64(w, (int64_t)(int32_t)(uint32_t)r.p[3]); w.ch('"');
         break;
@@ -1098,6 +1174,7 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
     KTJ_PUT(w, ", \"stream\": "); put_i64(w, r.res);
     KTJ_PUT(w, ", \"correlation\": "); w.dec((uint64_t)r.flow_id);
     KTJ_PUT(w, ", \"bytes\": "); w.dec(r.p[0]);
+    w.relief();
     if (r.dur != 0) {
       const double bw = (double)r.p[0] / (double)r.dur;
       uint64_t bits; __builtin_memcpy(&bits, &bw, 8);
@@ -1116,6 +1193,7 @@ template <class W> KTJ_HD KTJ_FI inline void put_fragment(W& w, const MatRow& r,
   KTJ_PUT(w, ", \"stream\": "); put_i64(w, r.res);
   KTJ_PUT(w, ", \"hsa_queue\": "); w.dec(r.p[3]);
   KTJ_PUT(w, ", \"correlation\": "); w.dec((uint64_t)r.flow_id);
+  w.relief();
   if (kind == KTJ_DOM_MEMORY_COPY) { KTJ_PUT(w, ", \"kind\": \""); put_copy_kind(w, r.aux); w.ch('"'); }
   else KTJ_PUT(w, ", \"kind\": \"Dispatch Kernel\"");
   if (r.meta & KTJ_M_HAS_SIZE) {
@@ -1298,6 +1376,7 @@ template <class W> KTJ_HD KTJ_FI inline void format_head(W& w, const MatRow& r, 
   put_category(w, type);
   KTJ_PUT(w, "\",\n    \"name\": \"");
   put_name(w, r, c);
+  w.relief();
   KTJ_PUT(w, "\",\n    \"pid\": "); if (st.pid_neg) w.ch('-'); w.num(st.pid);
   KTJ_PUT(w, ",\n    \"tid\": "); w.num(st.tidn);
   KTJ_PUT(w, ",\n    \"ts\": "); put_ts(w, rel);
@@ -1328,6 +1407,7 @@ template <class W> KTJ_HD KTJ_FI inline void format_flow(W& w, const MatRow& r, 
   put_i64(w, r.flow_id);
   KTJ_PUT(w, ",\n    \"pid\": "); if (st.pid_neg) w.ch('-'); w.num(st.pid);
   KTJ_PUT(w, ",\n    \"tid\": "); w.num(st.tidn);
+  w.relief();
   KTJ_PUT(w, ",\n    \"ts\": "); put_ts(w, frel);
   if (r.meta & KTJ_M_FLOW_FWDBWD) KTJ_PUT(w, ",\n    \"cat\": \"fwdbwd\",\n    \"name\": \"fwdbwd\"\n    ");
   else KTJ_PUT(w, ",\n    \"cat\": \"ac2g\",\n    \"name\": \"ac2g\"\n    ");

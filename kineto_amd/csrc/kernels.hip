@@ -2434,14 +2434,15 @@ k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n
 }
 
 /* Direct variant: one lane per activity; blocks of 16 bytes, aligned in the document (see
- * BlockWriter for who writes the blocks that two activities share).  Finished blocks wait in LDS
- * and leave at the three points where the whole wavefront meets: after the head of the event,
- * after its args and after the flow event; there four neighbouring lanes store four consecutive
- * blocks of one activity at a time, whole 128-byte lines only until the last of the three (a line
- * written in two pieces some microseconds apart leaves the L2 cache twice).  Lanes without an
- * activity stay until the end for that.  The
- * document's prefix and suffix are already in place when this kernel runs; the first and the last
- * activity merge with them. */
+ * BlockWriter for who writes the blocks that two activities share).  Finished blocks wait in the
+ * lane's stage in LDS, one 128-byte line of the document and the beginning of the next, and a line
+ * leaves when it is complete (a line written in pieces some microseconds apart leaves the L2 cache
+ * once per piece): at the three points where the whole wavefront meets — after the head of the
+ * event, after its args and after the flow event — the four lanes of a quad store each other's
+ * blocks, 64 contiguous bytes per quad and instruction, and in between a lane whose stage is nearly
+ * full stores its line itself (BlockWriter::relief).  Lanes without an activity stay until the end
+ * for the quads' sake.  The document's prefix and suffix are already in place when this kernel
+ * runs; the first and the last activity merge with them. */
 __global__ void __launch_bounds__(KTJ_BLOCK) __attribute__((amdgpu_waves_per_eu(3)))
 k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, const uint8_t* kind_sorted, uint64_t n_rows,
               EmitCtx ctx, char* out, uint64_t prefix_len) {
@@ -2457,6 +2458,7 @@ k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, con
   if (active) {
     m = mat[row];
     w.begin(out, prefix_len + o, i ? kind_sorted[i - 1] : 0u, i == 0);
+    w.stage_follow();
     format_head(w, m, ctx, parts);
   }
   w.flush(false);
