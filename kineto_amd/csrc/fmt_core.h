@@ -618,6 +618,13 @@ struct BlockWriter {
     stage_cap = KTJ_STAGE_BLOCKS;
 #endif
   }
+  /* the same, but only if some lane's stage is full or closed: where the part that follows is short
+   * enough for the stages of most wavefronts, the flush costs more than it saves */
+  __device__ KTJ_FI void flush_if_full() {
+#if defined(__HIP_DEVICE_COMPILE__)
+    if (__any(stage_cap == 0 || q_end >= KTJ_STAGE_BLOCKS)) flush(false);
+#endif
+  }
   /* Between flushes, wherever the formatter calls it: when a lane's stage is nearly full, every lane
    * that is here with a complete line writes it out (whole quads together, other lanes each on its
    * own).  Without this a full stage sends the blocks that follow straight to the document one at a

@@ -2437,10 +2437,10 @@ k_emit(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, uint64_t n
  * BlockWriter for who writes the blocks that two activities share).  Finished blocks wait in the
  * lane's stage in LDS, one 128-byte line of the document and the beginning of the next, and a line
  * leaves when it is complete (a line written in pieces some microseconds apart leaves the L2 cache
- * once per piece): at the three points where the whole wavefront meets — after the head of the
- * event, after its args and after the flow event — the four lanes of a quad store each other's
- * blocks, 64 contiguous bytes per quad and instruction, and in between a lane whose stage is nearly
- * full stores its line itself (BlockWriter::relief).  Lanes without an activity stay until the end
+ * once per piece): at the points where the whole wavefront meets — after the head of the event,
+ * after its args if some lane's stage is full by then, and after the flow event — the four lanes
+ * of a quad store each other's blocks, 64 contiguous bytes per quad and instruction, and in between
+ * a lane whose stage is nearly full stores its line itself (BlockWriter::relief).  Lanes without an activity stay until the end
  * for the quads' sake.  The document's prefix and suffix are already in place when this kernel
  * runs; the first and the last activity merge with them. */
 __global__ void __launch_bounds__(KTJ_BLOCK) __attribute__((amdgpu_waves_per_eu(3)))
@@ -2463,7 +2463,7 @@ k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, con
   }
   w.flush(false);
   if (active) format_args(w, m, ctx, parts);
-  w.flush(false);
+  w.flush_if_full();
   if (active) {
     format_flow(w, m, ctx, parts);
     w.end(i + 1 == n_rows);
