@@ -444,9 +444,9 @@ extern __shared__ __attribute__((aligned(16))) char ktj_stage_lds[];
 #endif
 
 /* Pass B: one lane formats one activity straight into the document in device memory.  Bytes are
- * gathered in a 128-bit accumulator and leave as aligned 16-byte stores; literal text is appended
- * sixteen bytes at a time, so that all lanes of a wavefront complete a block at the same append
- * and the wave issues one full store there, whatever the lanes' phases.  Dictionary strings are
+ * gathered in a 128-bit accumulator and leave as aligned 16-byte blocks (on the device through the
+ * lane's stage in LDS, see below); literal text is appended sixteen bytes at a time, so that all
+ * lanes of a wavefront complete a block at the same append, whatever their phases.  Dictionary strings are
  * appended inline through a funnel shift over aligned 8-byte loads (dictionary blobs are padded by
  * 16 bytes so that the last load stays inside the allocation).  Every block of the document has exactly one writer who knows all of
  * its bytes: a block that holds the end of activity A and the start of activity B is written
