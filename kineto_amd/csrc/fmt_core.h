@@ -425,7 +425,9 @@ static __device__ __attribute__((noinline)) void cooperative_word_copy(const cha
         v.x = (w0 >> sh) | (w1 << (64u - sh));
         v.y = (w1 >> sh) | (w2 << (64u - sh));
       }
-      d[k] = v;
+      /* whole lines that nobody reads again: stored past the L2's usual replacement, so that the
+       * dictionary the next strings come from stays in it (config 5: emit 3.64 -> 3.27 ms) */
+      __builtin_nontemporal_store(v, &d[k]);
     }
   }
 }
