@@ -1595,6 +1595,7 @@ k_radix_scatter(const uint64_t* keys_in, const uint32_t* vals_in, uint64_t* keys
 
 /* counts per (digit, tile) plus the digits' totals; below SORTP_SMALL_N keys the packed sort's tiles are 512 keys */
 #define SORTP_SMALL_N (1ull << 19)
+#define SORTP_STREAM_N (1ull << 24)
 uint64_t radix_tmp_elems(uint64_t n) {
   const uint64_t tiles = n < SORTP_SMALL_N ? (n + 511) / 512 : (n + RADIX_TILE - 1) / RADIX_TILE;
   return 256ull * tiles + 256;
@@ -1766,10 +1767,21 @@ k_sortp_scatter(const uint64_t* in, uint64_t* words_out, uint32_t* perm_out, uin
   uint64_t word[P::ITEMS];
   uint32_t rank[P::ITEMS];
   uint16_t dig[P::ITEMS];
+  /* this pass is the last to read the words: where they are more than the last-level cache keeps
+   * between the count and the scatter anyway, they are loaded past the L2's usual replacement
+   * (config 3, 22 M words: 1.20 -> 1.11 ms for the sort; at 11 M words the hint costs 2 %) */
+  if (n > SORTP_STREAM_N) {
 #pragma unroll
-  for (int r = 0; r < P::ITEMS; ++r) {
-    const uint64_t i = chunk + (uint64_t)r * 64u + lane;
-    word[r] = i < n ? in[i] : ~0ULL;
+    for (int r = 0; r < P::ITEMS; ++r) {
+      const uint64_t i = chunk + (uint64_t)r * 64u + lane;
+      word[r] = i < n ? load_once(&in[i]) : ~0ULL;
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < P::ITEMS; ++r) {
+      const uint64_t i = chunk + (uint64_t)r * 64u + lane;
+      word[r] = i < n ? in[i] : ~0ULL;
+    }
   }
 #pragma unroll
   for (int r = 0; r < P::ITEMS; ++r) {
