@@ -50,11 +50,11 @@ struct DevBuf {
     return *this;
   }
   ~DevBuf() { release(); }
-  hipError_t ensure(size_t bytes) {
+  hipError_t ensure(size_t bytes, bool with_slack = true) {
     if (p != own) { p = own; cap = own_cap; } /* back from a borrowed range */
     if (bytes <= cap) return hipSuccess;
     if (own) { hipError_t e = hipFree(own); p = own = nullptr; cap = own_cap = 0; if (e != hipSuccess) return e; }
-    size_t want = bytes + bytes / 8 + 256;
+    size_t want = bytes + (with_slack ? bytes / 8 : 0) + 256;
     hipError_t e = hipMalloc(&own, want);
     if (e != hipSuccess) { p = own = nullptr; return e; }
     p = own;
@@ -106,6 +106,7 @@ struct HostCtl {
   uint32_t n_out;
   uint32_t pad;
 };
+#define KTJ_GUESS_BYTES_PER_ROW 480u /* the fixed text of an event with its flow event */
 #define KTJ_PINNED_SMALL_BYTES (256u << 10) /* header/footer text and small tables of a pass that may not allocate */
 
 enum { EV_START = 0, EV_DICT, EV_DECODE, EV_CONVERT, EV_JOIN, EV_SORT_A, EV_SORT_B, EV_SORT, EV_SIZE, EV_SCAN,
@@ -970,6 +971,15 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   HIPCHK(rank_distinct(sets, sc, st));
   HIPCHK(hipEventRecord(e->ev[EV_SORT_A], st));
   HIPCHK(publish(sc, nullptr, nullptr, 0, &e->h_ctl_dev->scalars, nullptr, nullptr, st));
+  if (!out_device && !e->noalloc && e->out.cap == 0) {
+    /* An engine's first pass has no document buffer yet, and how long the document is comes out of
+     * the scan.  A first guess is allocated here, while the GPU is busy with the join: per row the
+     * fixed text of an event and one string of average length, at most 2 KB.  If that turns out too
+     * small (or cannot be had) the buffer is allocated where its size is known, as in later passes. */
+    const uint64_t avg_string = e->n_strings ? e->blob_bytes / e->n_strings : 0;
+    const uint64_t per_row = KTJ_GUESS_BYTES_PER_ROW + avg_string < 2048 ? KTJ_GUESS_BYTES_PER_ROW + avg_string : 2048;
+    if (e->out.ensure(N * per_row + (1u << 20), false) != hipSuccess) (void)hipGetLastError();
+  }
   HIPCHK(hipStreamSynchronize(st));
   e->scalars = e->h_ctl->scalars;
   const unsigned distinct_overflow = e->scalars.error & (KTJ_DEVERR_DISTINCT_DEVICES | KTJ_DEVERR_DISTINCT_RESOURCES);
