@@ -243,6 +243,7 @@ struct CountWriter {
   KTJ_HD KTJ_FI void dec(uint64_t v) { n += (uint32_t)ndigits_u64(v); }
   KTJ_HD KTJ_FI void dec3(uint32_t) { n += 3; }
   KTJ_HD KTJ_FI void str(const char*, uint64_t len) { n += len; }
+  KTJ_HD KTJ_FI void name(const char*, uint64_t len) { n += len; }
   /* a number that is printed more than once is prepared once */
   typedef uint32_t Prepared;
   KTJ_HD KTJ_FI static Prepared prepare(uint64_t v) { return (uint32_t)ndigits_u64(v); }
@@ -362,6 +363,7 @@ struct TileWriter {
   KTJ_HD KTJ_FI void dec3(uint32_t x) { /* {:03} of 0..999 */
     append((uint64_t)(ascii4(x) >> 8), 3);
   }
+  KTJ_HD KTJ_FI void name(const char* src, uint64_t len) { str(src, len); }
   KTJ_HD KTJ_FI void str(const char* src, uint64_t len) {
     if (len == 0) return;
     end(); /* bytes gathered so far */
@@ -709,7 +711,10 @@ struct BlockWriter {
   KTJ_HD KTJ_FI void dec3(uint32_t x) { append((uint64_t)(ascii4(x) >> 8), 3); }
   /* a dictionary string copied by this lane: aligned 8-byte loads, funnel-shifted, sixteen bytes
    * per append while they last */
-  KTJ_HD KTJ_FI void str_own(const char* src, uint64_t len) {
+  KTJ_HD KTJ_FI void str_own(const char* src, uint64_t len) { str_own_t<false>(src, len); }
+  /* RELIEF: with a relief() every 32 bytes, for the one string of an activity that is often longer
+   * than the stage has room for (a kernel's name; everywhere else the call would only be code in the way) */
+  template <bool RELIEF> KTJ_HD KTJ_FI void str_own_t(const char* src, uint64_t len) {
     if (len == 0) return;
     const uintptr_t sa = (uintptr_t)src;
     const uint32_t sh = (uint32_t)(sa & 7u) * 8u;
@@ -725,6 +730,7 @@ struct BlockWriter {
     uint64_t k = 0;
     KTJ_NOUNROLL
     for (; k + 2 <= full; k += 2) {
+      if (RELIEF && (k & 2u) != 0) relief();
       const uint64_t n1 = sp[k + 1], n2 = sp[k + 2];
       append16(sh ? (cur >> sh) | (n1 << (64u - sh)) : cur, sh ? (n1 >> sh) | (n2 << (64u - sh)) : n1);
       cur = n2;
@@ -741,7 +747,10 @@ struct BlockWriter {
       append(v & ((1ULL << (8 * rem)) - 1ULL), rem);
     }
   }
-  KTJ_HD KTJ_FI void str(const char* src, uint64_t len) {
+  KTJ_HD KTJ_FI void str(const char* src, uint64_t len) { str_t<false>(src, len); }
+  /* an activity's name */
+  KTJ_HD KTJ_FI void name(const char* src, uint64_t len) { str_t<true>(src, len); }
+  template <bool RELIEF> KTJ_HD KTJ_FI void str_t(const char* src, uint64_t len) {
 #if defined(__HIP_DEVICE_COMPILE__)
     const bool big = len >= KTJ_COOP_MIN_BYTES;
     if (__any(big)) { /* see cooperative_word_copy */
@@ -758,13 +767,13 @@ struct BlockWriter {
         dst = wptr;
         stage_close();
         wptr += n_words;
-      } else str_own(src, len);
+      } else str_own_t<RELIEF>(src, len);
       cooperative_word_copy(body, dst, n_words);
       if (big) str_own(body + (uint64_t)n_words * 8u, tail);
       return;
     }
 #endif
-    str_own(src, len);
+    str_own_t<RELIEF>(src, len);
   }
 };
 
@@ -1241,7 +1250,7 @@ template <class W> KTJ_HD KTJ_FI inline void put_name(W& w, const MatRow& r, con
     return;
   }
   if (r.name_id < c.dict.n)
-    w.str(c.dict.name_blob + c.dict.name_off[r.name_id], c.dict.name_off[r.name_id + 1] - c.dict.name_off[r.name_id]);
+    w.name(c.dict.name_blob + c.dict.name_off[r.name_id], c.dict.name_off[r.name_id + 1] - c.dict.name_off[r.name_id]);
 }
 
 /* Generic rows only: marks a CUDA_SYNC activity named "Stream Sync" (output_json.cpp:915) and
