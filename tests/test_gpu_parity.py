@@ -239,6 +239,41 @@ def test_header_text_beyond_the_pinned_staging_buffer():
         _engine_vs_oracle(b.build())
 
 
+def test_document_longer_than_the_first_guess_of_its_buffer():
+    """An engine's first pass allocates the document's buffer from a guess (rows times the fixed text
+    of an event plus one string of average length) before the lengths are known.  Here every device
+    row carries the one long name of a dictionary of short strings, so the document is several times
+    the guess and the buffer has to be allocated again; a second pass on the same engine then finds
+    the buffer large enough.  Both documents must be the oracle's."""
+    import oracle_glue as og
+    from kineto_amd.engine import TraceEngine
+    from stream_builder import StreamBuilder, B
+    b = StreamBuilder(host_name="guess")
+    ids, plain_s = {}, b.s
+    b.s = lambda text: ids[text] if text in ids else ids.setdefault(text, plain_s(text))  # one dictionary entry per text
+    b.api(["hipLaunchKernel"], flow_start=[0])
+    long_name = "void long_kernel<" + ", ".join("T%d" % k for k in range(400)) + ">(int)"
+    assert len(long_name) > 2000
+    for k in range(3000):  # many short strings: the average stays small
+        b.add_generic("op%d" % k, 0, B + 1000 + 10 * k, B + 1005 + 10 * k, 7, 100 + (k % 4), id=k + 1)
+    for k in range(6000):
+        b.add_runtime(10 + k, B + 2000 + 20 * k, B + 2010 + 20 * k, 0, 7, 100 + (k % 4), kind=1, stream=1 + k % 3)
+        b.add_device(10 + k, B + 2020 + 20 * k, B + 2030 + 20 * k, domain=0, device=0, name=long_name, queue=1 + k % 3, stream=0)
+    b.add_span(B, B + 10**6, 50, 0, "PyTorch Profiler")
+    sp = b.build()
+    ora = og.OracleRun(sp)
+    want = ora.output()
+    ora.close()
+    assert len(want) > 6000 * 2000
+    with TraceEngine(sp.contents.trace_name.decode(), device=0) as eng:
+        eng.submit_stream(sp)
+        for attempt in range(2):
+            print(f"document of {len(want)} bytes, pass {attempt}", flush=True)
+            eng.process()
+            got = eng.output()
+            assert got == want, f"pass {attempt}: bytes differ at {_first_diff(got, want)}"
+
+
 def test_golden_digests_on_gpu():
     """The engine's document against the committed digests (tests/golden/digests.json, written where
     the checker's output had just been compared byte for byte with the reference logger's): no
