@@ -468,6 +468,14 @@ typedef struct ktj_engine ktj_engine;
  * KTJ_CREATE_CUDA12_ARGS prints the "graph id", "graph node id", "channel" and "channel_type" keys
  * of memset rows (ktj_memset_rec), which the reference compiles in for CUDA >= 12 only
  * (CuptiActivity.h:424-458).
+ *
+ * ktj_destroy leaves what every engine needs before its first record (its stream and events, the
+ * small page-locked buffers, 1 MiB of device memory for the inputs of small traces) and, while they
+ * are small (64 MiB together), the working memory and the document buffer of its last pass behind
+ * for the next ktj_create on the same device, which starts from them instead of allocating: one
+ * such set per device, held until the process ends.  A trace of a few records otherwise spends
+ * more time creating and destroying these than on the GPU.  Nothing is kept of an engine that saw
+ * a HIP error.
  * ---------------------------------------------------------------------------------------- */
 #define KTJ_CREATE_NO_FILE 0x1u
 #define KTJ_CREATE_TILE_EMIT 0x2u
@@ -519,7 +527,11 @@ int ktj_set_window(ktj_engine* e, int64_t start_ns, int64_t end_ns);
 /* Raw record submission: the bulk equivalent of the per-record handleActivity /
  * handleGenericActivity calls (output_json.cpp:837-971) and of the profiler's per-row handlers
  * (RocmActivityProfiler.cpp:150-213).  `packed` is host memory; the caller may free it when the
- * call returns.  Arrival order is: all generic records, then all runtime rows, then all device
+ * call returns (the copy to the device is ordered in front of the next pass, not necessarily
+ * finished: submissions of up to 64 KiB wait in a page-locked ring and are moved by one kernel
+ * launch for many of them; ordinary memory of 16 MiB and more is copied into page-locked chunks by
+ * several threads while the copy engine empties others; memory from ktj_host_alloc is copied from
+ * directly).  Arrival order is: all generic records, then all runtime rows, then all device
  * rows, each in submission order. */
 int ktj_submit_records(ktj_engine* e, int rec_class, const void* packed, size_t n_records);
 

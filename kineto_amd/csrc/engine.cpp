@@ -14,6 +14,8 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <mutex>
+#include <thread>
 #include <string>
 #include <unistd.h>
 #include <unordered_map>
@@ -32,6 +34,16 @@ using namespace ktj;
 using namespace ktj::gpu;
 
 namespace {
+
+#define KTJ_INPUT_ARENA_BYTES (1u << 20)   /* device memory for the inputs of small traces */
+#define KTJ_INPUT_PIECE_MAX (128u << 10)   /* largest array that takes a piece of it */
+#define KTJ_STAGE_SMALL_BYTES (256u << 10) /* pinned ring that small submissions pass through */
+#define KTJ_STAGE_SMALL_MAX (64u << 10)    /* largest submission that does */
+#define KTJ_STAGE_CHUNK (2ull << 20)       /* large submissions: pinned chunks, two per copying thread */
+#define KTJ_STAGE_BIG_MIN (16ull << 20)    /* smallest submission that is spread over threads */
+#define KTJ_STAGE_THREADS_MAX 8
+#define KTJ_KIT_DEVICE_BYTES_MAX (64ull << 20) /* working and document memory that waits for the next engine */
+#define KTJ_KIT_PINNED_BYTES_MAX (1ull << 20)  /* same, per pinned buffer sized by a document */
 
 /* One working buffer in device memory.  `p` is what the kernels use: either the buffer's own
  * allocation (freed with the engine; the engine's device is current then) or, for the entry point
@@ -66,29 +78,43 @@ struct DevBuf {
   template <typename T> T* as() const { return reinterpret_cast<T*>(p); }
 };
 
+/* Device memory for the inputs of a small trace: one allocation that the engine's small arrays are
+ * carved out of (a trace of a few records otherwise spends more time in hipMalloc than on the GPU).
+ * Pieces are never given back; a new engine that inherits the arena starts at its beginning. */
+struct InputArena {
+  DevBuf mem;
+  size_t used = 0;
+  void* take(size_t bytes) {
+    const size_t off = (used + 255) & ~(size_t)255;
+    if (bytes > KTJ_INPUT_PIECE_MAX || !mem.p || off > mem.cap || bytes > mem.cap - off) return nullptr;
+    used = off + bytes;
+    return static_cast<char*>(mem.p) + off;
+  }
+};
+
 /* append-only device array fed from host memory */
 struct DevVec {
   DevBuf buf;
   size_t bytes = 0;
-  hipError_t append(const void* src, size_t n, hipStream_t st) {
-    if (n == 0) return hipSuccess;
+  /* room for n more bytes behind what is there; what is there moves along.  A small array takes a
+   * piece of the engine's input arena instead of an allocation of its own. */
+  hipError_t reserve(size_t n, hipStream_t st, InputArena* arena) {
     if (bytes + n + 16 > buf.cap) { /* 16 spare bytes: string copies load whole aligned words */
       DevBuf nb;
       size_t want = (bytes + n) * 2 + 16;
-      hipError_t e = nb.ensure(want);
+      void* piece = arena ? arena->take(want) : nullptr;
+      hipError_t e = hipSuccess;
+      if (piece) nb.borrow(piece, want);
+      else e = nb.ensure(want);
       if (e != hipSuccess) return e;
       if (bytes) { e = hipMemcpyAsync(nb.p, buf.p, bytes, hipMemcpyDeviceToDevice, st); if (e != hipSuccess) return e; }
       e = hipStreamSynchronize(st);
       if (e != hipSuccess) return e;
       buf = std::move(nb);
     }
-    hipError_t e = hipMemcpyAsync(static_cast<char*>(buf.p) + bytes, src, n, hipMemcpyHostToDevice, st);
-    if (e != hipSuccess) return e;
-    e = hipStreamSynchronize(st); /* caller may free src when we return */
-    if (e != hipSuccess) return e;
-    bytes += n;
     return hipSuccess;
   }
+  char* end() const { return static_cast<char*>(buf.p) + bytes; }
   void release() { buf.release(); bytes = 0; }
 };
 
@@ -185,6 +211,15 @@ struct ktj_engine {
   size_t file_stage_cap[2] = {0, 0};
   hipEvent_t ev_file_stage[2] = {};
   bool host_copy_valid = false;
+  /* submissions from ordinary host memory: small ones pass through a pinned ring and are not waited
+   * for (the stream orders them before the pass), large ones through pinned chunks that several
+   * threads fill while the copy engine empties others */
+  InputArena input_arena;
+  char* stage_small = nullptr; char* stage_small_dev = nullptr; size_t stage_small_used = 0;
+  PieceJobs pieces{}; /* small submissions in the ring that no kernel has moved yet */
+  char* stage_big = nullptr; size_t stage_big_chunks = 0;
+  hipEvent_t ev_stage_big[2 * KTJ_STAGE_THREADS_MAX] = {};
+  bool hip_failed = false; /* a HIP call failed at some point: nothing of this engine is handed on */
 
   /* results */
   uint64_t N = 0, prefix_len = 0, act_bytes = 0, total_bytes = 0;
@@ -197,6 +232,7 @@ struct ktj_engine {
 namespace {
 
 int fail_hip(ktj_engine* e, hipError_t err, const char* what) {
+  e->hip_failed = true;
   e->last_error = std::string(what) + ": " + hipGetErrorString(err);
   return KTJ_ERR_HIP;
 }
@@ -285,6 +321,109 @@ int upload_small(ktj_engine* e, DevBuf& dst, const void* src, size_t bytes) {
   }
   if (bytes) HIPCHK(hipMemcpyAsync(dst.p, src, bytes, hipMemcpyHostToDevice, e->stream));
   HIPCHK(hipStreamSynchronize(e->stream));
+  return KTJ_OK;
+}
+
+/* The small submissions gathered in the pinned ring go to their places on the device: one launch for
+ * all of them, ordered on the engine's stream like everything else.  Before a pass, before an array
+ * they belong to moves, and when the ring or the list is full. */
+int put_pending_pieces(ktj_engine* e) {
+  if (e->pieces.count == 0) return KTJ_OK;
+  HIPCHK(put_pieces(e->pieces, e->stream));
+  e->pieces.count = 0;
+  return KTJ_OK;
+}
+
+/* Is this host memory page-locked for the GPU (ktj_host_alloc, or the caller's own hipHostMalloc)?
+ * Such memory is copied from directly. */
+bool is_pinned_host(const void* p) {
+  hipPointerAttribute_t a;
+  memset(&a, 0, sizeof a);
+  if (hipPointerGetAttributes(&a, p) != hipSuccess) { (void)hipGetLastError(); return false; }
+  return a.type == hipMemoryTypeHost;
+}
+
+/* n bytes of host memory behind a device array.  The caller may free or reuse src when this
+ * returns; the copy itself is only ordered on the engine's stream, in front of the next pass.
+ *   - up to KTJ_STAGE_SMALL_MAX bytes: into the pinned ring, from where one kernel launch takes all
+ *     such pieces to their places (put_pending_pieces; a trace of a few records pays a dozen copies
+ *     and stream synchronisations otherwise);
+ *   - from KTJ_STAGE_BIG_MIN bytes of ordinary memory: threads copy chunks into pinned buffers, two
+ *     per thread, and hand each to the copy engine as soon as it is full (one thread's copy through
+ *     the runtime's own staging reaches about half of what the link carries);
+ *   - everything else, and page-locked sources: one copy, waited for. */
+int append_from_host(ktj_engine* e, DevVec& v, const void* src, size_t n) {
+  if (n == 0) return KTJ_OK;
+  hipStream_t st = e->stream;
+  if (v.bytes + n + 16 > v.buf.cap) { /* the array is about to move: the pieces on their way to it go first */
+    const int rc = put_pending_pieces(e);
+    if (rc != KTJ_OK) return rc;
+  }
+  HIPCHK(v.reserve(n, st, &e->input_arena));
+  char* dst = v.end();
+  if (n <= KTJ_STAGE_SMALL_MAX && e->stage_small) {
+    /* the piece sits in the ring where its place on the device does, modulo 16 */
+    size_t off = ((e->stage_small_used + 63) & ~(size_t)63) + ((uintptr_t)dst & 15u);
+    if (off + n > KTJ_STAGE_SMALL_BYTES || e->pieces.count == KTJ_MAX_PIECES) {
+      const int rc = put_pending_pieces(e);
+      if (rc != KTJ_OK) return rc;
+    }
+    if (off + n > KTJ_STAGE_SMALL_BYTES) { /* the ring is full: what is in it has to be on the device first */
+      HIPCHK(hipStreamSynchronize(st));
+      off = (uintptr_t)dst & 15u;
+    }
+    memcpy(e->stage_small + off, src, n);
+    const uint32_t k = e->pieces.count++;
+    e->pieces.src[k] = e->stage_small_dev + off;
+    e->pieces.dst[k] = dst;
+    e->pieces.n[k] = n;
+    e->stage_small_used = off + n;
+    v.bytes += n;
+    return KTJ_OK;
+  }
+  unsigned n_threads = std::thread::hardware_concurrency() / 2;
+  if (n_threads > KTJ_STAGE_THREADS_MAX) n_threads = KTJ_STAGE_THREADS_MAX;
+  if (n >= KTJ_STAGE_BIG_MIN && n_threads >= 2 && !is_pinned_host(src)) {
+    const size_t slots = 2 * (size_t)n_threads;
+    if (e->stage_big_chunks < slots) {
+      if (e->stage_big) HIPCHK(hipHostFree(e->stage_big));
+      e->stage_big = nullptr; e->stage_big_chunks = 0;
+      void* p = nullptr;
+      HIPCHK(hipHostMalloc(&p, slots * KTJ_STAGE_CHUNK, hipHostMallocDefault));
+      e->stage_big = static_cast<char*>(p);
+      e->stage_big_chunks = slots;
+    }
+    for (size_t k = 0; k < slots; ++k)
+      if (!e->ev_stage_big[k]) HIPCHK(hipEventCreateWithFlags(&e->ev_stage_big[k], hipEventDisableTiming));
+    const size_t n_chunks = (n + KTJ_STAGE_CHUNK - 1) / KTJ_STAGE_CHUNK;
+    hipError_t err[KTJ_STAGE_THREADS_MAX];
+    auto worker = [&](unsigned t) {
+      err[t] = hipSetDevice(e->device);
+      /* thread t takes chunks t, t + T, ...; its two pinned slots alternate */
+      for (size_t c = t, turn = 0; c < n_chunks && err[t] == hipSuccess; c += n_threads, ++turn) {
+        const size_t slot = 2 * (size_t)t + (turn & 1);
+        char* stage = e->stage_big + slot * KTJ_STAGE_CHUNK;
+        const size_t off = c * KTJ_STAGE_CHUNK, len = n - off < KTJ_STAGE_CHUNK ? n - off : KTJ_STAGE_CHUNK;
+        if (turn >= 2) { err[t] = hipEventSynchronize(e->ev_stage_big[slot]); if (err[t] != hipSuccess) break; }
+        memcpy(stage, static_cast<const char*>(src) + off, len);
+        err[t] = hipMemcpyAsync(dst + off, stage, len, hipMemcpyHostToDevice, st);
+        if (err[t] == hipSuccess) err[t] = hipEventRecord(e->ev_stage_big[slot], st);
+      }
+    };
+    std::vector<std::thread> pool;
+    for (unsigned t = 1; t < n_threads; ++t) pool.emplace_back(worker, t);
+    worker(0);
+    for (auto& th : pool) th.join();
+    /* the slots are free for the next call once the stream has passed them */
+    const hipError_t done = hipStreamSynchronize(st);
+    for (unsigned t = 0; t < n_threads; ++t) HIPCHK(err[t]);
+    HIPCHK(done);
+    v.bytes += n;
+    return KTJ_OK;
+  }
+  HIPCHK(hipMemcpyAsync(dst, src, n, hipMemcpyHostToDevice, st));
+  HIPCHK(hipStreamSynchronize(st)); /* the caller may free src when we return */
+  v.bytes += n;
   return KTJ_OK;
 }
 
@@ -390,6 +529,90 @@ int synthesise_user_spans(ktj_engine* e, Columns c, const EmitCtx& ctx, Table t_
   return KTJ_OK;
 }
 
+
+/* What every engine needs before its first record — a stream, its events, the pinned buffers of the
+ * hand-over, the input arena — and what its first pass allocates (the pool of working buffers and
+ * the document, while they are small) costs several times what a trace of a few records takes on
+ * the GPU.  ktj_destroy leaves one such set per device behind for the next ktj_create, which takes
+ * it whole; a second engine alive at the same time makes its own.  Nothing of an engine that saw a
+ * HIP error is kept.  Device and pinned memory that is kept: at most KTJ_KIT_DEVICE_BYTES_MAX of
+ * working and document memory, the input arena, the small pinned buffers; it is held until the
+ * process ends. */
+struct Kit {
+  bool full = false;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev[EV_COUNT] = {};
+  hipEvent_t ev_d2h[2] = {};
+  hipEvent_t ev_file_stage[2] = {};
+  hipEvent_t ev_stage_big[2 * KTJ_STAGE_THREADS_MAX] = {};
+  void* pinned_small = nullptr; size_t pinned_small_cap = 0; char* pinned_small_dev = nullptr;
+  HostCtl* h_ctl = nullptr; HostCtl* h_ctl_dev = nullptr;
+  char* pinned_out = nullptr; size_t pinned_out_cap = 0;
+  char* file_stage[2] = {nullptr, nullptr}; size_t file_stage_cap[2] = {0, 0};
+  char* stage_small = nullptr; char* stage_small_dev = nullptr;
+  char* stage_big = nullptr; size_t stage_big_chunks = 0;
+  DevBuf d_scalars, pool, out, arena_mem;
+};
+std::mutex g_kit_mutex;
+std::map<int, Kit*>& kits() { static auto* m = new std::map<int, Kit*>(); return *m; } /* never destroyed: the runtime may be gone by then */
+
+/* the engine's device is current */
+bool take_kit(ktj_engine* e) {
+  std::lock_guard<std::mutex> lock(g_kit_mutex);
+  auto it = kits().find(e->device);
+  if (it == kits().end() || !it->second->full) return false;
+  Kit& k = *it->second;
+  e->stream = k.stream;
+  memcpy(e->ev, k.ev, sizeof k.ev); memcpy(e->ev_d2h, k.ev_d2h, sizeof k.ev_d2h);
+  memcpy(e->ev_file_stage, k.ev_file_stage, sizeof k.ev_file_stage);
+  memcpy(e->ev_stage_big, k.ev_stage_big, sizeof k.ev_stage_big);
+  e->pinned_small = k.pinned_small; e->pinned_small_cap = k.pinned_small_cap; e->pinned_small_dev = k.pinned_small_dev;
+  e->h_ctl = k.h_ctl; e->h_ctl_dev = k.h_ctl_dev;
+  e->pinned_out = k.pinned_out; e->pinned_out_cap = k.pinned_out_cap;
+  for (int i = 0; i < 2; ++i) { e->file_stage[i] = k.file_stage[i]; e->file_stage_cap[i] = k.file_stage_cap[i]; }
+  e->stage_small = k.stage_small; e->stage_small_dev = k.stage_small_dev;
+  e->stage_big = k.stage_big; e->stage_big_chunks = k.stage_big_chunks;
+  e->d_scalars = std::move(k.d_scalars); e->pool = std::move(k.pool); e->out = std::move(k.out);
+  e->input_arena.mem = std::move(k.arena_mem);
+  k = Kit();
+  return true;
+}
+
+/* the engine's device is current and its stream is idle; whatever is not taken stays with the engine */
+void give_kit(ktj_engine* e) {
+  if (e->hip_failed || !e->stream || !e->h_ctl || !e->pinned_small || !e->stage_small || !e->d_scalars.own) return;
+  for (auto& ev : e->ev) if (!ev) return;
+  for (auto& ev : e->ev_d2h) if (!ev) return;
+  std::lock_guard<std::mutex> lock(g_kit_mutex);
+  Kit*& slot = kits()[e->device];
+  if (!slot) slot = new (std::nothrow) Kit();
+  if (!slot || slot->full) return;
+  Kit& k = *slot;
+  k.stream = e->stream; e->stream = nullptr;
+  memcpy(k.ev, e->ev, sizeof k.ev); memset(e->ev, 0, sizeof e->ev);
+  memcpy(k.ev_d2h, e->ev_d2h, sizeof k.ev_d2h); memset(e->ev_d2h, 0, sizeof e->ev_d2h);
+  memcpy(k.ev_file_stage, e->ev_file_stage, sizeof k.ev_file_stage); memset(e->ev_file_stage, 0, sizeof e->ev_file_stage);
+  memcpy(k.ev_stage_big, e->ev_stage_big, sizeof k.ev_stage_big); memset(e->ev_stage_big, 0, sizeof e->ev_stage_big);
+  k.pinned_small = e->pinned_small; k.pinned_small_cap = e->pinned_small_cap; k.pinned_small_dev = e->pinned_small_dev;
+  e->pinned_small = nullptr;
+  k.h_ctl = e->h_ctl; k.h_ctl_dev = e->h_ctl_dev; e->h_ctl = nullptr;
+  if (e->pinned_out_cap <= KTJ_KIT_PINNED_BYTES_MAX) { k.pinned_out = e->pinned_out; k.pinned_out_cap = e->pinned_out_cap; e->pinned_out = nullptr; }
+  for (int i = 0; i < 2; ++i)
+    if (e->file_stage_cap[i] <= KTJ_KIT_PINNED_BYTES_MAX) { k.file_stage[i] = e->file_stage[i]; k.file_stage_cap[i] = e->file_stage_cap[i]; e->file_stage[i] = nullptr; }
+  k.stage_small = e->stage_small; k.stage_small_dev = e->stage_small_dev; e->stage_small = nullptr;
+  k.stage_big = e->stage_big; k.stage_big_chunks = e->stage_big_chunks; e->stage_big = nullptr;
+  k.d_scalars = std::move(e->d_scalars);
+  if (e->pool.own_cap + e->out.own_cap <= KTJ_KIT_DEVICE_BYTES_MAX) {
+    /* back from whatever they were lent (the pool never is; the document may sit in a caller's buffer) */
+    e->pool.p = e->pool.own; e->pool.cap = e->pool.own_cap;
+    e->out.p = e->out.own; e->out.cap = e->out.own_cap;
+    k.pool = std::move(e->pool);
+    k.out = std::move(e->out);
+  }
+  k.arena_mem = std::move(e->input_arena.mem);
+  k.full = true;
+}
+
 }  // namespace
 
 extern "C" {
@@ -414,23 +637,29 @@ int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int
     if (!e->sink) { e->bad_sink = true; e->last_error = "Failed to open '" + e->out_path + "': " + strerror(errno); }
   }
   HIPCHK(hipSetDevice(hip_device));
-  HIPCHK(hipStreamCreate(&e->stream));
-  for (auto& ev : e->ev) HIPCHK(hipEventCreate(&ev));
-  for (auto& ev : e->ev_d2h) HIPCHK(hipEventCreate(&ev));
-  HIPCHK(e->d_scalars.ensure(sizeof(Scalars)));
-  HIPCHK(hipHostMalloc(&e->pinned_small, KTJ_PINNED_SMALL_BYTES, hipHostMallocDefault));
-  e->pinned_small_cap = KTJ_PINNED_SMALL_BYTES;
-  {
+  if (!take_kit(e)) {
+    HIPCHK(hipStreamCreate(&e->stream));
+    for (auto& ev : e->ev) HIPCHK(hipEventCreate(&ev));
+    for (auto& ev : e->ev_d2h) HIPCHK(hipEventCreate(&ev));
+    HIPCHK(e->d_scalars.ensure(sizeof(Scalars)));
+    HIPCHK(hipHostMalloc(&e->pinned_small, KTJ_PINNED_SMALL_BYTES, hipHostMallocDefault));
+    e->pinned_small_cap = KTJ_PINNED_SMALL_BYTES;
     void* p = nullptr;
     HIPCHK(hipHostMalloc(&p, sizeof(HostCtl), hipHostMallocDefault));
     e->h_ctl = static_cast<HostCtl*>(p);
-    memset(e->h_ctl, 0, sizeof(HostCtl));
     void* d = nullptr;
     HIPCHK(hipHostGetDevicePointer(&d, e->h_ctl, 0));
     e->h_ctl_dev = static_cast<HostCtl*>(d);
     HIPCHK(hipHostGetDevicePointer(&d, e->pinned_small, 0));
     e->pinned_small_dev = static_cast<char*>(d);
+    p = nullptr;
+    HIPCHK(hipHostMalloc(&p, KTJ_STAGE_SMALL_BYTES, hipHostMallocDefault));
+    e->stage_small = static_cast<char*>(p);
+    HIPCHK(hipHostGetDevicePointer(&d, e->stage_small, 0));
+    e->stage_small_dev = static_cast<char*>(d);
+    HIPCHK(e->input_arena.mem.ensure(KTJ_INPUT_ARENA_BYTES, false));
   }
+  memset(e->h_ctl, 0, sizeof(HostCtl));
   { /* this device's copy of the static scratch array (ktj_process_noalloc) */
     void* p = nullptr;
     size_t bytes = 0;
@@ -445,12 +674,16 @@ void ktj_destroy(ktj_engine* e) {
   if (!e) return;
   (void)hipSetDevice(e->device);
   if (e->stream) (void)hipStreamSynchronize(e->stream);
+  give_kit(e); /* what the next engine on this device can start from; the rest is freed here */
   /* device buffers free themselves when the engine is deleted below */
   if (e->pinned_small) (void)hipHostFree(e->pinned_small);
   if (e->h_ctl) (void)hipHostFree(e->h_ctl);
   if (e->pinned_out) (void)hipHostFree(e->pinned_out);
+  if (e->stage_small) (void)hipHostFree(e->stage_small);
+  if (e->stage_big) (void)hipHostFree(e->stage_big);
   for (auto& p : e->file_stage) if (p) (void)hipHostFree(p);
   for (auto& ev : e->ev_file_stage) if (ev) (void)hipEventDestroy(ev);
+  for (auto& ev : e->ev_stage_big) if (ev) (void)hipEventDestroy(ev);
   for (auto& ev : e->ev) if (ev) (void)hipEventDestroy(ev);
   for (auto& ev : e->ev_d2h) if (ev) (void)hipEventDestroy(ev);
   if (e->stream) (void)hipStreamDestroy(e->stream);
@@ -482,9 +715,13 @@ int ktj_intern_strings(ktj_engine* e, const char* blob, const uint64_t* offsets,
     if (offsets[i] < src0 || (i && offsets[i] < offsets[i - 1])) return KTJ_ERR_ARG;
     abs_off[i] = e->blob_bytes + (offsets[i] - src0);
   }
-  HIPCHK(e->str_blob.append(blob + src0, nbytes, e->stream));
-  if (e->n_strings == 0) HIPCHK(e->str_off.append(abs_off.data(), (n + 1) * 8, e->stream));
-  else HIPCHK(e->str_off.append(abs_off.data() + 1, n * 8, e->stream)); /* entry n_strings already equals blob_bytes */
+  { const int rc = append_from_host(e, e->str_blob, blob + src0, nbytes); if (rc != KTJ_OK) return rc; }
+  {
+    /* entry n_strings already equals blob_bytes */
+    const int rc = e->n_strings == 0 ? append_from_host(e, e->str_off, abs_off.data(), (n + 1) * 8)
+                                     : append_from_host(e, e->str_off, abs_off.data() + 1, n * 8);
+    if (rc != KTJ_OK) return rc;
+  }
   e->n_strings += n;
   e->blob_bytes += nbytes;
   e->processed = false;
@@ -533,7 +770,7 @@ int ktj_submit_args(ktj_engine* e, const uint64_t* slots, size_t n_slots, uint64
   if (first_slot) *first_slot = e->n_args;
   if (e->bad_sink || n_slots == 0) return KTJ_OK;
   HIPCHK(hipSetDevice(e->device));
-  HIPCHK(e->args.append(slots, n_slots * 8, e->stream));
+  { const int rc = append_from_host(e, e->args, slots, n_slots * 8); if (rc != KTJ_OK) return rc; }
   e->n_args += n_slots;
   e->processed = false;
   return KTJ_OK;
@@ -597,7 +834,7 @@ int ktj_submit_records(ktj_engine* e, int rec_class, const void* packed, size_t 
   }
   if (set->external) return KTJ_ERR_STATE;
   HIPCHK(hipSetDevice(e->device));
-  HIPCHK(set->owned.append(packed, n_records * rs, e->stream));
+  { const int rc = append_from_host(e, set->owned, packed, n_records * rs); if (rc != KTJ_OK) return rc; }
   set->n += n_records;
   if (rec_class == KTJ_REC_GENERIC || rec_class == KTJ_REC_RUNTIME || rec_class == KTJ_REC_DEVICE) e->activities_begun = true;
   e->processed = false;
@@ -775,6 +1012,7 @@ int ktj_submit_info(ktj_engine* e, int info_kind, const void* info) {
 static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, uint64_t out_cap) {
   HIPCHK(hipSetDevice(e->device));
   hipStream_t st = e->stream;
+  { const int rc = put_pending_pieces(e); if (rc != KTJ_OK) return rc; }
   e->arena_used = 0;
   e->processed = false;
   e->total_bytes = 0;

@@ -168,6 +168,15 @@ struct ApiTable {
 hipError_t publish(const Scalars* sc, const uint64_t* total, const uint32_t* list, uint32_t n_list, Scalars* h_sc,
                    uint64_t* h_total, uint32_t* h_list, hipStream_t st);
 hipError_t put_text(const char* src_a, char* dst_a, uint64_t n_a, const char* src_b, char* dst_b, uint64_t n_b, hipStream_t st);
+/* pieces of page-locked host memory to their places in device memory, in one launch */
+#define KTJ_MAX_PIECES 16u
+struct PieceJobs {
+  const char* src[KTJ_MAX_PIECES];
+  char* dst[KTJ_MAX_PIECES];
+  uint64_t n[KTJ_MAX_PIECES];
+  uint32_t count;
+};
+hipError_t put_pieces(const PieceJobs& jobs, hipStream_t st);
 /* ---- utilities ---- */
 hipError_t fill_u64(uint64_t* p, uint64_t v, uint64_t n, hipStream_t st);
 hipError_t fill_u32(uint32_t* p, uint32_t v, uint64_t n, hipStream_t st);

@@ -2577,6 +2577,34 @@ hipError_t put_text(const char* src_a, char* dst_a, uint64_t n_a, const char* sr
   return KTJ_LAUNCH_CHECK();
 }
 
+/* up to KTJ_MAX_PIECES pieces of page-locked host memory, each to its place in device memory (the
+ * small submissions an engine has gathered); source and destination of a piece agree modulo 16 */
+__global__ void k_put_pieces(PieceJobs jobs) {
+  const char* src = jobs.src[blockIdx.y];
+  char* dst = jobs.dst[blockIdx.y];
+  const uint64_t n = jobs.n[blockIdx.y];
+  uint64_t head = (16u - (uint32_t)((uintptr_t)dst & 15u)) & 15u;
+  if (head > n) head = n;
+  const uint64_t body = (n - head) >> 4, tail = (n - head) & 15u;
+  const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  if (t < head) dst[t] = src[t];
+  const uint4* sv = reinterpret_cast<const uint4*>(src + head);
+  uint4* dv = reinterpret_cast<uint4*>(dst + head);
+  for (uint64_t k = t; k < body; k += stride) dv[k] = sv[k];
+  if (t < tail) dst[head + body * 16u + t] = src[head + body * 16u + t];
+}
+hipError_t put_pieces(const PieceJobs& jobs, hipStream_t st) {
+  if (jobs.count == 0) return hipSuccess;
+  if (jobs.count > KTJ_MAX_PIECES) return hipErrorInvalidValue;
+  uint64_t most = 0;
+  for (uint32_t k = 0; k < jobs.count; ++k) {
+    if (((uintptr_t)jobs.src[k] ^ (uintptr_t)jobs.dst[k]) & 15u) return hipErrorInvalidValue;
+    if (jobs.n[k] > most) most = jobs.n[k];
+  }
+  hipLaunchKernelGGL(k_put_pieces, dim3(grid_stride_for((most >> 4) + 1, KTJ_BLOCK), jobs.count), dim3(KTJ_BLOCK), 0, st, jobs);
+  return KTJ_LAUNCH_CHECK();
+}
+
 /* plain 16-byte-per-lane copy of known size: the yardstick for the HBM counters */
 __global__ void k_copy_reference(const uint4* src, uint4* dst, uint64_t n16) {
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * blockDim.x) dst[i] = src[i];

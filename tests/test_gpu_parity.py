@@ -429,6 +429,55 @@ def test_device_resident_submission():
     assert got == want
 
 
+def test_records_submitted_in_many_pieces():
+    """The same stream handed over a few records at a time (small submissions wait in a page-locked
+    ring and are moved by one kernel launch per sixteen pieces; the arrays they go to grow and move
+    in between), by two engines that are alive at the same time and by one created after both were
+    destroyed (it starts from what they left behind): every document equals the checker's."""
+    import oracle_glue as og
+    from kineto_amd.engine import TraceEngine
+    sp, release = abi.synth_stream(3, 20000, host_name="gpubox")
+    s = sp.contents
+    ora = og.OracleRun(sp)
+    want = ora.output()
+    ora.close()
+    sets = ((abi.REC_GENERIC, s.generic, s.n_generic, 64), (abi.REC_RUNTIME, s.runtime, s.n_runtime, 96),
+            (abi.REC_DEVICE, s.device, s.n_device, 64), (abi.REC_EXTCORR, s.extcorr, s.n_extcorr, 16))
+    counts = (s.n_generic, s.n_runtime, s.n_device, s.n_extcorr)
+
+    def feed(eng, step):
+        s.n_generic = s.n_runtime = s.n_device = s.n_extcorr = 0   # submit_stream then sends no records
+        try:
+            eng.submit_stream(sp)
+        finally:
+            s.n_generic, s.n_runtime, s.n_device, s.n_extcorr = counts
+        for cls, ptr, n, size in sets:
+            base = C.cast(ptr, C.c_void_p).value
+            k = 0
+            while k < n:
+                m = min(step + (k % 7), n - k)   # ragged piece sizes
+                assert eng.lib.ktj_submit_records(eng.h, cls, C.c_void_p(base + k * size), m) == 0
+                k += m
+
+    a = TraceEngine(s.trace_name.decode(), device=0)
+    b = TraceEngine(s.trace_name.decode(), device=0)
+    feed(a, 37)
+    feed(b, 611)      # pieces just below the ring's limit per submission
+    b.process()
+    a.process()
+    got_a, got_b = a.output(), b.output()
+    a.close()
+    b.close()
+    with TraceEngine(s.trace_name.decode(), device=0) as c:
+        feed(c, 5)
+        c.process()
+        got_c = c.output()
+    release()
+    assert got_a == want
+    assert got_b == want
+    assert got_c == want
+
+
 @pytest.mark.parametrize("cfg", [3, 2, 4, 5])
 def test_full_size_config_digest(cfg):
     """Configurations 2 to 5 at their full sizes (1 is at its full size among the cases above): the
