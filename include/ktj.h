@@ -470,8 +470,9 @@ typedef struct ktj_engine ktj_engine;
  * (CuptiActivity.h:424-458).
  *
  * ktj_destroy leaves what every engine needs before its first record (its stream and events, the
- * small page-locked buffers, 1 MiB of device memory for the inputs of small traces) and, while they
- * are small (64 MiB together), the working memory and the document buffer of its last pass behind
+ * small page-locked buffers, 1 MiB of device memory for the inputs of small traces), the 64 MiB of
+ * page-locked staging for large submissions if the engine made one, and, while they are small
+ * (64 MiB together), the working memory and the document buffer of its last pass behind
  * for the next ktj_create on the same device, which starts from them instead of allocating: one
  * such set per device, held until the process ends.  A trace of a few records otherwise spends
  * more time creating and destroying these than on the GPU.  Nothing is kept of an engine that saw
