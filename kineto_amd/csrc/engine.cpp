@@ -414,9 +414,15 @@ int append_from_host(ktj_engine* e, DevVec& v, const void* src, size_t n) {
         if (err[t] == hipSuccess) err[t] = hipEventRecord(e->ev_stage_big[slot], st);
       }
     };
+    for (auto& x : err) x = hipSuccess;
     std::vector<std::thread> pool;
-    for (unsigned t = 1; t < n_threads; ++t) pool.emplace_back(worker, t);
+    unsigned started = 1; /* thread 0 is this one; a thread that cannot be started has its chunks copied here */
+    try {
+      pool.reserve(n_threads);
+      for (; started < n_threads; ++started) pool.emplace_back(worker, started);
+    } catch (...) {}
     worker(0);
+    for (unsigned t = started; t < n_threads; ++t) worker(t);
     for (auto& th : pool) th.join();
     /* the slots are free for the next call once the stream has passed them */
     const hipError_t done = hipStreamSynchronize(st);
@@ -585,12 +591,17 @@ bool take_kit(ktj_engine* e) {
 /* the engine's device is current and its stream is idle; whatever is not taken stays with the engine */
 void give_kit(ktj_engine* e) {
   if (e->hip_failed || !e->stream || !e->h_ctl || !e->pinned_small || !e->stage_small || !e->d_scalars.own) return;
+  if (e->pinned_small_cap > KTJ_KIT_PINNED_BYTES_MAX) return; /* grown for an unusually long header: not worth holding */
   for (auto& ev : e->ev) if (!ev) return;
   for (auto& ev : e->ev_d2h) if (!ev) return;
   std::lock_guard<std::mutex> lock(g_kit_mutex);
-  Kit*& slot = kits()[e->device];
-  if (!slot) slot = new (std::nothrow) Kit();
-  if (!slot || slot->full) return;
+  Kit* slot = nullptr;
+  try {
+    Kit*& entry = kits()[e->device];
+    if (!entry) entry = new Kit();
+    slot = entry;
+  } catch (...) { return; }
+  if (slot->full) return;
   Kit& k = *slot;
   k.stream = e->stream; e->stream = nullptr;
   memcpy(k.ev, e->ev, sizeof k.ev); memset(e->ev, 0, sizeof e->ev);
