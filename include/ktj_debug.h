@@ -38,6 +38,11 @@ int ktj_debug_fetch(ktj_engine* e, int what, void* dst, uint64_t cap, uint64_t* 
  * second run's time: the achievable-bandwidth yardstick and the scale for the HBM counters. */
 int ktj_debug_copy_reference(ktj_engine* e, uint64_t n_bytes, float* ms);
 
+/* on != 0: a trace of one sort tile (up to 4096 rows) is sorted by the launches of a large trace
+ * (keys, then one scatter per pass) instead of by the one launch that does it all; for the tests
+ * that run small cases through both.  Process-wide. */
+void ktj_debug_force_sort_passes(int on);
+
 #ifdef __cplusplus
 }
 #endif

@@ -279,6 +279,8 @@ def load_engine():
         lib.ktj_version.argtypes = []
         lib.ktj_debug_fetch.restype = C.c_int
         lib.ktj_debug_fetch.argtypes = [vp, C.c_int, C.c_void_p, C.c_uint64, C.POINTER(C.c_uint64)]
+        lib.ktj_debug_force_sort_passes.restype = None
+        lib.ktj_debug_force_sort_passes.argtypes = [C.c_int]
         lib.ktj_debug_copy_reference.restype = C.c_int
         lib.ktj_debug_copy_reference.argtypes = [vp, C.c_uint64, C.POINTER(C.c_float)]
         _engine = lib

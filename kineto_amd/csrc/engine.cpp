@@ -1606,6 +1606,8 @@ int ktj_get_stats(ktj_engine* e, ktj_stats* out) {
   return KTJ_OK;
 }
 
+void ktj_debug_force_sort_passes(int on) { sort_packed_force_passes(on != 0); }
+
 int ktj_debug_copy_reference(ktj_engine* e, uint64_t n_bytes, float* ms) {
   if (!e || !ms) return KTJ_ERR_ARG;
   HIPCHK(hipSetDevice(e->device));

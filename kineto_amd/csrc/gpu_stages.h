@@ -302,6 +302,7 @@ hipError_t clear_error_bits(Scalars* sc, unsigned int bits, hipStream_t st);
 /* The composite-key sort on single 64-bit words (key above the arrival index); perm receives the
  * arrival index per sorted position.  Usable when sort_packed_fits(n, key_bits). */
 bool sort_packed_fits(uint64_t n, uint32_t key_bits);
+void sort_packed_force_passes(bool on); /* tests: no one-launch sort of a single tile */
 hipError_t sort_packed(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits,
                        uint32_t key_bits, uint64_t* buf_a, uint64_t* buf_b, uint32_t* perm, uint32_t* hist, uint64_t* scan_tmp,
                        hipStream_t st);

@@ -1862,6 +1862,107 @@ k_sortp_scatter(const uint64_t* in, uint64_t* words_out, uint32_t* perm_out, uin
   }
 }
 
+/* A trace of one tile: keys, every pass and the permutation in one launch of one workgroup (six
+ * launches of a few microseconds each otherwise).  Keys and arrival indices stay in registers and
+ * LDS between the passes; a pass ranks the keys as k_sortp_scatter does (ballots among the lanes of
+ * a wavefront, running counts per wavefront and digit) and puts them in LDS in the new order, from
+ * where every thread takes the keys of its positions for the next pass. */
+template <int BITS, int THREADS, int ITEMS>
+__global__ void __launch_bounds__(THREADS)
+k_sortp_single(Columns c, uint32_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits, uint32_t key_bits,
+               uint32_t* perm_out) {
+  using P = SortP<BITS, THREADS, ITEMS>;
+  __shared__ uint64_t s_key[P::TILE];
+  __shared__ uint16_t s_idx[P::TILE];
+  __shared__ uint32_t wave_run[P::WAVES][P::NB];
+  __shared__ uint32_t digit_start[P::NB];
+  __shared__ uint32_t wave_tot[P::WAVES];
+  static_assert(P::TILE <= 65536, "arrival indices are kept as 16 bits");
+  static_assert(P::NB == THREADS, "a thread owns one digit");
+  const uint32_t w = threadIdx.x >> 6, lane = lane_id();
+  const uint64_t lt = lanemask_lt();
+  const uint32_t chunk = w * P::WAVE_KEYS;
+  typedef volatile __attribute__((address_space(3))) uint32_t* lds_counts;
+  lds_counts my_run = (lds_counts)&wave_run[w][0];
+  uint64_t key[P::ITEMS];
+  uint16_t idx[P::ITEMS];
+  uint32_t rank[P::ITEMS];
+  uint16_t dig[P::ITEMS];
+  const uint64_t ts_min = sc->ts_min_biased;
+#pragma unroll
+  for (int r = 0; r < P::ITEMS; ++r) {
+    const uint32_t a = chunk + (uint32_t)r * 64u + lane;
+    uint64_t k = 1ULL << key_bits; /* dropped rows sort behind everything */
+    if (a < n && (c.meta[a] & KTJ_M_VALID)) {
+      const uint64_t rd = set_rank(s.dev_keys, s.dev_rank, (uint64_t)c.dev[a]);
+      const uint64_t rr = set_rank(s.res_keys, s.res_rank, (uint64_t)c.res[a]);
+      const uint64_t rel = ((uint64_t)c.ts[a] ^ 0x8000000000000000ULL) - ts_min;
+      k = ((((rd << res_bits) | rr)) << ts_bits) | rel;
+    }
+    key[r] = k;
+    idx[r] = (uint16_t)a;
+  }
+  const uint32_t passes = (key_bits + 1u + BITS - 1u) / BITS;
+  for (uint32_t pass = 0; pass < passes; ++pass) {
+    const uint32_t shift = pass * BITS;
+    wave_run[0][threadIdx.x] = 0;
+#pragma unroll
+    for (int k = 1; k < P::WAVES; ++k) wave_run[k][threadIdx.x] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < P::ITEMS; ++r) {
+      const bool valid = chunk + (uint32_t)r * 64u + lane < n;
+      const uint32_t digit = (uint32_t)(key[r] >> shift) & (P::NB - 1u);
+      dig[r] = (uint16_t)digit;
+      uint64_t peers = __ballot(valid ? 1 : 0);
+#pragma unroll
+      for (int b = 0; b < BITS; ++b) {
+        const uint64_t bal = __ballot((digit >> b) & 1u);
+        peers &= ((digit >> b) & 1u) ? bal : ~bal;
+      }
+      const uint32_t rank_in_wave = (uint32_t)__popcll(peers & lt);
+      const uint32_t before = my_run[digit];
+      rank[r] = before + rank_in_wave;
+      if (valid && rank_in_wave == 0) my_run[digit] = before + (uint32_t)__popcll(peers);
+    }
+    __syncthreads();
+    {
+      /* thread d: the wavefronts' counts of digit d become their starts inside the digit's run, the
+       * digit's total goes into the scan that gives the run's start inside the tile */
+      const int d = (int)threadIdx.x;
+      uint32_t t = 0;
+#pragma unroll
+      for (int k = 0; k < P::WAVES; ++k) { const uint32_t cnt = wave_run[k][d]; wave_run[k][d] = t; t += cnt; }
+      uint32_t inc = t;
+      for (int o = 1; o < 64; o <<= 1) { const uint32_t v = __shfl_up(inc, o); if (lane >= (uint32_t)o) inc += v; }
+      if (lane == 63) wave_tot[w] = inc;
+      __syncthreads();
+      uint32_t start = inc - t;
+      for (uint32_t k = 0; k < w; ++k) start += wave_tot[k];
+      digit_start[d] = start;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < P::ITEMS; ++r) {
+      if (chunk + (uint32_t)r * 64u + lane < n) {
+        const uint32_t digit = dig[r];
+        const uint32_t p = digit_start[digit] + wave_run[w][digit] + rank[r];
+        s_key[p] = key[r];
+        s_idx[p] = idx[r];
+      }
+    }
+    __syncthreads();
+    if (pass + 1 == passes) break;
+#pragma unroll
+    for (int r = 0; r < P::ITEMS; ++r) {
+      const uint32_t a = chunk + (uint32_t)r * 64u + lane;
+      if (a < n) { key[r] = s_key[a]; idx[r] = s_idx[a]; }
+    }
+    __syncthreads();
+  }
+  for (uint32_t p = threadIdx.x; p < n; p += THREADS) perm_out[p] = s_idx[p];
+}
+
 template <int BITS, int THREADS, int ITEMS>
 static hipError_t sort_packed_t(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits,
                                 uint32_t key_bits, uint32_t idx_bits, uint64_t* buf_a, uint64_t* buf_b, uint32_t* perm,
@@ -1906,6 +2007,9 @@ static hipError_t sort_packed_t(Columns c, uint64_t n, SortSets s, const Scalars
 }
 #define SORTP_BITS 8
 #define SORTP_THREADS 256
+/* tests: the one-launch sort of a single tile switched off, so that such a trace takes the passes of a large one */
+static bool g_sortp_no_single = false;
+void sort_packed_force_passes(bool on) { g_sortp_no_single = on; }
 bool sort_packed_fits(uint64_t n, uint32_t key_bits) {
   const uint32_t total_bits = key_bits + 1u;
   const uint32_t idx_bits = (uint32_t)(64 - __builtin_clzll(n > 1 ? n - 1 : 1));
@@ -1916,6 +2020,11 @@ hipError_t sort_packed(Columns c, uint64_t n, SortSets s, const Scalars* sc, uin
                        hipStream_t st) {
   if (n == 0) return hipSuccess;
   const uint32_t idx_bits = (uint32_t)(64 - __builtin_clzll(n > 1 ? n - 1 : 1));
+  if (n <= (uint64_t)SORTP_THREADS * 16u && !g_sortp_no_single) {
+    hipLaunchKernelGGL((k_sortp_single<SORTP_BITS, SORTP_THREADS, 16>), dim3(1), dim3(SORTP_THREADS), 0, st, c, (uint32_t)n, s, sc, ts_bits,
+                       res_bits, key_bits, perm);
+    return KTJ_LAUNCH_CHECK();
+  }
   /* a few thousand keys are one tile; up to SORTP_SMALL_N keys, tiles of 512 spread over the GPU
    * finish a pass sooner than the few 4096-key tiles would (30 000 keys: 76 against 130 us for the
    * sort, 330 000 keys: 113 against 155 us; from a million keys on the large tiles win) */

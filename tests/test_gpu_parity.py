@@ -330,6 +330,32 @@ def test_empty_and_tiny_streams_on_gpu():
     _engine_vs_oracle(b.build())
 
 
+def test_small_traces_through_the_passes_of_a_large_one():
+    """A trace of up to 4096 rows is sorted by one launch of one workgroup; with that switched off it
+    takes the key and scatter launches of a large trace.  Both forms, on the smallest cases, the
+    known-answer cases, a tile that is exactly full and one row more, and seeded
+    random streams: same permutation, same document."""
+    import kat_cases
+    import random_streams
+    lib = abi.load_engine()
+    sizes = [(1, 1), (5, 3), (1, 1365), (1, 1366), (3, 1300), (4, 1000), (2, 900)]   # (1, 1365): 4095 rows; (1, 1366): 4098
+    try:
+        for forced in (1, 0):
+            lib.ktj_debug_force_sort_passes(forced)
+            for cfg, n in sizes:
+                print(f"forced={forced} config={cfg} n={n}", flush=True)
+                run_case(cfg, n)
+            for case in kat_cases.SUBSTRING_CASES:
+                print(f"forced={forced} case {case.__name__}", flush=True)
+                b, expect = case()
+                _engine_vs_oracle(b.build(), expect)
+            for seed in (3, 11, 14):
+                sp = random_streams.random_stream(seed, wide_ids=seed % 2 == 1, unique_runtime_ids=seed % 3 == 2).build()
+                _engine_vs_oracle(sp)
+    finally:
+        lib.ktj_debug_force_sort_passes(0)
+
+
 def test_process_is_repeatable_and_file_output(tmp_path):
     import hashlib
     import oracle_glue as og
