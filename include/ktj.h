@@ -468,6 +468,9 @@ typedef struct ktj_engine ktj_engine;
  * KTJ_CREATE_CUDA12_ARGS prints the "graph id", "graph node id", "channel" and "channel_type" keys
  * of memset rows (ktj_memset_rec), which the reference compiles in for CUDA >= 12 only
  * (CuptiActivity.h:424-458).
+ * KTJ_CREATE_NO_STAGE_TIMES leaves the events between the stages of a pass out: ktj_stats then
+ * reports the time of the whole pass only (stage_ms[KTJ_STAGE_TOTAL_GPU]), and a trace of a few
+ * records is finished a tenth sooner.
  *
  * ktj_destroy leaves what every engine needs before its first record (its stream and events, the
  * small page-locked buffers, 1 MiB of device memory for the inputs of small traces), the 64 MiB of
@@ -484,6 +487,7 @@ typedef struct ktj_engine ktj_engine;
 #define KTJ_CREATE_PAIR_SORT 0x8u
 #define KTJ_CREATE_DISPLAY_NS 0x10u
 #define KTJ_CREATE_CUDA12_ARGS 0x20u
+#define KTJ_CREATE_NO_STAGE_TIMES 0x40u
 int ktj_create(ktj_engine** out, const char* out_path, int64_t base_time_ns, int hip_device,
                uint32_t flags);
 void ktj_destroy(ktj_engine* e);

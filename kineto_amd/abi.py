@@ -16,6 +16,7 @@ KTJ_CREATE_HASH_JOIN = 0x4
 KTJ_CREATE_PAIR_SORT = 0x8
 KTJ_CREATE_DISPLAY_NS = 0x10
 KTJ_CREATE_CUDA12_ARGS = 0x20
+KTJ_CREATE_NO_STAGE_TIMES = 0x40
 KTJ_GF_WIDE_DEVICE = 0x04
 
 REC_GENERIC, REC_RUNTIME, REC_DEVICE, REC_EXTCORR, REC_USERCORR = 0, 1, 2, 3, 4

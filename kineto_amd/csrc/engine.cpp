@@ -1121,6 +1121,9 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   const ktj_device_rec* d_recs = static_cast<const ktj_device_rec*>(e->devrows.ptr());
   const ktj_extcorr_rec* x_recs = static_cast<const ktj_extcorr_rec*>(e->extcorr.ptr());
 
+  /* an event on the stream costs the GPU a microsecond or two between two kernels: a trace of a few
+   * records can do without the ten that separate the stages (KTJ_CREATE_NO_STAGE_TIMES) */
+  const bool stage_times = !(e->flags & KTJ_CREATE_NO_STAGE_TIMES);
   HIPCHK(hipEventRecord(e->ev[EV_START], st));
   HIPCHK(init_scalars(sc, st));
 
@@ -1164,7 +1167,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
                       e->d_arg_off.as<uint64_t>(), e->d_sflags.as<uint32_t>(), e->d_name_blob.as<char>(),
                       e->d_arg_blob.as<char>(), st));
   }
-  HIPCHK(hipEventRecord(e->ev[EV_DICT], st));
+  if (stage_times) HIPCHK(hipEventRecord(e->ev[EV_DICT], st));
 
   /* ---- stage 1: decode ---- */
   KeyRange* parts = e->range_parts.as<KeyRange>(); /* [generic | runtime | runtime narrowed | device] */
@@ -1178,8 +1181,8 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
                         e->win_start, e->win_end, sc, st));
   HIPCHK(decode_device(d_recs, nd, c, ng + nr, e->dev_brief.as<DevBrief>(), parts + decode_blocks(ng) + 2 * decode_blocks(nr), clk,
                        e->win_start, e->win_end, sc, st));
-  HIPCHK(hipEventRecord(e->ev[EV_DECODE], st));
-  HIPCHK(hipEventRecord(e->ev[EV_CONVERT], st));
+  if (stage_times) HIPCHK(hipEventRecord(e->ev[EV_DECODE], st));
+  if (stage_times) HIPCHK(hipEventRecord(e->ev[EV_CONVERT], st));
 
   /* ---- stage 2b: joins ---- */
   Table tf{e->t_full.as<uint64_t>(), cap_full - 1, 0u, &sc->plan.ctl[KTJ_TBL_FULL]};
@@ -1217,12 +1220,12 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
     N += e->n_spans;
     e->N = N;
   }
-  HIPCHK(hipEventRecord(e->ev[EV_JOIN], st));
+  if (stage_times) HIPCHK(hipEventRecord(e->ev[EV_JOIN], st));
 
   /* ---- stage 3: canonical order ---- */
   HIPCHK(collect_distinct(c, N, sets, sc, st));
   HIPCHK(rank_distinct(sets, sc, st));
-  HIPCHK(hipEventRecord(e->ev[EV_SORT_A], st));
+  if (stage_times) HIPCHK(hipEventRecord(e->ev[EV_SORT_A], st));
   HIPCHK(publish(sc, nullptr, nullptr, 0, &e->h_ctl_dev->scalars, nullptr, nullptr, st));
   if (!out_device && !e->noalloc && e->out.cap == 0) {
     /* An engine's first pass has no document buffer yet, and how long the document is comes out of
@@ -1248,7 +1251,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
     key_bits = ts_bits + res_bits + dev_bits;
     rank_bits = res_bits + dev_bits;
   }
-  HIPCHK(hipEventRecord(e->ev[EV_SORT_B], st));
+  if (stage_times) HIPCHK(hipEventRecord(e->ev[EV_SORT_B], st));
   {
     uint64_t* ka = e->keys_a.as<uint64_t>(); uint32_t* va = e->vals_a.as<uint32_t>();
     uint64_t* kb = e->keys_b.as<uint64_t>(); uint32_t* vb = e->vals_b.as<uint32_t>();
@@ -1288,7 +1291,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
       if (rc != KTJ_OK) return rc;
     }
   }
-  HIPCHK(hipEventRecord(e->ev[EV_SORT], st));
+  if (stage_times) HIPCHK(hipEventRecord(e->ev[EV_SORT], st));
 
   /* ---- stage 4a: joined rows + lengths ---- */
   const uint32_t* sync_first = nullptr;
@@ -1305,11 +1308,11 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   HIPCHK(mat_device_rows(d_recs, nd, c, ng + nr, e->dev_link.as<DevLink>(), ctx, mat, e->len.as<uint32_t>(), sc, st));
   HIPCHK(gather_len(e->perm, e->len.as<uint32_t>(), N, e->len_sorted.as<uint32_t>(), e->kind_sorted.as<uint8_t>(), st));
   if (n_coll) HIPCHK(collective_first(mat, e->perm, e->scalars.n_valid, n_coll, e->d_coll_first.as<uint32_t>(), st));
-  HIPCHK(hipEventRecord(e->ev[EV_SIZE], st));
+  if (stage_times) HIPCHK(hipEventRecord(e->ev[EV_SIZE], st));
 
   /* ---- scan ---- */
   HIPCHK(scan_u32_to_u64(e->len_sorted.as<uint32_t>(), e->offs.as<uint64_t>(), N, e->scan_tmp.as<uint64_t>(), st));
-  HIPCHK(hipEventRecord(e->ev[EV_SCAN], st));
+  if (stage_times) HIPCHK(hipEventRecord(e->ev[EV_SCAN], st));
   uint64_t act_bytes = 0;
   e->coll_first.assign(2ull * n_coll, 0xFFFFFFFFu);
   const bool list_fits = 2ull * n_coll * 4 <= e->pinned_small_cap; /* through the engine's pinned buffer when it fits */
@@ -1381,7 +1384,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
   }
   const uint32_t tile = emit_tile_bytes(act_bytes, e->scalars.n_valid);
   NEED(e->tile_start, (emit_tile_count(e->prefix_len, act_bytes, tile) + 2) * 4);
-  HIPCHK(hipEventRecord(e->ev[EV_EMIT_START], st));
+  if (stage_times) HIPCHK(hipEventRecord(e->ev[EV_EMIT_START], st));
   {
     if (e->flags & KTJ_CREATE_TILE_EMIT)
       HIPCHK(emit(mat, e->perm, e->offs.as<uint64_t>(), N, ctx, e->out.as<char>(), e->prefix_len, act_bytes, tile,
@@ -1415,6 +1418,7 @@ static int process_pass(ktj_engine* e, int64_t end_time_ns, void* out_device, ui
       {KTJ_STAGE_SIZE, EV_SORT, EV_SIZE},        {KTJ_STAGE_SCAN, EV_SIZE, EV_SCAN},
       {KTJ_STAGE_EMIT, EV_EMIT_START, EV_EMIT}};
   for (const auto& sp : spans) {
+    if (!stage_times) break;
     float ms = 0;
     HIPCHK(hipEventElapsedTime(&ms, e->ev[sp.from], e->ev[sp.to]));
     s.stage_ms[sp.stage] += ms;

@@ -22,10 +22,10 @@ class EngineError(RuntimeError):
 
 
 class TraceEngine:
-    def __init__(self, out_path, base_time_ns=abi.DEFAULT_BASE_TIME_NS, device=0, no_file=True, tile_emit=False, hash_join=False, pair_sort=False, display_ns=False, cuda12_args=False):
+    def __init__(self, out_path, base_time_ns=abi.DEFAULT_BASE_TIME_NS, device=0, no_file=True, tile_emit=False, hash_join=False, pair_sort=False, display_ns=False, cuda12_args=False, no_stage_times=False):
         self.lib = abi.load_engine()
         self.h = C.c_void_p()
-        flags = (abi.KTJ_CREATE_NO_FILE if no_file else 0) | (abi.KTJ_CREATE_TILE_EMIT if tile_emit else 0) | (abi.KTJ_CREATE_HASH_JOIN if hash_join else 0) | (abi.KTJ_CREATE_PAIR_SORT if pair_sort else 0) | (abi.KTJ_CREATE_DISPLAY_NS if display_ns else 0) | (abi.KTJ_CREATE_CUDA12_ARGS if cuda12_args else 0)
+        flags = (abi.KTJ_CREATE_NO_FILE if no_file else 0) | (abi.KTJ_CREATE_TILE_EMIT if tile_emit else 0) | (abi.KTJ_CREATE_HASH_JOIN if hash_join else 0) | (abi.KTJ_CREATE_PAIR_SORT if pair_sort else 0) | (abi.KTJ_CREATE_DISPLAY_NS if display_ns else 0) | (abi.KTJ_CREATE_CUDA12_ARGS if cuda12_args else 0) | (abi.KTJ_CREATE_NO_STAGE_TIMES if no_stage_times else 0)
         rc = self.lib.ktj_create(C.byref(self.h), out_path.encode(), base_time_ns, device, flags)
         if rc != 0:
             msg = self.lib.ktj_last_error(self.h).decode() if self.h else "allocation failed"

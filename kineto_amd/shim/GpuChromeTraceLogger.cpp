@@ -87,7 +87,7 @@ struct GpuChromeTraceLogger::Packed {
 GpuChromeTraceLogger::GpuChromeTraceLogger(const std::string& traceFileName, int hipDevice)
     : fileName_(traceFileName), staging_(new Packed) {
   /* the engine applies the default-file-name rule (output_json.cpp:481-483) for an empty name */
-  uint32_t flags = 0;
+  uint32_t flags = KTJ_CREATE_NO_STAGE_TIMES; /* a logger reports no stage times */
 #ifdef DISPLAY_TRACE_IN_NS /* the reference's compile-time switch (output_json.cpp:451-454) */
   flags |= KTJ_CREATE_DISPLAY_NS;
 #endif
