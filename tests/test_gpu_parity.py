@@ -504,6 +504,46 @@ def test_records_submitted_in_many_pieces():
     assert got_c == want
 
 
+def test_engines_on_several_threads():
+    """Four threads create, feed, run and destroy engines at the same time (a profiler finishes traces
+    on background threads): the stream, events and buffers that a destroyed engine leaves for the next
+    one change hands between the threads; every document equals the checker's."""
+    import threading
+    import oracle_glue as og
+    from kineto_amd.engine import TraceEngine
+    cases = [(1, 300), (3, 2000), (4, 900), (5, 200), (2, 3000), (3, 40000)]
+    streams, want = {}, {}
+    for key in cases:
+        sp, release = abi.synth_stream(*key, host_name="gpubox")
+        ora = og.OracleRun(sp)
+        want[key] = ora.output()
+        ora.close()
+        streams[key] = (sp, release)
+    bad = []
+
+    def work(tid):
+        try:
+            for it in range(12):
+                key = cases[(tid + it) % len(cases)]
+                sp = streams[key][0]
+                with TraceEngine(sp.contents.trace_name.decode(), device=0, no_stage_times=it % 2 == 0) as eng:
+                    eng.submit_stream(sp)
+                    eng.process()
+                    if eng.output() != want[key]:
+                        bad.append((tid, it, key))
+        except Exception as ex:   # noqa: BLE001 - reported by the assertion below
+            bad.append((tid, repr(ex)))
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for sp, release in streams.values():
+        release()
+    assert not bad, bad
+
+
 @pytest.mark.parametrize("cfg", [3, 2, 4, 5])
 def test_full_size_config_digest(cfg):
     """Configurations 2 to 5 at their full sizes (1 is at its full size among the cases above): the
