@@ -113,6 +113,9 @@ struct Columns {
 };
 
 /* small block of scalars the kernels update and the host reads back */
+#ifndef KTJ_COUNTER_SHARDS
+#define KTJ_COUNTER_SHARDS 64u
+#endif
 struct Scalars {
   unsigned long long ts_min_biased;   /* min over valid rows of ts ^ 2^63 */
   unsigned long long ts_max_biased;
@@ -136,7 +139,15 @@ struct Scalars {
   unsigned int ext_ids_repeat;        /* two external-correlation records share a correlation id */
   alignas(256) JoinPlan plan;         /* key ranges and modes of the join tables: read by every row of the join
                                          kernels, so kept off the cache lines that take the counters' atomics */
+  /* The counters that most workgroups add to (KTJ_CNT_*) are kept in KTJ_COUNTER_SHARDS copies, one
+   * 128-byte line each; a workgroup adds to the copy of its index.  Atomics on one address are carried
+   * out one after the other, and tens of thousands of workgroups adding to the same few words cost the
+   * join more than its table lookups.  k_publish sums the copies into the fields above, which nothing
+   * on the device reads; it hands the host everything in front of this array. */
+  alignas(128) unsigned long long shard[KTJ_COUNTER_SHARDS][16];
 };
+enum { KTJ_CNT_OUT_OF_RANGE = 0, KTJ_CNT_OUT_OF_ORDER, KTJ_CNT_FLOW, KTJ_CNT_LINKED, KTJ_CNT_BLANK_NAMES, KTJ_CNT_VALID,
+       KTJ_CNT_SYNC_TYPED, KTJ_CNT_COUNT };
 #define KTJ_DEVERR_TABLE_FULL 1u         /* a join table sized from the record counts filled up (a defect) */
 #define KTJ_DEVERR_DISTINCT_DEVICES 2u   /* more distinct deviceId values than the rank set holds: the sort
                                             takes its slower path without ranks, no error reaches the caller */
@@ -165,7 +176,7 @@ struct ApiTable {
 /* read-backs and text of a pass without the copy engine: sc, *total (may be null) and list[0..n_list)
  * into pinned host memory (device-visible addresses); two pieces of host text to their places in the
  * document (source and destination of a piece must agree modulo 16) */
-hipError_t publish(const Scalars* sc, const uint64_t* total, const uint32_t* list, uint32_t n_list, Scalars* h_sc,
+hipError_t publish(Scalars* sc, const uint64_t* total, const uint32_t* list, uint32_t n_list, Scalars* h_sc,
                    uint64_t* h_total, uint32_t* h_list, hipStream_t st);
 hipError_t put_text(const char* src_a, char* dst_a, uint64_t n_a, const char* src_b, char* dst_b, uint64_t n_b, hipStream_t st);
 /* pieces of page-locked host memory to their places in device memory, in one launch */

@@ -163,18 +163,26 @@ __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
 }
 /* Sums a per-thread count over the workgroup and adds it to a global counter with one atomic per
  * workgroup (a single hot address serialises atomics in L2, so they must be rare).  Must be
- * reached by every thread of the workgroup. */
-__device__ __forceinline__ void block_add(unsigned long long* counter, uint32_t mine) {
+ * reached by every thread of the workgroup.  block_add_to: a counter of its own address, for counts
+ * that are zero in nearly every workgroup; block_add: one of the sharded counters of Scalars. */
+__device__ __forceinline__ uint32_t block_sum(uint32_t mine) { /* the sum, in thread 0 */
   __shared__ uint32_t partial[KTJ_BLOCK >> 6];
   const uint32_t w = wave_sum_u32(mine);
   __syncthreads();
   if (lane_id() == 0) partial[threadIdx.x >> 6] = w;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    uint32_t t = 0;
+  uint32_t t = 0;
+  if (threadIdx.x == 0)
     for (uint32_t k = 0; k < (blockDim.x >> 6); ++k) t += partial[k];
-    if (t) atomicAdd(counter, (unsigned long long)t);
-  }
+  return t;
+}
+__device__ __forceinline__ void block_add_to(unsigned long long* counter, uint32_t mine) {
+  const uint32_t t = block_sum(mine);
+  if (threadIdx.x == 0 && t) atomicAdd(counter, (unsigned long long)t);
+}
+__device__ __forceinline__ void block_add(Scalars* sc, int which, uint32_t mine) {
+  const uint32_t t = block_sum(mine);
+  if (threadIdx.x == 0 && t) atomicAdd(&sc->shard[blockIdx.x & (KTJ_COUNTER_SHARDS - 1u)][which], (unsigned long long)t);
 }
 /* grid-stride kernels: enough workgroups to fill 256 CUs several times over */
 #define KTJ_MAX_GRID 4096u
@@ -188,6 +196,9 @@ __global__ void k_fill_u32(uint32_t* p, uint32_t v, uint64_t n) {
   if (i < n) p[i] = v;
 }
 __global__ void k_init_scalars(Scalars* s) {
+  if (blockIdx.x == 0)
+    for (uint32_t c = threadIdx.x; c < KTJ_COUNTER_SHARDS; c += blockDim.x)
+      for (int k = 0; k < 16; ++k) s->shard[c][k] = 0;
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     s->ts_min_biased = ~0ULL; s->ts_max_biased = 0;
     s->out_of_range = 0; s->out_of_order = 0; s->n_flow = 0; s->n_linked = 0; s->n_blank_names = 0; s->n_valid = 0;
@@ -237,6 +248,7 @@ hipError_t fill_many(const FillJobs& jobs, hipStream_t st) {
   return KTJ_LAUNCH_CHECK();
 }
 hipError_t init_scalars(Scalars* s, hipStream_t st) {
+  static_assert((KTJ_COUNTER_SHARDS & (KTJ_COUNTER_SHARDS - 1u)) == 0, "a workgroup's copy is its index modulo the number of copies");
   hipLaunchKernelGGL(k_init_scalars, dim3(1), dim3(64), 0, st, s);
   return KTJ_LAUNCH_CHECK();
 }
@@ -569,7 +581,7 @@ __global__ void k_decode_generic(const ktj_generic_rec* recs, uint64_t n, Column
   const ktj_generic_rec* l = stage_records(recs, n, stage, &cnt);
   /* rows that may need a Stream Sync row of their own are rare: the extra passes run only if any */
   const bool sync_typed = threadIdx.x < cnt && l[threadIdx.x].type == KTJ_TYPE_CUDA_SYNC;
-  if (__syncthreads_or(sync_typed ? 1 : 0)) block_add(&sc->n_sync_typed, sync_typed ? 1u : 0u);
+  if (__syncthreads_or(sync_typed ? 1 : 0)) block_add(sc, KTJ_CNT_SYNC_TYPED, sync_typed ? 1u : 0u);
   if (id_range) block_key_range(threadIdx.x < cnt, threadIdx.x < cnt ? (uint64_t)(int64_t)l[threadIdx.x].id : 0, id_range);
   if (threadIdx.x >= cnt) return;
   const ktj_generic_rec g = l[threadIdx.x];
@@ -615,7 +627,7 @@ __global__ void k_decode_runtime(const ktj_runtime_rec* recs, uint64_t n, Column
               (oor ? 0u : KTJ_M_VALID);
   c.ext[a] = 0;
   }
-  block_add(&sc->out_of_range, oor);
+  block_add(sc, KTJ_CNT_OUT_OF_RANGE, oor);
 }
 __global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns c, uint64_t first, DevBrief* brief,
                                 KeyRange* id_range, ClockDev clk, int64_t win_start, int64_t win_end, Scalars* sc) {
@@ -644,7 +656,7 @@ __global__ void k_decode_device(const ktj_device_rec* recs, uint64_t n, Columns 
   br.queue = d->queue; br.device = d->device; br.domain = dom;
   brief[a - first] = br;
   }
-  block_add(&sc->out_of_range, oor);
+  block_add(sc, KTJ_CNT_OUT_OF_RANGE, oor);
 }
 
 uint64_t decode_blocks(uint64_t n) { return grid_for(n, KTJ_BLOCK); }
@@ -961,10 +973,10 @@ __global__ void k_link_device(uint64_t n, Columns c, uint64_t first_device, Tabl
     }
     if (is_async_op(domain) && res == 0) ++n_unresolved;
   }
-  block_add(&sc->n_linked, n_linked);
-  block_add(&sc->out_of_order, n_bad);
-  block_add(&sc->n_unresolved, n_unresolved);
-  block_add(&sc->n_device_orphans, n_orphans);
+  block_add(sc, KTJ_CNT_LINKED, n_linked);
+  block_add(sc, KTJ_CNT_OUT_OF_ORDER, n_bad);
+  block_add_to(&sc->n_unresolved, n_unresolved);
+  block_add_to(&sc->n_device_orphans, n_orphans);
 }
 /* Only when some in-window device row has an id that no runtime row has: such a row is checked
  * against the first device row of its id (act1 = this row, act2 = the first one). */
@@ -983,7 +995,7 @@ __global__ void k_device_orphans(uint64_t n, Columns c, uint64_t first_device, T
       if (t2 != 0 && t1 > t2) ++n_bad;
     }
   }
-  block_add(&sc->out_of_order, n_bad);
+  block_add(sc, KTJ_CNT_OUT_OF_ORDER, n_bad);
 }
 
 hipError_t build_cpu_ids(const ktj_generic_rec* g, uint64_t n, Table cpu, uint32_t* cpu_row, Scalars* sc, hipStream_t st) {
@@ -1351,7 +1363,7 @@ __global__ void k_collect_distinct(Columns c, uint64_t n, SortSets s, Scalars* s
       atomicMax(&sc->ts_max_biased, (unsigned long long)mx);
     }
   }
-  block_add(&sc->n_valid, n_valid);
+  block_add(sc, KTJ_CNT_VALID, n_valid);
 }
 /* one workgroup per set: rank of each distinct value = number of smaller values (signed) */
 __global__ void k_rank_distinct(SortSets s, Scalars* sc) {
@@ -2093,8 +2105,8 @@ __device__ __forceinline__ void count_row_stats(const MatRow& m, const EmitCtx& 
     ++rs->n_blank;
 }
 __device__ __forceinline__ void flush_row_stats(const RowStats& rs, Scalars* sc) {
-  block_add(&sc->n_flow, rs.n_flow);
-  block_add(&sc->n_blank_names, rs.n_blank);
+  block_add(sc, KTJ_CNT_FLOW, rs.n_flow);
+  block_add(sc, KTJ_CNT_BLANK_NAMES, rs.n_blank);
 }
 
 /* Stream Sync rows (output_json.cpp:913-943): which activity is the first of its (device, row) key
@@ -2325,7 +2337,7 @@ __global__ void KX_JOIN_ATTR k_join_runtime(const ktj_runtime_rec* r, uint64_t n
     if (any_repeat) sc->runtime_ids_repeat = 1;
   }
   flush_row_stats(rs, sc);
-  block_add(&sc->n_linked, n_linked);
+  block_add(sc, KTJ_CNT_LINKED, n_linked);
 }
 /* Only when runtime rows share slots: which row of a slot the device rows take each value from
  * (the last row that carries a stream; the last in-window kernel launch; the last in-window copy
@@ -2382,7 +2394,7 @@ __global__ void k_republish_runtime(const ktj_runtime_rec* r, uint64_t n, Column
       }
     }
   }
-  block_add(&sc->out_of_order, n_bad);
+  block_add(sc, KTJ_CNT_OUT_OF_ORDER, n_bad);
 }
 __global__ void k_mat_device(const ktj_device_rec* d, uint64_t n, Columns c, uint64_t first, const DevLink* link,
                              EmitCtx ctx, MatRow* mat, uint32_t* len, Scalars* sc) {
@@ -2646,19 +2658,38 @@ hipError_t emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* 
 /* What the host needs during a pass goes straight into its pinned memory, and the text it made
  * (header, infos, footer) comes straight out of it: one small kernel each instead of one copy
  * engine transfer per value. */
-__global__ void k_publish(const Scalars* sc, const uint64_t* total, const uint32_t* list, uint32_t n_list, Scalars* h_sc,
+__global__ void k_publish(Scalars* sc, const uint64_t* total, const uint32_t* list, uint32_t n_list, Scalars* h_sc,
                           uint64_t* h_total, uint32_t* h_list) {
   const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x, stride = gridDim.x * blockDim.x;
-  static_assert(sizeof(Scalars) % 4 == 0, "copied as 32-bit words");
-  const uint32_t* src = reinterpret_cast<const uint32_t*>(sc);
-  uint32_t* dst = reinterpret_cast<uint32_t*>(h_sc);
-  for (uint32_t k = t; k < sizeof(Scalars) / 4; k += stride) dst[k] = src[k];
+  if (blockIdx.x == 0) {
+    /* the sharded counters: their sums so far into the fields the host reads (written, not added:
+     * a pass publishes twice) */
+    if (threadIdx.x < KTJ_CNT_COUNT) {
+      unsigned long long sum = 0;
+      for (uint32_t k = 0; k < KTJ_COUNTER_SHARDS; ++k) sum += sc->shard[k][threadIdx.x];
+      switch (threadIdx.x) {
+        case KTJ_CNT_OUT_OF_RANGE: sc->out_of_range = sum; break;
+        case KTJ_CNT_OUT_OF_ORDER: sc->out_of_order = sum; break;
+        case KTJ_CNT_FLOW: sc->n_flow = sum; break;
+        case KTJ_CNT_LINKED: sc->n_linked = sum; break;
+        case KTJ_CNT_BLANK_NAMES: sc->n_blank_names = sum; break;
+        case KTJ_CNT_VALID: sc->n_valid = sum; break;
+        default: sc->n_sync_typed = sum; break;
+      }
+    }
+    __syncthreads();
+    constexpr uint32_t head_words = (uint32_t)(offsetof(Scalars, shard) / 4);
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(sc);
+    uint32_t* dst = reinterpret_cast<uint32_t*>(h_sc);
+    for (uint32_t k = threadIdx.x; k < head_words; k += blockDim.x) dst[k] = src[k];
+  }
   for (uint32_t k = t; k < n_list; k += stride) h_list[k] = list[k];
   if (t == 0 && total != nullptr) *h_total = *total;
   __threadfence_system();
 }
-hipError_t publish(const Scalars* sc, const uint64_t* total, const uint32_t* list, uint32_t n_list, Scalars* h_sc,
+hipError_t publish(Scalars* sc, const uint64_t* total, const uint32_t* list, uint32_t n_list, Scalars* h_sc,
                    uint64_t* h_total, uint32_t* h_list, hipStream_t st) {
+  static_assert(KTJ_CNT_COUNT == 7, "k_publish names every sharded counter");
   hipLaunchKernelGGL(k_publish, dim3(n_list > 4096 ? 16 : 1), dim3(KTJ_BLOCK), 0, st, sc, total, list, n_list, h_sc, h_total, h_list);
   return KTJ_LAUNCH_CHECK();
 }
