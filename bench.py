@@ -228,6 +228,46 @@ def host_to_file_legs(sp, n_records):
     return out
 
 
+def small_trace_legs():
+    """What a trace of a few records and configuration 1 at its full size (30 000 records) cost: the
+    fixed cost of the pass (some forty short kernels and two read-backs), not throughput.  Median over
+    repeated passes on a warm engine, with and without the events between the stages
+    (KTJ_CREATE_NO_STAGE_TIMES, which the ActivityLogger shim sets), and from ktj_create to
+    ktj_destroy on engines that start from what the previous one left behind."""
+    import statistics
+    from kineto_amd import abi
+    from kineto_amd.engine import TraceEngine
+    out = {}
+    for label, cfg, n in (("fifteen_records", 1, 5), ("config1_full", 1, FULL_SIZE[1])):
+        sp, release = abi.synth_stream(cfg, n, host_name="bench")
+        s = sp.contents
+        leg = {"records": int(s.n_generic + s.n_runtime + s.n_device)}
+        for key, nst in (("warm_pass_ms", False), ("warm_pass_no_stage_times_ms", True)):
+            with TraceEngine(s.trace_name.decode(), device=0, no_stage_times=nst) as eng:
+                eng.submit_stream(sp)
+                for _ in range(5):
+                    eng.process()
+                ts = []
+                for _ in range(100):
+                    t0 = time.perf_counter()
+                    eng.process()
+                    ts.append((time.perf_counter() - t0) * 1e3)
+                leg[key] = statistics.median(ts)
+        ts = []
+        for k in range(30):
+            t0 = time.perf_counter()
+            with TraceEngine(s.trace_name.decode(), device=0, no_stage_times=True) as eng:
+                eng.submit_stream(sp)
+                eng.process()
+                eng.output()
+            if k >= 5:
+                ts.append((time.perf_counter() - t0) * 1e3)
+        leg["create_to_destroy_ms"] = statistics.median(ts)   # includes this script's ctypes calls
+        release()
+        out[label] = leg
+    return out
+
+
 def host_cpu():
     model = None
     try:
@@ -458,6 +498,7 @@ def main():
     eng.close()
     host_legs = None if args.no_host_legs else host_to_file_legs(sp, n_records)
     release()
+    small = None if args.no_host_legs else small_trace_legs()
 
     # algorithmic bytes of a stage / its time, as a fraction of the HBM peak (the three stages the
     # per-kernel target of this path is stated for, and the rest beside them)
@@ -497,6 +538,7 @@ def main():
         "pcie": {"h2d_submit_s": h2d_s, "d2h_document_ms": d2h_ms, "d2h_wall_s": d2h_s,
                  "records_per_s_incl_d2h": (n_records / (ms_per_step * 1e-3 + (d2h_ms or 0) * 1e-3)) if d2h_ms else None},
         "host_legs": host_legs,
+        "small_traces": small,
         "generate_s": gen_s,
         "copy_kernel_gb_per_s": copy_gbs,
     }
