@@ -1408,6 +1408,23 @@ __device__ __forceinline__ uint64_t set_rank(const uint64_t* keys, const uint32_
   const uint32_t slot = table_find(keys, KTJ_SET_CAP - 1u, v);
   return slot != KTJ_NOSLOT ? rank[slot] : 0;
 }
+/* The same for a thread that looks up one row after the other: rows that follow each other in a
+ * record buffer mostly belong to one stream or thread, so the last wavefront-wide value and its rank
+ * are kept, and a lookup (two dependent loads at least) is only made when the value changes.  A
+ * lane's memo is a (value, rank) pair that it took part in looking up, or nothing. */
+struct RankMemo { uint64_t key; uint32_t rank; bool have; };
+__device__ __forceinline__ uint64_t set_rank_memo(const uint64_t* keys, const uint32_t* rank, uint64_t v, RankMemo& m) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  const uint64_t first = ((uint64_t)hi << 32) | lo;
+  if (__ballot(v != first) == 0) {
+    if (m.have && m.key == first) return m.rank;
+    const uint32_t slot = table_find(keys, KTJ_SET_CAP - 1u, first);
+    m.key = first; m.rank = slot != KTJ_NOSLOT ? rank[slot] : 0; m.have = true;
+    return m.rank;
+  }
+  const uint32_t slot = table_find(keys, KTJ_SET_CAP - 1u, v);
+  return slot != KTJ_NOSLOT ? rank[slot] : 0;
+}
 __global__ void k_make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t ts_bits, uint32_t res_bits,
                             uint32_t key_bits, uint64_t* keys, uint32_t* vals) {
   const uint64_t a = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1667,6 +1684,7 @@ k_sortp_make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t
   const uint64_t base = (uint64_t)blockIdx.x * P::TILE;
   const uint64_t ts_min = sc->ts_min_biased;
   constexpr int G = ITEMS < 4 ? ITEMS : 4; /* rows per thread whose loads are in flight together */
+  RankMemo memo_dev{0, 0, false}, memo_res{0, 0, false};
   for (int r0 = 0; r0 < P::ITEMS; r0 += G) {
     uint32_t meta[G];
     uint64_t dev[G], res[G], ts[G];
@@ -1685,8 +1703,8 @@ k_sortp_make_keys(Columns c, uint64_t n, SortSets s, const Scalars* sc, uint32_t
       if (a >= n) continue;
       uint64_t key = 1ULL << key_bits; /* dropped rows sort behind everything */
       if (meta[g] & KTJ_M_VALID) {
-        const uint64_t rd = set_rank(s.dev_keys, s.dev_rank, dev[g]);
-        const uint64_t rr = set_rank(s.res_keys, s.res_rank, res[g]);
+        const uint64_t rd = set_rank_memo(s.dev_keys, s.dev_rank, dev[g], memo_dev);
+        const uint64_t rr = set_rank_memo(s.res_keys, s.res_rank, res[g], memo_res);
         const uint64_t rel = (ts[g] ^ 0x8000000000000000ULL) - ts_min;
         key = ((((rd << res_bits) | rr)) << ts_bits) | rel;
       }
