@@ -2646,16 +2646,18 @@ k_emit_direct(const MatRow* mat, const uint32_t* perm, const uint64_t* offs, con
   /* A wavefront that has just started comes first on its SIMD until the loads of its joined row are
    * on their way (two dependent loads with a few instructions between them, which would otherwise
    * queue behind the formatting of the two older wavefronts): config 3 4.70 -> 4.61 ms, config 4
-   * 2.12 -> 2.07 ms.  Kept up until the name is copied, or lowered in steps: slower. */
+   * 2.12 -> 2.07 ms.  Priority 1, 2 or 3: the same.  Kept up until the name is copied, lowered in
+   * steps, lowered behind the branch below or before the row's loads: slower or no gain; a
+   * scheduling barrier in place of the priority: no gain. */
   __builtin_amdgcn_s_setprio(3);
   if (active) { row = perm[i]; o = offs[i]; active = offs[i + 1] != o; } /* one wait for both */
   MatRow m;
   BlockWriter w;
   w.stage_init((uint32_t)threadIdx.x * (KTJ_STAGE_BLOCKS * 16u));
   ActivityParts<BlockWriter> parts;
-  if (active) m = mat[row];
-  __builtin_amdgcn_s_setprio(0);
   if (active) {
+    m = mat[row];
+    __builtin_amdgcn_s_setprio(0); /* (a wavefront without any activity keeps it: it ends at once) */
     w.begin(out, prefix_len + o, i ? kind_sorted[i - 1] : 0u, i == 0);
     w.stage_follow();
     format_head(w, m, ctx, parts);
